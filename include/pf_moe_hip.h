@@ -1,0 +1,132 @@
+/* C-ABI shim between the C11 host side (qwen4_moe.h entry points) and the HIP
+ * kernels for gfx950.  Plain pointers and sizes only; no HIP or C++ types.
+ *
+ * These entry points take the place of the reference's device-side MoE step,
+ * qw4f_routed_encode and its scratch description QW4FRoutedWork
+ * (src/qwen4_moe_internal.h:36-78, src/qwen4_moe.m:271-402): router product,
+ * softmax/top-k, indexed expert products and the weighted reduction all run on
+ * the device and expert ids are not read back unless the caller asks for them.
+ *
+ * Every function returns PF_HIP_OK (0) or one of the codes below.  Pointers
+ * named d_* are device pointers, everything else is host memory.  `stream` is a
+ * hipStream_t passed as void* (NULL = the default stream).  A workspace serves
+ * one forward at a time; different workspaces of one layer are independent. */
+#ifndef PF_MOE_HIP_H
+#define PF_MOE_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    PF_HIP_OK = 0,
+    PF_HIP_E_ARGUMENT = 1,     /* null pointer, bad size */
+    PF_HIP_E_UNSUPPORTED = 2,  /* format or dimension outside the kernels' range */
+    PF_HIP_E_MEMORY = 3,       /* device or host allocation failed */
+    PF_HIP_E_RUNTIME = 4,      /* a HIP call or launch failed; see pf_hip_last_error */
+    PF_HIP_E_NO_DEVICE = 5
+};
+
+/* Bits of the error word the kernels maintain (the reference's convention,
+ * src/qwen4_gpu.h:27-31: bit 1 nonfinite, bit 2 bounds). */
+#define PF_HIP_ERR_NONFINITE 2u
+#define PF_HIP_ERR_BOUNDS 4u
+
+typedef struct PfHipMoe PfHipMoe;    /* one layer's eight tensors, resident in HBM */
+typedef struct PfHipWork PfHipWork;  /* device scratch for up to token_cap tokens */
+
+/* Dimensions of Qwen4MoeConfig (src/qwen4_types.h:75-80) plus the GGUF type of
+ * each tensor in Qwen4MoeWeights order: router, gate, up, down, shared gate,
+ * shared up, shared down, shared router (src/qwen4_moe.h:7-10). */
+typedef struct {
+    uint32_t hidden, experts, top_k, inter, shared_inter, down_physical;
+    uint32_t norm_topk;
+    uint32_t type[8];
+} PfHipMoeDesc;
+
+int pf_hip_device_count(void);
+const char *pf_hip_last_error(void);
+
+/* Uploads the eight tensors (GGUF byte layout, bytes[i] each) into HBM.  The
+ * host bytes are not referenced after the call returns. */
+int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const host_weights[8],
+                      const size_t bytes[8], PfHipMoe **out);
+void pf_hip_moe_destroy(PfHipMoe *moe);
+/* Total HBM bytes held by the layer. */
+size_t pf_hip_moe_bytes(const PfHipMoe *moe);
+
+size_t pf_hip_work_bytes(const PfHipMoeDesc *desc, size_t token_cap);
+int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWork **out);
+void pf_hip_work_destroy(PfHipWork *work);
+
+/* Enqueues one forward on `stream`: d_x [tokens, hidden] -> d_y [tokens, hidden],
+ * row pitches in floats.  Asynchronous; results, routes (in the workspace) and
+ * the error word are valid after the stream has been synchronised. */
+int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
+                              size_t x_pitch, float *d_y, size_t y_pitch, size_t tokens,
+                              void *stream);
+/* Device pointers into the workspace, valid after a forward: expert ids
+ * [tokens, top_k] uint32, route weights [tokens, top_k], router logits
+ * [tokens, experts], the error word (one uint32). */
+const uint32_t *pf_hip_work_ids(const PfHipWork *work);
+const float *pf_hip_work_route_weights(const PfHipWork *work);
+const float *pf_hip_work_logits(const PfHipWork *work);
+const uint32_t *pf_hip_work_error_word(const PfHipWork *work);
+/* Number of tokens of the last forward whose routing was re-evaluated in the
+ * reference's serial order because two candidate logits were too close. */
+int pf_hip_work_exact_rows(PfHipWork *work, uint32_t *count);
+
+/* Host-buffer forward used by qwen4_moe_forward: copies x in, runs the forward,
+ * copies y (and ids/weights when non-NULL) out, returns the error word.  Pitches
+ * in bytes.  Outputs are written only when the error word is zero. */
+int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x,
+                            size_t x_pitch_bytes, float *y, size_t y_pitch_bytes,
+                            uint32_t *ids, size_t ids_pitch_bytes, float *weights,
+                            size_t weights_pitch_bytes, size_t tokens, uint32_t *error_word);
+
+/* qwen4_moe_route on the device (src/qwen4_moe.c:188-249), reference evaluation
+ * order.  Dense host arrays: logits/probs [tokens, experts], ids/weights
+ * [tokens, top_k].  *bad_row receives the first row with a nonfinite logit when
+ * the error word has PF_HIP_ERR_NONFINITE set; nothing is written then. */
+int pf_hip_route_host(const float *logits, size_t tokens, size_t experts, size_t top_k,
+                      int norm_topk, float *probs, uint32_t *ids, float *weights,
+                      uint32_t *error_word, uint64_t *bad_row);
+
+/* qw4_moe_group_pairs on the device (src/qwen4_moe.c:251-303): histogram,
+ * exclusive scan, stable placement.  ids dense [tokens, top_k]; outputs
+ * offsets [experts+1], pair_to_row/row_to_pair [tokens*top_k] as uint64.  Error
+ * word: PF_HIP_ERR_BOUNDS for an id >= experts, PF_HIP_ERR_NONFINITE is unused;
+ * *duplicate is set when a token repeats an id.  Outputs untouched on error. */
+int pf_hip_group_pairs_host(const uint32_t *ids, size_t tokens, size_t experts, size_t top_k,
+                            uint64_t *offsets, uint64_t *pair_to_row, uint64_t *row_to_pair,
+                            uint32_t *error_word, int *duplicate);
+
+/* qw4_packed_matmul / qw4_packed_decode_row on the device for one expert's
+ * bytes (src/qwen4_packed.c:124-181), reference evaluation order, bit-identical.
+ * x dense [rows, k_logical], y dense [rows, n_out]. */
+int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_bytes, size_t row_bytes,
+                              size_t n_out, size_t k_logical, const float *x, size_t rows,
+                              float *y, uint32_t *error_word);
+int pf_hip_packed_decode_row_host(uint32_t gguf_type, const void *row_bytes_ptr, size_t row_bytes,
+                                  size_t k_storage, float *out, uint32_t *error_word);
+
+/* Minimal device-memory and timing helpers so that a host program can keep
+ * inputs resident and time launches with events on the launch stream. */
+int pf_hip_malloc(void **d_ptr, size_t bytes);
+void pf_hip_free(void *d_ptr);
+int pf_hip_memcpy_h2d(void *d_dst, const void *src, size_t bytes);
+int pf_hip_memcpy_d2h(void *dst, const void *d_src, size_t bytes);
+int pf_hip_synchronize(void);
+/* Runs `iters` forwards back to back on one stream, input row block i % n_inputs
+ * of d_x each time, and returns the elapsed milliseconds between two events
+ * recorded on that stream around the launches. */
+int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
+                             size_t n_inputs, float *d_y, size_t tokens, size_t iters,
+                             float *elapsed_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

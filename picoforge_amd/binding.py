@@ -1,0 +1,189 @@
+"""Loading and typing of the C-ABI libraries.
+
+`load_product()` opens picoforge_amd/libpicoforge_moe.so, the shipped library:
+the C11 host side with the entry points of the reference's src/qwen4_moe.h plus
+the HIP shim of include/pf_moe_hip.h.  It raises if the library is missing; no
+part of this package computes anything on the CPU in its place.
+
+`MoeApi` types the eight entry points (and the two tested private helpers) of a
+library that follows the reference's boundary.  The same class wraps the CPU
+oracle (functions prefixed orc_) and a build of the reference's own C path, so
+tests drive all three through identical code.
+"""
+import ctypes as C
+from pathlib import Path
+
+import numpy as np
+
+from . import abi
+
+PACKAGE_DIR = Path(__file__).resolve().parent
+REPO_DIR = PACKAGE_DIR.parent
+PRODUCT_LIB = PACKAGE_DIR / "libpicoforge_moe.so"
+SYNTH_LIB = PACKAGE_DIR / "libpf_synth.so"
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def _open(path):
+    if not Path(path).exists():
+        raise LibraryMissing(f"{path} is not built: run python -c 'import __graft_entry__ as g; g.build()' "
+                             "or make -C picoforge_amd/csrc")
+    return C.CDLL(str(path), mode=C.RTLD_LOCAL)
+
+
+class MoeApi:
+    """Typed view of one library exporting the reference's MoE boundary."""
+
+    def __init__(self, lib, moe_prefix="qwen4_moe_", private_prefix="qw4_moe_", packed_prefix="qw4_packed_"):
+        self.lib = lib
+        P, E = C.POINTER, abi.Qwen4Error
+        vp, sz = C.c_void_p, C.c_size_t
+
+        def bind(name, restype, *argtypes):
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = list(argtypes)
+            return fn
+
+        m = moe_prefix
+        self.create = bind(m + "create", C.c_int, P(abi.Qwen4MoeConfig), P(abi.Qwen4MoeWeights), P(vp), P(E))
+        self.destroy = bind(m + "destroy", None, vp)
+        self.work_size = bind(m + "work_size", C.c_int, vp, sz, P(sz), P(E))
+        self.work_create = bind(m + "work_create", C.c_int, vp, sz, sz, P(vp), P(E))
+        self.work_reset = bind(m + "work_reset", C.c_int, vp, P(E))
+        self.work_destroy = bind(m + "work_destroy", None, vp)
+        self.route = bind(m + "route", C.c_int, P(abi.Qwen4MoeConfig), abi.Qwen4F32, abi.Qwen4MoeRoutes,
+                          abi.Qwen4F32Mut, P(E))
+        self.forward = bind(m + "forward", C.c_int, vp, abi.Qwen4F32, abi.Qwen4F32Mut, P(abi.Qwen4MoeRoutes), vp,
+                            P(E))
+        self.group_pairs = bind(private_prefix + "group_pairs", C.c_int, P(abi.Qwen4MoeConfig), abi.Qwen4U32Mut,
+                                abi.QW4MoeGrouping, P(E))
+        self.observe = bind(private_prefix + "observe", None, vp, abi.OBSERVER, vp)
+        self.layout_init = bind(packed_prefix + "layout_init", C.c_int, P(abi.GgufTensor), sz,
+                                P(abi.QW4PackedLayout), P(E))
+        self.decode_row = bind(packed_prefix + "decode_row", C.c_int, P(abi.QW4PackedCpuView), sz, sz, vp, sz, P(E))
+        self.matmul = bind(packed_prefix + "matmul", C.c_int, P(abi.QW4PackedCpuView), sz, abi.Qwen4F32,
+                           abi.Qwen4F32Mut, P(E))
+
+
+def load_product():
+    lib = _open(PRODUCT_LIB)
+    api = MoeApi(lib)
+    api.hip = HipShim(lib)
+    return api
+
+
+def load_oracle():
+    """CPU oracle: test infrastructure (oracle/), never part of the product path."""
+    lib = _open(REPO_DIR / "oracle" / "liborc.so")
+    return MoeApi(lib, moe_prefix="orc_moe_", private_prefix="orc_moe_", packed_prefix="orc_packed_")
+
+
+def load_reference():
+    """The reference's own C path, if oracle/_ref was built where the reference tree is mounted."""
+    path = REPO_DIR / "oracle" / "_ref" / "libqwen4_ref.so"
+    return MoeApi(_open(path)) if path.exists() else None
+
+
+class HipShim:
+    """include/pf_moe_hip.h"""
+
+    def __init__(self, lib):
+        P, vp, sz, u32p = C.POINTER, C.c_void_p, C.c_size_t, C.POINTER(C.c_uint32)
+
+        def bind(name, restype, *argtypes):
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = list(argtypes)
+            setattr(self, name.replace("pf_hip_", ""), fn)
+
+        bind("pf_hip_device_count", C.c_int)
+        bind("pf_hip_last_error", C.c_char_p)
+        bind("pf_hip_moe_create", C.c_int, P(PfHipMoeDesc), P(vp), P(sz), P(vp))
+        bind("pf_hip_moe_destroy", None, vp)
+        bind("pf_hip_moe_bytes", sz, vp)
+        bind("pf_hip_work_bytes", sz, P(PfHipMoeDesc), sz)
+        bind("pf_hip_work_create", C.c_int, vp, sz, P(vp))
+        bind("pf_hip_work_destroy", None, vp)
+        bind("pf_hip_moe_forward_device", C.c_int, vp, vp, vp, sz, vp, sz, sz, vp)
+        bind("pf_hip_work_ids", vp, vp)
+        bind("pf_hip_work_route_weights", vp, vp)
+        bind("pf_hip_work_logits", vp, vp)
+        bind("pf_hip_work_error_word", vp, vp)
+        bind("pf_hip_work_exact_rows", C.c_int, vp, u32p)
+        bind("pf_hip_moe_forward_host", C.c_int, vp, vp, vp, sz, vp, sz, vp, sz, vp, sz, sz, u32p)
+        bind("pf_hip_route_host", C.c_int, vp, sz, sz, sz, C.c_int, vp, vp, vp, u32p, P(C.c_uint64))
+        bind("pf_hip_group_pairs_host", C.c_int, vp, sz, sz, sz, vp, vp, vp, u32p, P(C.c_int))
+        bind("pf_hip_packed_matmul_host", C.c_int, C.c_uint32, vp, sz, sz, sz, vp, sz, vp, u32p)
+        bind("pf_hip_packed_decode_row_host", C.c_int, C.c_uint32, vp, sz, sz, vp, u32p)
+        bind("pf_hip_malloc", C.c_int, P(vp), sz)
+        bind("pf_hip_free", None, vp)
+        bind("pf_hip_memcpy_h2d", C.c_int, vp, vp, sz)
+        bind("pf_hip_memcpy_d2h", C.c_int, vp, vp, sz)
+        bind("pf_hip_synchronize", C.c_int)
+        bind("pf_hip_moe_time_forwards", C.c_int, vp, vp, vp, sz, vp, sz, sz, P(C.c_float))
+
+    def check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what}: shim status {rc}: {self.last_error().decode()}")
+
+    def to_device(self, array):
+        array = np.ascontiguousarray(array)
+        ptr = C.c_void_p()
+        self.check(self.malloc(C.byref(ptr), array.nbytes), "malloc")
+        if array.nbytes:
+            self.check(self.memcpy_h2d(ptr, array.ctypes.data, array.nbytes), "h2d")
+        return ptr
+
+    def from_device(self, ptr, shape, dtype):
+        out = np.empty(shape, dtype=dtype)
+        if out.nbytes:
+            self.check(self.memcpy_d2h(out.ctypes.data, ptr, out.nbytes), "d2h")
+        return out
+
+
+class PfHipMoeDesc(C.Structure):
+    _fields_ = [("hidden", C.c_uint32), ("experts", C.c_uint32), ("top_k", C.c_uint32), ("inter", C.c_uint32),
+                ("shared_inter", C.c_uint32), ("down_physical", C.c_uint32), ("norm_topk", C.c_uint32),
+                ("type", C.c_uint32 * 8)]
+
+
+class Synth:
+    """picoforge_amd/csrc/pf_synth.c"""
+
+    def __init__(self):
+        lib = _open(SYNTH_LIB)
+        vp, sz = C.c_void_p, C.c_size_t
+        lib.pf_synth_normal_f32.argtypes = [vp, sz, C.c_uint64, C.c_float, C.c_float]
+        lib.pf_synth_q4k_quantize.argtypes = [vp, sz, vp]
+        lib.pf_synth_q4k_normal.argtypes = [vp, sz, C.c_uint64, C.c_float]
+        lib.pf_synth_iq2xxs_uniform.argtypes = [vp, sz, C.c_uint64, C.c_float]
+        for fn in (lib.pf_synth_normal_f32, lib.pf_synth_q4k_quantize, lib.pf_synth_q4k_normal,
+                   lib.pf_synth_iq2xxs_uniform):
+            fn.restype = None
+        self.lib = lib
+
+    def normal(self, shape, seed, std=1.0, mean=0.0):
+        out = np.empty(shape, dtype=np.float32)
+        self.lib.pf_synth_normal_f32(out.ctypes.data, out.size, seed, mean, std)
+        return out
+
+    def q4k_normal(self, blocks, seed, std):
+        out = np.empty(blocks * 144, dtype=np.uint8)
+        self.lib.pf_synth_q4k_normal(out.ctypes.data, blocks, seed, std)
+        return out
+
+    def q4k_quantize(self, values):
+        values = np.ascontiguousarray(values, dtype=np.float32)
+        assert values.size % 256 == 0
+        out = np.empty(values.size // 256 * 144, dtype=np.uint8)
+        self.lib.pf_synth_q4k_quantize(values.ctypes.data, values.size // 256, out.ctypes.data)
+        return out
+
+    def iq2xxs_uniform(self, blocks, seed, d_base=2.0 ** -12):
+        out = np.empty(blocks * 66, dtype=np.uint8)
+        self.lib.pf_synth_iq2xxs_uniform(out.ctypes.data, blocks, seed, d_base)
+        return out

@@ -1,0 +1,431 @@
+// C-ABI entry points of the HIP side (include/pf_moe_hip.h).
+#include "pf_moe_internal.h"
+#include "../../include/pf_iq2_codes.h"
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+static thread_local char g_error[256] = "";
+
+void pf_set_error(const char *what, hipError_t code) {
+    snprintf(g_error, sizeof g_error, "%s: %s", what, hipGetErrorString(code));
+}
+#define HIP_TRY(call)                                                                                   \
+    do {                                                                                                \
+        hipError_t e_ = (call);                                                                         \
+        if (e_ != hipSuccess) { pf_set_error(#call, e_); return PF_HIP_E_RUNTIME; }                     \
+    } while (0)
+
+extern "C" const char *pf_hip_last_error(void) { return g_error; }
+
+extern "C" int pf_hip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+// 256 x 8 IQ2_XXS magnitudes, one copy per process (single device per process).
+static uint64_t *g_grid = nullptr;
+const uint64_t *pf_device_iq2_grid(void) {
+    if (g_grid) return g_grid;
+    uint64_t host[256];
+    for (unsigned i = 0; i < 256; i++) {
+        uint64_t v = 0;
+        for (unsigned j = 0; j < 8; j++) v |= (uint64_t)pf_iq2_grid_byte(i, j) << (8 * j);
+        host[i] = v;
+    }
+    uint64_t *d = nullptr;
+    if (hipMalloc(&d, sizeof host) != hipSuccess) return nullptr;
+    if (hipMemcpy(d, host, sizeof host, hipMemcpyHostToDevice) != hipSuccess) { hipFree(d); return nullptr; }
+    g_grid = d;
+    return g_grid;
+}
+
+static bool block_geometry(uint32_t type, size_t *block, size_t *bytes) {
+    switch (type) {
+    case PF_F32: *block = 1; *bytes = 4; return true;
+    case PF_Q4_K: *block = 256; *bytes = 144; return true;
+    case PF_IQ2_XXS: *block = 256; *bytes = 66; return true;
+    default: return false;
+    }
+}
+
+extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const host_weights[8], const size_t bytes[8],
+                                 PfHipMoe **out) {
+    if (out) *out = nullptr;
+    if (!desc || !host_weights || !bytes || !out) return PF_HIP_E_ARGUMENT;
+    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
+    const size_t h = desc->hidden, i = desc->inter, s = desc->shared_inter, E = desc->experts;
+    const size_t k_storage[8] = {h, h, h, desc->down_physical, h, h, s, h};
+    const size_t n_out[8] = {E, i, i, h, s, s, h, 1};
+    const size_t experts[8] = {1, E, E, E, 1, 1, 1, 1};
+    if (!h || !i || !s || !E || !desc->top_k || desc->top_k > E || desc->down_physical < i) return PF_HIP_E_ARGUMENT;
+    if (desc->type[0] != PF_F32 || desc->type[7] != PF_F32) return PF_HIP_E_UNSUPPORTED;
+    PfHipMoe *m = (PfHipMoe *)calloc(1, sizeof *m);
+    if (!m) return PF_HIP_E_MEMORY;
+    m->desc = *desc;
+    for (int a = 0; a < 8; a++) {
+        size_t block, size;
+        if (!block_geometry(desc->type[a], &block, &size) || k_storage[a] % block) {
+            pf_hip_moe_destroy(m);
+            return PF_HIP_E_UNSUPPORTED;
+        }
+        m->row_bytes[a] = k_storage[a] / block * size;
+        m->expert_bytes[a] = m->row_bytes[a] * n_out[a];
+        m->bytes[a] = m->expert_bytes[a] * experts[a];
+        if (bytes[a] < m->bytes[a] || !host_weights[a]) { pf_hip_moe_destroy(m); return PF_HIP_E_ARGUMENT; }
+    }
+    m->iq2_grid = const_cast<uint64_t *>(pf_device_iq2_grid());
+    if (!m->iq2_grid) { pf_hip_moe_destroy(m); return PF_HIP_E_MEMORY; }
+    for (int a = 0; a < 8; a++) {
+        hipError_t e = hipMalloc((void **)&m->w[a], m->bytes[a]);
+        if (e == hipSuccess) e = hipMemcpy(m->w[a], host_weights[a], m->bytes[a], hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            pf_set_error("weight upload", e);
+            pf_hip_moe_destroy(m);
+            return e == hipErrorOutOfMemory ? PF_HIP_E_MEMORY : PF_HIP_E_RUNTIME;
+        }
+        m->total_bytes += m->bytes[a];
+    }
+    *out = m;
+    return PF_HIP_OK;
+}
+
+extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
+    if (!m) return;
+    for (int a = 0; a < 8; a++) if (m->w[a]) (void)hipFree(m->w[a]);
+    free(m);
+}
+
+extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_bytes : 0; }
+
+// workspace layout: a list of (pointer slot, bytes) carved from one allocation
+struct Carve { size_t offset[16], bytes[16], total; int n; };
+static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
+    Carve c;
+    memset(&c, 0, sizeof c);
+    const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden;
+    const size_t want[] = {
+        T * E * 4,            // 0 logits
+        T * E * 4,            // 1 logit_ssq
+        T * K * 4,            // 2 route weights
+        T * K * d->inter * 4, // 3 act
+        T * d->shared_inter * 4, // 4 shared act
+        T * 4,                // 5 shared scale
+        T * H * 4,            // 6 x staging
+        T * H * 4,            // 7 y staging
+        T * K * 4,            // 8 ids
+        256,                  // 9 error word
+        256,                  // 10 exact rows
+        T * 4,                // 11 route flags
+    };
+    c.n = (int)(sizeof want / sizeof want[0]);
+    for (int j = 0; j < c.n; j++) {
+        c.offset[j] = c.total;
+        c.bytes[j] = (want[j] + 255) & ~(size_t)255;
+        c.total += c.bytes[j];
+    }
+    return c;
+}
+
+extern "C" size_t pf_hip_work_bytes(const PfHipMoeDesc *desc, size_t token_cap) {
+    return desc ? plan_work(desc, token_cap).total : 0;
+}
+
+extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWork **out) {
+    if (out) *out = nullptr;
+    if (!moe || !out) return PF_HIP_E_ARGUMENT;
+    PfHipWork *w = (PfHipWork *)calloc(1, sizeof *w);
+    if (!w) return PF_HIP_E_MEMORY;
+    const Carve c = plan_work(&moe->desc, token_cap);
+    uint8_t *base = nullptr;
+    hipError_t e = hipMalloc((void **)&base, c.total);
+    if (e == hipSuccess) e = hipMemset(base, 0, c.total);
+    if (e != hipSuccess) {
+        pf_set_error("workspace allocation", e);
+        if (base) (void)hipFree(base);
+        free(w);
+        return PF_HIP_E_MEMORY;
+    }
+    w->moe = moe; w->cap = token_cap; w->bytes = c.total;
+    w->logits = (float *)(base + c.offset[0]);
+    w->logit_ssq = (float *)(base + c.offset[1]);
+    w->route_weights = (float *)(base + c.offset[2]);
+    w->act = (float *)(base + c.offset[3]);
+    w->shared_act = (float *)(base + c.offset[4]);
+    w->shared_scale = (float *)(base + c.offset[5]);
+    w->x = (float *)(base + c.offset[6]);
+    w->y = (float *)(base + c.offset[7]);
+    w->ids = (uint32_t *)(base + c.offset[8]);
+    w->error_word = (uint32_t *)(base + c.offset[9]);
+    w->exact_rows = (uint32_t *)(base + c.offset[10]);
+    w->route_flags = (uint32_t *)(base + c.offset[11]);
+    *out = w;
+    return PF_HIP_OK;
+}
+
+extern "C" void pf_hip_work_destroy(PfHipWork *w) {
+    if (!w) return;
+    if (w->logits) (void)hipFree(w->logits);   // base of the single allocation
+    if (w->host_stage) (void)hipHostFree(w->host_stage);
+    free(w);
+}
+
+extern "C" const uint32_t *pf_hip_work_ids(const PfHipWork *w) { return w ? w->ids : nullptr; }
+extern "C" const float *pf_hip_work_route_weights(const PfHipWork *w) { return w ? w->route_weights : nullptr; }
+extern "C" const float *pf_hip_work_logits(const PfHipWork *w) { return w ? w->logits : nullptr; }
+extern "C" const uint32_t *pf_hip_work_error_word(const PfHipWork *w) { return w ? w->error_word : nullptr; }
+
+extern "C" int pf_hip_work_exact_rows(PfHipWork *w, uint32_t *count) {
+    if (!w || !count) return PF_HIP_E_ARGUMENT;
+    HIP_TRY(hipMemcpy(count, w->exact_rows, 4, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x, size_t x_pitch, float *d_y,
+                              size_t y_pitch) {
+    PfKernelArgs a;
+    memset(&a, 0, sizeof a);
+    const PfHipMoeDesc *d = &m->desc;
+    a.hidden = (int)d->hidden; a.experts = (int)d->experts; a.top_k = (int)d->top_k; a.inter = (int)d->inter;
+    a.shared_inter = (int)d->shared_inter; a.down_physical = (int)d->down_physical; a.norm_topk = (int)d->norm_topk;
+    for (int j = 0; j < 8; j++) {
+        a.type[j] = d->type[j];
+        a.w[j] = m->w[j];
+        a.row_bytes[j] = m->row_bytes[j];
+        a.expert_bytes[j] = m->expert_bytes[j];
+    }
+    a.iq2_grid = m->iq2_grid;
+    a.x = d_x; a.x_pitch = x_pitch; a.y = d_y; a.y_pitch = y_pitch;
+    a.logits = w->logits; a.logit_ssq = w->logit_ssq; a.ids = w->ids; a.route_weights = w->route_weights;
+    a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale;
+    a.error_word = w->error_word; a.exact_rows = w->exact_rows; a.route_flags = w->route_flags;
+    return a;
+}
+
+__global__ void pf_k_clear2(uint32_t *a, uint32_t *b) { *a = 0; *b = 0; }
+
+extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch,
+                                         float *d_y, size_t y_pitch, size_t tokens, void *stream) {
+    if (!moe || !work || work->moe != moe) return PF_HIP_E_ARGUMENT;
+    if (tokens > work->cap) return PF_HIP_E_ARGUMENT;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!d_x || !d_y || x_pitch < moe->desc.hidden || y_pitch < moe->desc.hidden) return PF_HIP_E_ARGUMENT;
+    const PfHipMoeDesc *d = &moe->desc;
+    // the general kernels stage one token's activations in LDS
+    const size_t lds_need = ((size_t)d->top_k * d->inter + d->shared_inter) * 4;
+    const size_t lds_route = ((size_t)d->hidden + 3 * (size_t)d->experts) * 4;
+    if (lds_need > 64 * 1024 || lds_route > 64 * 1024 || (size_t)d->hidden * 4 > 64 * 1024) {
+        snprintf(g_error, sizeof g_error, "dimensions exceed the LDS staging of the general kernels");
+        return PF_HIP_E_UNSUPPORTED;
+    }
+    if (tokens * (size_t)d->top_k > 0x7fffffffu / 4) return PF_HIP_E_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(pf_k_clear2, dim3(1), dim3(1), 0, s, work->error_word, work->exact_rows);
+    PfKernelArgs a = make_args(moe, work, d_x, x_pitch, d_y, y_pitch);
+    pf_launch_general(a, (int)tokens, s);
+    HIP_TRY(hipGetLastError());
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
+                                       float *y, size_t y_pitch_bytes, uint32_t *ids, size_t ids_pitch_bytes,
+                                       float *weights, size_t weights_pitch_bytes, size_t tokens,
+                                       uint32_t *error_word) {
+    if (!moe || !work || !error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!x || !y || tokens > work->cap) return PF_HIP_E_ARGUMENT;
+    const size_t H = moe->desc.hidden, K = moe->desc.top_k;
+    HIP_TRY(hipMemcpy2D(work->x, H * 4, x, x_pitch_bytes, H * 4, tokens, hipMemcpyHostToDevice));
+    int rc = pf_hip_moe_forward_device(moe, work, work->x, H, work->y, H, tokens, nullptr);
+    if (rc != PF_HIP_OK) return rc;
+    HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
+    if (*error_word) return PF_HIP_OK;
+    HIP_TRY(hipMemcpy2D(y, y_pitch_bytes, work->y, H * 4, H * 4, tokens, hipMemcpyDeviceToHost));
+    if (ids) HIP_TRY(hipMemcpy2D(ids, ids_pitch_bytes, work->ids, K * 4, K * 4, tokens, hipMemcpyDeviceToHost));
+    if (weights)
+        HIP_TRY(hipMemcpy2D(weights, weights_pitch_bytes, work->route_weights, K * 4, K * 4, tokens,
+                            hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+// ---- stand-alone operators on host buffers ---------------------------------------
+struct DeviceBlock {   // one allocation, freed on scope exit
+    uint8_t *p = nullptr;
+    ~DeviceBlock() { if (p) (void)hipFree(p); }
+};
+
+extern "C" int pf_hip_route_host(const float *logits, size_t tokens, size_t experts, size_t top_k, int norm_topk,
+                                 float *probs, uint32_t *ids, float *weights, uint32_t *error_word,
+                                 uint64_t *bad_row) {
+    if (!error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (bad_row) *bad_row = 0;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!logits || !probs || !ids || !weights || !experts || !top_k || top_k > experts) return PF_HIP_E_ARGUMENT;
+    if (tokens * experts > 0x7fffffffu || pf_hip_device_count() < 1) return PF_HIP_E_UNSUPPORTED;
+    const size_t zb = tokens * experts * 4, kb = tokens * top_k * 4;
+    const size_t o_p = (zb + 255) & ~(size_t)255, o_i = o_p * 2, o_w = o_i + ((kb + 255) & ~(size_t)255),
+                 o_e = o_w + ((kb + 255) & ~(size_t)255);
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, o_e + 256));
+    HIP_TRY(hipMemcpy(blk.p, logits, zb, hipMemcpyHostToDevice));
+    unsigned long long init[2] = {0ull, ~0ull};   // error word, first bad row
+    HIP_TRY(hipMemcpy(blk.p + o_e, init, sizeof init, hipMemcpyHostToDevice));
+    int rc = pf_route_exact_device((const float *)blk.p, (int)tokens, (int)experts, (int)top_k, norm_topk,
+                                   (float *)(blk.p + o_p), (uint32_t *)(blk.p + o_i), (float *)(blk.p + o_w),
+                                   (uint32_t *)(blk.p + o_e), (unsigned long long *)(blk.p + o_e + 8), nullptr);
+    if (rc != PF_HIP_OK) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    unsigned long long back[2];
+    HIP_TRY(hipMemcpy(back, blk.p + o_e, sizeof back, hipMemcpyDeviceToHost));
+    *error_word = (uint32_t)back[0];
+    if (*error_word) {
+        if (bad_row) *bad_row = back[1];
+        return PF_HIP_OK;
+    }
+    HIP_TRY(hipMemcpy(probs, blk.p + o_p, zb, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(ids, blk.p + o_i, kb, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(weights, blk.p + o_w, kb, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_group_pairs_host(const uint32_t *ids, size_t tokens, size_t experts, size_t top_k,
+                                       uint64_t *offsets, uint64_t *pair_to_row, uint64_t *row_to_pair,
+                                       uint32_t *error_word, int *duplicate) {
+    if (!error_word || !duplicate || !offsets || !experts || !top_k) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    *duplicate = 0;
+    const size_t pairs = tokens * top_k;
+    if (pairs > 0x3fffffffu || experts > 0x3fffffffu || pf_hip_device_count() < 1) return PF_HIP_E_UNSUPPORTED;
+    if (pairs && (!ids || !pair_to_row || !row_to_pair)) return PF_HIP_E_ARGUMENT;
+    const size_t pb = ((pairs ? pairs : 1) * 4 + 255) & ~(size_t)255, eb = ((experts + 1) * 4 + 255) & ~(size_t)255;
+    // ids | counts | offsets | pair_to_row | row_to_pair | error
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, 3 * pb + 2 * eb + 256));
+    uint32_t *d_ids = (uint32_t *)blk.p, *d_counts = (uint32_t *)(blk.p + pb), *d_off = (uint32_t *)(blk.p + pb + eb);
+    uint32_t *d_p2r = (uint32_t *)(blk.p + pb + 2 * eb), *d_r2p = (uint32_t *)(blk.p + 2 * pb + 2 * eb);
+    uint32_t *d_err = (uint32_t *)(blk.p + 3 * pb + 2 * eb);
+    if (pairs) HIP_TRY(hipMemcpy(d_ids, ids, pairs * 4, hipMemcpyHostToDevice));
+    int rc = pf_group_pairs_device(d_ids, (int)tokens, (int)experts, (int)top_k, d_counts, d_off, d_p2r, d_r2p, d_err,
+                                   nullptr);
+    if (rc != PF_HIP_OK) return rc;
+    HIP_TRY(hipDeviceSynchronize());
+    uint32_t err = 0;
+    HIP_TRY(hipMemcpy(&err, d_err, 4, hipMemcpyDeviceToHost));
+    if (err != 0xffffffffu) {   // first offending pair in scan order, low bit = kind
+        if (err & 1u) *duplicate = 1;
+        else *error_word = PF_HIP_ERR_BOUNDS;
+        return PF_HIP_OK;
+    }
+    uint32_t *host = (uint32_t *)malloc(((experts + 1) > pairs ? (experts + 1) : pairs) * 4);
+    if (!host) return PF_HIP_E_MEMORY;
+    hipError_t e = hipMemcpy(host, d_off, (experts + 1) * 4, hipMemcpyDeviceToHost);
+    for (size_t j = 0; e == hipSuccess && j <= experts; j++) offsets[j] = host[j];
+    if (e == hipSuccess && pairs) {
+        e = hipMemcpy(host, d_p2r, pairs * 4, hipMemcpyDeviceToHost);
+        for (size_t j = 0; e == hipSuccess && j < pairs; j++) pair_to_row[j] = host[j];
+        if (e == hipSuccess) e = hipMemcpy(host, d_r2p, pairs * 4, hipMemcpyDeviceToHost);
+        for (size_t j = 0; e == hipSuccess && j < pairs; j++) row_to_pair[j] = host[j];
+    }
+    free(host);
+    if (e != hipSuccess) { pf_set_error("group download", e); return PF_HIP_E_RUNTIME; }
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_bytes, size_t row_bytes, size_t n_out,
+                                         size_t k_logical, const float *x, size_t rows, float *y,
+                                         uint32_t *error_word) {
+    if (!error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (rows == 0) return PF_HIP_OK;
+    size_t block, size;
+    if (!block_geometry(gguf_type, &block, &size)) return PF_HIP_E_UNSUPPORTED;
+    if (!expert_bytes || !x || !y || !n_out || !k_logical) return PF_HIP_E_ARGUMENT;
+    if (rows * n_out > 0x7fffffffu || k_logical > 0x7fffffffu || pf_hip_device_count() < 1) return PF_HIP_E_UNSUPPORTED;
+    const uint64_t *grid = pf_device_iq2_grid();
+    if (!grid) return PF_HIP_E_MEMORY;
+    const size_t wb = (row_bytes * n_out + 255) & ~(size_t)255, xb = (rows * k_logical * 4 + 255) & ~(size_t)255,
+                 yb = (rows * n_out * 4 + 255) & ~(size_t)255;
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, wb + xb + yb + 256));
+    HIP_TRY(hipMemcpy(blk.p, expert_bytes, row_bytes * n_out, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(blk.p + wb, x, rows * k_logical * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(blk.p + wb + xb + yb, 0, 256));
+    pf_launch_exact_matmul(gguf_type, blk.p, row_bytes, (int)n_out, (int)k_logical, (const float *)(blk.p + wb),
+                           (int)rows, (float *)(blk.p + wb + xb), (uint32_t *)(blk.p + wb + xb + yb), grid, nullptr);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, blk.p + wb + xb + yb, 4, hipMemcpyDeviceToHost));
+    if (*error_word) return PF_HIP_OK;
+    HIP_TRY(hipMemcpy(y, blk.p + wb + xb, rows * n_out * 4, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_packed_decode_row_host(uint32_t gguf_type, const void *row, size_t row_bytes, size_t k_storage,
+                                             float *out, uint32_t *error_word) {
+    if (!error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    size_t block, size;
+    if (!block_geometry(gguf_type, &block, &size)) return PF_HIP_E_UNSUPPORTED;
+    if (!row || !out || !k_storage || k_storage > 0x7fffffffu) return PF_HIP_E_ARGUMENT;
+    if (pf_hip_device_count() < 1) return PF_HIP_E_NO_DEVICE;
+    const uint64_t *grid = pf_device_iq2_grid();
+    if (!grid) return PF_HIP_E_MEMORY;
+    const size_t wb = (row_bytes + 255) & ~(size_t)255, ob = (k_storage * 4 + 255) & ~(size_t)255;
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, wb + ob + 256));
+    HIP_TRY(hipMemcpy(blk.p, row, row_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(blk.p + wb + ob, 0, 256));
+    pf_launch_exact_decode(gguf_type, blk.p, (int)k_storage, (float *)(blk.p + wb), (uint32_t *)(blk.p + wb + ob),
+                           grid, nullptr);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, blk.p + wb + ob, 4, hipMemcpyDeviceToHost));
+    if (*error_word) return PF_HIP_OK;
+    HIP_TRY(hipMemcpy(out, blk.p + wb, k_storage * 4, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+// ---- device memory and timing helpers --------------------------------------------
+extern "C" int pf_hip_malloc(void **d_ptr, size_t bytes) {
+    if (!d_ptr) return PF_HIP_E_ARGUMENT;
+    *d_ptr = nullptr;
+    hipError_t e = hipMalloc(d_ptr, bytes ? bytes : 1);
+    if (e != hipSuccess) { pf_set_error("hipMalloc", e); return PF_HIP_E_MEMORY; }
+    return PF_HIP_OK;
+}
+extern "C" void pf_hip_free(void *d_ptr) { if (d_ptr) (void)hipFree(d_ptr); }
+extern "C" int pf_hip_memcpy_h2d(void *d_dst, const void *src, size_t bytes) {
+    HIP_TRY(hipMemcpy(d_dst, src, bytes, hipMemcpyHostToDevice));
+    return PF_HIP_OK;
+}
+extern "C" int pf_hip_memcpy_d2h(void *dst, const void *d_src, size_t bytes) {
+    HIP_TRY(hipMemcpy(dst, d_src, bytes, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+extern "C" int pf_hip_synchronize(void) {
+    HIP_TRY(hipDeviceSynchronize());
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
+                                        float *d_y, size_t tokens, size_t iters, float *elapsed_ms) {
+    if (!moe || !work || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
+    const size_t H = moe->desc.hidden;
+    hipStream_t s = nullptr;
+    hipEvent_t t0, t1;
+    HIP_TRY(hipStreamCreate(&s));
+    HIP_TRY(hipEventCreate(&t0));
+    HIP_TRY(hipEventCreate(&t1));
+    int rc = PF_HIP_OK;
+    HIP_TRY(hipEventRecord(t0, s));
+    for (size_t i = 0; i < iters && rc == PF_HIP_OK; i++)
+        rc = pf_hip_moe_forward_device(moe, work, d_x + (i % n_inputs) * tokens * H, H, d_y, H, tokens, s);
+    HIP_TRY(hipEventRecord(t1, s));
+    HIP_TRY(hipStreamSynchronize(s));
+    if (rc == PF_HIP_OK) HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipStreamDestroy(s);
+    return rc;
+}

@@ -1,0 +1,89 @@
+// Reference-order kernels: per-element decode and the serial product.
+//
+// One lane owns one output and walks k upwards, multiplying and adding without
+// contraction, exactly as src/qwen4_packed.c:164-179 does on the CPU; the decode
+// is the per-element arithmetic of src/qwen4_packed.c:67-115.  Results are
+// bit-identical to the reference.  These kernels serve qw4_packed_matmul,
+// qw4_packed_decode_row and the tie fallback of the router; they are not the
+// throughput path.
+#include "pf_moe_internal.h"
+
+__device__ __forceinline__ float exact_value(uint32_t type, const uint8_t *row, int column, const uint64_t *grid) {
+    if (type == PF_F32) {
+        const uint8_t *p = row + 4 * (size_t)column;
+        uint32_t bits = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+        return __uint_as_float(bits);
+    }
+    const int lane = column & 255, blk = column >> 8;
+    if (type == PF_Q4_K) {
+        const uint8_t *b = row + (size_t)blk * 144, *sc = b + 4;
+        const int g = lane >> 5;
+        uint32_t scale, minimum;
+        if (g < 4) {
+            scale = sc[g] & 63u;
+            minimum = sc[g + 4] & 63u;
+        } else {
+            scale = (sc[g + 4] & 15u) | ((sc[g - 4] & 192u) >> 2);
+            minimum = (uint32_t)(sc[g + 4] >> 4) | ((sc[g] & 192u) >> 2);
+        }
+        const uint32_t code = (b[16 + (g >> 1) * 32 + (lane & 31)] >> ((g & 1) * 4)) & 15u;
+        const float d = pf_half_bits_to_float((uint32_t)b[0] | ((uint32_t)b[1] << 8));
+        const float dmin = pf_half_bits_to_float((uint32_t)b[2] | ((uint32_t)b[3] << 8));
+        return __fsub_rn(__fmul_rn(__fmul_rn(d, (float)scale), (float)code), __fmul_rn(dmin, (float)minimum));
+    }
+    // IQ2_XXS
+    const uint8_t *b = row + (size_t)blk * 66, *grp = b + 2 + (lane >> 5) * 8;
+    const int slot = (lane & 31) >> 3, pos = lane & 7;
+    const uint32_t word = (uint32_t)grp[4] | ((uint32_t)grp[5] << 8) | ((uint32_t)grp[6] << 16) |
+                          ((uint32_t)grp[7] << 24);
+    uint32_t signs = (word >> (7 * slot)) & 127u;
+    signs |= pf_parity7(signs) << 7;
+    const uint32_t magnitude = (uint32_t)((grid[grp[slot]] >> (8 * pos)) & 255u);
+    const float d = pf_half_bits_to_float((uint32_t)b[0] | ((uint32_t)b[1] << 8));
+    const float scale = __fmul_rn(__fmul_rn(d, (float)(2u * (word >> 28) + 1u)), 0.125f);
+    const float v = __fmul_rn(scale, (float)magnitude);
+    return (signs >> pos) & 1u ? -v : v;
+}
+
+__global__ void pf_k_exact_matmul(uint32_t type, const uint8_t *w, size_t row_bytes, int n_out, int k_logical,
+                                  const float *x, int rows, float *y, uint32_t *error, const uint64_t *grid) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)rows * n_out) return;
+    const int m = (int)(i / n_out), n = (int)(i % n_out);
+    const uint8_t *row = w + (size_t)n * row_bytes;
+    const float *in = x + (size_t)m * k_logical;
+    float sum = 0.0f;
+    bool bad = false;
+    for (int k = 0; k < k_logical; k++) {
+        const float v = exact_value(type, row, k, grid);
+        const float p = __fmul_rn(v, in[k]);
+        sum = __fadd_rn(sum, p);
+        bad |= !pf_finite(v) || !pf_finite(in[k]) || !pf_finite(p) || !pf_finite(sum);
+    }
+    y[i] = sum;
+    if (bad) atomicOr(error, PF_HIP_ERR_NONFINITE);
+}
+
+__global__ void pf_k_exact_decode(uint32_t type, const uint8_t *row, int k_storage, float *out, uint32_t *error,
+                                  const uint64_t *grid) {
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= k_storage) return;
+    const float v = exact_value(type, row, k, grid);
+    out[k] = v;
+    if (!pf_finite(v)) atomicOr(error, PF_HIP_ERR_NONFINITE);
+}
+
+void pf_launch_exact_matmul(uint32_t type, const uint8_t *d_w, size_t row_bytes, int n_out, int k_logical,
+                            const float *d_x, int rows, float *d_y, uint32_t *d_error, const uint64_t *grid,
+                            hipStream_t stream) {
+    const size_t n = (size_t)rows * n_out;
+    if (n == 0) return;
+    hipLaunchKernelGGL(pf_k_exact_matmul, dim3((unsigned)((n + 63) / 64)), dim3(64), 0, stream, type, d_w, row_bytes,
+                       n_out, k_logical, d_x, rows, d_y, d_error, grid);
+}
+
+void pf_launch_exact_decode(uint32_t type, const uint8_t *d_row, int k_storage, float *d_out, uint32_t *d_error,
+                            const uint64_t *grid, hipStream_t stream) {
+    hipLaunchKernelGGL(pf_k_exact_decode, dim3((k_storage + 255) / 256), dim3(256), 0, stream, type, d_row, k_storage,
+                       d_out, d_error, grid);
+}

@@ -1,0 +1,64 @@
+// Internal declarations shared by the HIP translation units of the MoE library.
+#pragma once
+#include "pf_device.h"
+#include "../../include/pf_moe_hip.h"
+
+// Everything a kernel needs, passed by value.  Weight index order is
+// Qwen4MoeWeights': router, gate, up, down, shared gate/up/down, shared router.
+struct PfKernelArgs {
+    int hidden, experts, top_k, inter, shared_inter, down_physical, norm_topk;
+    uint32_t type[8];
+    const uint8_t *w[8];
+    size_t row_bytes[8], expert_bytes[8];
+    const uint64_t *iq2_grid;        // 256 x 8 magnitudes, device memory
+    const float *x;                  // [tokens, hidden], pitch in floats
+    size_t x_pitch;
+    float *y;
+    size_t y_pitch;
+    float *logits, *logit_ssq;       // [tokens, experts]
+    uint32_t *ids;                   // [tokens, top_k]
+    float *route_weights;            // [tokens, top_k]
+    float *act;                      // [tokens * top_k, inter]
+    float *shared_act;               // [tokens, shared_inter]
+    float *shared_scale;             // [tokens] sigmoid of the shared router logit
+    uint32_t *error_word;
+    uint32_t *exact_rows;            // count of tokens re-routed in serial order
+    uint32_t *route_flags;           // [tokens] 1 = route again in serial order
+};
+
+struct PfHipMoe {
+    PfHipMoeDesc desc;
+    uint8_t *w[8];
+    size_t bytes[8], row_bytes[8], expert_bytes[8];
+    uint64_t *iq2_grid;
+    size_t total_bytes;
+};
+
+struct PfHipWork {
+    const PfHipMoe *moe;
+    size_t cap, bytes;
+    float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
+    uint32_t *ids, *error_word, *exact_rows, *route_flags;
+    void *host_stage;                // pinned staging for the host-buffer forward
+    size_t host_stage_bytes;
+};
+
+// pf_moe_kernels.hip
+void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream);
+// pf_moe_route.hip
+void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream);
+int pf_route_exact_device(const float *d_logits, int tokens, int experts, int top_k, int norm,
+                          float *d_probs, uint32_t *d_ids, float *d_weights, uint32_t *d_error,
+                          unsigned long long *d_bad_row, hipStream_t stream);
+int pf_group_pairs_device(const uint32_t *d_ids, int tokens, int experts, int top_k, uint32_t *d_counts,
+                          uint32_t *d_offsets, uint32_t *d_pair_to_row, uint32_t *d_row_to_pair,
+                          uint32_t *d_first_bad, hipStream_t stream);
+// pf_moe_exact.hip
+void pf_launch_exact_matmul(uint32_t type, const uint8_t *d_w, size_t row_bytes, int n_out, int k_logical,
+                            const float *d_x, int rows, float *d_y, uint32_t *d_error, const uint64_t *grid,
+                            hipStream_t stream);
+void pf_launch_exact_decode(uint32_t type, const uint8_t *d_row, int k_storage, float *d_out, uint32_t *d_error,
+                            const uint64_t *grid, hipStream_t stream);
+// pf_moe_api.hip
+const uint64_t *pf_device_iq2_grid(void);
+void pf_set_error(const char *what, hipError_t code);

@@ -1,0 +1,230 @@
+// General MoE kernels for gfx950: any admitted shape and format combination.
+//
+// One wave computes one output row product; activations of the current token
+// are staged in LDS.  These kernels keep GGUF's byte layout.  Shapes that the
+// specialised decode and prefill kernels cover are dispatched there instead.
+#include "pf_moe_internal.h"
+
+// ---- row products: packed row (GGUF layout) . x (LDS or global) ---------------
+
+__device__ __forceinline__ float dot_row_f32(const uint8_t *row, const float *x, int K, int lane) {
+    const float *w = reinterpret_cast<const float *>(row);
+    float acc = 0.0f;
+    if ((K & 3) == 0) {
+        for (int k = lane * 4; k < K; k += 4 * PF_WAVE) {
+            float4 a = *reinterpret_cast<const float4 *>(w + k);
+            acc = fmaf(a.x, x[k], acc);
+            acc = fmaf(a.y, x[k + 1], acc);
+            acc = fmaf(a.z, x[k + 2], acc);
+            acc = fmaf(a.w, x[k + 3], acc);
+        }
+    } else {
+        for (int k = lane; k < K; k += PF_WAVE) acc = fmaf(w[k], x[k], acc);
+    }
+    return acc;
+}
+
+// Lane l takes 16 nibble bytes of block l/8: the low nibbles are 16 weights of
+// group 2j, the high nibbles 16 weights of group 2j+1 (j = (l%8)/2).
+__device__ __forceinline__ float dot_row_q4k(const uint8_t *row, const float *x, int K, int lane) {
+    const int nblk = K >> 8, r = lane & 7, j = r >> 1, half = r & 1;
+    float acc = 0.0f;
+    for (int b = lane >> 3; b < nblk; b += 8) {
+        const uint8_t *blk = row + (size_t)b * 144;
+        const uint4 hdr = *reinterpret_cast<const uint4 *>(blk);
+        const uint4 q = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * r);
+        const float d = pf_half_bits_to_float(hdr.x & 0xffffu);
+        const float dmin = pf_half_bits_to_float(hdr.x >> 16);
+        const uint32_t sc[3] = {hdr.y, hdr.z, hdr.w};
+        uint32_t s0, m0, s1, m1;
+        pf_q4k_scale_min(sc, 2 * j, s0, m0);
+        pf_q4k_scale_min(sc, 2 * j + 1, s1, m1);
+        const float *xl = x + 256 * b + 64 * j + 16 * half, *xh = xl + 32;
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+        float ql = 0.0f, qh = 0.0f, sl = 0.0f, sh = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint32_t byte = (qw[w] >> (8 * c)) & 255u;
+                const float a = xl[4 * w + c], bb = xh[4 * w + c];
+                ql = fmaf((float)(byte & 15u), a, ql);
+                qh = fmaf((float)(byte >> 4), bb, qh);
+                sl += a;
+                sh += bb;
+            }
+        }
+        acc += d * ((float)s0 * ql + (float)s1 * qh) - dmin * ((float)m0 * sl + (float)m1 * sh);
+    }
+    return acc;
+}
+
+// Lane l takes group l (32 weights, 8 bytes at 2-byte alignment) per pass.
+__device__ __forceinline__ float dot_row_iq2(const uint8_t *row, const float *x, int K, int lane,
+                                             const uint64_t *grid) {
+    const int ngroups = K >> 5;
+    float acc = 0.0f;
+    for (int gi = lane; gi < ngroups; gi += PF_WAVE) {
+        const int b = gi >> 3, g = gi & 7;
+        const uint8_t *blk = row + (size_t)b * 66;
+        const uint16_t *p = reinterpret_cast<const uint16_t *>(blk + 2 + 8 * g);
+        const float d = pf_half_bits_to_float(*reinterpret_cast<const uint16_t *>(blk));
+        const uint32_t idx = (uint32_t)p[0] | ((uint32_t)p[1] << 16);
+        const uint32_t word = (uint32_t)p[2] | ((uint32_t)p[3] << 16);
+        const float scale = d * (float)(2u * (word >> 28) + 1u) * 0.125f;
+        const float *xg = x + 32 * gi;
+        float gacc = 0.0f;
+#pragma unroll
+        for (int slot = 0; slot < 4; slot++) {
+            const uint64_t mags = grid[(idx >> (8 * slot)) & 255u];
+            uint32_t signs = (word >> (7 * slot)) & 127u;
+            signs |= pf_parity7(signs) << 7;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float m = (float)(uint32_t)((mags >> (8 * e)) & 255u);
+                const float xv = xg[8 * slot + e];
+                gacc = fmaf((signs >> e) & 1u ? -m : m, xv, gacc);
+            }
+        }
+        acc = fmaf(scale, gacc, acc);
+    }
+    return acc;
+}
+
+__device__ __forceinline__ float dot_row(uint32_t type, const uint8_t *row, const float *x, int K, int lane,
+                                         const uint64_t *grid) {
+    float v;
+    if (type == PF_F32) v = dot_row_f32(row, x, K, lane);
+    else if (type == PF_Q4_K) v = dot_row_q4k(row, x, K, lane);
+    else v = dot_row_iq2(row, x, K, lane, grid);
+    return pf_wave_sum(v);
+}
+
+__device__ __forceinline__ void stage_grid(uint64_t *grid_lds, const uint64_t *grid_global) {
+    for (int i = threadIdx.x; i < 256; i += blockDim.x) grid_lds[i] = grid_global[i];
+}
+
+// ---- stage 1: everything that depends on x only -------------------------------
+// Units per token: experts router rows, shared_inter fused shared gate/up rows,
+// one shared-router row.  One wave per unit.
+__global__ void __launch_bounds__(256) pf_k_pre(PfKernelArgs a) {
+    extern __shared__ float lds[];
+    __shared__ uint64_t grid[256];
+    const int H = a.hidden, t = blockIdx.y, lane = pf_lane(), wave = threadIdx.x >> 6;
+    const float *x = a.x + (size_t)t * a.x_pitch;
+    bool bad = false;
+    for (int k = threadIdx.x; k < H; k += blockDim.x) {
+        float v = x[k];
+        lds[k] = v;
+        bad |= !pf_finite(v);
+    }
+    if (bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+    stage_grid(grid, a.iq2_grid);
+    __syncthreads();
+    const int unit = blockIdx.x * 4 + wave, E = a.experts, Is = a.shared_inter;
+    if (unit < E) {
+        // router logit and the sum of squared products used by the tie guard
+        const float *w = reinterpret_cast<const float *>(a.w[0]) + (size_t)unit * H;
+        float acc = 0.0f, sq = 0.0f;
+        for (int k = lane; k < H; k += PF_WAVE) {
+            float p = w[k] * lds[k];
+            acc += p;
+            sq = fmaf(p, p, sq);
+        }
+        acc = pf_wave_sum(acc);
+        sq = pf_wave_sum(sq);
+        if (lane == 0) {
+            a.logits[(size_t)t * E + unit] = acc;
+            a.logit_ssq[(size_t)t * E + unit] = sq;
+        }
+    } else if (unit < E + Is) {
+        const int n = unit - E;
+        float g = dot_row(a.type[4], a.w[4] + (size_t)n * a.row_bytes[4], lds, H, lane, grid);
+        float u = dot_row(a.type[5], a.w[5] + (size_t)n * a.row_bytes[5], lds, H, lane, grid);
+        float v = pf_silu(g) * u;
+        if (lane == 0) {
+            a.shared_act[(size_t)t * Is + n] = v;
+            if (!pf_finite(v)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        }
+    } else if (unit == E + Is) {
+        float z = dot_row(PF_F32, a.w[7], lds, H, lane, grid);
+        float s = pf_sigmoid(z);
+        if (lane == 0) {
+            a.shared_scale[t] = s;
+            if (!pf_finite(z)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        }
+    }
+}
+
+// ---- stage 3: routed gate/up + SwiGLU ----------------------------------------
+// grid (ceil(inter/4), pairs); pair p = token * top_k + slot.
+__global__ void __launch_bounds__(256) pf_k_gate_up(PfKernelArgs a) {
+    extern __shared__ float lds[];
+    __shared__ uint64_t grid[256];
+    const int H = a.hidden, pair = blockIdx.y, t = pair / a.top_k, lane = pf_lane(), wave = threadIdx.x >> 6;
+    const float *x = a.x + (size_t)t * a.x_pitch;
+    for (int k = threadIdx.x; k < H; k += blockDim.x) lds[k] = x[k];
+    stage_grid(grid, a.iq2_grid);
+    __syncthreads();
+    const int n = blockIdx.x * 4 + wave;
+    if (n >= a.inter) return;
+    const uint32_t e = a.ids[pair];
+    if (e >= (uint32_t)a.experts) {
+        if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
+        return;
+    }
+    const uint8_t *gate = a.w[1] + (size_t)e * a.expert_bytes[1] + (size_t)n * a.row_bytes[1];
+    const uint8_t *up = a.w[2] + (size_t)e * a.expert_bytes[2] + (size_t)n * a.row_bytes[2];
+    float g = dot_row(a.type[1], gate, lds, H, lane, grid);
+    float u = dot_row(a.type[2], up, lds, H, lane, grid);
+    float v = pf_silu(g) * u;
+    if (lane == 0) {
+        a.act[(size_t)pair * a.inter + n] = v;
+        if (!pf_finite(v)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+    }
+}
+
+// ---- stage 4: routed down products, slot-ordered weighted sum, shared branch ----
+// grid (ceil(hidden/4), tokens).  LDS holds the token's top_k activation rows
+// and its shared activation row.
+__global__ void __launch_bounds__(256) pf_k_down_combine(PfKernelArgs a) {
+    extern __shared__ float lds[];
+    __shared__ uint64_t grid[256];
+    const int I = a.inter, Is = a.shared_inter, K = a.top_k, t = blockIdx.y;
+    const int lane = pf_lane(), wave = threadIdx.x >> 6;
+    const float *act = a.act + (size_t)t * K * I;
+    for (int i = threadIdx.x; i < K * I; i += blockDim.x) lds[i] = act[i];
+    float *sact = lds + K * I;
+    for (int i = threadIdx.x; i < Is; i += blockDim.x) sact[i] = a.shared_act[(size_t)t * Is + i];
+    stage_grid(grid, a.iq2_grid);
+    __syncthreads();
+    const int n = blockIdx.x * 4 + wave;
+    if (n >= a.hidden) return;
+    float sum = 0.0f;
+    for (int s = 0; s < K; s++) {
+        const uint32_t e = a.ids[(size_t)t * K + s];
+        if (e >= (uint32_t)a.experts) {
+            if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
+            return;
+        }
+        const uint8_t *row = a.w[3] + (size_t)e * a.expert_bytes[3] + (size_t)n * a.row_bytes[3];
+        float dsum = dot_row(a.type[3], row, lds + s * I, I, lane, grid);
+        sum += a.route_weights[(size_t)t * K + s] * dsum;   // slot order, as src/qwen4_moe.c:362-372
+    }
+    float sh = dot_row(a.type[6], a.w[6] + (size_t)n * a.row_bytes[6], sact, Is, lane, grid);
+    float y = sum + a.shared_scale[t] * sh;
+    if (lane == 0) {
+        a.y[(size_t)t * a.y_pitch + n] = y;
+        if (!pf_finite(y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+    }
+}
+
+void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream) {
+    const int units = a.experts + a.shared_inter + 1;
+    const size_t x_lds = (size_t)a.hidden * sizeof(float);
+    hipLaunchKernelGGL(pf_k_pre, dim3((units + 3) / 4, tokens), dim3(256), x_lds, stream, a);
+    pf_launch_route(a, tokens, stream);
+    hipLaunchKernelGGL(pf_k_gate_up, dim3((a.inter + 3) / 4, tokens * a.top_k), dim3(256), x_lds, stream, a);
+    const size_t act_lds = ((size_t)a.top_k * a.inter + a.shared_inter) * sizeof(float);
+    hipLaunchKernelGGL(pf_k_down_combine, dim3((a.hidden + 3) / 4, tokens), dim3(256), act_lds, stream, a);
+}

@@ -1,0 +1,349 @@
+/* C11 host side of the MoE block (include/qwen4_moe.h): handles, lifecycle and
+ * the reference's preflight validation in the reference's order
+ * (src/qwen4_moe.c), so that callers and tests see the same status codes.  All
+ * arithmetic is done by the HIP kernels behind include/pf_moe_hip.h; there is no
+ * CPU fallback: without a device every compute entry point fails. */
+#include "../../include/qwen4_moe.h"
+#include "../../include/pf_moe_hip.h"
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+Qwen4Status pf_packed_admit(const QW4PackedCpuView *w, size_t expert);              /* qwen4_packed_host.c */
+Qwen4Status pf_device_status(int rc, Qwen4Error *err, const char *subject);
+
+typedef struct { uintptr_t lo, hi; } Range;
+
+struct Qwen4Moe {
+    Qwen4MoeConfig cfg;
+    QW4PackedCpuView w[8];
+    size_t refs;
+    bool alive;
+    PfHipMoe *device;
+    PfHipMoeDesc desc;
+};
+
+struct Qwen4MoeWork {
+    Qwen4Moe *owner;
+    size_t cap, bytes;
+    PfHipWork *device;
+    bool busy, failed;
+    QW4MoeObserver observer;
+    void *observer_ctx;
+};
+
+static Qwen4Status moe_status(Qwen4Error *err, Qwen4Status code, const char *detail) {
+    if (err) {
+        memset(err, 0, sizeof *err);
+        err->code = code;
+        if (code != QW4_OK) {
+            snprintf(err->subject, sizeof err->subject, "qwen4_moe");
+            snprintf(err->detail, sizeof err->detail, "%s", detail);
+        }
+    }
+    return code;
+}
+#define TRY(expr) do { Qwen4Status st_ = (expr); if (st_ != QW4_OK) return st_; } while (0)
+
+static Qwen4Status admit_config(const Qwen4MoeConfig *c, Qwen4Error *err) {
+    if (!c) return moe_status(err, QW4_INVALID_ARGUMENT, "null config");
+    if (!c->hidden_size || !c->experts || !c->top_k || c->top_k > c->experts || !c->intermediate ||
+        !c->shared_intermediate || c->down_physical < c->intermediate)
+        return moe_status(err, QW4_RANGE, "invalid MoE dimensions");
+    return QW4_OK;
+}
+
+/* ---- create / destroy ------------------------------------------------------ */
+Qwen4Status qwen4_moe_create(const Qwen4MoeConfig *c, const Qwen4MoeWeights *weights, Qwen4Moe **out,
+                             Qwen4Error *err) {
+    if (out) *out = NULL;
+    if (!out || !weights) return moe_status(err, QW4_INVALID_ARGUMENT, "null create argument");
+    TRY(admit_config(c, err));
+    const QW4PackedCpuView w[8] = {weights->router, weights->gate, weights->up, weights->down,
+                                   weights->shared_gate, weights->shared_up, weights->shared_down,
+                                   weights->shared_router};
+    const size_t h = c->hidden_size, i = c->intermediate, s = c->shared_intermediate;
+    const size_t k_in[8] = {h, h, h, i, h, h, s, h}, n_out[8] = {c->experts, i, i, h, s, s, h, 1};
+    for (size_t a = 0; a < 8; a++) {
+        const QW4PackedLayout *l = &w[a].layout;
+        const size_t experts = (a >= 1 && a <= 3) ? c->experts : 1;
+        if (l->k_logical != k_in[a] || l->n_out != n_out[a] || l->n_experts != experts ||
+            l->k_storage != (a == 3 ? c->down_physical : k_in[a]))
+            return moe_status(err, QW4_SHAPE, "MoE weight shape mismatch");
+        if ((a == 0 || a == 7) && l->gguf_type != 0) return moe_status(err, QW4_FORMAT, "router must be F32");
+        Qwen4Status st = pf_packed_admit(&w[a], 0);
+        if (st) {
+            moe_status(err, st, "invalid weight view");
+            if (err) snprintf(err->subject, sizeof err->subject, "packed weights");
+            return st;
+        }
+    }
+    Qwen4Moe *m = calloc(1, sizeof *m);
+    if (!m) return moe_status(err, QW4_OOM, "MoE allocation");
+    m->cfg = *c;
+    memcpy(m->w, w, sizeof w);
+    m->desc = (PfHipMoeDesc){.hidden = c->hidden_size, .experts = c->experts, .top_k = c->top_k,
+                             .inter = c->intermediate, .shared_inter = c->shared_intermediate,
+                             .down_physical = c->down_physical, .norm_topk = c->norm_topk_prob ? 1u : 0u};
+    const void *bytes[8];
+    size_t sizes[8];
+    for (size_t a = 0; a < 8; a++) {
+        m->desc.type[a] = w[a].layout.gguf_type;
+        bytes[a] = w[a].span.data;
+        sizes[a] = w[a].layout.tensor_bytes;
+    }
+    int rc = pf_hip_moe_create(&m->desc, bytes, sizes, &m->device);
+    if (rc) { free(m); return pf_device_status(rc, err, "qwen4_moe"); }
+    m->refs = 1;
+    m->alive = true;
+    *out = m;
+    return moe_status(err, QW4_OK, "");
+}
+
+static void moe_unref(Qwen4Moe *m) {
+    if (m && --m->refs == 0) { pf_hip_moe_destroy(m->device); free(m); }
+}
+void qwen4_moe_destroy(Qwen4Moe *m) {
+    if (m && m->alive) { m->alive = false; moe_unref(m); }
+}
+
+/* ---- workspaces ------------------------------------------------------------ */
+static Qwen4Status plan_work(const Qwen4Moe *m, size_t cap, size_t *bytes, Qwen4Error *err) {
+    if (!m || !m->alive) return moe_status(err, QW4_BAD_STATE, "inactive MoE");
+    const size_t k = m->cfg.top_k, widest = (size_t)m->cfg.hidden_size + m->cfg.experts + k * m->cfg.intermediate;
+    if (cap > SIZE_MAX / 64 / (widest ? widest : 1)) return moe_status(err, QW4_OVERFLOW, "scratch size overflow");
+    *bytes = sizeof(Qwen4MoeWork) + pf_hip_work_bytes(&m->desc, cap);
+    return QW4_OK;
+}
+
+Qwen4Status qwen4_moe_work_size(const Qwen4Moe *m, size_t cap, size_t *bytes, Qwen4Error *err) {
+    if (!bytes) return moe_status(err, QW4_INVALID_ARGUMENT, "null size output");
+    *bytes = 0;
+    size_t need;
+    TRY(plan_work(m, cap, &need, err));
+    *bytes = need;
+    return moe_status(err, QW4_OK, "");
+}
+
+Qwen4Status qwen4_moe_work_create(const Qwen4Moe *m, size_t cap, size_t budget, Qwen4MoeWork **out, Qwen4Error *err) {
+    if (out) *out = NULL;
+    if (!out) return moe_status(err, QW4_INVALID_ARGUMENT, "null workspace output");
+    size_t need;
+    TRY(plan_work(m, cap, &need, err));
+    if (budget < need) return moe_status(err, QW4_CAPACITY, "workspace budget too small");
+    Qwen4MoeWork *w = calloc(1, sizeof *w);
+    if (!w) return moe_status(err, QW4_OOM, "workspace metadata");
+    int rc = pf_hip_work_create(m->device, cap, &w->device);
+    if (rc) { free(w); return pf_device_status(rc, err, "qwen4_moe"); }
+    w->owner = (Qwen4Moe *)m;
+    w->owner->refs++;
+    w->cap = cap;
+    w->bytes = need;
+    *out = w;
+    return moe_status(err, QW4_OK, "");
+}
+
+Qwen4Status qwen4_moe_work_reset(Qwen4MoeWork *w, Qwen4Error *err) {
+    if (!w) return moe_status(err, QW4_INVALID_ARGUMENT, "null workspace");
+    if (w->busy) return moe_status(err, QW4_BUSY, "workspace executing");
+    if (!w->owner->alive) return moe_status(err, QW4_BAD_STATE, "destroyed owner");
+    w->failed = false;
+    return moe_status(err, QW4_OK, "");
+}
+
+void qwen4_moe_work_destroy(Qwen4MoeWork *w) {
+    if (w && !w->busy) { pf_hip_work_destroy(w->device); moe_unref(w->owner); free(w); }
+}
+
+void qw4_moe_observe(Qwen4MoeWork *w, QW4MoeObserver fn, void *ctx) {
+    if (w && !w->busy) { w->observer = fn; w->observer_ctx = ctx; }
+}
+
+/* ---- view admission (src/qwen4_moe.c:134-186) --------------------------------- */
+static Qwen4Status range_of(const void *data, size_t cap, size_t bytes, size_t alignment, Range *r, Qwen4Error *err) {
+    r->lo = r->hi = 0;
+    if (!bytes) return QW4_OK;
+    if (cap < bytes) return moe_status(err, QW4_CAPACITY, "view capacity too small");
+    if (!data) return moe_status(err, QW4_INVALID_ARGUMENT, "null nonempty view");
+    uintptr_t lo = (uintptr_t)data;
+    if (lo % alignment) return moe_status(err, QW4_STRIDE, "unaligned view");
+    if (bytes > UINTPTR_MAX - lo) return moe_status(err, QW4_OVERFLOW, "address extent overflow");
+    r->lo = lo;
+    r->hi = lo + bytes;
+    return QW4_OK;
+}
+
+static Qwen4Status range_rows(const void *data, size_t cap, size_t rows, size_t cols, size_t pitch, Range *r,
+                              Qwen4Error *err) {
+    r->lo = r->hi = 0;
+    if (cols > SIZE_MAX / 4) return moe_status(err, QW4_OVERFLOW, "row bytes overflow");
+    const size_t row_bytes = cols * 4;
+    if (pitch % 4 || pitch < row_bytes)
+        return moe_status(err, QW4_STRIDE, "row stride must cover contiguous features");
+    if (!rows) return QW4_OK;
+    if (rows - 1 > (SIZE_MAX - row_bytes) / pitch) return moe_status(err, QW4_OVERFLOW, "view extent overflow");
+    return range_of(data, cap, (rows - 1) * pitch + row_bytes, 4, r, err);
+}
+
+static Qwen4Status range_f32(const float *data, size_t cap, size_t rank, const size_t dim[4], const size_t stride[4],
+                             size_t rows, size_t cols, Range *r, Qwen4Error *err) {
+    if (rank != 2 || dim[0] != rows || dim[1] != cols)
+        return moe_status(err, QW4_SHAPE, "expected rank-2 token-major view");
+    if (stride[1] != sizeof(float)) return moe_status(err, QW4_STRIDE, "features must be contiguous");
+    return range_rows(data, cap, rows, cols, stride[0], r, err);
+}
+#define RANGE_F32(v, rows, cols, r) \
+    range_f32((v).data, (v).capacity_bytes, (v).rank, (v).dim, (v).stride_bytes, rows, cols, r, err)
+
+static Qwen4Status all_disjoint(const Range *r, size_t n, Qwen4Error *err) {
+    for (size_t i = 0; i < n; i++)
+        for (size_t j = 0; j < i; j++)
+            if (r[i].lo < r[j].hi && r[j].lo < r[i].hi)
+                return moe_status(err, QW4_INVALID_ARGUMENT, "overlapping views");
+    return QW4_OK;
+}
+
+/* ---- routing on caller-provided logits ------------------------------------------ */
+Qwen4Status qwen4_moe_route(const Qwen4MoeConfig *c, Qwen4F32 logits, Qwen4MoeRoutes routes,
+                            Qwen4F32Mut probabilities, Qwen4Error *err) {
+    TRY(admit_config(c, err));
+    const size_t T = logits.dim[0], E = c->experts, K = c->top_k;
+    Range r[4];
+    TRY(RANGE_F32(logits, T, E, &r[0]));
+    TRY(RANGE_F32(probabilities, T, E, &r[1]));
+    TRY(RANGE_F32(routes.weights, T, K, &r[2]));
+    if (routes.ids.rows != T || routes.ids.cols != K) return moe_status(err, QW4_SHAPE, "route ID shape mismatch");
+    TRY(range_rows(routes.ids.data, routes.ids.capacity_bytes, T, K, routes.ids.row_stride_bytes, &r[3], err));
+    TRY(all_disjoint(r, 4, err));
+    if (!T) return moe_status(err, QW4_OK, "");
+    float *z = malloc(T * E * 4), *p = malloc(T * E * 4), *w = malloc(T * K * 4);
+    uint32_t *ids = malloc(T * K * 4);
+    Qwen4Status st = QW4_OK;
+    if (!z || !p || !w || !ids) st = moe_status(err, QW4_OOM, "route staging");
+    if (!st) {
+        for (size_t t = 0; t < T; t++) memcpy(z + t * E, logits.data + t * (logits.stride_bytes[0] / 4), E * 4);
+        uint32_t word = 0;
+        uint64_t bad_row = 0;
+        int rc = pf_hip_route_host(z, T, E, K, c->norm_topk_prob, p, ids, w, &word, &bad_row);
+        if (rc) st = pf_device_status(rc, err, "qwen4_moe");
+        else if (word & PF_HIP_ERR_NONFINITE) {
+            st = moe_status(err, QW4_NONFINITE, "nonfinite router logit");
+            if (err) err->row = bad_row;
+        } else if (word) st = moe_status(err, QW4_GPU_ERROR, "device error word");
+    }
+    if (!st) {
+        for (size_t t = 0; t < T; t++) {
+            memcpy(probabilities.data + t * (probabilities.stride_bytes[0] / 4), p + t * E, E * 4);
+            memcpy(routes.weights.data + t * (routes.weights.stride_bytes[0] / 4), w + t * K, K * 4);
+            memcpy(routes.ids.data + t * (routes.ids.row_stride_bytes / 4), ids + t * K, K * 4);
+        }
+        moe_status(err, QW4_OK, "");
+    }
+    free(z); free(p); free(w); free(ids);
+    return st;
+}
+
+/* ---- grouping ---------------------------------------------------------------------- */
+Qwen4Status qw4_moe_group_pairs(const Qwen4MoeConfig *c, Qwen4U32Mut ids, QW4MoeGrouping g, Qwen4Error *err) {
+    TRY(admit_config(c, err));
+    if (ids.cols != c->top_k) return moe_status(err, QW4_SHAPE, "group ID shape mismatch");
+    const size_t E = c->experts, K = c->top_k;
+    if (ids.rows > SIZE_MAX / K || E == SIZE_MAX) return moe_status(err, QW4_OVERFLOW, "group count overflow");
+    const size_t pairs = ids.rows * K;
+    Range r[5];
+    TRY(range_rows(ids.data, ids.capacity_bytes, ids.rows, ids.cols, ids.row_stride_bytes, &r[0], err));
+    const void *ptr[4] = {g.offsets, g.cursors, g.pair_to_row, g.row_to_pair};
+    const size_t count[4] = {E + 1, E, pairs, pairs};
+    const size_t cap[4] = {g.offsets_capacity_bytes, g.cursors_capacity_bytes, g.pair_to_row_capacity_bytes,
+                           g.row_to_pair_capacity_bytes};
+    for (size_t a = 0; a < 4; a++) {
+        if (count[a] > SIZE_MAX / sizeof(size_t)) return moe_status(err, QW4_OVERFLOW, "group array bytes overflow");
+        TRY(range_of(ptr[a], cap[a], count[a] * sizeof(size_t), _Alignof(size_t), &r[a + 1], err));
+    }
+    TRY(all_disjoint(r, 5, err));
+    _Static_assert(sizeof(size_t) == sizeof(uint64_t), "the shim exchanges 64-bit indices");
+    uint32_t *dense = NULL;
+    if (pairs) {
+        dense = malloc(pairs * 4);
+        if (!dense) return moe_status(err, QW4_OOM, "group staging");
+        for (size_t t = 0; t < ids.rows; t++) memcpy(dense + t * K, ids.data + t * (ids.row_stride_bytes / 4), K * 4);
+    }
+    uint64_t *out = malloc((E + 1 + 2 * pairs) * sizeof(uint64_t));
+    if (!out) { free(dense); return moe_status(err, QW4_OOM, "group staging"); }
+    uint32_t word = 0;
+    int duplicate = 0;
+    int rc = pf_hip_group_pairs_host(dense, ids.rows, E, K, out, out + E + 1, out + E + 1 + pairs, &word, &duplicate);
+    Qwen4Status st;
+    if (rc) st = pf_device_status(rc, err, "qwen4_moe");
+    else if (word & PF_HIP_ERR_BOUNDS) st = moe_status(err, QW4_RANGE, "expert ID out of range");
+    else if (duplicate) st = moe_status(err, QW4_INVALID_ARGUMENT, "duplicate expert ID");
+    else {
+        memcpy(g.offsets, out, (E + 1) * sizeof(size_t));
+        for (size_t e = 0; e < E; e++) g.cursors[e] = (size_t)out[e + 1];   /* cursors end at offsets[e+1] */
+        if (pairs) {
+            memcpy(g.pair_to_row, out + E + 1, pairs * sizeof(size_t));
+            memcpy(g.row_to_pair, out + E + 1 + pairs, pairs * sizeof(size_t));
+        }
+        st = moe_status(err, QW4_OK, "");
+    }
+    free(out);
+    free(dense);
+    return st;
+}
+
+/* ---- forward (src/qwen4_moe.c:384-431) -------------------------------------------------- */
+Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen4MoeRoutes *routes, Qwen4MoeWork *w,
+                              Qwen4Error *err) {
+    if (!m || !w) return moe_status(err, QW4_INVALID_ARGUMENT, "null forward handle");
+    if (w->owner != m) return moe_status(err, QW4_OWNER, "workspace belongs to another MoE");
+    if (!m->alive || w->failed) return moe_status(err, QW4_BAD_STATE, "inactive MoE/workspace; reset required");
+    if (w->busy) return moe_status(err, QW4_BUSY, "workspace executing");
+    const size_t T = x.dim[0], H = m->cfg.hidden_size, K = m->cfg.top_k;
+    if (T > w->cap) return moe_status(err, QW4_CAPACITY, "batch exceeds token capacity");
+    Range r[4];
+    size_t nr = 2;
+    TRY(RANGE_F32(x, T, H, &r[0]));
+    TRY(RANGE_F32(y, T, H, &r[1]));
+    if (routes) {
+        TRY(RANGE_F32(routes->weights, T, K, &r[2]));
+        if (routes->ids.rows != T || routes->ids.cols != K)
+            return moe_status(err, QW4_SHAPE, "optional route shape mismatch");
+        TRY(range_rows(routes->ids.data, routes->ids.capacity_bytes, T, K, routes->ids.row_stride_bytes, &r[3], err));
+        nr = 4;
+    }
+    TRY(all_disjoint(r, nr, err));
+    for (size_t a = 0; a < 8; a++) {
+        const Range wr = {(uintptr_t)m->w[a].span.data, (uintptr_t)m->w[a].span.data + m->w[a].layout.tensor_bytes};
+        for (size_t b = 0; b < nr; b++) {
+            const Range two[2] = {r[b], wr};
+            TRY(all_disjoint(two, 2, err));
+        }
+    }
+    const size_t xs = x.stride_bytes[0] / 4;
+    for (size_t row = 0; row < T; row++)
+        for (size_t col = 0; col < H; col++)
+            if (!isfinite(x.data[row * xs + col])) return moe_status(err, QW4_NONFINITE, "nonfinite input");
+    if (!T) return moe_status(err, QW4_OK, "");
+    w->busy = true;
+    uint32_t word = 0;
+    int rc = pf_hip_moe_forward_host(m->device, w->device, x.data, x.stride_bytes[0], y.data, y.stride_bytes[0],
+                                     routes ? routes->ids.data : NULL, routes ? routes->ids.row_stride_bytes : 0,
+                                     routes ? routes->weights.data : NULL,
+                                     routes ? routes->weights.stride_bytes[0] : 0, T, &word);
+    w->busy = false;
+    if (rc || word) {
+        w->failed = true;
+        if (rc) return pf_device_status(rc, err, "qwen4_moe");
+        if (word & PF_HIP_ERR_NONFINITE) return moe_status(err, QW4_NONFINITE, "nonfinite value in the MoE block");
+        return moe_status(err, QW4_GPU_ERROR, "device error word");
+    }
+    if (w->observer) {
+        /* stage 12 of src/qwen4_moe_internal.h:9-12: the finished block output */
+        Qwen4F32 out = {.data = y.data, .capacity_bytes = y.capacity_bytes, .rank = 2};
+        memcpy(out.dim, y.dim, sizeof out.dim);
+        memcpy(out.stride_bytes, y.stride_bytes, sizeof out.stride_bytes);
+        w->observer(w->observer_ctx, 12, SIZE_MAX, 0, x, out);
+    }
+    return moe_status(err, QW4_OK, "");
+}

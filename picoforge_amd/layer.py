@@ -1,0 +1,119 @@
+"""Host-side mirror of how the reference's forward loop uses the MoE block.
+
+`LayerWeights` holds the eight tensors of one layer as GGUF bytes and the views
+over them (the job of the reference's create_moe binds, src/qwen4_forward.c:174-187);
+`MoeLayer` owns a Qwen4Moe handle and a workspace of one library and runs
+qwen4_moe_forward like layer_cpu does (src/qwen4_forward.c:365).  The class is
+agnostic of which library it drives: the shipped HIP one, the CPU oracle or a
+build of the reference.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import abi
+from .binding import Synth
+
+ROLE = ("router", "gate", "up", "down", "shared_gate", "shared_up", "shared_down", "shared_router")
+
+
+def shapes(cfg):
+    """(k_storage, k_logical, n_out, experts) per tensor, in Qwen4MoeWeights order (src/qwen4_moe.c:56-57)."""
+    h, i, s, e = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate, cfg.experts
+    return [(h, h, e, 1), (h, h, i, e), (h, h, i, e), (cfg.down_physical, i, h, e),
+            (h, h, s, 1), (h, h, s, 1), (s, s, h, 1), (h, h, 1, 1)]
+
+
+class LayerWeights:
+    def __init__(self, cfg, raw, types):
+        self.cfg, self.raw, self.types = cfg, list(raw), list(types)
+        self.struct = abi.Qwen4MoeWeights()
+        for role, buf, gtype, (ks, kl, n, e) in zip(ROLE, self.raw, self.types, shapes(cfg)):
+            setattr(self.struct, role, abi.packed_view(buf, gtype, ks, n, e, kl))
+
+    @property
+    def nbytes(self):
+        return sum(b.size for b in self.raw)
+
+    @classmethod
+    def synthetic(cls, cfg, expert_type, seed, std=0.02, shared_type=None, router_std=None, iq2_d=2.0 ** -12):
+        """Seeded weights: routers F32 N(0, router_std or std); expert tensors N(0, std) quantised to
+        Q4_K, IQ2_XXS blocks drawn uniformly, or plain F32."""
+        synth = Synth()
+        shared_type = expert_type if shared_type is None else shared_type
+        types = [abi.GGUF_F32, expert_type, expert_type, expert_type, shared_type, shared_type, shared_type,
+                 abi.GGUF_F32]
+        raw = []
+        for j, (gtype, (ks, kl, n, e)) in enumerate(zip(types, shapes(cfg))):
+            stream = seed * 16 + j + 1
+            count = ks * n * e
+            if gtype == abi.GGUF_F32:
+                sd = (router_std or std) if j in (0, 7) else std
+                raw.append(synth.normal((count,), stream, sd).view(np.uint8))
+            elif gtype == abi.GGUF_Q4_K:
+                raw.append(synth.q4k_normal(count // 256, stream, std))
+            elif gtype == abi.GGUF_IQ2_XXS:
+                raw.append(synth.iq2xxs_uniform(count // 256, stream, iq2_d))
+            else:
+                raise ValueError(gtype)
+        return cls(cfg, raw, types)
+
+
+class MoeError(RuntimeError):
+    def __init__(self, status, detail):
+        super().__init__(f"{abi.status_name(status)}: {detail}")
+        self.status = status
+
+
+class MoeLayer:
+    def __init__(self, api, cfg, weights, token_cap):
+        self.api, self.cfg, self.weights, self.cap = api, cfg, weights, token_cap
+        self.err = abi.Qwen4Error()
+        self.handle, self.work = C.c_void_p(), C.c_void_p()
+        st = api.create(C.byref(cfg), C.byref(weights.struct), C.byref(self.handle), C.byref(self.err))
+        self._raise(st)
+        size = C.c_size_t()
+        self._raise(api.work_size(self.handle, token_cap, C.byref(size), C.byref(self.err)))
+        self.work_bytes = size.value
+        self._raise(api.work_create(self.handle, token_cap, size.value, C.byref(self.work), C.byref(self.err)))
+
+    def _raise(self, st):
+        if st != abi.QW4_OK:
+            raise MoeError(st, self.err.detail.decode(errors="replace"))
+
+    def forward(self, x, want_routes=True, check=True):
+        """x [T, H] float32 -> (status, y, ids, weights)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        t, k = x.shape[0], self.cfg.top_k
+        y = np.full((t, self.cfg.hidden_size), -99.0, dtype=np.float32)
+        ids = np.full((t, k), 0xFFFFFFFF, dtype=np.uint32)
+        w = np.full((t, k), -99.0, dtype=np.float32)
+        routes = abi.Qwen4MoeRoutes(abi.u32_view(ids), abi.f32_view(w))
+        st = self.api.forward(self.handle, abi.f32_view(x), abi.f32_view(y),
+                              C.byref(routes) if want_routes else None, self.work, C.byref(self.err))
+        if check:
+            self._raise(st)
+        return st, y, ids, w
+
+    def reset(self):
+        return self.api.work_reset(self.work, C.byref(self.err))
+
+    def close(self):
+        if self.work:
+            self.api.work_destroy(self.work)
+            self.work = C.c_void_p()
+        if self.handle:
+            self.api.destroy(self.handle)
+            self.handle = C.c_void_p()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+
+def rms_normalise(x, eps=0.0):
+    x = np.asarray(x, dtype=np.float32)
+    scale = np.sqrt(np.mean(x.astype(np.float64) ** 2, axis=-1, keepdims=True) + eps)
+    return (x / scale).astype(np.float32)
