@@ -36,7 +36,7 @@ const uint64_t *pf_device_iq2_grid(void) {
     }
     uint64_t *d = nullptr;
     if (hipMalloc(&d, sizeof host) != hipSuccess) return nullptr;
-    if (hipMemcpy(d, host, sizeof host, hipMemcpyHostToDevice) != hipSuccess) { hipFree(d); return nullptr; }
+    if (hipMemcpy(d, host, sizeof host, hipMemcpyHostToDevice) != hipSuccess) { (void)hipFree(d); return nullptr; }
     g_grid = d;
     return g_grid;
 }

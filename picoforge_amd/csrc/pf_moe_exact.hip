@@ -7,6 +7,14 @@
 // qw4_packed_decode_row and the tie fallback of the router; they are not the
 // throughput path.
 #include "pf_moe_internal.h"
+// Reference-order arithmetic: a*b+c must stay two roundings.  HIP's __fmul_rn and
+// __fadd_rn are plain operators compiled with contraction allowed, so they fuse
+// after inlining; the helpers below are compiled with contraction off instead.
+#pragma clang fp contract(off)
+static __device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
+static __device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
+static __device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
+static __device__ __forceinline__ float div_rn(float a, float b) { return a / b; }
 
 __device__ __forceinline__ float exact_value(uint32_t type, const uint8_t *row, int column, const uint64_t *grid) {
     if (type == PF_F32) {
@@ -29,7 +37,7 @@ __device__ __forceinline__ float exact_value(uint32_t type, const uint8_t *row, 
         const uint32_t code = (b[16 + (g >> 1) * 32 + (lane & 31)] >> ((g & 1) * 4)) & 15u;
         const float d = pf_half_bits_to_float((uint32_t)b[0] | ((uint32_t)b[1] << 8));
         const float dmin = pf_half_bits_to_float((uint32_t)b[2] | ((uint32_t)b[3] << 8));
-        return __fsub_rn(__fmul_rn(__fmul_rn(d, (float)scale), (float)code), __fmul_rn(dmin, (float)minimum));
+        return sub_rn(mul_rn(mul_rn(d, (float)scale), (float)code), mul_rn(dmin, (float)minimum));
     }
     // IQ2_XXS
     const uint8_t *b = row + (size_t)blk * 66, *grp = b + 2 + (lane >> 5) * 8;
@@ -40,8 +48,8 @@ __device__ __forceinline__ float exact_value(uint32_t type, const uint8_t *row, 
     signs |= pf_parity7(signs) << 7;
     const uint32_t magnitude = (uint32_t)((grid[grp[slot]] >> (8 * pos)) & 255u);
     const float d = pf_half_bits_to_float((uint32_t)b[0] | ((uint32_t)b[1] << 8));
-    const float scale = __fmul_rn(__fmul_rn(d, (float)(2u * (word >> 28) + 1u)), 0.125f);
-    const float v = __fmul_rn(scale, (float)magnitude);
+    const float scale = mul_rn(mul_rn(d, (float)(2u * (word >> 28) + 1u)), 0.125f);
+    const float v = mul_rn(scale, (float)magnitude);
     return (signs >> pos) & 1u ? -v : v;
 }
 
@@ -56,8 +64,8 @@ __global__ void pf_k_exact_matmul(uint32_t type, const uint8_t *w, size_t row_by
     bool bad = false;
     for (int k = 0; k < k_logical; k++) {
         const float v = exact_value(type, row, k, grid);
-        const float p = __fmul_rn(v, in[k]);
-        sum = __fadd_rn(sum, p);
+        const float p = mul_rn(v, in[k]);
+        sum = add_rn(sum, p);
         bad |= !pf_finite(v) || !pf_finite(in[k]) || !pf_finite(p) || !pf_finite(sum);
     }
     y[i] = sum;

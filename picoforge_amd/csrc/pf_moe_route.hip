@@ -7,6 +7,14 @@
 // exact path, which recomputes its logits in the reference's serial order
 // (src/qwen4_packed.c:164-179) and follows src/qwen4_moe.c:219-247 step by step.
 #include "pf_moe_internal.h"
+// Reference-order arithmetic: a*b+c must stay two roundings.  HIP's __fmul_rn and
+// __fadd_rn are plain operators compiled with contraction allowed, so they fuse
+// after inlining; the helpers below are compiled with contraction off instead.
+#pragma clang fp contract(off)
+static __device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
+static __device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
+static __device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
+static __device__ __forceinline__ float div_rn(float a, float b) { return a / b; }
 #include <math.h>
 
 #define ROUTE_MAX_FAST_EXPERTS 1024
@@ -35,13 +43,13 @@ __device__ void route_exact_wave(const float *z, float *p, float *q, int E, int 
     for (int e = lane; e < E; e += PF_WAVE) top = fmaxf(top, z[e]);
     top = pf_wave_max(top);
     // exponent in double, rounded once: the correctly rounded expf
-    for (int e = lane; e < E; e += PF_WAVE) p[e] = (float)exp((double)__fsub_rn(z[e], top));
+    for (int e = lane; e < E; e += PF_WAVE) p[e] = (float)exp((double)sub_rn(z[e], top));
     wave_lds_fence();
     float sum = 0.0f;
-    for (int e = 0; e < E; e++) sum = __fadd_rn(sum, p[e]);   // serial, expert ascending
+    for (int e = 0; e < E; e++) sum = add_rn(sum, p[e]);   // serial, expert ascending
     wave_lds_fence();
     for (int e = lane; e < E; e += PF_WAVE) {
-        float v = __fdiv_rn(p[e], sum);
+        float v = div_rn(p[e], sum);
         p[e] = v;
         q[e] = v;
     }
@@ -57,11 +65,11 @@ __device__ void route_exact_wave(const float *z, float *p, float *q, int E, int 
         wave_argmax(best, best_id);
         if ((int)(best_id & (PF_WAVE - 1)) == lane) q[best_id] = -1.0f;
         wave_lds_fence();
-        chosen = __fadd_rn(chosen, best);
+        chosen = add_rn(chosen, best);
         if (lane == 0) { ids_out[slot] = best_id; w_out[slot] = best; }
     }
     if (norm && lane == 0)
-        for (int slot = 0; slot < K; slot++) w_out[slot] = __fdiv_rn(w_out[slot], chosen);
+        for (int slot = 0; slot < K; slot++) w_out[slot] = div_rn(w_out[slot], chosen);
 }
 
 // ---- fast routing inside a forward --------------------------------------------
@@ -149,7 +157,7 @@ __global__ void __launch_bounds__(256) pf_k_route_fix(PfKernelArgs a) {
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
         const float *w = reinterpret_cast<const float *>(a.w[0]) + (size_t)e * H;
         float sum = 0.0f;
-        for (int k = 0; k < H; k++) sum = __fadd_rn(sum, __fmul_rn(w[k], xs[k]));
+        for (int k = 0; k < H; k++) sum = add_rn(sum, mul_rn(w[k], xs[k]));
         z[e] = sum;
         a.logits[(size_t)t * E + e] = sum;
     }
