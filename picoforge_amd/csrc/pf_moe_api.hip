@@ -264,7 +264,8 @@ extern "C" int pf_hip_route_host(const float *logits, size_t tokens, size_t expe
     if (bad_row) *bad_row = 0;
     if (tokens == 0) return PF_HIP_OK;
     if (!logits || !probs || !ids || !weights || !experts || !top_k || top_k > experts) return PF_HIP_E_ARGUMENT;
-    if (tokens * experts > 0x7fffffffu || pf_hip_device_count() < 1) return PF_HIP_E_UNSUPPORTED;
+    if (tokens * experts > 0x7fffffffu) return PF_HIP_E_UNSUPPORTED;
+    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
     const size_t zb = tokens * experts * 4, kb = tokens * top_k * 4;
     const size_t o_p = (zb + 255) & ~(size_t)255, o_i = o_p * 2, o_w = o_i + ((kb + 255) & ~(size_t)255),
                  o_e = o_w + ((kb + 255) & ~(size_t)255);
@@ -298,7 +299,8 @@ extern "C" int pf_hip_group_pairs_host(const uint32_t *ids, size_t tokens, size_
     *error_word = 0;
     *duplicate = 0;
     const size_t pairs = tokens * top_k;
-    if (pairs > 0x3fffffffu || experts > 0x3fffffffu || pf_hip_device_count() < 1) return PF_HIP_E_UNSUPPORTED;
+    if (pairs > 0x3fffffffu || experts > 0x3fffffffu) return PF_HIP_E_UNSUPPORTED;
+    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
     if (pairs && (!ids || !pair_to_row || !row_to_pair)) return PF_HIP_E_ARGUMENT;
     const size_t pb = ((pairs ? pairs : 1) * 4 + 255) & ~(size_t)255, eb = ((experts + 1) * 4 + 255) & ~(size_t)255;
     // ids | counts | offsets | pair_to_row | row_to_pair | error
@@ -343,7 +345,8 @@ extern "C" int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_
     size_t block, size;
     if (!block_geometry(gguf_type, &block, &size)) return PF_HIP_E_UNSUPPORTED;
     if (!expert_bytes || !x || !y || !n_out || !k_logical) return PF_HIP_E_ARGUMENT;
-    if (rows * n_out > 0x7fffffffu || k_logical > 0x7fffffffu || pf_hip_device_count() < 1) return PF_HIP_E_UNSUPPORTED;
+    if (rows * n_out > 0x7fffffffu || k_logical > 0x7fffffffu) return PF_HIP_E_UNSUPPORTED;
+    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
     const uint64_t *grid = pf_device_iq2_grid();
     if (!grid) return PF_HIP_E_MEMORY;
     const size_t wb = (row_bytes * n_out + 255) & ~(size_t)255, xb = (rows * k_logical * 4 + 255) & ~(size_t)255,
