@@ -126,6 +126,13 @@ int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *
                              size_t n_inputs, float *d_y, size_t tokens, size_t iters,
                              float *elapsed_ms);
 
+/* Same loop, synchronising after every forward and reading events placed between
+ * the four stages of the general path: stage_ms[0] router + shared gate/up,
+ * [1] routing, [2] routed gate/up, [3] down + combine; averages over iters. */
+int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
+                              size_t n_inputs, float *d_y, size_t tokens, size_t iters,
+                              float stage_ms[4]);
+
 #ifdef __cplusplus
 }
 #endif

@@ -223,9 +223,36 @@ extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, c
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(pf_k_clear2, dim3(1), dim3(1), 0, s, work->error_word, work->exact_rows);
     PfKernelArgs a = make_args(moe, work, d_x, x_pitch, d_y, y_pitch);
-    pf_launch_general(a, (int)tokens, s);
+    pf_launch_general(a, (int)tokens, s, (hipEvent_t *)work->marks);
     HIP_TRY(hipGetLastError());
     return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
+                                         float *d_y, size_t tokens, size_t iters, float stage_ms[4]) {
+    if (!moe || !work || !d_x || !d_y || !n_inputs || !stage_ms) return PF_HIP_E_ARGUMENT;
+    const size_t H = moe->desc.hidden;
+    hipStream_t s = nullptr;
+    hipEvent_t marks[5];
+    HIP_TRY(hipStreamCreate(&s));
+    for (int j = 0; j < 5; j++) HIP_TRY(hipEventCreate(&marks[j]));
+    for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
+    int rc = PF_HIP_OK;
+    work->marks = marks;
+    for (size_t i = 0; i < iters && rc == PF_HIP_OK; i++) {
+        rc = pf_hip_moe_forward_device(moe, work, d_x + (i % n_inputs) * tokens * H, H, d_y, H, tokens, s);
+        if (rc == PF_HIP_OK && hipStreamSynchronize(s) != hipSuccess) rc = PF_HIP_E_RUNTIME;
+        for (int j = 0; j < 4 && rc == PF_HIP_OK; j++) {
+            float ms = 0.0f;
+            if (hipEventElapsedTime(&ms, marks[j], marks[j + 1]) != hipSuccess) rc = PF_HIP_E_RUNTIME;
+            stage_ms[j] += ms;
+        }
+    }
+    work->marks = nullptr;
+    for (int j = 0; j < 4; j++) stage_ms[j] /= (float)(iters ? iters : 1);
+    for (int j = 0; j < 5; j++) (void)hipEventDestroy(marks[j]);
+    (void)hipStreamDestroy(s);
+    return rc;
 }
 
 extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,

@@ -41,10 +41,11 @@ struct PfHipWork {
     uint32_t *ids, *error_word, *exact_rows, *route_flags;
     void *host_stage;                // pinned staging for the host-buffer forward
     size_t host_stage_bytes;
+    void *marks;                     // hipEvent_t[5] while stage profiling, else null
 };
 
 // pf_moe_kernels.hip
-void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream);
+void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks);
 // pf_moe_route.hip
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream);
 int pf_route_exact_device(const float *d_logits, int tokens, int experts, int top_k, int norm,
