@@ -78,6 +78,13 @@ const uint32_t *pf_hip_work_error_word(const PfHipWork *work);
  * reference's serial order because two candidate logits were too close. */
 int pf_hip_work_exact_rows(PfHipWork *work, uint32_t *count);
 
+/* The error word and the re-route counter accumulate over forwards (a forward only
+ * enqueues kernels, so it can be captured into a graph); this clears both. */
+int pf_hip_work_clear_status(PfHipWork *work);
+/* Tests: route every batch size through the general kernels (on != 0) instead of the
+ * specialised decode kernels. */
+void pf_hip_work_force_general(PfHipWork *work, int on);
+
 /* Host-buffer forward used by qwen4_moe_forward: copies x in, runs the forward,
  * copies y (and ids/weights when non-NULL) out, returns the error word.  Pitches
  * in bytes.  Outputs are written only when the error word is zero. */

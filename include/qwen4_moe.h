@@ -99,6 +99,13 @@ typedef void (*QW4MoeObserver)(void *ctx, size_t stage, size_t expert, size_t to
                                Qwen4F32 input, Qwen4F32 output);
 void qw4_moe_observe(Qwen4MoeWork *work, QW4MoeObserver observer, void *ctx);
 
+/* Extension without a counterpart in the reference: the device-side handles behind a
+ * layer and a workspace (include/pf_moe_hip.h), for callers that keep activations
+ * resident in HBM and enqueue forwards on their own stream.  Owned by the handles
+ * they come from. */
+struct PfHipMoe *pf_moe_device_layer(const Qwen4Moe *moe);
+struct PfHipWork *pf_moe_device_work(Qwen4MoeWork *work);
+
 #ifdef __cplusplus
 }
 #endif

@@ -62,6 +62,9 @@ class MoeApi:
         self.group_pairs = bind(private_prefix + "group_pairs", C.c_int, P(abi.Qwen4MoeConfig), abi.Qwen4U32Mut,
                                 abi.QW4MoeGrouping, P(E))
         self.observe = bind(private_prefix + "observe", None, vp, abi.OBSERVER, vp)
+        if hasattr(lib, "pf_moe_device_layer"):
+            self.device_layer = bind("pf_moe_device_layer", vp, vp)
+            self.device_work = bind("pf_moe_device_work", vp, vp)
         self.layout_init = bind(packed_prefix + "layout_init", C.c_int, P(abi.GgufTensor), sz,
                                 P(abi.QW4PackedLayout), P(E))
         self.decode_row = bind(packed_prefix + "decode_row", C.c_int, P(abi.QW4PackedCpuView), sz, sz, vp, sz, P(E))
@@ -114,6 +117,8 @@ class HipShim:
         bind("pf_hip_work_logits", vp, vp)
         bind("pf_hip_work_error_word", vp, vp)
         bind("pf_hip_work_exact_rows", C.c_int, vp, u32p)
+        bind("pf_hip_work_clear_status", C.c_int, vp)
+        bind("pf_hip_work_force_general", None, vp, C.c_int)
         bind("pf_hip_moe_forward_host", C.c_int, vp, vp, vp, sz, vp, sz, vp, sz, vp, sz, sz, u32p)
         bind("pf_hip_route_host", C.c_int, vp, sz, sz, sz, C.c_int, vp, vp, vp, u32p, P(C.c_uint64))
         bind("pf_hip_group_pairs_host", C.c_int, vp, sz, sz, sz, vp, vp, vp, u32p, P(C.c_int))

@@ -24,22 +24,55 @@ extern "C" int pf_hip_device_count(void) {
     return n;
 }
 
-// 256 x 8 IQ2_XXS magnitudes, one copy per process (single device per process).
-static uint64_t *g_grid = nullptr;
-const uint64_t *pf_device_iq2_grid(void) {
-    if (g_grid) return g_grid;
-    uint64_t host[256];
-    for (unsigned i = 0; i < 256; i++) {
-        uint64_t v = 0;
-        for (unsigned j = 0; j < 8; j++) v |= (uint64_t)pf_iq2_grid_byte(i, j) << (8 * j);
-        host[i] = v;
-    }
-    uint64_t *d = nullptr;
-    if (hipMalloc(&d, sizeof host) != hipSuccess) return nullptr;
-    if (hipMemcpy(d, host, sizeof host, hipMemcpyHostToDevice) != hipSuccess) { (void)hipFree(d); return nullptr; }
-    g_grid = d;
-    return g_grid;
+static int need_device(void) {
+    if (pf_hip_device_count() >= 1) return PF_HIP_OK;
+    snprintf(g_error, sizeof g_error, "no HIP device");
+    return PF_HIP_E_NO_DEVICE;
 }
+
+// IQ2_XXS constants, one copy per process (one device per process): the 256 x 8
+// magnitudes, and for the integer dot products four signed magnitudes per (grid entry,
+// sign nibble): words [0, 4096) positions 0..3, words [4096, 8192) positions 4..7.
+static uint64_t *g_grid = nullptr;
+static uint32_t *g_signed = nullptr;
+
+static bool upload_constants(void) {
+    if (g_grid && g_signed) return true;
+    uint64_t grid[256];
+    uint32_t *tables = (uint32_t *)malloc(8192 * sizeof(uint32_t));
+    if (!tables) return false;
+    for (unsigned g = 0; g < 256; g++) {
+        uint64_t v = 0;
+        for (unsigned j = 0; j < 8; j++) v |= (uint64_t)pf_iq2_grid_byte(g, j) << (8 * j);
+        grid[g] = v;
+        for (unsigned s = 0; s < 16; s++)
+            for (unsigned half = 0; half < 2; half++) {
+                uint32_t word = 0;
+                for (unsigned j = 0; j < 4; j++) {
+                    int m = (int)pf_iq2_grid_byte(g, 4 * half + j);
+                    if ((s >> j) & 1u) m = -m;
+                    word |= ((uint32_t)m & 255u) << (8 * j);
+                }
+                tables[4096 * half + ((g << 4) | s)] = word;
+            }
+    }
+    uint64_t *dg = nullptr;
+    uint32_t *dt = nullptr;
+    bool ok = hipMalloc(&dg, sizeof grid) == hipSuccess && hipMalloc(&dt, 8192 * 4) == hipSuccess &&
+              hipMemcpy(dg, grid, sizeof grid, hipMemcpyHostToDevice) == hipSuccess &&
+              hipMemcpy(dt, tables, 8192 * 4, hipMemcpyHostToDevice) == hipSuccess;
+    free(tables);
+    if (!ok) {
+        if (dg) (void)hipFree(dg);
+        if (dt) (void)hipFree(dt);
+        return false;
+    }
+    g_grid = dg;
+    g_signed = dt;
+    return true;
+}
+const uint64_t *pf_device_iq2_grid(void) { return upload_constants() ? g_grid : nullptr; }
+const uint32_t *pf_device_iq2_signed(void) { return upload_constants() ? g_signed : nullptr; }
 
 static bool block_geometry(uint32_t type, size_t *block, size_t *bytes) {
     switch (type) {
@@ -54,9 +87,10 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
                                  PfHipMoe **out) {
     if (out) *out = nullptr;
     if (!desc || !host_weights || !bytes || !out) return PF_HIP_E_ARGUMENT;
-    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
     const size_t h = desc->hidden, i = desc->inter, s = desc->shared_inter, E = desc->experts;
     const size_t k_storage[8] = {h, h, h, desc->down_physical, h, h, s, h};
+    const size_t k_logical[8] = {h, h, h, i, h, h, s, h};
     const size_t n_out[8] = {E, i, i, h, s, s, h, 1};
     const size_t experts[8] = {1, E, E, E, 1, 1, 1, 1};
     if (!h || !i || !s || !E || !desc->top_k || desc->top_k > E || desc->down_physical < i) return PF_HIP_E_ARGUMENT;
@@ -64,22 +98,49 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
     PfHipMoe *m = (PfHipMoe *)calloc(1, sizeof *m);
     if (!m) return PF_HIP_E_MEMORY;
     m->desc = *desc;
+    size_t gguf_bytes[8];
     for (int a = 0; a < 8; a++) {
         size_t block, size;
-        if (!block_geometry(desc->type[a], &block, &size) || k_storage[a] % block) {
+        if (!block_geometry(desc->type[a], &block, &size) || k_storage[a] % block || k_storage[a] > 0x7fffffffu ||
+            n_out[a] > 0x7fffffffu) {
             pf_hip_moe_destroy(m);
             return PF_HIP_E_UNSUPPORTED;
         }
-        m->row_bytes[a] = k_storage[a] / block * size;
+        const size_t blocks_per_row = k_storage[a] / block, rows = n_out[a] * experts[a];
+        gguf_bytes[a] = blocks_per_row * size * rows;
+        if (bytes[a] < gguf_bytes[a] || !host_weights[a]) { pf_hip_moe_destroy(m); return PF_HIP_E_ARGUMENT; }
+        m->k_logical[a] = (int)k_logical[a];
+        m->n_out[a] = (int)n_out[a];
+        m->blocks_per_row[a] = (int)blocks_per_row;
+        if (desc->type[a] == PF_IQ2_XXS) {
+            // device layout: every block's 64-byte payload, then every block's half scale
+            m->row_bytes[a] = blocks_per_row * 64;
+            m->scale_offset[a] = (blocks_per_row * rows * 64 + 255) & ~(size_t)255;
+            m->bytes[a] = m->scale_offset[a] + blocks_per_row * rows * 2;
+        } else {
+            m->row_bytes[a] = blocks_per_row * size;
+            m->bytes[a] = gguf_bytes[a];
+        }
         m->expert_bytes[a] = m->row_bytes[a] * n_out[a];
-        m->bytes[a] = m->expert_bytes[a] * experts[a];
-        if (bytes[a] < m->bytes[a] || !host_weights[a]) { pf_hip_moe_destroy(m); return PF_HIP_E_ARGUMENT; }
     }
-    m->iq2_grid = const_cast<uint64_t *>(pf_device_iq2_grid());
-    if (!m->iq2_grid) { pf_hip_moe_destroy(m); return PF_HIP_E_MEMORY; }
+    if (!upload_constants()) { pf_hip_moe_destroy(m); return PF_HIP_E_MEMORY; }
+    m->iq2_grid = g_grid;
+    m->iq2_signed = g_signed;
     for (int a = 0; a < 8; a++) {
         hipError_t e = hipMalloc((void **)&m->w[a], m->bytes[a]);
-        if (e == hipSuccess) e = hipMemcpy(m->w[a], host_weights[a], m->bytes[a], hipMemcpyHostToDevice);
+        if (e == hipSuccess && desc->type[a] == PF_IQ2_XXS) {
+            uint8_t *staging = nullptr;
+            e = hipMalloc((void **)&staging, gguf_bytes[a]);
+            if (e == hipSuccess) e = hipMemcpy(staging, host_weights[a], gguf_bytes[a], hipMemcpyHostToDevice);
+            if (e == hipSuccess) {
+                pf_launch_iq2_split(staging, m->w[a], reinterpret_cast<uint16_t *>(m->w[a] + m->scale_offset[a]),
+                                    gguf_bytes[a] / 66, nullptr);
+                e = hipDeviceSynchronize();
+            }
+            if (staging) (void)hipFree(staging);
+        } else if (e == hipSuccess) {
+            e = hipMemcpy(m->w[a], host_weights[a], m->bytes[a], hipMemcpyHostToDevice);
+        }
         if (e != hipSuccess) {
             pf_set_error("weight upload", e);
             pf_hip_moe_destroy(m);
@@ -87,6 +148,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         }
         m->total_bytes += m->bytes[a];
     }
+    m->decode_ready = pf_decode_supported(*desc);
     *out = m;
     return PF_HIP_OK;
 }
@@ -99,31 +161,35 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
 
 extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_bytes : 0; }
 
-// workspace layout: a list of (pointer slot, bytes) carved from one allocation
-struct Carve { size_t offset[16], bytes[16], total; int n; };
+// workspace layout: buffers carved from one allocation, each 256-byte aligned
+enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_SOUT, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS,
+       W_IMAGES, W_COUNT };
+struct Carve { size_t offset[W_COUNT], total; };
 static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     Carve c;
     memset(&c, 0, sizeof c);
-    const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden;
-    const size_t want[] = {
-        T * E * 4,            // 0 logits
-        T * E * 4,            // 1 logit_ssq
-        T * K * 4,            // 2 route weights
-        T * K * d->inter * 4, // 3 act
-        T * d->shared_inter * 4, // 4 shared act
-        T * 4,                // 5 shared scale
-        T * H * 4,            // 6 x staging
-        T * H * 4,            // 7 y staging
-        T * K * 4,            // 8 ids
-        256,                  // 9 error word
-        256,                  // 10 exact rows
-        T * 4,                // 11 route flags
-    };
-    c.n = (int)(sizeof want / sizeof want[0]);
-    for (int j = 0; j < c.n; j++) {
+    const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden, I = d->inter;
+    const size_t Td = T < PF_DECODE_MAX_TOKENS ? T : PF_DECODE_MAX_TOKENS;   // tokens per decode launch
+    const size_t image = (3 * 20 * ((I + 63) / 64) + 2 * ((I + 31) / 32)) * 4;
+    size_t want[W_COUNT];
+    want[W_LOGITS] = T * E * 4;
+    want[W_SSQ] = T * E * 4;
+    want[W_RW] = T * K * 4;
+    want[W_ACT] = (T * K > Td * K * Td ? T * K : Td * K * Td) * I * 4;
+    want[W_SACT] = T * d->shared_inter * 4;
+    want[W_SSCALE] = T * 4;
+    want[W_SOUT] = Td * H * 4;
+    want[W_X] = T * H * 4;
+    want[W_Y] = T * H * 4;
+    want[W_IDS] = T * K * 4;
+    want[W_UNIQ] = (1 + 3 * Td * K) * 4;
+    want[W_ERR] = 256;
+    want[W_EXACT] = 256;
+    want[W_FLAGS] = T * 4;
+    want[W_IMAGES] = Td * K * Td * image;
+    for (int j = 0; j < W_COUNT; j++) {
         c.offset[j] = c.total;
-        c.bytes[j] = (want[j] + 255) & ~(size_t)255;
-        c.total += c.bytes[j];
+        c.total += (want[j] + 255) & ~(size_t)255;
     }
     return c;
 }
@@ -148,18 +214,21 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
         return PF_HIP_E_MEMORY;
     }
     w->moe = moe; w->cap = token_cap; w->bytes = c.total;
-    w->logits = (float *)(base + c.offset[0]);
-    w->logit_ssq = (float *)(base + c.offset[1]);
-    w->route_weights = (float *)(base + c.offset[2]);
-    w->act = (float *)(base + c.offset[3]);
-    w->shared_act = (float *)(base + c.offset[4]);
-    w->shared_scale = (float *)(base + c.offset[5]);
-    w->x = (float *)(base + c.offset[6]);
-    w->y = (float *)(base + c.offset[7]);
-    w->ids = (uint32_t *)(base + c.offset[8]);
-    w->error_word = (uint32_t *)(base + c.offset[9]);
-    w->exact_rows = (uint32_t *)(base + c.offset[10]);
-    w->route_flags = (uint32_t *)(base + c.offset[11]);
+    w->logits = (float *)(base + c.offset[W_LOGITS]);
+    w->logit_ssq = (float *)(base + c.offset[W_SSQ]);
+    w->route_weights = (float *)(base + c.offset[W_RW]);
+    w->act = (float *)(base + c.offset[W_ACT]);
+    w->shared_act = (float *)(base + c.offset[W_SACT]);
+    w->shared_scale = (float *)(base + c.offset[W_SSCALE]);
+    w->shared_out = (float *)(base + c.offset[W_SOUT]);
+    w->x = (float *)(base + c.offset[W_X]);
+    w->y = (float *)(base + c.offset[W_Y]);
+    w->ids = (uint32_t *)(base + c.offset[W_IDS]);
+    w->uniq = (uint32_t *)(base + c.offset[W_UNIQ]);
+    w->error_word = (uint32_t *)(base + c.offset[W_ERR]);
+    w->exact_rows = (uint32_t *)(base + c.offset[W_EXACT]);
+    w->route_flags = (uint32_t *)(base + c.offset[W_FLAGS]);
+    w->act_images = (int *)(base + c.offset[W_IMAGES]);
     *out = w;
     return PF_HIP_OK;
 }
@@ -167,7 +236,6 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
 extern "C" void pf_hip_work_destroy(PfHipWork *w) {
     if (!w) return;
     if (w->logits) (void)hipFree(w->logits);   // base of the single allocation
-    if (w->host_stage) (void)hipHostFree(w->host_stage);
     free(w);
 }
 
@@ -182,6 +250,15 @@ extern "C" int pf_hip_work_exact_rows(PfHipWork *w, uint32_t *count) {
     return PF_HIP_OK;
 }
 
+extern "C" int pf_hip_work_clear_status(PfHipWork *w) {
+    if (!w) return PF_HIP_E_ARGUMENT;
+    HIP_TRY(hipMemset(w->error_word, 0, 4));
+    HIP_TRY(hipMemset(w->exact_rows, 0, 4));
+    return PF_HIP_OK;
+}
+
+extern "C" void pf_hip_work_force_general(PfHipWork *w, int on) { if (w) w->force_general = on; }
+
 static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x, size_t x_pitch, float *d_y,
                               size_t y_pitch) {
     PfKernelArgs a;
@@ -194,17 +271,22 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
         a.w[j] = m->w[j];
         a.row_bytes[j] = m->row_bytes[j];
         a.expert_bytes[j] = m->expert_bytes[j];
+        a.scale_offset[j] = m->scale_offset[j];
+        a.k_logical[j] = m->k_logical[j];
+        a.blocks_per_row[j] = m->blocks_per_row[j];
+        a.n_out[j] = m->n_out[j];
     }
     a.iq2_grid = m->iq2_grid;
+    a.iq2_signed = m->iq2_signed;
     a.x = d_x; a.x_pitch = x_pitch; a.y = d_y; a.y_pitch = y_pitch;
     a.logits = w->logits; a.logit_ssq = w->logit_ssq; a.ids = w->ids; a.route_weights = w->route_weights;
-    a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale;
+    a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale; a.shared_out = w->shared_out;
+    a.act_images = w->act_images; a.uniq = w->uniq;
     a.error_word = w->error_word; a.exact_rows = w->exact_rows; a.route_flags = w->route_flags;
     return a;
 }
 
-__global__ void pf_k_clear2(uint32_t *a, uint32_t *b) { *a = 0; *b = 0; }
-
+// Enqueue only: no allocation, no synchronisation, no memset; safe under stream capture.
 extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch,
                                          float *d_y, size_t y_pitch, size_t tokens, void *stream) {
     if (!moe || !work || work->moe != moe) return PF_HIP_E_ARGUMENT;
@@ -212,47 +294,23 @@ extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, c
     if (tokens == 0) return PF_HIP_OK;
     if (!d_x || !d_y || x_pitch < moe->desc.hidden || y_pitch < moe->desc.hidden) return PF_HIP_E_ARGUMENT;
     const PfHipMoeDesc *d = &moe->desc;
-    // the general kernels stage one token's activations in LDS
-    const size_t lds_need = ((size_t)d->top_k * d->inter + d->shared_inter) * 4;
-    const size_t lds_route = ((size_t)d->hidden + 3 * (size_t)d->experts) * 4;
-    if (lds_need > 64 * 1024 || lds_route > 64 * 1024 || (size_t)d->hidden * 4 > 64 * 1024) {
-        snprintf(g_error, sizeof g_error, "dimensions exceed the LDS staging of the general kernels");
-        return PF_HIP_E_UNSUPPORTED;
-    }
     if (tokens * (size_t)d->top_k > 0x7fffffffu / 4) return PF_HIP_E_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
-    hipLaunchKernelGGL(pf_k_clear2, dim3(1), dim3(1), 0, s, work->error_word, work->exact_rows);
     PfKernelArgs a = make_args(moe, work, d_x, x_pitch, d_y, y_pitch);
-    pf_launch_general(a, (int)tokens, s, (hipEvent_t *)work->marks);
+    const bool aligned = (x_pitch % 4 == 0) && ((uintptr_t)d_x % 16 == 0);
+    if (moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS && aligned && !work->force_general) {
+        pf_launch_decode(a, (int)tokens, s, (hipEvent_t *)work->marks);
+    } else {
+        // the general kernels stage one token's activations in LDS
+        const size_t lds_route = ((size_t)d->hidden + 3 * (size_t)d->experts) * 4;
+        if (pf_general_lds_bytes(a) > 64 * 1024 || lds_route > 64 * 1024) {
+            snprintf(g_error, sizeof g_error, "dimensions exceed the LDS staging of the general kernels");
+            return PF_HIP_E_UNSUPPORTED;
+        }
+        pf_launch_general(a, (int)tokens, s, (hipEvent_t *)work->marks);
+    }
     HIP_TRY(hipGetLastError());
     return PF_HIP_OK;
-}
-
-extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
-                                         float *d_y, size_t tokens, size_t iters, float stage_ms[4]) {
-    if (!moe || !work || !d_x || !d_y || !n_inputs || !stage_ms) return PF_HIP_E_ARGUMENT;
-    const size_t H = moe->desc.hidden;
-    hipStream_t s = nullptr;
-    hipEvent_t marks[5];
-    HIP_TRY(hipStreamCreate(&s));
-    for (int j = 0; j < 5; j++) HIP_TRY(hipEventCreate(&marks[j]));
-    for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
-    int rc = PF_HIP_OK;
-    work->marks = marks;
-    for (size_t i = 0; i < iters && rc == PF_HIP_OK; i++) {
-        rc = pf_hip_moe_forward_device(moe, work, d_x + (i % n_inputs) * tokens * H, H, d_y, H, tokens, s);
-        if (rc == PF_HIP_OK && hipStreamSynchronize(s) != hipSuccess) rc = PF_HIP_E_RUNTIME;
-        for (int j = 0; j < 4 && rc == PF_HIP_OK; j++) {
-            float ms = 0.0f;
-            if (hipEventElapsedTime(&ms, marks[j], marks[j + 1]) != hipSuccess) rc = PF_HIP_E_RUNTIME;
-            stage_ms[j] += ms;
-        }
-    }
-    work->marks = nullptr;
-    for (int j = 0; j < 4; j++) stage_ms[j] /= (float)(iters ? iters : 1);
-    for (int j = 0; j < 5; j++) (void)hipEventDestroy(marks[j]);
-    (void)hipStreamDestroy(s);
-    return rc;
 }
 
 extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
@@ -265,10 +323,14 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
     if (!x || !y || tokens > work->cap) return PF_HIP_E_ARGUMENT;
     const size_t H = moe->desc.hidden, K = moe->desc.top_k;
     HIP_TRY(hipMemcpy2D(work->x, H * 4, x, x_pitch_bytes, H * 4, tokens, hipMemcpyHostToDevice));
+    // prefill-sized batches go through whole; 2..4 tokens use the decode path in one launch
     int rc = pf_hip_moe_forward_device(moe, work, work->x, H, work->y, H, tokens, nullptr);
     if (rc != PF_HIP_OK) return rc;
     HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
-    if (*error_word) return PF_HIP_OK;
+    if (*error_word) {
+        HIP_TRY(hipMemset(work->error_word, 0, 4));   // the word is sticky on the device; reading it clears it
+        return PF_HIP_OK;
+    }
     HIP_TRY(hipMemcpy2D(y, y_pitch_bytes, work->y, H * 4, H * 4, tokens, hipMemcpyDeviceToHost));
     if (ids) HIP_TRY(hipMemcpy2D(ids, ids_pitch_bytes, work->ids, K * 4, K * 4, tokens, hipMemcpyDeviceToHost));
     if (weights)
@@ -292,7 +354,7 @@ extern "C" int pf_hip_route_host(const float *logits, size_t tokens, size_t expe
     if (tokens == 0) return PF_HIP_OK;
     if (!logits || !probs || !ids || !weights || !experts || !top_k || top_k > experts) return PF_HIP_E_ARGUMENT;
     if (tokens * experts > 0x7fffffffu) return PF_HIP_E_UNSUPPORTED;
-    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
     const size_t zb = tokens * experts * 4, kb = tokens * top_k * 4;
     const size_t o_p = (zb + 255) & ~(size_t)255, o_i = o_p * 2, o_w = o_i + ((kb + 255) & ~(size_t)255),
                  o_e = o_w + ((kb + 255) & ~(size_t)255);
@@ -327,24 +389,24 @@ extern "C" int pf_hip_group_pairs_host(const uint32_t *ids, size_t tokens, size_
     *duplicate = 0;
     const size_t pairs = tokens * top_k;
     if (pairs > 0x3fffffffu || experts > 0x3fffffffu) return PF_HIP_E_UNSUPPORTED;
-    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
     if (pairs && (!ids || !pair_to_row || !row_to_pair)) return PF_HIP_E_ARGUMENT;
     const size_t pb = ((pairs ? pairs : 1) * 4 + 255) & ~(size_t)255, eb = ((experts + 1) * 4 + 255) & ~(size_t)255;
-    // ids | counts | offsets | pair_to_row | row_to_pair | error
+    // ids | counts | offsets | pair_to_row | row_to_pair | first offending pair
     DeviceBlock blk;
     HIP_TRY(hipMalloc((void **)&blk.p, 3 * pb + 2 * eb + 256));
     uint32_t *d_ids = (uint32_t *)blk.p, *d_counts = (uint32_t *)(blk.p + pb), *d_off = (uint32_t *)(blk.p + pb + eb);
     uint32_t *d_p2r = (uint32_t *)(blk.p + pb + 2 * eb), *d_r2p = (uint32_t *)(blk.p + 2 * pb + 2 * eb);
-    uint32_t *d_err = (uint32_t *)(blk.p + 3 * pb + 2 * eb);
+    uint32_t *d_bad = (uint32_t *)(blk.p + 3 * pb + 2 * eb);
     if (pairs) HIP_TRY(hipMemcpy(d_ids, ids, pairs * 4, hipMemcpyHostToDevice));
-    int rc = pf_group_pairs_device(d_ids, (int)tokens, (int)experts, (int)top_k, d_counts, d_off, d_p2r, d_r2p, d_err,
+    int rc = pf_group_pairs_device(d_ids, (int)tokens, (int)experts, (int)top_k, d_counts, d_off, d_p2r, d_r2p, d_bad,
                                    nullptr);
     if (rc != PF_HIP_OK) return rc;
     HIP_TRY(hipDeviceSynchronize());
-    uint32_t err = 0;
-    HIP_TRY(hipMemcpy(&err, d_err, 4, hipMemcpyDeviceToHost));
-    if (err != 0xffffffffu) {   // first offending pair in scan order, low bit = kind
-        if (err & 1u) *duplicate = 1;
+    uint32_t bad = 0;
+    HIP_TRY(hipMemcpy(&bad, d_bad, 4, hipMemcpyDeviceToHost));
+    if (bad != 0xffffffffu) {   // first offending pair in scan order, low bit = kind
+        if (bad & 1u) *duplicate = 1;
         else *error_word = PF_HIP_ERR_BOUNDS;
         return PF_HIP_OK;
     }
@@ -373,7 +435,7 @@ extern "C" int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_
     if (!block_geometry(gguf_type, &block, &size)) return PF_HIP_E_UNSUPPORTED;
     if (!expert_bytes || !x || !y || !n_out || !k_logical) return PF_HIP_E_ARGUMENT;
     if (rows * n_out > 0x7fffffffu || k_logical > 0x7fffffffu) return PF_HIP_E_UNSUPPORTED;
-    if (pf_hip_device_count() < 1) { snprintf(g_error, sizeof g_error, "no HIP device"); return PF_HIP_E_NO_DEVICE; }
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
     const uint64_t *grid = pf_device_iq2_grid();
     if (!grid) return PF_HIP_E_MEMORY;
     const size_t wb = (row_bytes * n_out + 255) & ~(size_t)255, xb = (rows * k_logical * 4 + 255) & ~(size_t)255,
@@ -399,7 +461,7 @@ extern "C" int pf_hip_packed_decode_row_host(uint32_t gguf_type, const void *row
     size_t block, size;
     if (!block_geometry(gguf_type, &block, &size)) return PF_HIP_E_UNSUPPORTED;
     if (!row || !out || !k_storage || k_storage > 0x7fffffffu) return PF_HIP_E_ARGUMENT;
-    if (pf_hip_device_count() < 1) return PF_HIP_E_NO_DEVICE;
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
     const uint64_t *grid = pf_device_iq2_grid();
     if (!grid) return PF_HIP_E_MEMORY;
     const size_t wb = (row_bytes + 255) & ~(size_t)255, ob = (k_storage * 4 + 255) & ~(size_t)255;
@@ -438,24 +500,71 @@ extern "C" int pf_hip_synchronize(void) {
     return PF_HIP_OK;
 }
 
+// `iters` forwards back to back on one stream.  The launches are captured into graphs of
+// up to 256 forwards (each with its own input block) and the graphs are replayed in order,
+// so the measured gap between dependent kernels is the device's, not the host's enqueue rate.
 extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
                                         float *d_y, size_t tokens, size_t iters, float *elapsed_ms) {
     if (!moe || !work || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
+    *elapsed_ms = 0.0f;
+    if (!iters) return PF_HIP_OK;
+    const size_t H = moe->desc.hidden, chunk = 256, n_graphs = (iters + chunk - 1) / chunk;
+    hipStream_t s = nullptr;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    HIP_TRY(hipStreamCreate(&s));
+    hipGraphExec_t *execs = (hipGraphExec_t *)calloc(n_graphs, sizeof *execs);
+    int rc = execs ? PF_HIP_OK : PF_HIP_E_MEMORY;
+    for (size_t g = 0; g < n_graphs && rc == PF_HIP_OK; g++) {
+        hipGraph_t graph = nullptr;
+        if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) { rc = PF_HIP_E_RUNTIME; break; }
+        for (size_t i = g * chunk; i < iters && i < (g + 1) * chunk && rc == PF_HIP_OK; i++)
+            rc = pf_hip_moe_forward_device(moe, work, d_x + (i % n_inputs) * tokens * H, H, d_y, H, tokens, s);
+        hipError_t e = hipStreamEndCapture(s, &graph);
+        if (e != hipSuccess && rc == PF_HIP_OK) { pf_set_error("hipStreamEndCapture", e); rc = PF_HIP_E_RUNTIME; }
+        if (rc == PF_HIP_OK && hipGraphInstantiate(&execs[g], graph, nullptr, nullptr, 0) != hipSuccess)
+            rc = PF_HIP_E_RUNTIME;
+        if (graph) (void)hipGraphDestroy(graph);
+    }
+    if (rc == PF_HIP_OK && (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess)) rc = PF_HIP_E_RUNTIME;
+    if (rc == PF_HIP_OK) {
+        hipError_t e = hipEventRecord(t0, s);
+        for (size_t g = 0; g < n_graphs && e == hipSuccess; g++) e = hipGraphLaunch(execs[g], s);
+        if (e == hipSuccess) e = hipEventRecord(t1, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+        if (e != hipSuccess) { pf_set_error("timed graph replay", e); rc = PF_HIP_E_RUNTIME; }
+    }
+    for (size_t g = 0; execs && g < n_graphs; g++) if (execs[g]) (void)hipGraphExecDestroy(execs[g]);
+    free(execs);
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    (void)hipStreamDestroy(s);
+    return rc;
+}
+
+extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
+                                         float *d_y, size_t tokens, size_t iters, float stage_ms[4]) {
+    if (!moe || !work || !d_x || !d_y || !n_inputs || !stage_ms) return PF_HIP_E_ARGUMENT;
     const size_t H = moe->desc.hidden;
     hipStream_t s = nullptr;
-    hipEvent_t t0, t1;
+    hipEvent_t marks[5];
     HIP_TRY(hipStreamCreate(&s));
-    HIP_TRY(hipEventCreate(&t0));
-    HIP_TRY(hipEventCreate(&t1));
+    for (int j = 0; j < 5; j++) HIP_TRY(hipEventCreate(&marks[j]));
+    for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
     int rc = PF_HIP_OK;
-    HIP_TRY(hipEventRecord(t0, s));
-    for (size_t i = 0; i < iters && rc == PF_HIP_OK; i++)
+    work->marks = marks;
+    for (size_t i = 0; i < iters && rc == PF_HIP_OK; i++) {
         rc = pf_hip_moe_forward_device(moe, work, d_x + (i % n_inputs) * tokens * H, H, d_y, H, tokens, s);
-    HIP_TRY(hipEventRecord(t1, s));
-    HIP_TRY(hipStreamSynchronize(s));
-    if (rc == PF_HIP_OK) HIP_TRY(hipEventElapsedTime(elapsed_ms, t0, t1));
-    (void)hipEventDestroy(t0);
-    (void)hipEventDestroy(t1);
+        if (rc == PF_HIP_OK && hipStreamSynchronize(s) != hipSuccess) rc = PF_HIP_E_RUNTIME;
+        for (int j = 0; j < 4 && rc == PF_HIP_OK; j++) {
+            float ms = 0.0f;
+            if (hipEventElapsedTime(&ms, marks[j], marks[j + 1]) != hipSuccess) rc = PF_HIP_E_RUNTIME;
+            stage_ms[j] += ms;
+        }
+    }
+    work->marks = nullptr;
+    for (int j = 0; j < 4; j++) stage_ms[j] /= (float)(iters ? iters : 1);
+    for (int j = 0; j < 5; j++) (void)hipEventDestroy(marks[j]);
     (void)hipStreamDestroy(s);
     return rc;
 }

@@ -1,0 +1,625 @@
+// Decode path: 1..4 tokens through one MoE layer as three dependent kernels.
+//
+//   pf_k_dec_pre      router logits (F32 rows), shared gate/up + SwiGLU, shared router
+//   pf_k_dec_gate_up  routing (every workgroup repeats it from the logits), the union
+//                     of the tokens' experts, routed gate/up + SwiGLU once per unique
+//                     expert, and the shared expert's down product
+//   pf_k_dec_down     routed down products, slot-ordered weighted sum, shared branch
+//
+// A dependent kernel boundary costs about 1.6 us on this GPU when replayed from a
+// graph; an in-kernel barrier across its eight L2 domains costs more, so the three
+// data dependencies of the block are kernel boundaries.
+//
+// Arithmetic.  A lane owns 64 consecutive weights of a row (two 32-weight groups:
+// one Q4_K nibble pair or two IQ2_XXS groups).  Activations are turned into block
+// fixed point once per vector: per 32-group a power-of-two step and, per value, a
+// 21-bit integer written as three balanced base-128 digits.  Weight codes are small
+// integers in both formats, so the group dot product is three v_dot4_i32_i8 chains
+// and exact; the group scales are applied in FP32 afterwards.  The activation error
+// is at most 2^-21 of the largest magnitude of its group.
+#include "pf_moe_internal.h"
+#include "pf_route_device.h"
+#include "pf_route_fast.h"
+
+#define SEG_STRIDE 20   // dwords per 64-value segment of a digit plane (16 used): spreads LDS banks
+
+// ---- digit images --------------------------------------------------------------------
+// Image of a K-vector: three digit planes of SEG_STRIDE * K/64 dwords, then K/32 group
+// steps (float), then K/32 group sums of the integer values.
+__host__ __device__ constexpr int image_words(int K) { return 3 * SEG_STRIDE * (K / 64) + 2 * (K / 32); }
+
+struct XSeg {          // one lane's 64 activations
+    int d0[16], d1[16], d2[16];
+    float step[2];
+    int sum[2];
+};
+
+__device__ __forceinline__ void xseg_load(XSeg &s, const int *img, int K, int seg) {
+    const int plane = SEG_STRIDE * (K / 64);
+    const int4 *p0 = reinterpret_cast<const int4 *>(img + SEG_STRIDE * seg);
+    const int4 *p1 = reinterpret_cast<const int4 *>(img + plane + SEG_STRIDE * seg);
+    const int4 *p2 = reinterpret_cast<const int4 *>(img + 2 * plane + SEG_STRIDE * seg);
+#pragma unroll
+    for (int m = 0; m < 4; m++) {
+        int4 a = p0[m], b = p1[m], c = p2[m];
+        s.d0[4 * m] = a.x; s.d0[4 * m + 1] = a.y; s.d0[4 * m + 2] = a.z; s.d0[4 * m + 3] = a.w;
+        s.d1[4 * m] = b.x; s.d1[4 * m + 1] = b.y; s.d1[4 * m + 2] = b.z; s.d1[4 * m + 3] = b.w;
+        s.d2[4 * m] = c.x; s.d2[4 * m + 1] = c.y; s.d2[4 * m + 2] = c.z; s.d2[4 * m + 3] = c.w;
+    }
+    const float *steps = reinterpret_cast<const float *>(img + 3 * plane);
+    const int *sums = img + 3 * plane + K / 32;
+    s.step[0] = steps[2 * seg]; s.step[1] = steps[2 * seg + 1];
+    s.sum[0] = sums[2 * seg]; s.sum[1] = sums[2 * seg + 1];
+}
+
+__device__ __forceinline__ int dpp_quad_xor1(int v) { return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true); }
+__device__ __forceinline__ int dpp_quad_xor2(int v) { return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true); }
+
+// power-of-two step for a group whose largest magnitude is m: |v| / step < 2^20
+__device__ __forceinline__ void group_step(float m, float &step, float &inv) {
+    int e = (__float_as_int(m) >> 23) & 255;
+    e = e < 21 ? 21 : e;
+    step = __int_as_float((e - 19) << 23);
+    inv = __int_as_float((273 - e) << 23);
+}
+
+__device__ __forceinline__ void split_digits(int q, int &d0, int &d1, int &d2) {
+    d0 = ((q + 64) & 127) - 64;
+    const int r = (q - d0) >> 7;
+    d1 = ((r + 64) & 127) - 64;
+    d2 = (r - d1) >> 7;
+}
+
+// All threads of the workgroup: image of src[0..K) (K % 32 == 0).  Thread j takes the
+// eight values 8j..8j+7; four neighbouring threads form one 32-group.
+__device__ __forceinline__ bool build_image(int *img, const float *src, int K) {
+    const int plane = SEG_STRIDE * (K / 64);
+    bool bad = false;
+    for (int j = threadIdx.x; j < K / 8; j += blockDim.x) {
+        const float4 a = reinterpret_cast<const float4 *>(src)[2 * j];
+        const float4 b = reinterpret_cast<const float4 *>(src)[2 * j + 1];
+        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        float m = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; c++) { m = fmaxf(m, fabsf(v[c])); bad |= !pf_finite(v[c]); }
+        m = fmaxf(m, __int_as_float(dpp_quad_xor1(__float_as_int(m))));
+        m = fmaxf(m, __int_as_float(dpp_quad_xor2(__float_as_int(m))));
+        float step, inv;
+        group_step(m, step, inv);
+        int w0[2] = {0, 0}, w1[2] = {0, 0}, w2[2] = {0, 0}, sum = 0;
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const int q = __float2int_rn(v[c] * inv);
+            sum += q;
+            int d0, d1, d2;
+            split_digits(q, d0, d1, d2);
+            w0[c >> 2] |= (d0 & 255) << (8 * (c & 3));
+            w1[c >> 2] |= (d1 & 255) << (8 * (c & 3));
+            w2[c >> 2] |= (d2 & 255) << (8 * (c & 3));
+        }
+        sum += dpp_quad_xor1(sum);
+        sum += dpp_quad_xor2(sum);
+        const int at = SEG_STRIDE * (j >> 3) + 2 * (j & 7);
+        img[at] = w0[0]; img[at + 1] = w0[1];
+        img[plane + at] = w1[0]; img[plane + at + 1] = w1[1];
+        img[2 * plane + at] = w2[0]; img[2 * plane + at + 1] = w2[1];
+        if ((j & 3) == 0) {
+            reinterpret_cast<float *>(img + 3 * plane)[j >> 2] = step;
+            img[3 * plane + K / 32 + (j >> 2)] = sum;
+        }
+    }
+    return bad;
+}
+
+// ---- one lane's 64 weights of a row --------------------------------------------------
+template <int FMT> struct WSeg;
+template <> struct WSeg<PF_Q4_K> { uint4 hdr, q0, q1; };
+template <> struct WSeg<PF_IQ2_XXS> { uint4 p; uint32_t dbits; };
+
+template <int FMT>
+__device__ __forceinline__ void wseg_load(WSeg<FMT> &w, const PfKernelArgs &a, int t, size_t e, size_t n, int seg);
+
+template <>
+__device__ __forceinline__ void wseg_load<PF_Q4_K>(WSeg<PF_Q4_K> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
+                                                   int seg) {
+    const uint8_t *blk = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + (size_t)(seg >> 2) * 144;
+    w.hdr = *reinterpret_cast<const uint4 *>(blk);
+    const uint4 *q = reinterpret_cast<const uint4 *>(blk + 16 + 32 * (seg & 3));
+    w.q0 = q[0];
+    w.q1 = q[1];
+}
+
+template <>
+__device__ __forceinline__ void wseg_load<PF_IQ2_XXS>(WSeg<PF_IQ2_XXS> &w, const PfKernelArgs &a, int t, size_t e,
+                                                      size_t n, int seg) {
+    const uint8_t *row = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t];
+    w.p = *reinterpret_cast<const uint4 *>(row + 16 * seg);
+    const uint16_t *scales = reinterpret_cast<const uint16_t *>(a.w[t] + a.scale_offset[t]);
+    w.dbits = scales[(e * a.n_out[t] + n) * a.blocks_per_row[t] + (seg >> 2)];
+}
+
+__device__ __forceinline__ float half_bits(uint32_t h) {
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
+}
+
+template <int FMT>
+__device__ __forceinline__ float wseg_dot(const WSeg<FMT> &w, const XSeg &x, int seg, const uint32_t *tables);
+
+// Q4_K: low nibbles of the 32 bytes are group 2j, high nibbles group 2j+1
+template <>
+__device__ __forceinline__ float wseg_dot<PF_Q4_K>(const WSeg<PF_Q4_K> &w, const XSeg &x, int seg, const uint32_t *) {
+    const uint32_t q[8] = {w.q0.x, w.q0.y, w.q0.z, w.q0.w, w.q1.x, w.q1.y, w.q1.z, w.q1.w};
+    int l0 = 0, l1 = 0, l2 = 0, h0 = 0, h1 = 0, h2 = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+        l0 = __builtin_amdgcn_sdot4(lo, x.d0[i], l0, false);
+        l1 = __builtin_amdgcn_sdot4(lo, x.d1[i], l1, false);
+        l2 = __builtin_amdgcn_sdot4(lo, x.d2[i], l2, false);
+        h0 = __builtin_amdgcn_sdot4(hi, x.d0[8 + i], h0, false);
+        h1 = __builtin_amdgcn_sdot4(hi, x.d1[8 + i], h1, false);
+        h2 = __builtin_amdgcn_sdot4(hi, x.d2[8 + i], h2, false);
+    }
+    const float tl = (float)(l0 + (l1 << 7) + (l2 << 14)), th = (float)(h0 + (h1 << 7) + (h2 << 14));
+    // 6-bit scales and minima of groups 2j, 2j+1 (j = seg % 4) from the 12 packed bytes
+    const int j = seg & 3, sh = 16 * (j & 1);
+    const uint32_t wa = w.hdr.y >> sh, wb = w.hdr.z >> sh, wc = w.hdr.w >> sh;
+    uint32_t s0, m0, s1, m1;
+    if (j < 2) {
+        s0 = wa & 63u; s1 = (wa >> 8) & 63u; m0 = wb & 63u; m1 = (wb >> 8) & 63u;
+    } else {
+        s0 = (wc & 15u) | ((wa >> 2) & 48u);
+        m0 = ((wc >> 4) & 15u) | ((wb >> 2) & 48u);
+        s1 = ((wc >> 8) & 15u) | ((wa >> 10) & 48u);
+        m1 = ((wc >> 12) & 15u) | ((wb >> 10) & 48u);
+    }
+    const float d = half_bits(w.hdr.x & 0xffffu), dmin = half_bits(w.hdr.x >> 16);
+    const float lo = x.step[0] * fmaf(d * (float)s0, tl, -(dmin * (float)m0) * (float)x.sum[0]);
+    const float hi = x.step[1] * fmaf(d * (float)s1, th, -(dmin * (float)m1) * (float)x.sum[1]);
+    return lo + hi;
+}
+
+// IQ2_XXS: tables[(g << 4) | s] holds the four signed magnitudes of positions 0..3 of grid
+// entry g under sign nibble s; tables[4096 + ...] positions 4..7 (bit 3 = the parity sign).
+template <>
+__device__ __forceinline__ float wseg_dot<PF_IQ2_XXS>(const WSeg<PF_IQ2_XXS> &w, const XSeg &x, int,
+                                                      const uint32_t *tables) {
+    float acc[2];
+#pragma unroll
+    for (int gg = 0; gg < 2; gg++) {
+        const uint32_t idx = gg ? w.p.z : w.p.x, word = gg ? w.p.w : w.p.y;
+        int a0 = 0, a1 = 0, a2 = 0;
+#pragma unroll
+        for (int slot = 0; slot < 4; slot++) {
+            const uint32_t g = (idx >> (8 * slot)) & 255u, s7 = (word >> (7 * slot)) & 127u;
+            const uint32_t par = __popc(s7) & 1u;
+            const int ml = (int)tables[(g << 4) | (s7 & 15u)];
+            const int mh = (int)tables[4096u + ((g << 4) | (s7 >> 4) | (par << 3))];
+            const int m = 8 * gg + 2 * slot;
+            a0 = __builtin_amdgcn_sdot4(ml, x.d0[m], a0, false);
+            a1 = __builtin_amdgcn_sdot4(ml, x.d1[m], a1, false);
+            a2 = __builtin_amdgcn_sdot4(ml, x.d2[m], a2, false);
+            a0 = __builtin_amdgcn_sdot4(mh, x.d0[m + 1], a0, false);
+            a1 = __builtin_amdgcn_sdot4(mh, x.d1[m + 1], a1, false);
+            a2 = __builtin_amdgcn_sdot4(mh, x.d2[m + 1], a2, false);
+        }
+        acc[gg] = x.step[gg] * (float)(2u * (word >> 28) + 1u) * (float)(a0 + (a1 << 7) + (a2 << 14));
+    }
+    return half_bits(w.dbits) * 0.125f * (acc[0] + acc[1]);
+}
+
+// sum over `width` neighbouring lanes (power of two, <= 32); result in the lowest lane of each span
+__device__ __forceinline__ float span_sum(float v, int width) {
+    for (int m = width >> 1; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+    return v;
+}
+
+__device__ __forceinline__ void stage_tables(uint32_t *lds, const uint32_t *global) {
+    const uint4 *src = reinterpret_cast<const uint4 *>(global);
+    uint4 *dst = reinterpret_cast<uint4 *>(lds);
+    for (int i = threadIdx.x; i < 2048; i += blockDim.x) dst[i] = src[i];
+}
+
+template <int FMT> __host__ __device__ constexpr int table_words() { return FMT == PF_IQ2_XXS ? 8192 : 0; }
+
+// ---- kernel 1: everything that depends on x only -------------------------------------------
+// blocks [0, router_blocks): one router row per wave, all tokens;
+// blocks [router_blocks, +shared_blocks): shared gate/up rows; last block: shared router row.
+template <int FMT, int NT>
+__global__ void __launch_bounds__(256) pf_k_dec_pre(PfKernelArgs a, int router_blocks, int shared_blocks) {
+    extern __shared__ int lds[];
+    const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
+    if ((int)blockIdx.x < router_blocks || (int)blockIdx.x == router_blocks + shared_blocks) {
+        const bool gate_row = (int)blockIdx.x == router_blocks + shared_blocks;
+        const int e = blockIdx.x * 4 + wave;
+        if (gate_row ? wave != 0 : e >= E) return;
+        const float4 *w = reinterpret_cast<const float4 *>(gate_row ? a.w[7] : a.w[0] + (size_t)e * H * 4);
+        float acc[NT], sq[NT];
+        bool bad = false;
+#pragma unroll
+        for (int t = 0; t < NT; t++) acc[t] = sq[t] = 0.0f;
+        for (int i = lane; i < H / 4; i += PF_WAVE) {
+            const float4 wv = w[i];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const float4 xv = reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch)[i];
+                const float p0 = wv.x * xv.x, p1 = wv.y * xv.y, p2 = wv.z * xv.z, p3 = wv.w * xv.w;
+                acc[t] += (p0 + p1) + (p2 + p3);
+                sq[t] = fmaf(p0, p0, fmaf(p1, p1, fmaf(p2, p2, fmaf(p3, p3, sq[t]))));
+                bad |= !pf_finite(xv.x) || !pf_finite(xv.y) || !pf_finite(xv.z) || !pf_finite(xv.w);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const float z = pf_wave_sum(acc[t]), s2 = pf_wave_sum(sq[t]);
+            if (lane == 0) {
+                if (gate_row) {
+                    a.shared_scale[t] = pf_sigmoid(z);
+                    if (!pf_finite(z)) bad = true;
+                } else {
+                    a.logits[(size_t)t * E + e] = z;
+                    a.logit_ssq[(size_t)t * E + e] = s2;
+                }
+            }
+        }
+        if (__any(bad) && lane == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        return;
+    }
+    // shared gate/up: lower half of the wave takes gate rows, upper half up rows
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
+    int *images = lds + table_words<FMT>();
+    if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
+    const int W = image_words(H);
+    for (int t = 0; t < NT; t++) build_image(images + t * W, a.x + (size_t)t * a.x_pitch, H);
+    __syncthreads();
+    const int LPR = H / 64, RPH = 32 / LPR, Is = a.shared_inter;
+    const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
+    const int base = ((blockIdx.x - router_blocks) * 4 + wave) * 2 * RPH;
+    WSeg<FMT> w[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+        const int n = min(base + s * RPH + r, Is - 1);
+        wseg_load<FMT>(w[s], a, 4 + half, 0, n, seg);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        XSeg x;
+        xseg_load(x, images + t * W, H, seg);
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const int n = base + s * RPH + r;
+            float v = span_sum(wseg_dot<FMT>(w[s], x, seg, tables), LPR);
+            const float u = __shfl(v, (lane & 31) + 32);
+            if (half == 0 && seg == 0 && n < Is) {
+                const float act = pf_silu(v) * u;
+                a.shared_act[(size_t)t * Is + n] = act;
+                if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+            }
+        }
+    }
+}
+
+// ---- kernel 2: routing, expert union, routed gate/up, shared down --------------------------
+struct RouteLds {
+    uint32_t ids[64];        // [token][slot]
+    float weights[64];
+    uint32_t uniq[64];       // unique experts in first-use order
+    uint32_t pair_slot[64];  // pair -> index into uniq
+    uint32_t mask[64];       // unique -> bit t set when token t uses it
+    uint32_t count, close_mask, bad;
+    float tile[PF_DECODE_MAX_TOKENS][32];
+};
+
+template <int NPL>
+__device__ __forceinline__ void route_tokens(const PfKernelArgs &a, RouteLds *R, float *scratch, int tokens) {
+    const int lane = pf_lane(), wave = threadIdx.x >> 6, E = a.experts, K = a.top_k;
+    if (threadIdx.x == 0) { R->close_mask = 0; R->bad = 0; }
+    __syncthreads();
+    if (wave < tokens) {
+        PfRouteResult r = pf_route_fast_wave<NPL>(a.logits + (size_t)wave * E, a.logit_ssq + (size_t)wave * E, E, K,
+                                                  a.norm_topk != 0, a.hidden, lane);
+        if (lane < K) {
+            R->ids[wave * K + lane] = r.id;
+            R->weights[wave * K + lane] = r.weight;
+        }
+        if (lane == 0) {
+            if (r.close) atomicOr(&R->close_mask, 1u << wave);
+            if (r.bad) R->bad = 1;
+        }
+    }
+    __syncthreads();
+    const uint32_t close = R->close_mask;
+    if (close) {
+        // reference-order logits and routing for the ambiguous tokens (rare)
+        const int H = a.hidden;
+        float *xs = scratch, *z = xs + H, *p = z + E, *q = p + E;
+        for (int t = 0; t < tokens; t++) {
+            if (!((close >> t) & 1u)) continue;
+            for (int k = threadIdx.x; k < H; k += blockDim.x) xs[k] = a.x[(size_t)t * a.x_pitch + k];
+            __syncthreads();
+            for (int e = threadIdx.x; e < E; e += blockDim.x)
+                z[e] = pf_serial_logit(reinterpret_cast<const float *>(a.w[0]) + (size_t)e * H, xs, H);
+            __syncthreads();
+            if (wave == 0) pf_route_exact_wave(z, p, q, E, K, a.norm_topk != 0, R->ids + t * K, R->weights + t * K, lane);
+            __syncthreads();
+        }
+    }
+    // union of the tokens' experts in first-use order (pairs <= 64)
+    if (wave == 0) {
+        const int P = tokens * K;
+        const uint32_t id = lane < P ? R->ids[lane] : 0xffffffffu;
+        bool first = lane < P;
+        for (int q = 0; q < P; q++) {
+            const uint32_t other = __shfl(id, q);
+            if (q < lane && other == id) first = false;
+        }
+        const unsigned long long firsts = __ballot(first);
+        const uint32_t my_index = __popcll(firsts & ((1ull << lane) - 1ull));
+        uint32_t slot = my_index, mask = 0;
+        for (int q = 0; q < P; q++) {
+            const uint32_t other = __shfl(id, q), other_index = __shfl(my_index, q);
+            const bool other_first = (firsts >> q) & 1ull;
+            if (other == id) {
+                if (other_first) slot = other_index;
+                mask |= 1u << (q / K);
+            }
+        }
+        if (lane < P) R->pair_slot[lane] = slot;
+        if (first) { R->uniq[my_index] = id; R->mask[my_index] = mask; }
+        if (lane == 0) R->count = __popcll(firsts);
+    }
+    __syncthreads();
+}
+
+template <int FMT, int NT, int NPL>
+__global__ void __launch_bounds__(256) pf_k_dec_gate_up(PfKernelArgs a, int routed_blocks) {
+    extern __shared__ int lds[];
+    __shared__ RouteLds R;
+    const int H = a.hidden, I = a.inter, K = a.top_k, lane = pf_lane(), wave = threadIdx.x >> 6;
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
+    int *images = lds + table_words<FMT>();
+    if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
+
+    if ((int)blockIdx.x >= routed_blocks) {
+        // shared expert's down product: shared_out[t][n] = shared_down[n] . shared_act[t]
+        const int Is = a.shared_inter, W = image_words(Is), LPR = Is / 64, rows = 64 / LPR;
+        bool bad = false;
+        for (int t = 0; t < NT; t++) bad |= build_image(images + t * W, a.shared_act + (size_t)t * Is, Is);
+        __syncthreads();
+        const int seg = lane & (LPR - 1);
+        const int n = ((blockIdx.x - routed_blocks) * 4 + wave) * rows + lane / LPR;
+        if (n - lane / LPR >= H) return;
+        WSeg<FMT> w;
+        wseg_load<FMT>(w, a, 6, 0, min(n, H - 1), seg);
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            XSeg x;
+            xseg_load(x, images + t * W, Is, seg);
+            const float v = span_sum(wseg_dot<FMT>(w, x, seg, tables), LPR);
+            if (seg == 0 && n < H) a.shared_out[(size_t)t * H + n] = v;
+        }
+        return;
+    }
+
+    const int W = image_words(H);
+    for (int t = 0; t < NT; t++) build_image(images + t * W, a.x + (size_t)t * a.x_pitch, H);
+    float *scratch = reinterpret_cast<float *>(images + NT * W);
+    route_tokens<NPL>(a, &R, scratch, NT);
+    const int P = NT * K, U = R.count;
+    if (blockIdx.x == 0) {
+        // publish the routes and the union for the next kernel and the caller
+        for (int p = threadIdx.x; p < P; p += blockDim.x) {
+            a.ids[p] = R.ids[p];
+            a.route_weights[p] = R.weights[p];
+            a.uniq[1 + p] = p < U ? R.uniq[p] : 0u;
+            a.uniq[1 + P + p] = R.pair_slot[p];
+            a.uniq[1 + 2 * P + p] = p < U ? R.mask[p] : 0u;
+        }
+        if (threadIdx.x == 0) {
+            a.uniq[0] = U;
+            if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+            if (R.close_mask) atomicAdd(a.exact_rows, __popc(R.close_mask));
+        }
+    }
+    const int tiles = I / 32, u = blockIdx.x / tiles, n0 = 32 * (blockIdx.x % tiles);
+    if (u >= U) return;
+    const uint32_t e = R.uniq[u], mask = R.mask[u];
+    if (e >= (uint32_t)a.experts) {   // only reachable with nonfinite logits
+        if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+        return;
+    }
+    const int LPR = H / 64, RPH = 32 / LPR;
+    const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
+    const int steps = 8 / RPH;                       // this wave's 8 units, RPH per step
+    XSeg x[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+        if ((mask >> t) & 1u) xseg_load(x[t], images + t * W, H, seg);
+    for (int s0 = 0; s0 < steps; s0 += 4) {
+        WSeg<FMT> w[4];
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+            if (s0 + s < steps) wseg_load<FMT>(w[s], a, 1 + half, e, n0 + wave * 8 + (s0 + s) * RPH + r, seg);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            if (s0 + s >= steps) break;
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                if (!((mask >> t) & 1u)) continue;
+                float v = span_sum(wseg_dot<FMT>(w[s], x[t], seg, tables), LPR);
+                const float up = __shfl(v, (lane & 31) + 32);
+                if (half == 0 && seg == 0) R.tile[t][wave * 8 + (s0 + s) * RPH + r] = pf_silu(v) * up;
+            }
+        }
+    }
+    __syncthreads();
+    // 32 activations per token: FP32 copy and digit image for the down kernel
+    if (wave < NT && ((mask >> wave) & 1u) && lane < 32) {
+        const int t = wave, WI = image_words(I), plane = SEG_STRIDE * (I / 64);
+        const float v = R.tile[t][lane];
+        if (!pf_finite(v)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        a.act[((size_t)u * NT + t) * I + n0 + lane] = v;
+        float m = fabsf(v);
+        for (int k = 16; k >= 1; k >>= 1) m = fmaxf(m, __shfl_xor(m, k));
+        float step, inv;
+        group_step(m, step, inv);
+        const int q = __float2int_rn(v * inv);
+        int d0, d1, d2, sum = q;
+        split_digits(q, d0, d1, d2);
+        const int sh = 8 * (lane & 3);
+        int w0 = (d0 & 255) << sh, w1 = (d1 & 255) << sh, w2 = (d2 & 255) << sh;
+        w0 |= dpp_quad_xor1(w0); w0 |= dpp_quad_xor2(w0);
+        w1 |= dpp_quad_xor1(w1); w1 |= dpp_quad_xor2(w1);
+        w2 |= dpp_quad_xor1(w2); w2 |= dpp_quad_xor2(w2);
+        for (int k = 16; k >= 1; k >>= 1) sum += __shfl_xor(sum, k);
+        int *img = reinterpret_cast<int *>(a.act_images) + ((size_t)u * NT + t) * WI;
+        if ((lane & 3) == 0) {
+            const int nn = n0 + lane, at = SEG_STRIDE * (nn >> 6) + ((nn & 63) >> 2);
+            img[at] = w0;
+            img[plane + at] = w1;
+            img[2 * plane + at] = w2;
+        }
+        if (lane == 0) {
+            reinterpret_cast<float *>(img + 3 * plane)[n0 >> 5] = step;
+            img[3 * plane + I / 32 + (n0 >> 5)] = sum;
+        }
+    }
+}
+
+// ---- kernel 3: routed down products and the combine ------------------------------------------
+// block = (token, 16 output rows ... ) with one wave per slot; blockIdx.x = t * row_blocks + nb
+template <int FMT, int NT>
+__global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_blocks, int rows_per_block) {
+    __shared__ float partial[16][64];
+    extern __shared__ int lds[];
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
+    if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
+    const int I = a.inter, H = a.hidden, K = a.top_k, lane = pf_lane(), s = threadIdx.x >> 6;
+    const int t = blockIdx.x / row_blocks, nb = blockIdx.x % row_blocks, P = NT * K;
+    const int LPR = I / 64, rows = 64 / LPR, steps = rows_per_block / rows;
+    const int seg = lane & (LPR - 1), r = lane / LPR;
+    uint32_t e = a.ids[t * K + s], u = a.uniq[1 + P + t * K + s];
+    if (e >= (uint32_t)a.experts || u >= (uint32_t)P) {   // only reachable with nonfinite logits
+        if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+        e = 0;
+        u = 0;
+    }
+    const int n_base = nb * rows_per_block;
+    WSeg<FMT> w[4];
+#pragma unroll
+    for (int st = 0; st < 4; st++)
+        if (st < steps) wseg_load<FMT>(w[st], a, 3, e, min(n_base + st * rows + r, H - 1), seg);
+    XSeg x;
+    xseg_load(x, reinterpret_cast<const int *>(a.act_images) + ((size_t)u * NT + t) * image_words(I), I, seg);
+    if (FMT == PF_IQ2_XXS) __syncthreads();
+#pragma unroll
+    for (int st = 0; st < 4; st++) {
+        if (st >= steps) break;
+        const float v = span_sum(wseg_dot<FMT>(w[st], x, seg, tables), LPR);
+        if (seg == 0) partial[s][st * rows + r] = v;
+    }
+    __syncthreads();
+    const int n = n_base + threadIdx.x;
+    if ((int)threadIdx.x < rows_per_block && n < H) {
+        float sum = 0.0f;
+        for (int slot = 0; slot < K; slot++)   // slot order, as src/qwen4_moe.c:362-372
+            sum += a.route_weights[t * K + slot] * partial[slot][threadIdx.x];
+        const float y = sum + a.shared_scale[t] * a.shared_out[(size_t)t * H + n];
+        a.y[(size_t)t * a.y_pitch + n] = y;
+        if (!pf_finite(y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+    }
+}
+
+// ---- IQ2_XXS upload split -------------------------------------------------------------------------
+__global__ void pf_k_iq2_split(const uint8_t *gguf, uint8_t *payload, uint16_t *scales, size_t blocks) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;   // one 16-bit word of a block per thread
+    const size_t b = i / 33, h = i % 33;
+    if (b >= blocks) return;
+    const uint16_t v = reinterpret_cast<const uint16_t *>(gguf)[b * 33 + h];
+    if (h == 0) scales[b] = v;
+    else reinterpret_cast<uint16_t *>(payload)[b * 32 + (h - 1)] = v;
+}
+
+void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
+                         hipStream_t stream) {
+    const size_t threads = blocks * 33;
+    if (!threads) return;
+    hipLaunchKernelGGL(pf_k_iq2_split, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, d_gguf,
+                       d_payload, d_scales, blocks);
+}
+
+// ---- dispatch ----------------------------------------------------------------------------------------
+static bool pow2_between(uint32_t v, uint32_t lo, uint32_t hi) { return v >= lo && v <= hi && (v & (v - 1)) == 0; }
+
+bool pf_decode_supported(const PfHipMoeDesc &d) {
+    const uint32_t fmt = d.type[1];
+    if (fmt != PF_Q4_K && fmt != PF_IQ2_XXS) return false;
+    for (int j = 1; j <= 6; j++)
+        if (d.type[j] != fmt) return false;
+    if (!pow2_between(d.hidden, 512, 2048) || !pow2_between(d.inter, 256, 2048) ||
+        !pow2_between(d.shared_inter, 256, 2048) || d.down_physical != d.inter)
+        return false;
+    if (d.experts > 1024 || d.top_k > 16 || d.top_k * PF_DECODE_MAX_TOKENS > 64 || d.top_k >= d.experts) return false;
+    return true;
+}
+
+template <int FMT, int NT>
+static void launch_decode(const PfKernelArgs &a, hipStream_t stream, hipEvent_t *marks) {
+    const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
+    const size_t tab = table_words<FMT>() * 4;
+    // kernel 1
+    const int router_blocks = (E + 3) / 4, rph = 32 / (H / 64), shared_blocks = (Is + 8 * rph - 1) / (8 * rph);
+    const size_t lds1 = tab + (size_t)NT * image_words(H) * 4;
+    if (marks) (void)hipEventRecord(marks[0], stream);
+    hipLaunchKernelGGL((pf_k_dec_pre<FMT, NT>), dim3(router_blocks + shared_blocks + 1), dim3(256), lds1, stream, a,
+                       router_blocks, shared_blocks);
+    if (marks) { (void)hipEventRecord(marks[1], stream); (void)hipEventRecord(marks[2], stream); }
+    // kernel 2
+    const int routed_blocks = NT * K * (I / 32), down_rows = 64 / (Is / 64);
+    const int shared_down_blocks = (H + 4 * down_rows - 1) / (4 * down_rows);
+    const size_t img2 = (size_t)NT * image_words(H > Is ? H : Is) * 4, fix = ((size_t)H + 3 * (size_t)E) * 4;
+    const size_t lds2 = tab + img2 + fix;
+    const int npl = (E + 63) / 64;
+    dim3 g2(routed_blocks + shared_down_blocks);
+    static bool big_lds = false;   // once per instantiation: allow more than the default 64 KB of dynamic LDS
+    if (!big_lds) {
+        const int limit = 128 * 1024;
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 2>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 4>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 8>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 16>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_pre<FMT, NT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
+        big_lds = true;
+    }
+    if (npl <= 2) hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 2>), g2, dim3(256), lds2, stream, a, routed_blocks);
+    else if (npl <= 4) hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 4>), g2, dim3(256), lds2, stream, a, routed_blocks);
+    else if (npl <= 8) hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 8>), g2, dim3(256), lds2, stream, a, routed_blocks);
+    else hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 16>), g2, dim3(256), lds2, stream, a, routed_blocks);
+    if (marks) (void)hipEventRecord(marks[3], stream);
+    // kernel 3
+    const int rows = 64 / (I / 64), rows_per_block = 2 * rows > 64 ? 64 : 2 * rows;
+    const int row_blocks = (H + rows_per_block - 1) / rows_per_block;
+    hipLaunchKernelGGL((pf_k_dec_down<FMT, NT>), dim3(NT * row_blocks), dim3(64 * K), tab, stream, a, row_blocks,
+                       rows_per_block);
+    if (marks) (void)hipEventRecord(marks[4], stream);
+}
+
+template <int FMT>
+static void launch_decode_tokens(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks) {
+    switch (tokens) {
+    case 1: launch_decode<FMT, 1>(a, stream, marks); break;
+    case 2: launch_decode<FMT, 2>(a, stream, marks); break;
+    case 3: launch_decode<FMT, 3>(a, stream, marks); break;
+    default: launch_decode<FMT, 4>(a, stream, marks); break;
+    }
+}
+
+void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks) {
+    if (a.type[1] == PF_Q4_K) launch_decode_tokens<PF_Q4_K>(a, tokens, stream, marks);
+    else launch_decode_tokens<PF_IQ2_XXS>(a, tokens, stream, marks);
+}

@@ -3,14 +3,19 @@
 #include "pf_device.h"
 #include "../../include/pf_moe_hip.h"
 
+#define PF_DECODE_MAX_TOKENS 4
+
 // Everything a kernel needs, passed by value.  Weight index order is
 // Qwen4MoeWeights': router, gate, up, down, shared gate/up/down, shared router.
 struct PfKernelArgs {
     int hidden, experts, top_k, inter, shared_inter, down_physical, norm_topk;
     uint32_t type[8];
     const uint8_t *w[8];
-    size_t row_bytes[8], expert_bytes[8];
+    size_t row_bytes[8], expert_bytes[8];   // of the payload (IQ2_XXS: 64 bytes per block)
+    size_t scale_offset[8];                 // IQ2_XXS: byte offset of the half scales in the tensor buffer
+    int k_logical[8], blocks_per_row[8], n_out[8];
     const uint64_t *iq2_grid;        // 256 x 8 magnitudes, device memory
+    const uint32_t *iq2_signed;      // 2 x 4096 words: four signed magnitudes per (grid entry, sign nibble)
     const float *x;                  // [tokens, hidden], pitch in floats
     size_t x_pitch;
     float *y;
@@ -18,9 +23,12 @@ struct PfKernelArgs {
     float *logits, *logit_ssq;       // [tokens, experts]
     uint32_t *ids;                   // [tokens, top_k]
     float *route_weights;            // [tokens, top_k]
-    float *act;                      // [tokens * top_k, inter]
+    float *act;                      // general path [tokens * top_k, inter]; decode path [unique, tokens, inter]
     float *shared_act;               // [tokens, shared_inter]
     float *shared_scale;             // [tokens] sigmoid of the shared router logit
+    float *shared_out;               // [tokens, hidden] shared expert's down product (decode path)
+    int *act_images;                 // decode path: digit image of every [unique, token] activation row
+    uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
     uint32_t *error_word;
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
     uint32_t *route_flags;           // [tokens] 1 = route again in serial order
@@ -29,23 +37,27 @@ struct PfKernelArgs {
 struct PfHipMoe {
     PfHipMoeDesc desc;
     uint8_t *w[8];
-    size_t bytes[8], row_bytes[8], expert_bytes[8];
+    size_t bytes[8], row_bytes[8], expert_bytes[8], scale_offset[8];
+    int k_logical[8], blocks_per_row[8], n_out[8];
     uint64_t *iq2_grid;
+    uint32_t *iq2_signed;
     size_t total_bytes;
+    bool decode_ready;               // shapes and formats the specialised decode kernels cover
 };
 
 struct PfHipWork {
     const PfHipMoe *moe;
     size_t cap, bytes;
-    float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
-    uint32_t *ids, *error_word, *exact_rows, *route_flags;
-    void *host_stage;                // pinned staging for the host-buffer forward
-    size_t host_stage_bytes;
+    float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *shared_out, *x, *y;
+    uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags;
+    int *act_images;
     void *marks;                     // hipEvent_t[5] while stage profiling, else null
+    int force_general;               // tests: run the general kernels even where the decode path applies
 };
 
 // pf_moe_kernels.hip
 void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks);
+size_t pf_general_lds_bytes(const PfKernelArgs &a);
 // pf_moe_route.hip
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream);
 int pf_route_exact_device(const float *d_logits, int tokens, int experts, int top_k, int norm,
@@ -60,6 +72,12 @@ void pf_launch_exact_matmul(uint32_t type, const uint8_t *d_w, size_t row_bytes,
                             hipStream_t stream);
 void pf_launch_exact_decode(uint32_t type, const uint8_t *d_row, int k_storage, float *d_out, uint32_t *d_error,
                             const uint64_t *grid, hipStream_t stream);
+// pf_moe_decode.hip
+bool pf_decode_supported(const PfHipMoeDesc &d);
+void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks);
+void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
+                         hipStream_t stream);
 // pf_moe_api.hip
 const uint64_t *pf_device_iq2_grid(void);
+const uint32_t *pf_device_iq2_signed(void);
 void pf_set_error(const char *what, hipError_t code);

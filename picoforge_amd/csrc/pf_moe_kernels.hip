@@ -1,11 +1,16 @@
 // General MoE kernels for gfx950: any admitted shape and format combination.
 //
 // One wave computes one output row product; activations of the current token
-// are staged in LDS.  These kernels keep GGUF's byte layout.  Shapes that the
-// specialised decode and prefill kernels cover are dispatched there instead.
+// are staged in LDS (zero-padded to the stored row length, so the stored padding
+// of a row multiplies zeros).  Shapes that the specialised decode and prefill
+// kernels cover are dispatched there instead.
+//
+// Device layout of the tensors: F32 and Q4_K keep GGUF's bytes.  IQ2_XXS tensors
+// are split at upload into 64-byte block payloads (all blocks, row-major)
+// followed by the blocks' half scales, so that payload loads are aligned.
 #include "pf_moe_internal.h"
 
-// ---- row products: packed row (GGUF layout) . x (LDS or global) ---------------
+// ---- row products: packed row . x (LDS) -----------------------------------------
 
 __device__ __forceinline__ float dot_row_f32(const uint8_t *row, const float *x, int K, int lane) {
     const float *w = reinterpret_cast<const float *>(row);
@@ -26,8 +31,8 @@ __device__ __forceinline__ float dot_row_f32(const uint8_t *row, const float *x,
 
 // Lane l takes 16 nibble bytes of block l/8: the low nibbles are 16 weights of
 // group 2j, the high nibbles 16 weights of group 2j+1 (j = (l%8)/2).
-__device__ __forceinline__ float dot_row_q4k(const uint8_t *row, const float *x, int K, int lane) {
-    const int nblk = K >> 8, r = lane & 7, j = r >> 1, half = r & 1;
+__device__ __forceinline__ float dot_row_q4k(const uint8_t *row, const float *x, int nblk, int lane) {
+    const int r = lane & 7, j = r >> 1, half = r & 1;
     float acc = 0.0f;
     for (int b = lane >> 3; b < nblk; b += 8) {
         const uint8_t *blk = row + (size_t)b * 144;
@@ -59,18 +64,15 @@ __device__ __forceinline__ float dot_row_q4k(const uint8_t *row, const float *x,
     return acc;
 }
 
-// Lane l takes group l (32 weights, 8 bytes at 2-byte alignment) per pass.
-__device__ __forceinline__ float dot_row_iq2(const uint8_t *row, const float *x, int K, int lane,
-                                             const uint64_t *grid) {
-    const int ngroups = K >> 5;
+// Lane l takes group l (32 weights, one aligned 8-byte payload word) per pass.
+__device__ __forceinline__ float dot_row_iq2(const uint8_t *payload, const uint16_t *scales, const float *x, int nblk,
+                                             int lane, const uint64_t *grid) {
+    const int ngroups = nblk * 8;
     float acc = 0.0f;
     for (int gi = lane; gi < ngroups; gi += PF_WAVE) {
-        const int b = gi >> 3, g = gi & 7;
-        const uint8_t *blk = row + (size_t)b * 66;
-        const uint16_t *p = reinterpret_cast<const uint16_t *>(blk + 2 + 8 * g);
-        const float d = pf_half_bits_to_float(*reinterpret_cast<const uint16_t *>(blk));
-        const uint32_t idx = (uint32_t)p[0] | ((uint32_t)p[1] << 16);
-        const uint32_t word = (uint32_t)p[2] | ((uint32_t)p[3] << 16);
+        const uint2 p = *reinterpret_cast<const uint2 *>(payload + 8 * (size_t)gi);
+        const float d = pf_half_bits_to_float(scales[gi >> 3]);
+        const uint32_t idx = p.x, word = p.y;
         const float scale = d * (float)(2u * (word >> 28) + 1u) * 0.125f;
         const float *xg = x + 32 * gi;
         float gacc = 0.0f;
@@ -91,17 +93,34 @@ __device__ __forceinline__ float dot_row_iq2(const uint8_t *row, const float *x,
     return acc;
 }
 
-__device__ __forceinline__ float dot_row(uint32_t type, const uint8_t *row, const float *x, int K, int lane,
-                                         const uint64_t *grid) {
+// Row n of expert e of tensor t against x (LDS, padded to the stored length).
+__device__ __forceinline__ float dot_tensor_row(const PfKernelArgs &a, int t, size_t e, size_t n, const float *x,
+                                                int lane, const uint64_t *grid) {
+    const uint8_t *row = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t];
     float v;
-    if (type == PF_F32) v = dot_row_f32(row, x, K, lane);
-    else if (type == PF_Q4_K) v = dot_row_q4k(row, x, K, lane);
-    else v = dot_row_iq2(row, x, K, lane, grid);
+    if (a.type[t] == PF_F32) v = dot_row_f32(row, x, a.k_logical[t], lane);
+    else if (a.type[t] == PF_Q4_K) v = dot_row_q4k(row, x, a.blocks_per_row[t], lane);
+    else {
+        const uint16_t *scales = reinterpret_cast<const uint16_t *>(a.w[t] + a.scale_offset[t]) +
+                                 (e * a.n_out[t] + n) * a.blocks_per_row[t];
+        v = dot_row_iq2(row, scales, x, a.blocks_per_row[t], lane, grid);
+    }
     return pf_wave_sum(v);
 }
 
 __device__ __forceinline__ void stage_grid(uint64_t *grid_lds, const uint64_t *grid_global) {
     for (int i = threadIdx.x; i < 256; i += blockDim.x) grid_lds[i] = grid_global[i];
+}
+
+// copies `count` floats and zero-fills up to `padded`
+__device__ __forceinline__ bool stage_row(float *dst, const float *src, int count, int padded) {
+    bool bad = false;
+    for (int k = threadIdx.x; k < padded; k += blockDim.x) {
+        float v = k < count ? src[k] : 0.0f;
+        dst[k] = v;
+        bad |= !pf_finite(v);
+    }
+    return bad;
 }
 
 // ---- stage 1: everything that depends on x only -------------------------------
@@ -111,14 +130,7 @@ __global__ void __launch_bounds__(256) pf_k_pre(PfKernelArgs a) {
     extern __shared__ float lds[];
     __shared__ uint64_t grid[256];
     const int H = a.hidden, t = blockIdx.y, lane = pf_lane(), wave = threadIdx.x >> 6;
-    const float *x = a.x + (size_t)t * a.x_pitch;
-    bool bad = false;
-    for (int k = threadIdx.x; k < H; k += blockDim.x) {
-        float v = x[k];
-        lds[k] = v;
-        bad |= !pf_finite(v);
-    }
-    if (bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+    if (stage_row(lds, a.x + (size_t)t * a.x_pitch, H, H)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     stage_grid(grid, a.iq2_grid);
     __syncthreads();
     const int unit = blockIdx.x * 4 + wave, E = a.experts, Is = a.shared_inter;
@@ -139,15 +151,15 @@ __global__ void __launch_bounds__(256) pf_k_pre(PfKernelArgs a) {
         }
     } else if (unit < E + Is) {
         const int n = unit - E;
-        float g = dot_row(a.type[4], a.w[4] + (size_t)n * a.row_bytes[4], lds, H, lane, grid);
-        float u = dot_row(a.type[5], a.w[5] + (size_t)n * a.row_bytes[5], lds, H, lane, grid);
+        float g = dot_tensor_row(a, 4, 0, n, lds, lane, grid);
+        float u = dot_tensor_row(a, 5, 0, n, lds, lane, grid);
         float v = pf_silu(g) * u;
         if (lane == 0) {
             a.shared_act[(size_t)t * Is + n] = v;
             if (!pf_finite(v)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
         }
     } else if (unit == E + Is) {
-        float z = dot_row(PF_F32, a.w[7], lds, H, lane, grid);
+        float z = dot_tensor_row(a, 7, 0, 0, lds, lane, grid);
         float s = pf_sigmoid(z);
         if (lane == 0) {
             a.shared_scale[t] = s;
@@ -162,8 +174,7 @@ __global__ void __launch_bounds__(256) pf_k_gate_up(PfKernelArgs a) {
     extern __shared__ float lds[];
     __shared__ uint64_t grid[256];
     const int H = a.hidden, pair = blockIdx.y, t = pair / a.top_k, lane = pf_lane(), wave = threadIdx.x >> 6;
-    const float *x = a.x + (size_t)t * a.x_pitch;
-    for (int k = threadIdx.x; k < H; k += blockDim.x) lds[k] = x[k];
+    stage_row(lds, a.x + (size_t)t * a.x_pitch, H, H);
     stage_grid(grid, a.iq2_grid);
     __syncthreads();
     const int n = blockIdx.x * 4 + wave;
@@ -173,10 +184,8 @@ __global__ void __launch_bounds__(256) pf_k_gate_up(PfKernelArgs a) {
         if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
         return;
     }
-    const uint8_t *gate = a.w[1] + (size_t)e * a.expert_bytes[1] + (size_t)n * a.row_bytes[1];
-    const uint8_t *up = a.w[2] + (size_t)e * a.expert_bytes[2] + (size_t)n * a.row_bytes[2];
-    float g = dot_row(a.type[1], gate, lds, H, lane, grid);
-    float u = dot_row(a.type[2], up, lds, H, lane, grid);
+    float g = dot_tensor_row(a, 1, e, n, lds, lane, grid);
+    float u = dot_tensor_row(a, 2, e, n, lds, lane, grid);
     float v = pf_silu(g) * u;
     if (lane == 0) {
         a.act[(size_t)pair * a.inter + n] = v;
@@ -186,16 +195,15 @@ __global__ void __launch_bounds__(256) pf_k_gate_up(PfKernelArgs a) {
 
 // ---- stage 4: routed down products, slot-ordered weighted sum, shared branch ----
 // grid (ceil(hidden/4), tokens).  LDS holds the token's top_k activation rows
-// and its shared activation row.
+// (each padded to the stored row length of the down tensor) and its shared row.
 __global__ void __launch_bounds__(256) pf_k_down_combine(PfKernelArgs a) {
     extern __shared__ float lds[];
     __shared__ uint64_t grid[256];
-    const int I = a.inter, Is = a.shared_inter, K = a.top_k, t = blockIdx.y;
+    const int I = a.inter, Ip = a.down_physical, Is = a.shared_inter, K = a.top_k, t = blockIdx.y;
     const int lane = pf_lane(), wave = threadIdx.x >> 6;
-    const float *act = a.act + (size_t)t * K * I;
-    for (int i = threadIdx.x; i < K * I; i += blockDim.x) lds[i] = act[i];
-    float *sact = lds + K * I;
-    for (int i = threadIdx.x; i < Is; i += blockDim.x) sact[i] = a.shared_act[(size_t)t * Is + i];
+    for (int s = 0; s < K; s++) stage_row(lds + s * Ip, a.act + ((size_t)t * K + s) * I, I, Ip);
+    float *sact = lds + K * Ip;
+    stage_row(sact, a.shared_act + (size_t)t * Is, Is, Is);
     stage_grid(grid, a.iq2_grid);
     __syncthreads();
     const int n = blockIdx.x * 4 + wave;
@@ -207,16 +215,21 @@ __global__ void __launch_bounds__(256) pf_k_down_combine(PfKernelArgs a) {
             if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
             return;
         }
-        const uint8_t *row = a.w[3] + (size_t)e * a.expert_bytes[3] + (size_t)n * a.row_bytes[3];
-        float dsum = dot_row(a.type[3], row, lds + s * I, I, lane, grid);
+        float dsum = dot_tensor_row(a, 3, e, n, lds + s * Ip, lane, grid);
         sum += a.route_weights[(size_t)t * K + s] * dsum;   // slot order, as src/qwen4_moe.c:362-372
     }
-    float sh = dot_row(a.type[6], a.w[6] + (size_t)n * a.row_bytes[6], sact, Is, lane, grid);
+    float sh = dot_tensor_row(a, 6, 0, n, sact, lane, grid);
     float y = sum + a.shared_scale[t] * sh;
     if (lane == 0) {
         a.y[(size_t)t * a.y_pitch + n] = y;
         if (!pf_finite(y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
+}
+
+size_t pf_general_lds_bytes(const PfKernelArgs &a) {
+    const size_t down = ((size_t)a.top_k * a.down_physical + a.shared_inter) * sizeof(float);
+    const size_t x = (size_t)a.hidden * sizeof(float);
+    return down > x ? down : x;
 }
 
 void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks) {
@@ -230,7 +243,7 @@ void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, hi
     if (marks) (void)hipEventRecord(marks[2], stream);
     hipLaunchKernelGGL(pf_k_gate_up, dim3((a.inter + 3) / 4, tokens * a.top_k), dim3(256), x_lds, stream, a);
     if (marks) (void)hipEventRecord(marks[3], stream);
-    const size_t act_lds = ((size_t)a.top_k * a.inter + a.shared_inter) * sizeof(float);
+    const size_t act_lds = ((size_t)a.top_k * a.down_physical + a.shared_inter) * sizeof(float);
     hipLaunchKernelGGL(pf_k_down_combine, dim3((a.hidden + 3) / 4, tokens), dim3(256), act_lds, stream, a);
     if (marks) (void)hipEventRecord(marks[4], stream);
 }

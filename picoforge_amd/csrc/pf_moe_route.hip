@@ -1,148 +1,29 @@
 // Routing (softmax, top-k, renormalisation) and expert grouping kernels.
 //
 // Two routing paths exist.  The fast one keeps a token's logits in the registers
-// of one wave and sums the exponentials with a tree.  It also measures how close
-// the k+1 best logits are; when two of them are closer than the rounding noise a
+// of one wave and selects in logit space.  It also measures how close the k+1
+// best logits are; when two of them are closer than the rounding noise a
 // differently ordered logit sum could have, the token is routed again by the
 // exact path, which recomputes its logits in the reference's serial order
 // (src/qwen4_packed.c:164-179) and follows src/qwen4_moe.c:219-247 step by step.
 #include "pf_moe_internal.h"
-// Reference-order arithmetic: a*b+c must stay two roundings.  HIP's __fmul_rn and
-// __fadd_rn are plain operators compiled with contraction allowed, so they fuse
-// after inlining; the helpers below are compiled with contraction off instead.
-#pragma clang fp contract(off)
-static __device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
-static __device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
-static __device__ __forceinline__ float sub_rn(float a, float b) { return a - b; }
-static __device__ __forceinline__ float div_rn(float a, float b) { return a / b; }
-#include <math.h>
+#include "pf_route_device.h"
+#include "pf_route_fast.h"
 
 #define ROUTE_MAX_FAST_EXPERTS 1024
 
-__device__ __forceinline__ void wave_lds_fence() {
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-}
-
-// (p, id) arg-max over the wave: larger p wins, equal p goes to the lower id,
-// which is what an ascending scan with a strict comparison selects.
-__device__ __forceinline__ void wave_argmax(float &p, uint32_t &id) {
-    for (int m = 1; m < PF_WAVE; m <<= 1) {
-        float op = __shfl_xor(p, m);
-        uint32_t oid = __shfl_xor(id, m);
-        if (op > p || (op == p && oid < id)) { p = op; id = oid; }
-    }
-}
-
-// Reference-order routing of one token by one wave.  z, p, q: LDS arrays of E
-// floats (q is scratch).  Writes ids/weights (top_k entries) and leaves the
-// probabilities in p.
-__device__ void route_exact_wave(const float *z, float *p, float *q, int E, int K, bool norm, uint32_t *ids_out,
-                                 float *w_out, int lane) {
-    float top = -INFINITY;
-    for (int e = lane; e < E; e += PF_WAVE) top = fmaxf(top, z[e]);
-    top = pf_wave_max(top);
-    // exponent in double, rounded once: the correctly rounded expf
-    for (int e = lane; e < E; e += PF_WAVE) p[e] = (float)exp((double)sub_rn(z[e], top));
-    wave_lds_fence();
-    float sum = 0.0f;
-    for (int e = 0; e < E; e++) sum = add_rn(sum, p[e]);   // serial, expert ascending
-    wave_lds_fence();
-    for (int e = lane; e < E; e += PF_WAVE) {
-        float v = div_rn(p[e], sum);
-        p[e] = v;
-        q[e] = v;
-    }
-    wave_lds_fence();
-    float chosen = 0.0f;
-    for (int slot = 0; slot < K; slot++) {
-        float best = -2.0f;
-        uint32_t best_id = 0xffffffffu;
-        for (int e = lane; e < E; e += PF_WAVE) {
-            float v = q[e];
-            if (v > best) { best = v; best_id = (uint32_t)e; }
-        }
-        wave_argmax(best, best_id);
-        if ((int)(best_id & (PF_WAVE - 1)) == lane) q[best_id] = -1.0f;
-        wave_lds_fence();
-        chosen = add_rn(chosen, best);
-        if (lane == 0) { ids_out[slot] = best_id; w_out[slot] = best; }
-    }
-    if (norm && lane == 0)
-        for (int slot = 0; slot < K; slot++) w_out[slot] = div_rn(w_out[slot], chosen);
-}
-
-// ---- fast routing inside a forward --------------------------------------------
+// ---- fast routing inside a forward (general path) --------------------------------
 template <int NPL>
 __global__ void __launch_bounds__(64) pf_k_route_fast(PfKernelArgs a) {
     const int t = blockIdx.x, lane = threadIdx.x, E = a.experts, K = a.top_k;
-    const float *zr = a.logits + (size_t)t * E, *sr = a.logit_ssq + (size_t)t * E;
-    float z[NPL], s2[NPL], p[NPL];
-    float top = -INFINITY;
-    bool bad = false;
-#pragma unroll
-    for (int i = 0; i < NPL; i++) {
-        const int e = lane + PF_WAVE * i;
-        const bool in = e < E;
-        z[i] = in ? zr[e] : -INFINITY;
-        s2[i] = in ? sr[e] : 0.0f;
-        bad |= in && !pf_finite(z[i]);
-        top = fmaxf(top, z[i]);
-    }
-    if (bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-    top = pf_wave_max(top);
-    float sum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < NPL; i++) {
-        p[i] = (lane + PF_WAVE * i < E) ? expf(z[i] - top) : -1.0f;
-        sum += fmaxf(p[i], 0.0f);
-    }
-    sum = pf_wave_sum(sum);
-#pragma unroll
-    for (int i = 0; i < NPL; i++) if (p[i] >= 0.0f) p[i] = p[i] / sum;
-    // k rounds, plus one more to see the runner-up's logit
-    const int rounds = K < E ? K + 1 : K;
-    float chosen = 0.0f, prev_z = 0.0f, prev_s2 = 0.0f, my_w = 0.0f;
-    uint32_t my_id = 0;
-    bool close = false;
-    for (int r = 0; r < rounds; r++) {
-        float best = -2.0f;
-        uint32_t best_id = 0xffffffffu;
-#pragma unroll
-        for (int i = 0; i < NPL; i++)
-            if (p[i] > best) { best = p[i]; best_id = (uint32_t)(lane + PF_WAVE * i); }
-        wave_argmax(best, best_id);
-        const int owner = best_id & (PF_WAVE - 1), slot_i = best_id >> 6;
-        float zo = 0.0f, so = 0.0f;
-#pragma unroll
-        for (int i = 0; i < NPL; i++)
-            if (i == slot_i) {
-                zo = z[i];
-                so = s2[i];
-                if (lane == owner) p[i] = -1.0f;
-            }
-        zo = __shfl(zo, owner);
-        so = __shfl(so, owner);
-        if (r > 0) {
-            // Noise model of a K-term FP32 sum in any order: standard deviation
-            // u * sqrt(K * sum(products^2) / 6); eight of those per logit, plus the
-            // rounding of z - max and of the exponential.
-            const float u = 5.9604645e-8f, hk = (float)a.hidden / 6.0f;
-            float tol = 8.0f * u * (sqrtf(hk * so) + sqrtf(hk * prev_s2)) + 4e-6f * fmaxf(1.0f, top - zo);
-            close |= !(prev_z - zo > tol);
-        }
-        prev_z = zo;
-        prev_s2 = so;
-        if (r < K) {
-            chosen += best;
-            if (lane == r) { my_id = best_id; my_w = best; }   // top_k <= 64: lane s keeps slot s
-        }
-    }
+    PfRouteResult r = pf_route_fast_wave<NPL>(a.logits + (size_t)t * E, a.logit_ssq + (size_t)t * E, E, K,
+                                              a.norm_topk != 0, a.hidden, lane);
+    if (r.bad && lane == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     if (lane < K) {
-        a.ids[(size_t)t * K + lane] = my_id;
-        a.route_weights[(size_t)t * K + lane] = a.norm_topk ? my_w / chosen : my_w;
+        a.ids[(size_t)t * K + lane] = r.id;
+        a.route_weights[(size_t)t * K + lane] = r.weight;
     }
-    if (lane == 0) a.route_flags[t] = close ? 1u : 0u;
+    if (lane == 0) a.route_flags[t] = r.close ? 1u : 0u;
 }
 
 // Serial-order recomputation for flagged tokens: thread e owns expert e.
@@ -155,16 +36,14 @@ __global__ void __launch_bounds__(256) pf_k_route_fix(PfKernelArgs a) {
     for (int k = threadIdx.x; k < H; k += blockDim.x) xs[k] = x[k];
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
-        const float *w = reinterpret_cast<const float *>(a.w[0]) + (size_t)e * H;
-        float sum = 0.0f;
-        for (int k = 0; k < H; k++) sum = add_rn(sum, mul_rn(w[k], xs[k]));
+        const float sum = pf_serial_logit(reinterpret_cast<const float *>(a.w[0]) + (size_t)e * H, xs, H);
         z[e] = sum;
         a.logits[(size_t)t * E + e] = sum;
     }
     __syncthreads();
     if (threadIdx.x < PF_WAVE) {
-        route_exact_wave(z, p, q, E, a.top_k, a.norm_topk != 0, a.ids + (size_t)t * a.top_k,
-                         a.route_weights + (size_t)t * a.top_k, threadIdx.x);
+        pf_route_exact_wave(z, p, q, E, a.top_k, a.norm_topk != 0, a.ids + (size_t)t * a.top_k,
+                            a.route_weights + (size_t)t * a.top_k, threadIdx.x);
         if (threadIdx.x == 0) atomicAdd(a.exact_rows, 1u);
     }
 }
@@ -176,10 +55,9 @@ __global__ void pf_k_flag_all(uint32_t *flags, int n) {
 }
 
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
-    uint32_t *flags = a.route_flags;
     const int npl = (a.experts + PF_WAVE - 1) / PF_WAVE;
-    if (a.experts > ROUTE_MAX_FAST_EXPERTS || a.top_k > PF_WAVE)
-        hipLaunchKernelGGL(pf_k_flag_all, dim3((tokens + 255) / 256), dim3(256), 0, stream, flags, tokens);
+    if (a.experts > ROUTE_MAX_FAST_EXPERTS || a.top_k >= PF_WAVE)
+        hipLaunchKernelGGL(pf_k_flag_all, dim3((tokens + 255) / 256), dim3(256), 0, stream, a.route_flags, tokens);
     else if (npl <= 1) hipLaunchKernelGGL(pf_k_route_fast<1>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 2) hipLaunchKernelGGL(pf_k_route_fast<2>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 4) hipLaunchKernelGGL(pf_k_route_fast<4>, dim3(tokens), dim3(64), 0, stream, a);
@@ -204,9 +82,8 @@ __global__ void __launch_bounds__(64) pf_k_route_exact(const float *logits, int 
     const int t = blockIdx.x, lane = threadIdx.x;
     float *z = lds, *p = z + E, *q = p + E;
     for (int e = lane; e < E; e += PF_WAVE) z[e] = logits[(size_t)t * E + e];
-    wave_lds_fence();
-    route_exact_wave(z, p, q, E, K, norm != 0, ids + (size_t)t * K, weights + (size_t)t * K, lane);
-    wave_lds_fence();
+    pf_wave_lds_fence();
+    pf_route_exact_wave(z, p, q, E, K, norm != 0, ids + (size_t)t * K, weights + (size_t)t * K, lane);
     for (int e = lane; e < E; e += PF_WAVE) probs[(size_t)t * E + e] = p[e];
 }
 

@@ -156,6 +156,9 @@ void qwen4_moe_work_destroy(Qwen4MoeWork *w) {
     if (w && !w->busy) { pf_hip_work_destroy(w->device); moe_unref(w->owner); free(w); }
 }
 
+PfHipMoe *pf_moe_device_layer(const Qwen4Moe *m) { return m ? m->device : NULL; }
+PfHipWork *pf_moe_device_work(Qwen4MoeWork *w) { return w ? w->device : NULL; }
+
 void qw4_moe_observe(Qwen4MoeWork *w, QW4MoeObserver fn, void *ctx) {
     if (w && !w->busy) { w->observer = fn; w->observer_ctx = ctx; }
 }

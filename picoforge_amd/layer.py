@@ -95,6 +95,19 @@ class MoeLayer:
             self._raise(st)
         return st, y, ids, w
 
+    def device_handles(self):
+        """(PfHipMoe*, PfHipWork*) behind this layer: shipped library only."""
+        return self.api.device_layer(self.handle), self.api.device_work(self.work)
+
+    def force_general(self, on=True):
+        """Route every batch size through the general kernels (tests of both kernel families)."""
+        self.api.hip.work_force_general(self.api.device_work(self.work), 1 if on else 0)
+
+    def serial_order_reroutes(self):
+        count = C.c_uint32()
+        self.api.hip.work_exact_rows(self.api.device_work(self.work), C.byref(count))
+        return count.value
+
     def reset(self):
         return self.api.work_reset(self.work, C.byref(self.err))
 
