@@ -40,7 +40,8 @@ WORKLOADS = {
     "q4k_decode": dict(type=abi.GGUF_Q4_K, tokens=1, label="Q4_K experts, decode batch 1"),
     "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
 }
-STAGES = ["router+shared_gate_up", "route", "routed_gate_up", "down+combine"]
+STAGES = ["pf_k_dec_pre (router logits, shared gate/up)", "pf_k_dec_gate_up (routing, routed gate/up, shared down)",
+          "pf_k_dec_down (routed down, combine)"]
 
 
 def device_forward_sample(api, layer, x, tokens):
@@ -85,15 +86,7 @@ def main():
     prep_s = time.time() - t0
 
     layer = pf.MoeLayer(api, cfg, weights, tokens)
-    # device-resident handles of the same layer for the timed loop
-    desc = pf.binding.PfHipMoeDesc(cfg.hidden_size, cfg.experts, cfg.top_k, cfg.intermediate, cfg.shared_intermediate,
-                                   cfg.down_physical, 1)
-    desc.type[:] = weights.types
-    ptrs = (C.c_void_p * 8)(*[w.ctypes.data for w in weights.raw])
-    sizes = (C.c_size_t * 8)(*[w.size for w in weights.raw])
-    moe, work = C.c_void_p(), C.c_void_p()
-    hip.check(hip.moe_create(C.byref(desc), ptrs, sizes, C.byref(moe)), "moe_create")
-    hip.check(hip.work_create(moe, tokens, C.byref(work)), "work_create")
+    moe, work = layer.device_handles()     # the layer's HBM-resident tensors and scratch, for the timed loop
     d_x = hip.to_device(x)
     d_y = hip.to_device(np.zeros((tokens, cfg.hidden_size), dtype=np.float32))
 
@@ -110,19 +103,24 @@ def main():
     exact = C.c_uint32()
     hip.work_exact_rows(work, C.byref(exact))
 
+    # Per-kernel durations: HIP events on the launch stream around each of the three decode
+    # kernels, minus the same measurement of an empty kernel (the fixed dispatch cost).
     stage = (C.c_float * 4)()
     hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(args.steps, 500), stage), "stages")
-    stage_us = [float(v) * 1e3 for v in stage]
+    empty = C.c_float()
+    hip.check(hip.event_overhead(200, C.byref(empty)), "event overhead")
+    overhead_us = float(empty.value) * 1e3
+    raw_us = [float(stage[0]) * 1e3, float(stage[2]) * 1e3, float(stage[3]) * 1e3]
+    stage_us = [max(v - overhead_us, 0.05) for v in raw_us]
 
     alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique)
-    # dominant kernel: routed gate/up + SwiGLU reads 2/3 of the selected experts' bytes
     block, size = abi.BLOCK[wl["type"]]
-    gate_up_bytes = unique * 2 * cfg.intermediate * cfg.hidden_size // block * size
-    dom = int(np.argmax(stage_us))
-    stage_bytes = [(cfg.experts + 1) * cfg.hidden_size * 4 + 2 * cfg.shared_intermediate * cfg.hidden_size // block * size,
-                   tokens * cfg.experts * 8,
-                   gate_up_bytes,
-                   (unique + 1) * cfg.hidden_size * cfg.intermediate // block * size]
+    h, i, s_i = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate
+    # algorithmic bytes per launch: what each kernel must read once
+    stage_bytes = [(cfg.experts + 1) * h * 4 + 2 * s_i * h // block * size,
+                   unique * 2 * i * h // block * size + h * s_i // block * size,
+                   unique * h * i // block * size]
+    dom = int(np.argmax(stage_bytes))
     achieved = stage_bytes[dom] / (stage_us[dom] * 1e-6) / 1e9
 
     # CPU baseline and parity on a bounded sample of the same inputs
@@ -159,7 +157,9 @@ def main():
         "roofline": {"bound": "hbm", "kernel": STAGES[dom], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "bytes_per_launch": int(stage_bytes[dom]), "us_per_launch": round(stage_us[dom], 3)},
-        "stage_us": dict(zip(STAGES, [round(v, 3) for v in stage_us])),
+        "kernel_us": dict(zip(STAGES, [round(v, 3) for v in stage_us])),
+        "kernel_bytes": dict(zip(STAGES, [int(b) for b in stage_bytes])),
+        "event_overhead_us": round(overhead_us, 3),
         "cpu_baseline": {"value": round(cpu_s / (sample * tokens) * 1e6, 1), "unit": "us/layer/token", "cores": 1,
                          "kind": kind, "sample": f"first {sample} steps ({sample * tokens} tokens) of the same inputs, "
                                                    f"{cpu_s:.1f} s"},

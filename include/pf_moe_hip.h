@@ -140,6 +140,11 @@ int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float 
                               size_t n_inputs, float *d_y, size_t tokens, size_t iters,
                               float stage_ms[4]);
 
+/* Average milliseconds between two events recorded around an empty kernel, measured
+ * the way pf_hip_moe_profile_stages measures a stage: the fixed cost inside every
+ * stage time. */
+int pf_hip_event_overhead(size_t iters, float *ms_per_kernel);
+
 #ifdef __cplusplus
 }
 #endif

@@ -162,7 +162,7 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
 extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_bytes : 0; }
 
 // workspace layout: buffers carved from one allocation, each 256-byte aligned
-enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_SOUT, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS,
+enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_SIMAGES, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS,
        W_IMAGES, W_COUNT };
 struct Carve { size_t offset[W_COUNT], total; };
 static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
@@ -178,7 +178,7 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_ACT] = (T * K > Td * K * Td ? T * K : Td * K * Td) * I * 4;
     want[W_SACT] = T * d->shared_inter * 4;
     want[W_SSCALE] = T * 4;
-    want[W_SOUT] = Td * H * 4;
+    want[W_SIMAGES] = Td * (3 * 20 * ((d->shared_inter + 63) / 64) + 2 * ((d->shared_inter + 31) / 32)) * 4;
     want[W_X] = T * H * 4;
     want[W_Y] = T * H * 4;
     want[W_IDS] = T * K * 4;
@@ -220,7 +220,7 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     w->act = (float *)(base + c.offset[W_ACT]);
     w->shared_act = (float *)(base + c.offset[W_SACT]);
     w->shared_scale = (float *)(base + c.offset[W_SSCALE]);
-    w->shared_out = (float *)(base + c.offset[W_SOUT]);
+    w->shared_images = (int *)(base + c.offset[W_SIMAGES]);
     w->x = (float *)(base + c.offset[W_X]);
     w->y = (float *)(base + c.offset[W_Y]);
     w->ids = (uint32_t *)(base + c.offset[W_IDS]);
@@ -257,6 +257,14 @@ extern "C" int pf_hip_work_clear_status(PfHipWork *w) {
     return PF_HIP_OK;
 }
 
+#ifdef PF_TIMING
+extern "C" int pf_hip_debug_read(PfHipWork *w, void *out, size_t bytes) {
+    HIP_TRY(hipDeviceSynchronize());
+    HIP_TRY(hipMemcpy(out, w->exact_rows, bytes, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+#endif
+
 extern "C" void pf_hip_work_force_general(PfHipWork *w, int on) { if (w) w->force_general = on; }
 
 static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x, size_t x_pitch, float *d_y,
@@ -280,8 +288,8 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.iq2_signed = m->iq2_signed;
     a.x = d_x; a.x_pitch = x_pitch; a.y = d_y; a.y_pitch = y_pitch;
     a.logits = w->logits; a.logit_ssq = w->logit_ssq; a.ids = w->ids; a.route_weights = w->route_weights;
-    a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale; a.shared_out = w->shared_out;
-    a.act_images = w->act_images; a.uniq = w->uniq;
+    a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale;
+    a.act_images = w->act_images; a.shared_images = w->shared_images; a.uniq = w->uniq;
     a.error_word = w->error_word; a.exact_rows = w->exact_rows; a.route_flags = w->route_flags;
     return a;
 }
@@ -538,6 +546,38 @@ extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, co
     free(execs);
     if (t0) (void)hipEventDestroy(t0);
     if (t1) (void)hipEventDestroy(t1);
+    (void)hipStreamDestroy(s);
+    return rc;
+}
+
+__global__ void pf_k_nothing(uint32_t *p) { if (p && threadIdx.x == 0xffffffffu) *p = 0; }
+
+// Average time between two events recorded around an empty kernel, measured the same way
+// pf_hip_moe_profile_stages measures a stage: the fixed cost to subtract from a stage time
+// to estimate the kernel's own duration.
+extern "C" int pf_hip_event_overhead(size_t iters, float *ms_per_kernel) {
+    if (!ms_per_kernel || !iters) return PF_HIP_E_ARGUMENT;
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
+    hipStream_t s = nullptr;
+    hipEvent_t a = nullptr, b = nullptr;
+    HIP_TRY(hipStreamCreate(&s));
+    HIP_TRY(hipEventCreate(&a));
+    HIP_TRY(hipEventCreate(&b));
+    float total = 0.0f;
+    int rc = PF_HIP_OK;
+    for (size_t i = 0; i < iters + 3 && rc == PF_HIP_OK; i++) {
+        float ms = 0.0f;
+        hipError_t e = hipEventRecord(a, s);
+        hipLaunchKernelGGL(pf_k_nothing, dim3(256), dim3(256), 0, s, (uint32_t *)nullptr);
+        if (e == hipSuccess) e = hipEventRecord(b, s);
+        if (e == hipSuccess) e = hipStreamSynchronize(s);
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, a, b);
+        if (e != hipSuccess) { pf_set_error("event overhead", e); rc = PF_HIP_E_RUNTIME; }
+        if (i >= 3) total += ms;
+    }
+    *ms_per_kernel = total / (float)iters;
+    (void)hipEventDestroy(a);
+    (void)hipEventDestroy(b);
     (void)hipStreamDestroy(s);
     return rc;
 }

@@ -1,10 +1,12 @@
 // Decode path: 1..4 tokens through one MoE layer as three dependent kernels.
 //
-//   pf_k_dec_pre      router logits (F32 rows), shared gate/up + SwiGLU, shared router
-//   pf_k_dec_gate_up  routing (every workgroup repeats it from the logits), the union
-//                     of the tokens' experts, routed gate/up + SwiGLU once per unique
-//                     expert, and the shared expert's down product
-//   pf_k_dec_down     routed down products, slot-ordered weighted sum, shared branch
+//   pf_k_dec_router   router logits (F32 rows) and the shared router's sigmoid
+//   pf_k_dec_gate_up  routing (every workgroup repeats it from the logits: candidate
+//                     lists by several waves, merged by one), the union of the tokens'
+//                     experts, gate/up + SwiGLU once per unique routed expert and for
+//                     the shared expert, activations written as FP32 and as digit images
+//   pf_k_dec_down     down products of the routed slots and of the shared expert (one
+//                     wave each), slot-ordered weighted sum, shared branch added last
 //
 // A dependent kernel boundary costs about 1.6 us on this GPU when replayed from a
 // graph; an in-kernel barrier across its eight L2 domains costs more, so the three
@@ -21,6 +23,11 @@
 #include "pf_route_device.h"
 #include "pf_route_fast.h"
 
+#ifdef PF_TIMING
+#define STAMP(i) do { if (blockIdx.x == PF_TIMING && threadIdx.x == 0) reinterpret_cast<unsigned long long *>(a.exact_rows + 2)[i] = wall_clock64(); } while (0)
+#else
+#define STAMP(i) do {} while (0)
+#endif
 #define SEG_STRIDE 20   // dwords per 64-value segment of a digit plane (16 used): spreads LDS banks
 
 // ---- digit images --------------------------------------------------------------------
@@ -72,10 +79,13 @@ __device__ __forceinline__ void split_digits(int q, int &d0, int &d1, int &d2) {
 
 // All threads of the workgroup: image of src[0..K) (K % 32 == 0).  Thread j takes the
 // eight values 8j..8j+7; four neighbouring threads form one 32-group.
-__device__ __forceinline__ bool build_image(int *img, const float *src, int K) {
+__device__ __forceinline__ bool build_image(int *img, const float *src, int K, int first_thread = 0,
+                                            int thread_count = 1 << 30) {
     const int plane = SEG_STRIDE * (K / 64);
     bool bad = false;
-    for (int j = threadIdx.x; j < K / 8; j += blockDim.x) {
+    const int j0 = (int)threadIdx.x - first_thread, stride = min(thread_count, (int)blockDim.x - first_thread);
+    if (j0 < 0 || j0 >= stride) return false;
+    for (int j = j0; j < K / 8; j += stride) {
         const float4 a = reinterpret_cast<const float4 *>(src)[2 * j];
         const float4 b = reinterpret_cast<const float4 *>(src)[2 * j + 1];
         const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -209,8 +219,13 @@ __device__ __forceinline__ float wseg_dot<PF_IQ2_XXS>(const WSeg<PF_IQ2_XXS> &w,
 }
 
 // sum over `width` neighbouring lanes (power of two, <= 32); result in the lowest lane of each span
+// (width is uniform; the DPP steps leave the span total in every lane of the span)
 __device__ __forceinline__ float span_sum(float v, int width) {
-    for (int m = width >> 1; m >= 1; m >>= 1) v += __shfl_xor(v, m);
+    if (width >= 2) v = pf_dpp_add(v, 0);    // quad_perm [1,0,3,2]
+    if (width >= 4) v = pf_dpp_add(v, 1);    // quad_perm [2,3,0,1]
+    if (width >= 8) v = pf_dpp_add(v, 2);    // row_half_mirror
+    if (width >= 16) v = pf_dpp_add(v, 3);   // row_mirror
+    if (width >= 32) v += __shfl_xor(v, 16);
     return v;
 }
 
@@ -222,84 +237,61 @@ __device__ __forceinline__ void stage_tables(uint32_t *lds, const uint32_t *glob
 
 template <int FMT> __host__ __device__ constexpr int table_words() { return FMT == PF_IQ2_XXS ? 8192 : 0; }
 
-// ---- kernel 1: everything that depends on x only -------------------------------------------
-// blocks [0, router_blocks): one router row per wave, all tokens;
-// blocks [router_blocks, +shared_blocks): shared gate/up rows; last block: shared router row.
-template <int FMT, int NT>
-__global__ void __launch_bounds__(256) pf_k_dec_pre(PfKernelArgs a, int router_blocks, int shared_blocks) {
-    extern __shared__ int lds[];
+// ---- kernel 1: router logits -----------------------------------------------------------------
+// One F32 row per wave, all tokens: blocks [0, router_blocks) take the experts' rows, the
+// last block's first wave the shared router row (its sigmoid scales the shared expert).
+template <int NT>
+__global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks) {
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
-    if ((int)blockIdx.x < router_blocks || (int)blockIdx.x == router_blocks + shared_blocks) {
-        const bool gate_row = (int)blockIdx.x == router_blocks + shared_blocks;
-        const int e = blockIdx.x * 4 + wave;
-        if (gate_row ? wave != 0 : e >= E) return;
-        const float4 *w = reinterpret_cast<const float4 *>(gate_row ? a.w[7] : a.w[0] + (size_t)e * H * 4);
-        float acc[NT], sq[NT];
-        bool bad = false;
+    const bool gate_row = (int)blockIdx.x == router_blocks;
+    const int e = blockIdx.x * 4 + wave;
+    if (gate_row ? wave != 0 : e >= E) return;
+    const float4 *w = reinterpret_cast<const float4 *>(gate_row ? a.w[7] : a.w[0] + (size_t)e * H * 4);
+    float acc[NT], sq[NT];
+    bool bad = false;
 #pragma unroll
-        for (int t = 0; t < NT; t++) acc[t] = sq[t] = 0.0f;
-        for (int i = lane; i < H / 4; i += PF_WAVE) {
-            const float4 wv = w[i];
+    for (int t = 0; t < NT; t++) acc[t] = sq[t] = 0.0f;
+    // the whole row (hidden <= 2048: eight 16-byte chunks per lane) is requested before any use
+    float4 wv[8];
 #pragma unroll
-            for (int t = 0; t < NT; t++) {
-                const float4 xv = reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch)[i];
-                const float p0 = wv.x * xv.x, p1 = wv.y * xv.y, p2 = wv.z * xv.z, p3 = wv.w * xv.w;
-                acc[t] += (p0 + p1) + (p2 + p3);
-                sq[t] = fmaf(p0, p0, fmaf(p1, p1, fmaf(p2, p2, fmaf(p3, p3, sq[t]))));
-                bad |= !pf_finite(xv.x) || !pf_finite(xv.y) || !pf_finite(xv.z) || !pf_finite(xv.w);
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const float z = pf_wave_sum(acc[t]), s2 = pf_wave_sum(sq[t]);
-            if (lane == 0) {
-                if (gate_row) {
-                    a.shared_scale[t] = pf_sigmoid(z);
-                    if (!pf_finite(z)) bad = true;
-                } else {
-                    a.logits[(size_t)t * E + e] = z;
-                    a.logit_ssq[(size_t)t * E + e] = s2;
-                }
-            }
-        }
-        if (__any(bad) && lane == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-        return;
-    }
-    // shared gate/up: lower half of the wave takes gate rows, upper half up rows
-    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
-    int *images = lds + table_words<FMT>();
-    if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
-    const int W = image_words(H);
-    for (int t = 0; t < NT; t++) build_image(images + t * W, a.x + (size_t)t * a.x_pitch, H);
-    __syncthreads();
-    const int LPR = H / 64, RPH = 32 / LPR, Is = a.shared_inter;
-    const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
-    const int base = ((blockIdx.x - router_blocks) * 4 + wave) * 2 * RPH;
-    WSeg<FMT> w[2];
-#pragma unroll
-    for (int s = 0; s < 2; s++) {
-        const int n = min(base + s * RPH + r, Is - 1);
-        wseg_load<FMT>(w[s], a, 4 + half, 0, n, seg);
+    for (int c = 0; c < 8; c++) {
+        const int i = lane + PF_WAVE * c;
+        wv[c] = i < H / 4 ? w[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        XSeg x;
-        xseg_load(x, images + t * W, H, seg);
+        float4 xv[8];
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            const int n = base + s * RPH + r;
-            float v = span_sum(wseg_dot<FMT>(w[s], x, seg, tables), LPR);
-            const float u = __shfl(v, (lane & 31) + 32);
-            if (half == 0 && seg == 0 && n < Is) {
-                const float act = pf_silu(v) * u;
-                a.shared_act[(size_t)t * Is + n] = act;
-                if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        for (int c = 0; c < 8; c++) {
+            const int i = lane + PF_WAVE * c;
+            xv[c] = i < H / 4 ? reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch)[i]
+                              : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const float p0 = wv[c].x * xv[c].x, p1 = wv[c].y * xv[c].y, p2 = wv[c].z * xv[c].z, p3 = wv[c].w * xv[c].w;
+            acc[t] += (p0 + p1) + (p2 + p3);
+            sq[t] = fmaf(p0, p0, fmaf(p1, p1, fmaf(p2, p2, fmaf(p3, p3, sq[t]))));
+            bad |= !pf_finite(xv[c].x) || !pf_finite(xv[c].y) || !pf_finite(xv[c].z) || !pf_finite(xv[c].w);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        const float z = pf_wave_sum(acc[t]), s2 = pf_wave_sum(sq[t]);
+        if (lane == 0) {
+            if (gate_row) {
+                a.shared_scale[t] = pf_sigmoid(z);
+                if (!pf_finite(z)) bad = true;
+            } else {
+                a.logits[(size_t)t * E + e] = z;
+                a.logit_ssq[(size_t)t * E + e] = s2;
             }
         }
     }
+    if (__any(bad) && lane == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
 }
 
-// ---- kernel 2: routing, expert union, routed gate/up, shared down --------------------------
+// ---- kernel 2: routing, expert union, gate/up + SwiGLU of the routed and the shared expert ------
 struct RouteLds {
     uint32_t ids[64];        // [token][slot]
     float weights[64];
@@ -307,33 +299,26 @@ struct RouteLds {
     uint32_t pair_slot[64];  // pair -> index into uniq
     uint32_t mask[64];       // unique -> bit t set when token t uses it
     uint32_t count, close_mask, bad;
+    uint32_t close[PF_DECODE_MAX_TOKENS], nonfinite[PF_DECODE_MAX_TOKENS];
     float tile[PF_DECODE_MAX_TOKENS][32];
+    PfRouteCands cands[PF_DECODE_MAX_TOKENS];
 };
 
-template <int NPL>
-__device__ __forceinline__ void route_tokens(const PfKernelArgs &a, RouteLds *R, float *scratch, int tokens) {
+// Entered by the whole block after the fast routing: reference-order routing of the
+// ambiguous tokens (rare), then the union of the tokens' experts.  Ends with a block barrier.
+template <int NT>
+__device__ __forceinline__ void route_finish(const PfKernelArgs &a, RouteLds *R, float *scratch) {
     const int lane = pf_lane(), wave = threadIdx.x >> 6, E = a.experts, K = a.top_k;
-    if (threadIdx.x == 0) { R->close_mask = 0; R->bad = 0; }
-    __syncthreads();
-    if (wave < tokens) {
-        PfRouteResult r = pf_route_fast_wave<NPL>(a.logits + (size_t)wave * E, a.logit_ssq + (size_t)wave * E, E, K,
-                                                  a.norm_topk != 0, a.hidden, lane);
-        if (lane < K) {
-            R->ids[wave * K + lane] = r.id;
-            R->weights[wave * K + lane] = r.weight;
-        }
-        if (lane == 0) {
-            if (r.close) atomicOr(&R->close_mask, 1u << wave);
-            if (r.bad) R->bad = 1;
-        }
+    uint32_t close = 0, bad = 0;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        close |= R->close[t] << t;
+        bad |= R->nonfinite[t];
     }
-    __syncthreads();
-    const uint32_t close = R->close_mask;
     if (close) {
-        // reference-order logits and routing for the ambiguous tokens (rare)
         const int H = a.hidden;
         float *xs = scratch, *z = xs + H, *p = z + E, *q = p + E;
-        for (int t = 0; t < tokens; t++) {
+        for (int t = 0; t < NT; t++) {
             if (!((close >> t) & 1u)) continue;
             for (int k = threadIdx.x; k < H; k += blockDim.x) xs[k] = a.x[(size_t)t * a.x_pitch + k];
             __syncthreads();
@@ -344,121 +329,130 @@ __device__ __forceinline__ void route_tokens(const PfKernelArgs &a, RouteLds *R,
             __syncthreads();
         }
     }
-    // union of the tokens' experts in first-use order (pairs <= 64)
     if (wave == 0) {
-        const int P = tokens * K;
-        const uint32_t id = lane < P ? R->ids[lane] : 0xffffffffu;
-        bool first = lane < P;
-        for (int q = 0; q < P; q++) {
-            const uint32_t other = __shfl(id, q);
-            if (q < lane && other == id) first = false;
-        }
-        const unsigned long long firsts = __ballot(first);
-        const uint32_t my_index = __popcll(firsts & ((1ull << lane) - 1ull));
-        uint32_t slot = my_index, mask = 0;
-        for (int q = 0; q < P; q++) {
-            const uint32_t other = __shfl(id, q), other_index = __shfl(my_index, q);
-            const bool other_first = (firsts >> q) & 1ull;
-            if (other == id) {
-                if (other_first) slot = other_index;
-                mask |= 1u << (q / K);
+        const int P = NT * K;
+        if (NT == 1) {
+            if (lane < P) { R->uniq[lane] = R->ids[lane]; R->pair_slot[lane] = lane; R->mask[lane] = 1u; }
+            if (lane == 0) R->count = P;
+        } else {
+            // first-use order: pair p is a first use when no earlier pair names its expert
+            const uint32_t id = lane < P ? R->ids[lane] : 0xffffffffu;
+            int first_at = lane;
+            uint32_t mask = 0;
+            for (int q = P - 1; q >= 0; q--) {
+                if (R->ids[q] == id) { first_at = q; mask |= 1u << (q / K); }
             }
+            const bool first = lane < P && first_at == lane;
+            const unsigned long long firsts = __ballot(first);
+            const uint32_t slot = __popcll(firsts & ((1ull << first_at) - 1ull));
+            if (lane < P) R->pair_slot[lane] = slot;
+            if (first) { R->uniq[slot] = id; R->mask[slot] = mask; }
+            if (lane == 0) R->count = __popcll(firsts);
         }
-        if (lane < P) R->pair_slot[lane] = slot;
-        if (first) { R->uniq[my_index] = id; R->mask[my_index] = mask; }
-        if (lane == 0) R->count = __popcll(firsts);
+        if (lane == 0) { R->close_mask = close; R->bad = bad; }
     }
     __syncthreads();
 }
 
+// 1024 threads.  Routed block b: unique slot b / tiles, units [32 * (b % tiles), +32) of that
+// expert; shared blocks follow.  Every wave owns two units (a unit = gate row + up row:
+// lower half-wave the gate row, upper half-wave the up row).  Waves 0..parts*NT-1 first
+// reduce the logits to candidates, waves 12..15 turn the activations into digit images.
 template <int FMT, int NT, int NPL>
-__global__ void __launch_bounds__(256) pf_k_dec_gate_up(PfKernelArgs a, int routed_blocks) {
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int routed_blocks, int parts, int chunk) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
-    const int H = a.hidden, I = a.inter, K = a.top_k, lane = pf_lane(), wave = threadIdx.x >> 6;
+    const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
     int *images = lds + table_words<FMT>();
+    const int W = image_words(H), P = NT * K;
+    const bool shared = (int)blockIdx.x >= routed_blocks;
+    STAMP(0);
     if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
-
-    if ((int)blockIdx.x >= routed_blocks) {
-        // shared expert's down product: shared_out[t][n] = shared_down[n] . shared_act[t]
-        const int Is = a.shared_inter, W = image_words(Is), LPR = Is / 64, rows = 64 / LPR;
-        bool bad = false;
-        for (int t = 0; t < NT; t++) bad |= build_image(images + t * W, a.shared_act + (size_t)t * Is, Is);
+    const int rounds = K + 1;
+    if (!shared && wave < parts * NT) {
+        const int t = wave / parts;
+        pf_route_stage1<NPL>(a.logits + (size_t)t * E, a.logit_ssq + (size_t)t * E, E, wave % parts, chunk, rounds,
+                             a.norm_topk != 0, &R.cands[t], lane);
+    }
+    STAMP(1);
+    for (int t = 0; t < NT; t++) build_image(images + t * W, a.x + (size_t)t * a.x_pitch, H, 768, 256);
+    __syncthreads();
+    STAMP(2);
+    int u, n0, I, gate_tensor;
+    uint32_t e, mask;
+    if (shared) {
+        u = P; n0 = 32 * (blockIdx.x - routed_blocks); I = a.shared_inter; gate_tensor = 4;
+        e = 0; mask = (1u << NT) - 1u;
+    } else {
+        if (wave < NT) {
+            PfRouteResult r = pf_route_stage2(&R.cands[wave], parts, K, rounds, a.norm_topk != 0, H, lane);
+            if (lane < K) { R.ids[wave * K + lane] = r.id; R.weights[wave * K + lane] = r.weight; }
+            if (lane == 0) { R.close[wave] = r.close ? 1u : 0u; R.nonfinite[wave] = r.bad ? 1u : 0u; }
+        }
         __syncthreads();
-        const int seg = lane & (LPR - 1);
-        const int n = ((blockIdx.x - routed_blocks) * 4 + wave) * rows + lane / LPR;
-        if (n - lane / LPR >= H) return;
-        WSeg<FMT> w;
-        wseg_load<FMT>(w, a, 6, 0, min(n, H - 1), seg);
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            XSeg x;
-            xseg_load(x, images + t * W, Is, seg);
-            const float v = span_sum(wseg_dot<FMT>(w, x, seg, tables), LPR);
-            if (seg == 0 && n < H) a.shared_out[(size_t)t * H + n] = v;
+        STAMP(3);
+        route_finish<NT>(a, &R, reinterpret_cast<float *>(images + NT * W));
+        const int U = R.count;
+        if (blockIdx.x == 0) {
+            // publish the routes and the union for the next kernel and the caller
+            for (int p = threadIdx.x; p < P; p += blockDim.x) {
+                a.ids[p] = R.ids[p];
+                a.route_weights[p] = R.weights[p];
+                a.uniq[1 + p] = p < U ? R.uniq[p] : 0u;
+                a.uniq[1 + P + p] = R.pair_slot[p];
+                a.uniq[1 + 2 * P + p] = p < U ? R.mask[p] : 0u;
+            }
+            if (threadIdx.x == 0) {
+                a.uniq[0] = U;
+                if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+                if (R.close_mask) atomicAdd(a.exact_rows, __popc(R.close_mask));
+            }
         }
-        return;
-    }
-
-    const int W = image_words(H);
-    for (int t = 0; t < NT; t++) build_image(images + t * W, a.x + (size_t)t * a.x_pitch, H);
-    float *scratch = reinterpret_cast<float *>(images + NT * W);
-    route_tokens<NPL>(a, &R, scratch, NT);
-    const int P = NT * K, U = R.count;
-    if (blockIdx.x == 0) {
-        // publish the routes and the union for the next kernel and the caller
-        for (int p = threadIdx.x; p < P; p += blockDim.x) {
-            a.ids[p] = R.ids[p];
-            a.route_weights[p] = R.weights[p];
-            a.uniq[1 + p] = p < U ? R.uniq[p] : 0u;
-            a.uniq[1 + P + p] = R.pair_slot[p];
-            a.uniq[1 + 2 * P + p] = p < U ? R.mask[p] : 0u;
-        }
-        if (threadIdx.x == 0) {
-            a.uniq[0] = U;
-            if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-            if (R.close_mask) atomicAdd(a.exact_rows, __popc(R.close_mask));
+        I = a.inter; gate_tensor = 1;
+        const int tiles = I / 32;
+        u = blockIdx.x / tiles; n0 = 32 * (blockIdx.x % tiles);
+        if (u >= U) return;
+        e = R.uniq[u]; mask = R.mask[u];
+        if (e >= (uint32_t)E) {   // only reachable with nonfinite logits
+            if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+            return;
         }
     }
-    const int tiles = I / 32, u = blockIdx.x / tiles, n0 = 32 * (blockIdx.x % tiles);
-    if (u >= U) return;
-    const uint32_t e = R.uniq[u], mask = R.mask[u];
-    if (e >= (uint32_t)a.experts) {   // only reachable with nonfinite logits
-        if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
-        return;
-    }
+    STAMP(4);
     const int LPR = H / 64, RPH = 32 / LPR;
     const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
-    const int steps = 8 / RPH;                       // this wave's 8 units, RPH per step
-    XSeg x[NT];
+    // the tile's 32 units over 16 waves: two per wave, RPH per wave step
+    const int per_wave = RPH > 2 ? RPH : 2, steps = per_wave / RPH, unit0 = wave * per_wave;
+    if (unit0 < 32) {
+        WSeg<FMT> w[2];
 #pragma unroll
-    for (int t = 0; t < NT; t++)
-        if ((mask >> t) & 1u) xseg_load(x[t], images + t * W, H, seg);
-    for (int s0 = 0; s0 < steps; s0 += 4) {
-        WSeg<FMT> w[4];
+        for (int s = 0; s < 2; s++)
+            if (s < steps) wseg_load<FMT>(w[s], a, gate_tensor + half, e, n0 + unit0 + s * RPH + r, seg);
 #pragma unroll
-        for (int s = 0; s < 4; s++)
-            if (s0 + s < steps) wseg_load<FMT>(w[s], a, 1 + half, e, n0 + wave * 8 + (s0 + s) * RPH + r, seg);
+        for (int t = 0; t < NT; t++) {
+            if (!((mask >> t) & 1u)) continue;
+            XSeg x;
+            xseg_load(x, images + t * W, H, seg);
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-            if (s0 + s >= steps) break;
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                if (!((mask >> t) & 1u)) continue;
-                float v = span_sum(wseg_dot<FMT>(w[s], x[t], seg, tables), LPR);
+            for (int s = 0; s < 2; s++) {
+                if (s >= steps) break;
+                float v = span_sum(wseg_dot<FMT>(w[s], x, seg, tables), LPR);
                 const float up = __shfl(v, (lane & 31) + 32);
-                if (half == 0 && seg == 0) R.tile[t][wave * 8 + (s0 + s) * RPH + r] = pf_silu(v) * up;
+                if (half == 0 && seg == 0) R.tile[t][unit0 + s * RPH + r] = pf_silu(v) * up;
             }
         }
     }
+    STAMP(5);
     __syncthreads();
+    STAMP(6);
     // 32 activations per token: FP32 copy and digit image for the down kernel
     if (wave < NT && ((mask >> wave) & 1u) && lane < 32) {
         const int t = wave, WI = image_words(I), plane = SEG_STRIDE * (I / 64);
         const float v = R.tile[t][lane];
         if (!pf_finite(v)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-        a.act[((size_t)u * NT + t) * I + n0 + lane] = v;
+        if (shared) a.shared_act[(size_t)t * I + n0 + lane] = v;
+        else a.act[((size_t)u * NT + t) * I + n0 + lane] = v;
         float m = fabsf(v);
         for (int k = 16; k >= 1; k >>= 1) m = fmaxf(m, __shfl_xor(m, k));
         float step, inv;
@@ -472,7 +466,7 @@ __global__ void __launch_bounds__(256) pf_k_dec_gate_up(PfKernelArgs a, int rout
         w1 |= dpp_quad_xor1(w1); w1 |= dpp_quad_xor2(w1);
         w2 |= dpp_quad_xor1(w2); w2 |= dpp_quad_xor2(w2);
         for (int k = 16; k >= 1; k >>= 1) sum += __shfl_xor(sum, k);
-        int *img = reinterpret_cast<int *>(a.act_images) + ((size_t)u * NT + t) * WI;
+        int *img = shared ? a.shared_images + (size_t)t * WI : a.act_images + ((size_t)u * NT + t) * WI;
         if ((lane & 3) == 0) {
             const int nn = n0 + lane, at = SEG_STRIDE * (nn >> 6) + ((nn & 63) >> 2);
             img[at] = w0;
@@ -484,47 +478,61 @@ __global__ void __launch_bounds__(256) pf_k_dec_gate_up(PfKernelArgs a, int rout
             img[3 * plane + I / 32 + (n0 >> 5)] = sum;
         }
     }
+    STAMP(7);
 }
 
-// ---- kernel 3: routed down products and the combine ------------------------------------------
-// block = (token, 16 output rows ... ) with one wave per slot; blockIdx.x = t * row_blocks + nb
+// ---- kernel 3: down products and the combine ---------------------------------------------------
+// blockIdx.x = t * row_blocks + nb; one wave per slot plus one for the shared expert; a routed
+// wave covers the block's rows in one step.
 template <int FMT, int NT>
 __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_blocks, int rows_per_block) {
-    __shared__ float partial[16][64];
+    __shared__ float partial[17][64];
     extern __shared__ int lds[];
     uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
     if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
-    const int I = a.inter, H = a.hidden, K = a.top_k, lane = pf_lane(), s = threadIdx.x >> 6;
+    const int H = a.hidden, K = a.top_k, lane = pf_lane(), s = threadIdx.x >> 6;
     const int t = blockIdx.x / row_blocks, nb = blockIdx.x % row_blocks, P = NT * K;
-    const int LPR = I / 64, rows = 64 / LPR, steps = rows_per_block / rows;
+    const bool shared = s == K;
+    const int I = shared ? a.shared_inter : a.inter, tensor = shared ? 6 : 3;
+    const int LPR = I / 64, rows = 64 / LPR, steps = rows >= rows_per_block ? 1 : rows_per_block / rows;
     const int seg = lane & (LPR - 1), r = lane / LPR;
-    uint32_t e = a.ids[t * K + s], u = a.uniq[1 + P + t * K + s];
-    if (e >= (uint32_t)a.experts || u >= (uint32_t)P) {   // only reachable with nonfinite logits
-        if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
-        e = 0;
-        u = 0;
+    uint32_t e = 0, u = 0;
+    if (!shared) {
+        e = a.ids[t * K + s];
+        u = a.uniq[1 + P + t * K + s];
+        if (e >= (uint32_t)a.experts || u >= (uint32_t)P) {   // only reachable with nonfinite logits
+            if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+            e = 0;
+            u = 0;
+        }
     }
     const int n_base = nb * rows_per_block;
-    WSeg<FMT> w[4];
-#pragma unroll
-    for (int st = 0; st < 4; st++)
-        if (st < steps) wseg_load<FMT>(w[st], a, 3, e, min(n_base + st * rows + r, H - 1), seg);
+    WSeg<FMT> w;   // further steps (a shared expert wider than the routed ones) load as they go
+    wseg_load<FMT>(w, a, tensor, e, min(n_base + r, H - 1), seg);
     XSeg x;
-    xseg_load(x, reinterpret_cast<const int *>(a.act_images) + ((size_t)u * NT + t) * image_words(I), I, seg);
-    if (FMT == PF_IQ2_XXS) __syncthreads();
+    const int *image = shared ? a.shared_images + (size_t)t * image_words(I)
+                              : a.act_images + ((size_t)u * NT + t) * image_words(I);
+    xseg_load(x, image, I, seg);
+    // operands of the final combine, requested now so that they arrive with the weights
+    float rw[16];
 #pragma unroll
-    for (int st = 0; st < 4; st++) {
-        if (st >= steps) break;
-        const float v = span_sum(wseg_dot<FMT>(w[st], x, seg, tables), LPR);
-        if (seg == 0) partial[s][st * rows + r] = v;
+    for (int slot = 0; slot < 16; slot++) rw[slot] = slot < K ? a.route_weights[t * K + slot] : 0.0f;
+    const float shared_scale = a.shared_scale[t];
+    if (FMT == PF_IQ2_XXS) __syncthreads();
+    for (int st = 0; st < steps; st++) {
+        const float v = span_sum(wseg_dot<FMT>(w, x, seg, tables), LPR);
+        const int row = st * rows + r;
+        if (seg == 0 && row < rows_per_block) partial[s][row] = v;
+        if (st + 1 < steps) wseg_load<FMT>(w, a, tensor, e, min(n_base + (st + 1) * rows + r, H - 1), seg);
     }
     __syncthreads();
     const int n = n_base + threadIdx.x;
     if ((int)threadIdx.x < rows_per_block && n < H) {
         float sum = 0.0f;
-        for (int slot = 0; slot < K; slot++)   // slot order, as src/qwen4_moe.c:362-372
-            sum += a.route_weights[t * K + slot] * partial[slot][threadIdx.x];
-        const float y = sum + a.shared_scale[t] * a.shared_out[(size_t)t * H + n];
+#pragma unroll
+        for (int slot = 0; slot < 16; slot++)   // slot order, as src/qwen4_moe.c:362-372
+            if (slot < K) sum += rw[slot] * partial[slot][threadIdx.x];
+        const float y = sum + shared_scale * partial[K][threadIdx.x];
         a.y[(size_t)t * a.y_pitch + n] = y;
         if (!pf_finite(y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
@@ -557,10 +565,22 @@ bool pf_decode_supported(const PfHipMoeDesc &d) {
     for (int j = 1; j <= 6; j++)
         if (d.type[j] != fmt) return false;
     if (!pow2_between(d.hidden, 512, 2048) || !pow2_between(d.inter, 256, 2048) ||
-        !pow2_between(d.shared_inter, 256, 2048) || d.down_physical != d.inter)
+        !pow2_between(d.shared_inter, 256, 2048) || d.down_physical != d.inter || d.shared_inter > 4 * d.inter)
         return false;
-    if (d.experts > 1024 || d.top_k > 16 || d.top_k * PF_DECODE_MAX_TOKENS > 64 || d.top_k >= d.experts) return false;
+    if (d.experts > 1024 || d.top_k > 15 || d.top_k * PF_DECODE_MAX_TOKENS > 64 || d.top_k >= d.experts) return false;
     return true;
+}
+
+template <int FMT, int NT, int NPL>
+static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks,
+                           int parts, int chunk) {
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, NPL>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, NPL>), grid, dim3(1024), lds, stream, a, routed_blocks, parts, chunk);
 }
 
 template <int FMT, int NT>
@@ -568,43 +588,25 @@ static void launch_decode(const PfKernelArgs &a, hipStream_t stream, hipEvent_t 
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
     const size_t tab = table_words<FMT>() * 4;
     // kernel 1
-    const int router_blocks = (E + 3) / 4, rph = 32 / (H / 64), shared_blocks = (Is + 8 * rph - 1) / (8 * rph);
-    const size_t lds1 = tab + (size_t)NT * image_words(H) * 4;
+    const int router_blocks = (E + 3) / 4;
     if (marks) (void)hipEventRecord(marks[0], stream);
-    hipLaunchKernelGGL((pf_k_dec_pre<FMT, NT>), dim3(router_blocks + shared_blocks + 1), dim3(256), lds1, stream, a,
-                       router_blocks, shared_blocks);
+    hipLaunchKernelGGL((pf_k_dec_router<NT>), dim3(router_blocks + 1), dim3(256), 0, stream, a, router_blocks);
     if (marks) { (void)hipEventRecord(marks[1], stream); (void)hipEventRecord(marks[2], stream); }
-    // kernel 2
-    const int routed_blocks = NT * K * (I / 32), down_rows = 64 / (Is / 64);
-    const int shared_down_blocks = (H + 4 * down_rows - 1) / (4 * down_rows);
-    const size_t img2 = (size_t)NT * image_words(H > Is ? H : Is) * 4, fix = ((size_t)H + 3 * (size_t)E) * 4;
-    const size_t lds2 = tab + img2 + fix;
-    const int npl = (E + 63) / 64;
-    dim3 g2(routed_blocks + shared_down_blocks);
-    static bool big_lds = false;   // once per instantiation: allow more than the default 64 KB of dynamic LDS
-    if (!big_lds) {
-        const int limit = 128 * 1024;
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 2>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 4>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 8>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, 16>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_pre<FMT, NT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, limit);
-        big_lds = true;
-    }
-    if (npl <= 2) hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 2>), g2, dim3(256), lds2, stream, a, routed_blocks);
-    else if (npl <= 4) hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 4>), g2, dim3(256), lds2, stream, a, routed_blocks);
-    else if (npl <= 8) hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 8>), g2, dim3(256), lds2, stream, a, routed_blocks);
-    else hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, 16>), g2, dim3(256), lds2, stream, a, routed_blocks);
+    // kernel 2: the candidate stage uses up to 8 of waves 0..11 per token
+    const int routed_blocks = NT * K * (I / 32), shared_blocks = Is / 32;
+    const size_t lds2 = tab + (size_t)NT * image_words(H) * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+    int parts = NT == 1 ? 8 : NT == 2 ? 6 : NT == 3 ? 4 : 3;
+    while (parts > 1 && (E + parts - 1) / parts < 64) parts--;
+    const int chunk = (E + parts - 1) / parts, npl = (chunk + 63) / 64;
+    dim3 g2(routed_blocks + shared_blocks);
+    if (npl <= 1) launch_gate_up<FMT, NT, 1>(a, g2, lds2, stream, routed_blocks, parts, chunk);
+    else if (npl <= 2) launch_gate_up<FMT, NT, 2>(a, g2, lds2, stream, routed_blocks, parts, chunk);
+    else if (npl <= 4) launch_gate_up<FMT, NT, 4>(a, g2, lds2, stream, routed_blocks, parts, chunk);
+    else launch_gate_up<FMT, NT, 8>(a, g2, lds2, stream, routed_blocks, parts, chunk);   // experts <= 1024
     if (marks) (void)hipEventRecord(marks[3], stream);
     // kernel 3
-    const int rows = 64 / (I / 64), rows_per_block = 2 * rows > 64 ? 64 : 2 * rows;
-    const int row_blocks = (H + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((pf_k_dec_down<FMT, NT>), dim3(NT * row_blocks), dim3(64 * K), tab, stream, a, row_blocks,
+    const int rows_per_block = 64 / (I / 64), row_blocks = (H + rows_per_block - 1) / rows_per_block;
+    hipLaunchKernelGGL((pf_k_dec_down<FMT, NT>), dim3(NT * row_blocks), dim3(64 * (K + 1)), tab, stream, a, row_blocks,
                        rows_per_block);
     if (marks) (void)hipEventRecord(marks[4], stream);
 }

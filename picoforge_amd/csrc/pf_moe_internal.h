@@ -26,8 +26,8 @@ struct PfKernelArgs {
     float *act;                      // general path [tokens * top_k, inter]; decode path [unique, tokens, inter]
     float *shared_act;               // [tokens, shared_inter]
     float *shared_scale;             // [tokens] sigmoid of the shared router logit
-    float *shared_out;               // [tokens, hidden] shared expert's down product (decode path)
     int *act_images;                 // decode path: digit image of every [unique, token] activation row
+    int *shared_images;              // decode path: digit image of every token's shared activation row
     uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
     uint32_t *error_word;
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
@@ -48,9 +48,9 @@ struct PfHipMoe {
 struct PfHipWork {
     const PfHipMoe *moe;
     size_t cap, bytes;
-    float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *shared_out, *x, *y;
+    float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
     uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags;
-    int *act_images;
+    int *act_images, *shared_images;
     void *marks;                     // hipEvent_t[5] while stage profiling, else null
     int force_general;               // tests: run the general kernels even where the decode path applies
 };

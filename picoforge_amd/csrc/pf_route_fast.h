@@ -1,8 +1,15 @@
-// Fast routing of one token by one wave: logits in registers, selection in logit
-// space, and a closeness test that sends ambiguous tokens to the reference-order
-// path.  Selecting on logits equals selecting on probabilities (src/qwen4_moe.c:233-246)
-// whenever adjacent selected logits are further apart than the test's tolerance,
-// because exp and the division by a common sum are monotone up to a few ulps.
+// Fast routing: logits in registers, selection in logit space, and a closeness test that
+// sends ambiguous tokens to the reference-order path.  Selecting on logits equals selecting
+// on probabilities (src/qwen4_moe.c:233-246) whenever adjacent selected logits are further
+// apart than the test's tolerance, because exp and the division by a common sum are
+// monotone up to a few ulps.
+//
+// Two forms: one wave routes a whole token (pf_route_fast_wave), or several waves each
+// reduce a contiguous chunk of experts to their best k+1 candidates (pf_route_stage1) and
+// one wave merges the candidates (pf_route_stage2).  Expert e of a chunk lives in lane
+// e / NPL, register e % NPL, so the lowest lane holding the maximum also holds the lowest
+// expert id among equal logits: ties go to the lower id, as an ascending scan with a strict
+// comparison decides them.
 #pragma once
 #include "pf_device.h"
 
@@ -38,19 +45,49 @@ struct PfRouteResult {
     bool bad;        // uniform: a nonfinite logit was seen
 };
 
-// z_row, ssq_row: the token's E logits and sums of squared products.  Expert e
-// lives in lane e / NPL, register e % NPL, so the lowest lane holding the
-// maximum also holds the lowest expert id among equal logits.
+// One round of extraction: the largest remaining value of the wave, its holder and register.
+template <int NPL>
+__device__ __forceinline__ void pf_extract_max(float (&v)[NPL], int lane, float &wm, int &owner, int &jsel) {
+    float m = v[0];
+#pragma unroll
+    for (int j = 1; j < NPL; j++) m = fmaxf(m, v[j]);
+    wm = pf_wave_max_fast(m);
+    const unsigned long long holders = __ballot(m == wm);
+    owner = holders ? __ffsll((long long)holders) - 1 : 0;   // no holder: NaN logits, flagged as bad
+    int jl = NPL - 1;
+#pragma unroll
+    for (int j = NPL - 1; j >= 0; j--) jl = v[j] == wm ? j : jl;
+    jsel = NPL == 1 ? 0 : __builtin_amdgcn_readlane(jl, owner);
+#pragma unroll
+    for (int j = 0; j < NPL; j++) v[j] = (lane == owner && j == jsel) ? -INFINITY : v[j];
+}
+
+// Closeness test and route weights from the sorted k+1 best: lane r holds (my_z, my_s2).
+// total/top_all: softmax denominator and its reference maximum (only used when !norm).
+__device__ __forceinline__ void pf_route_finish_wave(float my_z, float my_s2, int K, int rounds, bool norm, int hidden,
+                                                     float total, float top_all, int lane, float &weight, bool &close) {
+    const float next_z = __shfl_down(my_z, 1), next_s2 = __shfl_down(my_s2, 1);
+    const float top = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_z), 0));
+    // Noise model of a K-term FP32 sum in any order: standard deviation
+    // u * sqrt(K * sum(products^2) / 6); eight of those per logit, plus the
+    // rounding of z - max and of the exponential.
+    const float u = 5.9604645e-8f, hk = (float)hidden / 6.0f;
+    const float tol = 8.0f * u * (sqrtf(hk * my_s2) + sqrtf(hk * next_s2)) + 4e-6f * fmaxf(1.0f, top - next_z);
+    close = __any(lane + 1 < rounds && !(my_z - next_z > tol));
+    const float e = lane < K ? expf(my_z - top) : 0.0f;
+    if (norm) weight = e / pf_wave_sum(e);
+    else weight = e * expf(top - top_all) / total;
+}
+
 template <int NPL>
 __device__ __forceinline__ PfRouteResult pf_route_fast_wave(const float *z_row, const float *ssq_row, int E, int K,
                                                             bool norm, int hidden, int lane) {
-    float v[NPL], s2[NPL];
+    float v[NPL];
     bool bad = false;
 #pragma unroll
     for (int j = 0; j < NPL; j++) {
         const int e = lane * NPL + j;
         v[j] = e < E ? z_row[e] : -INFINITY;
-        s2[j] = e < E ? ssq_row[e] : 0.0f;
         bad |= e < E && !pf_finite(v[j]);
     }
     bad = __any(bad);
@@ -68,45 +105,112 @@ __device__ __forceinline__ PfRouteResult pf_route_fast_wave(const float *z_row, 
     uint32_t my_id = 0;
     float my_z = 0.0f, my_s2 = 0.0f;
     for (int r = 0; r < rounds; r++) {
-        float m = v[0];
-#pragma unroll
-        for (int j = 1; j < NPL; j++) m = fmaxf(m, v[j]);
-        const float wm = pf_wave_max_fast(m);
-        const unsigned long long holders = __ballot(m == wm);
-        const int owner = holders ? __ffsll((long long)holders) - 1 : 0;   // no holder: NaN logits, flagged as bad
-        int jl = NPL - 1;
-#pragma unroll
-        for (int j = NPL - 1; j >= 0; j--) jl = v[j] == wm ? j : jl;
-        const int jsel = __builtin_amdgcn_readlane(jl, owner);
-        float s2sel = s2[0];
-#pragma unroll
-        for (int j = 1; j < NPL; j++) s2sel = j == jsel ? s2[j] : s2sel;
-        s2sel = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s2sel), owner));
-#pragma unroll
-        for (int j = 0; j < NPL; j++) v[j] = (lane == owner && j == jsel) ? -INFINITY : v[j];
+        float wm;
+        int owner, jsel;
+        pf_extract_max<NPL>(v, lane, wm, owner, jsel);
         if (lane == r) {
             my_id = (uint32_t)(owner * NPL + jsel);
             my_z = wm;
-            my_s2 = s2sel;
         }
     }
-    // closeness of neighbours in the sorted list of the k+1 best
-    const float next_z = __shfl_down(my_z, 1), next_s2 = __shfl_down(my_s2, 1);
-    const float top = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_z), 0));
-    // Noise model of a K-term FP32 sum in any order: standard deviation
-    // u * sqrt(K * sum(products^2) / 6); eight of those per logit, plus the
-    // rounding of z - max and of the exponential.
-    const float u = 5.9604645e-8f, hk = (float)hidden / 6.0f;
-    const float tol = 8.0f * u * (sqrtf(hk * my_s2) + sqrtf(hk * next_s2)) + 4e-6f * fmaxf(1.0f, top - next_z);
-    const bool close = __any(lane + 1 < rounds && !(my_z - next_z > tol));
-    float e = lane < K ? expf(my_z - top) : 0.0f;
-    float weight;
-    if (norm) weight = e / pf_wave_sum(e);
-    else weight = e * expf(top - top_all) / total;   // exp(z - top_all) / total, without overflow
+    if (lane < rounds && my_id < (uint32_t)E) my_s2 = ssq_row[my_id];
     PfRouteResult out;
+    pf_route_finish_wave(my_z, my_s2, K, rounds, norm, hidden, total, top_all, lane, out.weight, out.close);
     out.id = my_id;
-    out.weight = weight;
-    out.close = close;
+    out.bad = bad;
+    return out;
+}
+
+// ---- several waves per token -------------------------------------------------------------
+// Candidate lists in LDS: for each of `parts` waves, `rounds` entries sorted by (logit
+// descending, id ascending); entry = logit, id, sum of squared products.  part_max and
+// part_sum carry the pieces of the softmax denominator.
+struct PfRouteCands {
+    float z[160];
+    uint32_t id[160];
+    float s2[160];
+    float part_max[8], part_sum[8];
+    uint32_t bad[8];
+};
+
+template <int NPL>
+__device__ __forceinline__ void pf_route_stage1(const float *z_row, const float *ssq_row, int E, int part, int chunk,
+                                                int rounds, bool norm, PfRouteCands *c, int lane) {
+    const int base = part * chunk, len = min(chunk, E - base);
+    float v[NPL], s2[NPL];
+    bool bad = false;
+#pragma unroll
+    for (int j = 0; j < NPL; j++) {
+        const int i = lane * NPL + j;
+        v[j] = i < len ? z_row[base + i] : -INFINITY;
+        s2[j] = i < len ? ssq_row[base + i] : 0.0f;
+        bad |= i < len && !pf_finite(v[j]);
+    }
+    bad = __any(bad);
+    if (!norm) {
+        float m = v[0], sum = 0.0f;
+#pragma unroll
+        for (int j = 1; j < NPL; j++) m = fmaxf(m, v[j]);
+        m = pf_wave_max_fast(m);
+#pragma unroll
+        for (int j = 0; j < NPL; j++) sum += expf(v[j] - m);
+        sum = pf_wave_sum(sum);
+        if (lane == 0) { c->part_max[part] = m; c->part_sum[part] = sum; }
+    }
+    if (lane == 0) c->bad[part] = bad ? 1u : 0u;
+    for (int r = 0; r < rounds; r++) {
+        float wm;
+        int owner, jsel;
+        pf_extract_max<NPL>(v, lane, wm, owner, jsel);
+        const int at = part * rounds + r;
+        // the holder stores from its own registers: one predicated store per register, no
+        // register array indexed by a run-time value
+#pragma unroll
+        for (int j = 0; j < NPL; j++) {
+            if (lane == owner && j == jsel) {
+                c->z[at] = wm;
+                c->id[at] = wm == -INFINITY ? 0xffffffffu : (uint32_t)(base + lane * NPL + j);
+                c->s2[at] = s2[j];
+            }
+        }
+    }
+}
+
+// Merge by one wave: candidate p sits in lane p / 3, register p % 3 (at most 160 candidates).
+__device__ __forceinline__ PfRouteResult pf_route_stage2(const PfRouteCands *c, int parts, int K, int rounds, bool norm,
+                                                         int hidden, int lane) {
+    const int count = parts * rounds;
+    float v[3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int p = lane * 3 + j;
+        v[j] = p < count ? c->z[p] : -INFINITY;
+    }
+    float total = 0.0f, top_all = 0.0f;
+    bool bad = false;
+    for (int w = 0; w < parts; w++) bad |= c->bad[w] != 0;
+    if (!norm) {
+        top_all = c->part_max[0];
+        for (int w = 1; w < parts; w++) top_all = fmaxf(top_all, c->part_max[w]);
+        for (int w = 0; w < parts; w++) total += c->part_sum[w] * expf(c->part_max[w] - top_all);
+    }
+    int my_at = 0;
+    float my_z = 0.0f;
+    for (int r = 0; r < rounds; r++) {
+        float wm;
+        int owner, jsel;
+        pf_extract_max<3>(v, lane, wm, owner, jsel);
+        if (lane == r) {
+            my_at = owner * 3 + jsel;
+            my_z = wm;
+        }
+    }
+    my_at = my_at < count ? my_at : 0;
+    const uint32_t my_id = c->id[my_at];
+    const float my_s2 = c->s2[my_at];
+    PfRouteResult out;
+    pf_route_finish_wave(my_z, my_s2, K, rounds, norm, hidden, total, top_all, lane, out.weight, out.close);
+    out.id = my_id;
     out.bad = bad;
     return out;
 }
