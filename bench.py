@@ -11,8 +11,8 @@ token, hence other experts.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 Prints one JSON line.  `value` is microseconds per layer per token (lower is
-better).  `roofline` is for the dominant kernel, timed live with HIP events on
-the launch stream.  `cpu_baseline` times the CPU path (the reference's own
+better).  `roofline` is for the kernel that moves the most bytes, timed live
+with HIP events on the launch stream.  `cpu_baseline` times the CPU path (the reference's own
 compiled C when oracle/_ref is present, else the oracle port) on a bounded
 sample of the same tokens, single thread, and the same sample is used to check
 the GPU results (ids exact, outputs within 1e-3 + 1e-4 relative).
@@ -40,8 +40,8 @@ WORKLOADS = {
     "q4k_decode": dict(type=abi.GGUF_Q4_K, tokens=1, label="Q4_K experts, decode batch 1"),
     "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
 }
-STAGES = ["pf_k_dec_pre (router logits, shared gate/up)", "pf_k_dec_gate_up (routing, routed gate/up, shared down)",
-          "pf_k_dec_down (routed down, combine)"]
+STAGES = ["pf_k_dec_router (router logits)", "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
+          "pf_k_dec_down (down products, routed and shared, combine)"]
 
 
 def device_forward_sample(api, layer, x, tokens):
@@ -61,6 +61,8 @@ def main():
     ap.add_argument("--workload", default="iq2xxs_decode", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-sample", type=int, default=None, help="tokens timed on the CPU path (default ~15 s of work)")
     ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="also launch a plain copy kernel of this many MiB three times (byte-counter calibration)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); use --gpus 1")
@@ -103,23 +105,21 @@ def main():
     exact = C.c_uint32()
     hip.work_exact_rows(work, C.byref(exact))
 
-    # Per-kernel durations: HIP events on the launch stream around each of the three decode
-    # kernels, minus the same measurement of an empty kernel (the fixed dispatch cost).
+    # Per-kernel durations inside the dependent chain: graph replays of the first 1, 2, 3
+    # kernels of every forward, bracketed by HIP events on the launch stream; a kernel's
+    # duration is the difference between consecutive replays (it includes the dispatch gap
+    # before it, as a profiler's start-to-end time of a dependent kernel does).
     stage = (C.c_float * 4)()
-    hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(args.steps, 500), stage), "stages")
-    empty = C.c_float()
-    hip.check(hip.event_overhead(200, C.byref(empty)), "event overhead")
-    overhead_us = float(empty.value) * 1e3
-    raw_us = [float(stage[0]) * 1e3, float(stage[2]) * 1e3, float(stage[3]) * 1e3]
-    stage_us = [max(v - overhead_us, 0.05) for v in raw_us]
+    hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(args.steps, 2000), stage), "stages")
+    stage_us = [max(float(stage[j]) * 1e3, 1e-3) for j in range(3)]
 
     alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique)
     block, size = abi.BLOCK[wl["type"]]
     h, i, s_i = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate
     # algorithmic bytes per launch: what each kernel must read once
-    stage_bytes = [(cfg.experts + 1) * h * 4 + 2 * s_i * h // block * size,
-                   unique * 2 * i * h // block * size + h * s_i // block * size,
-                   unique * h * i // block * size]
+    stage_bytes = [(cfg.experts + 1) * h * 4,
+                   unique * 2 * i * h // block * size + 2 * s_i * h // block * size,
+                   unique * h * i // block * size + h * s_i // block * size]
     dom = int(np.argmax(stage_bytes))
     achieved = stage_bytes[dom] / (stage_us[dom] * 1e-6) / 1e9
 
@@ -138,6 +138,8 @@ def main():
     max_abs = max(float(np.abs(g[0] - c[0]).max()) for g, c in zip(gpu_out, cpu_out))
     within = all((np.abs(g[0] - c[0]) <= 1e-3 + 1e-4 * np.abs(c[0])).all() for g, c in zip(gpu_out, cpu_out))
     layer.close()
+    if args.copy_probe:
+        hip.check(hip.copy_probe(args.copy_probe << 20, 3), "copy probe")
 
     result = {
         "metric": "moe_decode_us_per_layer_token",
@@ -159,7 +161,6 @@ def main():
                      "bytes_per_launch": int(stage_bytes[dom]), "us_per_launch": round(stage_us[dom], 3)},
         "kernel_us": dict(zip(STAGES, [round(v, 3) for v in stage_us])),
         "kernel_bytes": dict(zip(STAGES, [int(b) for b in stage_bytes])),
-        "event_overhead_us": round(overhead_us, 3),
         "cpu_baseline": {"value": round(cpu_s / (sample * tokens) * 1e6, 1), "unit": "us/layer/token", "cores": 1,
                          "kind": kind, "sample": f"first {sample} steps ({sample * tokens} tokens) of the same inputs, "
                                                    f"{cpu_s:.1f} s"},

@@ -133,17 +133,20 @@ int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *
                              size_t n_inputs, float *d_y, size_t tokens, size_t iters,
                              float *elapsed_ms);
 
-/* Same loop, synchronising after every forward and reading events placed between
- * the four stages of the general path: stage_ms[0] router + shared gate/up,
- * [1] routing, [2] routed gate/up, [3] down + combine; averages over iters. */
+/* Average duration of each kernel inside the dependent chain: the same loop run
+ * with only the first 1, 2, ... kernels of every forward launched; stage_ms[j] is
+ * the difference between consecutive runs divided by iters.  Decode path (1..4
+ * tokens, supported shapes): [0] router logits, [1] routing + gate/up, [2] down +
+ * combine, [3] zero.  General path: [0] router + shared gate/up, [1] routing,
+ * [2] routed gate/up, [3] down + combine. */
 int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
                               size_t n_inputs, float *d_y, size_t tokens, size_t iters,
                               float stage_ms[4]);
 
-/* Average milliseconds between two events recorded around an empty kernel, measured
- * the way pf_hip_moe_profile_stages measures a stage: the fixed cost inside every
- * stage time. */
-int pf_hip_event_overhead(size_t iters, float *ms_per_kernel);
+/* Launches a plain device-to-device copy kernel (pf_k_copy_probe) of `bytes` bytes
+ * `launches` times: a kernel of known traffic (bytes read, bytes written) against
+ * which hardware byte counters read under a profiler can be scaled. */
+int pf_hip_copy_probe(size_t bytes, size_t launches);
 
 #ifdef __cplusplus
 }

@@ -307,7 +307,7 @@ extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, c
     PfKernelArgs a = make_args(moe, work, d_x, x_pitch, d_y, y_pitch);
     const bool aligned = (x_pitch % 4 == 0) && ((uintptr_t)d_x % 16 == 0);
     if (moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS && aligned && !work->force_general) {
-        pf_launch_decode(a, (int)tokens, s, (hipEvent_t *)work->marks);
+        pf_launch_decode(a, (int)tokens, s, work->stage_limit);
     } else {
         // the general kernels stage one token's activations in LDS
         const size_t lds_route = ((size_t)d->hidden + 3 * (size_t)d->experts) * 4;
@@ -315,7 +315,7 @@ extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, c
             snprintf(g_error, sizeof g_error, "dimensions exceed the LDS staging of the general kernels");
             return PF_HIP_E_UNSUPPORTED;
         }
-        pf_launch_general(a, (int)tokens, s, (hipEvent_t *)work->marks);
+        pf_launch_general(a, (int)tokens, s, work->stage_limit);
     }
     HIP_TRY(hipGetLastError());
     return PF_HIP_OK;
@@ -511,9 +511,8 @@ extern "C" int pf_hip_synchronize(void) {
 // `iters` forwards back to back on one stream.  The launches are captured into graphs of
 // up to 256 forwards (each with its own input block) and the graphs are replayed in order,
 // so the measured gap between dependent kernels is the device's, not the host's enqueue rate.
-extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
-                                        float *d_y, size_t tokens, size_t iters, float *elapsed_ms) {
-    if (!moe || !work || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
+static int time_graph_replay(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs, float *d_y,
+                             size_t tokens, size_t iters, int stage_limit, float *elapsed_ms) {
     *elapsed_ms = 0.0f;
     if (!iters) return PF_HIP_OK;
     const size_t H = moe->desc.hidden, chunk = 256, n_graphs = (iters + chunk - 1) / chunk;
@@ -522,6 +521,8 @@ extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, co
     HIP_TRY(hipStreamCreate(&s));
     hipGraphExec_t *execs = (hipGraphExec_t *)calloc(n_graphs, sizeof *execs);
     int rc = execs ? PF_HIP_OK : PF_HIP_E_MEMORY;
+    const int saved_limit = work->stage_limit;
+    work->stage_limit = stage_limit;
     for (size_t g = 0; g < n_graphs && rc == PF_HIP_OK; g++) {
         hipGraph_t graph = nullptr;
         if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) { rc = PF_HIP_E_RUNTIME; break; }
@@ -533,6 +534,7 @@ extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, co
             rc = PF_HIP_E_RUNTIME;
         if (graph) (void)hipGraphDestroy(graph);
     }
+    work->stage_limit = saved_limit;
     if (rc == PF_HIP_OK && (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess)) rc = PF_HIP_E_RUNTIME;
     if (rc == PF_HIP_OK) {
         hipError_t e = hipEventRecord(t0, s);
@@ -550,61 +552,56 @@ extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, co
     return rc;
 }
 
-__global__ void pf_k_nothing(uint32_t *p) { if (p && threadIdx.x == 0xffffffffu) *p = 0; }
-
-// Average time between two events recorded around an empty kernel, measured the same way
-// pf_hip_moe_profile_stages measures a stage: the fixed cost to subtract from a stage time
-// to estimate the kernel's own duration.
-extern "C" int pf_hip_event_overhead(size_t iters, float *ms_per_kernel) {
-    if (!ms_per_kernel || !iters) return PF_HIP_E_ARGUMENT;
-    if (need_device()) return PF_HIP_E_NO_DEVICE;
-    hipStream_t s = nullptr;
-    hipEvent_t a = nullptr, b = nullptr;
-    HIP_TRY(hipStreamCreate(&s));
-    HIP_TRY(hipEventCreate(&a));
-    HIP_TRY(hipEventCreate(&b));
-    float total = 0.0f;
-    int rc = PF_HIP_OK;
-    for (size_t i = 0; i < iters + 3 && rc == PF_HIP_OK; i++) {
-        float ms = 0.0f;
-        hipError_t e = hipEventRecord(a, s);
-        hipLaunchKernelGGL(pf_k_nothing, dim3(256), dim3(256), 0, s, (uint32_t *)nullptr);
-        if (e == hipSuccess) e = hipEventRecord(b, s);
-        if (e == hipSuccess) e = hipStreamSynchronize(s);
-        if (e == hipSuccess) e = hipEventElapsedTime(&ms, a, b);
-        if (e != hipSuccess) { pf_set_error("event overhead", e); rc = PF_HIP_E_RUNTIME; }
-        if (i >= 3) total += ms;
-    }
-    *ms_per_kernel = total / (float)iters;
-    (void)hipEventDestroy(a);
-    (void)hipEventDestroy(b);
-    (void)hipStreamDestroy(s);
-    return rc;
+extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
+                                        float *d_y, size_t tokens, size_t iters, float *elapsed_ms) {
+    if (!moe || !work || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
+    return time_graph_replay(moe, work, d_x, n_inputs, d_y, tokens, iters, 0, elapsed_ms);
 }
 
+// Kernel durations inside the dependent chain: the same graph replay with only the first
+// 1, 2, ... kernels of every forward launched; stage j's time is the difference between
+// the runs with j + 1 and with j kernels, divided by the forwards.  HIP events on the launch
+// stream bracket each replay.  The decode path has three kernels, the general path four
+// launches (the third being the routing pair); unused entries are zero.
 extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
                                          float *d_y, size_t tokens, size_t iters, float stage_ms[4]) {
-    if (!moe || !work || !d_x || !d_y || !n_inputs || !stage_ms) return PF_HIP_E_ARGUMENT;
-    const size_t H = moe->desc.hidden;
-    hipStream_t s = nullptr;
-    hipEvent_t marks[5];
-    HIP_TRY(hipStreamCreate(&s));
-    for (int j = 0; j < 5; j++) HIP_TRY(hipEventCreate(&marks[j]));
+    if (!moe || !work || !d_x || !d_y || !n_inputs || !stage_ms || !iters) return PF_HIP_E_ARGUMENT;
+    const bool decode = moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS && !work->force_general;
+    const int stages = decode ? 3 : 4;
+    float previous = 0.0f;
     for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
-    int rc = PF_HIP_OK;
-    work->marks = marks;
-    for (size_t i = 0; i < iters && rc == PF_HIP_OK; i++) {
-        rc = pf_hip_moe_forward_device(moe, work, d_x + (i % n_inputs) * tokens * H, H, d_y, H, tokens, s);
-        if (rc == PF_HIP_OK && hipStreamSynchronize(s) != hipSuccess) rc = PF_HIP_E_RUNTIME;
-        for (int j = 0; j < 4 && rc == PF_HIP_OK; j++) {
-            float ms = 0.0f;
-            if (hipEventElapsedTime(&ms, marks[j], marks[j + 1]) != hipSuccess) rc = PF_HIP_E_RUNTIME;
-            stage_ms[j] += ms;
-        }
+    for (int j = 0; j < stages; j++) {
+        float warm = 0.0f, ms = 0.0f;
+        int rc = time_graph_replay(moe, work, d_x, n_inputs, d_y, tokens, iters < 64 ? iters : 64, j + 1, &warm);
+        if (rc == PF_HIP_OK) rc = time_graph_replay(moe, work, d_x, n_inputs, d_y, tokens, iters, j + 1, &ms);
+        if (rc != PF_HIP_OK) return rc;
+        stage_ms[j] = (ms - previous) / (float)iters;
+        previous = ms;
     }
-    work->marks = nullptr;
-    for (int j = 0; j < 4; j++) stage_ms[j] /= (float)(iters ? iters : 1);
-    for (int j = 0; j < 5; j++) (void)hipEventDestroy(marks[j]);
-    (void)hipStreamDestroy(s);
+    return PF_HIP_OK;
+}
+
+
+
+// A plain copy of a known size: the reference point for hardware byte counters, which a
+// profiler reads in units that are easiest to pin against a kernel whose traffic is known.
+__global__ void pf_k_copy_probe(const uint4 *src, uint4 *dst, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+extern "C" int pf_hip_copy_probe(size_t bytes, size_t launches) {
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
+    bytes &= ~(size_t)15;
+    if (!bytes || !launches) return PF_HIP_E_ARGUMENT;
+    uint4 *src = nullptr, *dst = nullptr;
+    int rc = PF_HIP_OK;
+    if (hipMalloc((void **)&src, bytes) != hipSuccess || hipMalloc((void **)&dst, bytes) != hipSuccess) rc = PF_HIP_E_MEMORY;
+    if (rc == PF_HIP_OK && hipMemset(src, 1, bytes) != hipSuccess) rc = PF_HIP_E_RUNTIME;
+    for (size_t i = 0; i < launches && rc == PF_HIP_OK; i++)
+        hipLaunchKernelGGL(pf_k_copy_probe, dim3(2048), dim3(256), 0, nullptr, src, dst, bytes / 16);
+    if (rc == PF_HIP_OK && hipDeviceSynchronize() != hipSuccess) rc = PF_HIP_E_RUNTIME;
+    if (src) (void)hipFree(src);
+    if (dst) (void)hipFree(dst);
     return rc;
 }

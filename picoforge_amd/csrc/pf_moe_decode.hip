@@ -584,14 +584,13 @@ static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStre
 }
 
 template <int FMT, int NT>
-static void launch_decode(const PfKernelArgs &a, hipStream_t stream, hipEvent_t *marks) {
+static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_limit) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
     const size_t tab = table_words<FMT>() * 4;
-    // kernel 1
-    const int router_blocks = (E + 3) / 4;
-    if (marks) (void)hipEventRecord(marks[0], stream);
+    // kernel 1 (stage_limit, profiling: launch only the first so many kernels; 0 = all)
+    const int router_blocks = (E + 3) / 4, last = stage_limit ? stage_limit : 3;
     hipLaunchKernelGGL((pf_k_dec_router<NT>), dim3(router_blocks + 1), dim3(256), 0, stream, a, router_blocks);
-    if (marks) { (void)hipEventRecord(marks[1], stream); (void)hipEventRecord(marks[2], stream); }
+    if (last < 2) return;
     // kernel 2: the candidate stage uses up to 8 of waves 0..11 per token
     const int routed_blocks = NT * K * (I / 32), shared_blocks = Is / 32;
     const size_t lds2 = tab + (size_t)NT * image_words(H) * 4 + ((size_t)H + 3 * (size_t)E) * 4;
@@ -603,25 +602,24 @@ static void launch_decode(const PfKernelArgs &a, hipStream_t stream, hipEvent_t 
     else if (npl <= 2) launch_gate_up<FMT, NT, 2>(a, g2, lds2, stream, routed_blocks, parts, chunk);
     else if (npl <= 4) launch_gate_up<FMT, NT, 4>(a, g2, lds2, stream, routed_blocks, parts, chunk);
     else launch_gate_up<FMT, NT, 8>(a, g2, lds2, stream, routed_blocks, parts, chunk);   // experts <= 1024
-    if (marks) (void)hipEventRecord(marks[3], stream);
+    if (last < 3) return;
     // kernel 3
     const int rows_per_block = 64 / (I / 64), row_blocks = (H + rows_per_block - 1) / rows_per_block;
     hipLaunchKernelGGL((pf_k_dec_down<FMT, NT>), dim3(NT * row_blocks), dim3(64 * (K + 1)), tab, stream, a, row_blocks,
                        rows_per_block);
-    if (marks) (void)hipEventRecord(marks[4], stream);
 }
 
 template <int FMT>
-static void launch_decode_tokens(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks) {
+static void launch_decode_tokens(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     switch (tokens) {
-    case 1: launch_decode<FMT, 1>(a, stream, marks); break;
-    case 2: launch_decode<FMT, 2>(a, stream, marks); break;
-    case 3: launch_decode<FMT, 3>(a, stream, marks); break;
-    default: launch_decode<FMT, 4>(a, stream, marks); break;
+    case 1: launch_decode<FMT, 1>(a, stream, stage_limit); break;
+    case 2: launch_decode<FMT, 2>(a, stream, stage_limit); break;
+    case 3: launch_decode<FMT, 3>(a, stream, stage_limit); break;
+    default: launch_decode<FMT, 4>(a, stream, stage_limit); break;
     }
 }
 
-void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks) {
-    if (a.type[1] == PF_Q4_K) launch_decode_tokens<PF_Q4_K>(a, tokens, stream, marks);
-    else launch_decode_tokens<PF_IQ2_XXS>(a, tokens, stream, marks);
+void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    if (a.type[1] == PF_Q4_K) launch_decode_tokens<PF_Q4_K>(a, tokens, stream, stage_limit);
+    else launch_decode_tokens<PF_IQ2_XXS>(a, tokens, stream, stage_limit);
 }

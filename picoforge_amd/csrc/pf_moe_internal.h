@@ -51,12 +51,12 @@ struct PfHipWork {
     float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
     uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags;
     int *act_images, *shared_images;
-    void *marks;                     // hipEvent_t[5] while stage profiling, else null
+    int stage_limit;                 // profiling: launch only the first so many kernels of a forward; 0 = all
     int force_general;               // tests: run the general kernels even where the decode path applies
 };
 
 // pf_moe_kernels.hip
-void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks);
+void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 size_t pf_general_lds_bytes(const PfKernelArgs &a);
 // pf_moe_route.hip
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream);
@@ -74,7 +74,7 @@ void pf_launch_exact_decode(uint32_t type, const uint8_t *d_row, int k_storage, 
                             const uint64_t *grid, hipStream_t stream);
 // pf_moe_decode.hip
 bool pf_decode_supported(const PfHipMoeDesc &d);
-void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks);
+void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);
 // pf_moe_api.hip

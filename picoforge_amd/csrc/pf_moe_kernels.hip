@@ -232,18 +232,16 @@ size_t pf_general_lds_bytes(const PfKernelArgs &a) {
     return down > x ? down : x;
 }
 
-void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, hipEvent_t *marks) {
-    // marks (optional, 5 events): before stage 1 and after each of the four stages
-    const int units = a.experts + a.shared_inter + 1;
+void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    // stage_limit (profiling): launch only the first so many of the four stages; 0 = all
+    const int units = a.experts + a.shared_inter + 1, last = stage_limit ? stage_limit : 4;
     const size_t x_lds = (size_t)a.hidden * sizeof(float);
-    if (marks) (void)hipEventRecord(marks[0], stream);
     hipLaunchKernelGGL(pf_k_pre, dim3((units + 3) / 4, tokens), dim3(256), x_lds, stream, a);
-    if (marks) (void)hipEventRecord(marks[1], stream);
+    if (last < 2) return;
     pf_launch_route(a, tokens, stream);
-    if (marks) (void)hipEventRecord(marks[2], stream);
+    if (last < 3) return;
     hipLaunchKernelGGL(pf_k_gate_up, dim3((a.inter + 3) / 4, tokens * a.top_k), dim3(256), x_lds, stream, a);
-    if (marks) (void)hipEventRecord(marks[3], stream);
+    if (last < 4) return;
     const size_t act_lds = ((size_t)a.top_k * a.down_physical + a.shared_inter) * sizeof(float);
     hipLaunchKernelGGL(pf_k_down_combine, dim3((a.hidden + 3) / 4, tokens), dim3(256), act_lds, stream, a);
-    if (marks) (void)hipEventRecord(marks[4], stream);
 }
