@@ -4,18 +4,22 @@
 Default workload (the configuration the metric is quoted on): one MoE layer at
 hidden 2048 / 512 experts / top-10 / intermediate 512 with IQ2_XXS expert
 blocks, decode batch 1, seeded RMS-normalised tokens whose top-11 router logits
-are at least 1e-3 apart.  A step is one token through the layer; inputs and
+are at least 1e-3 apart.  A step is one token batch through the layer; inputs and
 weights are resident in HBM before the timed region; every step uses another
-token, hence other experts.
+input, hence other experts.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
+Workloads: iq2xxs_decode (default), q4k_decode, q4k_verify4 (4-token batches with
+about half of the experts shared between neighbours), q4k_prefill1024 (1024-token
+chunks, N(0,1) activations, Zipf(1.1) expert popularity).
+
 Prints one JSON line.  `value` is microseconds per layer per token (lower is
 better).  `roofline` is for the kernel that moves the most bytes, timed live
-with HIP events on the launch stream.  `cpu_baseline` times the CPU path (the reference's own
-compiled C when oracle/_ref is present, else the oracle port) on a bounded
-sample of the same tokens, single thread, and the same sample is used to check
-the GPU results (ids exact, outputs within 1e-3 + 1e-4 relative).
+with HIP events on the launch stream.  `cpu_baseline` times the CPU path (the
+reference's own compiled C when oracle/_ref is present, else the oracle port) on
+a bounded sample of the same tokens, single thread, and the same sample is used
+to check the GPU results (ids exact, outputs within 1e-3 + 1e-4 relative).
 """
 import argparse
 import ctypes as C
@@ -34,30 +38,31 @@ import picoforge_amd as pf  # noqa: E402
 from picoforge_amd import abi, workloads  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 
 WORKLOADS = {
-    "iq2xxs_decode": dict(type=abi.GGUF_IQ2_XXS, tokens=1, label="IQ2_XXS experts, decode batch 1"),
-    "q4k_decode": dict(type=abi.GGUF_Q4_K, tokens=1, label="Q4_K experts, decode batch 1"),
-    "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
+    "iq2xxs_decode": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=10000, warmup=200,
+                          label="IQ2_XXS experts, decode batch 1"),
+    "q4k_decode": dict(type=abi.GGUF_Q4_K, tokens=1, steps=10000, warmup=200, label="Q4_K experts, decode batch 1"),
+    "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, steps=2000, warmup=100,
+                        label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
+    "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10,
+                            label="Q4_K experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
 }
-STAGES = ["pf_k_dec_router (router logits)", "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
-          "pf_k_dec_down (down products, routed and shared, combine)"]
-
-
-def device_forward_sample(api, layer, x, tokens):
-    """Runs the first sample batches through the device path and returns y, ids, weights."""
-    outs = []
-    for b in range(len(x)):
-        _, y, ids, w = layer.forward(x[b].reshape(tokens, -1))
-        outs.append((y, ids, w))
-    return outs
+DECODE_STAGES = ["pf_k_dec_router (router logits)",
+                 "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
+                 "pf_k_dec_down (down products, routed and shared, combine)"]
+PREFILL_STAGES = ["pf_k_rows_to_half + pf_k_pf_router (fp16 copy of x, router logits by FP32 MFMA)",
+                  "routing + grouping (top-k, serial-order re-routes, histogram/scan/stable placement)",
+                  "pf_k_pf_gemm<gate_up> (grouped gate/up + SwiGLU by FP16 MFMA, then fp16 copy of the activations)",
+                  "pf_k_pf_gemm<down> + pf_k_pf_combine (grouped down by FP16 MFMA, slot-ordered combine)"]
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="iq2xxs_decode", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-sample", type=int, default=None, help="tokens timed on the CPU path (default ~15 s of work)")
     ap.add_argument("--seed", type=int, default=1)
@@ -68,21 +73,34 @@ def main():
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); use --gpus 1")
 
     wl = WORKLOADS[args.workload]
+    steps = args.steps if args.steps is not None else wl["steps"]
+    warmup = args.warmup if args.warmup is not None else wl["warmup"]
     api = pf.load_product()
     hip = api.hip
     if hip.device_count() < 1:
         sys.exit("no HIP device: the benchmark runs the HIP path only")
     cfg = workloads.measured_config()
     tokens = wl["tokens"]
+    prefill = tokens > 4
     t0 = time.time()
     weights = pf.LayerWeights.synthetic(cfg, wl["type"], seed=args.seed)
-    n_inputs = max(1, min(args.steps, 10000))
-    if tokens == 1:
+    if prefill:
+        # Zipf(1.1) popularity profile, flattened (logit bias -1.1 * 0.18 * ln rank) so that the busiest
+        # expert receives about 150 of the 1024 tokens, as the configuration states
+        workloads.zipf_router(weights, seed=args.seed, temperature=0.18)
+        n_inputs = max(1, min(steps, 4))
+        x = np.stack([workloads.prefill_chunk(weights, tokens, seed=args.seed + b) for b in range(n_inputs)])
+        load = workloads.expert_load(weights, x[0])
+        unique = float(np.count_nonzero(load))
+        info = {"active_experts_chunk0": int(unique), "max_tokens_per_expert": int(load.max()),
+                "median_tokens_per_expert": float(np.median(load)), "chunks": n_inputs}
+    elif tokens == 1:
+        n_inputs = max(1, min(steps, 10000))
         x, info = workloads.decode_tokens(weights, n_inputs, seed=args.seed)
         x = x.reshape(n_inputs, 1, cfg.hidden_size)
         unique = float(cfg.top_k)
     else:
-        n_inputs = min(n_inputs, 2000)
+        n_inputs = max(1, min(steps, 2000))
         x, info = workloads.verify_batches(weights, n_inputs, seed=args.seed)
         unique = info["mean_unique_experts"]
     prep_s = time.time() - t0
@@ -93,33 +111,55 @@ def main():
     d_y = hip.to_device(np.zeros((tokens, cfg.hidden_size), dtype=np.float32))
 
     ms = C.c_float()
-    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, args.warmup, C.byref(ms)), "warmup")
+    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, warmup, C.byref(ms)), "warmup")
     hip.check(hip.synchronize(), "sync")
     wall0 = time.perf_counter()
-    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, args.steps, C.byref(ms)), "timed loop")
+    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, steps, C.byref(ms)), "timed loop")
     hip.check(hip.synchronize(), "sync")
     wall_ms = (time.perf_counter() - wall0) * 1e3
-    ms_per_step = ms.value / args.steps
+    ms_per_step = ms.value / steps
     us_per_token = ms_per_step * 1e3 / tokens
     err_word = hip.from_device(hip.work_error_word(work), (1,), np.uint32)[0]
     exact = C.c_uint32()
     hip.work_exact_rows(work, C.byref(exact))
 
-    # Per-kernel durations inside the dependent chain: graph replays of the first 1, 2, 3
-    # kernels of every forward, bracketed by HIP events on the launch stream; a kernel's
-    # duration is the difference between consecutive replays (it includes the dispatch gap
-    # before it, as a profiler's start-to-end time of a dependent kernel does).
+    # Per-kernel durations inside the dependent chain: graph replays of the first 1, 2, ...
+    # kernels (stages) of every forward, bracketed by HIP events on the launch stream; a
+    # stage's duration is the difference between consecutive replays (it includes the dispatch
+    # gap before it, as a profiler's start-to-end time of a dependent kernel does).
     stage = (C.c_float * 4)()
-    hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(args.steps, 2000), stage), "stages")
-    stage_us = [max(float(stage[j]) * 1e3, 1e-3) for j in range(3)]
+    hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(steps, 2000), stage), "stages")
+    names = PREFILL_STAGES if prefill else DECODE_STAGES
+    stage_us = [max(float(stage[j]) * 1e3, 1e-3) for j in range(len(names))]
 
-    alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique)
     block, size = abi.BLOCK[wl["type"]]
-    h, i, s_i = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate
-    # algorithmic bytes per launch: what each kernel must read once
-    stage_bytes = [(cfg.experts + 1) * h * 4,
-                   unique * 2 * i * h // block * size + 2 * s_i * h // block * size,
-                   unique * h * i // block * size + h * s_i // block * size]
+    h, i, s_i, k = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate, cfg.top_k
+    extra = {}
+    if prefill:
+        # algorithmic bytes per launch: weights of the active experts once, activations once
+        pairs = tokens * k
+        stage_bytes = [tokens * h * 4 + (cfg.experts + 1) * h * 4 + tokens * h * 2,
+                       tokens * cfg.experts * 4 + pairs * 16,
+                       unique * 2 * i * h // block * size + 2 * s_i * h // block * size + (pairs + tokens) * h * 2
+                       + (pairs * i + tokens * s_i) * 4,
+                       unique * h * i // block * size + h * s_i // block * size + (pairs * i + tokens * s_i) * 2
+                       + (pairs + tokens) * h * 4 + tokens * h * 4]
+        alg_bytes = unique * 3 * i * h // block * size + 3 * s_i * h // block * size + (cfg.experts + 1) * h * 4 \
+            + 2 * tokens * h * 4
+        stage_flops = [2.0 * tokens * h * (cfg.experts + 1), 0.0, 2.0 * tokens * (k * 2 * h * i + 2 * h * s_i),
+                       2.0 * tokens * (k * i * h + s_i * h)]
+        flops = sum(stage_flops)
+        extra = {"prefill_tokens_per_s": round(tokens / (ms_per_step * 1e-3), 1),
+                 "flops_per_step": flops,
+                 "mfma_frac_of_fp16_dense_peak": round(flops / (ms_per_step * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                 "stage_tflops": {names[j].split()[0]: round(stage_flops[j] / (stage_us[j] * 1e-6) / 1e12, 1)
+                                  for j in (0, 2, 3)},
+                 "binding_roofline": "hbm: about 80 flop per weight byte at this chunk size, below the MFMA ridge"}
+    else:
+        alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique)
+        stage_bytes = [(cfg.experts + 1) * h * 4,
+                       unique * 2 * i * h // block * size + 2 * s_i * h // block * size,
+                       unique * h * i // block * size + h * s_i // block * size]
     dom = int(np.argmax(stage_bytes))
     achieved = stage_bytes[dom] / (stage_us[dom] * 1e-6) / 1e9
 
@@ -127,13 +167,25 @@ def main():
     ref = pf.load_reference()
     cpu_api, kind = (ref, "reference") if ref is not None else (pf.load_oracle(), "port")
     per_token_guess = 0.55 if wl["type"] == abi.GGUF_IQ2_XXS else 0.32
-    sample = args.cpu_sample or max(1, int(15.0 / per_token_guess / tokens))
-    sample = min(sample, n_inputs)
-    with pf.MoeLayer(cpu_api, cfg, weights, tokens) as cpu:
-        c0 = time.perf_counter()
-        cpu_out = [cpu.forward(x[b].reshape(tokens, -1))[1:] for b in range(sample)]
-        cpu_s = time.perf_counter() - c0
-    gpu_out = device_forward_sample(api, layer, x[:sample], tokens)
+    if prefill:
+        sample_tokens = min(tokens, args.cpu_sample or 48)
+        with pf.MoeLayer(cpu_api, cfg, weights, sample_tokens) as cpu:
+            c0 = time.perf_counter()
+            cpu_out = [cpu.forward(x[0][:sample_tokens])[1:]]
+            cpu_s = time.perf_counter() - c0
+        _, y, ids, w = layer.forward(x[0])
+        gpu_out = [(y[:sample_tokens], ids[:sample_tokens], w[:sample_tokens])]
+        sample_text = f"first {sample_tokens} tokens of chunk 0 (the CPU cost is linear in tokens), {cpu_s:.1f} s"
+    else:
+        sample = args.cpu_sample or max(1, int(15.0 / per_token_guess / tokens))
+        sample = min(sample, n_inputs)
+        sample_tokens = sample * tokens
+        with pf.MoeLayer(cpu_api, cfg, weights, tokens) as cpu:
+            c0 = time.perf_counter()
+            cpu_out = [cpu.forward(x[b].reshape(tokens, -1))[1:] for b in range(sample)]
+            cpu_s = time.perf_counter() - c0
+        gpu_out = [layer.forward(x[b].reshape(tokens, -1))[1:] for b in range(sample)]
+        sample_text = f"first {sample} steps ({sample_tokens} tokens) of the same inputs, {cpu_s:.1f} s"
     ids_equal = all((g[1] == c[1]).all() for g, c in zip(gpu_out, cpu_out))
     max_abs = max(float(np.abs(g[0] - c[0]).max()) for g, c in zip(gpu_out, cpu_out))
     within = all((np.abs(g[0] - c[0]) <= 1e-3 + 1e-4 * np.abs(c[0])).all() for g, c in zip(gpu_out, cpu_out))
@@ -141,29 +193,31 @@ def main():
     if args.copy_probe:
         hip.check(hip.copy_probe(args.copy_probe << 20, 3), "copy probe")
 
+    margins = "; top-11 logit margins >= 1e-3" if not prefill else ""
     result = {
-        "metric": "moe_decode_us_per_layer_token",
+        "metric": "moe_decode_us_per_layer_token" if not prefill else "moe_prefill_us_per_layer_token",
         "value": round(us_per_token, 3),
         "unit": "us/layer/token",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic",
+        "dtype": "f32" if not prefill else "f16 products, f32 accumulation",
+        "data": "synthetic",
         "config": {"workload": f"one MoE layer, hidden 2048, 512 experts, top-10, intermediate 512, shared 512; "
-                               f"{wl['label']}; {n_inputs} seeded inputs, top-11 logit margins >= 1e-3",
+                               f"{wl['label']}; {n_inputs} seeded inputs{margins}",
                    "tokens_per_step": tokens, "expert_format": {12: "Q4_K", 16: "IQ2_XXS"}[wl["type"]],
                    "unique_experts_per_step": unique, "inputs": info},
         "hbm_GBps_on_algorithmic_bytes": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         "algorithmic_bytes_per_step": int(alg_bytes),
         "tokens_per_s": round(tokens / (ms_per_step * 1e-3), 1),
-        "roofline": {"bound": "hbm", "kernel": STAGES[dom], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": names[dom], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "bytes_per_launch": int(stage_bytes[dom]), "us_per_launch": round(stage_us[dom], 3)},
-        "kernel_us": dict(zip(STAGES, [round(v, 3) for v in stage_us])),
-        "kernel_bytes": dict(zip(STAGES, [int(b) for b in stage_bytes])),
-        "cpu_baseline": {"value": round(cpu_s / (sample * tokens) * 1e6, 1), "unit": "us/layer/token", "cores": 1,
-                         "kind": kind, "sample": f"first {sample} steps ({sample * tokens} tokens) of the same inputs, "
-                                                   f"{cpu_s:.1f} s"},
+        "kernel_us": dict(zip(names, [round(v, 3) for v in stage_us])),
+        "kernel_bytes": dict(zip(names, [int(b) for b in stage_bytes])),
+        **extra,
+        "cpu_baseline": {"value": round(cpu_s / sample_tokens * 1e6, 1), "unit": "us/layer/token", "cores": 1,
+                         "kind": kind, "sample": sample_text},
         "parity_on_sample": {"ids_equal": bool(ids_equal), "within_1e-3_abs_1e-4_rel": bool(within),
                              "max_abs_err": max_abs, "error_word": int(err_word), "serial_order_reroutes": int(exact.value)},
         "wall_ms_timed_loop": round(wall_ms, 2), "prep_s": round(prep_s, 1),

@@ -149,6 +149,20 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         m->total_bytes += m->bytes[a];
     }
     m->decode_ready = pf_decode_supported(*desc);
+    // prefill path: squared norms of the router rows (the routing tolerance's bound)
+    m->prefill_ready = pf_prefill_supported(*desc);
+    if (m->prefill_ready) {
+        hipError_t e = hipMalloc((void **)&m->w_norm2, E * sizeof(float));
+        if (e == hipSuccess) {
+            pf_launch_row_norm2(reinterpret_cast<const float *>(m->w[0]), (int)E, (int)h, m->w_norm2, nullptr);
+            e = hipDeviceSynchronize();
+        }
+        if (e != hipSuccess) {
+            pf_set_error("prefill constants", e);
+            pf_hip_moe_destroy(m);
+            return e == hipErrorOutOfMemory ? PF_HIP_E_MEMORY : PF_HIP_E_RUNTIME;
+        }
+    }
     *out = m;
     return PF_HIP_OK;
 }
@@ -156,6 +170,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
 extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
     if (!m) return;
     for (int a = 0; a < 8; a++) if (m->w[a]) (void)hipFree(m->w[a]);
+    if (m->w_norm2) (void)hipFree(m->w_norm2);
     free(m);
 }
 
@@ -163,7 +178,8 @@ extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_byte
 
 // workspace layout: buffers carved from one allocation, each 256-byte aligned
 enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_SIMAGES, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS,
-       W_IMAGES, W_COUNT };
+       W_IMAGES, W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
+       W_P2R, W_R2P, W_GROUPBAD, W_TILES, W_COUNT };
 struct Carve { size_t offset[W_COUNT], total; };
 static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     Carve c;
@@ -187,6 +203,23 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_EXACT] = 256;
     want[W_FLAGS] = T * 4;
     want[W_IMAGES] = Td * K * Td * image;
+    // prefill path: fp16 copies, per-row scales, down products in expert order, grouping tables
+    const bool prefill = T > PF_DECODE_MAX_TOKENS && pf_prefill_supported(*d);
+    const size_t Tp = prefill ? T : 0, Is = d->shared_inter;
+    want[W_X16] = Tp * pf_prefill_half_row((int)H) * 2;
+    want[W_ACT16] = Tp * K * pf_prefill_half_row((int)I) * 2;
+    want[W_SACT16] = Tp * pf_prefill_half_row((int)Is) * 2;
+    want[W_XSCALE] = Tp * 4;
+    want[W_ACTSCALE] = Tp * K * 4;
+    want[W_SACTSCALE] = Tp * 4;
+    want[W_XMAX2] = Tp * 4;
+    want[W_DOWN] = (Tp * K + Tp) * H * 4;
+    want[W_COUNTS] = prefill ? E * 4 : 0;
+    want[W_OFFSETS] = prefill ? (E + 1) * 4 : 0;
+    want[W_P2R] = Tp * K * 4;
+    want[W_R2P] = Tp * K * 4;
+    want[W_GROUPBAD] = prefill ? 4 : 0;
+    want[W_TILES] = prefill ? (1 + (size_t)pf_prefill_max_tiles((int)T, (int)E, (int)K)) * 4 : 0;
     for (int j = 0; j < W_COUNT; j++) {
         c.offset[j] = c.total;
         c.total += (want[j] + 255) & ~(size_t)255;
@@ -229,6 +262,22 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     w->exact_rows = (uint32_t *)(base + c.offset[W_EXACT]);
     w->route_flags = (uint32_t *)(base + c.offset[W_FLAGS]);
     w->act_images = (int *)(base + c.offset[W_IMAGES]);
+    if (c.offset[W_GROUPBAD] != c.offset[W_X16]) {   // the prefill buffers were planned
+        w->x16 = (uint16_t *)(base + c.offset[W_X16]);
+        w->act16 = (uint16_t *)(base + c.offset[W_ACT16]);
+        w->sact16 = (uint16_t *)(base + c.offset[W_SACT16]);
+        w->x_scale = (float *)(base + c.offset[W_XSCALE]);
+        w->act_scale = (float *)(base + c.offset[W_ACTSCALE]);
+        w->sact_scale = (float *)(base + c.offset[W_SACTSCALE]);
+        w->x_max2 = (float *)(base + c.offset[W_XMAX2]);
+        w->down = (float *)(base + c.offset[W_DOWN]);
+        w->counts = (uint32_t *)(base + c.offset[W_COUNTS]);
+        w->offsets = (uint32_t *)(base + c.offset[W_OFFSETS]);
+        w->pair_to_row = (uint32_t *)(base + c.offset[W_P2R]);
+        w->row_to_pair = (uint32_t *)(base + c.offset[W_R2P]);
+        w->group_bad = (uint32_t *)(base + c.offset[W_GROUPBAD]);
+        w->tiles = (uint32_t *)(base + c.offset[W_TILES]);
+    }
     *out = w;
     return PF_HIP_OK;
 }
@@ -291,6 +340,11 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale;
     a.act_images = w->act_images; a.shared_images = w->shared_images; a.uniq = w->uniq;
     a.error_word = w->error_word; a.exact_rows = w->exact_rows; a.route_flags = w->route_flags;
+    a.x16 = w->x16; a.act16 = w->act16; a.sact16 = w->sact16;
+    a.x_scale = w->x_scale; a.act_scale = w->act_scale; a.sact_scale = w->sact_scale; a.x_max2 = w->x_max2;
+    a.w_norm2 = m->w_norm2; a.down = w->down;
+    a.counts = w->counts; a.offsets = w->offsets; a.pair_to_row = w->pair_to_row; a.row_to_pair = w->row_to_pair;
+    a.group_bad = w->group_bad; a.tiles = w->tiles;
     return a;
 }
 
@@ -308,6 +362,8 @@ extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, c
     const bool aligned = (x_pitch % 4 == 0) && ((uintptr_t)d_x % 16 == 0);
     if (moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS && aligned && !work->force_general) {
         pf_launch_decode(a, (int)tokens, s, work->stage_limit);
+    } else if (moe->prefill_ready && work->down && tokens > PF_DECODE_MAX_TOKENS && aligned && !work->force_general) {
+        pf_launch_prefill(a, (int)tokens, s, work->stage_limit);
     } else {
         // the general kernels stage one token's activations in LDS
         const size_t lds_route = ((size_t)d->hidden + 3 * (size_t)d->experts) * 4;

@@ -32,6 +32,14 @@ struct PfKernelArgs {
     uint32_t *error_word;
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
     uint32_t *route_flags;           // [tokens] 1 = route again in serial order
+    // prefill path
+    uint16_t *x16, *act16, *sact16;  // fp16 forms of x, act (pairs in expert order), shared act: per row the high
+                                     // parts, the low parts, then 8 + 8 group-sum parts per 256 columns
+    float *x_scale, *act_scale, *sact_scale;   // per row: the power of two the fp16 form was divided by
+    float *x_max2;                   // [tokens] largest squared magnitude of the row
+    const float *w_norm2;            // [experts] squared norm of each router row
+    float *down;                     // [pairs + tokens, hidden] down products in expert order, then the shared expert's
+    uint32_t *counts, *offsets, *pair_to_row, *row_to_pair, *group_bad, *tiles;
 };
 
 struct PfHipMoe {
@@ -43,6 +51,8 @@ struct PfHipMoe {
     uint32_t *iq2_signed;
     size_t total_bytes;
     bool decode_ready;               // shapes and formats the specialised decode kernels cover
+    bool prefill_ready;              // shapes and formats the matrix-core prefill kernels cover
+    float *w_norm2;                  // [experts] squared norm of each router row
 };
 
 struct PfHipWork {
@@ -51,7 +61,10 @@ struct PfHipWork {
     float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
     uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags;
     int *act_images, *shared_images;
-    int stage_limit;                 // profiling: launch only the first so many kernels of a forward; 0 = all
+    uint16_t *x16, *act16, *sact16;  // prefill buffers (allocated when cap exceeds the decode path's batch)
+    float *x_scale, *act_scale, *sact_scale, *x_max2, *down;
+    uint32_t *counts, *offsets, *pair_to_row, *row_to_pair, *group_bad, *tiles;
+    int stage_limit;                // profiling: launch only the first so many kernels of a forward; 0 = all
     int force_general;               // tests: run the general kernels even where the decode path applies
 };
 
@@ -77,6 +90,12 @@ bool pf_decode_supported(const PfHipMoeDesc &d);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);
+// pf_moe_prefill.hip
+bool pf_prefill_supported(const PfHipMoeDesc &d);
+void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_row_norm2(const float *d_w, int rows, int cols, float *d_out, hipStream_t stream);
+size_t pf_prefill_half_row(int cols);   // halfs per row of the fp16 form of a matrix with `cols` columns
+int pf_prefill_max_tiles(int tokens, int experts, int top_k);
 // pf_moe_api.hip
 const uint64_t *pf_device_iq2_grid(void);
 const uint32_t *pf_device_iq2_signed(void);

@@ -1,0 +1,478 @@
+// Prefill path: a chunk of tokens through one MoE layer as grouped matrix products on the
+// matrix cores.
+//
+//   pf_k_rows_to_half   f32 rows -> power-of-two scaled fp16 pairs (high + low part) and the
+//                       per-32-group sums, the scale, max^2, finite check
+//   pf_k_pf_router      router logits [T, E] (+ the shared router as column E) by FP32 MFMA
+//   routing, grouping   the kernels of pf_moe_route.hip (serial-order re-route of close tokens,
+//                       histogram / scan / stable placement)
+//   pf_k_pf_gemm        grouped product over the rows of each expert (the shared expert is
+//                       expert E with every token) on v_mfma_f32_32x32x16_f16; gate/up with
+//                       the SwiGLU epilogue, or down
+//   pf_k_pf_combine     slot-ordered weighted sum of the down rows, then the shared branch
+//
+// Numerics.  A Q4_K weight is d * (scale * code) - dmin * min (src/qwen4_packed.c:86-93) with
+// 6-bit scale and min and a 4-bit code, so scale * code <= 945 and min <= 63 are integers that
+// fp16 holds exactly.  The matrix cores therefore multiply exact integer weight operands:
+// P = sum_k (scale * code)_k x_k over a 256-block and Q = sum_g min_g * (sum of x over group g),
+// and the block's d and dmin are applied in FP32: acc += d * P - dmin * Q.  Activations are
+// scaled per row by a power of two so that the largest magnitude lies in [0.5, 1) and split
+// into two fp16 parts x = hi + lo (22 significant bits); every product is exact in the FP32
+// accumulators, so the result differs from the reference's serial FP32 sum by accumulation
+// order and the 2^-22 activation rounding only.
+#include "pf_moe_internal.h"
+
+typedef _Float16 half_t;
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+#define A_PITCH 264   // halfs per LDS row of a 256-wide activation tile: 528 bytes, 33 sixteen-byte slots
+#define S_PITCH 24    // halfs per LDS row of the group sums (16 used)
+
+// halfs per row of a converted matrix: high parts, low parts, per 256-block 8 + 8 group sums
+__host__ __device__ constexpr size_t pf_half_row(int cols) { return 2 * (size_t)cols + (size_t)cols / 16; }
+
+// ---- rows to scaled fp16 pairs ------------------------------------------------------------------
+// One workgroup per row (cols a multiple of 256).  scale = 2^e with max|row| / scale in
+// [0.5, 1) (1 for a zero row).  Thread j converts the eight values 8j..8j+7; four neighbouring
+// threads form one 32-group.
+__global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_t src_pitch, int cols, half_t *dst,
+                                                         float *scale_out, float *max2_out, uint32_t *error_word) {
+    __shared__ float part[4];
+    const size_t row = blockIdx.x;
+    const float *s = src + row * src_pitch;
+    float m = 0.0f;
+    bool bad = false;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        const float v = s[c];
+        bad |= !pf_finite(v);
+        m = fmaxf(m, fabsf(v));
+    }
+    m = pf_wave_max(m);
+    if (pf_lane() == 0) part[threadIdx.x >> 6] = m;
+    if (__any(bad) && pf_lane() == 0) atomicOr(error_word, PF_HIP_ERR_NONFINITE);
+    __syncthreads();
+    m = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
+    int e = (__float_as_int(m) >> 23) & 255;                  // m in [2^(e-127), 2^(e-126))
+    e = (e == 0 || e == 255) ? 126 : min(e, 252);             // zero, subnormal or nonfinite row: scale 1
+    const float scale = __int_as_float((e + 1) << 23);        // 2^(e-126)
+    const float inv = __int_as_float((253 - e) << 23);        // 2^(126-e)
+    half_t *out = dst + row * pf_half_row(cols);
+    for (int j = threadIdx.x; j < cols / 8; j += blockDim.x) {
+        const float4 a = reinterpret_cast<const float4 *>(s)[2 * j], b = reinterpret_cast<const float4 *>(s)[2 * j + 1];
+        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        half8v hi, lo;
+        float sum = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const float x = v[c] * inv;
+            const half_t h = (half_t)x, l = (half_t)(x - (float)h);
+            hi[c] = h;
+            lo[c] = l;
+            sum += (float)h + (float)l;
+        }
+        *reinterpret_cast<half8v *>(out + 8 * j) = hi;
+        *reinterpret_cast<half8v *>(out + cols + 8 * j) = lo;
+        sum += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sum), 0xB1, 0xF, 0xF, true));   // quad xor 1
+        sum += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sum), 0x4E, 0xF, 0xF, true));   // quad xor 2
+        if ((j & 3) == 0) {
+            const int g = j >> 2;
+            const half_t sh = (half_t)sum, sl = (half_t)(sum - (float)sh);
+            out[2 * cols + 16 * (g >> 3) + (g & 7)] = sh;
+            out[2 * cols + 16 * (g >> 3) + 8 + (g & 7)] = sl;
+        }
+    }
+    if (threadIdx.x == 0) {
+        scale_out[row] = scale;
+        if (max2_out) max2_out[row] = m * m;
+    }
+}
+
+// squared norm of every router row (once, at upload)
+__global__ void __launch_bounds__(64) pf_k_row_norm2(const float *w, int cols, float *out) {
+    const float *r = w + (size_t)blockIdx.x * cols;
+    float s = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += 64) s = fmaf(r[c], r[c], s);
+    s = pf_wave_sum(s);
+    if (threadIdx.x == 0) out[blockIdx.x] = s;
+}
+
+void pf_launch_row_norm2(const float *d_w, int rows, int cols, float *d_out, hipStream_t stream) {
+    hipLaunchKernelGGL(pf_k_row_norm2, dim3(rows), dim3(64), 0, stream, d_w, cols, d_out);
+}
+
+// ---- router logits by FP32 MFMA ----------------------------------------------------------------
+// Workgroup = 2 x 2 waves, each a 32-token x 32-expert tile; operands straight from global memory
+// (the lines a lane touches are consumed over the following iterations from the vector cache).
+// Column E is the shared router.  Also writes the routing tolerance's bound on the sum of
+// squared products, max(x)^2 * |w_e|^2.
+__global__ void __launch_bounds__(256) pf_k_pf_router(PfKernelArgs a, int tokens) {
+    const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
+    const int t0 = blockIdx.x * 64 + 32 * (wave & 1), e0 = blockIdx.y * 64 + 32 * (wave >> 1);
+    if (t0 >= tokens || e0 > E) return;
+    const int i = lane & 31, kk = lane >> 5;
+    const int t = min(t0 + i, tokens - 1), e = min(e0 + i, E);
+    const float4 *xp = reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch) + kk;
+    const float4 *wp = reinterpret_cast<const float4 *>(e < E ? a.w[0] + (size_t)e * H * 4 : a.w[7]) + kk;
+    float16v acc = {0};
+#pragma unroll 4
+    for (int q = 0; q < H / 8; q++) {
+        const float4 xv = xp[2 * q], wv = wp[2 * q];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.x, wv.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.y, wv.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.z, wv.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.w, wv.w, acc, 0, 0, 0);
+    }
+    const int col = e0 + i;   // this lane's expert
+    const float wn = col < E ? a.w_norm2[col] : 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int row = t0 + 8 * (r >> 2) + 4 * kk + (r & 3);
+        if (row >= tokens || col > E) continue;
+        const float z = acc[r];
+        if (col < E) {
+            a.logits[(size_t)row * E + col] = z;
+            a.logit_ssq[(size_t)row * E + col] = a.x_max2[row] * wn;
+        } else {
+            a.shared_scale[row] = pf_sigmoid(z);
+            if (!pf_finite(z)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        }
+    }
+}
+
+// ---- grouped product ------------------------------------------------------------------------------
+enum { PF_GEMM_GATE_UP = 0, PF_GEMM_DOWN = 1 };
+
+struct Q4Raw { uint4 hdr; uint4 q[4]; };   // one lane's share of a row's 144-byte block: header + 16 bytes per 64 weights
+
+__device__ __forceinline__ void q4_load(Q4Raw &r, const uint8_t *block, int h) {
+    r.hdr = *reinterpret_cast<const uint4 *>(block);
+#pragma unroll
+    for (int j = 0; j < 4; j++) r.q[j] = *reinterpret_cast<const uint4 *>(block + 16 + 32 * j + 16 * h);
+}
+
+// 6-bit scale and min of group g from the 12 packed bytes (src/qwen4_packed.c:88-91)
+__device__ __forceinline__ void q4_scale_min(const Q4Raw &r, int g, uint32_t &sc, uint32_t &mn) {
+    const uint32_t w[3] = {r.hdr.y, r.hdr.z, r.hdr.w};
+    const int sh = 8 * (g & 3);
+    if (g < 4) {
+        sc = (w[0] >> sh) & 63u;
+        mn = (w[1] >> sh) & 63u;
+    } else {
+        const uint32_t hi = (w[2] >> sh) & 255u, lo_s = (w[0] >> sh) & 255u, lo_m = (w[1] >> sh) & 255u;
+        sc = (hi & 15u) | ((lo_s & 192u) >> 2);
+        mn = (hi >> 4) | ((lo_m & 192u) >> 2);
+    }
+}
+
+// eight codes (two dwords of nibbles, nibble position nib) times the group's scale, exact in fp16:
+// a nibble under the exponent byte 0x64 reads as 1024 + q, and (1024 + q) * s - 1024 * s = q * s
+__device__ __forceinline__ half8v q4_scaled_codes(uint32_t w0, uint32_t w1, int nib, half2v s2, half2v c1024) {
+    const uint32_t q0 = (w0 >> (4 * nib)) & 0x0F0F0F0Fu, q1 = (w1 >> (4 * nib)) & 0x0F0F0F0Fu;
+    const uint32_t bias = 0x64646464u;
+    const half2v p0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q0, 0x04010400u));
+    const half2v p1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q0, 0x04030402u));
+    const half2v p2 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q1, 0x04010400u));
+    const half2v p3 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q1, 0x04030402u));
+    const half2v v0 = p0 * s2 - c1024, v1 = p1 * s2 - c1024, v2 = p2 * s2 - c1024, v3 = p3 * s2 - c1024;
+    return half8v{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+}
+
+// One pass: MT row tiles of 32 rows against this wave's two 32-row weight tiles, all K.
+// Lane (n = lane % 32, h = lane / 32) owns weight row n of its tiles and, per 64 weights, the
+// 16 bytes [16h, 16h + 16) of the 32-byte nibble run: chunk c = 2h + c2 (c2 = 0, 1) of nibble
+// position nib is k = 64j + 32 nib + 8c + 0..7, one MFMA per (c2, nib) and activation part.
+template <int MT>
+__device__ __forceinline__ void gemm_pass(half_t *tile_h, half_t *tile_l, half_t *tile_s, const uint32_t *src_row,
+                                          const half_t *a16, int a_cols, const uint8_t *wrow0, const uint8_t *wrow1,
+                                          int kblocks, int rows_here, float16v (&acc)[2][MT]) {
+    const int lane = pf_lane(), n = lane & 31, h = lane >> 5;
+    const size_t a_pitch = pf_half_row(a_cols);
+    Q4Raw raw0, raw1;
+    q4_load(raw0, wrow0, h);
+    q4_load(raw1, wrow1, h);
+    for (int kb = 0; kb < kblocks; kb++) {
+        __syncthreads();   // the previous tile has been consumed
+        // activation tile: per row 32 + 32 sixteen-byte chunks of the two parts and 2 of the group sums
+        for (int i = threadIdx.x; i < 32 * MT * 66; i += 256) {
+            const int m = i / 66, c = i % 66;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            const half_t *row = a16 + (size_t)src_row[m] * a_pitch;
+            if (c < 32) {
+                if (m < rows_here) v = *reinterpret_cast<const uint4 *>(row + 256 * kb + 8 * c);
+                *reinterpret_cast<uint4 *>(tile_h + m * A_PITCH + 8 * c) = v;
+            } else if (c < 64) {
+                if (m < rows_here) v = *reinterpret_cast<const uint4 *>(row + a_cols + 256 * kb + 8 * (c - 32));
+                *reinterpret_cast<uint4 *>(tile_l + m * A_PITCH + 8 * (c - 32)) = v;
+            } else {
+                if (m < rows_here) v = *reinterpret_cast<const uint4 *>(row + 2 * a_cols + 16 * kb + 8 * (c - 64));
+                *reinterpret_cast<uint4 *>(tile_s + m * S_PITCH + 8 * (c - 64)) = v;
+            }
+        }
+        const Q4Raw cur0 = raw0, cur1 = raw1;
+        if (kb + 1 < kblocks) {   // next block's bytes travel while this one is multiplied
+            q4_load(raw0, wrow0 + 144 * (kb + 1), h);
+            q4_load(raw1, wrow1 + 144 * (kb + 1), h);
+        }
+        __syncthreads();
+        const float d0 = pf_half_bits_to_float(cur0.hdr.x & 0xffffu), m0 = pf_half_bits_to_float(cur0.hdr.x >> 16);
+        const float d1 = pf_half_bits_to_float(cur1.hdr.x & 0xffffu), m1 = pf_half_bits_to_float(cur1.hdr.x >> 16);
+        // Q: the eight minima against the eight group sums (high parts in k 0..7, low parts in k 8..15)
+        half8v min0, min1;
+        half2v s2[2][8], c2k[2][8];
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            uint32_t sc, mn;
+            q4_scale_min(cur0, g, sc, mn);
+            min0[g] = (half_t)(int)mn;
+            s2[0][g] = half2v{(half_t)(int)sc, (half_t)(int)sc};
+            c2k[0][g] = half2v{(half_t)(int)(sc << 10), (half_t)(int)(sc << 10)};
+            q4_scale_min(cur1, g, sc, mn);
+            min1[g] = (half_t)(int)mn;
+            s2[1][g] = half2v{(half_t)(int)sc, (half_t)(int)sc};
+            c2k[1][g] = half2v{(half_t)(int)(sc << 10), (half_t)(int)(sc << 10)};
+        }
+        float16v part[2][MT];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+            const half8v as = *reinterpret_cast<const half8v *>(tile_s + (32 * mt + n) * S_PITCH + 8 * h);
+            const float16v zero = {0};
+            const float16v q0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min0, zero, 0, 0, 0);
+            const float16v q1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min1, zero, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[0][mt][r] = fmaf(-m0, q0[r], acc[0][mt][r]);
+                acc[1][mt][r] = fmaf(-m1, q1[r], acc[1][mt][r]);
+            }
+            part[0][mt] = zero;
+            part[1][mt] = zero;
+        }
+        // P: scale * code against both activation parts
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+#pragma unroll
+            for (int nib = 0; nib < 2; nib++) {
+                const int g = 2 * j + nib;
+#pragma unroll
+                for (int c2 = 0; c2 < 2; c2++) {
+                    const uint4 w0 = cur0.q[j], w1 = cur1.q[j];
+                    const half8v b0 = q4_scaled_codes(c2 ? w0.z : w0.x, c2 ? w0.w : w0.y, nib, s2[0][g], c2k[0][g]);
+                    const half8v b1 = q4_scaled_codes(c2 ? w1.z : w1.x, c2 ? w1.w : w1.y, nib, s2[1][g], c2k[1][g]);
+                    const int k = 64 * j + 32 * nib + 16 * h + 8 * c2;
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        const half8v ah = *reinterpret_cast<const half8v *>(tile_h + (32 * mt + n) * A_PITCH + k);
+                        const half8v al = *reinterpret_cast<const half8v *>(tile_l + (32 * mt + n) * A_PITCH + k);
+                        part[0][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, part[0][mt], 0, 0, 0);
+                        part[1][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, part[1][mt], 0, 0, 0);
+                        part[0][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b0, part[0][mt], 0, 0, 0);
+                        part[1][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b1, part[1][mt], 0, 0, 0);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc[0][mt][r] = fmaf(d0, part[0][mt][r], acc[0][mt][r]);
+                acc[1][mt][r] = fmaf(d1, part[1][mt][r], acc[1][mt][r]);
+            }
+        }
+    }
+}
+
+struct GemmTarget {   // what one workgroup of the grouped product works on
+    bool shared;
+    int first, count, inter, kblocks, a_cols, slab;
+    const uint8_t *w0, *w1;
+    const half_t *a16;
+    const float *a_scale;
+};
+
+template <int MODE, int MT>
+__device__ __forceinline__ void gemm_rows(const PfKernelArgs &a, const GemmTarget &g, int m0, int rows_here, half_t *tile_h,
+                                          half_t *tile_l, half_t *tile_s, uint32_t *src_row, float *row_scale) {
+    const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5, K = a.top_k;
+    __syncthreads();
+    for (int m = threadIdx.x; m < 32 * MT; m += 256) {
+        uint32_t src = 0;
+        float sc = 0.0f;
+        if (m < rows_here) {
+            if (MODE == PF_GEMM_GATE_UP) src = g.shared ? (uint32_t)(m0 + m) : a.row_to_pair[g.first + m0 + m] / (uint32_t)K;
+            else src = g.shared ? (uint32_t)(m0 + m) : (uint32_t)(g.first + m0 + m);
+            sc = g.a_scale[src];
+        }
+        src_row[m] = src;
+        row_scale[m] = sc;
+    }
+    float16v acc[2][MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) { acc[0][mt] = float16v{0}; acc[1][mt] = float16v{0}; }
+    gemm_pass<MT>(tile_h, tile_l, tile_s, src_row, g.a16, g.a_cols, g.w0, g.w1, g.kblocks, rows_here, acc);
+    // epilogue: the lane holds column n of its two tiles; register r of tile mt is row
+    // 32 mt + 8 (r / 4) + 4 h + r % 4
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = 32 * mt + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (m >= rows_here) continue;
+            const float rs = row_scale[m];
+            if (MODE == PF_GEMM_GATE_UP) {
+                const int unit = 128 * g.slab + 32 * wave + n;
+                if (unit >= g.inter) continue;
+                const float gate = acc[0][mt][r] * rs, up = acc[1][mt][r] * rs;
+                const float v = pf_silu(gate) * up;
+                if (g.shared) a.shared_act[(size_t)(m0 + m) * g.inter + unit] = v;
+                else a.act[(size_t)(g.first + m0 + m) * g.inter + unit] = v;
+            } else {
+                const int r0 = 256 * g.slab + 64 * wave + n;
+                float *out = a.down + (size_t)(g.first + m0 + m) * a.hidden;
+                if (r0 < a.hidden) out[r0] = acc[0][mt][r] * rs;
+                if (r0 + 32 < a.hidden) out[r0 + 32] = acc[1][mt][r] * rs;
+            }
+        }
+    }
+}
+
+// Row tiles: every expert's rows (the shared expert = expert E with all tokens) cut into tiles of
+// 32; tiles[0] = count, tiles[1 + i] = expert | (tile index within the expert) << 16.
+__global__ void __launch_bounds__(256) pf_k_pf_tiles(const uint32_t *offsets, int E, int tokens, uint32_t *tiles) {
+    __shared__ uint32_t part[256];
+    const int tid = threadIdx.x, per = (E + 1 + 255) / 256, lo = tid * per, hi = min(E + 1, lo + per);
+    uint32_t s = 0;
+    for (int e = lo; e < hi; e++) s += ((e < E ? offsets[e + 1] - offsets[e] : (uint32_t)tokens) + 31u) / 32u;
+    part[tid] = s;
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t run = 0;
+        for (int i = 0; i < 256; i++) { const uint32_t v = part[i]; part[i] = run; run += v; }
+        tiles[0] = run;
+    }
+    __syncthreads();
+    uint32_t at = part[tid];
+    for (int e = lo; e < hi; e++) {
+        const uint32_t n = ((e < E ? offsets[e + 1] - offsets[e] : (uint32_t)tokens) + 31u) / 32u;
+        for (uint32_t i = 0; i < n; i++) tiles[1 + at + i] = (uint32_t)e | (i << 16);
+        at += n;
+    }
+}
+
+// Workgroup (row tile, slab): 4 waves, each with two 32-row weight tiles (gate + up of 32 units,
+// or 2 x 32 down rows) against the tile's 32 rows.
+template <int MODE>
+__global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, int slabs) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    half_t *tile_h = reinterpret_cast<half_t *>(lds_raw), *tile_l = tile_h + 32 * A_PITCH, *tile_s = tile_l + 32 * A_PITCH;
+    __shared__ uint32_t src_row[32];
+    __shared__ float row_scale[32];
+    const int E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31;
+    const uint32_t tile = blockIdx.x / slabs;
+    if (tile >= a.tiles[0]) return;
+    const uint32_t entry = a.tiles[1 + tile];
+    const int expert = entry & 0xffffu, m0 = 32 * (int)(entry >> 16);
+    GemmTarget g;
+    g.slab = blockIdx.x % slabs;
+    g.shared = expert == E;
+    const int P = tokens * a.top_k;
+    g.first = g.shared ? P : (int)a.offsets[expert];
+    g.count = g.shared ? tokens : (int)a.offsets[expert + 1] - g.first;
+    if (g.count <= m0) return;
+    g.inter = g.shared ? a.shared_inter : a.inter;
+    const size_t ex = g.shared ? 0 : (size_t)expert;
+    if (MODE == PF_GEMM_GATE_UP) {
+        const int tg = g.shared ? 4 : 1;
+        if (128 * g.slab >= g.inter) return;
+        const int u = min(128 * g.slab + 32 * wave + n, g.inter - 1);
+        g.w0 = a.w[tg] + ex * a.expert_bytes[tg] + (size_t)u * a.row_bytes[tg];
+        g.w1 = a.w[tg + 1] + ex * a.expert_bytes[tg + 1] + (size_t)u * a.row_bytes[tg + 1];
+        g.kblocks = a.hidden / 256; g.a_cols = a.hidden;
+        g.a16 = reinterpret_cast<const half_t *>(a.x16); g.a_scale = a.x_scale;
+    } else {
+        const int td = g.shared ? 6 : 3, r0 = 256 * g.slab + 64 * wave + n;
+        g.w0 = a.w[td] + ex * a.expert_bytes[td] + (size_t)min(r0, a.hidden - 1) * a.row_bytes[td];
+        g.w1 = a.w[td] + ex * a.expert_bytes[td] + (size_t)min(r0 + 32, a.hidden - 1) * a.row_bytes[td];
+        g.kblocks = g.inter / 256; g.a_cols = g.inter;
+        g.a16 = reinterpret_cast<const half_t *>(g.shared ? a.sact16 : a.act16);
+        g.a_scale = g.shared ? a.sact_scale : a.act_scale;
+    }
+    gemm_rows<MODE, 1>(a, g, m0, min(32, g.count - m0), tile_h, tile_l, tile_s, src_row, row_scale);
+}
+
+// ---- combine ---------------------------------------------------------------------------------------
+// y[t] = sum over slots in order of weight * down row, then + sigmoid * shared down row
+// (src/qwen4_moe.c:362-372)
+__global__ void __launch_bounds__(256) pf_k_pf_combine(PfKernelArgs a, int tokens) {
+    const int t = blockIdx.x, H = a.hidden, K = a.top_k, P = tokens * K;
+    __shared__ uint32_t rows[64];
+    __shared__ float weights[64];
+    if ((int)threadIdx.x < K) {
+        rows[threadIdx.x] = a.pair_to_row[(size_t)t * K + threadIdx.x];
+        weights[threadIdx.x] = a.route_weights[(size_t)t * K + threadIdx.x];
+    }
+    __syncthreads();
+    const float ss = a.shared_scale[t];
+    bool bad = false;
+    for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        float sum = 0.0f;
+        for (int s = 0; s < K; s++) {
+            const float term = weights[s] * a.down[(size_t)rows[s] * H + c];
+            sum += term;
+        }
+        const float y = sum + ss * a.down[(size_t)(P + t) * H + c];
+        bad |= !pf_finite(y);
+        a.y[(size_t)t * a.y_pitch + c] = y;
+    }
+    if (__any(bad) && pf_lane() == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+}
+
+// ---- dispatch --------------------------------------------------------------------------------------
+bool pf_prefill_supported(const PfHipMoeDesc &d) {
+    for (int j = 1; j <= 6; j++)
+        if (d.type[j] != PF_Q4_K) return false;
+    if (d.hidden % 256 || d.inter % 256 || d.shared_inter % 256 || d.down_physical != d.inter) return false;
+    if (d.top_k > 64 || d.top_k >= d.experts || d.experts >= 65535) return false;
+    return true;
+}
+
+size_t pf_prefill_half_row(int cols) { return pf_half_row(cols); }
+// sum over experts of ceil(rows / 32) <= pairs / 32 + experts, plus the shared expert's tiles
+int pf_prefill_max_tiles(int tokens, int experts, int top_k) {
+    return (int)(((size_t)tokens * top_k) / 32 + experts + (tokens + 31) / 32 + 1);
+}
+
+template <int MODE>
+static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_t stream) {
+    const size_t lds = (size_t)(2 * 32 * A_PITCH + 32 * S_PITCH) * sizeof(half_t);
+    // the tile count is only known on the device: launch its upper bound, surplus workgroups exit at once
+    const int max_tiles = pf_prefill_max_tiles(tokens, a.experts, a.top_k);
+    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3(max_tiles * slabs), dim3(256), lds, stream, a, tokens, slabs);
+}
+
+void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    const int H = a.hidden, E = a.experts, K = a.top_k, I = a.inter, Is = a.shared_inter, P = tokens * K;
+    const int last = stage_limit ? stage_limit : 4;
+    // stage 1: fp16 parts of x, router logits
+    hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.x, a.x_pitch, H, (half_t *)a.x16, a.x_scale,
+                       a.x_max2, a.error_word);
+    hipLaunchKernelGGL(pf_k_pf_router, dim3((tokens + 63) / 64, (E + 1 + 63) / 64), dim3(256), 0, stream, a, tokens);
+    if (last < 2) return;
+    // stage 2: routes and grouping
+    pf_launch_route(a, tokens, stream);
+    pf_group_pairs_device(a.ids, tokens, E, K, a.counts, a.offsets, a.pair_to_row, a.row_to_pair, a.group_bad, stream);
+    hipLaunchKernelGGL(pf_k_pf_tiles, dim3(1), dim3(256), 0, stream, a.offsets, E, tokens, a.tiles);
+    if (last < 3) return;
+    // stage 3: gate/up + SwiGLU, then fp16 parts of the activation rows
+    const int gi = I > Is ? I : Is;
+    launch_gemm<PF_GEMM_GATE_UP>(a, tokens, (gi + 127) / 128, stream);
+    hipLaunchKernelGGL(pf_k_rows_to_half, dim3(P), dim3(256), 0, stream, a.act, (size_t)I, I, (half_t *)a.act16, a.act_scale,
+                       (float *)nullptr, a.error_word);
+    hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.shared_act, (size_t)Is, Is,
+                       (half_t *)a.sact16, a.sact_scale, (float *)nullptr, a.error_word);
+    if (last < 4) return;
+    // stage 4: down and combine
+    launch_gemm<PF_GEMM_DOWN>(a, tokens, (H + 255) / 256, stream);
+    hipLaunchKernelGGL(pf_k_pf_combine, dim3(tokens), dim3(256), 0, stream, a, tokens);
+}

@@ -73,7 +73,9 @@ __device__ __forceinline__ void pf_route_finish_wave(float my_z, float my_s2, in
     // rounding of z - max and of the exponential.
     const float u = 5.9604645e-8f, hk = (float)hidden / 6.0f;
     const float tol = 8.0f * u * (sqrtf(hk * my_s2) + sqrtf(hk * next_s2)) + 4e-6f * fmaxf(1.0f, top - next_z);
-    close = __any(lane + 1 < rounds && !(my_z - next_z > tol));
+    // Far below the maximum exp() reaches the subnormals and zero, where distinct logits give
+    // equal probabilities and the reference's tie rule (lower id) decides: serial-order path.
+    close = __any((lane + 1 < rounds && !(my_z - next_z > tol)) || (lane < rounds && !(top - my_z < 80.0f)));
     const float e = lane < K ? expf(my_z - top) : 0.0f;
     if (norm) weight = e / pf_wave_sum(e);
     else weight = e * expf(top - top_all) / total;

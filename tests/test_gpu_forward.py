@@ -59,6 +59,76 @@ def test_decode_kernels_match_oracle_and_general_kernels(product, oracle, h, e, 
         assert_parity(y, ids, w, *want, label="general kernels on a decode shape")
 
 
+# shapes the matrix-core prefill kernels cover (Q4_K experts, widths in whole 256-blocks), more than 4 tokens
+PREFILL = [
+    (256, 16, 4, 256, 256, 5), (256, 16, 4, 256, 256, 33), (512, 8, 3, 256, 512, 70),
+    (256, 16, 4, 512, 256, 400),          # about 100 rows per expert: several passes of 64 rows
+    (768, 40, 5, 256, 256, 129),
+]
+
+
+@pytest.mark.parametrize("h,e,k,i,s,tokens", PREFILL)
+def test_prefill_kernels_match_oracle_and_general_kernels(product, oracle, h, e, k, i, s, tokens):
+    print(f"case prefill h={h} e={e} k={k} i={i} s={s} T={tokens}", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s)
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, tokens, seed=h + e + tokens)
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, tokens) as layer:
+        _, y, ids, w = layer.forward(x)
+        worst = assert_parity(y, ids, w, *want, label=f"prefill T={tokens}")
+        print(f"  max abs err {worst:.2e}, serial-order reroutes {layer.serial_order_reroutes()}", flush=True)
+        _, y2, ids2, _ = layer.forward(x)
+        np.testing.assert_array_equal(y, y2, err_msg="prefill path is not deterministic")
+        layer.force_general()
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y, ids, w, *want, label="general kernels on a prefill shape")
+
+
+def test_prefill_rows_of_very_different_magnitude(product, oracle):
+    """Per-row power-of-two scaling: rows spanning 1e-6 .. 1e6 keep the relative accuracy."""
+    cfg = abi.moe_config(256, 16, 4, 256, 256)
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 24, seed=77, normalise=False)
+    scales = np.logspace(-6, 6, 24).astype(np.float32)
+    x = (x / np.abs(x).max(axis=1, keepdims=True)) * scales[:, None]
+    want = forward_with(oracle, cfg, weights, x)
+    got = forward_with(product, cfg, weights, x)
+    np.testing.assert_array_equal(got[1], want[1])
+    rel = np.abs(got[0] - want[0]).max(axis=1) / np.maximum(np.abs(want[0]).max(axis=1), 1e-30)
+    print("relative row errors", rel, flush=True)
+    # fp16 operands: about 2^-11 per rounding, relative to the row's largest output, at every scale
+    assert (rel < 4e-3).all() and rel.max() < 3 * rel.min() + 1e-3
+
+
+def test_saturated_softmax_follows_the_reference_tie_rule(product, oracle):
+    """Logits so far apart that exp() underflows: the reference picks the remaining experts by
+    lowest id (equal zero probabilities), not by logit."""
+    cfg = abi.moe_config(512, 32, 6, 256, 256)
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 4, seed=91)
+    x = x * np.float32(3e4)
+    want = forward_with(oracle, cfg, weights, x)
+    assert (want[2] == 0).any(), "the case must contain underflowed probabilities"
+    for tokens in (1, 4):
+        got = forward_with(product, cfg, weights, x[:tokens])
+        np.testing.assert_array_equal(got[1], want[1][:tokens])
+        np.testing.assert_allclose(got[2], want[2][:tokens], atol=2e-6, rtol=2e-5)
+        rel = np.abs(got[0] - want[0][:tokens]).max() / np.abs(want[0]).max()
+        assert rel < 1e-4, rel
+
+
+def test_full_size_prefill_rows_match_oracle(product, oracle):
+    from picoforge_amd import workloads
+    cfg = workloads.measured_config()
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 48, seed=5)
+    print("full-size prefill, 48 tokens", flush=True)
+    want = forward_with(oracle, cfg, weights, x[:6])      # the CPU path costs 0.14 s per token
+    with pf.MoeLayer(product, cfg, weights, 48) as layer:
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y[:6], ids[:6], w[:6], *want, label="full-size prefill")
+        layer.force_general()
+        _, yg, idsg, wg = layer.forward(x)
+        assert_parity(y, ids, w, yg, idsg, wg, label="prefill against general kernels, all 48 rows")
+
+
 @pytest.mark.parametrize("norm", [True, False])
 def test_decode_unnormalised_weights_and_repeat_calls(product, oracle, norm):
     cfg = abi.moe_config(512, 64, 4, 256, 256, norm=norm)
