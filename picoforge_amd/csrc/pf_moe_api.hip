@@ -148,6 +148,19 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         }
         m->total_bytes += m->bytes[a];
     }
+    {   // transposed router copy for the serial-order re-routing
+        hipError_t e = hipMalloc((void **)&m->router_t, E * h * sizeof(float));
+        if (e == hipSuccess) {
+            pf_launch_transpose(reinterpret_cast<const float *>(m->w[0]), (int)E, (int)h, m->router_t, nullptr);
+            e = hipDeviceSynchronize();
+        }
+        if (e != hipSuccess) {
+            pf_set_error("router copy", e);
+            pf_hip_moe_destroy(m);
+            return e == hipErrorOutOfMemory ? PF_HIP_E_MEMORY : PF_HIP_E_RUNTIME;
+        }
+        m->total_bytes += E * h * sizeof(float);
+    }
     m->decode_ready = pf_decode_supported(*desc);
     // prefill path: squared norms of the router rows (the routing tolerance's bound)
     m->prefill_ready = pf_prefill_supported(*desc);
@@ -171,6 +184,7 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
     if (!m) return;
     for (int a = 0; a < 8; a++) if (m->w[a]) (void)hipFree(m->w[a]);
     if (m->w_norm2) (void)hipFree(m->w_norm2);
+    if (m->router_t) (void)hipFree(m->router_t);
     free(m);
 }
 
@@ -206,9 +220,10 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     // prefill path: fp16 copies, per-row scales, down products in expert order, grouping tables
     const bool prefill = T > PF_DECODE_MAX_TOKENS && pf_prefill_supported(*d);
     const size_t Tp = prefill ? T : 0, Is = d->shared_inter;
-    want[W_X16] = Tp * pf_prefill_half_row((int)H) * 2;
-    want[W_ACT16] = Tp * K * pf_prefill_half_row((int)I) * 2;
-    want[W_SACT16] = Tp * pf_prefill_half_row((int)Is) * 2;
+    // one more row each, never written after the workspace's initial memset: the all-zero row
+    want[W_X16] = prefill ? (Tp + 1) * pf_prefill_half_row((int)H) * 2 : 0;
+    want[W_ACT16] = prefill ? (Tp * K + 1) * pf_prefill_half_row((int)I) * 2 : 0;
+    want[W_SACT16] = prefill ? (Tp + 1) * pf_prefill_half_row((int)Is) * 2 : 0;
     want[W_XSCALE] = Tp * 4;
     want[W_ACTSCALE] = Tp * K * 4;
     want[W_SACTSCALE] = Tp * 4;
@@ -345,6 +360,8 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.w_norm2 = m->w_norm2; a.down = w->down;
     a.counts = w->counts; a.offsets = w->offsets; a.pair_to_row = w->pair_to_row; a.row_to_pair = w->row_to_pair;
     a.group_bad = w->group_bad; a.tiles = w->tiles;
+    a.token_cap = (uint32_t)w->cap;
+    a.router_t = m->router_t;
     return a;
 }
 

@@ -14,6 +14,7 @@ struct PfKernelArgs {
     size_t row_bytes[8], expert_bytes[8];   // of the payload (IQ2_XXS: 64 bytes per block)
     size_t scale_offset[8];                 // IQ2_XXS: byte offset of the half scales in the tensor buffer
     int k_logical[8], blocks_per_row[8], n_out[8];
+    const float *router_t;           // router transposed to [hidden][experts] (serial-order re-routing)
     const uint64_t *iq2_grid;        // 256 x 8 magnitudes, device memory
     const uint32_t *iq2_signed;      // 2 x 4096 words: four signed magnitudes per (grid entry, sign nibble)
     const float *x;                  // [tokens, hidden], pitch in floats
@@ -33,6 +34,7 @@ struct PfKernelArgs {
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
     uint32_t *route_flags;           // [tokens] 1 = route again in serial order
     // prefill path
+    uint32_t token_cap;              // rows the workspace holds; row token_cap (token_cap * top_k for act16) of an fp16 form is all zero
     uint16_t *x16, *act16, *sact16;  // fp16 forms of x, act (pairs in expert order), shared act: per row the high
                                      // parts, the low parts, then 8 + 8 group-sum parts per 256 columns
     float *x_scale, *act_scale, *sact_scale;   // per row: the power of two the fp16 form was divided by
@@ -53,6 +55,7 @@ struct PfHipMoe {
     bool decode_ready;               // shapes and formats the specialised decode kernels cover
     bool prefill_ready;              // shapes and formats the matrix-core prefill kernels cover
     float *w_norm2;                  // [experts] squared norm of each router row
+    float *router_t;                 // [hidden][experts] transposed copy of the router
 };
 
 struct PfHipWork {
@@ -73,6 +76,7 @@ void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, in
 size_t pf_general_lds_bytes(const PfKernelArgs &a);
 // pf_moe_route.hip
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream);
+void pf_launch_transpose(const float *d_src, int rows, int cols, float *d_dst, hipStream_t stream);
 int pf_route_exact_device(const float *d_logits, int tokens, int experts, int top_k, int norm,
                           float *d_probs, uint32_t *d_ids, float *d_weights, uint32_t *d_error,
                           unsigned long long *d_bad_row, hipStream_t stream);

@@ -103,27 +103,38 @@ void pf_launch_row_norm2(const float *d_w, int rows, int cols, float *d_out, hip
 }
 
 // ---- router logits by FP32 MFMA ----------------------------------------------------------------
-// Workgroup = 2 x 2 waves, each a 32-token x 32-expert tile; operands straight from global memory
-// (the lines a lane touches are consumed over the following iterations from the vector cache).
+// Workgroup = one 32-token x 32-expert tile, its four waves a quarter of the columns each (the
+// partial tiles are added in wave order); operands straight from global memory (the lines a
+// lane touches are consumed over the following iterations from the vector cache).
 // Column E is the shared router.  Also writes the routing tolerance's bound on the sum of
 // squared products, max(x)^2 * |w_e|^2.
 __global__ void __launch_bounds__(256) pf_k_pf_router(PfKernelArgs a, int tokens) {
+    __shared__ float partial[3][16][64];
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
-    const int t0 = blockIdx.x * 64 + 32 * (wave & 1), e0 = blockIdx.y * 64 + 32 * (wave >> 1);
-    if (t0 >= tokens || e0 > E) return;
+    const int t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
     const int i = lane & 31, kk = lane >> 5;
     const int t = min(t0 + i, tokens - 1), e = min(e0 + i, E);
+    // the four waves share the tile and split the columns into quarters (hidden is a multiple of 32)
+    const int q0 = wave * (H / 32), q1 = q0 + H / 32;
     const float4 *xp = reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch) + kk;
     const float4 *wp = reinterpret_cast<const float4 *>(e < E ? a.w[0] + (size_t)e * H * 4 : a.w[7]) + kk;
     float16v acc = {0};
 #pragma unroll 4
-    for (int q = 0; q < H / 8; q++) {
+    for (int q = q0; q < q1; q++) {
         const float4 xv = xp[2 * q], wv = wp[2 * q];
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.x, wv.x, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.y, wv.y, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.z, wv.z, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.w, wv.w, acc, 0, 0, 0);
     }
+    if (wave > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) partial[wave - 1][r][lane] = acc[r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = ((acc[r] + partial[0][r][lane]) + partial[1][r][lane]) + partial[2][r][lane];
     const int col = e0 + i;   // this lane's expert
     const float wn = col < E ? a.w_norm2[col] : 0.0f;
 #pragma unroll
@@ -168,8 +179,11 @@ __device__ __forceinline__ void q4_scale_min(const Q4Raw &r, int g, uint32_t &sc
 
 // eight codes (two dwords of nibbles, nibble position nib) times the group's scale, exact in fp16:
 // a nibble under the exponent byte 0x64 reads as 1024 + q, and (1024 + q) * s - 1024 * s = q * s
+// (the high nibbles stay in place: 1024 + 16 q against s / 16 and 64 s, both exact for a 6-bit s;
+// the caller passes the pair of constants that belongs to the nibble position)
 __device__ __forceinline__ half8v q4_scaled_codes(uint32_t w0, uint32_t w1, int nib, half2v s2, half2v c1024) {
-    const uint32_t q0 = (w0 >> (4 * nib)) & 0x0F0F0F0Fu, q1 = (w1 >> (4 * nib)) & 0x0F0F0F0Fu;
+    const uint32_t mask = nib ? 0xF0F0F0F0u : 0x0F0F0F0Fu;
+    const uint32_t q0 = w0 & mask, q1 = w1 & mask;
     const uint32_t bias = 0x64646464u;
     const half2v p0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q0, 0x04010400u));
     const half2v p1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q0, 0x04030402u));
@@ -183,121 +197,151 @@ __device__ __forceinline__ half8v q4_scaled_codes(uint32_t w0, uint32_t w1, int 
 // Lane (n = lane % 32, h = lane / 32) owns weight row n of its tiles and, per 64 weights, the
 // 16 bytes [16h, 16h + 16) of the 32-byte nibble run: chunk c = 2h + c2 (c2 = 0, 1) of nibble
 // position nib is k = 64j + 32 nib + 8c + 0..7, one MFMA per (c2, nib) and activation part.
+//
+// The activation tile of a 256-block travels from global memory straight into LDS (16 bytes per
+// lane, 64 consecutive chunks per wave instruction), one block ahead of the products, into the
+// other of two buffers.  Chunk p of a buffer: [0, 1056) high parts, row p / 33, column chunk
+// p % 33 (the 33rd is padding); [1056, 2112) low parts likewise; [2112, 2208) group sums, row
+// q / 3, chunk q % 3 (the third is padding); the rest, the padding and the rows beyond the
+// tile's last read the matrix's all-zero row (index zero_row).
+#define TILE_LOADS 35                      // wave instructions per tile
+#define TILE_HALFS (TILE_LOADS * 64 * 8)   // 35 840 bytes
+#define TILE_LOW (1056 * 8)                // half offsets of the low parts and of the sums in a buffer
+#define TILE_SUMS (2112 * 8)
+
+__device__ __forceinline__ uint32_t tile_source(int p, const uint32_t *src_row, uint32_t a_pitch, int a_cols,
+                                                uint32_t zero_row) {
+    int m, c, base;
+    if (p < 2112) {
+        const int q = p < 1056 ? p : p - 1056;
+        m = q / 33; c = q % 33;
+        base = p < 1056 ? 0 : a_cols;
+        if (c == 32) m = 32;
+    } else {
+        const int q = p - 2112;
+        m = q / 3; c = q % 3;
+        base = 2 * a_cols;
+        if (c == 2) m = 32;
+    }
+    const uint32_t row = m < 32 ? src_row[m] : zero_row;   // src_row holds zero_row beyond the tile's rows
+    return row * a_pitch + (uint32_t)base + (row == zero_row ? 0u : 8u * (uint32_t)c);
+}
+
 template <int MT>
-__device__ __forceinline__ void gemm_pass(half_t *tile_h, half_t *tile_l, half_t *tile_s, const uint32_t *src_row,
-                                          const half_t *a16, int a_cols, const uint8_t *wrow0, const uint8_t *wrow1,
-                                          int kblocks, int rows_here, float16v (&acc)[2][MT]) {
-    const int lane = pf_lane(), n = lane & 31, h = lane >> 5;
-    const size_t a_pitch = pf_half_row(a_cols);
-    Q4Raw raw0, raw1;
-    q4_load(raw0, wrow0, h);
-    q4_load(raw1, wrow1, h);
-    for (int kb = 0; kb < kblocks; kb++) {
-        __syncthreads();   // the previous tile has been consumed
-        // activation tile: per row 32 + 32 sixteen-byte chunks of the two parts and 2 of the group sums
-        for (int i = threadIdx.x; i < 32 * MT * 66; i += 256) {
-            const int m = i / 66, c = i % 66;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            const half_t *row = a16 + (size_t)src_row[m] * a_pitch;
-            if (c < 32) {
-                if (m < rows_here) v = *reinterpret_cast<const uint4 *>(row + 256 * kb + 8 * c);
-                *reinterpret_cast<uint4 *>(tile_h + m * A_PITCH + 8 * c) = v;
-            } else if (c < 64) {
-                if (m < rows_here) v = *reinterpret_cast<const uint4 *>(row + a_cols + 256 * kb + 8 * (c - 32));
-                *reinterpret_cast<uint4 *>(tile_l + m * A_PITCH + 8 * (c - 32)) = v;
-            } else {
-                if (m < rows_here) v = *reinterpret_cast<const uint4 *>(row + 2 * a_cols + 16 * kb + 8 * (c - 64));
-                *reinterpret_cast<uint4 *>(tile_s + m * S_PITCH + 8 * (c - 64)) = v;
-            }
+__device__ __forceinline__ void gemm_pass(half_t *tiles, const uint32_t *src_row, const half_t *a16, int a_cols,
+                                          uint32_t zero_row, const uint8_t *wrow0, const uint8_t *wrow1, int kblocks,
+                                          float16v (&acc)[2][MT]) {
+    static_assert(MT == 1, "one 32-row tile per pass");
+    const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
+    const uint32_t a_pitch = (uint32_t)pf_half_row(a_cols);
+    // this wave's loads of a tile: instruction i = wave + 4 ii covers chunks [64 i, 64 i + 64)
+    uint32_t source[9];
+#pragma unroll
+    for (int ii = 0; ii < 9; ii++) source[ii] = tile_source(64 * (wave + 4 * ii) + lane, src_row, a_pitch, a_cols, zero_row);
+    auto issue_tile = [&](int kb, half_t *buffer) {
+#pragma unroll
+        for (int ii = 0; ii < 9; ii++) {
+            const int i = wave + 4 * ii;
+            if (i >= TILE_LOADS) break;
+            const uint32_t step = 64 * i < 2112 ? 256u : 16u;   // halfs per 256-block in this region (uniform per load)
+            __builtin_amdgcn_global_load_lds(a16 + source[ii] + step * (uint32_t)kb, buffer + 512 * i, 16, 0, 0);
         }
-        const Q4Raw cur0 = raw0, cur1 = raw1;
+    };
+    // One 256-block: wait for its bytes, start the next block's, multiply.  The weight bytes
+    // alternate between two register sets (cur / next) from block to block.
+    auto block_step = [&](int kb, const Q4Raw &cur0, const Q4Raw &cur1, Q4Raw &next0, Q4Raw &next1) {
+        half_t *tile_h = tiles + (kb & 1) * TILE_HALFS, *tile_l = tile_h + TILE_LOW, *tile_s = tile_h + TILE_SUMS;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's part of the tile and its weight bytes have arrived
+        __syncthreads();                                    // every wave's part; and the other buffer has been consumed
         if (kb + 1 < kblocks) {   // next block's bytes travel while this one is multiplied
-            q4_load(raw0, wrow0 + 144 * (kb + 1), h);
-            q4_load(raw1, wrow1 + 144 * (kb + 1), h);
+            issue_tile(kb + 1, tiles + ((kb + 1) & 1) * TILE_HALFS);
+            q4_load(next0, wrow0 + 144 * (kb + 1), h);
+            q4_load(next1, wrow1 + 144 * (kb + 1), h);
         }
-        __syncthreads();
-        const float d0 = pf_half_bits_to_float(cur0.hdr.x & 0xffffu), m0 = pf_half_bits_to_float(cur0.hdr.x >> 16);
-        const float d1 = pf_half_bits_to_float(cur1.hdr.x & 0xffffu), m1 = pf_half_bits_to_float(cur1.hdr.x >> 16);
-        // Q: the eight minima against the eight group sums (high parts in k 0..7, low parts in k 8..15)
+        const half_t *row_h = tile_h + n * A_PITCH + 16 * h, *row_l = tile_l + n * A_PITCH + 16 * h;
+        // first activation fragments, requested before the scale arithmetic
+        half8v ah = *reinterpret_cast<const half8v *>(row_h), al = *reinterpret_cast<const half8v *>(row_l);
+        const half8v as = *reinterpret_cast<const half8v *>(tile_s + n * S_PITCH + 8 * h);
+        // the hardware conversion is exact for every binary16 value, subnormals included
+        const half2v dm0 = __builtin_bit_cast(half2v, cur0.hdr.x), dm1 = __builtin_bit_cast(half2v, cur1.hdr.x);
+        const float d0 = (float)dm0.x, m0 = (float)dm0.y, d1 = (float)dm1.x, m1 = (float)dm1.y;
         half8v min0, min1;
         half2v s2[2][8], c2k[2][8];
 #pragma unroll
         for (int g = 0; g < 8; g++) {
+            // even groups sit in the low nibbles (1024 + q, times s, minus 1024 s), odd groups in
+            // the high ones (1024 + 16 q, times s / 16, minus 64 s)
+            const half_t unit = (g & 1) ? (half_t)0.0625f : (half_t)1.0f;
+            const int bias_shift = (g & 1) ? 6 : 10;
             uint32_t sc, mn;
             q4_scale_min(cur0, g, sc, mn);
             min0[g] = (half_t)(int)mn;
-            s2[0][g] = half2v{(half_t)(int)sc, (half_t)(int)sc};
-            c2k[0][g] = half2v{(half_t)(int)(sc << 10), (half_t)(int)(sc << 10)};
+            const half_t s0 = (half_t)(int)sc * unit;
+            s2[0][g] = half2v{s0, s0};
+            c2k[0][g] = half2v{(half_t)(int)(sc << bias_shift), (half_t)(int)(sc << bias_shift)};
             q4_scale_min(cur1, g, sc, mn);
             min1[g] = (half_t)(int)mn;
-            s2[1][g] = half2v{(half_t)(int)sc, (half_t)(int)sc};
-            c2k[1][g] = half2v{(half_t)(int)(sc << 10), (half_t)(int)(sc << 10)};
+            const half_t s1 = (half_t)(int)sc * unit;
+            s2[1][g] = half2v{s1, s1};
+            c2k[1][g] = half2v{(half_t)(int)(sc << bias_shift), (half_t)(int)(sc << bias_shift)};
         }
-        float16v part[2][MT];
+        // Q: the eight minima against the eight group sums (high parts in k 0..7, low parts in k 8..15)
+        const float16v zero = {0};
+        const float16v q0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min0, zero, 0, 0, 0);
+        const float16v q1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min1, zero, 0, 0, 0);
+        // P: scale * code against both activation parts; step s = (j, nib, c2) covers
+        // k = 64 j + 32 nib + 16 h + 8 c2 + 0..7, and its fragments are requested one step ahead
+        float16v part0 = zero, part1 = zero;
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            const half8v as = *reinterpret_cast<const half8v *>(tile_s + (32 * mt + n) * S_PITCH + 8 * h);
-            const float16v zero = {0};
-            const float16v q0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min0, zero, 0, 0, 0);
-            const float16v q1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min1, zero, 0, 0, 0);
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                acc[0][mt][r] = fmaf(-m0, q0[r], acc[0][mt][r]);
-                acc[1][mt][r] = fmaf(-m1, q1[r], acc[1][mt][r]);
+        for (int s = 0; s < 16; s++) {
+            const int j = s >> 2, nib = (s >> 1) & 1, c2 = s & 1, g = 2 * j + nib;
+            half8v nh = ah, nl = al;
+            if (s < 15) {
+                const int sn = s + 1, kn = 64 * (sn >> 2) + 32 * ((sn >> 1) & 1) + 8 * (sn & 1);
+                nh = *reinterpret_cast<const half8v *>(row_h + kn);
+                nl = *reinterpret_cast<const half8v *>(row_l + kn);
             }
-            part[0][mt] = zero;
-            part[1][mt] = zero;
-        }
-        // P: scale * code against both activation parts
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-#pragma unroll
-            for (int nib = 0; nib < 2; nib++) {
-                const int g = 2 * j + nib;
-#pragma unroll
-                for (int c2 = 0; c2 < 2; c2++) {
-                    const uint4 w0 = cur0.q[j], w1 = cur1.q[j];
-                    const half8v b0 = q4_scaled_codes(c2 ? w0.z : w0.x, c2 ? w0.w : w0.y, nib, s2[0][g], c2k[0][g]);
-                    const half8v b1 = q4_scaled_codes(c2 ? w1.z : w1.x, c2 ? w1.w : w1.y, nib, s2[1][g], c2k[1][g]);
-                    const int k = 64 * j + 32 * nib + 16 * h + 8 * c2;
-#pragma unroll
-                    for (int mt = 0; mt < MT; mt++) {
-                        const half8v ah = *reinterpret_cast<const half8v *>(tile_h + (32 * mt + n) * A_PITCH + k);
-                        const half8v al = *reinterpret_cast<const half8v *>(tile_l + (32 * mt + n) * A_PITCH + k);
-                        part[0][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, part[0][mt], 0, 0, 0);
-                        part[1][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, part[1][mt], 0, 0, 0);
-                        part[0][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b0, part[0][mt], 0, 0, 0);
-                        part[1][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b1, part[1][mt], 0, 0, 0);
-                    }
-                }
-            }
+            const uint4 w0 = cur0.q[j], w1 = cur1.q[j];
+            const half8v b0 = q4_scaled_codes(c2 ? w0.z : w0.x, c2 ? w0.w : w0.y, nib, s2[0][g], c2k[0][g]);
+            const half8v b1 = q4_scaled_codes(c2 ? w1.z : w1.x, c2 ? w1.w : w1.y, nib, s2[1][g], c2k[1][g]);
+            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, part0, 0, 0, 0);
+            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, part1, 0, 0, 0);
+            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b0, part0, 0, 0, 0);
+            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b1, part1, 0, 0, 0);
+            ah = nh;
+            al = nl;
         }
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                acc[0][mt][r] = fmaf(d0, part[0][mt][r], acc[0][mt][r]);
-                acc[1][mt][r] = fmaf(d1, part[1][mt][r], acc[1][mt][r]);
-            }
+        for (int r = 0; r < 16; r++) {
+            acc[0][0][r] = fmaf(d0, part0[r], fmaf(-m0, q0[r], acc[0][0][r]));
+            acc[1][0][r] = fmaf(d1, part1[r], fmaf(-m1, q1[r], acc[1][0][r]));
         }
+    };
+    Q4Raw a0, a1, b0, b1;
+    q4_load(a0, wrow0, h);
+    q4_load(a1, wrow1, h);
+    issue_tile(0, tiles);
+    for (int kb = 0; kb < kblocks; kb += 2) {
+        block_step(kb, a0, a1, b0, b1);
+        if (kb + 1 < kblocks) block_step(kb + 1, b0, b1, a0, a1);
     }
 }
 
 struct GemmTarget {   // what one workgroup of the grouped product works on
     bool shared;
     int first, count, inter, kblocks, a_cols, slab;
+    uint32_t zero_row;   // index of the all-zero row that ends the fp16 form of the activation matrix
     const uint8_t *w0, *w1;
     const half_t *a16;
     const float *a_scale;
 };
 
 template <int MODE, int MT>
-__device__ __forceinline__ void gemm_rows(const PfKernelArgs &a, const GemmTarget &g, int m0, int rows_here, half_t *tile_h,
-                                          half_t *tile_l, half_t *tile_s, uint32_t *src_row, float *row_scale) {
+__device__ __forceinline__ void gemm_rows(const PfKernelArgs &a, const GemmTarget &g, int m0, int rows_here, half_t *tiles,
+                                          uint32_t *src_row, float *row_scale) {
     const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5, K = a.top_k;
-    __syncthreads();
     for (int m = threadIdx.x; m < 32 * MT; m += 256) {
-        uint32_t src = 0;
+        uint32_t src = g.zero_row;
         float sc = 0.0f;
         if (m < rows_here) {
             if (MODE == PF_GEMM_GATE_UP) src = g.shared ? (uint32_t)(m0 + m) : a.row_to_pair[g.first + m0 + m] / (uint32_t)K;
@@ -310,7 +354,8 @@ __device__ __forceinline__ void gemm_rows(const PfKernelArgs &a, const GemmTarge
     float16v acc[2][MT];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++) { acc[0][mt] = float16v{0}; acc[1][mt] = float16v{0}; }
-    gemm_pass<MT>(tile_h, tile_l, tile_s, src_row, g.a16, g.a_cols, g.w0, g.w1, g.kblocks, rows_here, acc);
+    __syncthreads();   // src_row is read by every wave's tile loads
+    gemm_pass<MT>(tiles, src_row, g.a16, g.a_cols, g.zero_row, g.w0, g.w1, g.kblocks, acc);
     // epilogue: the lane holds column n of its two tiles; register r of tile mt is row
     // 32 mt + 8 (r / 4) + 4 h + r % 4
 #pragma unroll
@@ -365,7 +410,7 @@ __global__ void __launch_bounds__(256) pf_k_pf_tiles(const uint32_t *offsets, in
 template <int MODE>
 __global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, int slabs) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    half_t *tile_h = reinterpret_cast<half_t *>(lds_raw), *tile_l = tile_h + 32 * A_PITCH, *tile_s = tile_l + 32 * A_PITCH;
+    half_t *tiles = reinterpret_cast<half_t *>(lds_raw);   // two buffers of TILE_HALFS
     __shared__ uint32_t src_row[32];
     __shared__ float row_scale[32];
     const int E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31;
@@ -390,6 +435,7 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, 
         g.w1 = a.w[tg + 1] + ex * a.expert_bytes[tg + 1] + (size_t)u * a.row_bytes[tg + 1];
         g.kblocks = a.hidden / 256; g.a_cols = a.hidden;
         g.a16 = reinterpret_cast<const half_t *>(a.x16); g.a_scale = a.x_scale;
+        g.zero_row = a.token_cap;
     } else {
         const int td = g.shared ? 6 : 3, r0 = 256 * g.slab + 64 * wave + n;
         g.w0 = a.w[td] + ex * a.expert_bytes[td] + (size_t)min(r0, a.hidden - 1) * a.row_bytes[td];
@@ -397,8 +443,9 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, 
         g.kblocks = g.inter / 256; g.a_cols = g.inter;
         g.a16 = reinterpret_cast<const half_t *>(g.shared ? a.sact16 : a.act16);
         g.a_scale = g.shared ? a.sact_scale : a.act_scale;
+        g.zero_row = g.shared ? a.token_cap : a.token_cap * (uint32_t)a.top_k;
     }
-    gemm_rows<MODE, 1>(a, g, m0, min(32, g.count - m0), tile_h, tile_l, tile_s, src_row, row_scale);
+    gemm_rows<MODE, 1>(a, g, m0, min(32, g.count - m0), tiles, src_row, row_scale);
 }
 
 // ---- combine ---------------------------------------------------------------------------------------
@@ -445,7 +492,13 @@ int pf_prefill_max_tiles(int tokens, int experts, int top_k) {
 
 template <int MODE>
 static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_t stream) {
-    const size_t lds = (size_t)(2 * 32 * A_PITCH + 32 * S_PITCH) * sizeof(half_t);
+    const size_t lds = 2 * (size_t)TILE_HALFS * sizeof(half_t);
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_pf_gemm<MODE>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        configured = true;
+    }
     // the tile count is only known on the device: launch its upper bound, surplus workgroups exit at once
     const int max_tiles = pf_prefill_max_tiles(tokens, a.experts, a.top_k);
     hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3(max_tiles * slabs), dim3(256), lds, stream, a, tokens, slabs);
@@ -457,7 +510,7 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     // stage 1: fp16 parts of x, router logits
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.x, a.x_pitch, H, (half_t *)a.x16, a.x_scale,
                        a.x_max2, a.error_word);
-    hipLaunchKernelGGL(pf_k_pf_router, dim3((tokens + 63) / 64, (E + 1 + 63) / 64), dim3(256), 0, stream, a, tokens);
+    hipLaunchKernelGGL(pf_k_pf_router, dim3((tokens + 31) / 32, (E + 1 + 31) / 32), dim3(256), 0, stream, a, tokens);
     if (last < 2) return;
     // stage 2: routes and grouping
     pf_launch_route(a, tokens, stream);

@@ -26,26 +26,74 @@ __global__ void __launch_bounds__(64) pf_k_route_fast(PfKernelArgs a) {
     if (lane == 0) a.route_flags[t] = r.close ? 1u : 0u;
 }
 
-// Serial-order recomputation for flagged tokens: thread e owns expert e.
-__global__ void __launch_bounds__(256) pf_k_route_fix(PfKernelArgs a) {
-    extern __shared__ float lds[];
-    const int t = blockIdx.x, E = a.experts, H = a.hidden;
+// Serial-order recomputation for flagged tokens, in two kernels so that a token's logits
+// spread over many compute units: one wave per (token, 64 experts), lane e owns expert e and
+// walks k in order over the transposed router copy [hidden][experts], so that every step is
+// one coalesced 256-byte load; then one wave per token selects.
+__global__ void __launch_bounds__(64) pf_k_route_fix_logits(PfKernelArgs a) {
+#pragma clang fp contract(off)
+    const int t = blockIdx.x, E = a.experts, H = a.hidden, e = blockIdx.y * PF_WAVE + threadIdx.x;
     if (!a.route_flags[t]) return;
-    float *xs = lds, *z = lds + H, *p = z + E, *q = p + E;
-    const float *x = a.x + (size_t)t * a.x_pitch;
-    for (int k = threadIdx.x; k < H; k += blockDim.x) xs[k] = x[k];
-    __syncthreads();
-    for (int e = threadIdx.x; e < E; e += blockDim.x) {
-        const float sum = pf_serial_logit(reinterpret_cast<const float *>(a.w[0]) + (size_t)e * H, xs, H);
-        z[e] = sum;
-        a.logits[(size_t)t * E + e] = sum;
+    extern __shared__ float xs[];
+    const float *w = a.router_t + min(e, E - 1), *x = a.x + (size_t)t * a.x_pitch;
+    for (int k = threadIdx.x; k < H; k += PF_WAVE) xs[k] = x[k];
+    pf_wave_lds_fence();
+    if (e >= E) return;
+    // The sum is one dependent chain; the loads are not.  They are requested 128 at a time, one
+    // batch ahead of the chain, so that the chain rarely waits for memory.
+    float sum = 0.0f, wa[128], wb[128];
+    const int batches = H / 128;
+    auto load = [&](float (&dst)[128], int b) {
+#pragma unroll
+        for (int j = 0; j < 128; j++) dst[j] = w[(size_t)(128 * b + j) * E];
+    };
+    auto chain = [&](const float (&src)[128], int b) {
+#pragma unroll
+        for (int j = 0; j < 128; j++) {
+            const float p = src[j] * xs[128 * b + j];
+            sum = sum + p;
+        }
+    };
+    if (batches > 0) load(wa, 0);
+    for (int b = 0; b < batches; b += 2) {
+        if (b + 1 < batches) load(wb, b + 1);
+        chain(wa, b);
+        if (b + 2 < batches) load(wa, b + 2);
+        if (b + 1 < batches) chain(wb, b + 1);
     }
-    __syncthreads();
-    if (threadIdx.x < PF_WAVE) {
-        pf_route_exact_wave(z, p, q, E, a.top_k, a.norm_topk != 0, a.ids + (size_t)t * a.top_k,
-                            a.route_weights + (size_t)t * a.top_k, threadIdx.x);
-        if (threadIdx.x == 0) atomicAdd(a.exact_rows, 1u);
+    for (int k = 128 * batches; k < H; k++) {
+        const float p = w[(size_t)k * E] * xs[k];
+        sum = sum + p;
     }
+    a.logits[(size_t)t * E + e] = sum;
+}
+
+// router [experts][hidden] -> [hidden][experts], once at upload
+__global__ void pf_k_transpose(const float *src, int rows, int cols, float *dst) {
+    __shared__ float tile[32][33];
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32, tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    for (int j = ty; j < 32; j += 8)
+        if (r0 + j < rows && c0 + tx < cols) tile[j][tx] = src[(size_t)(r0 + j) * cols + c0 + tx];
+    __syncthreads();
+    for (int j = ty; j < 32; j += 8)
+        if (c0 + j < cols && r0 + tx < rows) dst[(size_t)(c0 + j) * rows + r0 + tx] = tile[tx][j];
+}
+
+void pf_launch_transpose(const float *d_src, int rows, int cols, float *d_dst, hipStream_t stream) {
+    hipLaunchKernelGGL(pf_k_transpose, dim3((cols + 31) / 32, (rows + 31) / 32), dim3(256), 0, stream, d_src, rows, cols,
+                       d_dst);
+}
+
+__global__ void __launch_bounds__(64) pf_k_route_fix_select(PfKernelArgs a) {
+    extern __shared__ float lds[];
+    const int t = blockIdx.x, E = a.experts;
+    if (!a.route_flags[t]) return;
+    float *z = lds, *p = z + E, *q = p + E;
+    for (int e = threadIdx.x; e < E; e += PF_WAVE) z[e] = a.logits[(size_t)t * E + e];
+    pf_wave_lds_fence();
+    pf_route_exact_wave(z, p, q, E, a.top_k, a.norm_topk != 0, a.ids + (size_t)t * a.top_k,
+                        a.route_weights + (size_t)t * a.top_k, threadIdx.x);
+    if (threadIdx.x == 0) atomicAdd(a.exact_rows, 1u);
 }
 
 // Every token through the exact path (expert counts the fast kernel cannot hold).
@@ -63,8 +111,10 @@ void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     else if (npl <= 4) hipLaunchKernelGGL(pf_k_route_fast<4>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 8) hipLaunchKernelGGL(pf_k_route_fast<8>, dim3(tokens), dim3(64), 0, stream, a);
     else hipLaunchKernelGGL(pf_k_route_fast<16>, dim3(tokens), dim3(64), 0, stream, a);
-    const size_t lds = ((size_t)a.hidden + 3 * (size_t)a.experts) * sizeof(float);
-    hipLaunchKernelGGL(pf_k_route_fix, dim3(tokens), dim3(256), lds, stream, a);
+    hipLaunchKernelGGL(pf_k_route_fix_logits, dim3(tokens, (a.experts + PF_WAVE - 1) / PF_WAVE), dim3(PF_WAVE),
+                       (size_t)a.hidden * sizeof(float), stream, a);
+    hipLaunchKernelGGL(pf_k_route_fix_select, dim3(tokens), dim3(PF_WAVE), 3 * (size_t)a.experts * sizeof(float), stream,
+                       a);
 }
 
 // ---- qwen4_moe_route on caller-provided logits ----------------------------------
@@ -154,20 +204,27 @@ __global__ void __launch_bounds__(256) pf_k_group_scan(const uint32_t *counts, i
 // same expert, so placement is stable without ordered atomics
 __global__ void __launch_bounds__(256) pf_k_group_place(const uint32_t *ids, int pairs, int E, const uint32_t *offsets,
                                                         uint32_t *pair_to_row, uint32_t *row_to_pair) {
+    __shared__ uint32_t staged[8192];   // the ids pass through LDS in pieces: the scan then waits on no global load
     const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = pf_lane();
-    if (e >= E) return;
-    uint32_t base = offsets[e];
-    if (offsets[e + 1] == base) return;
-    for (int p0 = 0; p0 < pairs; p0 += PF_WAVE) {
-        const int p = p0 + lane;
-        const bool hit = p < pairs && ids[p] == (uint32_t)e;
-        const unsigned long long mask = __ballot(hit);
-        if (hit) {
-            const uint32_t row = base + __popcll(mask & ((1ull << lane) - 1ull));
-            pair_to_row[p] = row;
-            row_to_pair[row] = (uint32_t)p;
+    const bool active = e < E && offsets[min(e, E - 1) + 1] != offsets[min(e, E - 1)];
+    uint32_t base = e < E ? offsets[e] : 0u;
+    for (int piece = 0; piece < pairs; piece += 8192) {
+        const int len = min(8192, pairs - piece);
+        __syncthreads();
+        for (int i = threadIdx.x; i < len; i += blockDim.x) staged[i] = ids[piece + i];
+        __syncthreads();
+        if (!active) continue;
+        for (int p0 = 0; p0 < len; p0 += PF_WAVE) {
+            const int p = p0 + lane;
+            const bool hit = p < len && staged[p] == (uint32_t)e;
+            const unsigned long long mask = __ballot(hit);
+            if (hit) {
+                const uint32_t row = base + __popcll(mask & ((1ull << lane) - 1ull));
+                pair_to_row[piece + p] = row;
+                row_to_pair[row] = (uint32_t)(piece + p);
+            }
+            base += __popcll(mask);
         }
-        base += __popcll(mask);
     }
 }
 
