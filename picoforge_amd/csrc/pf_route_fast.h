@@ -12,6 +12,7 @@
 // comparison decides them.
 #pragma once
 #include "pf_device.h"
+#include "pf_route_device.h"
 
 __device__ __forceinline__ float pf_dpp_max_step(float v, const int which) {
     int moved;
@@ -125,16 +126,32 @@ __device__ __forceinline__ PfRouteResult pf_route_fast_wave(const float *z_row, 
 
 // ---- several waves per token -------------------------------------------------------------
 // Candidate lists in LDS: for each of `parts` waves, `rounds` entries sorted by (logit
-// descending, id ascending); entry = logit, id, sum of squared products.  part_max and
-// part_sum carry the pieces of the softmax denominator.
+// descending, id ascending); entry = sort key, logit, id, sum of squared products.  part_max
+// and part_sum carry the pieces of the softmax denominator.  `first` receives the merged
+// k + 1 best.
 struct PfRouteCands {
-    float z[160];
-    uint32_t id[160];
-    float s2[160];
+    unsigned long long key[128];
+    float z[128];
+    uint32_t id[128];
+    float s2[128];
+    float first_z[16], first_s2[16];
+    uint32_t first_id[16];
     float part_max[8], part_sum[8];
     uint32_t bad[8];
 };
 
+// Larger key = earlier in the order: the logit as an order-preserving integer (-0 counted as
+// +0), then the lower id.  Equal logits among the k + 1 best always take the serial-order
+// path, so the id part only makes the order total.
+__device__ __forceinline__ unsigned long long pf_route_key(float z, uint32_t id) {
+    uint32_t u = __float_as_uint(z + 0.0f);
+    u ^= (u >> 31) ? 0xffffffffu : 0x80000000u;
+    return ((unsigned long long)u << 32) | (uint32_t)~id;
+}
+
+// Stage 1 by ranking: every value's rank = how many of the chunk's values have a larger key.
+// The other values come as wave-uniform operands (v_readlane), so one comparison and one
+// carry-add per pair and no dependent chain across lanes.
 template <int NPL>
 __device__ __forceinline__ void pf_route_stage1(const float *z_row, const float *ssq_row, int E, int part, int chunk,
                                                 int rounds, bool norm, PfRouteCands *c, int lane) {
@@ -160,6 +177,39 @@ __device__ __forceinline__ void pf_route_stage1(const float *z_row, const float 
         if (lane == 0) { c->part_max[part] = m; c->part_sum[part] = sum; }
     }
     if (lane == 0) c->bad[part] = bad ? 1u : 0u;
+    if (NPL == 1) {   // wider chunks keep the extraction below (the unrolled ranking would spill)
+        unsigned long long key[NPL];
+        uint32_t hi[NPL];
+        int rank[NPL];
+#pragma unroll
+        for (int j = 0; j < NPL; j++) {
+            key[j] = pf_route_key(v[j], (uint32_t)(base + lane * NPL + j));
+            hi[j] = (uint32_t)(key[j] >> 32);
+            rank[j] = 0;
+        }
+#pragma unroll
+        for (int l = 0; l < PF_WAVE; l++) {
+#pragma unroll
+            for (int jj = 0; jj < NPL; jj++) {
+                const unsigned long long other =
+                    ((unsigned long long)(uint32_t)__builtin_amdgcn_readlane((int)hi[jj], l) << 32) |
+                    (uint32_t)~(uint32_t)(base + l * NPL + jj);
+#pragma unroll
+                for (int j = 0; j < NPL; j++) rank[j] += other > key[j] ? 1 : 0;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NPL; j++) {
+            if (rank[j] < rounds) {
+                const int at = part * rounds + rank[j];
+                c->key[at] = key[j];
+                c->z[at] = v[j];
+                c->id[at] = v[j] == -INFINITY ? 0xffffffffu : (uint32_t)(base + lane * NPL + j);
+                c->s2[at] = s2[j];
+            }
+        }
+        return;
+    }
     for (int r = 0; r < rounds; r++) {
         float wm;
         int owner, jsel;
@@ -170,6 +220,7 @@ __device__ __forceinline__ void pf_route_stage1(const float *z_row, const float 
 #pragma unroll
         for (int j = 0; j < NPL; j++) {
             if (lane == owner && j == jsel) {
+                c->key[at] = pf_route_key(wm, (uint32_t)(base + lane * NPL + j));
                 c->z[at] = wm;
                 c->id[at] = wm == -INFINITY ? 0xffffffffu : (uint32_t)(base + lane * NPL + j);
                 c->s2[at] = s2[j];
@@ -178,16 +229,13 @@ __device__ __forceinline__ void pf_route_stage1(const float *z_row, const float 
     }
 }
 
-// Merge by one wave: candidate p sits in lane p / 3, register p % 3 (at most 160 candidates).
-__device__ __forceinline__ PfRouteResult pf_route_stage2(const PfRouteCands *c, int parts, int K, int rounds, bool norm,
+// Merge by one wave, again by ranking: candidate p and p + 64 sit in lane p (at most 128
+// candidates); the other candidates' keys are read from LDS at wave-uniform addresses.
+__device__ __forceinline__ PfRouteResult pf_route_stage2(PfRouteCands *c, int parts, int K, int rounds, bool norm,
                                                          int hidden, int lane) {
     const int count = parts * rounds;
-    float v[3];
-#pragma unroll
-    for (int j = 0; j < 3; j++) {
-        const int p = lane * 3 + j;
-        v[j] = p < count ? c->z[p] : -INFINITY;
-    }
+    const unsigned long long k0 = lane < count ? c->key[lane] : 0ull;
+    const unsigned long long k1 = lane + 64 < count ? c->key[lane + 64] : 0ull;
     float total = 0.0f, top_all = 0.0f;
     bool bad = false;
     for (int w = 0; w < parts; w++) bad |= c->bad[w] != 0;
@@ -196,20 +244,21 @@ __device__ __forceinline__ PfRouteResult pf_route_stage2(const PfRouteCands *c, 
         for (int w = 1; w < parts; w++) top_all = fmaxf(top_all, c->part_max[w]);
         for (int w = 0; w < parts; w++) total += c->part_sum[w] * expf(c->part_max[w] - top_all);
     }
-    int my_at = 0;
-    float my_z = 0.0f;
-    for (int r = 0; r < rounds; r++) {
-        float wm;
-        int owner, jsel;
-        pf_extract_max<3>(v, lane, wm, owner, jsel);
-        if (lane == r) {
-            my_at = owner * 3 + jsel;
-            my_z = wm;
-        }
+    int r0 = 0, r1 = 0;
+#pragma unroll 8
+    for (int l = 0; l < count; l++) {
+        const unsigned long long other = c->key[l];
+        r0 += other > k0 ? 1 : 0;
+        r1 += other > k1 ? 1 : 0;
     }
-    my_at = my_at < count ? my_at : 0;
-    const uint32_t my_id = c->id[my_at];
-    const float my_s2 = c->s2[my_at];
+    if (lane < count && r0 < rounds) { c->first_z[r0] = c->z[lane]; c->first_id[r0] = c->id[lane]; c->first_s2[r0] = c->s2[lane]; }
+    if (lane + 64 < count && r1 < rounds) {
+        c->first_z[r1] = c->z[lane + 64]; c->first_id[r1] = c->id[lane + 64]; c->first_s2[r1] = c->s2[lane + 64];
+    }
+    pf_wave_lds_fence();
+    const int at = lane < rounds ? lane : 0;
+    const float my_z = c->first_z[at], my_s2 = c->first_s2[at];
+    const uint32_t my_id = c->first_id[at];
     PfRouteResult out;
     pf_route_finish_wave(my_z, my_s2, K, rounds, norm, hidden, total, top_all, lane, out.weight, out.close);
     out.id = my_id;
