@@ -291,6 +291,38 @@ __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int route
     if (__any(bad) && lane == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
 }
 
+// Warms the L2 of this workgroup's XCD with the down-projection rows the next kernel will read
+// there.  Workgroups go to the eight XCDs round robin by index, in this kernel and in the next;
+// the next kernel's workgroup nb (rows [nb * rows_per_block, +rows_per_block) of every slot)
+// therefore runs on XCD nb % 8.  Run by workgroups that have no other work (compute units the
+// gate/up tiles leave idle): workgroup `order` of the `per_xcd` on its XCD takes every per_xcd-th
+// (slot, row block) item of that XCD; slot `uniques` is the shared expert.  The loaded values
+// are not used: a wrong guess about the placement costs time, not results.
+template <int FMT>
+__device__ __forceinline__ void prefetch_down(const PfKernelArgs &a, const uint32_t *uniq, int uniques, int order,
+                                              int per_xcd, int rows_per_block, int row_blocks) {
+    const int xcd = blockIdx.x % 8, per_slot = row_blocks / 8, items = (uniques + 1) * per_slot;
+    const int mine = (items - order + per_xcd - 1) / per_xcd;
+    const size_t widest = (size_t)rows_per_block * max(a.row_bytes[3], a.row_bytes[6]);
+    const int lines = (int)((widest + 127) / 128) + (FMT == PF_IQ2_XXS ? 1 : 0);
+    uint32_t sink = 0;
+    for (int i = threadIdx.x; i < mine * lines; i += blockDim.x) {
+        const int item = order + per_xcd * (i / lines), l = i % lines;
+        const int slot = item / per_slot, nb = xcd + 8 * (item % per_slot);
+        const int tensor = slot == uniques ? 6 : 3;
+        const size_t e = slot == uniques ? 0 : uniq[slot], row0 = (size_t)nb * rows_per_block;
+        if (e >= (size_t)a.experts) continue;
+        const size_t bytes = (size_t)rows_per_block * a.row_bytes[tensor];
+        const uint8_t *p = a.w[tensor] + e * a.expert_bytes[tensor] + row0 * a.row_bytes[tensor];
+        if (FMT == PF_IQ2_XXS && l == lines - 1)
+            p = a.w[tensor] + a.scale_offset[tensor] + (e * a.n_out[tensor] + row0) * a.blocks_per_row[tensor] * 2;
+        else
+            p += min((size_t)l * 128, bytes - 4);
+        sink |= *reinterpret_cast<const volatile uint32_t *>((uintptr_t)p & ~(uintptr_t)3);
+    }
+    if (sink == 0x9e3779b9u && a.hidden < 0) atomicOr(a.error_word, 0u);   // keeps the loads; never true
+}
+
 // ---- kernel 2: routing, expert union, gate/up + SwiGLU of the routed and the shared expert ------
 struct RouteLds {
     uint32_t ids[64];        // [token][slot]
@@ -300,7 +332,6 @@ struct RouteLds {
     uint32_t mask[64];       // unique -> bit t set when token t uses it
     uint32_t count, close_mask, bad;
     uint32_t close[PF_DECODE_MAX_TOKENS], nonfinite[PF_DECODE_MAX_TOKENS];
-    float tile[PF_DECODE_MAX_TOKENS][32];
     PfRouteCands cands[PF_DECODE_MAX_TOKENS];
 };
 
@@ -354,23 +385,28 @@ __device__ __forceinline__ void route_finish(const PfKernelArgs &a, RouteLds *R,
     __syncthreads();
 }
 
-// 1024 threads.  Routed block b: unique slot b / tiles, units [32 * (b % tiles), +32) of that
-// expert; shared blocks follow.  Every wave owns two units (a unit = gate row + up row:
-// lower half-wave the gate row, upper half-wave the up row).  Waves 0..parts*NT-1 first
-// reduce the logits to candidates, waves 12..15 turn the activations into digit images.
+// 1024 threads.  Routed block b: unique slot b / tiles, units [tile * (b % tiles), +tile) of
+// that expert (tile = 16 or 32); shared blocks follow.  A wave owns tile / 16 units (a unit =
+// gate row + up row: lower half-wave the gate rows, upper half-wave the up rows) and writes its
+// activations itself, so no wave waits for another after the routing.  Waves 0..parts*NT-1 first reduce
+// the logits to candidates, waves 12..15 turn the token rows into digit images.
 template <int FMT, int NT, int NPL>
-__global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int routed_blocks, int parts, int chunk) {
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int routed_blocks, int shared_blocks, int parts, int chunk, int tile,
+                                                         int mode) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
     const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
     int *images = lds + table_words<FMT>();
     const int W = image_words(H), P = NT * K;
-    const bool shared = (int)blockIdx.x >= routed_blocks;
+    const bool prefetcher = (int)blockIdx.x >= routed_blocks + shared_blocks;   // no tile: warms the L2 for the next kernel
+    const bool shared = (int)blockIdx.x >= routed_blocks && !prefetcher;
     STAMP(0);
     if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
     const int rounds = K + 1;
-    if (!shared && wave < parts * NT) {
+    // mode 0: every workgroup routes; 1: this launch only routes and publishes (one workgroup);
+    // 2: the routes were published by an earlier launch
+    if (!shared && mode != 2 && wave < parts * NT) {
         const int t = wave / parts;
         pf_route_stage1<NPL>(a.logits + (size_t)t * E, a.logit_ssq + (size_t)t * E, E, wave % parts, chunk, rounds,
                              a.norm_topk != 0, &R.cands[t], lane);
@@ -382,8 +418,19 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
     int u, n0, I, gate_tensor;
     uint32_t e, mask;
     if (shared) {
-        u = P; n0 = 32 * (blockIdx.x - routed_blocks); I = a.shared_inter; gate_tensor = 4;
+        u = P; n0 = tile * (blockIdx.x - routed_blocks); I = a.shared_inter; gate_tensor = 4;
         e = 0; mask = (1u << NT) - 1u;
+    } else if (mode == 2) {
+        const int U = (int)a.uniq[0];
+        I = a.inter; gate_tensor = 1;
+        const int tiles = I / tile;
+        u = blockIdx.x / tiles; n0 = tile * (blockIdx.x % tiles);
+        if (u >= U) return;
+        e = a.uniq[1 + u]; mask = a.uniq[1 + 2 * P + u];
+        if (e >= (uint32_t)E) {   // only reachable with nonfinite logits
+            if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+            return;
+        }
     } else {
         if (wave < NT) {
             PfRouteResult r = pf_route_stage2(&R.cands[wave], parts, K, rounds, a.norm_topk != 0, H, lane);
@@ -409,9 +456,16 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
                 if (R.close_mask) atomicAdd(a.exact_rows, __popc(R.close_mask));
             }
         }
+        if (mode == 1) return;
+        if (prefetcher) {
+            const int rows_next = 64 / (a.inter / 64), first = routed_blocks + shared_blocks;
+            prefetch_down<FMT>(a, R.uniq, U, ((int)blockIdx.x - first) / 8, ((int)gridDim.x - first) / 8, rows_next,
+                               (H + rows_next - 1) / rows_next);
+            return;
+        }
         I = a.inter; gate_tensor = 1;
-        const int tiles = I / 32;
-        u = blockIdx.x / tiles; n0 = 32 * (blockIdx.x % tiles);
+        const int tiles = I / tile;
+        u = blockIdx.x / tiles; n0 = tile * (blockIdx.x % tiles);
         if (u >= U) return;
         e = R.uniq[u]; mask = R.mask[u];
         if (e >= (uint32_t)E) {   // only reachable with nonfinite logits
@@ -422,70 +476,42 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
     STAMP(4);
     const int LPR = H / 64, RPH = 32 / LPR;
     const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
-    // the tile's 32 units over 16 waves: two per wave, RPH per wave step
-    const int per_wave = RPH > 2 ? RPH : 2, steps = per_wave / RPH, unit0 = wave * per_wave;
-    if (unit0 < 32) {
+    // the tile's units over 16 waves: RPH per wave step, one or two steps
+    const int per_wave = max(RPH, tile / 16), steps = per_wave / RPH, unit0 = wave * per_wave;
+    if (unit0 < tile) {
         WSeg<FMT> w[2];
 #pragma unroll
-        for (int s = 0; s < 2; s++)
-            if (s < steps) wseg_load<FMT>(w[s], a, gate_tensor + half, e, n0 + unit0 + s * RPH + r, seg);
+        for (int st = 0; st < 2; st++)
+            if (st < steps) wseg_load<FMT>(w[st], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg);
 #pragma unroll
         for (int t = 0; t < NT; t++) {
             if (!((mask >> t) & 1u)) continue;
             XSeg x;
             xseg_load(x, images + t * W, H, seg);
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                if (s >= steps) break;
-                float v = span_sum(wseg_dot<FMT>(w[s], x, seg, tables), LPR);
+            for (int st = 0; st < 2; st++) {
+                if (st >= steps) break;
+                const float v = span_sum(wseg_dot<FMT>(w[st], x, seg, tables), LPR);
                 const float up = __shfl(v, (lane & 31) + 32);
-                if (half == 0 && seg == 0) R.tile[t][unit0 + s * RPH + r] = pf_silu(v) * up;
+                if (half == 0 && seg == 0) {
+                    const float act = pf_silu(v) * up;
+                    const int unit = unit0 + st * RPH + r;
+                    if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+                    if (shared) a.shared_act[(size_t)t * I + n0 + unit] = act;
+                    else a.act[((size_t)u * NT + t) * I + n0 + unit] = act;
+                }
             }
         }
     }
     STAMP(5);
-    __syncthreads();
-    STAMP(6);
-    // 32 activations per token: FP32 copy and digit image for the down kernel
-    if (wave < NT && ((mask >> wave) & 1u) && lane < 32) {
-        const int t = wave, WI = image_words(I), plane = SEG_STRIDE * (I / 64);
-        const float v = R.tile[t][lane];
-        if (!pf_finite(v)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-        if (shared) a.shared_act[(size_t)t * I + n0 + lane] = v;
-        else a.act[((size_t)u * NT + t) * I + n0 + lane] = v;
-        float m = fabsf(v);
-        for (int k = 16; k >= 1; k >>= 1) m = fmaxf(m, __shfl_xor(m, k));
-        float step, inv;
-        group_step(m, step, inv);
-        const int q = __float2int_rn(v * inv);
-        int d0, d1, d2, sum = q;
-        split_digits(q, d0, d1, d2);
-        const int sh = 8 * (lane & 3);
-        int w0 = (d0 & 255) << sh, w1 = (d1 & 255) << sh, w2 = (d2 & 255) << sh;
-        w0 |= dpp_quad_xor1(w0); w0 |= dpp_quad_xor2(w0);
-        w1 |= dpp_quad_xor1(w1); w1 |= dpp_quad_xor2(w1);
-        w2 |= dpp_quad_xor1(w2); w2 |= dpp_quad_xor2(w2);
-        for (int k = 16; k >= 1; k >>= 1) sum += __shfl_xor(sum, k);
-        int *img = shared ? a.shared_images + (size_t)t * WI : a.act_images + ((size_t)u * NT + t) * WI;
-        if ((lane & 3) == 0) {
-            const int nn = n0 + lane, at = SEG_STRIDE * (nn >> 6) + ((nn & 63) >> 2);
-            img[at] = w0;
-            img[plane + at] = w1;
-            img[2 * plane + at] = w2;
-        }
-        if (lane == 0) {
-            reinterpret_cast<float *>(img + 3 * plane)[n0 >> 5] = step;
-            img[3 * plane + I / 32 + (n0 >> 5)] = sum;
-        }
-    }
-    STAMP(7);
 }
 
 // ---- kernel 3: down products and the combine ---------------------------------------------------
 // blockIdx.x = t * row_blocks + nb; one wave per slot plus one for the shared expert; a routed
-// wave covers the block's rows in one step.
+// wave covers the block's rows in one step.  Every wave turns its slot's activation row into a
+// digit image in LDS while its weight bytes are on their way.
 template <int FMT, int NT>
-__global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_blocks, int rows_per_block) {
+__global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_blocks, int rows_per_block, int image_pitch) {
     __shared__ float partial[17][64];
     extern __shared__ int lds[];
     uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
@@ -509,16 +535,17 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_bl
     const int n_base = nb * rows_per_block;
     WSeg<FMT> w;   // further steps (a shared expert wider than the routed ones) load as they go
     wseg_load<FMT>(w, a, tensor, e, min(n_base + r, H - 1), seg);
-    XSeg x;
-    const int *image = shared ? a.shared_images + (size_t)t * image_words(I)
-                              : a.act_images + ((size_t)u * NT + t) * image_words(I);
-    xseg_load(x, image, I, seg);
+    int *image = lds + table_words<FMT>() + s * image_pitch;
+    build_image(image, shared ? a.shared_act + (size_t)t * I : a.act + ((size_t)u * NT + t) * I, I, 64 * s, 64);
     // operands of the final combine, requested now so that they arrive with the weights
     float rw[16];
 #pragma unroll
     for (int slot = 0; slot < 16; slot++) rw[slot] = slot < K ? a.route_weights[t * K + slot] : 0.0f;
     const float shared_scale = a.shared_scale[t];
     if (FMT == PF_IQ2_XXS) __syncthreads();
+    else pf_wave_lds_fence();
+    XSeg x;
+    xseg_load(x, image, I, seg);
     for (int st = 0; st < steps; st++) {
         const float v = span_sum(wseg_dot<FMT>(w, x, seg, tables), LPR);
         const int row = st * rows + r;
@@ -568,19 +595,28 @@ bool pf_decode_supported(const PfHipMoeDesc &d) {
         !pow2_between(d.shared_inter, 256, 2048) || d.down_physical != d.inter || d.shared_inter > 4 * d.inter)
         return false;
     if (d.experts > 1024 || d.top_k > 15 || d.top_k * PF_DECODE_MAX_TOKENS > 64 || d.top_k >= d.experts) return false;
+    // the down kernel keeps one digit image per slot (and the IQ2_XXS tables) in LDS
+    const uint32_t widest = d.inter > d.shared_inter ? d.inter : d.shared_inter;
+    if ((size_t)(d.top_k + 1) * image_words((int)widest) * 4 + 32 * 1024 > 140 * 1024) return false;
     return true;
 }
 
 template <int FMT, int NT, int NPL>
 static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks,
-                           int parts, int chunk) {
+                           int shared_blocks, int parts, int chunk, int tile) {
+    // more workgroups than compute units: routing once, in a launch of its own, beats every workgroup repeating it
+    const bool split = grid.x > 256;
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, NPL>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
         configured = true;
     }
-    hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, NPL>), grid, dim3(1024), lds, stream, a, routed_blocks, parts, chunk);
+    if (split)
+        hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, NPL>), dim3(1), dim3(1024), lds, stream, a, routed_blocks, shared_blocks,
+                           parts, chunk, tile, 1);
+    hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, NPL>), grid, dim3(1024), lds, stream, a, routed_blocks, shared_blocks, parts,
+                       chunk, tile, split ? 2 : 0);
 }
 
 template <int FMT, int NT>
@@ -592,21 +628,37 @@ static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_l
     hipLaunchKernelGGL((pf_k_dec_router<NT>), dim3(router_blocks + 1), dim3(256), 0, stream, a, router_blocks);
     if (last < 2) return;
     // kernel 2: the candidate stage uses up to 8 of waves 0..11 per token
-    const int routed_blocks = NT * K * (I / 32), shared_blocks = Is / 32;
+    // 32 units per workgroup: every workgroup repeats the routing, and one workgroup per compute
+    // unit measured faster than two half as long
+    const int tile = 32;
+    const int routed_blocks = NT * K * (I / tile), shared_blocks = Is / tile;
     const size_t lds2 = tab + (size_t)NT * image_words(H) * 4 + ((size_t)H + 3 * (size_t)E) * 4;
     int parts = NT == 1 ? 8 : NT == 2 ? 6 : NT == 3 ? 4 : 3;
     while (parts > 1 && (E + parts - 1) / parts < 64) parts--;
     const int chunk = (E + parts - 1) / parts, npl = (chunk + 63) / 64;
-    dim3 g2(routed_blocks + shared_blocks);
-    if (npl <= 1) launch_gate_up<FMT, NT, 1>(a, g2, lds2, stream, routed_blocks, parts, chunk);
-    else if (npl <= 2) launch_gate_up<FMT, NT, 2>(a, g2, lds2, stream, routed_blocks, parts, chunk);
-    else if (npl <= 4) launch_gate_up<FMT, NT, 4>(a, g2, lds2, stream, routed_blocks, parts, chunk);
-    else launch_gate_up<FMT, NT, 8>(a, g2, lds2, stream, routed_blocks, parts, chunk);   // experts <= 1024
+    // compute units left over by the tiles (256 on this GPU) warm the L2 for the down kernel, whose
+    // row blocks must then spread evenly over the eight XCDs
+    const int rows_next = 64 / (I / 64), row_blocks_next = (H + rows_next - 1) / rows_next;
+    int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
+    if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
+    dim3 g2(routed_blocks + shared_blocks + prefetch_blocks);
+    if (npl <= 1) launch_gate_up<FMT, NT, 1>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else if (npl <= 2) launch_gate_up<FMT, NT, 2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else if (npl <= 4) launch_gate_up<FMT, NT, 4>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else launch_gate_up<FMT, NT, 8>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024
     if (last < 3) return;
     // kernel 3
     const int rows_per_block = 64 / (I / 64), row_blocks = (H + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL((pf_k_dec_down<FMT, NT>), dim3(NT * row_blocks), dim3(64 * (K + 1)), tab, stream, a, row_blocks,
-                       rows_per_block);
+    const int image_pitch = image_words(I > Is ? I : Is);
+    const size_t lds3 = tab + (size_t)(K + 1) * image_pitch * 4;
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down<FMT, NT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL((pf_k_dec_down<FMT, NT>), dim3(NT * row_blocks), dim3(64 * (K + 1)), lds3, stream, a, row_blocks,
+                       rows_per_block, image_pitch);
 }
 
 template <int FMT>
