@@ -49,6 +49,11 @@ WORKLOADS = {
     "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10,
                             label="Q4_K experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
 }
+# HBM bytes per launch of each workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE scaled by the same counters on a plain 256 MiB copy (profiles/*.txt hold the runs).
+# A counter result cannot be read live; None where no such run exists for the workload.
+MEASURED_TRAFFIC = {"iq2xxs_decode": 9832986, "q4k_decode": 19831587, "q4k_verify4": None,
+                    "q4k_prefill1024": 1027142930}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
@@ -211,7 +216,8 @@ def main():
         "algorithmic_bytes_per_step": int(alg_bytes),
         "tokens_per_s": round(tokens / (ms_per_step * 1e-3), 1),
         "roofline": {"bound": "hbm", "kernel": names[dom], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get(args.workload),
                      "bytes_per_launch": int(stage_bytes[dom]), "us_per_launch": round(stage_us[dom], 3)},
         "kernel_us": dict(zip(names, [round(v, 3) for v in stage_us])),
         "kernel_bytes": dict(zip(names, [int(b) for b in stage_bytes])),

@@ -191,8 +191,8 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
 extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_bytes : 0; }
 
 // workspace layout: buffers carved from one allocation, each 256-byte aligned
-enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_SIMAGES, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS,
-       W_IMAGES, W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
+enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS,
+       W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
        W_P2R, W_R2P, W_GROUPBAD, W_TILES, W_COUNT };
 struct Carve { size_t offset[W_COUNT], total; };
 static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
@@ -200,7 +200,6 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     memset(&c, 0, sizeof c);
     const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden, I = d->inter;
     const size_t Td = T < PF_DECODE_MAX_TOKENS ? T : PF_DECODE_MAX_TOKENS;   // tokens per decode launch
-    const size_t image = (3 * 20 * ((I + 63) / 64) + 2 * ((I + 31) / 32)) * 4;
     size_t want[W_COUNT];
     want[W_LOGITS] = T * E * 4;
     want[W_SSQ] = T * E * 4;
@@ -208,7 +207,6 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_ACT] = (T * K > Td * K * Td ? T * K : Td * K * Td) * I * 4;
     want[W_SACT] = T * d->shared_inter * 4;
     want[W_SSCALE] = T * 4;
-    want[W_SIMAGES] = Td * (3 * 20 * ((d->shared_inter + 63) / 64) + 2 * ((d->shared_inter + 31) / 32)) * 4;
     want[W_X] = T * H * 4;
     want[W_Y] = T * H * 4;
     want[W_IDS] = T * K * 4;
@@ -216,7 +214,6 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_ERR] = 256;
     want[W_EXACT] = 256;
     want[W_FLAGS] = T * 4;
-    want[W_IMAGES] = Td * K * Td * image;
     // prefill path: fp16 copies, per-row scales, down products in expert order, grouping tables
     const bool prefill = T > PF_DECODE_MAX_TOKENS && pf_prefill_supported(*d);
     const size_t Tp = prefill ? T : 0, Is = d->shared_inter;
@@ -268,7 +265,6 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     w->act = (float *)(base + c.offset[W_ACT]);
     w->shared_act = (float *)(base + c.offset[W_SACT]);
     w->shared_scale = (float *)(base + c.offset[W_SSCALE]);
-    w->shared_images = (int *)(base + c.offset[W_SIMAGES]);
     w->x = (float *)(base + c.offset[W_X]);
     w->y = (float *)(base + c.offset[W_Y]);
     w->ids = (uint32_t *)(base + c.offset[W_IDS]);
@@ -276,7 +272,6 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     w->error_word = (uint32_t *)(base + c.offset[W_ERR]);
     w->exact_rows = (uint32_t *)(base + c.offset[W_EXACT]);
     w->route_flags = (uint32_t *)(base + c.offset[W_FLAGS]);
-    w->act_images = (int *)(base + c.offset[W_IMAGES]);
     if (c.offset[W_GROUPBAD] != c.offset[W_X16]) {   // the prefill buffers were planned
         w->x16 = (uint16_t *)(base + c.offset[W_X16]);
         w->act16 = (uint16_t *)(base + c.offset[W_ACT16]);
@@ -353,7 +348,7 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.x = d_x; a.x_pitch = x_pitch; a.y = d_y; a.y_pitch = y_pitch;
     a.logits = w->logits; a.logit_ssq = w->logit_ssq; a.ids = w->ids; a.route_weights = w->route_weights;
     a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale;
-    a.act_images = w->act_images; a.shared_images = w->shared_images; a.uniq = w->uniq;
+    a.uniq = w->uniq;
     a.error_word = w->error_word; a.exact_rows = w->exact_rows; a.route_flags = w->route_flags;
     a.x16 = w->x16; a.act16 = w->act16; a.sact16 = w->sact16;
     a.x_scale = w->x_scale; a.act_scale = w->act_scale; a.sact_scale = w->sact_scale; a.x_max2 = w->x_max2;

@@ -27,8 +27,6 @@ struct PfKernelArgs {
     float *act;                      // general path [tokens * top_k, inter]; decode path [unique, tokens, inter]
     float *shared_act;               // [tokens, shared_inter]
     float *shared_scale;             // [tokens] sigmoid of the shared router logit
-    int *act_images;                 // decode path: digit image of every [unique, token] activation row
-    int *shared_images;              // decode path: digit image of every token's shared activation row
     uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
     uint32_t *error_word;
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
@@ -63,7 +61,6 @@ struct PfHipWork {
     size_t cap, bytes;
     float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
     uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags;
-    int *act_images, *shared_images;
     uint16_t *x16, *act16, *sact16;  // prefill buffers (allocated when cap exceeds the decode path's batch)
     float *x_scale, *act_scale, *sact_scale, *x_max2, *down;
     uint32_t *counts, *offsets, *pair_to_row, *row_to_pair, *group_bad, *tiles;

@@ -414,12 +414,14 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, 
     __shared__ uint32_t src_row[32];
     __shared__ float row_scale[32];
     const int E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31;
-    const uint32_t tile = blockIdx.x / slabs;
+    // Workgroups go to the eight XCDs round robin by index.  The slabs of one row tile read the
+    // same activation rows, so they are given indices eight apart: one XCD, one L2.
+    const uint32_t xcd = blockIdx.x % 8, turn = blockIdx.x / 8, tile = (turn / slabs) * 8 + xcd;
     if (tile >= a.tiles[0]) return;
     const uint32_t entry = a.tiles[1 + tile];
     const int expert = entry & 0xffffu, m0 = 32 * (int)(entry >> 16);
     GemmTarget g;
-    g.slab = blockIdx.x % slabs;
+    g.slab = turn % slabs;
     g.shared = expert == E;
     const int P = tokens * a.top_k;
     g.first = g.shared ? P : (int)a.offsets[expert];
@@ -501,7 +503,7 @@ static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_
     }
     // the tile count is only known on the device: launch its upper bound, surplus workgroups exit at once
     const int max_tiles = pf_prefill_max_tiles(tokens, a.experts, a.top_k);
-    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3(max_tiles * slabs), dim3(256), lds, stream, a, tokens, slabs);
+    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3((max_tiles + 7) / 8 * 8 * slabs), dim3(256), lds, stream, a, tokens, slabs);
 }
 
 void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
