@@ -35,6 +35,13 @@ def product():
 
 
 @pytest.fixture(scope="session")
+def product_host():
+    """The shipped library for tests of its host logic: no device needed, none assumed."""
+    import picoforge_amd as pf
+    return pf.load_product()
+
+
+@pytest.fixture(scope="session")
 def synth():
     import picoforge_amd as pf
     return pf.Synth()
