@@ -77,6 +77,8 @@ void pf_launch_transpose(const float *d_src, int rows, int cols, float *d_dst, h
 int pf_route_exact_device(const float *d_logits, int tokens, int experts, int top_k, int norm,
                           float *d_probs, uint32_t *d_ids, float *d_weights, uint32_t *d_error,
                           unsigned long long *d_bad_row, hipStream_t stream);
+void pf_launch_group_place(const uint32_t *d_ids, int pairs, int experts, const uint32_t *d_offsets,
+                           uint32_t *d_pair_to_row, uint32_t *d_row_to_pair, hipStream_t stream);
 int pf_group_pairs_device(const uint32_t *d_ids, int tokens, int experts, int top_k, uint32_t *d_counts,
                           uint32_t *d_offsets, uint32_t *d_pair_to_row, uint32_t *d_row_to_pair,
                           uint32_t *d_first_bad, hipStream_t stream);

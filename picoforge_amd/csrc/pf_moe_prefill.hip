@@ -382,24 +382,50 @@ __device__ __forceinline__ void gemm_rows(const PfKernelArgs &a, const GemmTarge
     }
 }
 
-// Row tiles: every expert's rows (the shared expert = expert E with all tokens) cut into tiles of
-// 32; tiles[0] = count, tiles[1 + i] = expert | (tile index within the expert) << 16.
-__global__ void __launch_bounds__(256) pf_k_pf_tiles(const uint32_t *offsets, int E, int tokens, uint32_t *tiles) {
-    __shared__ uint32_t part[256];
+// Histogram of the routed pairs.  counts[] is zero on entry: the workspace starts zeroed and
+// pf_k_pf_scan_tiles clears it again once it has been read.
+__global__ void pf_k_pf_count(const uint32_t *ids, int pairs, int E, uint32_t *counts) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < pairs && ids[p] < (uint32_t)E) atomicAdd(&counts[ids[p]], 1u);
+}
+
+// One workgroup: exclusive scan of counts[E] into offsets[E + 1], and the row tiles: every
+// expert's rows (the shared expert = expert E with all tokens) cut into tiles of 32; tiles[0] =
+// count, tiles[1 + i] = expert | (tile index within the expert) << 16.  Leaves counts[] zero.
+__global__ void __launch_bounds__(256) pf_k_pf_scan_tiles(uint32_t *counts, int E, int tokens, uint32_t *offsets,
+                                                          uint32_t *tiles) {
+    __shared__ uint32_t rows_before[256], tiles_before[256];
     const int tid = threadIdx.x, per = (E + 1 + 255) / 256, lo = tid * per, hi = min(E + 1, lo + per);
-    uint32_t s = 0;
-    for (int e = lo; e < hi; e++) s += ((e < E ? offsets[e + 1] - offsets[e] : (uint32_t)tokens) + 31u) / 32u;
-    part[tid] = s;
+    uint32_t rows = 0, ntiles = 0;
+    for (int e = lo; e < hi; e++) {
+        const uint32_t c = e < E ? counts[e] : (uint32_t)tokens;
+        if (e < E) rows += c;
+        ntiles += (c + 31u) / 32u;
+    }
+    rows_before[tid] = rows;
+    tiles_before[tid] = ntiles;
     __syncthreads();
     if (tid == 0) {
-        uint32_t run = 0;
-        for (int i = 0; i < 256; i++) { const uint32_t v = part[i]; part[i] = run; run += v; }
-        tiles[0] = run;
+        uint32_t run_rows = 0, run_tiles = 0;
+        for (int i = 0; i < 256; i++) {
+            const uint32_t r = rows_before[i], n = tiles_before[i];
+            rows_before[i] = run_rows;
+            tiles_before[i] = run_tiles;
+            run_rows += r;
+            run_tiles += n;
+        }
+        offsets[E] = run_rows;
+        tiles[0] = run_tiles;
     }
     __syncthreads();
-    uint32_t at = part[tid];
+    uint32_t row = rows_before[tid], at = tiles_before[tid];
     for (int e = lo; e < hi; e++) {
-        const uint32_t n = ((e < E ? offsets[e + 1] - offsets[e] : (uint32_t)tokens) + 31u) / 32u;
+        const uint32_t c = e < E ? counts[e] : (uint32_t)tokens, n = (c + 31u) / 32u;
+        if (e < E) {
+            offsets[e] = row;
+            row += c;
+            counts[e] = 0;
+        }
         for (uint32_t i = 0; i < n; i++) tiles[1 + at + i] = (uint32_t)e | (i << 16);
         at += n;
     }
@@ -516,8 +542,9 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     if (last < 2) return;
     // stage 2: routes and grouping
     pf_launch_route(a, tokens, stream);
-    pf_group_pairs_device(a.ids, tokens, E, K, a.counts, a.offsets, a.pair_to_row, a.row_to_pair, a.group_bad, stream);
-    hipLaunchKernelGGL(pf_k_pf_tiles, dim3(1), dim3(256), 0, stream, a.offsets, E, tokens, a.tiles);
+    hipLaunchKernelGGL(pf_k_pf_count, dim3((P + 255) / 256), dim3(256), 0, stream, a.ids, P, E, a.counts);
+    hipLaunchKernelGGL(pf_k_pf_scan_tiles, dim3(1), dim3(256), 0, stream, a.counts, E, tokens, a.offsets, a.tiles);
+    pf_launch_group_place(a.ids, P, E, a.offsets, a.pair_to_row, a.row_to_pair, stream);
     if (last < 3) return;
     // stage 3: gate/up + SwiGLU, then fp16 parts of the activation rows
     const int gi = I > Is ? I : Is;

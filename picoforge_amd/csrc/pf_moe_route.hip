@@ -28,44 +28,54 @@ __global__ void __launch_bounds__(64) pf_k_route_fast(PfKernelArgs a) {
 
 // Serial-order recomputation for flagged tokens, in two kernels so that a token's logits
 // spread over many compute units: one wave per (token, 64 experts), lane e owns expert e and
-// walks k in order over the transposed router copy [hidden][experts], so that every step is
-// one coalesced 256-byte load; then one wave per token selects.
+// the sum runs over k in order, as the reference's, on the transposed router copy
+// [hidden][experts]: every step is one coalesced 256-byte load at a wave-uniform base plus the
+// lane's offset.  Then one wave per token selects.
 __global__ void __launch_bounds__(64) pf_k_route_fix_logits(PfKernelArgs a) {
 #pragma clang fp contract(off)
-    const int t = blockIdx.x, E = a.experts, H = a.hidden, e = blockIdx.y * PF_WAVE + threadIdx.x;
+    const int t = blockIdx.x, E = a.experts, H = a.hidden;
+    int e = blockIdx.y * PF_WAVE + threadIdx.x;
     if (!a.route_flags[t]) return;
-    extern __shared__ float xs[];
-    const float *w = a.router_t + min(e, E - 1), *x = a.x + (size_t)t * a.x_pitch;
-    for (int k = threadIdx.x; k < H; k += PF_WAVE) xs[k] = x[k];
-    pf_wave_lds_fence();
-    if (e >= E) return;
+    const float *__restrict__ xs = a.x + (size_t)t * a.x_pitch;
+    const float *__restrict__ wt = a.router_t;
+    const bool live = e < E;
+    e = min(e, E - 1);   // every lane keeps loading: the token's values are shared through v_readlane
     // The sum is one dependent chain; the loads are not.  They are requested 128 at a time, one
-    // batch ahead of the chain, so that the chain rarely waits for memory.
-    float sum = 0.0f, wa[128], wb[128];
-    const int batches = H / 128;
-    auto load = [&](float (&dst)[128], int b) {
-#pragma unroll
-        for (int j = 0; j < 128; j++) dst[j] = w[(size_t)(128 * b + j) * E];
-    };
-    auto chain = [&](const float (&src)[128], int b) {
+    // batch ahead of the chain, so that the chain rarely waits for memory.  The token's values
+    // travel the same way, 64 per register, and reach the chain through v_readlane.
+    float sum = 0.0f, wa[128], wb[128], xa[2], xb[2];
+    const int batches = H / 128, lane = threadIdx.x;
+    const uint32_t lane_bytes = 4u * (uint32_t)e;   // uniform row base + 32-bit lane offset: no per-load address arithmetic
+    auto load = [&](float (&dst)[128], float (&xdst)[2], int b) {
+        const char *row = reinterpret_cast<const char *>(wt + (size_t)(128 * b) * E);
+        xdst[0] = xs[128 * b + lane];
+        xdst[1] = xs[128 * b + 64 + lane];
 #pragma unroll
         for (int j = 0; j < 128; j++) {
-            const float p = src[j] * xs[128 * b + j];
+            dst[j] = *reinterpret_cast<const float *>(row + lane_bytes);
+            row += 4 * (size_t)E;
+        }
+    };
+    auto chain = [&](const float (&src)[128], const float (&xsrc)[2]) {
+#pragma unroll
+        for (int j = 0; j < 128; j++) {
+            const float xj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xsrc[j >> 6]), j & 63));
+            const float p = src[j] * xj;
             sum = sum + p;
         }
     };
-    if (batches > 0) load(wa, 0);
+    if (batches > 0) load(wa, xa, 0);
     for (int b = 0; b < batches; b += 2) {
-        if (b + 1 < batches) load(wb, b + 1);
-        chain(wa, b);
-        if (b + 2 < batches) load(wa, b + 2);
-        if (b + 1 < batches) chain(wb, b + 1);
+        if (b + 1 < batches) load(wb, xb, b + 1);
+        chain(wa, xa);
+        if (b + 2 < batches) load(wa, xa, b + 2);
+        if (b + 1 < batches) chain(wb, xb);
     }
     for (int k = 128 * batches; k < H; k++) {
-        const float p = w[(size_t)k * E] * xs[k];
+        const float p = (wt + (size_t)k * E)[e] * xs[k];
         sum = sum + p;
     }
-    a.logits[(size_t)t * E + e] = sum;
+    if (live) a.logits[(size_t)t * E + e] = sum;
 }
 
 // router [experts][hidden] -> [hidden][experts], once at upload
@@ -111,8 +121,7 @@ void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     else if (npl <= 4) hipLaunchKernelGGL(pf_k_route_fast<4>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 8) hipLaunchKernelGGL(pf_k_route_fast<8>, dim3(tokens), dim3(64), 0, stream, a);
     else hipLaunchKernelGGL(pf_k_route_fast<16>, dim3(tokens), dim3(64), 0, stream, a);
-    hipLaunchKernelGGL(pf_k_route_fix_logits, dim3(tokens, (a.experts + PF_WAVE - 1) / PF_WAVE), dim3(PF_WAVE),
-                       (size_t)a.hidden * sizeof(float), stream, a);
+    hipLaunchKernelGGL(pf_k_route_fix_logits, dim3(tokens, (a.experts + PF_WAVE - 1) / PF_WAVE), dim3(PF_WAVE), 0, stream, a);
     hipLaunchKernelGGL(pf_k_route_fix_select, dim3(tokens), dim3(PF_WAVE), 3 * (size_t)a.experts * sizeof(float), stream,
                        a);
 }
@@ -226,6 +235,12 @@ __global__ void __launch_bounds__(256) pf_k_group_place(const uint32_t *ids, int
             base += __popcll(mask);
         }
     }
+}
+
+void pf_launch_group_place(const uint32_t *d_ids, int pairs, int experts, const uint32_t *d_offsets,
+                           uint32_t *d_pair_to_row, uint32_t *d_row_to_pair, hipStream_t stream) {
+    hipLaunchKernelGGL(pf_k_group_place, dim3((experts + 3) / 4), dim3(256), 0, stream, d_ids, pairs, experts, d_offsets,
+                       d_pair_to_row, d_row_to_pair);
 }
 
 int pf_group_pairs_device(const uint32_t *d_ids, int tokens, int experts, int top_k, uint32_t *d_counts,
