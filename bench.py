@@ -48,6 +48,9 @@ WORKLOADS = {
                         label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
     "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10,
                             label="Q4_K experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
+    "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
+                        label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
+                              "uniform and Zipf(1.1) expert popularity"),
 }
 # HBM bytes per launch of each workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE scaled by the same counters on a plain 256 MiB copy (profiles/*.txt hold the runs).
@@ -63,6 +66,90 @@ PREFILL_STAGES = ["pf_k_rows_to_half + pf_k_pf_router (fp16 copy of x, router lo
                   "pf_k_pf_gemm<down> + pf_k_pf_combine (grouped down by FP16 MFMA, slot-ordered combine)"]
 
 
+def run_stack(args, api, hip, cfg, steps, warmup):
+    """A stack of independent layers, all resident: every token (or chunk) passes the layers in order, each
+    layer with its own seeded input, hence its own routing.  The popularity bias sits in router column 0
+    (workloads.zipf_router): inputs with coordinate 0 = 1 see Zipf(1.1) popularity, with 0 the plain router."""
+    layers_n, chunk = args.layers, 2048
+    t0 = time.time()
+    layers, sample = [], None
+    for l in range(layers_n):
+        weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=args.seed * 1000 + l)
+        workloads.zipf_router(weights, seed=args.seed * 1000 + l, temperature=0.18)
+        layers.append(pf.MoeLayer(api, cfg, weights, chunk))
+        if l == 0:
+            sample = weights
+        else:
+            layers[-1].weights = None      # the library copied the bytes into HBM at create
+    prep_s = time.time() - t0
+    moes = (C.c_void_p * layers_n)(*[l.device_handles()[0] for l in layers])
+    works = (C.c_void_p * layers_n)(*[l.device_handles()[1] for l in layers])
+    resident = sum(hip.moe_bytes(m) for m in moes)
+    synth = pf.Synth()
+    h = cfg.hidden_size
+    per_layer_tokens = 32
+    dec = pf.rms_normalise(synth.normal((per_layer_tokens * layers_n, h), 77 + args.seed))
+    pre = synth.normal((4 * chunk, h), 78 + args.seed)
+    d_y = hip.to_device(np.zeros((chunk, h), dtype=np.float32))
+    out = {}
+    ms = C.c_float()
+    for name, coord in (("uniform", 0.0), ("zipf", 1.0)):
+        dec[:, 0] = coord
+        pre[:, 0] = coord
+        d_dec, d_pre = hip.to_device(dec), hip.to_device(pre)
+        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_dec, len(dec), d_y, 1, warmup * layers_n, C.byref(ms)), "warmup")
+        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_dec, len(dec), d_y, 1, steps * layers_n, C.byref(ms)), "decode")
+        out[name + "_decode_us_per_token"] = ms.value * 1e3 / steps
+        chunks = max(2, steps // 50)
+        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_pre, 4, d_y, chunk, layers_n, C.byref(ms)), "warmup")
+        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_pre, 4, d_y, chunk, chunks * layers_n, C.byref(ms)), "prefill")
+        out[name + "_prefill_ms_per_chunk"] = ms.value / chunks
+        out[name + "_prefill_tokens_per_s"] = chunk / (ms.value / chunks * 1e-3)
+        hip.free(d_dec)
+        hip.free(d_pre)
+    errors = sum(int(hip.from_device(hip.work_error_word(w), (1,), np.uint32)[0]) for w in works)
+    # parity and the CPU cost per layer-token on layer 0; the stack's CPU time is that times the layers
+    ref = pf.load_reference()
+    cpu_api, kind = (ref, "reference") if ref is not None else (pf.load_oracle(), "port")
+    n = args.cpu_sample or 16
+    xs = dec[:n].copy()
+    with pf.MoeLayer(cpu_api, cfg, sample, n) as cpu:
+        c0 = time.perf_counter()
+        _, y0, ids0, _ = cpu.forward(xs)
+        cpu_s = time.perf_counter() - c0
+    _, y1, ids1, _ = layers[0].forward(xs)
+    ids_equal = bool((ids0 == ids1).all())
+    within = bool((np.abs(y1 - y0) <= 1e-3 + 1e-4 * np.abs(y0)).all())
+    for l in layers:
+        l.close()
+    us = out["uniform_decode_us_per_token"]
+    alg = layers_n * workloads.algorithmic_bytes_per_token(abi.GGUF_Q4_K)
+    result = {
+        "metric": "moe_stack_decode_us_per_token", "value": round(us, 2), "unit": "us/token (all layers)",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(us * 1e-3, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{layers_n} independent MoE layers (hidden 2048, 512 experts, top-10, intermediate 512, "
+                               f"shared 512, Q4_K), {resident / 1e9:.1f} GB resident in HBM; decode batch 1 and "
+                               f"{chunk}-token prefill chunks; per-layer seeded inputs and routers",
+                   "layers": layers_n, "tokens_per_step": 1},
+        "us_per_layer_token": round(us / layers_n, 3),
+        "hbm_GBps_on_algorithmic_bytes": round(alg / (us * 1e-6) / 1e9, 1),
+        "algorithmic_bytes_per_step": int(alg),
+        "roofline": {"bound": "hbm", "kernel": "whole stack: three decode kernels per layer", "achieved":
+                     round(alg / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None},
+        "stack": {k: round(v, 3) for k, v in out.items()},
+        "cpu_baseline": {"value": round(cpu_s / n * 1e6 * layers_n, 1), "unit": "us/token (all layers)", "cores": 1,
+                         "kind": kind, "sample": f"{n} tokens through layer 0 ({cpu_s:.1f} s), times {layers_n} layers: "
+                                                 "an extrapolation, the CPU cost is linear in layers and tokens"},
+        "parity_on_sample": {"ids_equal": ids_equal, "within_1e-3_abs_1e-4_rel": within, "error_word": errors},
+        "prep_s": round(prep_s, 1),
+    }
+    print(json.dumps(result))
+    if not (ids_equal and within and errors == 0):
+        sys.exit("parity check failed on the sample")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -71,6 +158,7 @@ def main():
     ap.add_argument("--workload", default="iq2xxs_decode", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-sample", type=int, default=None, help="tokens timed on the CPU path (default ~15 s of work)")
     ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--layers", type=int, default=48, help="layers of the q4k_stack48 workload")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="also launch a plain copy kernel of this many MiB three times (byte-counter calibration)")
     args = ap.parse_args()
@@ -85,6 +173,8 @@ def main():
     if hip.device_count() < 1:
         sys.exit("no HIP device: the benchmark runs the HIP path only")
     cfg = workloads.measured_config()
+    if args.workload == "q4k_stack48":
+        return run_stack(args, api, hip, cfg, steps, warmup)
     tokens = wl["tokens"]
     prefill = tokens > 4
     t0 = time.time()

@@ -133,6 +133,13 @@ int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *
                              size_t n_inputs, float *d_y, size_t tokens, size_t iters,
                              float *elapsed_ms);
 
+/* The same for a stack of layers of equal hidden size (works[l] belongs to moes[l]):
+ * forward i runs through layer i % layers with input row block i % n_inputs, so
+ * `iters` = tokens-through-the-stack x layers. */
+int pf_hip_stack_time_forwards(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers,
+                               const float *d_x, size_t n_inputs, float *d_y, size_t tokens,
+                               size_t iters, float *elapsed_ms);
+
 /* Average duration of each kernel inside the dependent chain: the same loop run
  * with only the first 1, 2, ... kernels of every forward launched; stage_ms[j] is
  * the difference between consecutive runs divided by iters.  Decode path (1..4

@@ -131,6 +131,7 @@ class HipShim:
         bind("pf_hip_synchronize", C.c_int)
         bind("pf_hip_moe_time_forwards", C.c_int, vp, vp, vp, sz, vp, sz, sz, P(C.c_float))
         bind("pf_hip_moe_profile_stages", C.c_int, vp, vp, vp, sz, vp, sz, sz, P(C.c_float))
+        bind("pf_hip_stack_time_forwards", C.c_int, P(vp), P(vp), sz, vp, sz, vp, sz, sz, P(C.c_float))
         bind("pf_hip_copy_probe", C.c_int, sz, sz)
 
     def check(self, rc, what):

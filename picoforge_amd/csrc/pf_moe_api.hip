@@ -579,30 +579,31 @@ extern "C" int pf_hip_synchronize(void) {
 // `iters` forwards back to back on one stream.  The launches are captured into graphs of
 // up to 256 forwards (each with its own input block) and the graphs are replayed in order,
 // so the measured gap between dependent kernels is the device's, not the host's enqueue rate.
-static int time_graph_replay(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs, float *d_y,
-                             size_t tokens, size_t iters, int stage_limit, float *elapsed_ms) {
+// Forward i goes through layer i % layers (a stack of layers in order, token after token).
+static int time_graph_replay(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers, const float *d_x,
+                             size_t n_inputs, float *d_y, size_t tokens, size_t iters, int stage_limit, float *elapsed_ms) {
     *elapsed_ms = 0.0f;
     if (!iters) return PF_HIP_OK;
-    const size_t H = moe->desc.hidden, chunk = 256, n_graphs = (iters + chunk - 1) / chunk;
+    const size_t H = moes[0]->desc.hidden, chunk = 256, n_graphs = (iters + chunk - 1) / chunk;
     hipStream_t s = nullptr;
     hipEvent_t t0 = nullptr, t1 = nullptr;
     HIP_TRY(hipStreamCreate(&s));
     hipGraphExec_t *execs = (hipGraphExec_t *)calloc(n_graphs, sizeof *execs);
     int rc = execs ? PF_HIP_OK : PF_HIP_E_MEMORY;
-    const int saved_limit = work->stage_limit;
-    work->stage_limit = stage_limit;
+    for (size_t l = 0; l < layers; l++) works[l]->stage_limit = stage_limit;
     for (size_t g = 0; g < n_graphs && rc == PF_HIP_OK; g++) {
         hipGraph_t graph = nullptr;
         if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) { rc = PF_HIP_E_RUNTIME; break; }
         for (size_t i = g * chunk; i < iters && i < (g + 1) * chunk && rc == PF_HIP_OK; i++)
-            rc = pf_hip_moe_forward_device(moe, work, d_x + (i % n_inputs) * tokens * H, H, d_y, H, tokens, s);
+            rc = pf_hip_moe_forward_device(moes[i % layers], works[i % layers], d_x + (i % n_inputs) * tokens * H, H, d_y, H,
+                                           tokens, s);
         hipError_t e = hipStreamEndCapture(s, &graph);
         if (e != hipSuccess && rc == PF_HIP_OK) { pf_set_error("hipStreamEndCapture", e); rc = PF_HIP_E_RUNTIME; }
         if (rc == PF_HIP_OK && hipGraphInstantiate(&execs[g], graph, nullptr, nullptr, 0) != hipSuccess)
             rc = PF_HIP_E_RUNTIME;
         if (graph) (void)hipGraphDestroy(graph);
     }
-    work->stage_limit = saved_limit;
+    for (size_t l = 0; l < layers; l++) works[l]->stage_limit = 0;
     if (rc == PF_HIP_OK && (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess)) rc = PF_HIP_E_RUNTIME;
     if (rc == PF_HIP_OK) {
         hipError_t e = hipEventRecord(t0, s);
@@ -623,7 +624,17 @@ static int time_graph_replay(const PfHipMoe *moe, PfHipWork *work, const float *
 extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
                                         float *d_y, size_t tokens, size_t iters, float *elapsed_ms) {
     if (!moe || !work || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
-    return time_graph_replay(moe, work, d_x, n_inputs, d_y, tokens, iters, 0, elapsed_ms);
+    return time_graph_replay(&moe, &work, 1, d_x, n_inputs, d_y, tokens, iters, 0, elapsed_ms);
+}
+
+extern "C" int pf_hip_stack_time_forwards(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers,
+                                          const float *d_x, size_t n_inputs, float *d_y, size_t tokens, size_t iters,
+                                          float *elapsed_ms) {
+    if (!moes || !works || !layers || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
+    for (size_t l = 0; l < layers; l++)
+        if (!moes[l] || !works[l] || works[l]->moe != moes[l] || moes[l]->desc.hidden != moes[0]->desc.hidden)
+            return PF_HIP_E_ARGUMENT;
+    return time_graph_replay(moes, works, layers, d_x, n_inputs, d_y, tokens, iters, 0, elapsed_ms);
 }
 
 // Kernel durations inside the dependent chain: the same graph replay with only the first
@@ -640,8 +651,8 @@ extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, c
     for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
     for (int j = 0; j < stages; j++) {
         float warm = 0.0f, ms = 0.0f;
-        int rc = time_graph_replay(moe, work, d_x, n_inputs, d_y, tokens, iters < 64 ? iters : 64, j + 1, &warm);
-        if (rc == PF_HIP_OK) rc = time_graph_replay(moe, work, d_x, n_inputs, d_y, tokens, iters, j + 1, &ms);
+        int rc = time_graph_replay(&moe, &work, 1, d_x, n_inputs, d_y, tokens, iters < 64 ? iters : 64, j + 1, &warm);
+        if (rc == PF_HIP_OK) rc = time_graph_replay(&moe, &work, 1, d_x, n_inputs, d_y, tokens, iters, j + 1, &ms);
         if (rc != PF_HIP_OK) return rc;
         stage_ms[j] = (ms - previous) / (float)iters;
         previous = ms;
