@@ -92,9 +92,10 @@ Qwen4Status qw4_moe_group_pairs(const Qwen4MoeConfig *config, Qwen4U32Mut ids,
 
 /* Replaces qw4_moe_observe (src/qwen4_moe.c:130-132).  Stage numbers follow
  * src/qwen4_moe_internal.h:9-12: 0..7 projections in weight order, 8 SiLU,
- * 9 product, 10 sigmoid, 11 routed, 12 y.  The device path reports stages
- * 0, 10, 11 and 12 for the whole batch and stages 1..9 per (token, slot) pair
- * with one input row each; views are host copies valid during the callback. */
+ * 9 product, 10 sigmoid, 11 routed, 12 y.  The intermediate stages stay on the
+ * device and are not copied out: this path reports stage 12 only (x as input,
+ * y as output, once per forward); views are the caller's, valid during the
+ * callback. */
 typedef void (*QW4MoeObserver)(void *ctx, size_t stage, size_t expert, size_t token,
                                Qwen4F32 input, Qwen4F32 output);
 void qw4_moe_observe(Qwen4MoeWork *work, QW4MoeObserver observer, void *ctx);

@@ -316,6 +316,8 @@ extern "C" int pf_hip_work_clear_status(PfHipWork *w) {
     return PF_HIP_OK;
 }
 
+// Instrumented builds only (-DPF_TIMING=<workgroup>): the decode kernels leave wall_clock64
+// stamps of their phases behind the re-route counter; this reads them back.
 #ifdef PF_TIMING
 extern "C" int pf_hip_debug_read(PfHipWork *w, void *out, size_t bytes) {
     HIP_TRY(hipDeviceSynchronize());
