@@ -175,6 +175,25 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             pf_hip_moe_destroy(m);
             return e == hipErrorOutOfMemory ? PF_HIP_E_MEMORY : PF_HIP_E_RUNTIME;
         }
+        // Second, tile-ordered copy of the expert tensors: the grouped product then reads whole cache
+        // lines once instead of 32-byte pieces of lines it meets again a stage later.  It doubles the
+        // expert bytes; PF_MOE_PREFILL_COPY=0 does without it (the same kernels read the row order).
+        const char *copy = getenv("PF_MOE_PREFILL_COPY");
+        if (!copy || strcmp(copy, "0") != 0) {
+            for (int a = 1; a <= 6 && e == hipSuccess; a++) {
+                e = hipMalloc((void **)&m->w_tiled[a], m->bytes[a]);
+                if (e == hipSuccess) {
+                    pf_launch_q4k_tile(m->w[a], m->w_tiled[a], (size_t)n_out[a] * experts[a], m->blocks_per_row[a], nullptr);
+                    m->total_bytes += m->bytes[a];
+                }
+            }
+            if (e == hipSuccess) e = hipDeviceSynchronize();
+            if (e != hipSuccess) {
+                pf_set_error("tile-ordered weights", e);
+                pf_hip_moe_destroy(m);
+                return e == hipErrorOutOfMemory ? PF_HIP_E_MEMORY : PF_HIP_E_RUNTIME;
+            }
+        }
     }
     *out = m;
     return PF_HIP_OK;
@@ -185,6 +204,7 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
     for (int a = 0; a < 8; a++) if (m->w[a]) (void)hipFree(m->w[a]);
     if (m->w_norm2) (void)hipFree(m->w_norm2);
     if (m->router_t) (void)hipFree(m->router_t);
+    for (int a = 0; a < 8; a++) if (m->w_tiled[a]) (void)hipFree(m->w_tiled[a]);
     free(m);
 }
 
@@ -359,6 +379,7 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.group_bad = w->group_bad; a.tiles = w->tiles;
     a.token_cap = (uint32_t)w->cap;
     a.router_t = m->router_t;
+    for (int j = 0; j < 8; j++) a.wt[j] = m->w_tiled[j];
     return a;
 }
 

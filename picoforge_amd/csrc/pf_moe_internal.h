@@ -14,6 +14,7 @@ struct PfKernelArgs {
     size_t row_bytes[8], expert_bytes[8];   // of the payload (IQ2_XXS: 64 bytes per block)
     size_t scale_offset[8];                 // IQ2_XXS: byte offset of the half scales in the tensor buffer
     int k_logical[8], blocks_per_row[8], n_out[8];
+    const uint8_t *wt[8];            // Q4_K expert tensors in tile order for the grouped product (null: not kept)
     const float *router_t;           // router transposed to [hidden][experts] (serial-order re-routing)
     const uint64_t *iq2_grid;        // 256 x 8 magnitudes, device memory
     const uint32_t *iq2_signed;      // 2 x 4096 words: four signed magnitudes per (grid entry, sign nibble)
@@ -54,6 +55,7 @@ struct PfHipMoe {
     bool prefill_ready;              // shapes and formats the matrix-core prefill kernels cover
     float *w_norm2;                  // [experts] squared norm of each router row
     float *router_t;                 // [hidden][experts] transposed copy of the router
+    uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
 };
 
 struct PfHipWork {
@@ -96,6 +98,7 @@ void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_
 // pf_moe_prefill.hip
 bool pf_prefill_supported(const PfHipMoeDesc &d);
 void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_q4k_tile(const uint8_t *d_src, uint8_t *d_dst, size_t rows, int blocks_per_row, hipStream_t stream);
 void pf_launch_row_norm2(const float *d_w, int rows, int cols, float *d_out, hipStream_t stream);
 size_t pf_prefill_half_row(int cols);   // halfs per row of the fp16 form of a matrix with `cols` columns
 int pf_prefill_max_tiles(int tokens, int experts, int top_k);

@@ -27,11 +27,36 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-#define A_PITCH 264   // halfs per LDS row of a 256-wide activation tile: 528 bytes, 33 sixteen-byte slots
-#define S_PITCH 24    // halfs per LDS row of the group sums (16 used)
-
-// halfs per row of a converted matrix: high parts, low parts, per 256-block 8 + 8 group sums
+// halfs per row of a converted matrix: high parts, low parts, per 256-block the 16 group-sum halfs
+// [even groups: 4 high, 4 low][odd groups: 4 high, 4 low]
 __host__ __device__ constexpr size_t pf_half_row(int cols) { return 2 * (size_t)cols + (size_t)cols / 16; }
+
+// ---- Q4_K tensors in tile order (once, at upload) ---------------------------------------------
+// The grouped product's loader moves one 32-row tile's share of a 256-block per instruction group.
+// In GGUF row order that is 32 pieces a row pitch apart; here the same bytes are regrouped so that
+// it is 4608 consecutive bytes: [32 headers of 16 bytes][run 0..3: 16-byte halves 0 of the 32 rows,
+// then halves 1].  One thread per 16-byte piece; rows is a multiple of 32.
+__global__ void pf_k_q4k_tile(const uint8_t *src, uint8_t *dst, size_t rows, int blocks_per_row) {
+    const size_t piece = (size_t)blockIdx.x * blockDim.x + threadIdx.x, pieces = rows * (size_t)blocks_per_row * 9;
+    if (piece >= pieces) return;
+    const size_t chunk = piece / 288, tile = chunk / blocks_per_row, kb = chunk % blocks_per_row;
+    const int p = (int)(piece % 288);
+    size_t n, off;
+    if (p < 32) {
+        n = p; off = 0;
+    } else {
+        const int q = p - 32;
+        n = q & 31; off = 16 + 32 * (q >> 6) + 16 * ((q >> 5) & 1);
+    }
+    const size_t row_bytes = (size_t)blocks_per_row * 144;
+    reinterpret_cast<uint4 *>(dst)[piece] =
+        *reinterpret_cast<const uint4 *>(src + (32 * tile + n) * row_bytes + 144 * kb + off);
+}
+
+void pf_launch_q4k_tile(const uint8_t *d_src, uint8_t *d_dst, size_t rows, int blocks_per_row, hipStream_t stream) {
+    const size_t pieces = rows * (size_t)blocks_per_row * 9;
+    hipLaunchKernelGGL(pf_k_q4k_tile, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, stream, d_src, d_dst, rows, blocks_per_row);
+}
 
 // ---- rows to scaled fp16 pairs ------------------------------------------------------------------
 // One workgroup per row (cols a multiple of 256).  scale = 2^e with max|row| / scale in
@@ -79,8 +104,9 @@ __global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_
         if ((j & 3) == 0) {
             const int g = j >> 2;
             const half_t sh = (half_t)sum, sl = (half_t)(sum - (float)sh);
-            out[2 * cols + 16 * (g >> 3) + (g & 7)] = sh;
-            out[2 * cols + 16 * (g >> 3) + 8 + (g & 7)] = sl;
+            half_t *sums = out + 2 * cols + 16 * (g >> 3) + 8 * (g & 1) + ((g & 7) >> 1);
+            sums[0] = sh;
+            sums[4] = sl;
         }
     }
     if (threadIdx.x == 0) {
@@ -155,229 +181,266 @@ __global__ void __launch_bounds__(256) pf_k_pf_router(PfKernelArgs a, int tokens
 // ---- grouped product ------------------------------------------------------------------------------
 enum { PF_GEMM_GATE_UP = 0, PF_GEMM_DOWN = 1 };
 
-struct Q4Raw { uint4 hdr; uint4 q[4]; };   // one lane's share of a row's 144-byte block: header + 16 bytes per 64 weights
+// Workgroup = one 32-row tile of an expert against 64 NW weight rows: NW compute waves, each
+// with two 32-row weight tiles (gate + up of 32 units, or 2 x 32 down rows), and 1 + NW / 4 loader
+// waves.
+//
+// Only the loader waves issue global loads.  They move the operands of one stage (64 of the K
+// columns) straight into LDS, 16 bytes per lane, up to five stages ahead of the products, through
+// a ring of six slots: with one workgroup per compute unit that keeps about 100 KB on their way,
+// what it takes to cover the memory latency at full bandwidth; a wave counts at most 63 loads, so
+// the stream is split over three loaders (activations; the weight runs of compute waves 0-3; of
+// 4-7).  A stalled memory pipeline holds up the loaders, never the waves that feed the matrix
+// cores.  One workgroup barrier per stage hands the landed slot to the compute waves and the slot
+// they have just left back to the loaders.
+//
+//   slot   [0, A_PART)            high parts of the 32 activation rows, 128 bytes each: four images
+//                                 of eight rows, chunk-major (16-byte chunk c of row r at 128 c + 16 r)
+//          [A_PART, 2 A_PART)     low parts likewise
+//          [SLOT_W, +2 NW KB)     the stage's 32-byte nibble run of every weight row: per tile the
+//                                 first halves of the 32 rows, then the second halves
+//   once per 256-block: the 16-byte block headers of the 2 NW tiles, the activation rows' group sums
+//
+// Matrix-core operands.  Lane (n = lane % 32, h = lane / 32) holds column n (a weight row) and
+// supplies K slots 8h..8h+7.  In stage j, step t, these are the codes 8t..8t+7 of group 2j + h
+// (h = 0: the low nibbles of the run, h = 1: the high nibbles), so a lane needs the scale and the
+// minimum of one group per stage, and activation columns 64 j + 32 h + 8 t + 0..7.
+#define NW 8                               // compute waves per workgroup
+#define NL (1 + NW / 4)                    // loader waves
+#define RING_SLOTS 5
+#define A_GROUP 1152                       // bytes between eight-row images: 1 KB + 128, neighbours start on opposite bank halves
+#define A_PART (4 * A_GROUP)
+#define SLOT_W (2 * A_PART)
+#define SLOT_BYTES (SLOT_W + 2 * NW * 1024)
+#define HDR_OFF (RING_SLOTS * SLOT_BYTES)
+#define BLOCK_BYTES (2 * NW * 512 + 1024)   // per 256-block: headers, then sums; two copies (blocks alternate)
+#define SUMS_OFF (HDR_OFF + 2 * NW * 512)
+#define GEMM_LDS (HDR_OFF + 2 * BLOCK_BYTES)   // 146 432 bytes with 8 compute waves: one workgroup per compute unit
+static_assert(RING_SLOTS == 5 && NW % 4 == 0, "the loaders' wait counts below assume three younger stages on their way");
 
-__device__ __forceinline__ void q4_load(Q4Raw &r, const uint8_t *block, int h) {
-    r.hdr = *reinterpret_cast<const uint4 *>(block);
-#pragma unroll
-    for (int j = 0; j < 4; j++) r.q[j] = *reinterpret_cast<const uint4 *>(block + 16 + 32 * j + 16 * h);
+__device__ __forceinline__ void to_lds(const void *global, unsigned char *lds) {
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(global), reinterpret_cast<uint32_t *>(lds), 16, 0, 0);
 }
 
-// 6-bit scale and min of group g from the 12 packed bytes (src/qwen4_packed.c:88-91)
-__device__ __forceinline__ void q4_scale_min(const Q4Raw &r, int g, uint32_t &sc, uint32_t &mn) {
-    const uint32_t w[3] = {r.hdr.y, r.hdr.z, r.hdr.w};
-    const int sh = 8 * (g & 3);
-    if (g < 4) {
-        sc = (w[0] >> sh) & 63u;
-        mn = (w[1] >> sh) & 63u;
+__device__ __forceinline__ void stage_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+struct GemmTarget {   // what one workgroup of the grouped product works on
+    bool shared;
+    int first, count, inter, kblocks, a_cols, slab;
+    int waves;            // compute waves whose weight rows exist (the last slab of a narrow matrix has fewer)
+    uint32_t zero_row;    // index of the all-zero row that ends the fp16 form of the activation matrix
+    uint32_t row_bytes;   // of the weight tensor(s)
+    uint32_t wave_rows;   // weight rows between the tiles of consecutive compute waves
+    bool tiled;           // weights in the tile order of pf_k_q4k_tile (else GGUF row order)
+    const uint8_t *w0, *w1;   // first weight row of compute wave 0's two tiles
+    const half_t *a16;
+    const float *a_scale;
+};
+
+// Loads of the stages that may still be on their way when stage s is handed over: the younger
+// stages issued so far, at most three.  Three consecutive stages hold one that opens a 256-block
+// (and carries `block_loads` more) unless stage s opens one itself; fewer than three only happens
+// at the end, inside the last block.
+#define WAIT_YOUNGER(younger, opens, per_stage, block_loads)                             \
+    do {                                                                                 \
+        if ((younger) >= 3 && (opens)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (per_stage) + (block_loads)) : "memory"); \
+        else if ((younger) >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * (per_stage)) : "memory");        \
+        else if ((younger) == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (per_stage)) : "memory");        \
+        else if ((younger) == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(1 * (per_stage)) : "memory");        \
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                            \
+    } while (0)
+
+// A loader wave.  ROLE 0 moves the activation images and the group sums; ROLE q >= 1 the weight
+// runs and block headers of compute waves 4 (q - 1) .. 4 (q - 1) + 3.  Every workgroup barrier
+// here pairs with one of gemm_compute.
+template <int ROLE>
+__device__ __forceinline__ void gemm_loader(unsigned char *ring, const uint32_t *src_row, const GemmTarget &g) {
+    const int lane = pf_lane(), stages = 4 * g.kblocks;
+    const uint32_t a_pitch = (uint32_t)pf_half_row(g.a_cols);
+    // activation images: instruction i carries rows 8i..8i+7, lane = 8 * chunk + row (rows beyond
+    // the tile's last are the matrix's all-zero row)
+    uint32_t a_off[4] = {0, 0, 0, 0}, s_off = 0;
+    if (ROLE == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) a_off[i] = src_row[8 * i + (lane & 7)] * a_pitch + 8u * (uint32_t)(lane >> 3);
+        s_off = src_row[lane & 31] * a_pitch + 2u * (uint32_t)g.a_cols + 8u * (uint32_t)(lane >> 5);
+    }
+    // weight runs: lane = 32 * half + row; headers: lane = 32 * (tile of the wave's pair) + row.
+    // Tile order: a 32-row tile's 256-block is 4608 consecutive bytes, the 32 headers, then per run
+    // the 1 KB image exactly as it lands in LDS; row order: 144-byte blocks at the row pitch.
+    const uint32_t w_off = g.tiled ? 16u * (uint32_t)lane : (uint32_t)(lane & 31) * g.row_bytes + 16u * (uint32_t)(lane >> 5);
+    const uint32_t h_off = g.tiled ? 16u * (uint32_t)(lane & 31) : (uint32_t)(lane & 31) * g.row_bytes;
+    const uint32_t block_step = g.tiled ? 4608u : 144u, run0 = g.tiled ? 512u : 16u, run_step = g.tiled ? 1024u : 32u;
+    const size_t wave_bytes = (size_t)g.wave_rows * g.row_bytes;
+    auto issue = [&](int s, int slot_index) {
+        const int kb = s >> 2, j = s & 3;
+        unsigned char *slot = ring + slot_index * SLOT_BYTES;
+        if (ROLE == 0) {
+            const half_t *ap = g.a16 + 256u * (uint32_t)kb + 64u * (uint32_t)j;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                to_lds(ap + a_off[i], slot + i * A_GROUP);
+                to_lds(ap + g.a_cols + a_off[i], slot + A_PART + i * A_GROUP);
+            }
+            if (j == 0) to_lds(g.a16 + s_off + 16u * (uint32_t)kb, ring + SUMS_OFF + (kb & 1) * BLOCK_BYTES);
+        } else {
+            const uint32_t run = block_step * (uint32_t)kb + run0 + run_step * (uint32_t)j;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int v = 4 * (ROLE - 1) + q;
+                const size_t at = (size_t)min(v, g.waves - 1) * wave_bytes;   // a wave without rows repeats the last one's
+                to_lds(g.w0 + at + run + w_off, slot + SLOT_W + (2 * v) * 1024);
+                to_lds(g.w1 + at + run + w_off, slot + SLOT_W + (2 * v + 1) * 1024);
+            }
+            if (j == 0) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int v = 4 * (ROLE - 1) + q;
+                    const size_t at = (size_t)min(v, g.waves - 1) * wave_bytes;
+                    to_lds(((lane >> 5) ? g.w1 : g.w0) + at + block_step * (uint32_t)kb + h_off, ring + HDR_OFF + (kb & 1) * BLOCK_BYTES + v * 1024);
+                }
+            }
+        }
+    };
+    // Before the barrier of stage s its loads have landed (loads complete in order).  After it,
+    // the slot of stage s - 1 is free for stage s + RING_SLOTS - 1.  A stage that opens a block also
+    // brings its headers and sums, into the copy that the block before the previous one used.
+    int slot_index = 0;
+    for (int s = 0; s < min(RING_SLOTS - 1, stages); s++) {
+        issue(s, slot_index);
+        slot_index = slot_index + 1 == RING_SLOTS ? 0 : slot_index + 1;
+    }
+    for (int s = 0; s < stages; s++) {
+        const int younger = min(stages - 1 - s, RING_SLOTS - 2);
+        const bool opens = (s & 3) != 0;   // one of stages s + 1 .. s + 3 opens a block
+        if (ROLE == 0) WAIT_YOUNGER(younger, opens, 8, 1);
+        else WAIT_YOUNGER(younger, opens, 8, 4);
+        stage_barrier();
+        if (s + RING_SLOTS - 1 < stages) {
+            issue(s + RING_SLOTS - 1, slot_index);
+            slot_index = slot_index + 1 == RING_SLOTS ? 0 : slot_index + 1;
+        }
+    }
+}
+
+// 6-bit scale and minimum of group 2 jj + h (h per lane) from the 12 packed bytes of a block
+// header (src/qwen4_packed.c:88-91)
+__device__ __forceinline__ void q4_scale_min(const uint4 &hdr, int jj, int h, uint32_t &sc, uint32_t &mn) {
+    const int sh = 16 * (jj & 1) + 8 * h;
+    if (jj < 2) {
+        sc = (hdr.y >> sh) & 63u;
+        mn = (hdr.z >> sh) & 63u;
     } else {
-        const uint32_t hi = (w[2] >> sh) & 255u, lo_s = (w[0] >> sh) & 255u, lo_m = (w[1] >> sh) & 255u;
+        const uint32_t hi = (hdr.w >> sh) & 255u, lo_s = (hdr.y >> sh) & 255u, lo_m = (hdr.z >> sh) & 255u;
         sc = (hi & 15u) | ((lo_s & 192u) >> 2);
         mn = (hi >> 4) | ((lo_m & 192u) >> 2);
     }
 }
 
-// eight codes (two dwords of nibbles, nibble position nib) times the group's scale, exact in fp16:
-// a nibble under the exponent byte 0x64 reads as 1024 + q, and (1024 + q) * s - 1024 * s = q * s
-// (the high nibbles stay in place: 1024 + 16 q against s / 16 and 64 s, both exact for a 6-bit s;
-// the caller passes the pair of constants that belongs to the nibble position)
-__device__ __forceinline__ half8v q4_scaled_codes(uint32_t w0, uint32_t w1, int nib, half2v s2, half2v c1024) {
-    const uint32_t mask = nib ? 0xF0F0F0F0u : 0x0F0F0F0Fu;
+// eight codes (the nibbles under mask in two dwords) times the group's scale, exact in fp16: a
+// nibble under the exponent byte 0x64 reads as 1024 + q (low nibble) or 1024 + 16 q (high nibble,
+// left in place), and (1024 + q) * s - 1024 * s = q * s, (1024 + 16 q) * (s / 16) - 64 s = q * s;
+// s2 and c are the pair of constants that belongs to the lane's nibble position
+__device__ __forceinline__ half8v q4_scaled_codes(uint32_t w0, uint32_t w1, uint32_t mask, half2v s2, half2v c) {
     const uint32_t q0 = w0 & mask, q1 = w1 & mask;
     const uint32_t bias = 0x64646464u;
     const half2v p0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q0, 0x04010400u));
     const half2v p1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q0, 0x04030402u));
     const half2v p2 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q1, 0x04010400u));
     const half2v p3 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, q1, 0x04030402u));
-    const half2v v0 = p0 * s2 - c1024, v1 = p1 * s2 - c1024, v2 = p2 * s2 - c1024, v3 = p3 * s2 - c1024;
+    const half2v v0 = p0 * s2 - c, v1 = p1 * s2 - c, v2 = p2 * s2 - c, v3 = p3 * s2 - c;
     return half8v{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
 }
 
-// One pass: MT row tiles of 32 rows against this wave's two 32-row weight tiles, all K.
-// Lane (n = lane % 32, h = lane / 32) owns weight row n of its tiles and, per 64 weights, the
-// 16 bytes [16h, 16h + 16) of the 32-byte nibble run: chunk c = 2h + c2 (c2 = 0, 1) of nibble
-// position nib is k = 64j + 32 nib + 8c + 0..7, one MFMA per (c2, nib) and activation part.
-//
-// The activation tile of a 256-block travels from global memory straight into LDS (16 bytes per
-// lane, 64 consecutive chunks per wave instruction), one block ahead of the products, into the
-// other of two buffers.  Chunk p of a buffer: [0, 1056) high parts, row p / 33, column chunk
-// p % 33 (the 33rd is padding); [1056, 2112) low parts likewise; [2112, 2208) group sums, row
-// q / 3, chunk q % 3 (the third is padding); the rest, the padding and the rows beyond the
-// tile's last read the matrix's all-zero row (index zero_row).
-#define TILE_LOADS 35                      // wave instructions per tile
-#define TILE_HALFS (TILE_LOADS * 64 * 8)   // 35 840 bytes
-#define TILE_LOW (1056 * 8)                // half offsets of the low parts and of the sums in a buffer
-#define TILE_SUMS (2112 * 8)
-
-__device__ __forceinline__ uint32_t tile_source(int p, const uint32_t *src_row, uint32_t a_pitch, int a_cols,
-                                                uint32_t zero_row) {
-    int m, c, base;
-    if (p < 2112) {
-        const int q = p < 1056 ? p : p - 1056;
-        m = q / 33; c = q % 33;
-        base = p < 1056 ? 0 : a_cols;
-        if (c == 32) m = 32;
-    } else {
-        const int q = p - 2112;
-        m = q / 3; c = q % 3;
-        base = 2 * a_cols;
-        if (c == 2) m = 32;
-    }
-    const uint32_t row = m < 32 ? src_row[m] : zero_row;   // src_row holds zero_row beyond the tile's rows
-    return row * a_pitch + (uint32_t)base + (row == zero_row ? 0u : 8u * (uint32_t)c);
-}
-
-template <int MT>
-__device__ __forceinline__ void gemm_pass(half_t *tiles, const uint32_t *src_row, const half_t *a16, int a_cols,
-                                          uint32_t zero_row, const uint8_t *wrow0, const uint8_t *wrow1, int kblocks,
-                                          float16v (&acc)[2][MT]) {
-    static_assert(MT == 1, "one 32-row tile per pass");
+// A compute wave: all K against its two weight tiles.  A 256-block's result is
+// d * P - dmin * Q with P = sum (scale * code) x and Q = sum_g min_g * (sum of x over group g).
+__device__ __forceinline__ void gemm_compute(const unsigned char *ring, int kblocks, float16v &acc0, float16v &acc1) {
     const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
-    const uint32_t a_pitch = (uint32_t)pf_half_row(a_cols);
-    // this wave's loads of a tile: instruction i = wave + 4 ii covers chunks [64 i, 64 i + 64)
-    uint32_t source[9];
+    const uint32_t mask = h ? 0xF0F0F0F0u : 0x0F0F0F0Fu;
+    const half_t unit = h ? (half_t)0.0625f : (half_t)1.0f;
+    const int bias_shift = h ? 6 : 10;
+    const unsigned char *a_lane = ring + (n >> 3) * A_GROUP + (4 * h) * 128 + (n & 7) * 16;
+    const unsigned char *w_lane = ring + SLOT_W + (2 * wave) * 1024 + n * 16;
+    const float16v zero = {0};
+    int slot_off = 0;
+    for (int kb = 0; kb < kblocks; kb++) {
+        float16v part0 = zero, part1 = zero, q0 = zero, q1 = zero;
+        float d0 = 0.0f, m0 = 0.0f, d1 = 0.0f, m1 = 0.0f;
+        half2v s2[2][4], c2[2][4];
 #pragma unroll
-    for (int ii = 0; ii < 9; ii++) source[ii] = tile_source(64 * (wave + 4 * ii) + lane, src_row, a_pitch, a_cols, zero_row);
-    auto issue_tile = [&](int kb, half_t *buffer) {
+        for (int j = 0; j < 4; j++) {
+            stage_barrier();
+            const unsigned char *slot_a = a_lane + slot_off, *slot_w = w_lane + slot_off;
+            slot_off = slot_off + SLOT_BYTES == RING_SLOTS * SLOT_BYTES ? 0 : slot_off + SLOT_BYTES;
+            // every LDS operand of the stage is requested up front (they return in order: the first
+            // product waits for the weight runs and one fragment pair, the rest arrive under way)
+            const uint4 wa0 = *reinterpret_cast<const uint4 *>(slot_w), wb0 = *reinterpret_cast<const uint4 *>(slot_w + 512);
+            const uint4 wa1 = *reinterpret_cast<const uint4 *>(slot_w + 1024), wb1 = *reinterpret_cast<const uint4 *>(slot_w + 1536);
+            half8v ah[4], al[4];
 #pragma unroll
-        for (int ii = 0; ii < 9; ii++) {
-            const int i = wave + 4 * ii;
-            if (i >= TILE_LOADS) break;
-            const uint32_t step = 64 * i < 2112 ? 256u : 16u;   // halfs per 256-block in this region (uniform per load)
-            __builtin_amdgcn_global_load_lds(a16 + source[ii] + step * (uint32_t)kb, buffer + 512 * i, 16, 0, 0);
-        }
-    };
-    // One 256-block: wait for its bytes, start the next block's, multiply.  The weight bytes
-    // alternate between two register sets (cur / next) from block to block.
-    auto block_step = [&](int kb, const Q4Raw &cur0, const Q4Raw &cur1, Q4Raw &next0, Q4Raw &next1) {
-        half_t *tile_h = tiles + (kb & 1) * TILE_HALFS, *tile_l = tile_h + TILE_LOW, *tile_s = tile_h + TILE_SUMS;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's part of the tile and its weight bytes have arrived
-        __syncthreads();                                    // every wave's part; and the other buffer has been consumed
-        if (kb + 1 < kblocks) {   // next block's bytes travel while this one is multiplied
-            issue_tile(kb + 1, tiles + ((kb + 1) & 1) * TILE_HALFS);
-            q4_load(next0, wrow0 + 144 * (kb + 1), h);
-            q4_load(next1, wrow1 + 144 * (kb + 1), h);
-        }
-        const half_t *row_h = tile_h + n * A_PITCH + 16 * h, *row_l = tile_l + n * A_PITCH + 16 * h;
-        // first activation fragments, requested before the scale arithmetic
-        half8v ah = *reinterpret_cast<const half8v *>(row_h), al = *reinterpret_cast<const half8v *>(row_l);
-        const half8v as = *reinterpret_cast<const half8v *>(tile_s + n * S_PITCH + 8 * h);
-        // the hardware conversion is exact for every binary16 value, subnormals included
-        const half2v dm0 = __builtin_bit_cast(half2v, cur0.hdr.x), dm1 = __builtin_bit_cast(half2v, cur1.hdr.x);
-        const float d0 = (float)dm0.x, m0 = (float)dm0.y, d1 = (float)dm1.x, m1 = (float)dm1.y;
-        half8v min0, min1;
-        half2v s2[2][8], c2k[2][8];
-#pragma unroll
-        for (int g = 0; g < 8; g++) {
-            // even groups sit in the low nibbles (1024 + q, times s, minus 1024 s), odd groups in
-            // the high ones (1024 + 16 q, times s / 16, minus 64 s)
-            const half_t unit = (g & 1) ? (half_t)0.0625f : (half_t)1.0f;
-            const int bias_shift = (g & 1) ? 6 : 10;
-            uint32_t sc, mn;
-            q4_scale_min(cur0, g, sc, mn);
-            min0[g] = (half_t)(int)mn;
-            const half_t s0 = (half_t)(int)sc * unit;
-            s2[0][g] = half2v{s0, s0};
-            c2k[0][g] = half2v{(half_t)(int)(sc << bias_shift), (half_t)(int)(sc << bias_shift)};
-            q4_scale_min(cur1, g, sc, mn);
-            min1[g] = (half_t)(int)mn;
-            const half_t s1 = (half_t)(int)sc * unit;
-            s2[1][g] = half2v{s1, s1};
-            c2k[1][g] = half2v{(half_t)(int)(sc << bias_shift), (half_t)(int)(sc << bias_shift)};
-        }
-        // Q: the eight minima against the eight group sums (high parts in k 0..7, low parts in k 8..15)
-        const float16v zero = {0};
-        const float16v q0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min0, zero, 0, 0, 0);
-        const float16v q1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, min1, zero, 0, 0, 0);
-        // P: scale * code against both activation parts; step s = (j, nib, c2) covers
-        // k = 64 j + 32 nib + 16 h + 8 c2 + 0..7, and its fragments are requested one step ahead
-        float16v part0 = zero, part1 = zero;
-#pragma unroll
-        for (int s = 0; s < 16; s++) {
-            const int j = s >> 2, nib = (s >> 1) & 1, c2 = s & 1, g = 2 * j + nib;
-            half8v nh = ah, nl = al;
-            if (s < 15) {
-                const int sn = s + 1, kn = 64 * (sn >> 2) + 32 * ((sn >> 1) & 1) + 8 * (sn & 1);
-                nh = *reinterpret_cast<const half8v *>(row_h + kn);
-                nl = *reinterpret_cast<const half8v *>(row_l + kn);
+            for (int t = 0; t < 4; t++) {
+                ah[t] = *reinterpret_cast<const half8v *>(slot_a + 128 * t);
+                al[t] = *reinterpret_cast<const half8v *>(slot_a + A_PART + 128 * t);
             }
-            const uint4 w0 = cur0.q[j], w1 = cur1.q[j];
-            const half8v b0 = q4_scaled_codes(c2 ? w0.z : w0.x, c2 ? w0.w : w0.y, nib, s2[0][g], c2k[0][g]);
-            const half8v b1 = q4_scaled_codes(c2 ? w1.z : w1.x, c2 ? w1.w : w1.y, nib, s2[1][g], c2k[1][g]);
-            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b0, part0, 0, 0, 0);
-            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, b1, part1, 0, 0, 0);
-            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b0, part0, 0, 0, 0);
-            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, b1, part1, 0, 0, 0);
-            ah = nh;
-            al = nl;
+            if (j == 0) {
+                const unsigned char *block = ring + (kb & 1) * BLOCK_BYTES;
+                const uint4 hdr0 = *reinterpret_cast<const uint4 *>(block + HDR_OFF + (2 * wave) * 512 + n * 16);
+                const uint4 hdr1 = *reinterpret_cast<const uint4 *>(block + HDR_OFF + (2 * wave + 1) * 512 + n * 16);
+                const half8v as = *reinterpret_cast<const half8v *>(block + SUMS_OFF + lane * 16);
+                asm volatile("" ::: "memory");   // the requests stay above the arithmetic
+                // the hardware conversion is exact for every binary16 value, subnormals included
+                const half2v dm0 = __builtin_bit_cast(half2v, hdr0.x), dm1 = __builtin_bit_cast(half2v, hdr1.x);
+                d0 = (float)dm0.x; m0 = (float)dm0.y; d1 = (float)dm1.x; m1 = (float)dm1.y;
+                half_t min0[4], min1[4];
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    uint32_t sc, mn;
+                    q4_scale_min(hdr0, jj, h, sc, mn);
+                    min0[jj] = (half_t)(int)mn;
+                    const half_t s0 = (half_t)(int)sc * unit, k0 = (half_t)(int)(sc << bias_shift);
+                    s2[0][jj] = half2v{s0, s0};
+                    c2[0][jj] = half2v{k0, k0};
+                    q4_scale_min(hdr1, jj, h, sc, mn);
+                    min1[jj] = (half_t)(int)mn;
+                    const half_t s1 = (half_t)(int)sc * unit, k1 = (half_t)(int)(sc << bias_shift);
+                    s2[1][jj] = half2v{s1, s1};
+                    c2[1][jj] = half2v{k1, k1};
+                }
+                // Q: K slots 8h..8h+3 hold the high parts of the sums of the lane's four groups,
+                // 8h+4..8h+7 the low parts; the four minima appear once against each
+                const half8v mv0 = {min0[0], min0[1], min0[2], min0[3], min0[0], min0[1], min0[2], min0[3]};
+                const half8v mv1 = {min1[0], min1[1], min1[2], min1[3], min1[0], min1[1], min1[2], min1[3]};
+                q0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, mv0, zero, 0, 0, 0);
+                q1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(as, mv1, zero, 0, 0, 0);
+            }
+            asm volatile("" ::: "memory");
+            const uint32_t w0[8] = {wa0.x, wa0.y, wa0.z, wa0.w, wb0.x, wb0.y, wb0.z, wb0.w};
+            const uint32_t w1[8] = {wa1.x, wa1.y, wa1.z, wa1.w, wb1.x, wb1.y, wb1.z, wb1.w};
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const half8v b0 = q4_scaled_codes(w0[2 * t], w0[2 * t + 1], mask, s2[0][j], c2[0][j]);
+                const half8v b1 = q4_scaled_codes(w1[2 * t], w1[2 * t + 1], mask, s2[1][j], c2[1][j]);
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[t], b0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[t], b1, part1, 0, 0, 0);
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[t], b0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[t], b1, part1, 0, 0, 0);
+            }
+            if (j == 0) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    acc0[r] = fmaf(-m0, q0[r], acc0[r]);
+                    acc1[r] = fmaf(-m1, q1[r], acc1[r]);
+                }
+            }
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            acc[0][0][r] = fmaf(d0, part0[r], fmaf(-m0, q0[r], acc[0][0][r]));
-            acc[1][0][r] = fmaf(d1, part1[r], fmaf(-m1, q1[r], acc[1][0][r]));
-        }
-    };
-    Q4Raw a0, a1, b0, b1;
-    q4_load(a0, wrow0, h);
-    q4_load(a1, wrow1, h);
-    issue_tile(0, tiles);
-    for (int kb = 0; kb < kblocks; kb += 2) {
-        block_step(kb, a0, a1, b0, b1);
-        if (kb + 1 < kblocks) block_step(kb + 1, b0, b1, a0, a1);
-    }
-}
-
-struct GemmTarget {   // what one workgroup of the grouped product works on
-    bool shared;
-    int first, count, inter, kblocks, a_cols, slab;
-    uint32_t zero_row;   // index of the all-zero row that ends the fp16 form of the activation matrix
-    const uint8_t *w0, *w1;
-    const half_t *a16;
-    const float *a_scale;
-};
-
-template <int MODE, int MT>
-__device__ __forceinline__ void gemm_rows(const PfKernelArgs &a, const GemmTarget &g, int m0, int rows_here, half_t *tiles,
-                                          uint32_t *src_row, float *row_scale) {
-    const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5, K = a.top_k;
-    for (int m = threadIdx.x; m < 32 * MT; m += 256) {
-        uint32_t src = g.zero_row;
-        float sc = 0.0f;
-        if (m < rows_here) {
-            if (MODE == PF_GEMM_GATE_UP) src = g.shared ? (uint32_t)(m0 + m) : a.row_to_pair[g.first + m0 + m] / (uint32_t)K;
-            else src = g.shared ? (uint32_t)(m0 + m) : (uint32_t)(g.first + m0 + m);
-            sc = g.a_scale[src];
-        }
-        src_row[m] = src;
-        row_scale[m] = sc;
-    }
-    float16v acc[2][MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) { acc[0][mt] = float16v{0}; acc[1][mt] = float16v{0}; }
-    __syncthreads();   // src_row is read by every wave's tile loads
-    gemm_pass<MT>(tiles, src_row, g.a16, g.a_cols, g.zero_row, g.w0, g.w1, g.kblocks, acc);
-    // epilogue: the lane holds column n of its two tiles; register r of tile mt is row
-    // 32 mt + 8 (r / 4) + 4 h + r % 4
-#pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int m = 32 * mt + 8 * (r >> 2) + 4 * h + (r & 3);
-            if (m >= rows_here) continue;
-            const float rs = row_scale[m];
-            if (MODE == PF_GEMM_GATE_UP) {
-                const int unit = 128 * g.slab + 32 * wave + n;
-                if (unit >= g.inter) continue;
-                const float gate = acc[0][mt][r] * rs, up = acc[1][mt][r] * rs;
-                const float v = pf_silu(gate) * up;
-                if (g.shared) a.shared_act[(size_t)(m0 + m) * g.inter + unit] = v;
-                else a.act[(size_t)(g.first + m0 + m) * g.inter + unit] = v;
-            } else {
-                const int r0 = 256 * g.slab + 64 * wave + n;
-                float *out = a.down + (size_t)(g.first + m0 + m) * a.hidden;
-                if (r0 < a.hidden) out[r0] = acc[0][mt][r] * rs;
-                if (r0 + 32 < a.hidden) out[r0 + 32] = acc[1][mt][r] * rs;
-            }
+            acc0[r] = fmaf(d0, part0[r], acc0[r]);
+            acc1[r] = fmaf(d1, part1[r], acc1[r]);
         }
     }
 }
@@ -431,15 +494,13 @@ __global__ void __launch_bounds__(256) pf_k_pf_scan_tiles(uint32_t *counts, int 
     }
 }
 
-// Workgroup (row tile, slab): 4 waves, each with two 32-row weight tiles (gate + up of 32 units,
-// or 2 x 32 down rows) against the tile's 32 rows.
+// Workgroup (row tile, slab): see the description above gemm_loader.
 template <int MODE>
-__global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, int slabs) {
-    extern __shared__ __align__(16) unsigned char lds_raw[];
-    half_t *tiles = reinterpret_cast<half_t *>(lds_raw);   // two buffers of TILE_HALFS
+__global__ void __launch_bounds__(64 * (NW + NL), 3) pf_k_pf_gemm(PfKernelArgs a, int tokens, int slabs) {
+    extern __shared__ __align__(16) unsigned char ring[];
     __shared__ uint32_t src_row[32];
     __shared__ float row_scale[32];
-    const int E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31;
+    const int E = a.experts, K = a.top_k, lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
     // Workgroups go to the eight XCDs round robin by index.  The slabs of one row tile read the
     // same activation rows, so they are given indices eight apart: one XCD, one L2.
     const uint32_t xcd = blockIdx.x % 8, turn = blockIdx.x / 8, tile = (turn / slabs) * 8 + xcd;
@@ -449,7 +510,7 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, 
     GemmTarget g;
     g.slab = turn % slabs;
     g.shared = expert == E;
-    const int P = tokens * a.top_k;
+    const int P = tokens * K;
     g.first = g.shared ? P : (int)a.offsets[expert];
     g.count = g.shared ? tokens : (int)a.offsets[expert + 1] - g.first;
     if (g.count <= m0) return;
@@ -457,23 +518,71 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm(PfKernelArgs a, int tokens, 
     const size_t ex = g.shared ? 0 : (size_t)expert;
     if (MODE == PF_GEMM_GATE_UP) {
         const int tg = g.shared ? 4 : 1;
-        if (128 * g.slab >= g.inter) return;
-        const int u = min(128 * g.slab + 32 * wave + n, g.inter - 1);
-        g.w0 = a.w[tg] + ex * a.expert_bytes[tg] + (size_t)u * a.row_bytes[tg];
-        g.w1 = a.w[tg + 1] + ex * a.expert_bytes[tg + 1] + (size_t)u * a.row_bytes[tg + 1];
+        if (32 * NW * g.slab >= g.inter) return;
+        g.row_bytes = (uint32_t)a.row_bytes[tg];
+        g.tiled = a.wt[tg] != nullptr;
+        g.w0 = (g.tiled ? a.wt[tg] : a.w[tg]) + ex * a.expert_bytes[tg] + (size_t)(32 * NW * g.slab) * g.row_bytes;
+        g.w1 = (g.tiled ? a.wt[tg + 1] : a.w[tg + 1]) + ex * a.expert_bytes[tg + 1] + (size_t)(32 * NW * g.slab) * g.row_bytes;
+        g.wave_rows = 32;
+        g.waves = min(NW, (g.inter - 32 * NW * g.slab) / 32);
         g.kblocks = a.hidden / 256; g.a_cols = a.hidden;
         g.a16 = reinterpret_cast<const half_t *>(a.x16); g.a_scale = a.x_scale;
         g.zero_row = a.token_cap;
     } else {
-        const int td = g.shared ? 6 : 3, r0 = 256 * g.slab + 64 * wave + n;
-        g.w0 = a.w[td] + ex * a.expert_bytes[td] + (size_t)min(r0, a.hidden - 1) * a.row_bytes[td];
-        g.w1 = a.w[td] + ex * a.expert_bytes[td] + (size_t)min(r0 + 32, a.hidden - 1) * a.row_bytes[td];
+        const int td = g.shared ? 6 : 3;
+        if (64 * NW * g.slab >= a.hidden) return;
+        g.row_bytes = (uint32_t)a.row_bytes[td];
+        g.tiled = a.wt[td] != nullptr;
+        g.w0 = (g.tiled ? a.wt[td] : a.w[td]) + ex * a.expert_bytes[td] + (size_t)(64 * NW * g.slab) * g.row_bytes;
+        g.w1 = g.w0 + (size_t)32 * g.row_bytes;
+        g.wave_rows = 64;
+        g.waves = min(NW, (a.hidden - 64 * NW * g.slab) / 64);
         g.kblocks = g.inter / 256; g.a_cols = g.inter;
         g.a16 = reinterpret_cast<const half_t *>(g.shared ? a.sact16 : a.act16);
         g.a_scale = g.shared ? a.sact_scale : a.act_scale;
-        g.zero_row = g.shared ? a.token_cap : a.token_cap * (uint32_t)a.top_k;
+        g.zero_row = g.shared ? a.token_cap : a.token_cap * (uint32_t)K;
     }
-    gemm_rows<MODE, 1>(a, g, m0, min(32, g.count - m0), tiles, src_row, row_scale);
+    const int rows_here = min(32, g.count - m0);
+    if (threadIdx.x < 32) {
+        const int m = threadIdx.x;
+        uint32_t src = g.zero_row;
+        float sc = 0.0f;
+        if (m < rows_here) {
+            if (MODE == PF_GEMM_GATE_UP) src = g.shared ? (uint32_t)(m0 + m) : a.row_to_pair[g.first + m0 + m] / (uint32_t)K;
+            else src = g.shared ? (uint32_t)(m0 + m) : (uint32_t)(g.first + m0 + m);
+            sc = g.a_scale[src];
+        }
+        src_row[m] = src;
+        row_scale[m] = sc;
+    }
+    __syncthreads();
+    if (wave >= NW) {
+        if (wave == NW) gemm_loader<0>(ring, src_row, g);
+        else if (wave == NW + 1) gemm_loader<1>(ring, src_row, g);
+        else gemm_loader<2>(ring, src_row, g);
+        return;
+    }
+    float16v acc0 = {0}, acc1 = {0};
+    gemm_compute(ring, g.kblocks, acc0, acc1);
+    // epilogue: the lane holds column n of its two tiles; register r is row 8 (r / 4) + 4 h + r % 4
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int m = 8 * (r >> 2) + 4 * h + (r & 3);
+        if (m >= rows_here || wave >= g.waves) continue;
+        const float rs = row_scale[m];
+        if (MODE == PF_GEMM_GATE_UP) {
+            const int unit = 32 * NW * g.slab + 32 * wave + n;
+            const float gate = acc0[r] * rs, up = acc1[r] * rs;
+            const float v = pf_silu(gate) * up;
+            if (g.shared) a.shared_act[(size_t)(m0 + m) * g.inter + unit] = v;
+            else a.act[(size_t)(g.first + m0 + m) * g.inter + unit] = v;
+        } else {
+            const int r0 = 64 * NW * g.slab + 64 * wave + n;
+            float *out = a.down + (size_t)(g.first + m0 + m) * a.hidden;
+            out[r0] = acc0[r] * rs;
+            out[r0 + 32] = acc1[r] * rs;
+        }
+    }
 }
 
 // ---- combine ---------------------------------------------------------------------------------------
@@ -520,7 +629,7 @@ int pf_prefill_max_tiles(int tokens, int experts, int top_k) {
 
 template <int MODE>
 static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_t stream) {
-    const size_t lds = 2 * (size_t)TILE_HALFS * sizeof(half_t);
+    const size_t lds = GEMM_LDS;
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_pf_gemm<MODE>),
@@ -529,7 +638,7 @@ static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_
     }
     // the tile count is only known on the device: launch its upper bound, surplus workgroups exit at once
     const int max_tiles = pf_prefill_max_tiles(tokens, a.experts, a.top_k);
-    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3((max_tiles + 7) / 8 * 8 * slabs), dim3(256), lds, stream, a, tokens, slabs);
+    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3((max_tiles + 7) / 8 * 8 * slabs), dim3(64 * (NW + NL)), lds, stream, a, tokens, slabs);
 }
 
 void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
@@ -548,13 +657,13 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     if (last < 3) return;
     // stage 3: gate/up + SwiGLU, then fp16 parts of the activation rows
     const int gi = I > Is ? I : Is;
-    launch_gemm<PF_GEMM_GATE_UP>(a, tokens, (gi + 127) / 128, stream);
+    launch_gemm<PF_GEMM_GATE_UP>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(P), dim3(256), 0, stream, a.act, (size_t)I, I, (half_t *)a.act16, a.act_scale,
                        (float *)nullptr, a.error_word);
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.shared_act, (size_t)Is, Is,
                        (half_t *)a.sact16, a.sact_scale, (float *)nullptr, a.error_word);
     if (last < 4) return;
     // stage 4: down and combine
-    launch_gemm<PF_GEMM_DOWN>(a, tokens, (H + 255) / 256, stream);
+    launch_gemm<PF_GEMM_DOWN>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
     hipLaunchKernelGGL(pf_k_pf_combine, dim3(tokens), dim3(256), 0, stream, a, tokens);
 }
