@@ -228,9 +228,10 @@ __device__ __forceinline__ void stage_barrier() {
     asm volatile("" ::: "memory");
 }
 
-struct GemmTarget {   // what one workgroup of the grouped product works on
+struct GemmTarget {   // one work item of the grouped product: a 32-row tile of an expert against one slab of weight rows
     bool shared;
     int first, count, inter, kblocks, a_cols, slab;
+    int m0, rows_here;    // first row of the tile within the expert's rows, rows in it
     int waves;            // compute waves whose weight rows exist (the last slab of a narrow matrix has fewer)
     uint32_t zero_row;    // index of the all-zero row that ends the fp16 form of the activation matrix
     uint32_t row_bytes;   // of the weight tensor(s)
@@ -240,6 +241,65 @@ struct GemmTarget {   // what one workgroup of the grouped product works on
     const half_t *a16;
     const float *a_scale;
 };
+
+// Work item q -> (row tile, slab).  Workgroups go to the eight XCDs round robin by index and a
+// workgroup's items are a multiple of eight apart, so the slabs of one row tile, which read the
+// same activation rows, are given item numbers eight apart: one XCD, one L2.  False: nothing to do
+// for q.  Every wave of the workgroup evaluates this for itself, with the same result.
+template <int MODE>
+__device__ __forceinline__ bool gemm_item(const PfKernelArgs &a, int tokens, int slabs, uint32_t q, GemmTarget &g) {
+    const int E = a.experts, K = a.top_k;
+    const uint32_t xcd = q % 8, turn = q / 8, tile = (turn / slabs) * 8 + xcd;
+    if (tile >= a.tiles[0]) return false;
+    const uint32_t entry = a.tiles[1 + tile];
+    const int expert = entry & 0xffffu;
+    g.m0 = 32 * (int)(entry >> 16);
+    g.slab = turn % slabs;
+    g.shared = expert == E;
+    const int P = tokens * K;
+    g.first = g.shared ? P : (int)a.offsets[expert];
+    g.count = g.shared ? tokens : (int)a.offsets[expert + 1] - g.first;
+    if (g.count <= g.m0) return false;
+    g.rows_here = min(32, g.count - g.m0);
+    g.inter = g.shared ? a.shared_inter : a.inter;
+    const size_t ex = g.shared ? 0 : (size_t)expert;
+    if (MODE == PF_GEMM_GATE_UP) {
+        const int tg = g.shared ? 4 : 1;
+        if (32 * NW * g.slab >= g.inter) return false;
+        g.row_bytes = (uint32_t)a.row_bytes[tg];
+        g.tiled = a.wt[tg] != nullptr;
+        g.w0 = (g.tiled ? a.wt[tg] : a.w[tg]) + ex * a.expert_bytes[tg] + (size_t)(32 * NW * g.slab) * g.row_bytes;
+        g.w1 = (g.tiled ? a.wt[tg + 1] : a.w[tg + 1]) + ex * a.expert_bytes[tg + 1] + (size_t)(32 * NW * g.slab) * g.row_bytes;
+        g.wave_rows = 32;
+        g.waves = min(NW, (g.inter - 32 * NW * g.slab) / 32);
+        g.kblocks = a.hidden / 256; g.a_cols = a.hidden;
+        g.a16 = reinterpret_cast<const half_t *>(a.x16); g.a_scale = a.x_scale;
+        g.zero_row = a.token_cap;
+    } else {
+        const int td = g.shared ? 6 : 3;
+        if (64 * NW * g.slab >= a.hidden) return false;
+        g.row_bytes = (uint32_t)a.row_bytes[td];
+        g.tiled = a.wt[td] != nullptr;
+        g.w0 = (g.tiled ? a.wt[td] : a.w[td]) + ex * a.expert_bytes[td] + (size_t)(64 * NW * g.slab) * g.row_bytes;
+        g.w1 = g.w0 + (size_t)32 * g.row_bytes;
+        g.wave_rows = 64;
+        g.waves = min(NW, (a.hidden - 64 * NW * g.slab) / 64);
+        g.kblocks = g.inter / 256; g.a_cols = g.inter;
+        g.a16 = reinterpret_cast<const half_t *>(g.shared ? a.sact16 : a.act16);
+        g.a_scale = g.shared ? a.sact_scale : a.act_scale;
+        g.zero_row = g.shared ? a.token_cap : a.token_cap * (uint32_t)K;
+    }
+    return true;
+}
+
+// first item at or after q (stepping by the grid size) that has work; false when the list is exhausted
+template <int MODE>
+__device__ __forceinline__ bool gemm_next_item(const PfKernelArgs &a, int tokens, int slabs, uint32_t items, uint32_t &q,
+                                               GemmTarget &g) {
+    for (; q < items; q += gridDim.x)
+        if (gemm_item<MODE>(a, tokens, slabs, q, g)) return true;
+    return false;
+}
 
 // Loads of the stages that may still be on their way when stage s is handed over: the younger
 // stages issued so far, at most three.  Three consecutive stages hold one that opens a 256-block
@@ -254,76 +314,113 @@ struct GemmTarget {   // what one workgroup of the grouped product works on
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                            \
     } while (0)
 
-// A loader wave.  ROLE 0 moves the activation images and the group sums; ROLE q >= 1 the weight
-// runs and block headers of compute waves 4 (q - 1) .. 4 (q - 1) + 3.  Every workgroup barrier
-// here pairs with one of gemm_compute.
-template <int ROLE>
-__device__ __forceinline__ void gemm_loader(unsigned char *ring, const uint32_t *src_row, const GemmTarget &g) {
-    const int lane = pf_lane(), stages = 4 * g.kblocks;
-    const uint32_t a_pitch = (uint32_t)pf_half_row(g.a_cols);
-    // activation images: instruction i carries rows 8i..8i+7, lane = 8 * chunk + row (rows beyond
-    // the tile's last are the matrix's all-zero row)
-    uint32_t a_off[4] = {0, 0, 0, 0}, s_off = 0;
-    if (ROLE == 0) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) a_off[i] = src_row[8 * i + (lane & 7)] * a_pitch + 8u * (uint32_t)(lane >> 3);
-        s_off = src_row[lane & 31] * a_pitch + 2u * (uint32_t)g.a_cols + 8u * (uint32_t)(lane >> 5);
-    }
-    // weight runs: lane = 32 * half + row; headers: lane = 32 * (tile of the wave's pair) + row.
-    // Tile order: a 32-row tile's 256-block is 4608 consecutive bytes, the 32 headers, then per run
-    // the 1 KB image exactly as it lands in LDS; row order: 144-byte blocks at the row pitch.
-    const uint32_t w_off = g.tiled ? 16u * (uint32_t)lane : (uint32_t)(lane & 31) * g.row_bytes + 16u * (uint32_t)(lane >> 5);
-    const uint32_t h_off = g.tiled ? 16u * (uint32_t)(lane & 31) : (uint32_t)(lane & 31) * g.row_bytes;
-    const uint32_t block_step = g.tiled ? 4608u : 144u, run0 = g.tiled ? 512u : 16u, run_step = g.tiled ? 1024u : 32u;
-    const size_t wave_bytes = (size_t)g.wave_rows * g.row_bytes;
-    auto issue = [&](int s, int slot_index) {
-        const int kb = s >> 2, j = s & 3;
-        unsigned char *slot = ring + slot_index * SLOT_BYTES;
+// A loader wave.  ROLE 0 moves the activation images and the group sums (and leaves the rows'
+// scales for the epilogue); ROLE q >= 1 the weight runs and block headers of compute waves
+// 4 (q - 1) .. 4 (q - 1) + 3.  It walks the workgroup's items as one stream of stages, up to
+// RING_SLOTS - 1 stages ahead of the compute waves, also across item boundaries: the ring never
+// drains between items.  Every workgroup barrier here pairs with one of gemm_compute.
+template <int MODE, int ROLE>
+__device__ __forceinline__ void gemm_loader(const PfKernelArgs &a, int tokens, int slabs, uint32_t items, unsigned char *ring,
+                                            float (*row_scale)[32]) {
+    const int lane = pf_lane(), K = a.top_k;
+    GemmTarget g;
+    uint32_t q = blockIdx.x;
+    bool more = gemm_next_item<MODE>(a, tokens, slabs, items, q, g);
+    int kb = 0, j = 0, slot_index = 0, block_parity = 0, item_index = 0;
+    uint32_t a_off[4] = {0, 0, 0, 0}, a_live[4] = {0, 0, 0, 0}, s_off = 0, s_live = 0, w_off = 0, h_off = 0, block_step = 0,
+             run0 = 0, run_step = 0;
+    size_t wave_bytes = 0;
+    auto open_item = [&]() {   // per-lane source offsets of the item the issue cursor has reached
         if (ROLE == 0) {
-            const half_t *ap = g.a16 + 256u * (uint32_t)kb + 64u * (uint32_t)j;
+            // activation images: instruction i carries rows 8i..8i+7, lane = 8 * chunk + row.  The
+            // lanes of rows beyond the tile's last all read the first 16 bytes of the matrix's
+            // all-zero row, whatever the stage: one cache line serves them (a_live masks the
+            // stage's column offset away), so padding costs no memory traffic.
+            const uint32_t a_pitch = (uint32_t)pf_half_row(g.a_cols);
+            auto source_row = [&](int m) -> uint32_t {
+                if (m >= g.rows_here) return g.zero_row;
+                if (g.shared) return (uint32_t)(g.m0 + m);
+                return MODE == PF_GEMM_GATE_UP ? a.row_to_pair[g.first + g.m0 + m] / (uint32_t)K : (uint32_t)(g.first + g.m0 + m);
+            };
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                to_lds(ap + a_off[i], slot + i * A_GROUP);
-                to_lds(ap + g.a_cols + a_off[i], slot + A_PART + i * A_GROUP);
+                const int m = 8 * i + (lane & 7);
+                a_live[i] = m < g.rows_here ? 0xffffffffu : 0u;
+                a_off[i] = source_row(m) * a_pitch + (8u * (uint32_t)(lane >> 3) & a_live[i]);
             }
-            if (j == 0) to_lds(g.a16 + s_off + 16u * (uint32_t)kb, ring + SUMS_OFF + (kb & 1) * BLOCK_BYTES);
+            const uint32_t mine = source_row(lane & 31);
+            s_live = (lane & 31) < g.rows_here ? 0xffffffffu : 0u;
+            s_off = mine * a_pitch + ((2u * (uint32_t)g.a_cols + 8u * (uint32_t)(lane >> 5)) & s_live);
+            // the rows' scales for the epilogue of this item (read many barriers later; four copies
+            // in turn, because this wave may open the item after next before the epilogue of the
+            // current one is over)
+            if (lane < 32) row_scale[item_index & 3][lane] = (lane < g.rows_here) ? g.a_scale[mine] : 0.0f;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        } else {
+            // weight runs: lane = 32 * half + row; headers: lane = 32 * (tile of the wave's pair) + row.
+            // Tile order: a 32-row tile's 256-block is 4608 consecutive bytes, the 32 headers, then per
+            // run the 1 KB image exactly as it lands in LDS; row order: 144-byte blocks at the row pitch.
+            w_off = g.tiled ? 16u * (uint32_t)lane : (uint32_t)(lane & 31) * g.row_bytes + 16u * (uint32_t)(lane >> 5);
+            h_off = g.tiled ? 16u * (uint32_t)(lane & 31) : (uint32_t)(lane & 31) * g.row_bytes;
+            block_step = g.tiled ? 4608u : 144u; run0 = g.tiled ? 512u : 16u; run_step = g.tiled ? 1024u : 32u;
+            wave_bytes = (size_t)g.wave_rows * g.row_bytes;
+        }
+        item_index++;
+    };
+    auto issue = [&]() {   // the stage under the issue cursor, then advance the cursor
+        unsigned char *slot = ring + slot_index * SLOT_BYTES;
+        unsigned char *block = ring + block_parity * BLOCK_BYTES;
+        if (ROLE == 0) {
+            const uint32_t high = 256u * (uint32_t)kb + 64u * (uint32_t)j, low = high + (uint32_t)g.a_cols;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                to_lds(g.a16 + a_off[i] + (high & a_live[i]), slot + i * A_GROUP);
+                to_lds(g.a16 + a_off[i] + (low & a_live[i]), slot + A_PART + i * A_GROUP);
+            }
+            if (j == 0) to_lds(g.a16 + s_off + (16u * (uint32_t)kb & s_live), block + SUMS_OFF);
         } else {
             const uint32_t run = block_step * (uint32_t)kb + run0 + run_step * (uint32_t)j;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int v = 4 * (ROLE - 1) + q;
+            for (int c = 0; c < 4; c++) {
+                const int v = 4 * (ROLE - 1) + c;
                 const size_t at = (size_t)min(v, g.waves - 1) * wave_bytes;   // a wave without rows repeats the last one's
                 to_lds(g.w0 + at + run + w_off, slot + SLOT_W + (2 * v) * 1024);
                 to_lds(g.w1 + at + run + w_off, slot + SLOT_W + (2 * v + 1) * 1024);
             }
             if (j == 0) {
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const int v = 4 * (ROLE - 1) + q;
+                for (int c = 0; c < 4; c++) {
+                    const int v = 4 * (ROLE - 1) + c;
                     const size_t at = (size_t)min(v, g.waves - 1) * wave_bytes;
-                    to_lds(((lane >> 5) ? g.w1 : g.w0) + at + block_step * (uint32_t)kb + h_off, ring + HDR_OFF + (kb & 1) * BLOCK_BYTES + v * 1024);
+                    to_lds(((lane >> 5) ? g.w1 : g.w0) + at + block_step * (uint32_t)kb + h_off, block + HDR_OFF + v * 1024);
                 }
             }
         }
+        slot_index = slot_index + 1 == RING_SLOTS ? 0 : slot_index + 1;
+        if (++j == 4) {
+            j = 0;
+            block_parity ^= 1;
+            if (++kb == g.kblocks) {
+                kb = 0;
+                q += gridDim.x;
+                more = gemm_next_item<MODE>(a, tokens, slabs, items, q, g);
+                if (more) open_item();
+            }
+        }
     };
+    if (more) open_item();
     // Before the barrier of stage s its loads have landed (loads complete in order).  After it,
     // the slot of stage s - 1 is free for stage s + RING_SLOTS - 1.  A stage that opens a block also
     // brings its headers and sums, into the copy that the block before the previous one used.
-    int slot_index = 0;
-    for (int s = 0; s < min(RING_SLOTS - 1, stages); s++) {
-        issue(s, slot_index);
-        slot_index = slot_index + 1 == RING_SLOTS ? 0 : slot_index + 1;
-    }
-    for (int s = 0; s < stages; s++) {
-        const int younger = min(stages - 1 - s, RING_SLOTS - 2);
-        const bool opens = (s & 3) != 0;   // one of stages s + 1 .. s + 3 opens a block
+    int issued = 0;
+    while (issued < RING_SLOTS - 1 && more) { issue(); issued++; }
+    for (int s = 0; s < issued; s++) {
+        const int younger = issued - s - 1;   // at most RING_SLOTS - 2
+        const bool opens = (s & 3) != 0;      // one of stages s + 1 .. s + 3 opens a block
         if (ROLE == 0) WAIT_YOUNGER(younger, opens, 8, 1);
         else WAIT_YOUNGER(younger, opens, 8, 4);
         stage_barrier();
-        if (s + RING_SLOTS - 1 < stages) {
-            issue(s + RING_SLOTS - 1, slot_index);
-            slot_index = slot_index + 1 == RING_SLOTS ? 0 : slot_index + 1;
-        }
+        if (more) { issue(); issued++; }
     }
 }
 
@@ -358,7 +455,9 @@ __device__ __forceinline__ half8v q4_scaled_codes(uint32_t w0, uint32_t w1, uint
 
 // A compute wave: all K against its two weight tiles.  A 256-block's result is
 // d * P - dmin * Q with P = sum (scale * code) x and Q = sum_g min_g * (sum of x over group g).
-__device__ __forceinline__ void gemm_compute(const unsigned char *ring, int kblocks, float16v &acc0, float16v &acc1) {
+// slot_off and block_parity carry the ring position from one item to the next.
+__device__ __forceinline__ void gemm_compute(const unsigned char *ring, int kblocks, float16v &acc0, float16v &acc1, int &slot_off,
+                                             int &block_parity) {
     const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
     const uint32_t mask = h ? 0xF0F0F0F0u : 0x0F0F0F0Fu;
     const half_t unit = h ? (half_t)0.0625f : (half_t)1.0f;
@@ -366,7 +465,6 @@ __device__ __forceinline__ void gemm_compute(const unsigned char *ring, int kblo
     const unsigned char *a_lane = ring + (n >> 3) * A_GROUP + (4 * h) * 128 + (n & 7) * 16;
     const unsigned char *w_lane = ring + SLOT_W + (2 * wave) * 1024 + n * 16;
     const float16v zero = {0};
-    int slot_off = 0;
     for (int kb = 0; kb < kblocks; kb++) {
         float16v part0 = zero, part1 = zero, q0 = zero, q1 = zero;
         float d0 = 0.0f, m0 = 0.0f, d1 = 0.0f, m1 = 0.0f;
@@ -387,7 +485,8 @@ __device__ __forceinline__ void gemm_compute(const unsigned char *ring, int kblo
                 al[t] = *reinterpret_cast<const half8v *>(slot_a + A_PART + 128 * t);
             }
             if (j == 0) {
-                const unsigned char *block = ring + (kb & 1) * BLOCK_BYTES;
+                const unsigned char *block = ring + block_parity * BLOCK_BYTES;
+                block_parity ^= 1;
                 const uint4 hdr0 = *reinterpret_cast<const uint4 *>(block + HDR_OFF + (2 * wave) * 512 + n * 16);
                 const uint4 hdr1 = *reinterpret_cast<const uint4 *>(block + HDR_OFF + (2 * wave + 1) * 512 + n * 16);
                 const half8v as = *reinterpret_cast<const half8v *>(block + SUMS_OFF + lane * 16);
@@ -494,94 +593,48 @@ __global__ void __launch_bounds__(256) pf_k_pf_scan_tiles(uint32_t *counts, int 
     }
 }
 
-// Workgroup (row tile, slab): see the description above gemm_loader.
+// One workgroup per compute unit; workgroup b takes items b, b + grid, b + 2 grid, ...
 template <int MODE>
 __global__ void __launch_bounds__(64 * (NW + NL), 3) pf_k_pf_gemm(PfKernelArgs a, int tokens, int slabs) {
     extern __shared__ __align__(16) unsigned char ring[];
-    __shared__ uint32_t src_row[32];
-    __shared__ float row_scale[32];
-    const int E = a.experts, K = a.top_k, lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
-    // Workgroups go to the eight XCDs round robin by index.  The slabs of one row tile read the
-    // same activation rows, so they are given indices eight apart: one XCD, one L2.
-    const uint32_t xcd = blockIdx.x % 8, turn = blockIdx.x / 8, tile = (turn / slabs) * 8 + xcd;
-    if (tile >= a.tiles[0]) return;
-    const uint32_t entry = a.tiles[1 + tile];
-    const int expert = entry & 0xffffu, m0 = 32 * (int)(entry >> 16);
-    GemmTarget g;
-    g.slab = turn % slabs;
-    g.shared = expert == E;
-    const int P = tokens * K;
-    g.first = g.shared ? P : (int)a.offsets[expert];
-    g.count = g.shared ? tokens : (int)a.offsets[expert + 1] - g.first;
-    if (g.count <= m0) return;
-    g.inter = g.shared ? a.shared_inter : a.inter;
-    const size_t ex = g.shared ? 0 : (size_t)expert;
-    if (MODE == PF_GEMM_GATE_UP) {
-        const int tg = g.shared ? 4 : 1;
-        if (32 * NW * g.slab >= g.inter) return;
-        g.row_bytes = (uint32_t)a.row_bytes[tg];
-        g.tiled = a.wt[tg] != nullptr;
-        g.w0 = (g.tiled ? a.wt[tg] : a.w[tg]) + ex * a.expert_bytes[tg] + (size_t)(32 * NW * g.slab) * g.row_bytes;
-        g.w1 = (g.tiled ? a.wt[tg + 1] : a.w[tg + 1]) + ex * a.expert_bytes[tg + 1] + (size_t)(32 * NW * g.slab) * g.row_bytes;
-        g.wave_rows = 32;
-        g.waves = min(NW, (g.inter - 32 * NW * g.slab) / 32);
-        g.kblocks = a.hidden / 256; g.a_cols = a.hidden;
-        g.a16 = reinterpret_cast<const half_t *>(a.x16); g.a_scale = a.x_scale;
-        g.zero_row = a.token_cap;
-    } else {
-        const int td = g.shared ? 6 : 3;
-        if (64 * NW * g.slab >= a.hidden) return;
-        g.row_bytes = (uint32_t)a.row_bytes[td];
-        g.tiled = a.wt[td] != nullptr;
-        g.w0 = (g.tiled ? a.wt[td] : a.w[td]) + ex * a.expert_bytes[td] + (size_t)(64 * NW * g.slab) * g.row_bytes;
-        g.w1 = g.w0 + (size_t)32 * g.row_bytes;
-        g.wave_rows = 64;
-        g.waves = min(NW, (a.hidden - 64 * NW * g.slab) / 64);
-        g.kblocks = g.inter / 256; g.a_cols = g.inter;
-        g.a16 = reinterpret_cast<const half_t *>(g.shared ? a.sact16 : a.act16);
-        g.a_scale = g.shared ? a.sact_scale : a.act_scale;
-        g.zero_row = g.shared ? a.token_cap : a.token_cap * (uint32_t)K;
-    }
-    const int rows_here = min(32, g.count - m0);
-    if (threadIdx.x < 32) {
-        const int m = threadIdx.x;
-        uint32_t src = g.zero_row;
-        float sc = 0.0f;
-        if (m < rows_here) {
-            if (MODE == PF_GEMM_GATE_UP) src = g.shared ? (uint32_t)(m0 + m) : a.row_to_pair[g.first + m0 + m] / (uint32_t)K;
-            else src = g.shared ? (uint32_t)(m0 + m) : (uint32_t)(g.first + m0 + m);
-            sc = g.a_scale[src];
-        }
-        src_row[m] = src;
-        row_scale[m] = sc;
-    }
-    __syncthreads();
+    __shared__ float row_scale[4][32];
+    const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
+    const uint32_t items = (a.tiles[0] + 7u) / 8u * 8u * (uint32_t)slabs;
     if (wave >= NW) {
-        if (wave == NW) gemm_loader<0>(ring, src_row, g);
-        else if (wave == NW + 1) gemm_loader<1>(ring, src_row, g);
-        else gemm_loader<2>(ring, src_row, g);
+        __builtin_amdgcn_s_setprio(3);   // the loaders issue little and everything waits for it
+        if (wave == NW) gemm_loader<MODE, 0>(a, tokens, slabs, items, ring, row_scale);
+        else if (wave == NW + 1) gemm_loader<MODE, 1>(a, tokens, slabs, items, ring, row_scale);
+        else gemm_loader<MODE, 2>(a, tokens, slabs, items, ring, row_scale);
         return;
     }
-    float16v acc0 = {0}, acc1 = {0};
-    gemm_compute(ring, g.kblocks, acc0, acc1);
-    // epilogue: the lane holds column n of its two tiles; register r is row 8 (r / 4) + 4 h + r % 4
+    GemmTarget g;
+    int slot_off = 0, block_parity = 0, item_index = 0;
+    uint32_t q = blockIdx.x;
+    while (gemm_next_item<MODE>(a, tokens, slabs, items, q, g)) {
+        float16v acc0 = {0}, acc1 = {0};
+        gemm_compute(ring, g.kblocks, acc0, acc1, slot_off, block_parity);
+        // epilogue: the lane holds column n of its two tiles; register r is row 8 (r / 4) + 4 h + r % 4
+        const float *scales = row_scale[item_index & 3];
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const int m = 8 * (r >> 2) + 4 * h + (r & 3);
-        if (m >= rows_here || wave >= g.waves) continue;
-        const float rs = row_scale[m];
-        if (MODE == PF_GEMM_GATE_UP) {
-            const int unit = 32 * NW * g.slab + 32 * wave + n;
-            const float gate = acc0[r] * rs, up = acc1[r] * rs;
-            const float v = pf_silu(gate) * up;
-            if (g.shared) a.shared_act[(size_t)(m0 + m) * g.inter + unit] = v;
-            else a.act[(size_t)(g.first + m0 + m) * g.inter + unit] = v;
-        } else {
-            const int r0 = 64 * NW * g.slab + 64 * wave + n;
-            float *out = a.down + (size_t)(g.first + m0 + m) * a.hidden;
-            out[r0] = acc0[r] * rs;
-            out[r0 + 32] = acc1[r] * rs;
+        for (int r = 0; r < 16; r++) {
+            const int m = 8 * (r >> 2) + 4 * h + (r & 3);
+            if (m >= g.rows_here || wave >= g.waves) continue;
+            const float rs = scales[m];
+            if (MODE == PF_GEMM_GATE_UP) {
+                const int unit = 32 * NW * g.slab + 32 * wave + n;
+                const float gate = acc0[r] * rs, up = acc1[r] * rs;
+                const float v = pf_silu(gate) * up;
+                if (g.shared) a.shared_act[(size_t)(g.m0 + m) * g.inter + unit] = v;
+                else a.act[(size_t)(g.first + g.m0 + m) * g.inter + unit] = v;
+            } else {
+                const int r0 = 64 * NW * g.slab + 64 * wave + n;
+                float *out = a.down + (size_t)(g.first + g.m0 + m) * a.hidden;
+                out[r0] = acc0[r] * rs;
+                out[r0 + 32] = acc1[r] * rs;
+            }
         }
+        item_index++;
+        q += gridDim.x;
     }
 }
 
@@ -631,14 +684,18 @@ template <int MODE>
 static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_t stream) {
     const size_t lds = GEMM_LDS;
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    static int grid = 0;
     if (!configured) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_pf_gemm<MODE>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        int device = 0, units = 0;
+        (void)hipGetDevice(&device);
+        (void)hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device);
+        grid = units >= 8 ? units / 8 * 8 : 8;   // one workgroup per compute unit (its LDS), a multiple of the XCD count
         configured = true;
     }
-    // the tile count is only known on the device: launch its upper bound, surplus workgroups exit at once
-    const int max_tiles = pf_prefill_max_tiles(tokens, a.experts, a.top_k);
-    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3((max_tiles + 7) / 8 * 8 * slabs), dim3(64 * (NW + NL)), lds, stream, a, tokens, slabs);
+    // the item count is only known on the device: every workgroup walks the list from its own index
+    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3(grid), dim3(64 * (NW + NL)), lds, stream, a, tokens, slabs);
 }
 
 void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
