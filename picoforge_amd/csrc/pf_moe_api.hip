@@ -148,10 +148,11 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         }
         m->total_bytes += m->bytes[a];
     }
-    {   // transposed router copy for the serial-order re-routing
-        hipError_t e = hipMalloc((void **)&m->router_t, E * h * sizeof(float));
+    {   // router copy in 64-expert slabs for the serial-order re-routing
+        const size_t slab_floats = pf_router_slab_floats((int)E, (int)h);
+        hipError_t e = hipMalloc((void **)&m->router_t, slab_floats * sizeof(float));
         if (e == hipSuccess) {
-            pf_launch_transpose(reinterpret_cast<const float *>(m->w[0]), (int)E, (int)h, m->router_t, nullptr);
+            pf_launch_router_slabs(reinterpret_cast<const float *>(m->w[0]), (int)E, (int)h, m->router_t, nullptr);
             e = hipDeviceSynchronize();
         }
         if (e != hipSuccess) {
@@ -159,7 +160,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             pf_hip_moe_destroy(m);
             return e == hipErrorOutOfMemory ? PF_HIP_E_MEMORY : PF_HIP_E_RUNTIME;
         }
-        m->total_bytes += E * h * sizeof(float);
+        m->total_bytes += slab_floats * sizeof(float);
     }
     m->decode_ready = pf_decode_supported(*desc);
     // prefill path: squared norms of the router rows (the routing tolerance's bound)

@@ -15,7 +15,7 @@ struct PfKernelArgs {
     size_t scale_offset[8];                 // IQ2_XXS: byte offset of the half scales in the tensor buffer
     int k_logical[8], blocks_per_row[8], n_out[8];
     const uint8_t *wt[8];            // Q4_K expert tensors in tile order for the grouped product (null: not kept)
-    const float *router_t;           // router transposed to [hidden][experts] (serial-order re-routing)
+    const float *router_t;           // router as [slab of 64 experts][hidden / 4][64][4] (serial-order re-routing)
     const uint64_t *iq2_grid;        // 256 x 8 magnitudes, device memory
     const uint32_t *iq2_signed;      // 2 x 4096 words: four signed magnitudes per (grid entry, sign nibble)
     const float *x;                  // [tokens, hidden], pitch in floats
@@ -54,7 +54,7 @@ struct PfHipMoe {
     bool decode_ready;               // shapes and formats the specialised decode kernels cover
     bool prefill_ready;              // shapes and formats the matrix-core prefill kernels cover
     float *w_norm2;                  // [experts] squared norm of each router row
-    float *router_t;                 // [hidden][experts] transposed copy of the router
+    float *router_t;                 // [slab of 64 experts][hidden / 4][64][4] copy of the router
     uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
 };
 
@@ -75,7 +75,8 @@ void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, in
 size_t pf_general_lds_bytes(const PfKernelArgs &a);
 // pf_moe_route.hip
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream);
-void pf_launch_transpose(const float *d_src, int rows, int cols, float *d_dst, hipStream_t stream);
+size_t pf_router_slab_floats(int experts, int hidden);
+void pf_launch_router_slabs(const float *d_src, int experts, int hidden, float *d_dst, hipStream_t stream);
 int pf_route_exact_device(const float *d_logits, int tokens, int experts, int top_k, int norm,
                           float *d_probs, uint32_t *d_ids, float *d_weights, uint32_t *d_error,
                           unsigned long long *d_bad_row, hipStream_t stream);

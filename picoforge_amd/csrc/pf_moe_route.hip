@@ -27,71 +27,82 @@ __global__ void __launch_bounds__(64) pf_k_route_fast(PfKernelArgs a) {
 }
 
 // Serial-order recomputation for flagged tokens, in two kernels so that a token's logits
-// spread over many compute units: one wave per (token, 64 experts), lane e owns expert e and
-// the sum runs over k in order, as the reference's, on the transposed router copy
-// [hidden][experts]: every step is one coalesced 256-byte load at a wave-uniform base plus the
-// lane's offset.  Then one wave per token selects.
+// spread over many compute units: one wave per (token, slab of 64 experts), lane e owns expert e
+// and the sum runs over k in order, as the reference's.  The router copy is laid out for this,
+// [slab][hidden / 4][64 experts][4 consecutive k]: four steps of a wave are one 1 KB load at a
+// uniform base plus the lane's offset, and the token's values are scalar operands.  The sum is
+// one dependent chain; the loads are not: they are requested well ahead of the chain (a wave can
+// have 63 of them on their way, 252 steps).
 __global__ void __launch_bounds__(64) pf_k_route_fix_logits(PfKernelArgs a) {
 #pragma clang fp contract(off)
-    const int t = blockIdx.x, E = a.experts, H = a.hidden;
-    int e = blockIdx.y * PF_WAVE + threadIdx.x;
+    const int t = blockIdx.x, E = a.experts, H = a.hidden, lane = threadIdx.x;
+    const int e = blockIdx.y * PF_WAVE + lane;
     if (!a.route_flags[t]) return;
     const float *__restrict__ xs = a.x + (size_t)t * a.x_pitch;
-    const float *__restrict__ wt = a.router_t;
-    const bool live = e < E;
-    e = min(e, E - 1);   // every lane keeps loading: the token's values are shared through v_readlane
-    // The sum is one dependent chain; the loads are not.  They are requested 128 at a time, one
-    // batch ahead of the chain, so that the chain rarely waits for memory.  The token's values
-    // travel the same way, 64 per register, and reach the chain through v_readlane.
-    float sum = 0.0f, wa[128], wb[128], xa[2], xb[2];
-    const int batches = H / 128, lane = threadIdx.x;
-    const uint32_t lane_bytes = 4u * (uint32_t)e;   // uniform row base + 32-bit lane offset: no per-load address arithmetic
-    auto load = [&](float (&dst)[128], float (&xdst)[2], int b) {
-        const char *row = reinterpret_cast<const char *>(wt + (size_t)(128 * b) * E);
-        xdst[0] = xs[128 * b + lane];
-        xdst[1] = xs[128 * b + 64 + lane];
+    const float4 *__restrict__ w = reinterpret_cast<const float4 *>(a.router_t) + (size_t)blockIdx.y * ((H + 3) / 4) * PF_WAVE + lane;
+    float sum = 0.0f;
+    float4 w0[16], w1[16], w2[16];
+    const int batches = H / 64;   // 64 steps = 16 loads
+    auto load = [&](float4 (&dst)[16], int b) {
+        if (b >= batches) return;
+        const float4 *row = w + (size_t)(16 * b) * PF_WAVE;
 #pragma unroll
-        for (int j = 0; j < 128; j++) {
-            dst[j] = *reinterpret_cast<const float *>(row + lane_bytes);
-            row += 4 * (size_t)E;
+        for (int j = 0; j < 16; j++) dst[j] = row[j * PF_WAVE];
+    };
+    auto chain = [&](const float4 (&src)[16], int b) {
+        if (b >= batches) return;
+        const float *x = xs + 64 * b;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const float p0 = src[j].x * x[4 * j];
+            sum = sum + p0;
+            const float p1 = src[j].y * x[4 * j + 1];
+            sum = sum + p1;
+            const float p2 = src[j].z * x[4 * j + 2];
+            sum = sum + p2;
+            const float p3 = src[j].w * x[4 * j + 3];
+            sum = sum + p3;
         }
     };
-    auto chain = [&](const float (&src)[128], const float (&xsrc)[2]) {
-#pragma unroll
-        for (int j = 0; j < 128; j++) {
-            const float xj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xsrc[j >> 6]), j & 63));
-            const float p = src[j] * xj;
-            sum = sum + p;
-        }
-    };
-    if (batches > 0) load(wa, xa, 0);
-    for (int b = 0; b < batches; b += 2) {
-        if (b + 1 < batches) load(wb, xb, b + 1);
-        chain(wa, xa);
-        if (b + 2 < batches) load(wa, xa, b + 2);
-        if (b + 1 < batches) chain(wb, xb);
+    // three batches rotate: two are on their way while one is summed
+    load(w0, 0);
+    load(w1, 1);
+    for (int b = 0; b < batches; b += 3) {
+        load(w2, b + 2);
+        chain(w0, b);
+        load(w0, b + 3);
+        chain(w1, b + 1);
+        load(w1, b + 4);
+        chain(w2, b + 2);
     }
-    for (int k = 128 * batches; k < H; k++) {
-        const float p = (wt + (size_t)k * E)[e] * xs[k];
+    const float *tail = reinterpret_cast<const float *>(w);
+    for (int k = 64 * batches; k < H; k++) {   // the lane's k-quad at 256 (k / 4) floats
+        const float p = tail[(size_t)(k / 4) * 4 * PF_WAVE + (k & 3)] * xs[k];
         sum = sum + p;
     }
-    if (live) a.logits[(size_t)t * E + e] = sum;
+    if (e < E) a.logits[(size_t)t * E + e] = sum;
 }
 
-// router [experts][hidden] -> [hidden][experts], once at upload
-__global__ void pf_k_transpose(const float *src, int rows, int cols, float *dst) {
-    __shared__ float tile[32][33];
-    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32, tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    for (int j = ty; j < 32; j += 8)
-        if (r0 + j < rows && c0 + tx < cols) tile[j][tx] = src[(size_t)(r0 + j) * cols + c0 + tx];
-    __syncthreads();
-    for (int j = ty; j < 32; j += 8)
-        if (c0 + j < cols && r0 + tx < rows) dst[(size_t)(c0 + j) * rows + r0 + tx] = tile[tx][j];
+// router [experts][hidden] -> [slab][ceil(hidden / 4)][64][4] (expert 64 * slab + lane, four
+// consecutive columns together; zeros beyond the last expert and the last column), once at upload
+size_t pf_router_slab_floats(int experts, int hidden) {
+    return (size_t)((experts + PF_WAVE - 1) / PF_WAVE) * ((hidden + 3) / 4) * 4 * PF_WAVE;
 }
 
-void pf_launch_transpose(const float *d_src, int rows, int cols, float *d_dst, hipStream_t stream) {
-    hipLaunchKernelGGL(pf_k_transpose, dim3((cols + 31) / 32, (rows + 31) / 32), dim3(256), 0, stream, d_src, rows, cols,
-                       d_dst);
+__global__ void pf_k_router_slabs(const float *src, int experts, int hidden, float *dst, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t quads = (size_t)(hidden + 3) / 4;
+    const int c = (int)(i & 3), lane = (int)((i >> 2) % PF_WAVE);
+    const size_t quad = (i / (4 * PF_WAVE)) % quads, slab = i / (4 * PF_WAVE * quads);
+    const size_t e = slab * PF_WAVE + lane, k = 4 * quad + c;
+    dst[i] = (e < (size_t)experts && k < (size_t)hidden) ? src[e * hidden + k] : 0.0f;
+}
+
+void pf_launch_router_slabs(const float *d_src, int experts, int hidden, float *d_dst, hipStream_t stream) {
+    const size_t total = pf_router_slab_floats(experts, hidden);
+    hipLaunchKernelGGL(pf_k_router_slabs, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, d_src, experts, hidden,
+                       d_dst, total);
 }
 
 __global__ void __launch_bounds__(64) pf_k_route_fix_select(PfKernelArgs a) {
@@ -210,29 +221,64 @@ __global__ void __launch_bounds__(256) pf_k_group_scan(const uint32_t *counts, i
 }
 
 // one wave per expert walks the pairs in order: rank = earlier pairs of the
-// same expert, so placement is stable without ordered atomics
+// same expert, so placement is stable without ordered atomics.  The ids pass through LDS in
+// pieces; a lane looks at four consecutive pairs per step (one 16-byte LDS read), two steps'
+// reads are requested together.
+#define PLACE_PIECE 8192
 __global__ void __launch_bounds__(256) pf_k_group_place(const uint32_t *ids, int pairs, int E, const uint32_t *offsets,
                                                         uint32_t *pair_to_row, uint32_t *row_to_pair) {
-    __shared__ uint32_t staged[8192];   // the ids pass through LDS in pieces: the scan then waits on no global load
+    __shared__ __align__(16) uint32_t staged[PLACE_PIECE];
     const int e = blockIdx.x * 4 + (threadIdx.x >> 6), lane = pf_lane();
     const bool active = e < E && offsets[min(e, E - 1) + 1] != offsets[min(e, E - 1)];
     uint32_t base = e < E ? offsets[e] : 0u;
-    for (int piece = 0; piece < pairs; piece += 8192) {
-        const int len = min(8192, pairs - piece);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    for (int piece = 0; piece < pairs; piece += PLACE_PIECE) {
+        const int len = min(PLACE_PIECE, pairs - piece), padded = (len + 511) & ~511;
         __syncthreads();
-        for (int i = threadIdx.x; i < len; i += blockDim.x) staged[i] = ids[piece + i];
+        // all of a thread's loads are requested before the first is stored (the piece starts on a
+        // 16-byte boundary of ids; its ragged end is read id by id)
+        uint4 held[PLACE_PIECE / 4 / 256];
+#pragma unroll
+        for (int j = 0; j < PLACE_PIECE / 4 / 256; j++) {
+            const int i = 4 * ((int)threadIdx.x + 256 * j);
+            uint4 v = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+            if (i + 4 <= len) {
+                v = *reinterpret_cast<const uint4 *>(ids + piece + i);
+            } else if (i < len) {
+                v.x = ids[piece + i];
+                if (i + 1 < len) v.y = ids[piece + i + 1];
+                if (i + 2 < len) v.z = ids[piece + i + 2];
+            }
+            held[j] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < PLACE_PIECE / 4 / 256; j++) {
+            const int i = 4 * ((int)threadIdx.x + 256 * j);
+            if (i < padded) *reinterpret_cast<uint4 *>(staged + i) = held[j];
+        }
         __syncthreads();
         if (!active) continue;
-        for (int p0 = 0; p0 < len; p0 += PF_WAVE) {
-            const int p = p0 + lane;
-            const bool hit = p < len && staged[p] == (uint32_t)e;
-            const unsigned long long mask = __ballot(hit);
-            if (hit) {
-                const uint32_t row = base + __popcll(mask & ((1ull << lane) - 1ull));
-                pair_to_row[piece + p] = row;
-                row_to_pair[row] = (uint32_t)(piece + p);
-            }
-            base += __popcll(mask);
+        // step: 256 pairs, lane l holds pairs 4l .. 4l + 3 of it
+        auto place = [&](const uint4 &v, int p0) {
+            const bool h0 = v.x == (uint32_t)e, h1 = v.y == (uint32_t)e, h2 = v.z == (uint32_t)e, h3 = v.w == (uint32_t)e;
+            const int mine = (int)h0 + (int)h1 + (int)h2 + (int)h3;
+            const unsigned long long any = __ballot(mine != 0);
+            if (!any) return;
+            // pairs of lower lanes come first, then this lane's own earlier ones
+            const unsigned long long m0 = __ballot(h0), m1 = __ballot(h1), m2 = __ballot(h2), m3 = __ballot(h3);
+            uint32_t row = base + __popcll(m0 & below) + __popcll(m1 & below) + __popcll(m2 & below) + __popcll(m3 & below);
+            const int p = piece + p0 + 4 * lane;
+            if (h0) { pair_to_row[p] = row; row_to_pair[row] = (uint32_t)p; row++; }
+            if (h1) { pair_to_row[p + 1] = row; row_to_pair[row] = (uint32_t)(p + 1); row++; }
+            if (h2) { pair_to_row[p + 2] = row; row_to_pair[row] = (uint32_t)(p + 2); row++; }
+            if (h3) { pair_to_row[p + 3] = row; row_to_pair[row] = (uint32_t)(p + 3); }
+            base += __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
+        };
+        const uint4 *quads = reinterpret_cast<const uint4 *>(staged);
+        for (int p0 = 0; p0 < padded; p0 += 512) {
+            const uint4 va = quads[p0 / 4 + lane], vb = quads[p0 / 4 + 64 + lane];
+            place(va, p0);
+            place(vb, p0 + 256);
         }
     }
 }

@@ -12,14 +12,28 @@ __device__ __forceinline__ void pf_wave_lds_fence() {
     __builtin_amdgcn_wave_barrier();
 }
 
-// (p, id) arg-max over the wave: larger p wins, equal p goes to the lower id,
-// which is what an ascending scan with a strict comparison selects.
+// (p, id) arg-max over the wave: larger p wins, equal p goes to the lower id, which is what an
+// ascending scan with a strict comparison selects.  p is a probability or negative (no candidate):
+// nonnegative floats order like their bit patterns, so the pair travels as one 64-bit key,
+// (bits of p) : (~id), through the DPP reduction steps; a lane without a candidate offers key 0.
 __device__ __forceinline__ void pf_wave_argmax(float &p, uint32_t &id) {
-    for (int m = 1; m < PF_WAVE; m <<= 1) {
-        float op = __shfl_xor(p, m);
-        uint32_t oid = __shfl_xor(id, m);
-        if (op > p || (op == p && oid < id)) { p = op; id = oid; }
-    }
+    uint32_t hi = p < 0.0f ? 0u : __float_as_uint(p), lo = p < 0.0f ? 0u : ~id;
+    auto step = [&](auto dpp) {
+        const uint32_t mh = (uint32_t)dpp((int)hi), ml = (uint32_t)dpp((int)lo);
+        const bool better = mh > hi || (mh == hi && ml > lo);
+        hi = better ? mh : hi;
+        lo = better ? ml : lo;
+    };
+    step([](int v) { return __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xF, 0xF, false); });    // quad_perm [1,0,3,2]
+    step([](int v) { return __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xF, 0xF, false); });    // quad_perm [2,3,0,1]
+    step([](int v) { return __builtin_amdgcn_update_dpp(v, v, 0x141, 0xF, 0xF, false); });   // row_half_mirror
+    step([](int v) { return __builtin_amdgcn_update_dpp(v, v, 0x140, 0xF, 0xF, false); });   // row_mirror
+    step([](int v) { return __builtin_amdgcn_update_dpp(v, v, 0x142, 0xA, 0xF, false); });   // row_bcast:15 into rows 1,3
+    step([](int v) { return __builtin_amdgcn_update_dpp(v, v, 0x143, 0xC, 0xF, false); });   // row_bcast:31 into rows 2,3
+    hi = (uint32_t)__builtin_amdgcn_readlane((int)hi, 63);
+    lo = (uint32_t)__builtin_amdgcn_readlane((int)lo, 63);
+    p = (hi | lo) ? __uint_as_float(hi) : -2.0f;
+    id = (hi | lo) ? ~lo : 0xffffffffu;
 }
 
 // One router logit in the reference's order: k ascending, product then sum.
@@ -49,7 +63,15 @@ __device__ __forceinline__ void pf_route_exact_wave(const float *z, float *p, fl
     }
     pf_wave_lds_fence();
     float sum = 0.0f;
-    for (int e = 0; e < E; e++) sum = sum + p[e];   // serial, expert ascending
+    int e0 = 0;
+    for (; e0 + 32 <= E; e0 += 32) {   // serial, expert ascending; the LDS reads of a batch are requested together
+        float v[32];
+#pragma unroll
+        for (int j = 0; j < 32; j++) v[j] = p[e0 + j];
+#pragma unroll
+        for (int j = 0; j < 32; j++) sum = sum + v[j];
+    }
+    for (int e = e0; e < E; e++) sum = sum + p[e];
     pf_wave_lds_fence();
     for (int e = lane; e < E; e += PF_WAVE) {
         float v = p[e] / sum;
@@ -57,7 +79,8 @@ __device__ __forceinline__ void pf_route_exact_wave(const float *z, float *p, fl
         q[e] = v;
     }
     pf_wave_lds_fence();
-    float chosen = 0.0f;
+    float chosen = 0.0f, mine = 0.0f;
+    uint32_t mine_id = 0;
     for (int slot = 0; slot < K; slot++) {
         float best = -2.0f;
         uint32_t best_id = 0xffffffffu;
@@ -69,10 +92,17 @@ __device__ __forceinline__ void pf_route_exact_wave(const float *z, float *p, fl
         if ((int)(best_id & (PF_WAVE - 1)) == lane) q[best_id] = -1.0f;
         pf_wave_lds_fence();
         chosen = chosen + best;
-        if (lane == 0) { ids_out[slot] = best_id; w_out[slot] = best; }
+        if ((slot & (PF_WAVE - 1)) == lane) { mine = best; mine_id = best_id; }   // lane r keeps slots r, r + 64, ...
+        // ids_out / w_out may be global memory: written from registers, 64 slots at a time
+        if ((slot & (PF_WAVE - 1)) == PF_WAVE - 1 || slot == K - 1) {
+            const int s = (slot & ~(PF_WAVE - 1)) + lane;
+            if (s <= slot) {
+                ids_out[s] = mine_id;
+                w_out[s] = (norm && K <= PF_WAVE) ? mine / chosen : mine;   // chosen is final here when K <= 64
+            }
+        }
     }
-    pf_wave_lds_fence();
-    if (norm && lane == 0)
-        for (int slot = 0; slot < K; slot++) w_out[slot] = w_out[slot] / chosen;
+    if (norm && K > PF_WAVE)   // each lane divides the slots it wrote itself
+        for (int s = lane; s < K; s += PF_WAVE) w_out[s] = w_out[s] / chosen;
     pf_wave_lds_fence();
 }
