@@ -567,19 +567,24 @@ __global__ void __launch_bounds__(256) pf_k_pf_scan_tiles(uint32_t *counts, int 
     rows_before[tid] = rows;
     tiles_before[tid] = ntiles;
     __syncthreads();
-    if (tid == 0) {
-        uint32_t run_rows = 0, run_tiles = 0;
-        for (int i = 0; i < 256; i++) {
-            const uint32_t r = rows_before[i], n = tiles_before[i];
-            rows_before[i] = run_rows;
-            tiles_before[i] = run_tiles;
-            run_rows += r;
-            run_tiles += n;
-        }
+    // inclusive scan of the 256 partial sums in eight doubling steps, then made exclusive
+    uint32_t run_rows = rows, run_tiles = ntiles;
+    for (int d = 1; d < 256; d <<= 1) {
+        const uint32_t add_rows = tid >= d ? rows_before[tid - d] : 0u, add_tiles = tid >= d ? tiles_before[tid - d] : 0u;
+        __syncthreads();
+        run_rows += add_rows;
+        run_tiles += add_tiles;
+        rows_before[tid] = run_rows;
+        tiles_before[tid] = run_tiles;
+        __syncthreads();
+    }
+    if (tid == 255) {
         offsets[E] = run_rows;
         tiles[0] = run_tiles;
     }
     __syncthreads();
+    rows_before[tid] = run_rows - rows;
+    tiles_before[tid] = run_tiles - ntiles;
     uint32_t row = rows_before[tid], at = tiles_before[tid];
     for (int e = lo; e < hi; e++) {
         const uint32_t c = e < E ? counts[e] : (uint32_t)tokens, n = (c + 31u) / 32u;
