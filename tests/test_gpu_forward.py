@@ -84,6 +84,25 @@ def test_prefill_kernels_match_oracle_and_general_kernels(product, oracle, h, e,
         assert_parity(y, ids, w, *want, label="general kernels on a prefill shape")
 
 
+def test_prefill_from_row_order_when_the_tile_ordered_copy_is_switched_off(product, oracle, monkeypatch):
+    """PF_MOE_PREFILL_COPY=0 at create: the grouped product reads the GGUF row order, same results bit for bit."""
+    cfg = abi.moe_config(512, 8, 3, 256, 512)
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 70, seed=590)
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, 70) as layer:
+        _, y_tiled, _, _ = layer.forward(x)
+    monkeypatch.setenv("PF_MOE_PREFILL_COPY", "0")
+    with pf.MoeLayer(product, cfg, weights, 70) as layer:
+        bytes_without = product.hip.moe_bytes(layer.device_handles()[0])
+        _, y, ids, w = layer.forward(x)
+    monkeypatch.delenv("PF_MOE_PREFILL_COPY")
+    with pf.MoeLayer(product, cfg, weights, 70) as layer:
+        bytes_with = product.hip.moe_bytes(layer.device_handles()[0])
+    assert_parity(y, ids, w, *want, label="prefill from the row order")
+    np.testing.assert_array_equal(y, y_tiled, err_msg="the two weight orders give different results")
+    assert bytes_with > bytes_without
+
+
 def test_prefill_rows_of_very_different_magnitude(product, oracle):
     """Per-row power-of-two scaling: rows spanning 1e-6 .. 1e6 keep the relative accuracy."""
     cfg = abi.moe_config(256, 16, 4, 256, 256)
