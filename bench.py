@@ -11,8 +11,9 @@ input, hence other experts.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 Workloads: iq2xxs_decode (default), q4k_decode, q4k_verify4 (4-token batches with
-about half of the experts shared between neighbours), q4k_prefill1024 (1024-token
-chunks, N(0,1) activations, Zipf(1.1) expert popularity).
+about half of the experts shared between neighbours), q4k_prefill1024 and
+iq2xxs_prefill1024 (1024-token chunks, N(0,1) activations, Zipf(1.1) expert
+popularity), q4k_stack48 (48 resident layers, decode and 2048-token chunks).
 
 Prints one JSON line.  `value` is microseconds per layer per token (lower is
 better).  `roofline` is for the kernel that moves the most bytes, timed live
@@ -48,6 +49,8 @@ WORKLOADS = {
                         label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
     "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10,
                             label="Q4_K experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
+    "iq2xxs_prefill1024": dict(type=abi.GGUF_IQ2_XXS, tokens=1024, steps=100, warmup=10,
+                               label="IQ2_XXS experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),

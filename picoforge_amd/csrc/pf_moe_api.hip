@@ -116,7 +116,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             // device layout: every block's 64-byte payload, then every block's half scale
             m->row_bytes[a] = blocks_per_row * 64;
             m->scale_offset[a] = (blocks_per_row * rows * 64 + 255) & ~(size_t)255;
-            m->bytes[a] = m->scale_offset[a] + blocks_per_row * rows * 2;
+            m->bytes[a] = m->scale_offset[a] + blocks_per_row * rows * 2 + 4;   // the prefill loader reads the dword around a scale
         } else {
             m->row_bytes[a] = blocks_per_row * size;
             m->bytes[a] = gguf_bytes[a];
@@ -180,7 +180,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         // lines once instead of 32-byte pieces of lines it meets again a stage later.  It doubles the
         // expert bytes; PF_MOE_PREFILL_COPY=0 does without it (the same kernels read the row order).
         const char *copy = getenv("PF_MOE_PREFILL_COPY");
-        if (!copy || strcmp(copy, "0") != 0) {
+        if (desc->type[1] == PF_Q4_K && (!copy || strcmp(copy, "0") != 0)) {
             for (int a = 1; a <= 6 && e == hipSuccess; a++) {
                 e = hipMalloc((void **)&m->w_tiled[a], m->bytes[a]);
                 if (e == hipSuccess) {

@@ -186,11 +186,10 @@ enum { PF_GEMM_GATE_UP = 0, PF_GEMM_DOWN = 1 };
 // waves.
 //
 // Only the loader waves issue global loads.  They move the operands of one stage (64 of the K
-// columns) straight into LDS, 16 bytes per lane, up to five stages ahead of the products, through
-// a ring of six slots: with one workgroup per compute unit that keeps about 100 KB on their way,
-// what it takes to cover the memory latency at full bandwidth; a wave counts at most 63 loads, so
-// the stream is split over three loaders (activations; the weight runs of compute waves 0-3; of
-// 4-7).  A stalled memory pipeline holds up the loaders, never the waves that feed the matrix
+// columns) straight into LDS, 16 bytes per lane, up to four stages ahead of the products, through
+// a ring of five slots: with one workgroup per compute unit that keeps about 100 KB on their way;
+// a wave counts at most 63 loads, so the stream is split over three loaders (activations; the
+// weight runs of compute waves 0-3; of 4-7).  A stalled memory pipeline holds up the loaders, never the waves that feed the matrix
 // cores.  One workgroup barrier per stage hands the landed slot to the compute waves and the slot
 // they have just left back to the loaders.
 //
@@ -200,6 +199,11 @@ enum { PF_GEMM_GATE_UP = 0, PF_GEMM_DOWN = 1 };
 //          [SLOT_W, +2 NW KB)     the stage's 32-byte nibble run of every weight row: per tile the
 //                                 first halves of the 32 rows, then the second halves
 //   once per 256-block: the 16-byte block headers of the 2 NW tiles, the activation rows' group sums
+//
+// IQ2_XXS differs in the weight bytes only: a row's stage is 16 bytes (two 32-groups of four grid
+// indices and one word of signs and scale), so a wave's two tiles are one 1 KB image
+// [tile][row][16 bytes]; per 256-block a row brings its fp16 scale (the dword around it); the
+// 256 x 8 magnitude grid and the 128 sign masks sit in LDS behind the ring.
 //
 // Matrix-core operands.  Lane (n = lane % 32, h = lane / 32) holds column n (a weight row) and
 // supplies K slots 8h..8h+7.  In stage j, step t, these are the codes 8t..8t+7 of group 2j + h
@@ -216,10 +220,17 @@ enum { PF_GEMM_GATE_UP = 0, PF_GEMM_DOWN = 1 };
 #define BLOCK_BYTES (2 * NW * 512 + 1024)   // per 256-block: headers, then sums; two copies (blocks alternate)
 #define SUMS_OFF (HDR_OFF + 2 * NW * 512)
 #define GEMM_LDS (HDR_OFF + 2 * BLOCK_BYTES)   // 146 432 bytes with 8 compute waves: one workgroup per compute unit
+#define IQ2_GRID_OFF GEMM_LDS                  // IQ2_XXS: 256 grid entries of 8 magnitudes, then 128 masks of 8 fp16 sign bits
+#define IQ2_SIGN_OFF (IQ2_GRID_OFF + 2048)
+#define GEMM_LDS_IQ2 (IQ2_SIGN_OFF + 2048)
 static_assert(RING_SLOTS == 5 && NW % 4 == 0, "the loaders' wait counts below assume three younger stages on their way");
 
 __device__ __forceinline__ void to_lds(const void *global, unsigned char *lds) {
     __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(global), reinterpret_cast<uint32_t *>(lds), 16, 0, 0);
+}
+
+__device__ __forceinline__ void to_lds_dword(const void *global, unsigned char *lds) {   // 4 bytes per lane, lane l at lds + 4 l
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(global), reinterpret_cast<uint32_t *>(lds), 4, 0, 0);
 }
 
 __device__ __forceinline__ void stage_barrier() {
@@ -238,6 +249,8 @@ struct GemmTarget {   // one work item of the grouped product: a 32-row tile of 
     uint32_t wave_rows;   // weight rows between the tiles of consecutive compute waves
     bool tiled;           // weights in the tile order of pf_k_q4k_tile (else GGUF row order)
     const uint8_t *w0, *w1;   // first weight row of compute wave 0's two tiles
+    const uint16_t *s0, *s1;  // IQ2_XXS: the tensors' fp16 block scales, and the index of the tiles' first row's first scale
+    uint32_t sidx0, sidx1, bpr;
     const half_t *a16;
     const float *a_scale;
 };
@@ -246,7 +259,7 @@ struct GemmTarget {   // one work item of the grouped product: a 32-row tile of 
 // workgroup's items are a multiple of eight apart, so the slabs of one row tile, which read the
 // same activation rows, are given item numbers eight apart: one XCD, one L2.  False: nothing to do
 // for q.  Every wave of the workgroup evaluates this for itself, with the same result.
-template <int MODE>
+template <int MODE, int FMT>
 __device__ __forceinline__ bool gemm_item(const PfKernelArgs &a, int tokens, int slabs, uint32_t q, GemmTarget &g) {
     const int E = a.experts, K = a.top_k;
     const uint32_t xcd = q % 8, turn = q / 8, tile = (turn / slabs) * 8 + xcd;
@@ -270,6 +283,12 @@ __device__ __forceinline__ bool gemm_item(const PfKernelArgs &a, int tokens, int
         g.tiled = a.wt[tg] != nullptr;
         g.w0 = (g.tiled ? a.wt[tg] : a.w[tg]) + ex * a.expert_bytes[tg] + (size_t)(32 * NW * g.slab) * g.row_bytes;
         g.w1 = (g.tiled ? a.wt[tg + 1] : a.w[tg + 1]) + ex * a.expert_bytes[tg + 1] + (size_t)(32 * NW * g.slab) * g.row_bytes;
+        if (FMT == PF_IQ2_XXS) {
+            g.bpr = (uint32_t)a.blocks_per_row[tg];
+            g.s0 = reinterpret_cast<const uint16_t *>(a.w[tg] + a.scale_offset[tg]);
+            g.s1 = reinterpret_cast<const uint16_t *>(a.w[tg + 1] + a.scale_offset[tg + 1]);
+            g.sidx0 = g.sidx1 = (uint32_t)((ex * a.n_out[tg] + 32 * NW * g.slab) * g.bpr);
+        }
         g.wave_rows = 32;
         g.waves = min(NW, (g.inter - 32 * NW * g.slab) / 32);
         g.kblocks = a.hidden / 256; g.a_cols = a.hidden;
@@ -282,6 +301,12 @@ __device__ __forceinline__ bool gemm_item(const PfKernelArgs &a, int tokens, int
         g.tiled = a.wt[td] != nullptr;
         g.w0 = (g.tiled ? a.wt[td] : a.w[td]) + ex * a.expert_bytes[td] + (size_t)(64 * NW * g.slab) * g.row_bytes;
         g.w1 = g.w0 + (size_t)32 * g.row_bytes;
+        if (FMT == PF_IQ2_XXS) {
+            g.bpr = (uint32_t)a.blocks_per_row[td];
+            g.s0 = g.s1 = reinterpret_cast<const uint16_t *>(a.w[td] + a.scale_offset[td]);
+            g.sidx0 = (uint32_t)((ex * a.n_out[td] + 64 * NW * g.slab) * g.bpr);
+            g.sidx1 = g.sidx0 + 32 * g.bpr;
+        }
         g.wave_rows = 64;
         g.waves = min(NW, (a.hidden - 64 * NW * g.slab) / 64);
         g.kblocks = g.inter / 256; g.a_cols = g.inter;
@@ -293,11 +318,11 @@ __device__ __forceinline__ bool gemm_item(const PfKernelArgs &a, int tokens, int
 }
 
 // first item at or after q (stepping by the grid size) that has work; false when the list is exhausted
-template <int MODE>
+template <int MODE, int FMT>
 __device__ __forceinline__ bool gemm_next_item(const PfKernelArgs &a, int tokens, int slabs, uint32_t items, uint32_t &q,
                                                GemmTarget &g) {
     for (; q < items; q += gridDim.x)
-        if (gemm_item<MODE>(a, tokens, slabs, q, g)) return true;
+        if (gemm_item<MODE, FMT>(a, tokens, slabs, q, g)) return true;
     return false;
 }
 
@@ -319,13 +344,13 @@ __device__ __forceinline__ bool gemm_next_item(const PfKernelArgs &a, int tokens
 // 4 (q - 1) .. 4 (q - 1) + 3.  It walks the workgroup's items as one stream of stages, up to
 // RING_SLOTS - 1 stages ahead of the compute waves, also across item boundaries: the ring never
 // drains between items.  Every workgroup barrier here pairs with one of gemm_compute.
-template <int MODE, int ROLE>
+template <int MODE, int FMT, int ROLE>
 __device__ __forceinline__ void gemm_loader(const PfKernelArgs &a, int tokens, int slabs, uint32_t items, unsigned char *ring,
                                             float (*row_scale)[32]) {
     const int lane = pf_lane(), K = a.top_k;
     GemmTarget g;
     uint32_t q = blockIdx.x;
-    bool more = gemm_next_item<MODE>(a, tokens, slabs, items, q, g);
+    bool more = gemm_next_item<MODE, FMT>(a, tokens, slabs, items, q, g);
     int kb = 0, j = 0, slot_index = 0, block_parity = 0, item_index = 0;
     uint32_t a_off[4] = {0, 0, 0, 0}, a_live[4] = {0, 0, 0, 0}, s_off = 0, s_live = 0, w_off = 0, h_off = 0, block_step = 0,
              run0 = 0, run_step = 0;
@@ -356,6 +381,12 @@ __device__ __forceinline__ void gemm_loader(const PfKernelArgs &a, int tokens, i
             // current one is over)
             if (lane < 32) row_scale[item_index & 3][lane] = (lane < g.rows_here) ? g.a_scale[mine] : 0.0f;
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        } else if (FMT == PF_IQ2_XXS) {
+            // lane = 32 * (tile of the wave's pair) + row: the row's two groups of the stage, and per
+            // block the dword that holds the row's fp16 scale
+            w_off = (uint32_t)(lane & 31) * g.row_bytes;
+            h_off = (uint32_t)(lane & 31) * g.bpr;
+            wave_bytes = (size_t)g.wave_rows * g.row_bytes;
         } else {
             // weight runs: lane = 32 * half + row; headers: lane = 32 * (tile of the wave's pair) + row.
             // Tile order: a 32-row tile's 256-block is 4608 consecutive bytes, the 32 headers, then per
@@ -378,6 +409,23 @@ __device__ __forceinline__ void gemm_loader(const PfKernelArgs &a, int tokens, i
                 to_lds(g.a16 + a_off[i] + (low & a_live[i]), slot + A_PART + i * A_GROUP);
             }
             if (j == 0) to_lds(g.a16 + s_off + (16u * (uint32_t)kb & s_live), block + SUMS_OFF);
+        } else if (FMT == PF_IQ2_XXS) {
+            const uint8_t *tile = (lane >> 5) ? g.w1 : g.w0;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const int v = 4 * (ROLE - 1) + c, vv = min(v, g.waves - 1);   // a wave without rows repeats the last one's
+                to_lds(tile + (size_t)vv * wave_bytes + w_off + 64u * (uint32_t)kb + 16u * (uint32_t)j, slot + SLOT_W + v * 1024);
+            }
+            if (j == 0) {
+                const uint16_t *scales = (lane >> 5) ? g.s1 : g.s0;
+                const uint32_t first = (lane >> 5) ? g.sidx1 : g.sidx0;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const int v = 4 * (ROLE - 1) + c, vv = min(v, g.waves - 1);
+                    const uint32_t at = first + (uint32_t)vv * g.wave_rows * g.bpr + h_off + (uint32_t)kb;
+                    to_lds_dword(scales + (at & ~1u), block + HDR_OFF + v * 256);
+                }
+            }
         } else {
             const uint32_t run = block_step * (uint32_t)kb + run0 + run_step * (uint32_t)j;
 #pragma unroll
@@ -403,7 +451,7 @@ __device__ __forceinline__ void gemm_loader(const PfKernelArgs &a, int tokens, i
             if (++kb == g.kblocks) {
                 kb = 0;
                 q += gridDim.x;
-                more = gemm_next_item<MODE>(a, tokens, slabs, items, q, g);
+                more = gemm_next_item<MODE, FMT>(a, tokens, slabs, items, q, g);
                 if (more) open_item();
             }
         }
@@ -418,6 +466,7 @@ __device__ __forceinline__ void gemm_loader(const PfKernelArgs &a, int tokens, i
         const int younger = issued - s - 1;   // at most RING_SLOTS - 2
         const bool opens = (s & 3) != 0;      // one of stages s + 1 .. s + 3 opens a block
         if (ROLE == 0) WAIT_YOUNGER(younger, opens, 8, 1);
+        else if (FMT == PF_IQ2_XXS) WAIT_YOUNGER(younger, opens, 4, 4);
         else WAIT_YOUNGER(younger, opens, 8, 4);
         stage_barrier();
         if (more) { issue(); issued++; }
@@ -544,6 +593,83 @@ __device__ __forceinline__ void gemm_compute(const unsigned char *ring, int kblo
     }
 }
 
+// The same for IQ2_XXS tiles (src/qwen4_packed.c:95-121): a weight is d / 8 * (2 s + 1) * magnitude * sign with a
+// 4-bit s per 32-group, magnitudes 8, 25 or 43 from the grid and d per 256-block, so
+// (2 s + 1) * magnitude <= 1333 is an exact fp16 operand: a magnitude byte under the exponent byte
+// 0x64 reads as 1024 + m, (1024 + m) * (2 s + 1) - 1024 * (2 s + 1) = m * (2 s + 1) in one fused step,
+// and the sign is a bit flip.  A 256-block's result is (d / 8) * P.  Lane (n, h) takes group 2 j + h in
+// stage j: step t is its grid entry t (8 weights) with the 7 sign bits t of the group's second word.
+// sidx0 / sidx1 / bpr locate the rows' fp16 block scales (which half of the loaded dword is theirs).
+__device__ __forceinline__ void gemm_compute_iq2(const unsigned char *ring, int kblocks, float16v &acc0, float16v &acc1,
+                                                 int &slot_off, int &block_parity, uint32_t sidx0, uint32_t sidx1, uint32_t bpr,
+                                                 int wave_rows) {
+    const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
+    const unsigned char *a_lane = ring + (n >> 3) * A_GROUP + (4 * h) * 128 + (n & 7) * 16;
+    const unsigned char *w_lane = ring + SLOT_W + wave * 1024 + n * 16 + 8 * h;
+    const uint2 *grid = reinterpret_cast<const uint2 *>(ring + IQ2_GRID_OFF);
+    const uint4 *signs = reinterpret_cast<const uint4 *>(ring + IQ2_SIGN_OFF);
+    // index of this lane's rows' first scale; the loader fetched the dword around scale index + kb
+    const uint32_t row0 = sidx0 + ((uint32_t)wave * wave_rows + n) * bpr, row1 = sidx1 + ((uint32_t)wave * wave_rows + n) * bpr;
+    const float16v zero = {0};
+    for (int kb = 0; kb < kblocks; kb++) {
+        float16v part0 = zero, part1 = zero;
+        float d0 = 0.0f, d1 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            stage_barrier();
+            const unsigned char *slot_a = a_lane + slot_off, *slot_w = w_lane + slot_off;
+            slot_off = slot_off + SLOT_BYTES == RING_SLOTS * SLOT_BYTES ? 0 : slot_off + SLOT_BYTES;
+            const uint2 g0 = *reinterpret_cast<const uint2 *>(slot_w), g1 = *reinterpret_cast<const uint2 *>(slot_w + 512);
+            half8v ah[4], al[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                ah[t] = *reinterpret_cast<const half8v *>(slot_a + 128 * t);
+                al[t] = *reinterpret_cast<const half8v *>(slot_a + A_PART + 128 * t);
+            }
+            if (j == 0) {
+                const unsigned char *block = ring + block_parity * BLOCK_BYTES;
+                block_parity ^= 1;
+                const uint32_t pair0 = *reinterpret_cast<const uint32_t *>(block + HDR_OFF + wave * 256 + 4 * n);
+                const uint32_t pair1 = *reinterpret_cast<const uint32_t *>(block + HDR_OFF + wave * 256 + 128 + 4 * n);
+                const uint32_t bits0 = ((row0 + (uint32_t)kb) & 1u) ? pair0 >> 16 : pair0 & 0xffffu;
+                const uint32_t bits1 = ((row1 + (uint32_t)kb) & 1u) ? pair1 >> 16 : pair1 & 0xffffu;
+                d0 = (float)__builtin_bit_cast(half_t, (unsigned short)bits0) * 0.125f;
+                d1 = (float)__builtin_bit_cast(half_t, (unsigned short)bits1) * 0.125f;
+            }
+            asm volatile("" ::: "memory");   // the requests stay above the arithmetic
+            const half_t s0 = (half_t)(int)(2u * (g0.y >> 28) + 1u), s1 = (half_t)(int)(2u * (g1.y >> 28) + 1u);
+            const half_t k0 = (half_t)(int)(1024u * (2u * (g0.y >> 28) + 1u)), k1 = (half_t)(int)(1024u * (2u * (g1.y >> 28) + 1u));
+            const half2v s20 = {s0, s0}, s21 = {s1, s1}, c20 = {k0, k0}, c21 = {k1, k1};
+            auto codes = [&](const uint2 &g, int t, half2v s2, half2v c) -> half8v {
+                const uint2 m = grid[(g.x >> (8 * t)) & 255u];
+                const uint4 flip = signs[(g.y >> (7 * t)) & 127u];
+                const uint32_t bias = 0x64646464u;
+                const half2v p0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, m.x, 0x04010400u));
+                const half2v p1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, m.x, 0x04030402u));
+                const half2v p2 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, m.y, 0x04010400u));
+                const half2v p3 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, m.y, 0x04030402u));
+                const half2v v0 = p0 * s2 - c, v1 = p1 * s2 - c, v2 = p2 * s2 - c, v3 = p3 * s2 - c;
+                const uint4 bits = {__builtin_bit_cast(uint32_t, v0) ^ flip.x, __builtin_bit_cast(uint32_t, v1) ^ flip.y,
+                                    __builtin_bit_cast(uint32_t, v2) ^ flip.z, __builtin_bit_cast(uint32_t, v3) ^ flip.w};
+                return __builtin_bit_cast(half8v, bits);
+            };
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const half8v b0 = codes(g0, t, s20, c20), b1 = codes(g1, t, s21, c21);
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[t], b0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[t], b1, part1, 0, 0, 0);
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[t], b0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[t], b1, part1, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            acc0[r] = fmaf(d0, part0[r], acc0[r]);
+            acc1[r] = fmaf(d1, part1[r], acc1[r]);
+        }
+    }
+}
+
 // Histogram of the routed pairs.  counts[] is zero on entry: the workspace starts zeroed and
 // pf_k_pf_scan_tiles clears it again once it has been read.
 __global__ void pf_k_pf_count(const uint32_t *ids, int pairs, int E, uint32_t *counts) {
@@ -599,25 +725,43 @@ __global__ void __launch_bounds__(256) pf_k_pf_scan_tiles(uint32_t *counts, int 
 }
 
 // One workgroup per compute unit; workgroup b takes items b, b + grid, b + 2 grid, ...
-template <int MODE>
+template <int MODE, int FMT>
 __global__ void __launch_bounds__(64 * (NW + NL), 3) pf_k_pf_gemm(PfKernelArgs a, int tokens, int slabs) {
     extern __shared__ __align__(16) unsigned char ring[];
     __shared__ float row_scale[4][32];
     const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
     const uint32_t items = (a.tiles[0] + 7u) / 8u * 8u * (uint32_t)slabs;
+    if (FMT == PF_IQ2_XXS) {
+        // grid magnitudes, and for every 7-bit sign field the fp16 sign bits of its eight weights
+        // (the eighth sign makes the number of negative weights even)
+        if (threadIdx.x < 256) reinterpret_cast<uint64_t *>(ring + IQ2_GRID_OFF)[threadIdx.x] = a.iq2_grid[threadIdx.x];
+        if (threadIdx.x >= 256 && threadIdx.x < 384) {
+            const uint32_t s7 = threadIdx.x - 256, s8 = s7 | ((__popc(s7) & 1u) << 7);
+            uint4 flip;
+            flip.x = ((s8 >> 0) & 1u) << 15 | ((s8 >> 1) & 1u) << 31;
+            flip.y = ((s8 >> 2) & 1u) << 15 | ((s8 >> 3) & 1u) << 31;
+            flip.z = ((s8 >> 4) & 1u) << 15 | ((s8 >> 5) & 1u) << 31;
+            flip.w = ((s8 >> 6) & 1u) << 15 | ((s8 >> 7) & 1u) << 31;
+            reinterpret_cast<uint4 *>(ring + IQ2_SIGN_OFF)[s7] = flip;
+        }
+        __syncthreads();
+    }
     if (wave >= NW) {
         __builtin_amdgcn_s_setprio(3);   // the loaders issue little and everything waits for it
-        if (wave == NW) gemm_loader<MODE, 0>(a, tokens, slabs, items, ring, row_scale);
-        else if (wave == NW + 1) gemm_loader<MODE, 1>(a, tokens, slabs, items, ring, row_scale);
-        else gemm_loader<MODE, 2>(a, tokens, slabs, items, ring, row_scale);
+        if (wave == NW) gemm_loader<MODE, FMT, 0>(a, tokens, slabs, items, ring, row_scale);
+        else if (wave == NW + 1) gemm_loader<MODE, FMT, 1>(a, tokens, slabs, items, ring, row_scale);
+        else gemm_loader<MODE, FMT, 2>(a, tokens, slabs, items, ring, row_scale);
         return;
     }
     GemmTarget g;
     int slot_off = 0, block_parity = 0, item_index = 0;
     uint32_t q = blockIdx.x;
-    while (gemm_next_item<MODE>(a, tokens, slabs, items, q, g)) {
+    while (gemm_next_item<MODE, FMT>(a, tokens, slabs, items, q, g)) {
         float16v acc0 = {0}, acc1 = {0};
-        gemm_compute(ring, g.kblocks, acc0, acc1, slot_off, block_parity);
+        if (FMT == PF_IQ2_XXS)
+            gemm_compute_iq2(ring, g.kblocks, acc0, acc1, slot_off, block_parity, g.sidx0, g.sidx1, g.bpr, (int)g.wave_rows);
+        else
+            gemm_compute(ring, g.kblocks, acc0, acc1, slot_off, block_parity);
         // epilogue: the lane holds column n of its two tiles; register r is row 8 (r / 4) + 4 h + r % 4
         const float *scales = row_scale[item_index & 3];
 #pragma unroll
@@ -672,8 +816,9 @@ __global__ void __launch_bounds__(256) pf_k_pf_combine(PfKernelArgs a, int token
 
 // ---- dispatch --------------------------------------------------------------------------------------
 bool pf_prefill_supported(const PfHipMoeDesc &d) {
+    if (d.type[1] != PF_Q4_K && d.type[1] != PF_IQ2_XXS) return false;
     for (int j = 1; j <= 6; j++)
-        if (d.type[j] != PF_Q4_K) return false;
+        if (d.type[j] != d.type[1]) return false;
     if (d.hidden % 256 || d.inter % 256 || d.shared_inter % 256 || d.down_physical != d.inter) return false;
     if (d.top_k > 64 || d.top_k >= d.experts || d.experts >= 65535) return false;
     return true;
@@ -685,13 +830,13 @@ int pf_prefill_max_tiles(int tokens, int experts, int top_k) {
     return (int)(((size_t)tokens * top_k) / 32 + experts + (tokens + 31) / 32 + 1);
 }
 
-template <int MODE>
+template <int MODE, int FMT>
 static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_t stream) {
-    const size_t lds = GEMM_LDS;
+    const size_t lds = FMT == PF_IQ2_XXS ? GEMM_LDS_IQ2 : GEMM_LDS;
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
     static int grid = 0;
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_pf_gemm<MODE>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_pf_gemm<MODE, FMT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         int device = 0, units = 0;
         (void)hipGetDevice(&device);
@@ -700,7 +845,7 @@ static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_
         configured = true;
     }
     // the item count is only known on the device: every workgroup walks the list from its own index
-    hipLaunchKernelGGL((pf_k_pf_gemm<MODE>), dim3(grid), dim3(64 * (NW + NL)), lds, stream, a, tokens, slabs);
+    hipLaunchKernelGGL((pf_k_pf_gemm<MODE, FMT>), dim3(grid), dim3(64 * (NW + NL)), lds, stream, a, tokens, slabs);
 }
 
 void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
@@ -719,13 +864,16 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     if (last < 3) return;
     // stage 3: gate/up + SwiGLU, then fp16 parts of the activation rows
     const int gi = I > Is ? I : Is;
-    launch_gemm<PF_GEMM_GATE_UP>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
+    const bool iq2 = a.type[1] == PF_IQ2_XXS;
+    if (iq2) launch_gemm<PF_GEMM_GATE_UP, PF_IQ2_XXS>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
+    else launch_gemm<PF_GEMM_GATE_UP, PF_Q4_K>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(P), dim3(256), 0, stream, a.act, (size_t)I, I, (half_t *)a.act16, a.act_scale,
                        (float *)nullptr, a.error_word);
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.shared_act, (size_t)Is, Is,
                        (half_t *)a.sact16, a.sact_scale, (float *)nullptr, a.error_word);
     if (last < 4) return;
     // stage 4: down and combine
-    launch_gemm<PF_GEMM_DOWN>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
+    if (iq2) launch_gemm<PF_GEMM_DOWN, PF_IQ2_XXS>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
+    else launch_gemm<PF_GEMM_DOWN, PF_Q4_K>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
     hipLaunchKernelGGL(pf_k_pf_combine, dim3(tokens), dim3(256), 0, stream, a, tokens);
 }

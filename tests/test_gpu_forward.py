@@ -59,7 +59,7 @@ def test_decode_kernels_match_oracle_and_general_kernels(product, oracle, h, e, 
         assert_parity(y, ids, w, *want, label="general kernels on a decode shape")
 
 
-# shapes the matrix-core prefill kernels cover (Q4_K experts, widths in whole 256-blocks), more than 4 tokens
+# shapes the matrix-core prefill kernels cover (Q4_K or IQ2_XXS experts, widths in whole 256-blocks), more than 4 tokens
 PREFILL = [
     (256, 16, 4, 256, 256, 5), (256, 16, 4, 256, 256, 33), (512, 8, 3, 256, 512, 70),
     (256, 16, 4, 512, 256, 400),          # about 100 rows per expert: several passes of 64 rows
@@ -67,11 +67,12 @@ PREFILL = [
 ]
 
 
+@pytest.mark.parametrize("gtype", [abi.GGUF_Q4_K, abi.GGUF_IQ2_XXS])
 @pytest.mark.parametrize("h,e,k,i,s,tokens", PREFILL)
-def test_prefill_kernels_match_oracle_and_general_kernels(product, oracle, h, e, k, i, s, tokens):
-    print(f"case prefill h={h} e={e} k={k} i={i} s={s} T={tokens}", flush=True)
+def test_prefill_kernels_match_oracle_and_general_kernels(product, oracle, h, e, k, i, s, tokens, gtype):
+    print(f"case prefill type={gtype} h={h} e={e} k={k} i={i} s={s} T={tokens}", flush=True)
     cfg = abi.moe_config(h, e, k, i, s)
-    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, tokens, seed=h + e + tokens)
+    weights, x = make_layer_inputs(cfg, gtype, tokens, seed=h + e + tokens)
     want = forward_with(oracle, cfg, weights, x)
     with pf.MoeLayer(product, cfg, weights, tokens) as layer:
         _, y, ids, w = layer.forward(x)
@@ -134,12 +135,13 @@ def test_saturated_softmax_follows_the_reference_tie_rule(product, oracle):
         assert rel < 1e-4, rel
 
 
-def test_full_size_prefill_rows_match_oracle(product, oracle):
+@pytest.mark.parametrize("gtype", [abi.GGUF_Q4_K, abi.GGUF_IQ2_XXS])
+def test_full_size_prefill_rows_match_oracle(product, oracle, gtype):
     from picoforge_amd import workloads
     cfg = workloads.measured_config()
-    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 48, seed=5)
-    print("full-size prefill, 48 tokens", flush=True)
-    want = forward_with(oracle, cfg, weights, x[:6])      # the CPU path costs 0.14 s per token
+    weights, x = make_layer_inputs(cfg, gtype, 48, seed=5)
+    print(f"full-size prefill, 48 tokens, type={gtype}", flush=True)
+    want = forward_with(oracle, cfg, weights, x[:6])      # the CPU path costs 0.14 .. 0.26 s per token
     with pf.MoeLayer(product, cfg, weights, 48) as layer:
         _, y, ids, w = layer.forward(x)
         assert_parity(y[:6], ids[:6], w[:6], *want, label="full-size prefill")
