@@ -150,6 +150,31 @@ def test_full_size_prefill_rows_match_oracle(product, oracle, gtype):
         assert_parity(y, ids, w, yg, idsg, wg, label="prefill against general kernels, all 48 rows")
 
 
+LARGER_PREFILL = [
+    # hidden, experts, top_k, inter, shared_inter, tokens, expert type: shapes where a workgroup walks several
+    # work items, slabs are partial (768 = 256 + 512 rows ... ) and experts have many row tiles
+    (1024, 128, 8, 768, 256, 777, abi.GGUF_Q4_K),
+    (768, 24, 6, 1024, 512, 1500, abi.GGUF_Q4_K),
+    (1024, 64, 4, 512, 768, 901, abi.GGUF_IQ2_XXS),
+    (2048, 512, 10, 512, 512, 640, abi.GGUF_IQ2_XXS),
+]
+
+
+@pytest.mark.parametrize("h,e,k,i,s,tokens,gtype", LARGER_PREFILL)
+def test_prefill_kernels_match_general_kernels_on_larger_shapes(product, h, e, k, i, s, tokens, gtype):
+    """The matrix-core path against the FP32 dequantise-and-FMA kernels of the same library (written
+    independently; each is checked against the oracle on smaller shapes)."""
+    print(f"case larger prefill type={gtype} h={h} e={e} k={k} i={i} s={s} T={tokens}", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s)
+    weights, x = make_layer_inputs(cfg, gtype, tokens, seed=h + e + tokens)
+    with pf.MoeLayer(product, cfg, weights, tokens) as layer:
+        _, y, ids, w = layer.forward(x)
+        layer.force_general()
+        _, yg, idsg, wg = layer.forward(x)
+    worst = assert_parity(y, ids, w, yg, idsg, wg, label="prefill against general kernels")
+    print(f"  max abs difference {worst:.2e} of the bound", flush=True)
+
+
 @pytest.mark.parametrize("norm", [True, False])
 def test_decode_unnormalised_weights_and_repeat_calls(product, oracle, norm):
     cfg = abi.moe_config(512, 64, 4, 256, 256, norm=norm)
