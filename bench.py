@@ -59,7 +59,7 @@ WORKLOADS = {
 # WRITE_SIZE scaled by the same counters on a plain 256 MiB copy (profiles/*.txt hold the runs).
 # A counter result cannot be read live; None where no such run exists for the workload.
 MEASURED_TRAFFIC = {"iq2xxs_decode": 9832986, "q4k_decode": 19831587, "q4k_verify4": None,
-                    "q4k_prefill1024": 816922171}
+                    "q4k_prefill1024": 816855693, "iq2xxs_prefill1024": 448880069}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
