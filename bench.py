@@ -13,7 +13,10 @@ input, hence other experts.
 Workloads: iq2xxs_decode (default), q4k_decode, q4k_verify4 (4-token batches with
 about half of the experts shared between neighbours), q4k_prefill1024 and
 iq2xxs_prefill1024 (1024-token chunks, N(0,1) activations, Zipf(1.1) expert
-popularity), q4k_stack48 (48 resident layers, decode and 2048-token chunks).
+popularity), q4k_stack48 (48 resident layers, decode and 2048-token chunks), and
+iq2xxs_decode_hc / q4k_decode_hc / q4k_prefill1024_hc: the same layer between its two
+hyper-connection steps (gated read of 4 residual streams before, injection into them
+after), with the injection folded into the block's last kernel and as a kernel of its own.
 
 Prints one JSON line.  `value` is microseconds per layer per token (lower is
 better).  `roofline` is for the kernel that moves the most bytes, timed live
@@ -51,6 +54,13 @@ WORKLOADS = {
                             label="Q4_K experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
     "iq2xxs_prefill1024": dict(type=abi.GGUF_IQ2_XXS, tokens=1024, steps=100, warmup=10,
                                label="IQ2_XXS experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
+    "iq2xxs_decode_hc": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=10000, warmup=200, hc=4,
+                             label="IQ2_XXS experts, decode batch 1, between the HC read and add of 4 residual streams"),
+    "q4k_decode_hc": dict(type=abi.GGUF_Q4_K, tokens=1, steps=10000, warmup=200, hc=4,
+                          label="Q4_K experts, decode batch 1, between the HC read and add of 4 residual streams"),
+    "q4k_prefill1024_hc": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10, hc=4,
+                               label="Q4_K experts, 1024-token prefill chunk, between the HC read and add of 4 residual "
+                                     "streams, Zipf(1.1) expert popularity"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),
@@ -153,6 +163,117 @@ def run_stack(args, api, hip, cfg, steps, warmup):
         sys.exit("parity check failed on the sample")
 
 
+def run_hc(args, api, hip, cfg, wl, steps, warmup):
+    """One layer between its two hyper-connection steps (src/qwen4_forward.c:362-367): per step a gated read
+    of [tokens, streams, hidden] normed streams and gate logits, the MoE block, and the injection of the
+    block's output into the [tokens, streams, hidden] residual.  Timed three ways on resident buffers: the
+    chain with the injection folded into the block's last kernel (`value`), the chain with the injection as
+    a kernel of its own, and the block alone on the same mixed rows."""
+    tokens, streams, h = wl["tokens"], wl["hc"], cfg.hidden_size
+    t0 = time.time()
+    weights = pf.LayerWeights.synthetic(cfg, wl["type"], seed=args.seed)
+    if tokens > 4:
+        workloads.zipf_router(weights, seed=args.seed, temperature=0.18)
+    n_inputs = max(1, min(steps, 4 if tokens > 4 else 2000))
+    rng = np.random.default_rng(args.seed)
+    # streams whose gated mix has about unit RMS, as the block sees after the norm
+    normed = (rng.standard_normal((n_inputs, tokens, streams, h)) * (2.0 * streams ** 0.5 / 1.12)).astype(np.float32)
+    logits = rng.standard_normal((n_inputs, tokens, streams, h)).astype(np.float32)
+    residual = rng.standard_normal((tokens, streams, h)).astype(np.float32)
+    inject = rng.uniform(0.0, 2.0 / streams, (tokens, streams)).astype(np.float32)
+    # the timed loop adds into one residual thousands of times: weights scaled down so that it stays small
+    inject_timed = inject * np.float32(1e-3)
+    prep_s = time.time() - t0
+    layer = pf.MoeLayer(api, cfg, weights, tokens)
+    moe, work = layer.device_handles()
+    d_n, d_g, d_i = hip.to_device(normed), hip.to_device(logits), hip.to_device(inject_timed)
+    d_r = hip.to_device(residual)
+    ms = C.c_float()
+    timed = {}
+    for name, fused in (("fused", 1), ("separate_add", 0)):
+        hip.check(hip.memcpy_h2d(d_r, residual.ctypes.data, residual.nbytes), "residual")
+        hip.check(hip.moe_time_forwards_hc(moe, work, d_n, d_g, n_inputs, d_r, d_i, streams, tokens, warmup, fused,
+                                           C.byref(ms)), "warmup")
+        hip.check(hip.moe_time_forwards_hc(moe, work, d_n, d_g, n_inputs, d_r, d_i, streams, tokens, steps, fused,
+                                           C.byref(ms)), "timed loop")
+        timed[name] = ms.value / steps
+    err_word = int(hip.from_device(hip.work_error_word(work), (1,), np.uint32)[0])
+    # the block alone on the mixed rows the read produces
+    shape = abi.Qwen4HcShape(streams, h, 1, 1e-6)
+    mixed = np.empty((n_inputs, tokens, h), dtype=np.float32)
+    for b in range(n_inputs):
+        st = api.hc.read(C.byref(shape), abi.f32_cube(normed[b]), abi.f32_cube(logits[b]), abi.f32_view(mixed[b]), None)
+        assert st == abi.QW4_OK, st
+    d_x = hip.to_device(mixed)
+    d_y = hip.to_device(np.zeros((tokens, h), dtype=np.float32))
+    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, warmup, C.byref(ms)), "warmup")
+    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, steps, C.byref(ms)), "block alone")
+    block_ms = ms.value / steps
+
+    # parity on a bounded sample, stage by stage on identical inputs: CPU read against the device's mixed rows,
+    # CPU block on those rows, CPU add of its output; the device's chained call against that residual
+    ref = pf.load_reference()
+    cpu_api, kind = (ref, "reference") if ref is not None else (pf.load_oracle(), "port")
+    sample = min(tokens, args.cpu_sample or (24 if wl["type"] == abi.GGUF_IQ2_XXS else 40))
+    steps_cpu = 1 if tokens > 1 else min(sample, n_inputs)
+    rows = sample if tokens > 1 else 1
+    ids_equal = within = read_close = True
+    max_abs = 0.0
+    cpu_s = 0.0
+    with pf.MoeLayer(cpu_api, cfg, weights, rows) as cpu:
+        for b in range(steps_cpu):
+            n_b, g_b = normed[b][:rows], logits[b][:rows]
+            want = residual[:rows].copy()
+            c0 = time.perf_counter()
+            _, ids_c, _ = cpu.forward_hc(n_b, g_b, want, inject[:rows], fused=False)
+            cpu_s += time.perf_counter() - c0
+            # the same chain with the CPU block fed the device's mixed rows (identical inputs to every stage)
+            _, y_c, ids_m, _ = cpu.forward(mixed[b][:rows])
+            want_m = residual[:rows].copy()
+            cpu_api.hc.add(C.byref(shape), abi.f32_cube(want_m), abi.f32_view(y_c), abi.f32_view(inject[:rows]), None)
+            got = residual.copy()
+            _, ids_g, _ = layer.forward_hc(normed[b], logits[b], got, inject)
+            ids_equal &= bool((ids_g[:rows] == ids_m).all())
+            bound = np.abs(inject[:rows])[:, :, None] * (1e-3 + 1e-4 * np.abs(y_c)[:, None, :]) + 1e-6 * np.abs(want_m)
+            within &= bool((np.abs(got[:rows] - want_m) <= bound).all())
+            max_abs = max(max_abs, float(np.abs(got[:rows] - want_m).max()))
+            read_close &= bool(np.allclose(want, want_m, atol=1e-5, rtol=1e-5))
+    layer.close()
+    sample_tokens = steps_cpu * rows
+    ms_per_step = timed["fused"]
+    block, size = abi.BLOCK[wl["type"]]
+    hc_bytes = tokens * h * 4 * (2 * streams + 1) + tokens * h * 4 * 2 * streams   # read in/out, residual in/out
+    result = {
+        "metric": "moe_hc_block_us_per_layer_token", "value": round(ms_per_step * 1e3 / tokens, 3),
+        "unit": "us/layer/token", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if tokens <= 4 else "f16 products, f32 accumulation", "data": "synthetic",
+        "config": {"workload": f"one MoE layer, hidden 2048, 512 experts, top-10, intermediate 512, shared 512; "
+                               f"{wl['label']}; {n_inputs} seeded inputs",
+                   "tokens_per_step": tokens, "streams": streams,
+                   "expert_format": {12: "Q4_K", 16: "IQ2_XXS"}[wl["type"]]},
+        "chain_us_per_step": {"read + block with the add folded in": round(timed["fused"] * 1e3, 3),
+                              "read + block + add kernel": round(timed["separate_add"] * 1e3, 3),
+                              "block alone": round(block_ms * 1e3, 3)},
+        "hc_bytes_per_step": int(hc_bytes),
+        "roofline": {"bound": "hbm", "kernel": "the two hyper-connection steps: chain minus block alone",
+                     "achieved": round(hc_bytes / max((timed["fused"] - block_ms) * 1e-3, 1e-9) / 1e9, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(hc_bytes / max((timed["fused"] - block_ms) * 1e-3, 1e-9) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": None},
+        "cpu_baseline": {"value": round(cpu_s / sample_tokens * 1e6, 1), "unit": "us/layer/token", "cores": 1,
+                         "kind": kind, "sample": f"{sample_tokens} tokens of the same inputs through read, block and add, "
+                                                 f"{cpu_s:.1f} s"},
+        "parity_on_sample": {"ids_equal": ids_equal, "residual_within_block_tolerance_times_inject": within,
+                             "cpu_read_vs_device_read_chain_close": read_close, "max_abs_err": max_abs,
+                             "error_word": err_word},
+        "prep_s": round(prep_s, 1),
+    }
+    print(json.dumps(result))
+    if not (ids_equal and within and err_word == 0):
+        sys.exit("parity check failed on the sample")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -178,6 +299,8 @@ def main():
     cfg = workloads.measured_config()
     if args.workload == "q4k_stack48":
         return run_stack(args, api, hip, cfg, steps, warmup)
+    if wl.get("hc"):
+        return run_hc(args, api, hip, cfg, wl, steps, warmup)
     tokens = wl["tokens"]
     prefill = tokens > 4
     t0 = time.time()

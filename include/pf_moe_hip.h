@@ -93,6 +93,52 @@ int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x
                             uint32_t *ids, size_t ids_pitch_bytes, float *weights,
                             size_t weights_pitch_bytes, size_t tokens, uint32_t *error_word);
 
+/* The hyper-connection steps either side of the block (src/qwen4_base.c:142-175).
+ * Device forms: enqueue only, pitches in FLOATS (token pitch, then stream pitch of
+ * the [tokens, streams, hidden] cubes; row pitch of matrices); d_error_word is a
+ * device uint32 that receives PF_HIP_ERR_NONFINITE for a nonfinite input or result.
+ *   read: d_mixed[t, j] = (sum_h d_normed[t, h, j] * sigmoid(d_logits[t, h, j])) / streams
+ *   add:  d_residual[t, h, j] += d_inject[t, h] * d_block[t, j]   (bit-identical to the reference) */
+int pf_hip_hc_read_device(const float *d_normed, size_t n_token_pitch, size_t n_stream_pitch,
+                          const float *d_logits, size_t g_token_pitch, size_t g_stream_pitch,
+                          float *d_mixed, size_t m_pitch, size_t tokens, size_t streams,
+                          size_t hidden, uint32_t *d_error_word, void *stream);
+int pf_hip_hc_add_device(float *d_residual, size_t r_token_pitch, size_t r_stream_pitch,
+                         const float *d_block, size_t b_pitch, const float *d_inject,
+                         size_t i_pitch, size_t tokens, size_t streams, size_t hidden,
+                         uint32_t *d_error_word, void *stream);
+/* read -> forward -> add as one enqueue: the read fills the workspace's input rows and
+ * the forward's last kernel adds weight * output into every residual stream instead of
+ * writing an output matrix (the reference's device path fuses the add the same way,
+ * src/qwen4_moe_internal.h:55-58).  d_inject is dense [tokens, streams].  Allocates
+ * nothing, synchronises nothing; errors accumulate in the workspace's error word. */
+int pf_hip_moe_forward_hc_device(const PfHipMoe *moe, PfHipWork *work, const float *d_normed,
+                                 size_t n_token_pitch, size_t n_stream_pitch,
+                                 const float *d_logits, size_t g_token_pitch,
+                                 size_t g_stream_pitch, float *d_residual, size_t r_token_pitch,
+                                 size_t r_stream_pitch, const float *d_inject, size_t streams,
+                                 size_t tokens, void *stream);
+/* Host-buffer forms used by qwen4_hc_read, qwen4_hc_add and pf_moe_forward_hc: copy
+ * in, run, copy out; pitches in BYTES; outputs written only when the returned error
+ * word is zero. */
+int pf_hip_hc_read_host(const float *normed, size_t n_token_pitch_bytes,
+                        size_t n_stream_pitch_bytes, const float *logits,
+                        size_t g_token_pitch_bytes, size_t g_stream_pitch_bytes, float *mixed,
+                        size_t m_pitch_bytes, size_t tokens, size_t streams, size_t hidden,
+                        uint32_t *error_word);
+int pf_hip_hc_add_host(float *residual, size_t r_token_pitch_bytes, size_t r_stream_pitch_bytes,
+                       const float *block, size_t b_pitch_bytes, const float *inject,
+                       size_t i_pitch_bytes, size_t tokens, size_t streams, size_t hidden,
+                       uint32_t *error_word);
+int pf_hip_moe_forward_hc_host(const PfHipMoe *moe, PfHipWork *work, const float *normed,
+                               size_t n_token_pitch_bytes, size_t n_stream_pitch_bytes,
+                               const float *logits, size_t g_token_pitch_bytes,
+                               size_t g_stream_pitch_bytes, float *residual,
+                               size_t r_token_pitch_bytes, size_t r_stream_pitch_bytes,
+                               const float *inject, size_t i_pitch_bytes, size_t streams,
+                               size_t tokens, uint32_t *ids, size_t ids_pitch_bytes,
+                               float *weights, size_t weights_pitch_bytes, uint32_t *error_word);
+
 /* qwen4_moe_route on the device (src/qwen4_moe.c:188-249), reference evaluation
  * order.  Dense host arrays: logits/probs [tokens, experts], ids/weights
  * [tokens, top_k].  *bad_row receives the first row with a nonfinite logit when
@@ -132,6 +178,15 @@ int pf_hip_synchronize(void);
 int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
                              size_t n_inputs, float *d_y, size_t tokens, size_t iters,
                              float *elapsed_ms);
+
+/* The block between its two hyper-connection steps, `iters` times: input block
+ * i % n_inputs of d_normed / d_logits (dense [tokens, streams, hidden] each) and one
+ * residual cube.  fused != 0 runs pf_hip_moe_forward_hc_device; fused == 0 runs the
+ * read, a forward into the workspace and the add as three enqueues. */
+int pf_hip_moe_time_forwards_hc(const PfHipMoe *moe, PfHipWork *work, const float *d_normed,
+                                const float *d_logits, size_t n_inputs, float *d_residual,
+                                const float *d_inject, size_t streams, size_t tokens,
+                                size_t iters, int fused, float *elapsed_ms);
 
 /* The same for a stack of layers of equal hidden size (works[l] belongs to moes[l]):
  * forward i runs through layer i % layers with input row block i % n_inputs, so

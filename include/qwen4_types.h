@@ -4,7 +4,9 @@
  * src/qwen4_moe.h and src/qwen4_packed.h use: a translation unit of the
  * reference compiled against this header sees the same enum values and the
  * same struct layouts, so handles and views cross the boundary unchanged.
- * Types of other blocks (attention, n-gram, recurrent state) are not here. */
+ * Qwen4HcShape serves the two hyper-connection steps either side of the block
+ * (include/qwen4_hc.h).  Types of other blocks (attention, n-gram, recurrent
+ * state) are not here. */
 #ifndef PF_QWEN4_TYPES_H
 #define PF_QWEN4_TYPES_H
 #include <stdbool.h>
@@ -92,5 +94,15 @@ typedef struct {
     bool norm_topk_prob;
     uint32_t trunk_type[3];
 } Qwen4MoeConfig;
+
+/* Hyper-connection dimensions (src/qwen4_types.h:69): `streams` residual streams of
+ * `hidden_size` floats per token; low_rank and rms_eps belong to the gate's low-rank
+ * projection and are only validated here (nonzero, eps finite and positive). */
+typedef struct {
+    size_t streams;
+    size_t hidden_size;
+    size_t low_rank;
+    float rms_eps;
+} Qwen4HcShape;
 
 #endif

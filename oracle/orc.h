@@ -15,6 +15,7 @@
 #ifndef PF_ORACLE_H
 #define PF_ORACLE_H
 #include "../include/qwen4_moe.h"
+#include "../include/qwen4_hc.h"
 
 typedef struct OrcMoe OrcMoe;
 typedef struct OrcMoeWork OrcMoeWork;
@@ -50,4 +51,10 @@ void orc_moe_work_destroy(OrcMoeWork *);
 void orc_moe_observe(OrcMoeWork *, QW4MoeObserver, void *);
 Qwen4Status orc_moe_forward(const OrcMoe *, Qwen4F32 x, Qwen4F32Mut y, Qwen4MoeRoutes *optional_routes,
                             OrcMoeWork *, Qwen4Error *);
+/* src/qwen4_base.c:142-160 and :161-175: the hyper-connection read before the block
+ * and the injection after it */
+Qwen4Status orc_hc_read(const Qwen4HcShape *, Qwen4F32 normed, Qwen4F32 gate_logits, Qwen4F32Mut mixed,
+                        Qwen4Error *);
+Qwen4Status orc_hc_add(const Qwen4HcShape *, Qwen4F32Mut residual, Qwen4F32 block_out, Qwen4F32 inject,
+                       Qwen4Error *);
 #endif

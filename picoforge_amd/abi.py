@@ -1,4 +1,4 @@
-"""ctypes mirror of the C boundary (include/qwen4_types.h, qwen4_packed.h, qwen4_moe.h).
+"""ctypes mirror of the C boundary (include/qwen4_types.h, qwen4_packed.h, qwen4_moe.h, qwen4_hc.h).
 
 The same structures serve the shipped library, the CPU oracle and a build of the
 reference, since all three use the reference's layouts (src/qwen4_types.h,
@@ -46,6 +46,11 @@ class Qwen4MoeConfig(C.Structure):
                 ("intermediate", C.c_uint32), ("shared_intermediate", C.c_uint32),
                 ("down_physical", C.c_uint32), ("norm_topk_prob", C.c_bool),
                 ("trunk_type", C.c_uint32 * 3)]
+
+
+class Qwen4HcShape(C.Structure):   # src/qwen4_types.h:69
+    _fields_ = [("streams", C.c_size_t), ("hidden_size", C.c_size_t), ("low_rank", C.c_size_t),
+                ("rms_eps", C.c_float)]
 
 
 class GgufTensor(C.Structure):
@@ -106,6 +111,24 @@ def f32_view(array, rows=None, cols=None, pitch_bytes=None, capacity=None):
         pitch = array.shape[1] * 4
     v.stride_bytes[:] = (pitch, 4, 0, 0)
     v.capacity_bytes = (array.shape[0] * pitch) if capacity is None else capacity
+    return v
+
+
+def f32_cube(array, dims=None):
+    """View of a 3-D float32 numpy array [tokens, streams, hidden]; token and stream axes may be
+    pitched (a slice of a larger array), the last axis is contiguous.  dims overrides the
+    dimensions the view declares."""
+    assert array.dtype == np.float32 and array.ndim == 3 and (array.size == 0 or array.strides[2] == 4)
+    v = Qwen4F32()
+    v.data = array.ctypes.data if array.size else None
+    v.rank = 3
+    d = tuple(array.shape) if dims is None else tuple(dims)
+    v.dim[:] = d + (1,)
+    s1 = array.strides[1] if array.shape[1] > 1 and array.size else d[2] * 4
+    s0 = array.strides[0] if array.shape[0] > 1 and array.size else max(d[1], 1) * s1
+    v.stride_bytes[:] = (s0, s1, 4, 0)
+    v.capacity_bytes = 0 if not array.size else (array.shape[0] - 1) * s0 + (array.shape[1] - 1) * s1 + \
+        array.shape[2] * 4
     return v
 
 

@@ -72,23 +72,48 @@ class MoeApi:
                            abi.Qwen4F32Mut, P(E))
 
 
+class HcApi:
+    """The hyper-connection read and add either side of the block (include/qwen4_hc.h,
+    src/qwen4_ops.h:43-48) and, where the library has it, the chained read -> MoE -> add."""
+
+    def __init__(self, lib, prefix="qwen4_hc_"):
+        P, E, vp = C.POINTER, abi.Qwen4Error, C.c_void_p
+        S, V = P(abi.Qwen4HcShape), abi.Qwen4F32
+        self.read = getattr(lib, prefix + "read")
+        self.read.restype, self.read.argtypes = C.c_int, [S, V, V, V, P(E)]
+        self.add = getattr(lib, prefix + "add")
+        self.add.restype, self.add.argtypes = C.c_int, [S, V, V, V, P(E)]
+        if hasattr(lib, "pf_moe_forward_hc"):
+            self.forward_hc = lib.pf_moe_forward_hc
+            self.forward_hc.restype = C.c_int
+            self.forward_hc.argtypes = [vp, S, V, V, V, V, P(abi.Qwen4MoeRoutes), vp, P(E)]
+
+
 def load_product():
     lib = _open(PRODUCT_LIB)
     api = MoeApi(lib)
     api.hip = HipShim(lib)
+    api.hc = HcApi(lib)
     return api
 
 
 def load_oracle():
     """CPU oracle: test infrastructure (oracle/), never part of the product path."""
     lib = _open(REPO_DIR / "oracle" / "liborc.so")
-    return MoeApi(lib, moe_prefix="orc_moe_", private_prefix="orc_moe_", packed_prefix="orc_packed_")
+    api = MoeApi(lib, moe_prefix="orc_moe_", private_prefix="orc_moe_", packed_prefix="orc_packed_")
+    api.hc = HcApi(lib, prefix="orc_hc_")
+    return api
 
 
 def load_reference():
     """The reference's own C path, if oracle/_ref was built where the reference tree is mounted."""
     path = REPO_DIR / "oracle" / "_ref" / "libqwen4_ref.so"
-    return MoeApi(_open(path)) if path.exists() else None
+    if not path.exists():
+        return None
+    lib = _open(path)
+    api = MoeApi(lib)
+    api.hc = HcApi(lib)
+    return api
 
 
 class HipShim:
@@ -133,6 +158,10 @@ class HipShim:
         bind("pf_hip_moe_profile_stages", C.c_int, vp, vp, vp, sz, vp, sz, sz, P(C.c_float))
         bind("pf_hip_stack_time_forwards", C.c_int, P(vp), P(vp), sz, vp, sz, vp, sz, sz, P(C.c_float))
         bind("pf_hip_copy_probe", C.c_int, sz, sz)
+        bind("pf_hip_hc_read_device", C.c_int, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, vp, vp)
+        bind("pf_hip_hc_add_device", C.c_int, vp, sz, sz, vp, sz, vp, sz, sz, sz, sz, vp, vp)
+        bind("pf_hip_moe_forward_hc_device", C.c_int, vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp)
+        bind("pf_hip_moe_time_forwards_hc", C.c_int, vp, vp, vp, vp, sz, vp, vp, sz, sz, sz, C.c_int, P(C.c_float))
 
     def check(self, rc, what):
         if rc != 0:

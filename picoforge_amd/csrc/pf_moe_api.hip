@@ -384,17 +384,22 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     return a;
 }
 
-// Enqueue only: no allocation, no synchronisation, no memset; safe under stream capture.
-extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch,
-                                         float *d_y, size_t y_pitch, size_t tokens, void *stream) {
-    if (!moe || !work || work->moe != moe) return PF_HIP_E_ARGUMENT;
-    if (tokens > work->cap) return PF_HIP_E_ARGUMENT;
-    if (tokens == 0) return PF_HIP_OK;
-    if (!d_x || !d_y || x_pitch < moe->desc.hidden || y_pitch < moe->desc.hidden) return PF_HIP_E_ARGUMENT;
+struct HcTarget {   // residual streams to inject into instead of writing y
+    float *residual;
+    size_t token_pitch, stream_pitch;
+    const float *inject;
+    int streams;
+};
+
+static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch, float *d_y,
+                           size_t y_pitch, size_t tokens, const HcTarget *hc, hipStream_t s) {
     const PfHipMoeDesc *d = &moe->desc;
     if (tokens * (size_t)d->top_k > 0x7fffffffu / 4) return PF_HIP_E_UNSUPPORTED;
-    hipStream_t s = (hipStream_t)stream;
     PfKernelArgs a = make_args(moe, work, d_x, x_pitch, d_y, y_pitch);
+    if (hc) {
+        a.hc_residual = hc->residual; a.hc_inject = hc->inject; a.hc_streams = hc->streams;
+        a.hc_token_pitch = hc->token_pitch; a.hc_stream_pitch = hc->stream_pitch;
+    }
     const bool aligned = (x_pitch % 4 == 0) && ((uintptr_t)d_x % 16 == 0);
     if (moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS && aligned && !work->force_general) {
         pf_launch_decode(a, (int)tokens, s, work->stage_limit);
@@ -411,6 +416,70 @@ extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, c
     }
     HIP_TRY(hipGetLastError());
     return PF_HIP_OK;
+}
+
+// Enqueue only: no allocation, no synchronisation, no memset; safe under stream capture.
+extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch,
+                                         float *d_y, size_t y_pitch, size_t tokens, void *stream) {
+    if (!moe || !work || work->moe != moe) return PF_HIP_E_ARGUMENT;
+    if (tokens > work->cap) return PF_HIP_E_ARGUMENT;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!d_x || !d_y || x_pitch < moe->desc.hidden || y_pitch < moe->desc.hidden) return PF_HIP_E_ARGUMENT;
+    return forward_enqueue(moe, work, d_x, x_pitch, d_y, y_pitch, tokens, nullptr, (hipStream_t)stream);
+}
+
+// ---- hyper-connection read and add (src/qwen4_base.c:142-175) -----------------------------------
+static bool hc_dims_ok(size_t tokens, size_t streams, size_t hidden) {
+    return streams && hidden && tokens <= 0x7fffffffu && streams <= 0x7fffffffu && hidden <= 0x7fffffffu;
+}
+
+extern "C" int pf_hip_hc_read_device(const float *d_normed, size_t n_token_pitch, size_t n_stream_pitch,
+                                     const float *d_logits, size_t g_token_pitch, size_t g_stream_pitch,
+                                     float *d_mixed, size_t m_pitch, size_t tokens, size_t streams, size_t hidden,
+                                     uint32_t *d_error_word, void *stream) {
+    if (!hc_dims_ok(tokens, streams, hidden) || !d_error_word) return PF_HIP_E_ARGUMENT;
+    if (!tokens) return PF_HIP_OK;
+    if (!d_normed || !d_logits || !d_mixed || n_stream_pitch < hidden || g_stream_pitch < hidden || m_pitch < hidden)
+        return PF_HIP_E_ARGUMENT;
+    pf_launch_hc_read(d_normed, n_token_pitch, n_stream_pitch, d_logits, g_token_pitch, g_stream_pitch, d_mixed,
+                      m_pitch, (int)tokens, (int)streams, (int)hidden, d_error_word, (hipStream_t)stream);
+    HIP_TRY(hipGetLastError());
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_hc_add_device(float *d_residual, size_t r_token_pitch, size_t r_stream_pitch,
+                                    const float *d_block, size_t b_pitch, const float *d_inject, size_t i_pitch,
+                                    size_t tokens, size_t streams, size_t hidden, uint32_t *d_error_word,
+                                    void *stream) {
+    if (!hc_dims_ok(tokens, streams, hidden) || !d_error_word) return PF_HIP_E_ARGUMENT;
+    if (!tokens) return PF_HIP_OK;
+    if (!d_residual || !d_block || !d_inject || r_stream_pitch < hidden || b_pitch < hidden || i_pitch < streams)
+        return PF_HIP_E_ARGUMENT;
+    pf_launch_hc_add(d_residual, r_token_pitch, r_stream_pitch, d_block, b_pitch, d_inject, i_pitch, (int)tokens,
+                     (int)streams, (int)hidden, d_error_word, (hipStream_t)stream);
+    HIP_TRY(hipGetLastError());
+    return PF_HIP_OK;
+}
+
+// Enqueue only, like pf_hip_moe_forward_device: the read writes the workspace's input rows, the
+// forward consumes them and its last kernel adds into the residual streams.
+extern "C" int pf_hip_moe_forward_hc_device(const PfHipMoe *moe, PfHipWork *work, const float *d_normed,
+                                            size_t n_token_pitch, size_t n_stream_pitch, const float *d_logits,
+                                            size_t g_token_pitch, size_t g_stream_pitch, float *d_residual,
+                                            size_t r_token_pitch, size_t r_stream_pitch, const float *d_inject,
+                                            size_t streams, size_t tokens, void *stream) {
+    if (!moe || !work || work->moe != moe || tokens > work->cap) return PF_HIP_E_ARGUMENT;
+    const size_t H = moe->desc.hidden;
+    if (!hc_dims_ok(tokens, streams, H)) return PF_HIP_E_ARGUMENT;
+    if (!tokens) return PF_HIP_OK;
+    if (!d_normed || !d_logits || !d_residual || !d_inject || n_stream_pitch < H || g_stream_pitch < H ||
+        r_stream_pitch < H)
+        return PF_HIP_E_ARGUMENT;
+    hipStream_t s = (hipStream_t)stream;
+    pf_launch_hc_read(d_normed, n_token_pitch, n_stream_pitch, d_logits, g_token_pitch, g_stream_pitch, work->x, H,
+                      (int)tokens, (int)streams, (int)H, work->error_word, s);
+    const HcTarget hc = {d_residual, r_token_pitch, r_stream_pitch, d_inject, (int)streams};
+    return forward_enqueue(moe, work, work->x, H, work->y, H, tokens, &hc, s);
 }
 
 extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
@@ -444,6 +513,120 @@ struct DeviceBlock {   // one allocation, freed on scope exit
     uint8_t *p = nullptr;
     ~DeviceBlock() { if (p) (void)hipFree(p); }
 };
+
+// A [tokens, streams, hidden] cube between host memory (byte pitches) and a dense device array.
+static hipError_t copy_cube(void *dense, void *host, size_t token_pitch, size_t stream_pitch, size_t T, size_t S,
+                            size_t H, bool to_device) {
+    const size_t row = H * 4;
+    const hipMemcpyKind kind = to_device ? hipMemcpyHostToDevice : hipMemcpyDeviceToHost;
+    if (T == 1 || S == 1 || token_pitch == S * stream_pitch) {   // one pitch describes every row
+        const size_t pitch = S == 1 ? token_pitch : stream_pitch;
+        return to_device ? hipMemcpy2D(dense, row, host, pitch, row, T * S, kind)
+                         : hipMemcpy2D(host, pitch, dense, row, row, T * S, kind);
+    }
+    for (size_t t = 0; t < T; t++) {
+        uint8_t *h = (uint8_t *)host + t * token_pitch, *d = (uint8_t *)dense + t * S * row;
+        const hipError_t e = to_device ? hipMemcpy2D(d, row, h, stream_pitch, row, S, kind)
+                                       : hipMemcpy2D(h, stream_pitch, d, row, row, S, kind);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+static size_t pad256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+extern "C" int pf_hip_hc_read_host(const float *normed, size_t n_token_pitch_bytes, size_t n_stream_pitch_bytes,
+                                   const float *logits, size_t g_token_pitch_bytes, size_t g_stream_pitch_bytes,
+                                   float *mixed, size_t m_pitch_bytes, size_t tokens, size_t streams, size_t hidden,
+                                   uint32_t *error_word) {
+    if (!error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (!hc_dims_ok(tokens, streams, hidden)) return PF_HIP_E_ARGUMENT;
+    if (!tokens) return PF_HIP_OK;
+    if (!normed || !logits || !mixed) return PF_HIP_E_ARGUMENT;
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
+    const size_t cube = pad256(tokens * streams * hidden * 4), out = pad256(tokens * hidden * 4);
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, 2 * cube + out + 256));
+    float *d_n = (float *)blk.p, *d_g = (float *)(blk.p + cube), *d_m = (float *)(blk.p + 2 * cube);
+    uint32_t *d_err = (uint32_t *)(blk.p + 2 * cube + out);
+    HIP_TRY(copy_cube(d_n, (void *)normed, n_token_pitch_bytes, n_stream_pitch_bytes, tokens, streams, hidden, true));
+    HIP_TRY(copy_cube(d_g, (void *)logits, g_token_pitch_bytes, g_stream_pitch_bytes, tokens, streams, hidden, true));
+    HIP_TRY(hipMemset(d_err, 0, 256));
+    pf_launch_hc_read(d_n, streams * hidden, hidden, d_g, streams * hidden, hidden, d_m, hidden, (int)tokens,
+                      (int)streams, (int)hidden, d_err, nullptr);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, d_err, 4, hipMemcpyDeviceToHost));
+    if (*error_word) return PF_HIP_OK;
+    HIP_TRY(hipMemcpy2D(mixed, m_pitch_bytes, d_m, hidden * 4, hidden * 4, tokens, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_hc_add_host(float *residual, size_t r_token_pitch_bytes, size_t r_stream_pitch_bytes,
+                                  const float *block, size_t b_pitch_bytes, const float *inject,
+                                  size_t i_pitch_bytes, size_t tokens, size_t streams, size_t hidden,
+                                  uint32_t *error_word) {
+    if (!error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (!hc_dims_ok(tokens, streams, hidden)) return PF_HIP_E_ARGUMENT;
+    if (!tokens) return PF_HIP_OK;
+    if (!residual || !block || !inject) return PF_HIP_E_ARGUMENT;
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
+    const size_t cube = pad256(tokens * streams * hidden * 4), rows = pad256(tokens * hidden * 4),
+                 gates = pad256(tokens * streams * 4);
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, cube + rows + gates + 256));
+    float *d_r = (float *)blk.p, *d_b = (float *)(blk.p + cube), *d_i = (float *)(blk.p + cube + rows);
+    uint32_t *d_err = (uint32_t *)(blk.p + cube + rows + gates);
+    HIP_TRY(copy_cube(d_r, residual, r_token_pitch_bytes, r_stream_pitch_bytes, tokens, streams, hidden, true));
+    HIP_TRY(hipMemcpy2D(d_b, hidden * 4, block, b_pitch_bytes, hidden * 4, tokens, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy2D(d_i, streams * 4, inject, i_pitch_bytes, streams * 4, tokens, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(d_err, 0, 256));
+    pf_launch_hc_add(d_r, streams * hidden, hidden, d_b, hidden, d_i, streams, (int)tokens, (int)streams, (int)hidden,
+                     d_err, nullptr);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, d_err, 4, hipMemcpyDeviceToHost));
+    if (*error_word) return PF_HIP_OK;
+    HIP_TRY(copy_cube(d_r, residual, r_token_pitch_bytes, r_stream_pitch_bytes, tokens, streams, hidden, false));
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_moe_forward_hc_host(const PfHipMoe *moe, PfHipWork *work, const float *normed,
+                                          size_t n_token_pitch_bytes, size_t n_stream_pitch_bytes,
+                                          const float *logits, size_t g_token_pitch_bytes,
+                                          size_t g_stream_pitch_bytes, float *residual, size_t r_token_pitch_bytes,
+                                          size_t r_stream_pitch_bytes, const float *inject, size_t i_pitch_bytes,
+                                          size_t streams, size_t tokens, uint32_t *ids, size_t ids_pitch_bytes,
+                                          float *weights, size_t weights_pitch_bytes, uint32_t *error_word) {
+    if (!moe || !work || !error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    const size_t H = moe->desc.hidden, K = moe->desc.top_k;
+    if (!hc_dims_ok(tokens, streams, H) || tokens > work->cap) return PF_HIP_E_ARGUMENT;
+    if (!tokens) return PF_HIP_OK;
+    if (!normed || !logits || !residual || !inject) return PF_HIP_E_ARGUMENT;
+    const size_t cube = pad256(tokens * streams * H * 4), gates = pad256(tokens * streams * 4);
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, 3 * cube + gates));
+    float *d_n = (float *)blk.p, *d_g = (float *)(blk.p + cube), *d_r = (float *)(blk.p + 2 * cube),
+          *d_i = (float *)(blk.p + 3 * cube);
+    HIP_TRY(copy_cube(d_n, (void *)normed, n_token_pitch_bytes, n_stream_pitch_bytes, tokens, streams, H, true));
+    HIP_TRY(copy_cube(d_g, (void *)logits, g_token_pitch_bytes, g_stream_pitch_bytes, tokens, streams, H, true));
+    HIP_TRY(copy_cube(d_r, residual, r_token_pitch_bytes, r_stream_pitch_bytes, tokens, streams, H, true));
+    HIP_TRY(hipMemcpy2D(d_i, streams * 4, inject, i_pitch_bytes, streams * 4, tokens, hipMemcpyHostToDevice));
+    int rc = pf_hip_moe_forward_hc_device(moe, work, d_n, streams * H, H, d_g, streams * H, H, d_r, streams * H, H,
+                                          d_i, streams, tokens, nullptr);
+    if (rc != PF_HIP_OK) return rc;
+    HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
+    if (*error_word) {
+        HIP_TRY(hipMemset(work->error_word, 0, 4));   // the word is sticky on the device; reading it clears it
+        return PF_HIP_OK;
+    }
+    HIP_TRY(copy_cube(d_r, residual, r_token_pitch_bytes, r_stream_pitch_bytes, tokens, streams, H, false));
+    if (ids) HIP_TRY(hipMemcpy2D(ids, ids_pitch_bytes, work->ids, K * 4, K * 4, tokens, hipMemcpyDeviceToHost));
+    if (weights)
+        HIP_TRY(hipMemcpy2D(weights, weights_pitch_bytes, work->route_weights, K * 4, K * 4, tokens,
+                            hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
 
 extern "C" int pf_hip_route_host(const float *logits, size_t tokens, size_t experts, size_t top_k, int norm_topk,
                                  float *probs, uint32_t *ids, float *weights, uint32_t *error_word,
@@ -604,11 +787,12 @@ extern "C" int pf_hip_synchronize(void) {
 // up to 256 forwards (each with its own input block) and the graphs are replayed in order,
 // so the measured gap between dependent kernels is the device's, not the host's enqueue rate.
 // Forward i goes through layer i % layers (a stack of layers in order, token after token).
-static int time_graph_replay(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers, const float *d_x,
-                             size_t n_inputs, float *d_y, size_t tokens, size_t iters, int stage_limit, float *elapsed_ms) {
+template <typename Enqueue>
+static int time_graph_replay_of(PfHipWork *const *works, size_t layers, size_t iters, int stage_limit,
+                                float *elapsed_ms, Enqueue enqueue) {
     *elapsed_ms = 0.0f;
     if (!iters) return PF_HIP_OK;
-    const size_t H = moes[0]->desc.hidden, chunk = 256, n_graphs = (iters + chunk - 1) / chunk;
+    const size_t chunk = 256, n_graphs = (iters + chunk - 1) / chunk;
     hipStream_t s = nullptr;
     hipEvent_t t0 = nullptr, t1 = nullptr;
     HIP_TRY(hipStreamCreate(&s));
@@ -619,8 +803,7 @@ static int time_graph_replay(const PfHipMoe *const *moes, PfHipWork *const *work
         hipGraph_t graph = nullptr;
         if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) { rc = PF_HIP_E_RUNTIME; break; }
         for (size_t i = g * chunk; i < iters && i < (g + 1) * chunk && rc == PF_HIP_OK; i++)
-            rc = pf_hip_moe_forward_device(moes[i % layers], works[i % layers], d_x + (i % n_inputs) * tokens * H, H, d_y, H,
-                                           tokens, s);
+            rc = enqueue(i, s);
         hipError_t e = hipStreamEndCapture(s, &graph);
         if (e != hipSuccess && rc == PF_HIP_OK) { pf_set_error("hipStreamEndCapture", e); rc = PF_HIP_E_RUNTIME; }
         if (rc == PF_HIP_OK && hipGraphInstantiate(&execs[g], graph, nullptr, nullptr, 0) != hipSuccess)
@@ -643,6 +826,42 @@ static int time_graph_replay(const PfHipMoe *const *moes, PfHipWork *const *work
     if (t1) (void)hipEventDestroy(t1);
     (void)hipStreamDestroy(s);
     return rc;
+}
+
+static int time_graph_replay(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers, const float *d_x,
+                             size_t n_inputs, float *d_y, size_t tokens, size_t iters, int stage_limit, float *elapsed_ms) {
+    const size_t H = moes[0]->desc.hidden;
+    return time_graph_replay_of(works, layers, iters, stage_limit, elapsed_ms, [&](size_t i, hipStream_t s) {
+        return pf_hip_moe_forward_device(moes[i % layers], works[i % layers], d_x + (i % n_inputs) * tokens * H, H, d_y, H,
+                                         tokens, s);
+    });
+}
+
+// The block between its two hyper-connection steps, `iters` times back to back: input block
+// i % n_inputs of d_normed / d_logits (dense [tokens, streams, hidden] each), one residual cube.
+// fused != 0: read, then a forward whose last kernel adds into the residual.  fused == 0: read,
+// forward into the workspace's output rows, then the add as a kernel of its own.
+extern "C" int pf_hip_moe_time_forwards_hc(const PfHipMoe *moe, PfHipWork *work, const float *d_normed,
+                                           const float *d_logits, size_t n_inputs, float *d_residual,
+                                           const float *d_inject, size_t streams, size_t tokens, size_t iters,
+                                           int fused, float *elapsed_ms) {
+    if (!moe || !work || work->moe != moe || !d_normed || !d_logits || !d_residual || !d_inject || !n_inputs ||
+        !elapsed_ms || !streams || tokens > work->cap)
+        return PF_HIP_E_ARGUMENT;
+    const size_t H = moe->desc.hidden, cube = tokens * streams * H;
+    return time_graph_replay_of(&work, 1, iters, 0, elapsed_ms, [&](size_t i, hipStream_t s) {
+        const float *n = d_normed + (i % n_inputs) * cube, *g = d_logits + (i % n_inputs) * cube;
+        if (fused)
+            return pf_hip_moe_forward_hc_device(moe, work, n, streams * H, H, g, streams * H, H, d_residual,
+                                                streams * H, H, d_inject, streams, tokens, s);
+        int rc = pf_hip_hc_read_device(n, streams * H, H, g, streams * H, H, work->x, H, tokens, streams, H,
+                                       work->error_word, s);
+        if (rc == PF_HIP_OK) rc = pf_hip_moe_forward_device(moe, work, work->x, H, work->y, H, tokens, s);
+        if (rc == PF_HIP_OK)
+            rc = pf_hip_hc_add_device(d_residual, streams * H, H, work->y, H, d_inject, streams, tokens, streams, H,
+                                      work->error_word, s);
+        return rc;
+    });
 }
 
 extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,

@@ -560,8 +560,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_bl
         for (int slot = 0; slot < 16; slot++)   // slot order, as src/qwen4_moe.c:362-372
             if (slot < K) sum += rw[slot] * partial[slot][threadIdx.x];
         const float y = sum + shared_scale * partial[K][threadIdx.x];
-        a.y[(size_t)t * a.y_pitch + n] = y;
-        if (!pf_finite(y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        if (!pf_emit_output(a, t, n, y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
 }
 

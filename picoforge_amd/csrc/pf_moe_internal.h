@@ -41,7 +41,33 @@ struct PfKernelArgs {
     const float *w_norm2;            // [experts] squared norm of each router row
     float *down;                     // [pairs + tokens, hidden] down products in expert order, then the shared expert's
     uint32_t *counts, *offsets, *pair_to_row, *row_to_pair, *group_bad, *tiles;
+    // injection into hyper-connection streams in place of writing y (null: y is written)
+    float *hc_residual;              // [tokens, streams, hidden], pitches in floats
+    const float *hc_inject;          // [tokens, streams], dense
+    size_t hc_token_pitch, hc_stream_pitch;
+    int hc_streams;
 };
+
+// One finished element of the block's output.  Normally y[t, n]; when the forward injects into the
+// residual streams, residual[t, h, n] += inject[t, h] * value for every stream h, product and sum
+// each rounded (src/qwen4_base.c:168-173).  Returns false if anything written is not finite.
+__device__ __forceinline__ bool pf_emit_output(const PfKernelArgs &a, int t, int n, float value) {
+#pragma clang fp contract(off)
+    if (!a.hc_residual) {
+        a.y[(size_t)t * a.y_pitch + n] = value;
+        return pf_finite(value);
+    }
+    bool ok = true;
+    float *r = a.hc_residual + (size_t)t * a.hc_token_pitch + n;
+    const float *w = a.hc_inject + (size_t)t * a.hc_streams;
+    for (int h = 0; h < a.hc_streams; h++) {
+        const float product = w[h] * value;
+        const float result = r[(size_t)h * a.hc_stream_pitch] + product;
+        r[(size_t)h * a.hc_stream_pitch] = result;
+        ok &= pf_finite(result);
+    }
+    return ok;
+}
 
 struct PfHipMoe {
     PfHipMoeDesc desc;
@@ -103,6 +129,13 @@ void pf_launch_q4k_tile(const uint8_t *d_src, uint8_t *d_dst, size_t rows, int b
 void pf_launch_row_norm2(const float *d_w, int rows, int cols, float *d_out, hipStream_t stream);
 size_t pf_prefill_half_row(int cols);   // halfs per row of the fp16 form of a matrix with `cols` columns
 int pf_prefill_max_tiles(int tokens, int experts, int top_k);
+// pf_moe_hc.hip
+void pf_launch_hc_read(const float *d_normed, size_t n_token_pitch, size_t n_stream_pitch, const float *d_logits,
+                       size_t g_token_pitch, size_t g_stream_pitch, float *d_mixed, size_t m_pitch, int tokens,
+                       int streams, int hidden, uint32_t *d_error, hipStream_t stream);
+void pf_launch_hc_add(float *d_residual, size_t r_token_pitch, size_t r_stream_pitch, const float *d_block,
+                      size_t b_pitch, const float *d_inject, size_t i_pitch, int tokens, int streams, int hidden,
+                      uint32_t *d_error, hipStream_t stream);
 // pf_moe_api.hip
 const uint64_t *pf_device_iq2_grid(void);
 const uint32_t *pf_device_iq2_signed(void);

@@ -221,8 +221,7 @@ __global__ void __launch_bounds__(256) pf_k_down_combine(PfKernelArgs a) {
     float sh = dot_tensor_row(a, 6, 0, n, sact, lane, grid);
     float y = sum + a.shared_scale[t] * sh;
     if (lane == 0) {
-        a.y[(size_t)t * a.y_pitch + n] = y;
-        if (!pf_finite(y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        if (!pf_emit_output(a, t, n, y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
 }
 

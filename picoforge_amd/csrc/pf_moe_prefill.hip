@@ -808,8 +808,7 @@ __global__ void __launch_bounds__(256) pf_k_pf_combine(PfKernelArgs a, int token
             sum += term;
         }
         const float y = sum + ss * a.down[(size_t)(P + t) * H + c];
-        bad |= !pf_finite(y);
-        a.y[(size_t)t * a.y_pitch + c] = y;
+        bad |= !pf_emit_output(a, t, c, y);
     }
     if (__any(bad) && pf_lane() == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
 }

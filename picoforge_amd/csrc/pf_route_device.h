@@ -89,7 +89,8 @@ __device__ __forceinline__ void pf_route_exact_wave(const float *z, float *p, fl
             if (v > best) { best = v; best_id = (uint32_t)e; }
         }
         pf_wave_argmax(best, best_id);
-        if ((int)(best_id & (PF_WAVE - 1)) == lane) q[best_id] = -1.0f;
+        // no candidate at all (every probability NaN): nothing to strike out, the id stays out of range
+        if (best_id != 0xffffffffu && (int)(best_id & (PF_WAVE - 1)) == lane) q[best_id] = -1.0f;
         pf_wave_lds_fence();
         chosen = chosen + best;
         if ((slot & (PF_WAVE - 1)) == lane) { mine = best; mine_id = best_id; }   // lane r keeps slots r, r + 64, ...

@@ -4,7 +4,9 @@
  * arithmetic is done by the HIP kernels behind include/pf_moe_hip.h; there is no
  * CPU fallback: without a device every compute entry point fails. */
 #include "../../include/qwen4_moe.h"
+#include "../../include/qwen4_hc.h"
 #include "../../include/pf_moe_hip.h"
+#include "pf_hc_host.h"
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -347,6 +349,64 @@ Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen
         memcpy(out.dim, y.dim, sizeof out.dim);
         memcpy(out.stride_bytes, y.stride_bytes, sizeof out.stride_bytes);
         w->observer(w->observer_ctx, 12, SIZE_MAX, 0, x, out);
+    }
+    return moe_status(err, QW4_OK, "");
+}
+
+/* ---- the block between its two hyper-connection steps (src/qwen4_forward.c:362-367) ------------
+ * Validation in the order of the three calls it stands for: the read's views, the forward's
+ * handles and routes, the add's views.  The arithmetic and the finite checks run on the device;
+ * the residual is written back only when the error word stayed clear. */
+Qwen4Status pf_moe_forward_hc(const Qwen4Moe *m, const Qwen4HcShape *s, Qwen4F32 normed, Qwen4F32 logits,
+                              Qwen4F32Mut residual, Qwen4F32 inject, Qwen4MoeRoutes *routes, Qwen4MoeWork *w,
+                              Qwen4Error *err) {
+    TRY(pf_hc_admit_shape(s, err));
+    size_t span[2], rspan;
+    TRY(pf_hc_admit_read_inputs(s, normed, logits, span, err));
+    if (!m || !w) return moe_status(err, QW4_INVALID_ARGUMENT, "null forward handle");
+    if (w->owner != m) return moe_status(err, QW4_OWNER, "workspace belongs to another MoE");
+    if (!m->alive || w->failed) return moe_status(err, QW4_BAD_STATE, "inactive MoE/workspace; reset required");
+    if (w->busy) return moe_status(err, QW4_BUSY, "workspace executing");
+    const size_t T = normed.dim[0], H = m->cfg.hidden_size, K = m->cfg.top_k;
+    if (s->hidden_size != H) return moe_status(err, QW4_SHAPE, "HC hidden size differs from the MoE's");
+    if (T > w->cap) return moe_status(err, QW4_CAPACITY, "batch exceeds token capacity");
+    Range r[5];
+    size_t nr = 0;
+    if (routes) {
+        TRY(RANGE_F32(routes->weights, T, K, &r[0]));
+        if (routes->ids.rows != T || routes->ids.cols != K)
+            return moe_status(err, QW4_SHAPE, "optional route shape mismatch");
+        TRY(range_rows(routes->ids.data, routes->ids.capacity_bytes, T, K, routes->ids.row_stride_bytes, &r[1], err));
+        nr = 2;
+    }
+    if (residual.dim[0] != T) return moe_status(err, QW4_SHAPE, "residual token count differs from the input's");
+    TRY(pf_hc_admit_add(s, residual, NULL, 0, inject, &rspan, err));
+    r[nr++] = (Range){(uintptr_t)residual.data, (uintptr_t)residual.data + rspan};
+    r[nr++] = (Range){(uintptr_t)normed.data, (uintptr_t)normed.data + span[0]};
+    r[nr++] = (Range){(uintptr_t)logits.data, (uintptr_t)logits.data + span[1]};
+    /* outputs (routes, residual) may not overlap each other or any input; the two read inputs may
+     * share memory with each other, as they may for qwen4_hc_read */
+    for (size_t i = 0; i + 2 < nr; i++)
+        for (size_t j = i + 1; j < nr; j++)
+            if (r[i].lo < r[j].hi && r[j].lo < r[i].hi)
+                return moe_status(err, QW4_INVALID_ARGUMENT, "overlapping views");
+    if (!T) return moe_status(err, QW4_OK, "");
+    w->busy = true;
+    uint32_t word = 0;
+    int rc = pf_hip_moe_forward_hc_host(m->device, w->device, normed.data, normed.stride_bytes[0],
+                                        normed.stride_bytes[1], logits.data, logits.stride_bytes[0],
+                                        logits.stride_bytes[1], residual.data, residual.stride_bytes[0],
+                                        residual.stride_bytes[1], inject.data, inject.stride_bytes[0], s->streams, T,
+                                        routes ? routes->ids.data : NULL, routes ? routes->ids.row_stride_bytes : 0,
+                                        routes ? routes->weights.data : NULL,
+                                        routes ? routes->weights.stride_bytes[0] : 0, &word);
+    w->busy = false;
+    if (rc || word) {
+        w->failed = true;
+        if (rc) return pf_device_status(rc, err, "qwen4_moe");
+        if (word & PF_HIP_ERR_NONFINITE)
+            return moe_status(err, QW4_NONFINITE, "nonfinite value in the hyper-connection steps or the MoE block");
+        return moe_status(err, QW4_GPU_ERROR, "device error word");
     }
     return moe_status(err, QW4_OK, "");
 }

@@ -95,6 +95,39 @@ class MoeLayer:
             self._raise(st)
         return st, y, ids, w
 
+    def forward_hc(self, normed, logits, residual, inject, fused=None, check=True, low_rank=1, eps=1e-6):
+        """The block between its two hyper-connection steps, as layer_cpu runs them
+        (src/qwen4_forward.c:362-367): read [T, S, H] -> MoE -> add into residual [T, S, H] in place.
+        fused=None uses the library's single call where it has one (the shipped library), the three
+        calls otherwise (the CPU oracle, a build of the reference).  Returns (status, ids, weights)."""
+        t, s, h = normed.shape
+        k = self.cfg.top_k
+        shape = abi.Qwen4HcShape(s, h, low_rank, eps)
+        ids = np.full((t, k), 0xFFFFFFFF, dtype=np.uint32)
+        w = np.full((t, k), -99.0, dtype=np.float32)
+        routes = abi.Qwen4MoeRoutes(abi.u32_view(ids), abi.f32_view(w))
+        hc = self.api.hc
+        if fused is None:
+            fused = hasattr(hc, "forward_hc")
+        if fused:
+            st = hc.forward_hc(self.handle, C.byref(shape), abi.f32_cube(normed), abi.f32_cube(logits),
+                               abi.f32_cube(residual), abi.f32_view(inject), C.byref(routes), self.work,
+                               C.byref(self.err))
+        else:
+            mixed = np.full((t, h), -99.0, dtype=np.float32)
+            block = np.full((t, h), -99.0, dtype=np.float32)
+            st = hc.read(C.byref(shape), abi.f32_cube(normed), abi.f32_cube(logits), abi.f32_view(mixed),
+                         C.byref(self.err))
+            if st == abi.QW4_OK:
+                st = self.api.forward(self.handle, abi.f32_view(mixed), abi.f32_view(block), C.byref(routes),
+                                      self.work, C.byref(self.err))
+            if st == abi.QW4_OK:
+                st = hc.add(C.byref(shape), abi.f32_cube(residual), abi.f32_view(block), abi.f32_view(inject),
+                            C.byref(self.err))
+        if check:
+            self._raise(st)
+        return st, ids, w
+
     def device_handles(self):
         """(PfHipMoe*, PfHipWork*) behind this layer: shipped library only."""
         return self.api.device_layer(self.handle), self.api.device_work(self.work)

@@ -12,7 +12,7 @@ import picoforge_amd as pf
 from picoforge_amd import abi, binding
 
 ROOT = Path(__file__).resolve().parents[1]
-HEADERS = ["qwen4_packed.h", "qwen4_moe.h", "pf_moe_hip.h"]
+HEADERS = ["qwen4_packed.h", "qwen4_moe.h", "qwen4_hc.h", "pf_moe_hip.h"]
 
 
 def declared_functions(header):
@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported():
         total += len(names)
         missing += [f"{header}:{n}" for n in names if not hasattr(lib, n)]
     assert not missing, missing
-    assert total >= 35
+    assert total >= 45
 
 
 def test_product_never_links_the_oracle():
@@ -51,11 +51,13 @@ def test_struct_layouts_match_a_c_compiler(tmp_path):
 #include <stdio.h>
 #include <stddef.h>
 #include "qwen4_moe.h"
+#include "qwen4_hc.h"
 #include "pf_moe_hip.h"
 int main(void) {
-    printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(Qwen4Error), sizeof(Qwen4F32), sizeof(Qwen4U32Mut),
+    printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(Qwen4Error), sizeof(Qwen4F32), sizeof(Qwen4U32Mut),
            sizeof(Qwen4MoeConfig), sizeof(GgufTensor), sizeof(QW4PackedLayout), sizeof(QW4PackedCpuView),
-           sizeof(Qwen4MoeWeights), sizeof(Qwen4MoeRoutes), sizeof(QW4MoeGrouping), sizeof(PfHipMoeDesc));
+           sizeof(Qwen4MoeWeights), sizeof(Qwen4MoeRoutes), sizeof(QW4MoeGrouping), sizeof(PfHipMoeDesc),
+           sizeof(Qwen4HcShape));
     printf("%zu %zu %zu %zu\n", offsetof(Qwen4Error, row), offsetof(Qwen4Error, subject),
            offsetof(Qwen4MoeConfig, trunk_type), offsetof(QW4PackedLayout, k_storage));
     return 0;
@@ -66,7 +68,7 @@ int main(void) {
                       subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.splitlines()]
     mirror = [abi.Qwen4Error, abi.Qwen4F32, abi.Qwen4U32Mut, abi.Qwen4MoeConfig, abi.GgufTensor,
               abi.QW4PackedLayout, abi.QW4PackedCpuView, abi.Qwen4MoeWeights, abi.Qwen4MoeRoutes,
-              abi.QW4MoeGrouping, binding.PfHipMoeDesc]
+              abi.QW4MoeGrouping, binding.PfHipMoeDesc, abi.Qwen4HcShape]
     assert sizes == [C.sizeof(t) for t in mirror]
     assert offsets == [abi.Qwen4Error.row.offset, abi.Qwen4Error.subject.offset,
                        abi.Qwen4MoeConfig.trunk_type.offset, abi.QW4PackedLayout.k_storage.offset]
@@ -91,6 +93,17 @@ int main(void) {
         subprocess.run(["gcc", "-std=c11", "-I", str(include), str(src), "-o", str(exe)], check=True)
         outputs.append(subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout)
     assert outputs[0] == outputs[1]
+    shapes = []
+    for name, include, header in (("mine_hc", ROOT / "include", "qwen4_hc.h"),
+                                  ("ref_hc", Path("/root/reference/src"), "qwen4_ops.h")):
+        src = tmp_path / f"{name}.c"
+        src.write_text(f'#include <stdio.h>\n#include <stddef.h>\n#include "{header}"\n' +
+                       'int main(void) { printf("%zu %zu %zu\\n", sizeof(Qwen4HcShape), offsetof(Qwen4HcShape, low_rank), '
+                       'offsetof(Qwen4HcShape, rms_eps)); return 0; }')
+        exe = tmp_path / name
+        subprocess.run(["gcc", "-std=c11", "-I", str(include), str(src), "-o", str(exe)], check=True)
+        shapes.append(subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout)
+    assert shapes[0] == shapes[1]
 
 
 def test_product_fails_loudly_without_a_device():

@@ -7,7 +7,10 @@ import ctypes as C
 import numpy as np
 
 import picoforge_amd as pf
+import pytest
 from picoforge_amd import abi
+
+from hc_cases import call_add, call_read, error_cases, hc_shape, random_case, run_error_case
 
 
 def _f32(buf, rows, cols, pitch):
@@ -124,3 +127,38 @@ def test_null_handles_give_the_oracle_codes(product_host, oracle):
         api.destroy(None)
         seen.append(codes)
     assert seen[0] == seen[1]
+
+
+# ---- hyper-connection read and add: every check made before the data is read ---------------------
+HC_PREFLIGHT = [c for c in error_cases() if c[2] != abi.QW4_NONFINITE or "eps" in c[0]]
+
+
+@pytest.mark.parametrize("op", ["read", "add"])
+@pytest.mark.parametrize("case", HC_PREFLIGHT, ids=lambda c: c[0])
+def test_hc_argument_errors_match_the_oracle(product_host, oracle, op, case):
+    _, mutate, status = case
+    st_o, out_o, err_o = run_error_case(oracle, op, mutate)
+    st_p, out_p, err_p = run_error_case(product_host, op, mutate)
+    assert st_p == st_o == status
+    assert (bytes(err_p.subject), bytes(err_p.detail)) == (bytes(err_o.subject), bytes(err_o.detail))
+    np.testing.assert_array_equal(out_p.view(np.uint32), out_o.view(np.uint32))   # untouched
+
+
+def test_hc_alias_and_empty_batches_need_no_device(product_host, oracle):
+    for api in (oracle, product_host):
+        normed, logits, block, inject = random_case(2, 4, 64, 21)
+        err = abi.Qwen4Error()
+        inside = normed[:, 0, :]
+        st = api.hc.read(C.byref(hc_shape(4, 64)), abi.f32_cube(normed), abi.f32_cube(logits),
+                         abi.f32_view(inside, pitch_bytes=normed.strides[0], capacity=normed.nbytes), C.byref(err))
+        assert st == abi.QW4_INVALID_ARGUMENT and b"alias" in err.detail
+        st = api.hc.add(C.byref(hc_shape(4, 64)), abi.f32_cube(normed),
+                        abi.f32_view(normed[:, 1, :], pitch_bytes=normed.strides[0], capacity=normed.nbytes),
+                        abi.f32_view(inject), C.byref(err))
+        assert st == abi.QW4_INVALID_ARGUMENT and b"alias" in err.detail
+        assert api.hc.read(None, abi.f32_cube(normed), abi.f32_cube(logits), abi.f32_view(block), None) == \
+            abi.QW4_INVALID_ARGUMENT
+        empty3 = np.zeros((0, 4, 64), dtype=np.float32)
+        empty2 = np.zeros((0, 64), dtype=np.float32)
+        assert call_read(api, empty3, empty3, empty2)[0] == abi.QW4_OK
+        assert call_add(api, empty3, empty2, np.zeros((0, 4), dtype=np.float32))[0] == abi.QW4_OK
