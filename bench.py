@@ -69,7 +69,9 @@ WORKLOADS = {
 # WRITE_SIZE scaled by the same counters on a plain 256 MiB copy (profiles/*.txt hold the runs).
 # A counter result cannot be read live; None where no such run exists for the workload.
 MEASURED_TRAFFIC = {"iq2xxs_decode": 9832986, "q4k_decode": 19831587, "q4k_verify4": None,
-                    "q4k_prefill1024": 816855693, "iq2xxs_prefill1024": 448880069}
+                    "q4k_prefill1024": 816855693, "iq2xxs_prefill1024": 448880069,
+                    # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
+                    "q4k_prefill1024_hc": 75633480, "iq2xxs_decode_hc": 117102, "q4k_decode_hc": None}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
@@ -210,6 +212,22 @@ def run_hc(args, api, hip, cfg, wl, steps, warmup):
     hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, steps, C.byref(ms)), "block alone")
     block_ms = ms.value / steps
 
+    # the two hyper-connection kernels alone, HIP events on the launch stream around back-to-back launches
+    # (the add runs with zero weights so that the residual stays put over the launches)
+    d_zero = hip.to_device(np.zeros_like(inject))
+    d_err = hip.to_device(np.zeros(64, dtype=np.uint32))
+    kernel_us = {}
+    n_launch = max(50, min(steps, 1000))
+    for which, name in ((0, "pf_k_hc_read"), (1, "pf_k_hc_add")):
+        for count in (10, n_launch):
+            hip.check(hip.hc_time_step(which, d_n if which == 0 else d_r, d_g, d_x if which == 0 else d_y,
+                                       d_zero, tokens, streams, h, count, d_err, C.byref(ms)), name)
+        kernel_us[name] = ms.value * 1e3 / n_launch
+    read_bytes = tokens * h * 4 * (2 * streams + 1)
+    add_bytes = tokens * h * 4 * (2 * streams + 1) + tokens * streams * 4
+    if args.copy_probe:
+        hip.check(hip.copy_probe(args.copy_probe << 20, 3), "copy probe")
+
     # parity on a bounded sample, stage by stage on identical inputs: CPU read against the device's mixed rows,
     # CPU block on those rows, CPU add of its output; the device's chained call against that residual
     ref = pf.load_reference()
@@ -256,11 +274,16 @@ def run_hc(args, api, hip, cfg, wl, steps, warmup):
                               "read + block + add kernel": round(timed["separate_add"] * 1e3, 3),
                               "block alone": round(block_ms * 1e3, 3)},
         "hc_bytes_per_step": int(hc_bytes),
-        "roofline": {"bound": "hbm", "kernel": "the two hyper-connection steps: chain minus block alone",
-                     "achieved": round(hc_bytes / max((timed["fused"] - block_ms) * 1e-3, 1e-9) / 1e9, 1),
+        "kernel_us": {k: round(v, 3) for k, v in kernel_us.items()},
+        "kernel_bytes": {"pf_k_hc_read": int(read_bytes), "pf_k_hc_add": int(add_bytes)},
+        "kernel_GBps": {"pf_k_hc_read": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9, 1),
+                        "pf_k_hc_add": round(add_bytes / (kernel_us["pf_k_hc_add"] * 1e-6) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "kernel": "pf_k_hc_read (gated mix of the residual streams)",
+                     "achieved": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(hc_bytes / max((timed["fused"] - block_ms) * 1e-3, 1e-9) / 1e9 / HBM_PEAK_GBPS, 4),
-                     "traffic": None},
+                     "frac": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC.get(args.workload), "bytes_per_launch": int(read_bytes),
+                     "us_per_launch": round(kernel_us["pf_k_hc_read"], 3)},
         "cpu_baseline": {"value": round(cpu_s / sample_tokens * 1e6, 1), "unit": "us/layer/token", "cores": 1,
                          "kind": kind, "sample": f"{sample_tokens} tokens of the same inputs through read, block and add, "
                                                  f"{cpu_s:.1f} s"},

@@ -188,6 +188,14 @@ int pf_hip_moe_time_forwards_hc(const PfHipMoe *moe, PfHipWork *work, const floa
                                 const float *d_inject, size_t streams, size_t tokens,
                                 size_t iters, int fused, float *elapsed_ms);
 
+/* One of the two hyper-connection kernels alone, `iters` launches back to back between
+ * two events on the launch stream.  which 0: the read of d_cube (normed) and d_logits,
+ * dense [tokens, streams, hidden], into d_rows [tokens, hidden]; which 1: the add of
+ * d_rows into d_cube with weights d_inject [tokens, streams]. */
+int pf_hip_hc_time_step(int which, float *d_cube, const float *d_logits, float *d_rows,
+                        const float *d_inject, size_t tokens, size_t streams, size_t hidden,
+                        size_t iters, uint32_t *d_error_word, float *elapsed_ms);
+
 /* The same for a stack of layers of equal hidden size (works[l] belongs to moes[l]):
  * forward i runs through layer i % layers with input row block i % n_inputs, so
  * `iters` = tokens-through-the-stack x layers. */

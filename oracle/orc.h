@@ -10,8 +10,11 @@
  * reference); functions carry an orc_ prefix so that the oracle, a build of the
  * reference and the product library can be loaded side by side.
  *
- * Pinning status (which independent check covers which function) is listed in
- * oracle/README.md; every function below is pinned. */
+ * Every function below is pinned by checks that do not restate its formula:
+ * tests/test_oracle_packed.py, tests/test_oracle_moe.py and tests/test_oracle_hc.py
+ * (known answers the reference's own tests hold, independent numpy evaluations,
+ * closed forms, and the reference's compiled C path bit for bit), and
+ * tests/test_golden.py (vectors written by that compiled path). */
 #ifndef PF_ORACLE_H
 #define PF_ORACLE_H
 #include "../include/qwen4_moe.h"

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include "pf_expf_libm.h"
 
 #define PF_WAVE 64
 
@@ -86,10 +87,10 @@ __device__ __forceinline__ uint32_t pf_parity7(uint32_t s) {
 }
 
 __device__ __forceinline__ float pf_sigmoid(float x) {
-    // two-branch form of src/qwen4_cpu_internal.h:103-106
-    if (x >= 0.0f) return 1.0f / (1.0f + expf(-x));
-    float z = expf(x);
-    return z / (1.0f + z);
+    // the two branches of src/qwen4_cpu_internal.h:103-106 share their exponential, expf(-|x|):
+    // 1 / (1 + e) for x >= 0, e / (1 + e) below; one evaluation whatever the lanes' signs
+    const float e = expf(-fabsf(x));
+    return (x >= 0.0f ? 1.0f : e) / (1.0f + e);
 }
 __device__ __forceinline__ float pf_silu(float x) { return x * pf_sigmoid(x); }
 

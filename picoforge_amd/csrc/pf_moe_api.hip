@@ -478,8 +478,17 @@ extern "C" int pf_hip_moe_forward_hc_device(const PfHipMoe *moe, PfHipWork *work
     hipStream_t s = (hipStream_t)stream;
     pf_launch_hc_read(d_normed, n_token_pitch, n_stream_pitch, d_logits, g_token_pitch, g_stream_pitch, work->x, H,
                       (int)tokens, (int)streams, (int)H, work->error_word, s);
-    const HcTarget hc = {d_residual, r_token_pitch, r_stream_pitch, d_inject, (int)streams};
-    return forward_enqueue(moe, work, work->x, H, work->y, H, tokens, &hc, s);
+    if (streams <= PF_HC_FOLD_MAX) {
+        const HcTarget hc = {d_residual, r_token_pitch, r_stream_pitch, d_inject, (int)streams};
+        return forward_enqueue(moe, work, work->x, H, work->y, H, tokens, &hc, s);
+    }
+    // more streams than the block's last kernel keeps in registers: the add runs as a kernel of its own
+    const int rc = forward_enqueue(moe, work, work->x, H, work->y, H, tokens, nullptr, s);
+    if (rc != PF_HIP_OK) return rc;
+    pf_launch_hc_add(d_residual, r_token_pitch, r_stream_pitch, work->y, H, d_inject, streams, (int)tokens,
+                     (int)streams, (int)H, work->error_word, s);
+    HIP_TRY(hipGetLastError());
+    return PF_HIP_OK;
 }
 
 extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
@@ -862,6 +871,40 @@ extern "C" int pf_hip_moe_time_forwards_hc(const PfHipMoe *moe, PfHipWork *work,
                                       work->error_word, s);
         return rc;
     });
+}
+
+// One of the two hyper-connection kernels alone, `iters` launches back to back on a stream of its own,
+// bracketed by two events on that stream.  which 0: the read (dense inputs, output into d_rows);
+// which 1: the add of d_rows into d_cube (dense), weights d_inject.
+extern "C" int pf_hip_hc_time_step(int which, float *d_cube, const float *d_logits, float *d_rows,
+                                   const float *d_inject, size_t tokens, size_t streams, size_t hidden, size_t iters,
+                                   uint32_t *d_error_word, float *elapsed_ms) {
+    if (!d_cube || !d_rows || !elapsed_ms || !d_error_word || !hc_dims_ok(tokens, streams, hidden) || !tokens ||
+        (which == 0 ? !d_logits : !d_inject))
+        return PF_HIP_E_ARGUMENT;
+    hipStream_t s = nullptr;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    HIP_TRY(hipStreamCreate(&s));
+    hipError_t e = hipEventCreate(&t0);
+    if (e == hipSuccess) e = hipEventCreate(&t1);
+    if (e == hipSuccess) e = hipEventRecord(t0, s);
+    for (size_t i = 0; i < iters && e == hipSuccess; i++) {
+        if (which == 0)
+            pf_launch_hc_read(d_cube, streams * hidden, hidden, d_logits, streams * hidden, hidden, d_rows, hidden,
+                              (int)tokens, (int)streams, (int)hidden, d_error_word, s);
+        else
+            pf_launch_hc_add(d_cube, streams * hidden, hidden, d_rows, hidden, d_inject, streams, (int)tokens,
+                             (int)streams, (int)hidden, d_error_word, s);
+        e = hipGetLastError();
+    }
+    if (e == hipSuccess) e = hipEventRecord(t1, s);
+    if (e == hipSuccess) e = hipStreamSynchronize(s);
+    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
+    (void)hipStreamDestroy(s);
+    if (e != hipSuccess) { pf_set_error("timed hyper-connection kernel", e); return PF_HIP_E_RUNTIME; }
+    return PF_HIP_OK;
 }
 
 extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,

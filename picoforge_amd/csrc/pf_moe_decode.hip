@@ -542,6 +542,9 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_bl
 #pragma unroll
     for (int slot = 0; slot < 16; slot++) rw[slot] = slot < K ? a.route_weights[t * K + slot] : 0.0f;
     const float shared_scale = a.shared_scale[t];
+    PfOutputRegs out_regs;
+    if ((int)threadIdx.x < rows_per_block && n_base + (int)threadIdx.x < H)
+        pf_output_prefetch(a, t, n_base + threadIdx.x, out_regs);
     if (FMT == PF_IQ2_XXS) __syncthreads();
     else pf_wave_lds_fence();
     XSeg x;
@@ -560,7 +563,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_bl
         for (int slot = 0; slot < 16; slot++)   // slot order, as src/qwen4_moe.c:362-372
             if (slot < K) sum += rw[slot] * partial[slot][threadIdx.x];
         const float y = sum + shared_scale * partial[K][threadIdx.x];
-        if (!pf_emit_output(a, t, n, y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        if (!pf_output_commit(a, t, n, y, out_regs)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
 }
 

@@ -49,9 +49,24 @@ struct PfKernelArgs {
 };
 
 // One finished element of the block's output.  Normally y[t, n]; when the forward injects into the
-// residual streams, residual[t, h, n] += inject[t, h] * value for every stream h, product and sum
-// each rounded (src/qwen4_base.c:168-173).  Returns false if anything written is not finite.
-__device__ __forceinline__ bool pf_emit_output(const PfKernelArgs &a, int t, int n, float value) {
+// residual streams (at most PF_HC_FOLD_MAX of them), residual[t, h, n] += inject[t, h] * value for
+// every stream h, product and sum each rounded (src/qwen4_base.c:168-173).  The residual values are
+// requested early (pf_output_prefetch, before the kernel's long loop) and used at the end
+// (pf_output_commit), so their latency hides behind the products.  commit returns false if
+// anything written is not finite.
+#define PF_HC_FOLD_MAX 4
+struct PfOutputRegs { float r[PF_HC_FOLD_MAX]; };
+
+__device__ __forceinline__ void pf_output_prefetch(const PfKernelArgs &a, int t, int n, PfOutputRegs &q) {
+    if (!a.hc_residual) return;
+    const float *r = a.hc_residual + (size_t)t * a.hc_token_pitch + n;
+#pragma unroll
+    for (int h = 0; h < PF_HC_FOLD_MAX; h++)
+        if (h < a.hc_streams) q.r[h] = r[(size_t)h * a.hc_stream_pitch];
+}
+
+__device__ __forceinline__ bool pf_output_commit(const PfKernelArgs &a, int t, int n, float value,
+                                                 const PfOutputRegs &q) {
 #pragma clang fp contract(off)
     if (!a.hc_residual) {
         a.y[(size_t)t * a.y_pitch + n] = value;
@@ -60,11 +75,14 @@ __device__ __forceinline__ bool pf_emit_output(const PfKernelArgs &a, int t, int
     bool ok = true;
     float *r = a.hc_residual + (size_t)t * a.hc_token_pitch + n;
     const float *w = a.hc_inject + (size_t)t * a.hc_streams;
-    for (int h = 0; h < a.hc_streams; h++) {
-        const float product = w[h] * value;
-        const float result = r[(size_t)h * a.hc_stream_pitch] + product;
-        r[(size_t)h * a.hc_stream_pitch] = result;
-        ok &= pf_finite(result);
+#pragma unroll
+    for (int h = 0; h < PF_HC_FOLD_MAX; h++) {
+        if (h < a.hc_streams) {
+            const float product = w[h] * value;
+            const float result = q.r[h] + product;
+            r[(size_t)h * a.hc_stream_pitch] = result;
+            ok &= pf_finite(result);
+        }
     }
     return ok;
 }

@@ -221,7 +221,9 @@ __global__ void __launch_bounds__(256) pf_k_down_combine(PfKernelArgs a) {
     float sh = dot_tensor_row(a, 6, 0, n, sact, lane, grid);
     float y = sum + a.shared_scale[t] * sh;
     if (lane == 0) {
-        if (!pf_emit_output(a, t, n, y)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        PfOutputRegs out_regs;
+        pf_output_prefetch(a, t, n, out_regs);
+        if (!pf_output_commit(a, t, n, y, out_regs)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
 }
 

@@ -802,13 +802,15 @@ __global__ void __launch_bounds__(256) pf_k_pf_combine(PfKernelArgs a, int token
     const float ss = a.shared_scale[t];
     bool bad = false;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
+        PfOutputRegs out_regs;
+        pf_output_prefetch(a, t, c, out_regs);
         float sum = 0.0f;
         for (int s = 0; s < K; s++) {
             const float term = weights[s] * a.down[(size_t)rows[s] * H + c];
             sum += term;
         }
         const float y = sum + ss * a.down[(size_t)(P + t) * H + c];
-        bad |= !pf_emit_output(a, t, c, y);
+        bad |= !pf_output_commit(a, t, c, y, out_regs);
     }
     if (__any(bad) && pf_lane() == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
 }

@@ -56,10 +56,10 @@ __device__ __forceinline__ void pf_route_exact_wave(const float *z, float *p, fl
     float top = -INFINITY;
     for (int e = lane; e < E; e += PF_WAVE) top = fmaxf(top, z[e]);
     top = pf_wave_max(top);
-    // exponent in double, rounded once: the correctly rounded expf
+    // the C library's expf, bit for bit (pf_expf_libm.h)
     for (int e = lane; e < E; e += PF_WAVE) {
         float shifted = z[e] - top;
-        p[e] = (float)exp((double)shifted);
+        p[e] = pf_expf_libm(shifted);
     }
     pf_wave_lds_fence();
     float sum = 0.0f;

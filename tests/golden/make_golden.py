@@ -20,6 +20,7 @@ sys.path.insert(0, str(ROOT / "tests"))
 import picoforge_amd as pf  # noqa: E402
 from picoforge_amd import abi  # noqa: E402
 from helpers import call_decode, call_group, call_route, forward_with, make_layer_inputs  # noqa: E402
+from hc_cases import call_add, call_read, random_case  # noqa: E402
 
 OUT = Path(__file__).resolve().parent
 
@@ -32,10 +33,31 @@ FORWARD_CASES = {
 }
 
 
+HC_CASES = [(5, 3, 7, 1.0), (3, 4, 256, 4.0), (2, 4, 64, 30.0)]   # tokens, streams, hidden, logit scale
+
+
+def write_hc(ref):
+    """qwen4_hc_read and qwen4_hc_add of the reference on seeded inputs, the exp branches included."""
+    arrays = {}
+    for n, (t, h, w, scale) in enumerate(HC_CASES):
+        normed, logits, block, inject = random_case(t, h, w, 26 + n, scale=scale)
+        logits.ravel()[:4] = (0.0, -0.0, 89.0, -104.0)
+        st, mixed, _ = call_read(ref, normed, logits)
+        assert st == 0
+        residual = normed.copy()
+        assert call_add(ref, residual, block, inject)[0] == 0
+        arrays.update({f"normed{n}": normed, f"logits{n}": logits, f"block{n}": block, f"inject{n}": inject,
+                       f"mixed_bits{n}": mixed.view(np.uint32), f"residual_bits{n}": residual.view(np.uint32)})
+    np.savez_compressed(OUT / "hc_read_add.npz", **arrays)
+
+
 def main():
     ref = pf.load_reference()
     if ref is None:
         sys.exit("oracle/_ref/libqwen4_ref.so missing: run make -C oracle where the reference is mounted")
+    write_hc(ref)
+    if "--only-hc" in sys.argv:
+        return
     for name, (h, e, k, i, s, gtype, tokens, seed) in FORWARD_CASES.items():
         cfg = abi.moe_config(h, e, k, i, s)
         weights, x = make_layer_inputs(cfg, gtype, tokens, seed=seed, std=0.02 if gtype else 0.2)

@@ -9,6 +9,7 @@ import pytest
 import picoforge_amd as pf
 from picoforge_amd import abi
 
+from hc_cases import call_add, call_read
 from helpers import assert_parity, call_decode, call_group, call_route, forward_with
 
 GOLDEN = Path(__file__).resolve().parent / "golden"
@@ -55,6 +56,29 @@ def test_oracle_reproduces_route_group_and_decode_fixtures(oracle):
             np.testing.assert_array_equal(out.view(np.uint32), data["rows_bits"][row])
 
 
+def replay_hc_fixture(api):
+    data = np.load(GOLDEN / "hc_read_add.npz", allow_pickle=False)
+    cases = sorted(int(k[6:]) for k in data.files if k.startswith("normed"))
+    assert len(cases) == 3
+    for n in cases:
+        normed, logits = data[f"normed{n}"].copy(), data[f"logits{n}"].copy()
+        st, mixed, _ = call_read(api, normed, logits)
+        assert st == abi.QW4_OK
+        np.testing.assert_array_equal(mixed.view(np.uint32), data[f"mixed_bits{n}"], err_msg=f"read, case {n}")
+        residual = normed.copy()
+        assert call_add(api, residual, data[f"block{n}"].copy(), data[f"inject{n}"].copy())[0] == abi.QW4_OK
+        np.testing.assert_array_equal(residual.view(np.uint32), data[f"residual_bits{n}"], err_msg=f"add, case {n}")
+
+
+def test_oracle_reproduces_hc_fixture(oracle):
+    replay_hc_fixture(oracle)
+
+
+@pytest.mark.gpu
+def test_hip_path_reproduces_hc_fixture_bit_for_bit(product):
+    replay_hc_fixture(product)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("name", FORWARD)
 def test_hip_path_reproduces_forward_fixture(product, name):
@@ -70,8 +94,8 @@ def test_hip_path_reproduces_route_group_and_decode_fixtures(product):
     st, p, ids, w, _ = call_route(product, cfg, data["logits"])
     assert st == abi.QW4_OK
     np.testing.assert_array_equal(ids, data["ids"])
-    np.testing.assert_allclose(p, data["p_bits"].view(np.float32), rtol=3e-7, atol=1e-38)
-    np.testing.assert_allclose(w, data["w_bits"].view(np.float32), rtol=5e-7, atol=1e-38)
+    np.testing.assert_array_equal(p.view(np.uint32), data["p_bits"])
+    np.testing.assert_array_equal(w.view(np.uint32), data["w_bits"])
     st, off, cur, p2r, r2p = call_group(product, cfg, data["ids"])
     np.testing.assert_array_equal(off[:513], data["offsets"])
     np.testing.assert_array_equal(p2r[:160], data["pair_to_row"])
