@@ -41,6 +41,8 @@ sys.path.insert(0, str(ROOT))
 import picoforge_amd as pf  # noqa: E402
 from picoforge_amd import abi, workloads  # noqa: E402
 
+FORMAT_LABEL = {12: "Q4_K", 16: "IQ2_XXS", "q2": "IQ2_XXS gate/up, Q2_K down, Q8_0 shared expert",
+                "q4": "Q4_K gate/up, MXFP4 down, Q8_0 shared expert"}
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
@@ -61,6 +63,10 @@ WORKLOADS = {
     "q4k_prefill1024_hc": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10, hc=4,
                                label="Q4_K experts, 1024-token prefill chunk, between the HC read and add of 4 residual "
                                      "streams, Zipf(1.1) expert popularity"),
+    "q2profile_decode": dict(type="q2", tokens=1, steps=5000, warmup=100,
+                             label="checkpoint profile Q2 (IQ2_XXS gate/up, Q2_K down, Q8_0 shared expert), decode batch 1"),
+    "q4profile_decode": dict(type="q4", tokens=1, steps=5000, warmup=100,
+                             label="checkpoint profile Q4 (Q4_K gate/up, MXFP4 down, Q8_0 shared expert), decode batch 1"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),
@@ -71,10 +77,15 @@ WORKLOADS = {
 MEASURED_TRAFFIC = {"iq2xxs_decode": 9832986, "q4k_decode": 19831587, "q4k_verify4": None,
                     "q4k_prefill1024": 816855693, "iq2xxs_prefill1024": 448880069,
                     # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
-                    "q4k_prefill1024_hc": 75633480, "iq2xxs_decode_hc": 117102, "q4k_decode_hc": None}
+                    "q4k_prefill1024_hc": 75633480, "iq2xxs_decode_hc": 117102, "q4k_decode_hc": None,
+                    "q2profile_decode": None, "q4profile_decode": None}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
+GENERAL_STAGES = ["pf_k_pre (router logits, shared gate/up + SwiGLU, shared gate)",
+                  "routing (top-k, serial-order re-routes)",
+                  "pf_k_gate_up (routed gate/up + SwiGLU)",
+                  "pf_k_down_combine (routed and shared down products, combine)"]
 PREFILL_STAGES = ["pf_k_rows_to_half + pf_k_pf_router (fp16 copy of x, router logits by FP32 MFMA)",
                   "routing + grouping (top-k, serial-order re-routes, histogram/scan/stable placement)",
                   "pf_k_pf_gemm<gate_up> (grouped gate/up + SwiGLU by FP16 MFMA, then fp16 copy of the activations)",
@@ -259,7 +270,6 @@ def run_hc(args, api, hip, cfg, wl, steps, warmup):
     layer.close()
     sample_tokens = steps_cpu * rows
     ms_per_step = timed["fused"]
-    block, size = abi.BLOCK[wl["type"]]
     hc_bytes = tokens * h * 4 * (2 * streams + 1) + tokens * h * 4 * 2 * streams   # read in/out, residual in/out
     result = {
         "metric": "moe_hc_block_us_per_layer_token", "value": round(ms_per_step * 1e3 / tokens, 3),
@@ -269,7 +279,7 @@ def run_hc(args, api, hip, cfg, wl, steps, warmup):
         "config": {"workload": f"one MoE layer, hidden 2048, 512 experts, top-10, intermediate 512, shared 512; "
                                f"{wl['label']}; {n_inputs} seeded inputs",
                    "tokens_per_step": tokens, "streams": streams,
-                   "expert_format": {12: "Q4_K", 16: "IQ2_XXS"}[wl["type"]]},
+                   "expert_format": FORMAT_LABEL[wl["type"]]},
         "chain_us_per_step": {"read + block with the add folded in": round(timed["fused"] * 1e3, 3),
                               "read + block + add kernel": round(timed["separate_add"] * 1e3, 3),
                               "block alone": round(block_ms * 1e3, 3)},
@@ -373,10 +383,11 @@ def main():
     # gap before it, as a profiler's start-to-end time of a dependent kernel does).
     stage = (C.c_float * 4)()
     hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(steps, 2000), stage), "stages")
-    names = PREFILL_STAGES if prefill else DECODE_STAGES
+    family = hip.moe_kernel_family(moe, work, tokens)
+    names = {0: GENERAL_STAGES, 1: DECODE_STAGES, 2: PREFILL_STAGES}[family]
     stage_us = [max(float(stage[j]) * 1e3, 1e-3) for j in range(len(names))]
 
-    block, size = abi.BLOCK[wl["type"]]
+    lb = workloads.layer_bytes(wl["type"], cfg)
     h, i, s_i, k = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate, cfg.top_k
     extra = {}
     if prefill:
@@ -384,11 +395,11 @@ def main():
         pairs = tokens * k
         stage_bytes = [tokens * h * 4 + (cfg.experts + 1) * h * 4 + tokens * h * 2,
                        tokens * cfg.experts * 4 + pairs * 16,
-                       unique * 2 * i * h // block * size + 2 * s_i * h // block * size + (pairs + tokens) * h * 2
+                       unique * lb["gate_up"] + lb["shared_gate_up"] + (pairs + tokens) * h * 2
                        + (pairs * i + tokens * s_i) * 4,
-                       unique * h * i // block * size + h * s_i // block * size + (pairs * i + tokens * s_i) * 2
+                       unique * lb["down"] + lb["shared_down"] + (pairs * i + tokens * s_i) * 2
                        + (pairs + tokens) * h * 4 + tokens * h * 4]
-        alg_bytes = unique * 3 * i * h // block * size + 3 * s_i * h // block * size + (cfg.experts + 1) * h * 4 \
+        alg_bytes = unique * (lb["gate_up"] + lb["down"]) + lb["shared_gate_up"] + lb["shared_down"] + lb["routers"] \
             + 2 * tokens * h * 4
         stage_flops = [2.0 * tokens * h * (cfg.experts + 1), 0.0, 2.0 * tokens * (k * 2 * h * i + 2 * h * s_i),
                        2.0 * tokens * (k * i * h + s_i * h)]
@@ -401,16 +412,18 @@ def main():
                  "binding_roofline": "hbm: about 80 flop per weight byte at this chunk size, below the MFMA ridge"}
     else:
         alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique)
-        stage_bytes = [(cfg.experts + 1) * h * 4,
-                       unique * 2 * i * h // block * size + 2 * s_i * h // block * size,
-                       unique * h * i // block * size + h * s_i // block * size]
+        stage_bytes = [lb["routers"], unique * lb["gate_up"] + lb["shared_gate_up"],
+                       unique * lb["down"] + lb["shared_down"]]
+        if family == 0:
+            stage_bytes = [lb["routers"] + lb["shared_gate_up"], tokens * cfg.experts * 8, unique * lb["gate_up"],
+                           unique * lb["down"] + lb["shared_down"]]
     dom = int(np.argmax(stage_bytes))
     achieved = stage_bytes[dom] / (stage_us[dom] * 1e-6) / 1e9
 
     # CPU baseline and parity on a bounded sample of the same inputs
     ref = pf.load_reference()
     cpu_api, kind = (ref, "reference") if ref is not None else (pf.load_oracle(), "port")
-    per_token_guess = 0.55 if wl["type"] == abi.GGUF_IQ2_XXS else 0.32
+    per_token_guess = 0.55 if wl["type"] in (abi.GGUF_IQ2_XXS, "q2") else 0.32
     if prefill:
         sample_tokens = min(tokens, args.cpu_sample or 48)
         with pf.MoeLayer(cpu_api, cfg, weights, sample_tokens) as cpu:
@@ -449,7 +462,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"one MoE layer, hidden 2048, 512 experts, top-10, intermediate 512, shared 512; "
                                f"{wl['label']}; {n_inputs} seeded inputs{margins}",
-                   "tokens_per_step": tokens, "expert_format": {12: "Q4_K", 16: "IQ2_XXS"}[wl["type"]],
+                   "tokens_per_step": tokens, "expert_format": FORMAT_LABEL[wl["type"]],
                    "unique_experts_per_step": unique, "inputs": info},
         "hbm_GBps_on_algorithmic_bytes": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         "algorithmic_bytes_per_step": int(alg_bytes),

@@ -67,6 +67,10 @@ void pf_hip_work_destroy(PfHipWork *work);
 int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
                               size_t x_pitch, float *d_y, size_t y_pitch, size_t tokens,
                               void *stream);
+/* Which kernels a forward of `tokens` tokens runs on this layer and workspace: 1 the
+ * decode kernels (1..4 tokens, supported shapes and formats), 2 the matrix-core
+ * prefill kernels, 0 the general kernels (any shape and format mix). */
+int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t tokens);
 /* Device pointers into the workspace, valid after a forward: expert ids
  * [tokens, top_k] uint32, route weights [tokens, top_k], router logits
  * [tokens, experts], the error word (one uint32). */

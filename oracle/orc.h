@@ -28,7 +28,7 @@ const GgufFormat *orc_format(uint32_t id);
 Qwen4Status orc_packed_layout_init(const GgufTensor *, size_t k_logical, QW4PackedLayout *, Qwen4Error *);
 /* src/qwen4_packed.c:54-66 */
 float orc_half_value(uint16_t bits);
-/* src/qwen4_packed.c:67-115 (types 0, 12, 16) */
+/* src/qwen4_packed.c:67-122 (F32, F16, Q8_0, Q2_K, Q4_K, IQ2_XXS, BF16, MXFP4) */
 float orc_packed_value(const unsigned char *row, size_t column, uint32_t type);
 /* src/qwen4_packed.c:124-143 and :145-181 */
 Qwen4Status orc_packed_decode_row(const QW4PackedCpuView *, size_t expert, size_t row,

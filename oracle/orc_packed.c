@@ -35,10 +35,11 @@ static bool ranges_overlap(const void *a, size_t na, const void *b, size_t nb) {
     return na != 0 && nb != 0 && pa < pb + nb && pb < pa + na;
 }
 
-/* src/gguf.c:12-16, restricted to the executable formats of this build */
+/* src/gguf.c:12-16 */
 const GgufFormat *orc_format(uint32_t id) {
     static const GgufFormat table[] = {
-        {0, "F32", 1, 4}, {12, "Q4_K", 256, 144}, {16, "IQ2_XXS", 256, 66},
+        {0, "F32", 1, 4}, {1, "F16", 1, 2}, {8, "Q8_0", 32, 34}, {10, "Q2_K", 256, 84},
+        {12, "Q4_K", 256, 144}, {16, "IQ2_XXS", 256, 66}, {30, "BF16", 1, 2}, {39, "MXFP4", 32, 17},
     };
     for (size_t i = 0; i < sizeof table / sizeof table[0]; i++)
         if (table[i].id == id) return &table[i];
@@ -119,14 +120,39 @@ float orc_half_value(uint16_t h) {
 
 static uint16_t le16(const unsigned char *p) { return (uint16_t)(p[0] | (p[1] << 8)); }
 
-/* src/qwen4_packed.c:67-78, :86-93, :102-115 */
+/* src/qwen4_packed.c:67-122 */
 float orc_packed_value(const unsigned char *row, size_t column, uint32_t type) {
-    if (type == 0) {
-        const unsigned char *p = row + 4 * column;
-        uint32_t bits = (uint32_t)le16(p) | ((uint32_t)le16(p + 2) << 16);
+    if (type == 0 || type == 30) {   /* F32; BF16 = the upper half of an F32 */
+        uint32_t bits;
+        if (type == 30) bits = (uint32_t)le16(row + 2 * column) << 16;
+        else bits = (uint32_t)le16(row + 4 * column) | ((uint32_t)le16(row + 4 * column + 2) << 16);
         float v;
         memcpy(&v, &bits, 4);
         return v;
+    }
+    if (type == 1) return orc_half_value(le16(row + 2 * column));
+    if (type == 8) {                 /* Q8_0: half scale, 32 signed bytes */
+        const unsigned char *blk = row + column / 32 * 34;
+        int code = blk[2 + column % 32];
+        if (code >= 128) code -= 256;
+        return orc_half_value(le16(blk)) * (float)code;
+    }
+    if (type == 39) {                /* MXFP4: one E8M0 scale byte, 32 E2M1 codes, low nibbles first */
+        static const float e2m1[16] = {0, .5f, 1, 1.5f, 2, 3, 4, 6, -0.0f, -.5f, -1, -1.5f, -2, -3, -4, -6};
+        const unsigned char *blk = row + column / 32 * 17;
+        unsigned lane = (unsigned)(column % 32), code = (blk[1 + lane % 16] >> ((lane / 16) * 4)) & 15u;
+        uint32_t bits = blk[0] ? (uint32_t)blk[0] << 23 : 0x00400000u;   /* 2^(e - 127); e = 0 is 2^-127 */
+        float scale;
+        memcpy(&scale, &bits, 4);
+        return e2m1[code] * scale;
+    }
+    if (type == 10) {                /* Q2_K: 16 scale/min nibble pairs, 64 bytes of 2-bit codes, d, dmin */
+        const unsigned char *blk = row + column / 256 * 84;
+        size_t lane = column % 256;
+        unsigned sm = blk[lane / 16];
+        unsigned code = (blk[16 + lane / 128 * 32 + lane % 32] >> (2 * (lane % 128 / 32))) & 3u;
+        return (orc_half_value(le16(blk + 80)) * (float)(sm & 15u)) * (float)code -
+               orc_half_value(le16(blk + 82)) * (float)(sm >> 4);
     }
     if (type == 12) {
         const unsigned char *blk = row + column / 256 * 144, *sc = blk + 4;

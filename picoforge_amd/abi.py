@@ -13,8 +13,11 @@ STATUS = ["OK", "INVALID_ARGUMENT", "MISSING", "TYPE", "RANGE", "SHAPE", "STRIDE
           "NONFINITE", "IO", "EOF", "CANCELLED", "GPU_ERROR"]
 globals().update({"QW4_" + name: value for value, name in enumerate(STATUS)})
 
-GGUF_F32, GGUF_Q4_K, GGUF_IQ2_XXS = 0, 12, 16
-BLOCK = {GGUF_F32: (1, 4), GGUF_Q4_K: (256, 144), GGUF_IQ2_XXS: (256, 66)}  # src/gguf.c:12-16
+GGUF_F32, GGUF_F16, GGUF_Q8_0, GGUF_Q2_K, GGUF_Q4_K, GGUF_IQ2_XXS, GGUF_BF16, GGUF_MXFP4 = 0, 1, 8, 10, 12, 16, 30, 39
+# (elements per block, bytes per block), src/gguf.c:12-16
+BLOCK = {GGUF_F32: (1, 4), GGUF_F16: (1, 2), GGUF_Q8_0: (32, 34), GGUF_Q2_K: (256, 84), GGUF_Q4_K: (256, 144),
+         GGUF_IQ2_XXS: (256, 66), GGUF_BF16: (1, 2), GGUF_MXFP4: (32, 17)}
+FORMAT_NAME = {0: "F32", 1: "F16", 8: "Q8_0", 10: "Q2_K", 12: "Q4_K", 16: "IQ2_XXS", 30: "BF16", 39: "MXFP4"}
 
 
 class Qwen4Error(C.Structure):

@@ -158,6 +158,7 @@ class HipShim:
         bind("pf_hip_moe_profile_stages", C.c_int, vp, vp, vp, sz, vp, sz, sz, P(C.c_float))
         bind("pf_hip_stack_time_forwards", C.c_int, P(vp), P(vp), sz, vp, sz, vp, sz, sz, P(C.c_float))
         bind("pf_hip_copy_probe", C.c_int, sz, sz)
+        bind("pf_hip_moe_kernel_family", C.c_int, vp, vp, sz)
         bind("pf_hip_hc_read_device", C.c_int, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_hc_add_device", C.c_int, vp, sz, sz, vp, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_moe_forward_hc_device", C.c_int, vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp)
@@ -199,8 +200,11 @@ class Synth:
         lib.pf_synth_q4k_quantize.argtypes = [vp, sz, vp]
         lib.pf_synth_q4k_normal.argtypes = [vp, sz, C.c_uint64, C.c_float]
         lib.pf_synth_iq2xxs_uniform.argtypes = [vp, sz, C.c_uint64, C.c_float]
+        for name in ("pf_synth_q8_0_normal", "pf_synth_q2k_normal", "pf_synth_mxfp4_normal"):
+            getattr(lib, name).argtypes = [vp, sz, C.c_uint64, C.c_float]
         for fn in (lib.pf_synth_normal_f32, lib.pf_synth_q4k_quantize, lib.pf_synth_q4k_normal,
-                   lib.pf_synth_iq2xxs_uniform):
+                   lib.pf_synth_iq2xxs_uniform, lib.pf_synth_q8_0_normal, lib.pf_synth_q2k_normal,
+                   lib.pf_synth_mxfp4_normal):
             fn.restype = None
         self.lib = lib
 
@@ -219,6 +223,14 @@ class Synth:
         assert values.size % 256 == 0
         out = np.empty(values.size // 256 * 144, dtype=np.uint8)
         self.lib.pf_synth_q4k_quantize(values.ctypes.data, values.size // 256, out.ctypes.data)
+        return out
+
+    def quantised_normal(self, gtype, elements, seed, std):
+        """N(0, std) weights quantised to Q8_0, Q2_K or MXFP4 blocks."""
+        name, (block, size) = {abi.GGUF_Q8_0: "q8_0", abi.GGUF_Q2_K: "q2k", abi.GGUF_MXFP4: "mxfp4"}[gtype], abi.BLOCK[gtype]
+        assert elements % block == 0
+        out = np.empty(elements // block * size, dtype=np.uint8)
+        getattr(self.lib, f"pf_synth_{name}_normal")(out.ctypes.data, elements // block, seed, std)
         return out
 
     def iq2xxs_uniform(self, blocks, seed, d_base=2.0 ** -12):

@@ -7,7 +7,7 @@
 #define PF_WAVE 64
 
 // GGUF type ids and block geometry (src/gguf.c:12-16 of the reference).
-enum { PF_F32 = 0, PF_Q4_K = 12, PF_IQ2_XXS = 16 };
+enum { PF_F32 = 0, PF_F16 = 1, PF_Q8_0 = 8, PF_Q2_K = 10, PF_Q4_K = 12, PF_IQ2_XXS = 16, PF_BF16 = 30, PF_MXFP4 = 39 };
 
 __device__ __forceinline__ int pf_lane() { return threadIdx.x & (PF_WAVE - 1); }
 
@@ -80,6 +80,16 @@ __device__ __forceinline__ void pf_q4k_scale_min(const uint32_t sc[3], int g, ui
         minimum = (pf_byte(sc, g + 4) >> 4) | ((pf_byte(sc, g) & 192u) >> 2);
     }
 }
+
+// E2M1 code of an MXFP4 block (src/qwen4_packed.c:97): magnitudes 0, .5, 1, 1.5, 2, 3, 4, 6; bit 3 the
+// sign (code 8 is -0).  Twice the magnitude is an integer: 0, 1, 2, 3, 4, 6, 8, 12.
+__device__ __forceinline__ float pf_e2m1_value(uint32_t code) {
+    const uint32_t m = code & 7u, twice = m < 4u ? m : (m == 4u ? 4u : m == 5u ? 6u : m == 6u ? 8u : 12u);
+    const float v = 0.5f * (float)twice;
+    return code & 8u ? -v : v;
+}
+// E8M0 scale byte: 2^(e - 127); e = 0 is 2^-127 (a subnormal float)
+__device__ __forceinline__ float pf_e8m0_scale(uint32_t e) { return __uint_as_float(e ? e << 23 : 0x00400000u); }
 
 __device__ __forceinline__ uint32_t pf_parity7(uint32_t s) {
     // eighth sign of an IQ2_XXS group: parity of the seven stored ones

@@ -77,10 +77,19 @@ const uint32_t *pf_device_iq2_signed(void) { return upload_constants() ? g_signe
 static bool block_geometry(uint32_t type, size_t *block, size_t *bytes) {
     switch (type) {
     case PF_F32: *block = 1; *bytes = 4; return true;
+    case PF_F16: case PF_BF16: *block = 1; *bytes = 2; return true;
+    case PF_Q8_0: *block = 32; *bytes = 34; return true;
+    case PF_Q2_K: *block = 256; *bytes = 84; return true;
     case PF_Q4_K: *block = 256; *bytes = 144; return true;
     case PF_IQ2_XXS: *block = 256; *bytes = 66; return true;
+    case PF_MXFP4: *block = 32; *bytes = 17; return true;
     default: return false;
     }
+}
+
+// Formats stored split on the device (payloads, then scales): bytes of a block's leading scale, else 0.
+static size_t split_header_bytes(uint32_t type) {
+    return type == PF_IQ2_XXS || type == PF_Q8_0 ? 2 : type == PF_MXFP4 ? 1 : 0;
 }
 
 extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const host_weights[8], const size_t bytes[8],
@@ -112,11 +121,13 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         m->k_logical[a] = (int)k_logical[a];
         m->n_out[a] = (int)n_out[a];
         m->blocks_per_row[a] = (int)blocks_per_row;
-        if (desc->type[a] == PF_IQ2_XXS) {
-            // device layout: every block's 64-byte payload, then every block's half scale
-            m->row_bytes[a] = blocks_per_row * 64;
-            m->scale_offset[a] = (blocks_per_row * rows * 64 + 255) & ~(size_t)255;
-            m->bytes[a] = m->scale_offset[a] + blocks_per_row * rows * 2 + 4;   // the prefill loader reads the dword around a scale
+        const size_t head = split_header_bytes(desc->type[a]);
+        if (head) {
+            // device layout: every block's payload (64, 32 or 16 bytes), then every block's scale
+            const size_t payload = size - head;
+            m->row_bytes[a] = blocks_per_row * payload;
+            m->scale_offset[a] = (blocks_per_row * rows * payload + 255) & ~(size_t)255;
+            m->bytes[a] = m->scale_offset[a] + blocks_per_row * rows * head + 4;   // the prefill loader reads the dword around a scale
         } else {
             m->row_bytes[a] = blocks_per_row * size;
             m->bytes[a] = gguf_bytes[a];
@@ -128,13 +139,20 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
     m->iq2_signed = g_signed;
     for (int a = 0; a < 8; a++) {
         hipError_t e = hipMalloc((void **)&m->w[a], m->bytes[a]);
-        if (e == hipSuccess && desc->type[a] == PF_IQ2_XXS) {
+        const size_t head = split_header_bytes(desc->type[a]);
+        if (e == hipSuccess && head) {
             uint8_t *staging = nullptr;
+            size_t block, size;
+            block_geometry(desc->type[a], &block, &size);
             e = hipMalloc((void **)&staging, gguf_bytes[a]);
             if (e == hipSuccess) e = hipMemcpy(staging, host_weights[a], gguf_bytes[a], hipMemcpyHostToDevice);
             if (e == hipSuccess) {
-                pf_launch_iq2_split(staging, m->w[a], reinterpret_cast<uint16_t *>(m->w[a] + m->scale_offset[a]),
-                                    gguf_bytes[a] / 66, nullptr);
+                if (desc->type[a] == PF_IQ2_XXS)
+                    pf_launch_iq2_split(staging, m->w[a], reinterpret_cast<uint16_t *>(m->w[a] + m->scale_offset[a]),
+                                        gguf_bytes[a] / 66, nullptr);
+                else
+                    pf_launch_block_split(staging, m->w[a], m->w[a] + m->scale_offset[a], gguf_bytes[a] / size,
+                                          (int)size, (int)head, nullptr);
                 e = hipDeviceSynchronize();
             }
             if (staging) (void)hipFree(staging);
@@ -416,6 +434,15 @@ static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_
     }
     HIP_TRY(hipGetLastError());
     return PF_HIP_OK;
+}
+
+// Which kernels a forward of `tokens` tokens (rows 16-byte aligned) runs: 1 the decode kernels,
+// 2 the matrix-core prefill kernels, 0 the general kernels.
+extern "C" int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t tokens) {
+    if (!moe || !work || work->force_general) return 0;
+    if (moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS) return 1;
+    if (moe->prefill_ready && work->down && tokens > PF_DECODE_MAX_TOKENS) return 2;
+    return 0;
 }
 
 // Enqueue only: no allocation, no synchronisation, no memset; safe under stream capture.
@@ -931,8 +958,7 @@ extern "C" int pf_hip_stack_time_forwards(const PfHipMoe *const *moes, PfHipWork
 extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
                                          float *d_y, size_t tokens, size_t iters, float stage_ms[4]) {
     if (!moe || !work || !d_x || !d_y || !n_inputs || !stage_ms || !iters) return PF_HIP_E_ARGUMENT;
-    const bool decode = moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS && !work->force_general;
-    const int stages = decode ? 3 : 4;
+    const int stages = pf_hip_moe_kernel_family(moe, work, tokens) == 1 ? 3 : 4;
     float previous = 0.0f;
     for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
     for (int j = 0; j < stages; j++) {

@@ -585,6 +585,27 @@ void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_
                        d_payload, d_scales, blocks);
 }
 
+// The same for any format whose block leads with its scale (Q8_0: 2 + 32 bytes, MXFP4: 1 + 16): one
+// byte per thread.
+__global__ void pf_k_block_split(const uint8_t *gguf, uint8_t *payload, uint8_t *scales, size_t blocks, int block_bytes,
+                                 int header_bytes) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t b = i / block_bytes;
+    const int h = (int)(i % block_bytes);
+    if (b >= blocks) return;
+    const uint8_t v = gguf[i];
+    if (h < header_bytes) scales[b * header_bytes + h] = v;
+    else payload[b * (block_bytes - header_bytes) + (h - header_bytes)] = v;
+}
+
+void pf_launch_block_split(const uint8_t *d_gguf, uint8_t *d_payload, uint8_t *d_scales, size_t blocks,
+                           int block_bytes, int header_bytes, hipStream_t stream) {
+    const size_t threads = blocks * block_bytes;
+    if (!threads) return;
+    hipLaunchKernelGGL(pf_k_block_split, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, d_gguf,
+                       d_payload, d_scales, blocks, block_bytes, header_bytes);
+}
+
 // ---- dispatch ----------------------------------------------------------------------------------------
 static bool pow2_between(uint32_t v, uint32_t lo, uint32_t hi) { return v >= lo && v <= hi && (v & (v - 1)) == 0; }
 

@@ -2,7 +2,7 @@
 //
 // One lane owns one output and walks k upwards, multiplying and adding without
 // contraction, exactly as src/qwen4_packed.c:164-179 does on the CPU; the decode
-// is the per-element arithmetic of src/qwen4_packed.c:67-115.  Results are
+// is the per-element arithmetic of src/qwen4_packed.c:67-122 (all eight formats).  Results are
 // bit-identical to the reference.  These kernels serve qw4_packed_matmul,
 // qw4_packed_decode_row and the tie fallback of the router; they are not the
 // throughput path.
@@ -22,7 +22,34 @@ __device__ __forceinline__ float exact_value(uint32_t type, const uint8_t *row, 
         uint32_t bits = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
         return __uint_as_float(bits);
     }
+    if (type == PF_BF16) {
+        const uint8_t *p = row + 2 * (size_t)column;
+        return __uint_as_float(((uint32_t)p[0] | ((uint32_t)p[1] << 8)) << 16);
+    }
+    if (type == PF_F16) {
+        const uint8_t *p = row + 2 * (size_t)column;
+        return pf_half_bits_to_float((uint32_t)p[0] | ((uint32_t)p[1] << 8));
+    }
+    if (type == PF_Q8_0) {   // src/qwen4_packed.c:80-85
+        const uint8_t *b = row + (size_t)(column >> 5) * 34;
+        const int code = (int)(int8_t)b[2 + (column & 31)];
+        return mul_rn(pf_half_bits_to_float((uint32_t)b[0] | ((uint32_t)b[1] << 8)), (float)code);
+    }
+    if (type == PF_MXFP4) {  // src/qwen4_packed.c:94-101
+        const uint8_t *b = row + (size_t)(column >> 5) * 17;
+        const int l = column & 31;
+        const uint32_t code = (b[1 + (l & 15)] >> ((l >> 4) * 4)) & 15u;
+        return mul_rn(pf_e2m1_value(code), pf_e8m0_scale(b[0]));
+    }
     const int lane = column & 255, blk = column >> 8;
+    if (type == PF_Q2_K) {   // src/qwen4_packed.c:116-121
+        const uint8_t *b = row + (size_t)blk * 84;
+        const uint32_t sm = b[lane >> 4];
+        const uint32_t code = (b[16 + (lane >> 7) * 32 + (lane & 31)] >> (2 * ((lane & 127) >> 5))) & 3u;
+        const float d = pf_half_bits_to_float((uint32_t)b[80] | ((uint32_t)b[81] << 8));
+        const float dmin = pf_half_bits_to_float((uint32_t)b[82] | ((uint32_t)b[83] << 8));
+        return sub_rn(mul_rn(mul_rn(d, (float)(sm & 15u)), (float)code), mul_rn(dmin, (float)(sm >> 4)));
+    }
     if (type == PF_Q4_K) {
         const uint8_t *b = row + (size_t)blk * 144, *sc = b + 4;
         const int g = lane >> 5;

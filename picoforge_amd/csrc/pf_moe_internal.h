@@ -140,6 +140,8 @@ bool pf_decode_supported(const PfHipMoeDesc &d);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);
+void pf_launch_block_split(const uint8_t *d_gguf, uint8_t *d_payload, uint8_t *d_scales, size_t blocks,
+                           int block_bytes, int header_bytes, hipStream_t stream);
 // pf_moe_prefill.hip
 bool pf_prefill_supported(const PfHipMoeDesc &d);
 void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);

@@ -5,9 +5,10 @@
 // of a row multiplies zeros).  Shapes that the specialised decode and prefill
 // kernels cover are dispatched there instead.
 //
-// Device layout of the tensors: F32 and Q4_K keep GGUF's bytes.  IQ2_XXS tensors
-// are split at upload into 64-byte block payloads (all blocks, row-major)
-// followed by the blocks' half scales, so that payload loads are aligned.
+// Device layout of the tensors: F32, F16, BF16, Q4_K and Q2_K keep GGUF's bytes.
+// IQ2_XXS, Q8_0 and MXFP4 tensors are split at upload into the blocks' payloads
+// (64, 32 and 16 bytes; all blocks, row-major) followed by the blocks' scales
+// (half, half, one byte), so that payload loads are aligned.
 #include "pf_moe_internal.h"
 
 // ---- row products: packed row . x (LDS) -----------------------------------------
@@ -93,17 +94,106 @@ __device__ __forceinline__ float dot_row_iq2(const uint8_t *payload, const uint1
     return acc;
 }
 
+// F16 / BF16 rows: two values per lane and step.
+template <bool BF>
+__device__ __forceinline__ float dot_row_16(const uint8_t *row, const float *x, int K, int lane) {
+    const uint16_t *w = reinterpret_cast<const uint16_t *>(row);
+    float acc = 0.0f;
+    for (int k = lane; k < K; k += PF_WAVE) {
+        const float v = BF ? __uint_as_float((uint32_t)w[k] << 16) : pf_half_bits_to_float(w[k]);
+        acc = fmaf(v, x[k], acc);
+    }
+    return acc;
+}
+
+// Q8_0, device layout: 32 code bytes per block (aligned), the half scales apart.  Lane l takes block l.
+__device__ __forceinline__ float dot_row_q8(const uint8_t *payload, const uint16_t *scales, const float *x, int nblk,
+                                            int lane) {
+    float acc = 0.0f;
+    for (int b = lane; b < nblk; b += PF_WAVE) {
+        const uint4 lo = *reinterpret_cast<const uint4 *>(payload + 32 * (size_t)b);
+        const uint4 hi = *reinterpret_cast<const uint4 *>(payload + 32 * (size_t)b + 16);
+        const uint32_t q[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        const float *xb = x + 32 * b;
+        float g = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 8; w++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) g = fmaf((float)(int)(int8_t)(q[w] >> (8 * c)), xb[4 * w + c], g);
+        acc = fmaf(pf_half_bits_to_float(scales[b]), g, acc);
+    }
+    return acc;
+}
+
+// MXFP4, device layout: 16 nibble bytes per block (aligned), the scale bytes apart.  Low nibbles are
+// values 0..15 of the block, high nibbles 16..31.
+__device__ __forceinline__ float dot_row_mxfp4(const uint8_t *payload, const uint8_t *scales, const float *x, int nblk,
+                                               int lane) {
+    float acc = 0.0f;
+    for (int b = lane; b < nblk; b += PF_WAVE) {
+        const uint4 p = *reinterpret_cast<const uint4 *>(payload + 16 * (size_t)b);
+        const uint32_t q[4] = {p.x, p.y, p.z, p.w};
+        const float *xb = x + 32 * b;
+        float g = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint32_t byte = (q[w] >> (8 * c)) & 255u;
+                g = fmaf(pf_e2m1_value(byte & 15u), xb[4 * w + c], g);
+                g = fmaf(pf_e2m1_value(byte >> 4), xb[16 + 4 * w + c], g);
+            }
+        acc = fmaf(pf_e8m0_scale(scales[b]), g, acc);
+    }
+    return acc;
+}
+
+// Q2_K (GGUF bytes): lane l takes the group of 16 values l of the row: 16 code bytes of one bit plane,
+// one scale | min << 4 byte.  Group g of a block: half g / 8, plane (g % 8) / 2, bytes (g % 2) * 16 ...
+__device__ __forceinline__ float dot_row_q2k(const uint8_t *row, const float *x, int nblk, int lane) {
+    float acc = 0.0f;
+    for (int gi = lane; gi < nblk * 16; gi += PF_WAVE) {
+        const uint8_t *blk = row + (size_t)(gi >> 4) * 84;
+        const int g = gi & 15, plane = (g & 7) >> 1;
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(blk + 16 + (g >> 3) * 32 + (g & 1) * 16);   // 4-byte aligned
+        const uint32_t q[4] = {p[0], p[1], p[2], p[3]};
+        const uint32_t sm = blk[g], dd = *reinterpret_cast<const uint32_t *>(blk + 80);
+        const float *xg = x + 16 * gi;
+        float dotq = 0.0f, sumx = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const float xv = xg[4 * w + c];
+                dotq = fmaf((float)((q[w] >> (8 * c + 2 * plane)) & 3u), xv, dotq);
+                sumx += xv;
+            }
+        acc += pf_half_bits_to_float(dd & 0xffffu) * (float)(sm & 15u) * dotq -
+               pf_half_bits_to_float(dd >> 16) * (float)(sm >> 4) * sumx;
+    }
+    return acc;
+}
+
 // Row n of expert e of tensor t against x (LDS, padded to the stored length).
 __device__ __forceinline__ float dot_tensor_row(const PfKernelArgs &a, int t, size_t e, size_t n, const float *x,
                                                 int lane, const uint64_t *grid) {
     const uint8_t *row = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t];
     float v;
-    if (a.type[t] == PF_F32) v = dot_row_f32(row, x, a.k_logical[t], lane);
-    else if (a.type[t] == PF_Q4_K) v = dot_row_q4k(row, x, a.blocks_per_row[t], lane);
-    else {
-        const uint16_t *scales = reinterpret_cast<const uint16_t *>(a.w[t] + a.scale_offset[t]) +
-                                 (e * a.n_out[t] + n) * a.blocks_per_row[t];
-        v = dot_row_iq2(row, scales, x, a.blocks_per_row[t], lane, grid);
+    const size_t first_block = (e * a.n_out[t] + n) * a.blocks_per_row[t];   // of the row, for the formats stored split
+    const uint8_t *scales = a.w[t] + a.scale_offset[t];
+    switch (a.type[t]) {
+    case PF_F32: v = dot_row_f32(row, x, a.k_logical[t], lane); break;
+    case PF_F16: v = dot_row_16<false>(row, x, a.k_logical[t], lane); break;
+    case PF_BF16: v = dot_row_16<true>(row, x, a.k_logical[t], lane); break;
+    case PF_Q4_K: v = dot_row_q4k(row, x, a.blocks_per_row[t], lane); break;
+    case PF_Q2_K: v = dot_row_q2k(row, x, a.blocks_per_row[t], lane); break;
+    case PF_Q8_0:
+        v = dot_row_q8(row, reinterpret_cast<const uint16_t *>(scales) + first_block, x, a.blocks_per_row[t], lane);
+        break;
+    case PF_MXFP4: v = dot_row_mxfp4(row, scales + first_block, x, a.blocks_per_row[t], lane); break;
+    default:
+        v = dot_row_iq2(row, reinterpret_cast<const uint16_t *>(scales) + first_block, x, a.blocks_per_row[t], lane,
+                        grid);
     }
     return pf_wave_sum(v);
 }

@@ -150,3 +150,85 @@ void pf_synth_iq2xxs_uniform(unsigned char *out, size_t blocks, uint64_t seed, f
         }
     }
 }
+
+/* ---- formats of the real checkpoints' other tensors ---------------------------------------- */
+static void normals(float *v, int n, uint64_t seed, size_t first, float std) {
+    for (int i = 0; i < n / 2; i++) {
+        normal_pair(seed, first / 2 + (size_t)i, &v[2 * i], &v[2 * i + 1]);
+        v[2 * i] *= std;
+        v[2 * i + 1] *= std;
+    }
+}
+
+/* Q8_0 blocks (half d, 32 signed bytes) of N(0, std) weights: d = largest magnitude / 127 */
+void pf_synth_q8_0_normal(unsigned char *out, size_t blocks, uint64_t seed, float std) {
+#pragma omp parallel for schedule(static)
+    for (size_t b = 0; b < blocks; b++) {
+        float v[32], top = 0;
+        normals(v, 32, seed, b * 32, std);
+        for (int i = 0; i < 32; i++) top = fmaxf(top, fabsf(v[i]));
+        uint16_t dh = half_bits(top / 127.0f);
+        float d = half_float(dh);
+        unsigned char *p = out + 34 * b;
+        p[0] = (unsigned char)(dh & 255u); p[1] = (unsigned char)(dh >> 8);
+        for (int i = 0; i < 32; i++) p[2 + i] = (unsigned char)(signed char)(d > 0 ? clampi((int)lrintf(v[i] / d), -127, 127) : 0);
+    }
+}
+
+/* Q2_K super-blocks (16 scale | min << 4 bytes, 64 bytes of 2-bit codes, half d, half dmin) of
+ * N(0, std) weights: per group of 16 a step (hi - lo) / 3 and an offset -lo, both in 4 bits. */
+void pf_synth_q2k_normal(unsigned char *out, size_t blocks, uint64_t seed, float std) {
+#pragma omp parallel for schedule(static)
+    for (size_t b = 0; b < blocks; b++) {
+        float v[256], step[16], lowest[16], max_step = 0, max_low = 0;
+        normals(v, 256, seed, b * 256, std);
+        for (int g = 0; g < 16; g++) {
+            float lo = 0, hi = 0;
+            for (int i = 0; i < 16; i++) { lo = fminf(lo, v[16 * g + i]); hi = fmaxf(hi, v[16 * g + i]); }
+            step[g] = (hi - lo) / 3.0f;
+            lowest[g] = -lo;
+            max_step = fmaxf(max_step, step[g]);
+            max_low = fmaxf(max_low, lowest[g]);
+        }
+        uint16_t dh = half_bits(max_step / 15.0f), mh = half_bits(max_low / 15.0f);
+        float d = half_float(dh), dmin = half_float(mh);
+        unsigned char *p = out + 84 * b;
+        memset(p, 0, 84);
+        for (int g = 0; g < 16; g++) {
+            unsigned sc = d > 0 ? (unsigned)clampi((int)lrintf(step[g] / d), 0, 15) : 0;
+            unsigned mn = dmin > 0 ? (unsigned)clampi((int)lrintf(lowest[g] / dmin), 0, 15) : 0;
+            p[g] = (unsigned char)(sc | (mn << 4));
+            float s = d * (float)sc, offset = dmin * (float)mn;
+            for (int i = 0; i < 16; i++) {
+                int lane = 16 * g + i, q = s > 0 ? clampi((int)lrintf((v[lane] + offset) / s), 0, 3) : 0;
+                p[16 + lane / 128 * 32 + lane % 32] |= (unsigned char)(q << (2 * (lane % 128 / 32)));
+            }
+        }
+        p[80] = (unsigned char)(dh & 255u); p[81] = (unsigned char)(dh >> 8);
+        p[82] = (unsigned char)(mh & 255u); p[83] = (unsigned char)(mh >> 8);
+    }
+}
+
+/* MXFP4 blocks (one E8M0 scale byte, 32 E2M1 codes, values 0..15 in the low nibbles) of N(0, std)
+ * weights: the scale is the power of two that brings the largest magnitude to at most 6. */
+void pf_synth_mxfp4_normal(unsigned char *out, size_t blocks, uint64_t seed, float std) {
+    static const float level[8] = {0, .5f, 1, 1.5f, 2, 3, 4, 6};
+#pragma omp parallel for schedule(static)
+    for (size_t b = 0; b < blocks; b++) {
+        float v[32], top = 0;
+        normals(v, 32, seed, b * 32, std);
+        for (int i = 0; i < 32; i++) top = fmaxf(top, fabsf(v[i]));
+        int e = top > 0 ? clampi((int)ceilf(log2f(top / 6.0f)) + 127, 1, 252) : 127;
+        float scale = ldexpf(1.0f, e - 127);
+        unsigned char *p = out + 17 * b;
+        memset(p, 0, 17);
+        p[0] = (unsigned char)e;
+        for (int i = 0; i < 32; i++) {
+            float a = fabsf(v[i]) / scale;
+            int best = 0;
+            for (int c = 1; c < 8; c++) if (fabsf(a - level[c]) < fabsf(a - level[best])) best = c;
+            unsigned code = (unsigned)best | (v[i] < 0 ? 8u : 0u);
+            p[1 + i % 16] |= (unsigned char)(code << ((i / 16) * 4));
+        }
+    }
+}

@@ -31,10 +31,10 @@ static bool intersects(const void *a, size_t na, const void *b, size_t nb) {
     uintptr_t pa = (uintptr_t)a, pb = (uintptr_t)b;
     return na && nb && pa < pb + nb && pb < pa + na;
 }
-static bool executable(uint32_t type) { return type == 0 || type == 12 || type == 16; }
+const GgufFormat *gguf_format(uint32_t id);
+static bool executable(uint32_t type) { return gguf_format(type) != NULL; }
 
-/* Block geometry of every format the reference registers (src/gguf.c:12-16);
- * only F32, Q4_K and IQ2_XXS have kernels here. */
+/* Block geometry of every format the reference registers (src/gguf.c:12-16); all have kernels here. */
 const GgufFormat *gguf_format(uint32_t id) {
     static const GgufFormat formats[] = {
         {0, "F32", 1, 4},      {1, "F16", 1, 2},          {8, "Q8_0", 32, 34},   {10, "Q2_K", 256, 84},

@@ -35,13 +35,22 @@ class LayerWeights:
     def nbytes(self):
         return sum(b.size for b in self.raw)
 
+    # the two profiles of real checkpoints (src/qwen4_config.c:197-216, src/qwen4_weights.c:91-99):
+    # routed gate/up, routed down, shared expert
+    PROFILE = {"q2": (abi.GGUF_IQ2_XXS, abi.GGUF_Q2_K, abi.GGUF_Q8_0), "q4": (abi.GGUF_Q4_K, abi.GGUF_MXFP4, abi.GGUF_Q8_0)}
+
     @classmethod
-    def synthetic(cls, cfg, expert_type, seed, std=0.02, shared_type=None, router_std=None, iq2_d=2.0 ** -12):
+    def synthetic(cls, cfg, expert_type, seed, std=0.02, shared_type=None, router_std=None, iq2_d=2.0 ** -12,
+                  down_type=None):
         """Seeded weights: routers F32 N(0, router_std or std); expert tensors N(0, std) quantised to
-        Q4_K, IQ2_XXS blocks drawn uniformly, or plain F32."""
+        Q4_K, Q8_0, Q2_K or MXFP4, IQ2_XXS blocks drawn uniformly, or plain F32 / F16 / BF16.
+        expert_type may name a checkpoint profile, "q2" or "q4"."""
         synth = Synth()
+        if expert_type in cls.PROFILE:
+            expert_type, down_type, shared_type = cls.PROFILE[expert_type]
         shared_type = expert_type if shared_type is None else shared_type
-        types = [abi.GGUF_F32, expert_type, expert_type, expert_type, shared_type, shared_type, shared_type,
+        down_type = expert_type if down_type is None else down_type
+        types = [abi.GGUF_F32, expert_type, expert_type, down_type, shared_type, shared_type, shared_type,
                  abi.GGUF_F32]
         raw = []
         for j, (gtype, (ks, kl, n, e)) in enumerate(zip(types, shapes(cfg))):
@@ -54,6 +63,12 @@ class LayerWeights:
                 raw.append(synth.q4k_normal(count // 256, stream, std))
             elif gtype == abi.GGUF_IQ2_XXS:
                 raw.append(synth.iq2xxs_uniform(count // 256, stream, iq2_d))
+            elif gtype in (abi.GGUF_Q8_0, abi.GGUF_Q2_K, abi.GGUF_MXFP4):
+                raw.append(synth.quantised_normal(gtype, count, stream, std))
+            elif gtype == abi.GGUF_F16:
+                raw.append(synth.normal((count,), stream, std).astype(np.float16).view(np.uint8))
+            elif gtype == abi.GGUF_BF16:
+                raw.append((synth.normal((count,), stream, std).view(np.uint32) >> 16).astype(np.uint16).view(np.uint8))
             else:
                 raise ValueError(gtype)
         return cls(cfg, raw, types)

@@ -17,15 +17,27 @@ def measured_config():
     return abi.moe_config(HIDDEN, EXPERTS, TOP_K, INTER, SHARED_INTER)
 
 
+def layer_bytes(expert_type, cfg=None):
+    """Stored bytes of one routed expert's gate + up rows and down rows, of the shared expert's, and of
+    the two routers.  expert_type: a GGUF type for every expert tensor, or a checkpoint profile
+    ("q2": IQ2_XXS gate/up, Q2_K down, Q8_0 shared; "q4": Q4_K gate/up, MXFP4 down, Q8_0 shared)."""
+    cfg = cfg or measured_config()
+    gate, down, shared = LayerWeights.PROFILE.get(expert_type, (expert_type,) * 3)
+
+    def size(gtype, k, n):
+        block, nbytes = abi.BLOCK[gtype]
+        return k // block * nbytes * n
+    h, i, s = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate
+    return {"gate_up": 2 * size(gate, h, i), "down": size(down, cfg.down_physical, h),
+            "shared_gate_up": 2 * size(shared, h, s), "shared_down": size(shared, s, h),
+            "routers": (cfg.experts + 1) * h * 4}
+
+
 def algorithmic_bytes_per_token(expert_type, unique_experts=TOP_K, cfg=None):
     """Bytes one decoded token must read: the selected experts' three tensors, the shared
     expert's, both routers (F32).  Q4_K: 23 666 688, IQ2_XXS: 13 123 584 at the measured shape."""
-    cfg = cfg or measured_config()
-    block, size = abi.BLOCK[expert_type]
-    per_expert = (2 * cfg.intermediate * cfg.hidden_size + cfg.hidden_size * cfg.down_physical) // block * size
-    shared = (2 * cfg.shared_intermediate * cfg.hidden_size + cfg.hidden_size * cfg.shared_intermediate) // block * size
-    routers = (cfg.experts + 1) * cfg.hidden_size * 4
-    return unique_experts * per_expert + shared + routers
+    b = layer_bytes(expert_type, cfg)
+    return unique_experts * (b["gate_up"] + b["down"]) + b["shared_gate_up"] + b["shared_down"] + b["routers"]
 
 
 def router_logits64(weights, x):

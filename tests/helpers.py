@@ -93,3 +93,31 @@ def call_decode(api, raw, gtype, k_storage, rows, row, experts=1, expert=0):
     err = abi.Qwen4Error()
     st = api.decode_row(C.byref(view), expert, row, out.ctypes.data, k_storage, C.byref(err))
     return st, out
+
+
+def random_blocks(gtype, elements, rng, scale=0.125):
+    """Random packed bytes of `elements` values in a format, every decoded value finite: block scales are
+    halves drawn from +-scale (Q8_0, Q2_K, Q4_K, IQ2_XXS), exponents 110..140 (MXFP4), finite patterns
+    (F16, BF16), N(0, 1) (F32)."""
+    block, size = abi.BLOCK[gtype]
+    assert elements % block == 0
+    n = elements // block
+    if gtype == abi.GGUF_F32:
+        return rng.normal(0, 1, elements).astype(np.float32).view(np.uint8)
+    if gtype in (abi.GGUF_F16, abi.GGUF_BF16):
+        v = rng.normal(0, 1, elements).astype(np.float32)
+        if gtype == abi.GGUF_F16:
+            return v.astype(np.float16).view(np.uint8)
+        return (v.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+    raw = rng.integers(0, 256, (n, size), dtype=np.uint8)
+    half = lambda: rng.uniform(-scale, scale, (n, 1)).astype(np.float16).view(np.uint8)  # noqa: E731
+    if gtype == abi.GGUF_Q2_K:
+        raw[:, 80:82] = half()
+        raw[:, 82:84] = half()
+    elif gtype == abi.GGUF_MXFP4:
+        raw[:, 0] = rng.integers(110, 141, n, dtype=np.uint8)
+    else:
+        raw[:, 0:2] = half()
+        if gtype == abi.GGUF_Q4_K:
+            raw[:, 2:4] = half()
+    return raw.reshape(-1)

@@ -1,0 +1,93 @@
+"""GPU parity on the formats real checkpoints use beside Q4_K and IQ2_XXS: F16, BF16, Q8_0 (shared
+expert), Q2_K and MXFP4 (routed down projections).  Operators in reference order are bit-exact; the MoE
+block on the two checkpoint profiles (src/qwen4_config.c:197-216: IQ2_XXS gate/up + Q2_K down, Q4_K
+gate/up + MXFP4 down, Q8_0 shared expert in both) is held to the path's bar against the CPU oracle."""
+import struct
+
+import numpy as np
+import pytest
+
+import picoforge_amd as pf
+from picoforge_amd import abi
+
+from helpers import assert_parity, call_decode, call_matmul, forward_with, make_layer_inputs, random_blocks
+
+pytestmark = pytest.mark.gpu
+ALL = sorted(abi.BLOCK)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+@pytest.mark.parametrize("gtype", ALL)
+def test_decode_and_product_bit_exact_on_every_format(product, oracle, gtype):
+    print(f"case format {abi.FORMAT_NAME[gtype]}", flush=True)
+    rng = np.random.default_rng(500 + gtype)
+    rows, k = 9, 768
+    raw = random_blocks(gtype, rows * k, rng, scale=1.0)
+    for row in range(rows):
+        st0, want = call_decode(oracle, raw, gtype, k, rows, row)
+        st1, got = call_decode(product, raw, gtype, k, rows, row)
+        assert st0 == st1 == abi.QW4_OK
+        np.testing.assert_array_equal(bits(got), bits(want))
+    x = rng.uniform(-1, 1, (5, 640)).astype(np.float32)
+    for expert in range(3):   # logical K 640 of 768 stored: padding is never read
+        st0, want = call_matmul(oracle, raw, gtype, k, 3, 3, expert, x, k_logical=640)
+        st1, got = call_matmul(product, raw, gtype, k, 3, 3, expert, x, k_logical=640)
+        assert st0 == st1 == abi.QW4_OK
+        np.testing.assert_array_equal(bits(got), bits(want))
+
+
+def test_closed_forms_of_the_reference_tests(product):
+    """tests/test_qwen4_packed.py:224-237, :362-367 through the device decoders."""
+    def decode(raw, gtype, columns=256, rows=1):
+        raw = np.frombuffer(bytes(raw), dtype=np.uint8).copy()
+        return np.stack([call_decode(product, raw, gtype, columns, rows, r)[1] for r in range(rows)])
+    raw = bytes([0x23]) * 16 + bytes([0xe4]) * 64 + struct.pack("<ee", 1, 0.5)
+    np.testing.assert_array_equal(decode(raw, abi.GGUF_Q2_K)[0], np.tile(np.repeat([-1, 2, 5, 8], 32), 2))
+    codes = np.arange(-128, 128, dtype=np.int16)
+    raw = b"".join(struct.pack("<e", 0.125) + codes[s:s + 32].astype("i1").tobytes() for s in range(0, 256, 32))
+    np.testing.assert_array_equal(bits(decode(raw, abi.GGUF_Q8_0)[0]), bits(codes.astype(np.float32) * 0.125))
+    nib = bytes(i | ((15 - i) << 4) for i in range(16))
+    got = decode(b"".join(bytes([e]) + nib for e in (0, 127, 252)), abi.GGUF_MXFP4, 32, 3)
+    table = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0.0, -.5, -1, -1.5, -2, -3, -4, -6], dtype=np.float32)
+    for row, e in enumerate((0, 127, 252)):
+        want = np.concatenate([table, table[::-1]]) * np.float32(2.0 ** (e - 127))
+        np.testing.assert_array_equal(bits(got[row]), bits(want))
+    r = np.frombuffer(bytes([254]) + nib, dtype=np.uint8).copy()
+    assert call_decode(product, r, abi.GGUF_MXFP4, 32, 1, 0)[0] == abi.QW4_NONFINITE
+
+
+PROFILES = [
+    # hidden, experts, top_k, inter, shared_inter, down_physical, profile, tokens
+    (256, 8, 3, 256, 256, 256, "q2", 5),
+    (512, 16, 4, 512, 256, 512, "q4", 3),
+    (256, 8, 3, 160, 96, 256, "q2", 2),      # logical K 160 stored in 256 (the checkpoint's 640 in 768)
+    (512, 32, 6, 256, 256, 256, "q4", 1),
+    (512, 32, 6, 256, 256, 256, "q2", 40),   # a chunk
+]
+
+
+@pytest.mark.parametrize("h,e,k,i,s,dp,profile,tokens", PROFILES)
+def test_checkpoint_profiles_match_oracle(product, oracle, h, e, k, i, s, dp, profile, tokens):
+    print(f"case profile {profile} h={h} e={e} k={k} i={i} s={s} down_physical={dp} T={tokens}", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s, down_physical=dp)
+    if profile == "q4" and dp != i:
+        pytest.skip("MXFP4 down tensors are stored at the logical width")
+    if s % 32 or (profile == "q2" and i % 32):
+        pytest.skip("block multiple")
+    weights, x = make_layer_inputs(cfg, profile, tokens, seed=700 + h + tokens)
+    want = forward_with(oracle, cfg, weights, x)
+    got = forward_with(product, cfg, weights, x)
+    worst = assert_parity(*got, *want, label=f"profile {profile}")
+    print(f"  max abs err {worst:.2e}", flush=True)
+
+
+@pytest.mark.parametrize("gtype", [abi.GGUF_F16, abi.GGUF_BF16, abi.GGUF_Q8_0])
+def test_uniform_layers_of_the_plain_formats(product, oracle, gtype):
+    cfg = abi.moe_config(128, 8, 2, 64, 32)
+    weights, x = make_layer_inputs(cfg, gtype, 6, seed=800 + gtype, std=0.1)
+    want = forward_with(oracle, cfg, weights, x)
+    got = forward_with(product, cfg, weights, x)
+    assert_parity(*got, *want, label=abi.FORMAT_NAME[gtype])
