@@ -148,6 +148,44 @@ __device__ __forceinline__ void wseg_load<PF_IQ2_XXS>(WSeg<PF_IQ2_XXS> &w, const
     w.dbits = scales[(e * a.n_out[t] + n) * a.blocks_per_row[t] + (seg >> 2)];
 }
 
+// Q8_0, device layout (32 code bytes per block, half scales apart): a segment is two blocks
+template <> struct WSeg<PF_Q8_0> { uint4 q[4]; uint32_t d2; };
+template <>
+__device__ __forceinline__ void wseg_load<PF_Q8_0>(WSeg<PF_Q8_0> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
+                                                   int seg) {
+    const uint4 *row = reinterpret_cast<const uint4 *>(a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + 64 * (size_t)seg);
+#pragma unroll
+    for (int i = 0; i < 4; i++) w.q[i] = row[i];
+    const uint16_t *scales = reinterpret_cast<const uint16_t *>(a.w[t] + a.scale_offset[t]);
+    w.d2 = *reinterpret_cast<const uint32_t *>(scales + (e * a.n_out[t] + n) * a.blocks_per_row[t] + 2 * seg);
+}
+
+// MXFP4, device layout (16 nibble bytes per block, scale bytes apart): a segment is two blocks
+template <> struct WSeg<PF_MXFP4> { uint4 q[2]; uint32_t e2; };
+template <>
+__device__ __forceinline__ void wseg_load<PF_MXFP4>(WSeg<PF_MXFP4> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
+                                                    int seg) {
+    const uint4 *row = reinterpret_cast<const uint4 *>(a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + 32 * (size_t)seg);
+    w.q[0] = row[0];
+    w.q[1] = row[1];
+    const uint8_t *scales = a.w[t] + a.scale_offset[t] + (e * a.n_out[t] + n) * a.blocks_per_row[t] + 2 * seg;
+    w.e2 = *reinterpret_cast<const uint16_t *>(scales);
+}
+
+// Q2_K, GGUF bytes (84-byte blocks, 4-byte aligned): a segment is a quarter of a block: 32 code
+// bytes read at two bit planes, four scale | min << 4 bytes, the block's d and dmin
+template <> struct WSeg<PF_Q2_K> { uint32_t q[8], sm, dd; };
+template <>
+__device__ __forceinline__ void wseg_load<PF_Q2_K>(WSeg<PF_Q2_K> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
+                                                   int seg) {
+    const uint8_t *blk = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + (size_t)(seg >> 2) * 84;
+    const uint32_t *codes = reinterpret_cast<const uint32_t *>(blk + 16 + 32 * ((seg & 3) >> 1));
+#pragma unroll
+    for (int i = 0; i < 8; i++) w.q[i] = codes[i];
+    w.sm = *reinterpret_cast<const uint32_t *>(blk + 4 * (seg & 3));
+    w.dd = *reinterpret_cast<const uint32_t *>(blk + 80);
+}
+
 __device__ __forceinline__ float half_bits(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
 }
@@ -216,6 +254,94 @@ __device__ __forceinline__ float wseg_dot<PF_IQ2_XXS>(const WSeg<PF_IQ2_XXS> &w,
         acc[gg] = x.step[gg] * (float)(2u * (word >> 28) + 1u) * (float)(a0 + (a1 << 7) + (a2 << 14));
     }
     return half_bits(w.dbits) * 0.125f * (acc[0] + acc[1]);
+}
+
+// Q8_0: signed byte codes against the three digit planes.  A group's integer can reach 2^32, so the
+// top digit's share is added in float (relative error 2^-24 of the group's partial sum).
+template <>
+__device__ __forceinline__ float wseg_dot<PF_Q8_0>(const WSeg<PF_Q8_0> &w, const XSeg &x, int, const uint32_t *) {
+    float out = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        const uint32_t q[8] = {w.q[2 * g].x, w.q[2 * g].y, w.q[2 * g].z, w.q[2 * g].w,
+                               w.q[2 * g + 1].x, w.q[2 * g + 1].y, w.q[2 * g + 1].z, w.q[2 * g + 1].w};
+        int a0 = 0, a1 = 0, a2 = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            a0 = __builtin_amdgcn_sdot4((int)q[i], x.d0[8 * g + i], a0, false);
+            a1 = __builtin_amdgcn_sdot4((int)q[i], x.d1[8 * g + i], a1, false);
+            a2 = __builtin_amdgcn_sdot4((int)q[i], x.d2[8 * g + i], a2, false);
+        }
+        const float total = (float)(a0 + (a1 << 7)) + 16384.0f * (float)a2;
+        out = fmaf(x.step[g] * half_bits((w.d2 >> (16 * g)) & 0xffffu), total, out);
+    }
+    return out;
+}
+
+// MXFP4: four E2M1 codes of a dword as signed bytes holding twice their value (0, 1, 2, 3, 4, 6, 8, 12):
+// one byte permute per sign, merged under the sign bits' byte mask
+__device__ __forceinline__ int e2m1_twice4(uint32_t nibbles) {
+    const uint32_t sel = nibbles & 0x07070707u;
+    const uint32_t pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
+    const uint32_t neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
+    const uint32_t mask = ((nibbles >> 3) & 0x01010101u) * 0xFFu;
+    return (int)((neg & mask) | (pos & ~mask));
+}
+
+template <>
+__device__ __forceinline__ float wseg_dot<PF_MXFP4>(const WSeg<PF_MXFP4> &w, const XSeg &x, int, const uint32_t *) {
+    float out = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        const uint32_t q[4] = {w.q[g].x, w.q[g].y, w.q[g].z, w.q[g].w};
+        int a0 = 0, a1 = 0, a2 = 0;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int lo = e2m1_twice4(q[i] & 0x0F0F0F0Fu), hi = e2m1_twice4((q[i] >> 4) & 0x0F0F0F0Fu);
+            a0 = __builtin_amdgcn_sdot4(lo, x.d0[8 * g + i], a0, false);
+            a1 = __builtin_amdgcn_sdot4(lo, x.d1[8 * g + i], a1, false);
+            a2 = __builtin_amdgcn_sdot4(lo, x.d2[8 * g + i], a2, false);
+            a0 = __builtin_amdgcn_sdot4(hi, x.d0[8 * g + 4 + i], a0, false);
+            a1 = __builtin_amdgcn_sdot4(hi, x.d1[8 * g + 4 + i], a1, false);
+            a2 = __builtin_amdgcn_sdot4(hi, x.d2[8 * g + 4 + i], a2, false);
+        }
+        const float scale = 0.5f * pf_e8m0_scale((w.e2 >> (8 * g)) & 255u);   // the integers are twice the values
+        out = fmaf(x.step[g] * scale, (float)(a0 + (a1 << 7) + (a2 << 14)), out);
+    }
+    return out;
+}
+
+// Q2_K: group gg of the segment reads bit plane 2 * (seg % 2) + gg of the 32 code bytes; bytes 0..15
+// and 16..31 are two sub-groups of 16 with their own scale and minimum, so the sums of the activation
+// integers are taken per sub-group here (dot products with ones).
+template <>
+__device__ __forceinline__ float wseg_dot<PF_Q2_K>(const WSeg<PF_Q2_K> &w, const XSeg &x, int seg, const uint32_t *) {
+    const float d = half_bits(w.dd & 0xffffu), dmin = half_bits(w.dd >> 16);
+    float out = 0.0f;
+#pragma unroll
+    for (int gg = 0; gg < 2; gg++) {
+        const int shift = 2 * (2 * (seg & 1) + gg);
+        float group = 0.0f;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            int c0 = 0, c1 = 0, c2 = 0, s0 = 0, s1 = 0, s2 = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int codes = (int)((w.q[4 * sub + i] >> shift) & 0x03030303u), m = 8 * gg + 4 * sub + i;
+                c0 = __builtin_amdgcn_sdot4(codes, x.d0[m], c0, false);
+                c1 = __builtin_amdgcn_sdot4(codes, x.d1[m], c1, false);
+                c2 = __builtin_amdgcn_sdot4(codes, x.d2[m], c2, false);
+                s0 = __builtin_amdgcn_sdot4(0x01010101, x.d0[m], s0, false);
+                s1 = __builtin_amdgcn_sdot4(0x01010101, x.d1[m], s1, false);
+                s2 = __builtin_amdgcn_sdot4(0x01010101, x.d2[m], s2, false);
+            }
+            const uint32_t sm = (w.sm >> (8 * (2 * gg + sub))) & 255u;
+            group += fmaf(d * (float)(sm & 15u), (float)(c0 + (c1 << 7) + (c2 << 14)),
+                          -(dmin * (float)(sm >> 4)) * (float)(s0 + (s1 << 7) + (s2 << 14)));
+        }
+        out = fmaf(x.step[gg], group, out);
+    }
+    return out;
 }
 
 // sum over `width` neighbouring lanes (power of two, <= 32); result in the lowest lane of each span
@@ -298,13 +424,12 @@ __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int route
 // gate/up tiles leave idle): workgroup `order` of the `per_xcd` on its XCD takes every per_xcd-th
 // (slot, row block) item of that XCD; slot `uniques` is the shared expert.  The loaded values
 // are not used: a wrong guess about the placement costs time, not results.
-template <int FMT>
 __device__ __forceinline__ void prefetch_down(const PfKernelArgs &a, const uint32_t *uniq, int uniques, int order,
                                               int per_xcd, int rows_per_block, int row_blocks) {
     const int xcd = blockIdx.x % 8, per_slot = row_blocks / 8, items = (uniques + 1) * per_slot;
     const int mine = (items - order + per_xcd - 1) / per_xcd;
     const size_t widest = (size_t)rows_per_block * max(a.row_bytes[3], a.row_bytes[6]);
-    const int lines = (int)((widest + 127) / 128) + (FMT == PF_IQ2_XXS ? 1 : 0);
+    const int lines = (int)((widest + 127) / 128) + 1;   // the last item: the rows' scales, where they are stored apart
     uint32_t sink = 0;
     for (int i = threadIdx.x; i < mine * lines; i += blockDim.x) {
         const int item = order + per_xcd * (i / lines), l = i % lines;
@@ -314,10 +439,13 @@ __device__ __forceinline__ void prefetch_down(const PfKernelArgs &a, const uint3
         if (e >= (size_t)a.experts) continue;
         const size_t bytes = (size_t)rows_per_block * a.row_bytes[tensor];
         const uint8_t *p = a.w[tensor] + e * a.expert_bytes[tensor] + row0 * a.row_bytes[tensor];
-        if (FMT == PF_IQ2_XXS && l == lines - 1)
-            p = a.w[tensor] + a.scale_offset[tensor] + (e * a.n_out[tensor] + row0) * a.blocks_per_row[tensor] * 2;
-        else
+        if (l == lines - 1) {
+            if (!a.scale_offset[tensor]) continue;
+            const size_t each = a.type[tensor] == PF_MXFP4 ? 1 : 2;
+            p = a.w[tensor] + a.scale_offset[tensor] + (e * a.n_out[tensor] + row0) * a.blocks_per_row[tensor] * each;
+        } else {
             p += min((size_t)l * 128, bytes - 4);
+        }
         sink |= *reinterpret_cast<const volatile uint32_t *>((uintptr_t)p & ~(uintptr_t)3);
     }
     if (sink == 0x9e3779b9u && a.hidden < 0) atomicOr(a.error_word, 0u);   // keeps the loads; never true
@@ -390,19 +518,57 @@ __device__ __forceinline__ void route_finish(const PfKernelArgs &a, RouteLds *R,
 // gate row + up row: lower half-wave the gate rows, upper half-wave the up rows) and writes its
 // activations itself, so no wave waits for another after the routing.  Waves 0..parts*NT-1 first reduce
 // the logits to candidates, waves 12..15 turn the token rows into digit images.
-template <int FMT, int NT, int NPL>
+// One tile's rows against the tokens' images: the part of kernel 2 that depends on the tensors' format.
+template <int FMT, int NT>
+__device__ __forceinline__ void gate_up_tile(const PfKernelArgs &a, const int *images, const uint32_t *tables, int W, int H,
+                                             int I, int gate_tensor, uint32_t e, uint32_t mask, int u, int n0, int tile,
+                                             bool shared) {
+    const int lane = pf_lane(), wave = threadIdx.x >> 6;
+    const int LPR = H / 64, RPH = 32 / LPR;
+    const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
+    // the tile's units over 16 waves: RPH per wave step, one or two steps
+    const int per_wave = max(RPH, tile / 16), steps = per_wave / RPH, unit0 = wave * per_wave;
+    if (unit0 >= tile) return;
+    WSeg<FMT> w[2];
+#pragma unroll
+    for (int st = 0; st < 2; st++)
+        if (st < steps) wseg_load<FMT>(w[st], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        if (!((mask >> t) & 1u)) continue;
+        XSeg x;
+        xseg_load(x, images + t * W, H, seg);
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            if (st >= steps) break;
+            const float v = span_sum(wseg_dot<FMT>(w[st], x, seg, tables), LPR);
+            const float up = __shfl(v, (lane & 31) + 32);
+            if (half == 0 && seg == 0) {
+                const float act = pf_silu(v) * up;
+                const int unit = unit0 + st * RPH + r;
+                if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+                if (shared) a.shared_act[(size_t)t * I + n0 + unit] = act;
+                else a.act[((size_t)u * NT + t) * I + n0 + unit] = act;
+            }
+        }
+    }
+}
+
+// FMT: format of the routed gate and up tensors; FMTS: of the shared expert's.
+template <int FMT, int FMTS, int NT, int NPL>
 __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int routed_blocks, int shared_blocks, int parts, int chunk, int tile,
                                                          int mode) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
     const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
-    int *images = lds + table_words<FMT>();
+    constexpr bool TABLES = FMT == PF_IQ2_XXS || FMTS == PF_IQ2_XXS;
+    int *images = lds + (TABLES ? 8192 : 0);
     const int W = image_words(H), P = NT * K;
     const bool prefetcher = (int)blockIdx.x >= routed_blocks + shared_blocks;   // no tile: warms the L2 for the next kernel
     const bool shared = (int)blockIdx.x >= routed_blocks && !prefetcher;
     STAMP(0);
-    if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
+    if (TABLES) stage_tables(tables, a.iq2_signed);
     const int rounds = K + 1;
     // mode 0: every workgroup routes; 1: this launch only routes and publishes (one workgroup);
     // 2: the routes were published by an earlier launch
@@ -459,7 +625,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
         if (mode == 1) return;
         if (prefetcher) {
             const int rows_next = 64 / (a.inter / 64), first = routed_blocks + shared_blocks;
-            prefetch_down<FMT>(a, R.uniq, U, ((int)blockIdx.x - first) / 8, ((int)gridDim.x - first) / 8, rows_next,
+            prefetch_down(a, R.uniq, U, ((int)blockIdx.x - first) / 8, ((int)gridDim.x - first) / 8, rows_next,
                                (H + rows_next - 1) / rows_next);
             return;
         }
@@ -474,35 +640,8 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
         }
     }
     STAMP(4);
-    const int LPR = H / 64, RPH = 32 / LPR;
-    const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
-    // the tile's units over 16 waves: RPH per wave step, one or two steps
-    const int per_wave = max(RPH, tile / 16), steps = per_wave / RPH, unit0 = wave * per_wave;
-    if (unit0 < tile) {
-        WSeg<FMT> w[2];
-#pragma unroll
-        for (int st = 0; st < 2; st++)
-            if (st < steps) wseg_load<FMT>(w[st], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg);
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            if (!((mask >> t) & 1u)) continue;
-            XSeg x;
-            xseg_load(x, images + t * W, H, seg);
-#pragma unroll
-            for (int st = 0; st < 2; st++) {
-                if (st >= steps) break;
-                const float v = span_sum(wseg_dot<FMT>(w[st], x, seg, tables), LPR);
-                const float up = __shfl(v, (lane & 31) + 32);
-                if (half == 0 && seg == 0) {
-                    const float act = pf_silu(v) * up;
-                    const int unit = unit0 + st * RPH + r;
-                    if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-                    if (shared) a.shared_act[(size_t)t * I + n0 + unit] = act;
-                    else a.act[((size_t)u * NT + t) * I + n0 + unit] = act;
-                }
-            }
-        }
-    }
+    if (shared) gate_up_tile<FMTS, NT>(a, images, tables, W, H, I, gate_tensor, e, mask, u, n0, tile, true);
+    else gate_up_tile<FMT, NT>(a, images, tables, W, H, I, gate_tensor, e, mask, u, n0, tile, false);
     STAMP(5);
 }
 
@@ -510,18 +649,41 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
 // blockIdx.x = t * row_blocks + nb; one wave per slot plus one for the shared expert; a routed
 // wave covers the block's rows in one step.  Every wave turns its slot's activation row into a
 // digit image in LDS while its weight bytes are on their way.
-template <int FMT, int NT>
+// One wave's products of kernel 3: its slot's rows of the block against its activation image.
+template <int FMT>
+__device__ __forceinline__ void down_rows(const PfKernelArgs &a, float *partial_row, int *image, const uint32_t *tables,
+                                          const float *act_row, bool block_sync, int tensor, uint32_t e, int I, int H,
+                                          int n_base, int rows_per_block, int s) {
+    const int lane = pf_lane();
+    const int LPR = I / 64, rows = 64 / LPR, steps = rows >= rows_per_block ? 1 : rows_per_block / rows;
+    const int seg = lane & (LPR - 1), r = lane / LPR;
+    WSeg<FMT> w;   // further steps (a shared expert wider than the routed ones) load as they go
+    wseg_load<FMT>(w, a, tensor, e, min(n_base + r, H - 1), seg);
+    build_image(image, act_row, I, 64 * s, 64);
+    if (block_sync) __syncthreads();   // the tables staged by the whole workgroup
+    else pf_wave_lds_fence();
+    XSeg x;
+    xseg_load(x, image, I, seg);
+    for (int st = 0; st < steps; st++) {
+        const float v = span_sum(wseg_dot<FMT>(w, x, seg, tables), LPR);
+        const int row = st * rows + r;
+        if (seg == 0 && row < rows_per_block) partial_row[row] = v;
+        if (st + 1 < steps) wseg_load<FMT>(w, a, tensor, e, min(n_base + (st + 1) * rows + r, H - 1), seg);
+    }
+}
+
+// FMT: format of the routed down tensor; FMTS: of the shared expert's.
+template <int FMT, int FMTS, int NT>
 __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_blocks, int rows_per_block, int image_pitch) {
     __shared__ float partial[17][64];
     extern __shared__ int lds[];
+    constexpr bool TABLES = FMT == PF_IQ2_XXS || FMTS == PF_IQ2_XXS;
     uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
-    if (FMT == PF_IQ2_XXS) stage_tables(tables, a.iq2_signed);
+    if (TABLES) stage_tables(tables, a.iq2_signed);
     const int H = a.hidden, K = a.top_k, lane = pf_lane(), s = threadIdx.x >> 6;
     const int t = blockIdx.x / row_blocks, nb = blockIdx.x % row_blocks, P = NT * K;
     const bool shared = s == K;
-    const int I = shared ? a.shared_inter : a.inter, tensor = shared ? 6 : 3;
-    const int LPR = I / 64, rows = 64 / LPR, steps = rows >= rows_per_block ? 1 : rows_per_block / rows;
-    const int seg = lane & (LPR - 1), r = lane / LPR;
+    const int I = shared ? a.shared_inter : a.inter;
     uint32_t e = 0, u = 0;
     if (!shared) {
         e = a.ids[t * K + s];
@@ -533,10 +695,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_bl
         }
     }
     const int n_base = nb * rows_per_block;
-    WSeg<FMT> w;   // further steps (a shared expert wider than the routed ones) load as they go
-    wseg_load<FMT>(w, a, tensor, e, min(n_base + r, H - 1), seg);
-    int *image = lds + table_words<FMT>() + s * image_pitch;
-    build_image(image, shared ? a.shared_act + (size_t)t * I : a.act + ((size_t)u * NT + t) * I, I, 64 * s, 64);
+    int *image = lds + (TABLES ? 8192 : 0) + s * image_pitch;
     // operands of the final combine, requested now so that they arrive with the weights
     float rw[16];
 #pragma unroll
@@ -545,16 +704,12 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_bl
     PfOutputRegs out_regs;
     if ((int)threadIdx.x < rows_per_block && n_base + (int)threadIdx.x < H)
         pf_output_prefetch(a, t, n_base + threadIdx.x, out_regs);
-    if (FMT == PF_IQ2_XXS) __syncthreads();
-    else pf_wave_lds_fence();
-    XSeg x;
-    xseg_load(x, image, I, seg);
-    for (int st = 0; st < steps; st++) {
-        const float v = span_sum(wseg_dot<FMT>(w, x, seg, tables), LPR);
-        const int row = st * rows + r;
-        if (seg == 0 && row < rows_per_block) partial[s][row] = v;
-        if (st + 1 < steps) wseg_load<FMT>(w, a, tensor, e, min(n_base + (st + 1) * rows + r, H - 1), seg);
-    }
+    if (shared)
+        down_rows<FMTS>(a, partial[s], image, tables, a.shared_act + (size_t)t * I, TABLES, 6, 0, I, H, n_base,
+                        rows_per_block, s);
+    else
+        down_rows<FMT>(a, partial[s], image, tables, a.act + ((size_t)u * NT + t) * I, TABLES, 3, e, I, H, n_base,
+                       rows_per_block, s);
     __syncthreads();
     const int n = n_base + threadIdx.x;
     if ((int)threadIdx.x < rows_per_block && n < H) {
@@ -609,11 +764,21 @@ void pf_launch_block_split(const uint8_t *d_gguf, uint8_t *d_payload, uint8_t *d
 // ---- dispatch ----------------------------------------------------------------------------------------
 static bool pow2_between(uint32_t v, uint32_t lo, uint32_t hi) { return v >= lo && v <= hi && (v & (v - 1)) == 0; }
 
+// The format combinations with decode kernels: one format throughout (Q4_K or IQ2_XXS), and the two
+// profiles of real checkpoints (src/qwen4_config.c:197-216, src/qwen4_weights.c:91-99): IQ2_XXS gate/up
+// with Q2_K down, Q4_K gate/up with MXFP4 down, the shared expert in Q8_0.
+static int decode_combination(const uint32_t type[8]) {
+    const uint32_t g = type[1], d = type[3], s = type[4];
+    if (type[2] != g || type[5] != s || type[6] != s) return 0;
+    if (g == PF_Q4_K && d == PF_Q4_K && s == PF_Q4_K) return 1;
+    if (g == PF_IQ2_XXS && d == PF_IQ2_XXS && s == PF_IQ2_XXS) return 2;
+    if (g == PF_IQ2_XXS && d == PF_Q2_K && s == PF_Q8_0) return 3;
+    if (g == PF_Q4_K && d == PF_MXFP4 && s == PF_Q8_0) return 4;
+    return 0;
+}
+
 bool pf_decode_supported(const PfHipMoeDesc &d) {
-    const uint32_t fmt = d.type[1];
-    if (fmt != PF_Q4_K && fmt != PF_IQ2_XXS) return false;
-    for (int j = 1; j <= 6; j++)
-        if (d.type[j] != fmt) return false;
+    if (!decode_combination(d.type)) return false;
     if (!pow2_between(d.hidden, 512, 2048) || !pow2_between(d.inter, 256, 2048) ||
         !pow2_between(d.shared_inter, 256, 2048) || d.down_physical != d.inter || d.shared_inter > 4 * d.inter)
         return false;
@@ -624,28 +789,30 @@ bool pf_decode_supported(const PfHipMoeDesc &d) {
     return true;
 }
 
-template <int FMT, int NT, int NPL>
+template <int FG, int FS, int NT, int NPL>
 static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks,
                            int shared_blocks, int parts, int chunk, int tile) {
     // more workgroups than compute units: routing once, in a launch of its own, beats every workgroup repeating it
     const bool split = grid.x > 256;
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FMT, NT, NPL>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FG, FS, NT, NPL>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
         configured = true;
     }
     if (split)
-        hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, NPL>), dim3(1), dim3(1024), lds, stream, a, routed_blocks, shared_blocks,
-                           parts, chunk, tile, 1);
-    hipLaunchKernelGGL((pf_k_dec_gate_up<FMT, NT, NPL>), grid, dim3(1024), lds, stream, a, routed_blocks, shared_blocks, parts,
-                       chunk, tile, split ? 2 : 0);
+        hipLaunchKernelGGL((pf_k_dec_gate_up<FG, FS, NT, NPL>), dim3(1), dim3(1024), lds, stream, a, routed_blocks,
+                           shared_blocks, parts, chunk, tile, 1);
+    hipLaunchKernelGGL((pf_k_dec_gate_up<FG, FS, NT, NPL>), grid, dim3(1024), lds, stream, a, routed_blocks, shared_blocks,
+                       parts, chunk, tile, split ? 2 : 0);
 }
 
-template <int FMT, int NT>
+// FG: format of the routed gate and up tensors, FD: of the routed down tensor, FS: of the shared expert
+template <int FG, int FD, int FS, int NT>
 static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_limit) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
-    const size_t tab = table_words<FMT>() * 4;
+    const size_t tab2 = (FG == PF_IQ2_XXS || FS == PF_IQ2_XXS) ? 8192 * 4 : 0;
+    const size_t tab3 = (FD == PF_IQ2_XXS || FS == PF_IQ2_XXS) ? 8192 * 4 : 0;
     // kernel 1 (stage_limit, profiling: launch only the first so many kernels; 0 = all)
     const int router_blocks = (E + 3) / 4, last = stage_limit ? stage_limit : 3;
     hipLaunchKernelGGL((pf_k_dec_router<NT>), dim3(router_blocks + 1), dim3(256), 0, stream, a, router_blocks);
@@ -655,7 +822,7 @@ static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_l
     // unit measured faster than two half as long
     const int tile = 32;
     const int routed_blocks = NT * K * (I / tile), shared_blocks = Is / tile;
-    const size_t lds2 = tab + (size_t)NT * image_words(H) * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+    const size_t lds2 = tab2 + (size_t)NT * image_words(H) * 4 + ((size_t)H + 3 * (size_t)E) * 4;
     int parts = NT == 1 ? 8 : NT == 2 ? 6 : NT == 3 ? 4 : 3;
     while (parts > 1 && (E + parts - 1) / parts < 64) parts--;
     const int chunk = (E + parts - 1) / parts, npl = (chunk + 63) / 64;
@@ -665,36 +832,41 @@ static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_l
     int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
     if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
     dim3 g2(routed_blocks + shared_blocks + prefetch_blocks);
-    if (npl <= 1) launch_gate_up<FMT, NT, 1>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
-    else if (npl <= 2) launch_gate_up<FMT, NT, 2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
-    else if (npl <= 4) launch_gate_up<FMT, NT, 4>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
-    else launch_gate_up<FMT, NT, 8>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024
+    if (npl <= 1) launch_gate_up<FG, FS, NT, 1>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else if (npl <= 2) launch_gate_up<FG, FS, NT, 2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else if (npl <= 4) launch_gate_up<FG, FS, NT, 4>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else launch_gate_up<FG, FS, NT, 8>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024
     if (last < 3) return;
     // kernel 3
     const int rows_per_block = 64 / (I / 64), row_blocks = (H + rows_per_block - 1) / rows_per_block;
     const int image_pitch = image_words(I > Is ? I : Is);
-    const size_t lds3 = tab + (size_t)(K + 1) * image_pitch * 4;
+    const size_t lds3 = tab3 + (size_t)(K + 1) * image_pitch * 4;
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down<FMT, NT>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down<FD, FS, NT>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
         configured = true;
     }
-    hipLaunchKernelGGL((pf_k_dec_down<FMT, NT>), dim3(NT * row_blocks), dim3(64 * (K + 1)), lds3, stream, a, row_blocks,
+    hipLaunchKernelGGL((pf_k_dec_down<FD, FS, NT>), dim3(NT * row_blocks), dim3(64 * (K + 1)), lds3, stream, a, row_blocks,
                        rows_per_block, image_pitch);
 }
 
-template <int FMT>
+template <int FG, int FD, int FS>
 static void launch_decode_tokens(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     switch (tokens) {
-    case 1: launch_decode<FMT, 1>(a, stream, stage_limit); break;
-    case 2: launch_decode<FMT, 2>(a, stream, stage_limit); break;
-    case 3: launch_decode<FMT, 3>(a, stream, stage_limit); break;
-    default: launch_decode<FMT, 4>(a, stream, stage_limit); break;
+    case 1: launch_decode<FG, FD, FS, 1>(a, stream, stage_limit); break;
+    case 2: launch_decode<FG, FD, FS, 2>(a, stream, stage_limit); break;
+    case 3: launch_decode<FG, FD, FS, 3>(a, stream, stage_limit); break;
+    default: launch_decode<FG, FD, FS, 4>(a, stream, stage_limit); break;
     }
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    if (a.type[1] == PF_Q4_K) launch_decode_tokens<PF_Q4_K>(a, tokens, stream, stage_limit);
-    else launch_decode_tokens<PF_IQ2_XXS>(a, tokens, stream, stage_limit);
+    switch (decode_combination(a.type)) {
+    case 1: launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit); break;
+    case 2: launch_decode_tokens<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit); break;
+    case 3: launch_decode_tokens<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit); break;
+    case 4: launch_decode_tokens<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit); break;
+    default: break;   // pf_decode_supported keeps other combinations away
+    }
 }

@@ -91,3 +91,32 @@ def test_uniform_layers_of_the_plain_formats(product, oracle, gtype):
     want = forward_with(oracle, cfg, weights, x)
     got = forward_with(product, cfg, weights, x)
     assert_parity(*got, *want, label=abi.FORMAT_NAME[gtype])
+
+
+# shapes the decode kernels cover, on the two checkpoint profiles, 1..4 tokens per call
+DECODE_PROFILES = [
+    (512, 32, 6, 256, 256, "q2"), (512, 32, 6, 256, 256, "q4"),
+    (1024, 96, 5, 512, 256, "q2"), (1024, 96, 5, 256, 1024, "q4"),     # a shared expert wider than the routed ones
+    (2048, 64, 10, 512, 512, "q2"), (2048, 64, 10, 512, 512, "q4"),    # the measured widths
+]
+
+
+@pytest.mark.parametrize("h,e,k,i,s,profile", DECODE_PROFILES)
+def test_decode_kernels_on_checkpoint_profiles(product, oracle, h, e, k, i, s, profile):
+    print(f"case decode profile {profile} h={h} e={e} k={k} i={i} s={s}", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s)
+    weights, x = make_layer_inputs(cfg, profile, 4, seed=h + e + len(profile))
+    x[3] = x[2]                                   # two identical tokens share every expert
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, 4) as layer:
+        moe, work = layer.device_handles()
+        assert product.hip.moe_kernel_family(moe, work, 1) == 1, "the decode kernels do not cover this layer"
+        for tokens in (1, 2, 3, 4):
+            print(f"  tokens={tokens}", flush=True)
+            _, y, ids, w = layer.forward(x[:tokens])
+            worst = assert_parity(y, ids, w, want[0][:tokens], want[1][:tokens], want[2][:tokens],
+                                  label=f"decode {profile} T={tokens}")
+        print(f"  max abs err {worst:.2e}", flush=True)
+        layer.force_general()
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y, ids, w, *want, label="general kernels on the same layer")
