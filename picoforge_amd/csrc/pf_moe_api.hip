@@ -198,8 +198,9 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         // lines once instead of 32-byte pieces of lines it meets again a stage later.  It doubles the
         // expert bytes; PF_MOE_PREFILL_COPY=0 does without it (the same kernels read the row order).
         const char *copy = getenv("PF_MOE_PREFILL_COPY");
-        if (desc->type[1] == PF_Q4_K && (!copy || strcmp(copy, "0") != 0)) {
+        if (!copy || strcmp(copy, "0") != 0) {
             for (int a = 1; a <= 6 && e == hipSuccess; a++) {
+                if (desc->type[a] != PF_Q4_K) continue;
                 e = hipMalloc((void **)&m->w_tiled[a], m->bytes[a]);
                 if (e == hipSuccess) {
                     pf_launch_q4k_tile(m->w[a], m->w_tiled[a], (size_t)n_out[a] * experts[a], m->blocks_per_row[a], nullptr);

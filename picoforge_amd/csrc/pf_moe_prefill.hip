@@ -276,6 +276,8 @@ __device__ __forceinline__ bool gemm_item(const PfKernelArgs &a, int tokens, int
     g.rows_here = min(32, g.count - g.m0);
     g.inter = g.shared ? a.shared_inter : a.inter;
     const size_t ex = g.shared ? 0 : (size_t)expert;
+    if (a.type[MODE == PF_GEMM_GATE_UP ? (g.shared ? 4 : 1) : (g.shared ? 6 : 3)] != (uint32_t)FMT)
+        return false;   // another format: the plain grouped product takes the item
     if (MODE == PF_GEMM_GATE_UP) {
         const int tg = g.shared ? 4 : 1;
         if (32 * NW * g.slab >= g.inter) return false;
@@ -787,6 +789,203 @@ __global__ void __launch_bounds__(64 * (NW + NL), 3) pf_k_pf_gemm(PfKernelArgs a
     }
 }
 
+// ---- the grouped product for the other formats of real checkpoints --------------------------------
+// Q8_0 (shared expert), Q2_K and MXFP4 (routed down projections) have no operand path in the ring
+// kernel above.  This kernel computes the same items with the same operands' arithmetic (exact
+// integer weight operands in fp16, two-part fp16 activations, FP32 accumulation, scales applied to
+// the partial sums in FP32) but without the LDS ring: a workgroup is one row tile against one slab
+// of 4 x 32 (gate/up) or 4 x 64 (down) weight rows, a wave takes its operands straight from global
+// memory (the activation fragments are shared through the caches by the four waves and the slabs).
+// Group scales that are not integers (Q8_0: a half per 32 weights; MXFP4: a power of two per 32)
+// multiply the group's partial sums; Q2_K folds its 4-bit scale into the operand (scale * code
+// <= 45) and obtains sum(min * x) from a second product with the minimum as the operand, as
+// d * P - dmin * Q per 256-block.
+
+// eight bytes as eight halfs, exact: a byte under the exponent byte 0x64 reads as 1024 + byte
+__device__ __forceinline__ half8v half8_of_bytes(uint32_t b0, uint32_t b1, half_t offset) {
+    const uint32_t bias = 0x64646464u;
+    const half2v c = {offset, offset};
+    const half2v v0 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, b0, 0x04010400u)) - c;
+    const half2v v1 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, b0, 0x04030402u)) - c;
+    const half2v v2 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, b1, 0x04010400u)) - c;
+    const half2v v3 = __builtin_bit_cast(half2v, __builtin_amdgcn_perm(bias, b1, 0x04030402u)) - c;
+    return half8v{v0.x, v0.y, v1.x, v1.y, v2.x, v2.y, v3.x, v3.y};
+}
+// signed bytes: flip the sign bit, read as unsigned, take 128 more away
+__device__ __forceinline__ half8v half8_of_signed_bytes(uint32_t b0, uint32_t b1) {
+    return half8_of_bytes(b0 ^ 0x80808080u, b1 ^ 0x80808080u, (half_t)1152.0f);
+}
+
+// four E2M1 codes (one per byte, low nibble) as signed bytes holding twice their value
+__device__ __forceinline__ uint32_t plain_e2m1_twice4(uint32_t nibbles) {
+    const uint32_t sel = nibbles & 0x07070707u;
+    const uint32_t pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
+    const uint32_t neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
+    const uint32_t mask = ((nibbles >> 3) & 0x01010101u) * 0xFFu;
+    return (neg & mask) | (pos & ~mask);
+}
+
+struct PlainRow {            // one weight row as the kernel reads it
+    const uint8_t *payload;  // first byte of the row (device layout of its format)
+    const uint8_t *scales;   // first scale of the row, for the formats stored split
+};
+
+__device__ __forceinline__ PlainRow plain_row(const PfKernelArgs &a, int t, size_t e, size_t row) {
+    const size_t index = e * a.n_out[t] + row;
+    PlainRow r;
+    r.payload = a.w[t] + index * a.row_bytes[t];
+    r.scales = a.w[t] + a.scale_offset[t] + index * a.blocks_per_row[t] * (a.type[t] == PF_MXFP4 ? 1 : 2);
+    return r;
+}
+
+// acc0 / acc1 += activation tile (rows of ahi: high parts at column k, low parts at a_cols + k) x rows r0 / r1
+template <int FMT>
+__device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow &r1, const half_t *ahi, int a_cols, int K,
+                                              int h, float16v &acc0, float16v &acc1) {
+    const float16v zero = {0};
+    const half_t *alo = ahi + a_cols;
+    if (FMT == PF_Q2_K) {
+        for (int b = 0; b < K / 256; b++) {
+            const uint8_t *blk0 = r0.payload + 84 * (size_t)b, *blk1 = r1.payload + 84 * (size_t)b;
+            const uint32_t dd0 = *reinterpret_cast<const uint32_t *>(blk0 + 80), dd1 = *reinterpret_cast<const uint32_t *>(blk1 + 80);
+            float16v part0 = zero, part1 = zero, low0 = zero, low1 = zero;
+            for (int gi = 0; gi < 16; gi++) {   // one group of 16 weights per product step
+                const int l = 16 * gi, at = 16 + 32 * (l >> 7) + (l & 31) + 8 * h, shift = 2 * ((l & 127) >> 5);
+                const uint32_t *q0 = reinterpret_cast<const uint32_t *>(blk0 + at), *q1 = reinterpret_cast<const uint32_t *>(blk1 + at);
+                const uint32_t sm0 = blk0[gi], sm1 = blk1[gi];
+                const int k = 256 * b + l + 8 * h;
+                const half8v xh = *reinterpret_cast<const half8v *>(ahi + k), xl = *reinterpret_cast<const half8v *>(alo + k);
+                // byte-wise scale * code: at most 15 * 3, no carry between bytes
+                const half8v w0 = half8_of_bytes(((q0[0] >> shift) & 0x03030303u) * (sm0 & 15u), ((q0[1] >> shift) & 0x03030303u) * (sm0 & 15u), (half_t)1024.0f);
+                const half8v w1 = half8_of_bytes(((q1[0] >> shift) & 0x03030303u) * (sm1 & 15u), ((q1[1] >> shift) & 0x03030303u) * (sm1 & 15u), (half_t)1024.0f);
+                const half_t m0 = (half_t)(int)(sm0 >> 4), m1 = (half_t)(int)(sm1 >> 4);
+                const half8v mv0 = {m0, m0, m0, m0, m0, m0, m0, m0}, mv1 = {m1, m1, m1, m1, m1, m1, m1, m1};
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w1, part1, 0, 0, 0);
+                low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv0, low0, 0, 0, 0);
+                low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv1, low1, 0, 0, 0);
+                low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv0, low0, 0, 0, 0);
+                low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv1, low1, 0, 0, 0);
+            }
+            const half2v h0 = __builtin_bit_cast(half2v, dd0), h1 = __builtin_bit_cast(half2v, dd1);
+            const float d0 = (float)h0.x, n0 = (float)h0.y, d1 = (float)h1.x, n1 = (float)h1.y;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc0[r] = fmaf(d0, part0[r], fmaf(-n0, low0[r], acc0[r]));
+                acc1[r] = fmaf(d1, part1[r], fmaf(-n1, low1[r], acc1[r]));
+            }
+        }
+        return;
+    }
+    for (int g = 0; g < K / 32; g++) {          // one scale per 32 weights: two product steps per group
+        float16v part0 = zero, part1 = zero;
+        float s0, s1;
+        if (FMT == PF_Q8_0) {
+            s0 = (float)__builtin_bit_cast(half_t, reinterpret_cast<const uint16_t *>(r0.scales)[g]);
+            s1 = (float)__builtin_bit_cast(half_t, reinterpret_cast<const uint16_t *>(r1.scales)[g]);
+        } else {
+            s0 = 0.5f * pf_e8m0_scale(r0.scales[g]);   // the operands are twice the values
+            s1 = 0.5f * pf_e8m0_scale(r1.scales[g]);
+        }
+        uint2 m0 = {0, 0}, m1 = {0, 0};
+        if (FMT == PF_MXFP4) {   // bytes 8h..8h+7 of the block: low nibbles values 8h.., high nibbles values 16 + 8h..
+            m0 = *reinterpret_cast<const uint2 *>(r0.payload + 16 * (size_t)g + 8 * h);
+            m1 = *reinterpret_cast<const uint2 *>(r1.payload + 16 * (size_t)g + 8 * h);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int k = 32 * g + 16 * t + 8 * h;
+            const half8v xh = *reinterpret_cast<const half8v *>(ahi + k), xl = *reinterpret_cast<const half8v *>(alo + k);
+            half8v w0, w1;
+            if (FMT == PF_Q8_0) {
+                const uint2 c0 = *reinterpret_cast<const uint2 *>(r0.payload + k), c1 = *reinterpret_cast<const uint2 *>(r1.payload + k);
+                w0 = half8_of_signed_bytes(c0.x, c0.y);
+                w1 = half8_of_signed_bytes(c1.x, c1.y);
+            } else {
+                const int sh = 4 * t;
+                w0 = half8_of_signed_bytes(plain_e2m1_twice4((m0.x >> sh) & 0x0F0F0F0Fu), plain_e2m1_twice4((m0.y >> sh) & 0x0F0F0F0Fu));
+                w1 = half8_of_signed_bytes(plain_e2m1_twice4((m1.x >> sh) & 0x0F0F0F0Fu), plain_e2m1_twice4((m1.y >> sh) & 0x0F0F0F0Fu));
+            }
+            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
+            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
+            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w0, part0, 0, 0, 0);
+            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w1, part1, 0, 0, 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            acc0[r] = fmaf(s0, part0[r], acc0[r]);
+            acc1[r] = fmaf(s1, part1[r], acc1[r]);
+        }
+    }
+}
+
+// grid: (row tiles the list can hold) x slabs; 4 waves.  Items whose tensors are in a format of the ring
+// kernel are skipped here, as the ring kernel skips these.
+template <int MODE>
+__global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int tokens, int slabs) {
+    const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
+    const int E = a.experts, K = a.top_k, P = tokens * K;
+    const uint32_t tile = blockIdx.x / slabs, slab = blockIdx.x % slabs;
+    if (tile >= a.tiles[0]) return;
+    const uint32_t entry = a.tiles[1 + tile];
+    const int expert = entry & 0xffffu, m0 = 32 * (int)(entry >> 16);
+    const bool shared = expert == E;
+    const int first = shared ? P : (int)a.offsets[expert];
+    const int count = shared ? tokens : (int)a.offsets[expert + 1] - first;
+    if (count <= m0) return;
+    const int rows_here = min(32, count - m0), inter = shared ? a.shared_inter : a.inter;
+    const size_t ex = shared ? 0 : (size_t)expert;
+    const int t0 = MODE == PF_GEMM_GATE_UP ? (shared ? 4 : 1) : (shared ? 6 : 3);
+    const uint32_t fmt = a.type[t0];
+    if (fmt != PF_Q8_0 && fmt != PF_Q2_K && fmt != PF_MXFP4) return;
+    // this lane's activation row as an operand (row n of the tile), and the rows' scales for the epilogue
+    const int a_cols = MODE == PF_GEMM_GATE_UP ? a.hidden : inter;
+    const half_t *a16 = reinterpret_cast<const half_t *>(MODE == PF_GEMM_GATE_UP ? a.x16 : shared ? a.sact16 : a.act16);
+    const float *a_scale = MODE == PF_GEMM_GATE_UP ? a.x_scale : shared ? a.sact_scale : a.act_scale;
+    auto source_row = [&](int m) -> uint32_t {
+        if (m >= rows_here) return MODE == PF_GEMM_GATE_UP || shared ? a.token_cap : a.token_cap * (uint32_t)K;   // the all-zero row
+        if (shared) return (uint32_t)(m0 + m);
+        return MODE == PF_GEMM_GATE_UP ? a.row_to_pair[first + m0 + m] / (uint32_t)K : (uint32_t)(first + m0 + m);
+    };
+    const half_t *ahi = a16 + (size_t)source_row(n) * pf_half_row(a_cols);
+    int row_a, row_b, t1, limit;
+    if (MODE == PF_GEMM_GATE_UP) {
+        limit = inter;
+        row_a = row_b = 128 * (int)slab + 32 * wave + n;   // the unit's gate row and up row
+        t1 = t0 + 1;
+    } else {
+        limit = a.hidden;
+        row_a = 256 * (int)slab + 64 * wave + n;
+        row_b = row_a + 32;
+        t1 = t0;
+    }
+    if (row_a - n >= limit) return;   // the whole wave: no barrier in this kernel
+    const PlainRow r0 = plain_row(a, t0, ex, min(row_a, limit - 1)), r1 = plain_row(a, t1, ex, min(row_b, limit - 1));
+    float16v acc0 = {0}, acc1 = {0};
+    if (fmt == PF_Q8_0) plain_product<PF_Q8_0>(r0, r1, ahi, a_cols, a_cols, h, acc0, acc1);
+    else if (fmt == PF_MXFP4) plain_product<PF_MXFP4>(r0, r1, ahi, a_cols, a_cols, h, acc0, acc1);
+    else plain_product<PF_Q2_K>(r0, r1, ahi, a_cols, a_cols, h, acc0, acc1);
+    // epilogue: the lane holds column n of its two tiles; register r is row 8 (r / 4) + 4 h + r % 4
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int m = 8 * (r >> 2) + 4 * h + (r & 3);
+        if (m >= rows_here) continue;
+        const float rs = a_scale[source_row(m)];
+        if (MODE == PF_GEMM_GATE_UP) {
+            if (row_a >= limit) continue;
+            const float v = pf_silu(acc0[r] * rs) * (acc1[r] * rs);
+            if (shared) a.shared_act[(size_t)(m0 + m) * inter + row_a] = v;
+            else a.act[(size_t)(first + m0 + m) * inter + row_a] = v;
+        } else {
+            float *out = a.down + (size_t)(first + m0 + m) * a.hidden;
+            if (row_a < limit) out[row_a] = acc0[r] * rs;
+            if (row_b < limit) out[row_b] = acc1[r] * rs;
+        }
+    }
+}
+
 // ---- combine ---------------------------------------------------------------------------------------
 // y[t] = sum over slots in order of weight * down row, then + sigmoid * shared down row
 // (src/qwen4_moe.c:362-372)
@@ -816,10 +1015,13 @@ __global__ void __launch_bounds__(256) pf_k_pf_combine(PfKernelArgs a, int token
 }
 
 // ---- dispatch --------------------------------------------------------------------------------------
+// Routed gate and up in Q4_K or IQ2_XXS (the ring kernel's operand paths); the routed down tensor and the
+// shared expert's three tensors in that same format or in Q2_K, MXFP4, Q8_0 (the plain grouped product).
 bool pf_prefill_supported(const PfHipMoeDesc &d) {
-    if (d.type[1] != PF_Q4_K && d.type[1] != PF_IQ2_XXS) return false;
-    for (int j = 1; j <= 6; j++)
-        if (d.type[j] != d.type[1]) return false;
+    const uint32_t g = d.type[1];
+    auto covered = [&](uint32_t t) { return t == g || t == PF_Q8_0 || t == PF_Q2_K || t == PF_MXFP4; };
+    if ((g != PF_Q4_K && g != PF_IQ2_XXS) || d.type[2] != g || !covered(d.type[3])) return false;
+    if (d.type[5] != d.type[4] || !covered(d.type[4]) || !covered(d.type[6])) return false;
     if (d.hidden % 256 || d.inter % 256 || d.shared_inter % 256 || d.down_physical != d.inter) return false;
     if (d.top_k > 64 || d.top_k >= d.experts || d.experts >= 65535) return false;
     return true;
@@ -864,17 +1066,30 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     pf_launch_group_place(a.ids, P, E, a.offsets, a.pair_to_row, a.row_to_pair, stream);
     if (last < 3) return;
     // stage 3: gate/up + SwiGLU, then fp16 parts of the activation rows
+    // the ring kernel takes the items whose tensors are in the routed gate's format, the plain kernel the rest
     const int gi = I > Is ? I : Is;
     const bool iq2 = a.type[1] == PF_IQ2_XXS;
+    const uint32_t ring_fmt = a.type[1];
+    const unsigned tile_cap = (unsigned)pf_prefill_max_tiles(tokens, E, K);
     if (iq2) launch_gemm<PF_GEMM_GATE_UP, PF_IQ2_XXS>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
     else launch_gemm<PF_GEMM_GATE_UP, PF_Q4_K>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
+    if (a.type[4] != ring_fmt) {
+        const int slabs = (gi + 127) / 128;
+        hipLaunchKernelGGL(pf_k_pf_gemm_plain<PF_GEMM_GATE_UP>, dim3(tile_cap * slabs), dim3(256), 0, stream, a, tokens, slabs);
+    }
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(P), dim3(256), 0, stream, a.act, (size_t)I, I, (half_t *)a.act16, a.act_scale,
                        (float *)nullptr, a.error_word);
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.shared_act, (size_t)Is, Is,
                        (half_t *)a.sact16, a.sact_scale, (float *)nullptr, a.error_word);
     if (last < 4) return;
     // stage 4: down and combine
-    if (iq2) launch_gemm<PF_GEMM_DOWN, PF_IQ2_XXS>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
-    else launch_gemm<PF_GEMM_DOWN, PF_Q4_K>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
+    if (a.type[3] == ring_fmt || a.type[6] == ring_fmt) {
+        if (iq2) launch_gemm<PF_GEMM_DOWN, PF_IQ2_XXS>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
+        else launch_gemm<PF_GEMM_DOWN, PF_Q4_K>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
+    }
+    if (a.type[3] != ring_fmt || a.type[6] != ring_fmt) {
+        const int slabs = (H + 255) / 256;
+        hipLaunchKernelGGL(pf_k_pf_gemm_plain<PF_GEMM_DOWN>, dim3(tile_cap * slabs), dim3(256), 0, stream, a, tokens, slabs);
+    }
     hipLaunchKernelGGL(pf_k_pf_combine, dim3(tokens), dim3(256), 0, stream, a, tokens);
 }

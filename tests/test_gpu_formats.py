@@ -65,7 +65,8 @@ PROFILES = [
     (512, 16, 4, 512, 256, 512, "q4", 3),
     (256, 8, 3, 160, 96, 256, "q2", 2),      # logical K 160 stored in 256 (the checkpoint's 640 in 768)
     (512, 32, 6, 256, 256, 256, "q4", 1),
-    (512, 32, 6, 256, 256, 256, "q2", 40),   # a chunk
+    (512, 32, 6, 256, 256, 256, "q2", 40),   # chunks: the matrix-core kernels
+    (512, 32, 6, 256, 256, 256, "q4", 37),
 ]
 
 
@@ -117,6 +118,35 @@ def test_decode_kernels_on_checkpoint_profiles(product, oracle, h, e, k, i, s, p
             worst = assert_parity(y, ids, w, want[0][:tokens], want[1][:tokens], want[2][:tokens],
                                   label=f"decode {profile} T={tokens}")
         print(f"  max abs err {worst:.2e}", flush=True)
+        layer.force_general()
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y, ids, w, *want, label="general kernels on the same layer")
+
+
+# chunks on the checkpoint profiles: the ring kernel for the routed gate/up tensors, the plain grouped
+# product for the Q8_0 shared expert and the Q2_K / MXFP4 down tensors
+PREFILL_PROFILES = [
+    (256, 16, 4, 256, 256, 5), (256, 16, 4, 256, 256, 33), (512, 8, 3, 256, 512, 70),
+    (256, 16, 4, 512, 256, 400),          # about 100 rows per expert: several row tiles
+    (768, 40, 5, 256, 256, 129),
+]
+
+
+@pytest.mark.parametrize("profile", ["q2", "q4"])
+@pytest.mark.parametrize("h,e,k,i,s,tokens", PREFILL_PROFILES)
+def test_prefill_kernels_on_checkpoint_profiles(product, oracle, h, e, k, i, s, tokens, profile):
+    print(f"case prefill profile {profile} h={h} e={e} k={k} i={i} s={s} T={tokens}", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s)
+    weights, x = make_layer_inputs(cfg, profile, tokens, seed=h + e + tokens)
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, tokens) as layer:
+        moe, work = layer.device_handles()
+        assert product.hip.moe_kernel_family(moe, work, tokens) == 2, "the prefill kernels do not cover this layer"
+        _, y, ids, w = layer.forward(x)
+        worst = assert_parity(y, ids, w, *want, label=f"prefill {profile} T={tokens}")
+        print(f"  max abs err {worst:.2e}", flush=True)
+        _, y2, _, _ = layer.forward(x)
+        np.testing.assert_array_equal(y, y2, err_msg="not deterministic")
         layer.force_general()
         _, y, ids, w = layer.forward(x)
         assert_parity(y, ids, w, *want, label="general kernels on the same layer")

@@ -142,6 +142,8 @@ CHAIN = [
     (768, 40, 5, 256, 256, abi.GGUF_Q4_K, 129, 2),
     (512, 32, 6, 256, 256, abi.GGUF_Q4_K, 2, 6),         # more streams than the last kernel folds in: separate add
     (256, 16, 4, 256, 256, abi.GGUF_IQ2_XXS, 33, 5),
+    (512, 32, 6, 256, 256, "q2", 3, 4),                  # checkpoint profiles on the decode kernels
+    (512, 32, 6, 256, 256, "q4", 9, 4),                  # ... a chunk, four tokens per launch
 ]
 
 
