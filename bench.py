@@ -14,6 +14,9 @@ Workloads: iq2xxs_decode (default), q4k_decode, q4k_verify4 (4-token batches wit
 about half of the experts shared between neighbours), q4k_prefill1024 and
 iq2xxs_prefill1024 (1024-token chunks, N(0,1) activations, Zipf(1.1) expert
 popularity), q4k_stack48 (48 resident layers, decode and 2048-token chunks), and
+q2profile_decode / q4profile_decode / q2profile_prefill1024 / q4profile_prefill1024 (the
+format mixes of real checkpoints: IQ2_XXS gate/up + Q2_K down, Q4_K gate/up + MXFP4 down,
+Q8_0 shared expert), and
 iq2xxs_decode_hc / q4k_decode_hc / q4k_prefill1024_hc: the same layer between its two
 hyper-connection steps (gated read of 4 residual streams before, injection into them
 after), with the injection folded into the block's last kernel and as a kernel of its own.
@@ -67,6 +70,12 @@ WORKLOADS = {
                              label="checkpoint profile Q2 (IQ2_XXS gate/up, Q2_K down, Q8_0 shared expert), decode batch 1"),
     "q4profile_decode": dict(type="q4", tokens=1, steps=5000, warmup=100,
                              label="checkpoint profile Q4 (Q4_K gate/up, MXFP4 down, Q8_0 shared expert), decode batch 1"),
+    "q2profile_prefill1024": dict(type="q2", tokens=1024, steps=50, warmup=5,
+                                  label="checkpoint profile Q2 (IQ2_XXS gate/up, Q2_K down, Q8_0 shared expert), 1024-token "
+                                        "prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
+    "q4profile_prefill1024": dict(type="q4", tokens=1024, steps=50, warmup=5,
+                                  label="checkpoint profile Q4 (Q4_K gate/up, MXFP4 down, Q8_0 shared expert), 1024-token "
+                                        "prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),
@@ -78,7 +87,8 @@ MEASURED_TRAFFIC = {"iq2xxs_decode": 9832986, "q4k_decode": 19831587, "q4k_verif
                     "q4k_prefill1024": 816855693, "iq2xxs_prefill1024": 448880069,
                     # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
                     "q4k_prefill1024_hc": 75633480, "iq2xxs_decode_hc": 117102, "q4k_decode_hc": None,
-                    "q2profile_decode": None, "q4profile_decode": None}
+                    "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None,
+                    "q4profile_prefill1024": None}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
@@ -90,6 +100,7 @@ PREFILL_STAGES = ["pf_k_rows_to_half + pf_k_pf_router (fp16 copy of x, router lo
                   "routing + grouping (top-k, serial-order re-routes, histogram/scan/stable placement)",
                   "pf_k_pf_gemm<gate_up> (grouped gate/up + SwiGLU by FP16 MFMA, then fp16 copy of the activations)",
                   "pf_k_pf_gemm<down> + pf_k_pf_combine (grouped down by FP16 MFMA, slot-ordered combine)"]
+# on the checkpoint profiles the Q8_0 / Q2_K / MXFP4 items of stages 3 and 4 run in pf_k_pf_gemm_plain
 
 
 def run_stack(args, api, hip, cfg, steps, warmup):

@@ -838,36 +838,48 @@ __device__ __forceinline__ PlainRow plain_row(const PfKernelArgs &a, int t, size
     return r;
 }
 
-// acc0 / acc1 += activation tile (rows of ahi: high parts at column k, low parts at a_cols + k) x rows r0 / r1
+// acc0 / acc1 += staged activation columns [c0, c0 + cols) x the same columns of weight rows r0 / r1.
+// ahi / alo: this lane's activation row in LDS (high and low parts of the staged columns).  The
+// weight bytes of several groups are requested before the first product of the batch.
+// A wave takes every `parts`-th batch (256-block for Q2_K) starting with batch `part`: with parts > 1 the
+// waves of a workgroup share one pair of rows and their partial sums are added afterwards.
 template <int FMT>
-__device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow &r1, const half_t *ahi, int a_cols, int K,
-                                              int h, float16v &acc0, float16v &acc1) {
+__device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow &r1, const half_t *ahi, const half_t *alo,
+                                              int c0, int cols, int h, int part, int parts, float16v &acc0, float16v &acc1) {
     const float16v zero = {0};
-    const half_t *alo = ahi + a_cols;
     if (FMT == PF_Q2_K) {
-        for (int b = 0; b < K / 256; b++) {
-            const uint8_t *blk0 = r0.payload + 84 * (size_t)b, *blk1 = r1.payload + 84 * (size_t)b;
+        for (int b = part; b < cols / 256; b += parts) {
+            const uint8_t *blk0 = r0.payload + 84 * (size_t)(c0 / 256 + b), *blk1 = r1.payload + 84 * (size_t)(c0 / 256 + b);
             const uint32_t dd0 = *reinterpret_cast<const uint32_t *>(blk0 + 80), dd1 = *reinterpret_cast<const uint32_t *>(blk1 + 80);
             float16v part0 = zero, part1 = zero, low0 = zero, low1 = zero;
-            for (int gi = 0; gi < 16; gi++) {   // one group of 16 weights per product step
-                const int l = 16 * gi, at = 16 + 32 * (l >> 7) + (l & 31) + 8 * h, shift = 2 * ((l & 127) >> 5);
-                const uint32_t *q0 = reinterpret_cast<const uint32_t *>(blk0 + at), *q1 = reinterpret_cast<const uint32_t *>(blk1 + at);
-                const uint32_t sm0 = blk0[gi], sm1 = blk1[gi];
-                const int k = 256 * b + l + 8 * h;
-                const half8v xh = *reinterpret_cast<const half8v *>(ahi + k), xl = *reinterpret_cast<const half8v *>(alo + k);
-                // byte-wise scale * code: at most 15 * 3, no carry between bytes
-                const half8v w0 = half8_of_bytes(((q0[0] >> shift) & 0x03030303u) * (sm0 & 15u), ((q0[1] >> shift) & 0x03030303u) * (sm0 & 15u), (half_t)1024.0f);
-                const half8v w1 = half8_of_bytes(((q1[0] >> shift) & 0x03030303u) * (sm1 & 15u), ((q1[1] >> shift) & 0x03030303u) * (sm1 & 15u), (half_t)1024.0f);
-                const half_t m0 = (half_t)(int)(sm0 >> 4), m1 = (half_t)(int)(sm1 >> 4);
-                const half8v mv0 = {m0, m0, m0, m0, m0, m0, m0, m0}, mv1 = {m1, m1, m1, m1, m1, m1, m1, m1};
-                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
-                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
-                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w0, part0, 0, 0, 0);
-                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w1, part1, 0, 0, 0);
-                low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv0, low0, 0, 0, 0);
-                low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv1, low1, 0, 0, 0);
-                low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv0, low0, 0, 0, 0);
-                low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv1, low1, 0, 0, 0);
+#pragma unroll
+            for (int half = 0; half < 2; half++) {   // eight groups of 16 weights per batch: one 32-byte half of the codes
+                const uint32_t *sw0 = reinterpret_cast<const uint32_t *>(blk0), *sw1 = reinterpret_cast<const uint32_t *>(blk1);   // 4-byte aligned
+                const uint32_t *q0 = reinterpret_cast<const uint32_t *>(blk0 + 16 + 32 * half + 8 * h);
+                const uint32_t *q1 = reinterpret_cast<const uint32_t *>(blk1 + 16 + 32 * half + 8 * h);
+                // bytes 8h..8h+7 and 16 + 8h..: the groups at l % 32 = 0 and 16, each at four bit planes
+                const uint32_t c0a[2] = {q0[0], q0[1]}, c0b[2] = {q0[4], q0[5]}, c1a[2] = {q1[0], q1[1]}, c1b[2] = {q1[4], q1[5]};
+                const uint32_t scales0[4] = {sw0[0], sw0[1], sw0[2], sw0[3]}, scales1[4] = {sw1[0], sw1[1], sw1[2], sw1[3]};
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int gi = 8 * half + j, shift = 2 * (j >> 1), k = 256 * b + 16 * gi + 8 * h;
+                    const uint32_t s0 = (scales0[gi >> 2] >> (8 * (gi & 3))) & 255u, s1 = (scales1[gi >> 2] >> (8 * (gi & 3))) & 255u;
+                    const uint32_t *w0c = (j & 1) ? c0b : c0a, *w1c = (j & 1) ? c1b : c1a;
+                    const half8v xh = *reinterpret_cast<const half8v *>(ahi + k), xl = *reinterpret_cast<const half8v *>(alo + k);
+                    // byte-wise scale * code: at most 15 * 3, no carry between bytes
+                    const half8v w0 = half8_of_bytes(((w0c[0] >> shift) & 0x03030303u) * (s0 & 15u), ((w0c[1] >> shift) & 0x03030303u) * (s0 & 15u), (half_t)1024.0f);
+                    const half8v w1 = half8_of_bytes(((w1c[0] >> shift) & 0x03030303u) * (s1 & 15u), ((w1c[1] >> shift) & 0x03030303u) * (s1 & 15u), (half_t)1024.0f);
+                    const half_t m0 = (half_t)(int)(s0 >> 4), m1 = (half_t)(int)(s1 >> 4);
+                    const half8v mv0 = {m0, m0, m0, m0, m0, m0, m0, m0}, mv1 = {m1, m1, m1, m1, m1, m1, m1, m1};
+                    part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
+                    part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
+                    part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w0, part0, 0, 0, 0);
+                    part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w1, part1, 0, 0, 0);
+                    low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv0, low0, 0, 0, 0);
+                    low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv1, low1, 0, 0, 0);
+                    low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv0, low0, 0, 0, 0);
+                    low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv1, low1, 0, 0, 0);
+                }
             }
             const half2v h0 = __builtin_bit_cast(half2v, dd0), h1 = __builtin_bit_cast(half2v, dd1);
             const float d0 = (float)h0.x, n0 = (float)h0.y, d1 = (float)h1.x, n1 = (float)h1.y;
@@ -879,57 +891,79 @@ __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow
         }
         return;
     }
-    for (int g = 0; g < K / 32; g++) {          // one scale per 32 weights: two product steps per group
-        float16v part0 = zero, part1 = zero;
-        float s0, s1;
-        if (FMT == PF_Q8_0) {
-            s0 = (float)__builtin_bit_cast(half_t, reinterpret_cast<const uint16_t *>(r0.scales)[g]);
-            s1 = (float)__builtin_bit_cast(half_t, reinterpret_cast<const uint16_t *>(r1.scales)[g]);
-        } else {
-            s0 = 0.5f * pf_e8m0_scale(r0.scales[g]);   // the operands are twice the values
-            s1 = 0.5f * pf_e8m0_scale(r1.scales[g]);
-        }
-        uint2 m0 = {0, 0}, m1 = {0, 0};
-        if (FMT == PF_MXFP4) {   // bytes 8h..8h+7 of the block: low nibbles values 8h.., high nibbles values 16 + 8h..
-            m0 = *reinterpret_cast<const uint2 *>(r0.payload + 16 * (size_t)g + 8 * h);
-            m1 = *reinterpret_cast<const uint2 *>(r1.payload + 16 * (size_t)g + 8 * h);
-        }
+    for (int g0 = 4 * part; g0 < cols / 32; g0 += 4 * parts) {   // batches of four groups of 32 weights (cols is a multiple of 256)
+        const int first = c0 / 32 + g0;            // of the row's groups
+        uint2 q0[4][2], q1[4][2];
+        float s0[4], s1[4];
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            const int k = 32 * g + 16 * t + 8 * h;
-            const half8v xh = *reinterpret_cast<const half8v *>(ahi + k), xl = *reinterpret_cast<const half8v *>(alo + k);
-            half8v w0, w1;
+        for (int j = 0; j < 4; j++) {
             if (FMT == PF_Q8_0) {
-                const uint2 c0 = *reinterpret_cast<const uint2 *>(r0.payload + k), c1 = *reinterpret_cast<const uint2 *>(r1.payload + k);
-                w0 = half8_of_signed_bytes(c0.x, c0.y);
-                w1 = half8_of_signed_bytes(c1.x, c1.y);
-            } else {
-                const int sh = 4 * t;
-                w0 = half8_of_signed_bytes(plain_e2m1_twice4((m0.x >> sh) & 0x0F0F0F0Fu), plain_e2m1_twice4((m0.y >> sh) & 0x0F0F0F0Fu));
-                w1 = half8_of_signed_bytes(plain_e2m1_twice4((m1.x >> sh) & 0x0F0F0F0Fu), plain_e2m1_twice4((m1.y >> sh) & 0x0F0F0F0Fu));
+                s0[j] = (float)__builtin_bit_cast(half_t, reinterpret_cast<const uint16_t *>(r0.scales)[first + j]);
+                s1[j] = (float)__builtin_bit_cast(half_t, reinterpret_cast<const uint16_t *>(r1.scales)[first + j]);
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    q0[j][t] = *reinterpret_cast<const uint2 *>(r0.payload + 32 * (size_t)(first + j) + 16 * t + 8 * h);
+                    q1[j][t] = *reinterpret_cast<const uint2 *>(r1.payload + 32 * (size_t)(first + j) + 16 * t + 8 * h);
+                }
+            } else {   // MXFP4: bytes 8h..8h+7 of the block: low nibbles values 8h.., high nibbles values 16 + 8h..
+                s0[j] = 0.5f * pf_e8m0_scale(r0.scales[first + j]);   // the operands are twice the values
+                s1[j] = 0.5f * pf_e8m0_scale(r1.scales[first + j]);
+                q0[j][0] = *reinterpret_cast<const uint2 *>(r0.payload + 16 * (size_t)(first + j) + 8 * h);
+                q1[j][0] = *reinterpret_cast<const uint2 *>(r1.payload + 16 * (size_t)(first + j) + 8 * h);
+                q0[j][1] = uint2{q0[j][0].x >> 4, q0[j][0].y >> 4};
+                q1[j][1] = uint2{q1[j][0].x >> 4, q1[j][0].y >> 4};
             }
-            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
-            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
-            part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w0, part0, 0, 0, 0);
-            part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w1, part1, 0, 0, 0);
         }
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            acc0[r] = fmaf(s0, part0[r], acc0[r]);
-            acc1[r] = fmaf(s1, part1[r], acc1[r]);
+        for (int j = 0; j < 4; j++) {
+            float16v part0 = zero, part1 = zero;
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const int k = 32 * (g0 + j) + 16 * t + 8 * h;
+                const half8v xh = *reinterpret_cast<const half8v *>(ahi + k), xl = *reinterpret_cast<const half8v *>(alo + k);
+                half8v w0, w1;
+                if (FMT == PF_Q8_0) {
+                    w0 = half8_of_signed_bytes(q0[j][t].x, q0[j][t].y);
+                    w1 = half8_of_signed_bytes(q1[j][t].x, q1[j][t].y);
+                } else {
+                    w0 = half8_of_signed_bytes(plain_e2m1_twice4(q0[j][t].x & 0x0F0F0F0Fu), plain_e2m1_twice4(q0[j][t].y & 0x0F0F0F0Fu));
+                    w1 = half8_of_signed_bytes(plain_e2m1_twice4(q1[j][t].x & 0x0F0F0F0Fu), plain_e2m1_twice4(q1[j][t].y & 0x0F0F0F0Fu));
+                }
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
+                part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w0, part0, 0, 0, 0);
+                part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w1, part1, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc0[r] = fmaf(s0[j], part0[r], acc0[r]);
+                acc1[r] = fmaf(s1[j], part1[r], acc1[r]);
+            }
         }
     }
 }
 
+#define PLAIN_CHUNK 512                     // activation columns staged per pass
+#define PLAIN_PITCH (PLAIN_CHUNK + 8)       // halfs between staged rows: 16 bytes of padding spread the rows over the banks
+#define PLAIN_LDS (2 * 32 * PLAIN_PITCH * 2)
+
 // grid: (row tiles the list can hold) x slabs; 4 waves.  Items whose tensors are in a format of the ring
-// kernel are skipped here, as the ring kernel skips these.
+// kernel are skipped here, as the ring kernel skips these.  Per pass the workgroup stages 512 columns
+// of the tile's 32 activation rows (high and low parts) in LDS, one 1 KB row part per load instruction.
+// split != 0 (gate/up only): the four waves share 32 units and take a quarter of the columns each; their
+// partial sums meet in LDS and wave 0 adds them in wave order.  For matrices with few row tiles (the
+// shared expert) that gives four times as many workgroups.
 template <int MODE>
-__global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int tokens, int slabs) {
+__global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int tokens, int slabs, int split) {
+    extern __shared__ __align__(16) unsigned char plain_lds[];
+    __shared__ uint32_t src_row[32];
+    __shared__ float src_scale[32];
+    half_t *tile = reinterpret_cast<half_t *>(plain_lds);
     const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
     const int E = a.experts, K = a.top_k, P = tokens * K;
-    const uint32_t tile = blockIdx.x / slabs, slab = blockIdx.x % slabs;
-    if (tile >= a.tiles[0]) return;
-    const uint32_t entry = a.tiles[1 + tile];
+    const uint32_t item_tile = blockIdx.x / slabs, slab = blockIdx.x % slabs;
+    if (item_tile >= a.tiles[0]) return;
+    const uint32_t entry = a.tiles[1 + item_tile];
     const int expert = entry & 0xffffu, m0 = 32 * (int)(entry >> 16);
     const bool shared = expert == E;
     const int first = shared ? P : (int)a.offsets[expert];
@@ -940,20 +974,11 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int to
     const int t0 = MODE == PF_GEMM_GATE_UP ? (shared ? 4 : 1) : (shared ? 6 : 3);
     const uint32_t fmt = a.type[t0];
     if (fmt != PF_Q8_0 && fmt != PF_Q2_K && fmt != PF_MXFP4) return;
-    // this lane's activation row as an operand (row n of the tile), and the rows' scales for the epilogue
-    const int a_cols = MODE == PF_GEMM_GATE_UP ? a.hidden : inter;
-    const half_t *a16 = reinterpret_cast<const half_t *>(MODE == PF_GEMM_GATE_UP ? a.x16 : shared ? a.sact16 : a.act16);
-    const float *a_scale = MODE == PF_GEMM_GATE_UP ? a.x_scale : shared ? a.sact_scale : a.act_scale;
-    auto source_row = [&](int m) -> uint32_t {
-        if (m >= rows_here) return MODE == PF_GEMM_GATE_UP || shared ? a.token_cap : a.token_cap * (uint32_t)K;   // the all-zero row
-        if (shared) return (uint32_t)(m0 + m);
-        return MODE == PF_GEMM_GATE_UP ? a.row_to_pair[first + m0 + m] / (uint32_t)K : (uint32_t)(first + m0 + m);
-    };
-    const half_t *ahi = a16 + (size_t)source_row(n) * pf_half_row(a_cols);
     int row_a, row_b, t1, limit;
+    const int slab_rows = MODE != PF_GEMM_GATE_UP ? 256 : split ? 32 : 128;
     if (MODE == PF_GEMM_GATE_UP) {
         limit = inter;
-        row_a = row_b = 128 * (int)slab + 32 * wave + n;   // the unit's gate row and up row
+        row_a = row_b = slab_rows * (int)slab + (split ? 0 : 32 * wave) + n;   // the unit's gate row and up row
         t1 = t0 + 1;
     } else {
         limit = a.hidden;
@@ -961,18 +986,73 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int to
         row_b = row_a + 32;
         t1 = t0;
     }
-    if (row_a - n >= limit) return;   // the whole wave: no barrier in this kernel
+    if (slab_rows * (int)slab >= limit) return;   // the slab starts beyond the matrix: the whole workgroup
+    const bool active = row_a - n < limit;        // this wave has rows (the others stay for the barriers)
+    const int part = split ? wave : 0, parts = split ? 4 : 1;
+    // the tile's activation rows (the all-zero row beyond the tile's last) and their scales
+    const int a_cols = MODE == PF_GEMM_GATE_UP ? a.hidden : inter;
+    const half_t *a16 = reinterpret_cast<const half_t *>(MODE == PF_GEMM_GATE_UP ? a.x16 : shared ? a.sact16 : a.act16);
+    const float *a_scale = MODE == PF_GEMM_GATE_UP ? a.x_scale : shared ? a.sact_scale : a.act_scale;
+    if (threadIdx.x < 32) {
+        const int m = threadIdx.x;
+        uint32_t src;
+        if (m >= rows_here) src = MODE == PF_GEMM_GATE_UP || shared ? a.token_cap : a.token_cap * (uint32_t)K;
+        else if (shared) src = (uint32_t)(m0 + m);
+        else src = MODE == PF_GEMM_GATE_UP ? a.row_to_pair[first + m0 + m] / (uint32_t)K : (uint32_t)(first + m0 + m);
+        src_row[m] = src;
+        src_scale[m] = m < rows_here ? a_scale[src] : 0.0f;
+    }
+    __syncthreads();
     const PlainRow r0 = plain_row(a, t0, ex, min(row_a, limit - 1)), r1 = plain_row(a, t1, ex, min(row_b, limit - 1));
+    const half_t *ahi = tile + (size_t)n * PLAIN_PITCH, *alo = ahi + 32 * PLAIN_PITCH;
     float16v acc0 = {0}, acc1 = {0};
-    if (fmt == PF_Q8_0) plain_product<PF_Q8_0>(r0, r1, ahi, a_cols, a_cols, h, acc0, acc1);
-    else if (fmt == PF_MXFP4) plain_product<PF_MXFP4>(r0, r1, ahi, a_cols, a_cols, h, acc0, acc1);
-    else plain_product<PF_Q2_K>(r0, r1, ahi, a_cols, a_cols, h, acc0, acc1);
+    for (int c0 = 0; c0 < a_cols; c0 += PLAIN_CHUNK) {
+        const int cols = min(PLAIN_CHUNK, a_cols - c0);
+        if (c0) __syncthreads();   // the previous pass has been consumed
+        // 64 row parts (32 rows, high and low) over the four waves; a lane moves 16 bytes of each
+#pragma unroll 4
+        for (int i = 0; i < 16; i++) {
+            const int part = 16 * wave + i, row = part & 31, low = part >> 5;
+            if (16 * lane < 2 * cols)
+                to_lds(a16 + (size_t)src_row[row] * pf_half_row(a_cols) + (size_t)low * a_cols + c0 + 8 * lane,
+                       reinterpret_cast<unsigned char *>(tile + ((size_t)low * 32 + row) * PLAIN_PITCH));
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (active) {
+            if (fmt == PF_Q8_0) plain_product<PF_Q8_0>(r0, r1, ahi, alo, c0, cols, h, part, parts, acc0, acc1);
+            else if (fmt == PF_MXFP4) plain_product<PF_MXFP4>(r0, r1, ahi, alo, c0, cols, h, part, parts, acc0, acc1);
+            else plain_product<PF_Q2_K>(r0, r1, ahi, alo, c0, cols, h, part, parts, acc0, acc1);
+        }
+    }
+    if (split) {   // every wave is active here: the partial sums of waves 1..3 go through LDS (over the staged columns)
+        __syncthreads();
+        float *sums = reinterpret_cast<float *>(plain_lds);
+        if (wave) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                sums[((wave - 1) * 32 + r) * 64 + lane] = acc0[r];
+                sums[((wave - 1) * 32 + 16 + r) * 64 + lane] = acc1[r];
+            }
+        }
+        __syncthreads();
+        if (wave) return;
+#pragma unroll
+        for (int w = 0; w < 3; w++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                acc0[r] += sums[(w * 32 + r) * 64 + lane];
+                acc1[r] += sums[(w * 32 + 16 + r) * 64 + lane];
+            }
+        }
+    }
+    if (!active) return;
     // epilogue: the lane holds column n of its two tiles; register r is row 8 (r / 4) + 4 h + r % 4
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         const int m = 8 * (r >> 2) + 4 * h + (r & 3);
         if (m >= rows_here) continue;
-        const float rs = a_scale[source_row(m)];
+        const float rs = src_scale[m];
         if (MODE == PF_GEMM_GATE_UP) {
             if (row_a >= limit) continue;
             const float v = pf_silu(acc0[r] * rs) * (acc1[r] * rs);
@@ -1051,6 +1131,17 @@ static void launch_gemm(const PfKernelArgs &a, int tokens, int slabs, hipStream_
     hipLaunchKernelGGL((pf_k_pf_gemm<MODE, FMT>), dim3(grid), dim3(64 * (NW + NL)), lds, stream, a, tokens, slabs);
 }
 
+template <int MODE>
+static void launch_gemm_plain(const PfKernelArgs &a, int tokens, unsigned tile_cap, int slabs, int split, hipStream_t stream) {
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_pf_gemm_plain<MODE>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, PLAIN_LDS);
+        configured = true;
+    }
+    hipLaunchKernelGGL(pf_k_pf_gemm_plain<MODE>, dim3(tile_cap * slabs), dim3(256), PLAIN_LDS, stream, a, tokens, slabs, split);
+}
+
 void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     const int H = a.hidden, E = a.experts, K = a.top_k, I = a.inter, Is = a.shared_inter, P = tokens * K;
     const int last = stage_limit ? stage_limit : 4;
@@ -1073,10 +1164,8 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     const unsigned tile_cap = (unsigned)pf_prefill_max_tiles(tokens, E, K);
     if (iq2) launch_gemm<PF_GEMM_GATE_UP, PF_IQ2_XXS>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
     else launch_gemm<PF_GEMM_GATE_UP, PF_Q4_K>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
-    if (a.type[4] != ring_fmt) {
-        const int slabs = (gi + 127) / 128;
-        hipLaunchKernelGGL(pf_k_pf_gemm_plain<PF_GEMM_GATE_UP>, dim3(tile_cap * slabs), dim3(256), 0, stream, a, tokens, slabs);
-    }
+    // only the shared expert's tiles (tokens / 32 of them) are left for this launch: columns split over the waves
+    if (a.type[4] != ring_fmt) launch_gemm_plain<PF_GEMM_GATE_UP>(a, tokens, tile_cap, (gi + 31) / 32, 1, stream);
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(P), dim3(256), 0, stream, a.act, (size_t)I, I, (half_t *)a.act16, a.act_scale,
                        (float *)nullptr, a.error_word);
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.shared_act, (size_t)Is, Is,
@@ -1087,9 +1176,6 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
         if (iq2) launch_gemm<PF_GEMM_DOWN, PF_IQ2_XXS>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
         else launch_gemm<PF_GEMM_DOWN, PF_Q4_K>(a, tokens, (H + 64 * NW - 1) / (64 * NW), stream);
     }
-    if (a.type[3] != ring_fmt || a.type[6] != ring_fmt) {
-        const int slabs = (H + 255) / 256;
-        hipLaunchKernelGGL(pf_k_pf_gemm_plain<PF_GEMM_DOWN>, dim3(tile_cap * slabs), dim3(256), 0, stream, a, tokens, slabs);
-    }
+    if (a.type[3] != ring_fmt || a.type[6] != ring_fmt) launch_gemm_plain<PF_GEMM_DOWN>(a, tokens, tile_cap, (H + 255) / 256, 0, stream);
     hipLaunchKernelGGL(pf_k_pf_combine, dim3(tokens), dim3(256), 0, stream, a, tokens);
 }
