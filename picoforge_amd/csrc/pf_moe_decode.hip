@@ -13,7 +13,9 @@
 // data dependencies of the block are kernel boundaries.
 //
 // Arithmetic.  A lane owns 64 consecutive weights of a row (two 32-weight groups:
-// one Q4_K nibble pair or two IQ2_XXS groups).  Activations are turned into block
+// one Q4_K nibble pair, two IQ2_XXS groups, two Q8_0 or MXFP4 blocks, a quarter of a
+// Q2_K block); the routed gate/up tensors, the routed down tensor and the shared
+// expert may each be in a format of their own.  Activations are turned into block
 // fixed point once per vector: per 32-group a power-of-two step and, per value, a
 // 21-bit integer written as three balanced base-128 digits.  Weight codes are small
 // integers in both formats, so the group dot product is three v_dot4_i32_i8 chains
