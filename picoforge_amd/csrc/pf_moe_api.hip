@@ -253,7 +253,7 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_UNIQ] = (1 + 3 * Td * K) * 4;
     want[W_ERR] = 256;
     want[W_EXACT] = 256;
-    want[W_FLAGS] = T * 4;
+    want[W_FLAGS] = (T + 1) * 4;
     // prefill path: fp16 copies, per-row scales, down products in expert order, grouping tables
     const bool prefill = T > PF_DECODE_MAX_TOKENS && pf_prefill_supported(*d);
     const size_t Tp = prefill ? T : 0, Is = d->shared_inter;

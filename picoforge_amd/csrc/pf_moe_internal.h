@@ -31,7 +31,8 @@ struct PfKernelArgs {
     uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
     uint32_t *error_word;
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
-    uint32_t *route_flags;           // [tokens] 1 = route again in serial order
+    uint32_t *route_flags;           // tokens to route again in serial order: [0] their number, then the tokens; the kernel
+                                     // before the routing clears [0]
     // prefill path
     uint32_t token_cap;              // rows the workspace holds; row token_cap (token_cap * top_k for act16) of an fp16 form is all zero
     uint16_t *x16, *act16, *sact16;  // fp16 forms of x, act (pairs in expert order), shared act: per row the high

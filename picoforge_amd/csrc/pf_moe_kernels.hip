@@ -220,6 +220,7 @@ __global__ void __launch_bounds__(256) pf_k_pre(PfKernelArgs a) {
     extern __shared__ float lds[];
     __shared__ uint64_t grid[256];
     const int H = a.hidden, t = blockIdx.y, lane = pf_lane(), wave = threadIdx.x >> 6;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) a.route_flags[0] = 0;   // the routing's list starts empty
     if (stage_row(lds, a.x + (size_t)t * a.x_pitch, H, H)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     stage_grid(grid, a.iq2_grid);
     __syncthreads();

@@ -138,6 +138,7 @@ __global__ void __launch_bounds__(256) pf_k_pf_router(PfKernelArgs a, int tokens
     __shared__ float partial[3][16][64];
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     const int t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) a.route_flags[0] = 0;   // the routing's list starts empty
     const int i = lane & 31, kk = lane >> 5;
     const int t = min(t0 + i, tokens - 1), e = min(e0 + i, E);
     // the four waves share the tile and split the columns into quarters (hidden is a multiple of 32)

@@ -23,64 +23,92 @@ __global__ void __launch_bounds__(64) pf_k_route_fast(PfKernelArgs a) {
         a.ids[(size_t)t * K + lane] = r.id;
         a.route_weights[(size_t)t * K + lane] = r.weight;
     }
-    if (lane == 0) a.route_flags[t] = r.close ? 1u : 0u;
+    if (lane == 0 && r.close) {   // onto the list of tokens to route again in serial order: [0] count, then the tokens
+        const uint32_t at = atomicAdd(a.route_flags, 1u);
+        a.route_flags[1 + at] = (uint32_t)t;
+    }
 }
 
 // Serial-order recomputation for flagged tokens, in two kernels so that a token's logits
-// spread over many compute units: one wave per (token, slab of 64 experts), lane e owns expert e
-// and the sum runs over k in order, as the reference's.  The router copy is laid out for this,
-// [slab][hidden / 4][64 experts][4 consecutive k]: four steps of a wave are one 1 KB load at a
-// uniform base plus the lane's offset, and the token's values are scalar operands.  The sum is
-// one dependent chain; the loads are not: they are requested well ahead of the chain (a wave can
-// have 63 of them on their way, 252 steps).
-__global__ void __launch_bounds__(64) pf_k_route_fix_logits(PfKernelArgs a) {
+// spread over many compute units: one workgroup per (token, slab of 64 experts), lane e of its
+// first wave owns expert e and the sum runs over k in order, as the reference's.  The router copy
+// is laid out for this, [slab][hidden / 4][64 experts][4 consecutive k]: four steps of the wave
+// are one 1 KB piece.  The sum is one dependent chain of 2 x hidden operations; what it must never
+// do is wait for memory, so two more waves stream the slab's pieces into an eight-batch LDS ring
+// (16 pieces = 64 steps per batch, six batches ahead: about 100 KB on their way) and the token's
+// row sits in LDS too, read as broadcasts.  One workgroup barrier per batch hands a batch over and
+// frees the one before it.
+#define FIX_RING 8
+#define FIX_AHEAD 6    // batches on their way or waiting in the ring beyond the one being handed over
+#define FIX_BATCH 16   // 1 KB pieces per batch
+__global__ void __launch_bounds__(192) pf_k_route_fix_logits(PfKernelArgs a) {
 #pragma clang fp contract(off)
-    const int t = blockIdx.x, E = a.experts, H = a.hidden, lane = threadIdx.x;
+    extern __shared__ __align__(16) unsigned char fix_lds[];   // the ring, then the token's row
+    const int E = a.experts, H = a.hidden, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int e = blockIdx.y * PF_WAVE + lane;
-    if (!a.route_flags[t]) return;
-    const float *__restrict__ xs = a.x + (size_t)t * a.x_pitch;
-    const float4 *__restrict__ w = reinterpret_cast<const float4 *>(a.router_t) + (size_t)blockIdx.y * ((H + 3) / 4) * PF_WAVE + lane;
+    float4 *ring = reinterpret_cast<float4 *>(fix_lds);
+    float *xs = reinterpret_cast<float *>(fix_lds + FIX_RING * FIX_BATCH * 1024);
+    const float4 *__restrict__ w = reinterpret_cast<const float4 *>(a.router_t) + (size_t)blockIdx.y * ((H + 3) / 4) * PF_WAVE;
+    const int batches = H / 64;
+    const uint32_t listed = a.route_flags[0];
+    for (uint32_t item = blockIdx.x; item < listed; item += gridDim.x) {   // the workgroup's share of the listed tokens
+    const int t = (int)a.route_flags[1 + item];
+    const float *__restrict__ row = a.x + (size_t)t * a.x_pitch;
+    __syncthreads();   // the previous token's row has been used up
+    for (int k = threadIdx.x; k < H; k += blockDim.x) xs[k] = row[k];
+    __syncthreads();
+    if (wave >= 1) {   // two loaders: wave 1 the even batches, wave 2 the odd ones, three batches each on their way
+        const int mine = wave - 1;
+        auto issue = [&](int b) {   // batch b into slot b % FIX_RING: piece j lands at [slot][j][lane]
+            const float4 *src = w + (size_t)(FIX_BATCH * b) * PF_WAVE + lane;
+            unsigned char *dst = fix_lds + (size_t)(b % FIX_RING) * FIX_BATCH * 1024;
+#pragma unroll
+            for (int j = 0; j < FIX_BATCH; j++)
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(src + j * PF_WAVE),
+                                                 reinterpret_cast<uint32_t *>(dst + j * 1024), 16, 0, 0);
+        };
+        for (int b = mine; b < FIX_AHEAD && b < batches; b += 2) issue(b);
+        for (int s = 0; s < batches; s++) {
+            if ((s & 1) == mine) {
+                // batch s has landed when only this wave's younger batches (s + 2, s + 4) are outstanding
+                if (s + 4 < batches) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * FIX_BATCH) : "memory");
+                else if (s + 2 < batches) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(FIX_BATCH) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();   // hands batch s over; batch s - 1 has been consumed
+            if ((s & 1) == mine && s + FIX_AHEAD < batches) issue(s + FIX_AHEAD);
+        }
+        continue;
+    }
     float sum = 0.0f;
-    float4 w0[16], w1[16], w2[16];
-    const int batches = H / 64;   // 64 steps = 16 loads
-    auto load = [&](float4 (&dst)[16], int b) {
-        if (b >= batches) return;
-        const float4 *row = w + (size_t)(16 * b) * PF_WAVE;
+    for (int s = 0; s < batches; s++) {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const float4 *slot = ring + (size_t)(s % FIX_RING) * FIX_BATCH * PF_WAVE + lane;
+        const float4 *x4 = reinterpret_cast<const float4 *>(xs + 64 * s);
+        float4 wv[FIX_BATCH], xv[FIX_BATCH];
 #pragma unroll
-        for (int j = 0; j < 16; j++) dst[j] = row[j * PF_WAVE];
-    };
-    auto chain = [&](const float4 (&src)[16], int b) {
-        if (b >= batches) return;
-        const float *x = xs + 64 * b;
+        for (int j = 0; j < FIX_BATCH; j++) { wv[j] = slot[j * PF_WAVE]; xv[j] = x4[j]; }
 #pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const float p0 = src[j].x * x[4 * j];
+        for (int j = 0; j < FIX_BATCH; j++) {
+            const float p0 = wv[j].x * xv[j].x;
             sum = sum + p0;
-            const float p1 = src[j].y * x[4 * j + 1];
+            const float p1 = wv[j].y * xv[j].y;
             sum = sum + p1;
-            const float p2 = src[j].z * x[4 * j + 2];
+            const float p2 = wv[j].z * xv[j].z;
             sum = sum + p2;
-            const float p3 = src[j].w * x[4 * j + 3];
+            const float p3 = wv[j].w * xv[j].w;
             sum = sum + p3;
         }
-    };
-    // three batches rotate: two are on their way while one is summed
-    load(w0, 0);
-    load(w1, 1);
-    for (int b = 0; b < batches; b += 3) {
-        load(w2, b + 2);
-        chain(w0, b);
-        load(w0, b + 3);
-        chain(w1, b + 1);
-        load(w1, b + 4);
-        chain(w2, b + 2);
     }
-    const float *tail = reinterpret_cast<const float *>(w);
+    const float *tail = reinterpret_cast<const float *>(w + lane);
     for (int k = 64 * batches; k < H; k++) {   // the lane's k-quad at 256 (k / 4) floats
         const float p = tail[(size_t)(k / 4) * 4 * PF_WAVE + (k & 3)] * xs[k];
         sum = sum + p;
     }
     if (e < E) a.logits[(size_t)t * E + e] = sum;
+    }
 }
 
 // router [experts][hidden] -> [slab][ceil(hidden / 4)][64][4] (expert 64 * slab + lane, four
@@ -107,20 +135,24 @@ void pf_launch_router_slabs(const float *d_src, int experts, int hidden, float *
 
 __global__ void __launch_bounds__(64) pf_k_route_fix_select(PfKernelArgs a) {
     extern __shared__ float lds[];
-    const int t = blockIdx.x, E = a.experts;
-    if (!a.route_flags[t]) return;
+    const int E = a.experts;
     float *z = lds, *p = z + E, *q = p + E;
-    for (int e = threadIdx.x; e < E; e += PF_WAVE) z[e] = a.logits[(size_t)t * E + e];
-    pf_wave_lds_fence();
-    pf_route_exact_wave(z, p, q, E, a.top_k, a.norm_topk != 0, a.ids + (size_t)t * a.top_k,
-                        a.route_weights + (size_t)t * a.top_k, threadIdx.x);
-    if (threadIdx.x == 0) atomicAdd(a.exact_rows, 1u);
+    const uint32_t listed = a.route_flags[0];
+    for (uint32_t item = blockIdx.x; item < listed; item += gridDim.x) {
+        const int t = (int)a.route_flags[1 + item];
+        for (int e = threadIdx.x; e < E; e += PF_WAVE) z[e] = a.logits[(size_t)t * E + e];
+        pf_wave_lds_fence();
+        pf_route_exact_wave(z, p, q, E, a.top_k, a.norm_topk != 0, a.ids + (size_t)t * a.top_k,
+                            a.route_weights + (size_t)t * a.top_k, threadIdx.x);
+        if (threadIdx.x == 0) atomicAdd(a.exact_rows, 1u);
+    }
 }
 
-// Every token through the exact path (expert counts the fast kernel cannot hold).
-__global__ void pf_k_flag_all(uint32_t *flags, int n) {
+// Every token through the exact path (expert counts the fast kernel cannot hold): the full list.
+__global__ void pf_k_flag_all(uint32_t *list, int n) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) flags[i] = 1u;
+    if (i == 0) list[0] = (uint32_t)n;
+    if (i < n) list[1 + i] = (uint32_t)i;
 }
 
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
@@ -132,8 +164,17 @@ void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     else if (npl <= 4) hipLaunchKernelGGL(pf_k_route_fast<4>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 8) hipLaunchKernelGGL(pf_k_route_fast<8>, dim3(tokens), dim3(64), 0, stream, a);
     else hipLaunchKernelGGL(pf_k_route_fast<16>, dim3(tokens), dim3(64), 0, stream, a);
-    hipLaunchKernelGGL(pf_k_route_fix_logits, dim3(tokens, (a.experts + PF_WAVE - 1) / PF_WAVE), dim3(PF_WAVE), 0, stream, a);
-    hipLaunchKernelGGL(pf_k_route_fix_select, dim3(tokens), dim3(PF_WAVE), 3 * (size_t)a.experts * sizeof(float), stream,
+    const size_t fix_lds = (size_t)FIX_RING * FIX_BATCH * 1024 + (size_t)a.hidden * sizeof(float);
+    static bool configured = false;   // more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_route_fix_logits),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        configured = true;
+    }
+    // the listed tokens are few: a fixed number of workgroups walks the list
+    const int workers = tokens < 256 ? tokens : 256;
+    hipLaunchKernelGGL(pf_k_route_fix_logits, dim3(workers, (a.experts + PF_WAVE - 1) / PF_WAVE), dim3(3 * PF_WAVE), fix_lds, stream, a);
+    hipLaunchKernelGGL(pf_k_route_fix_select, dim3(workers), dim3(PF_WAVE), 3 * (size_t)a.experts * sizeof(float), stream,
                        a);
 }
 
