@@ -162,6 +162,8 @@ class HipShim:
         bind("pf_hip_hc_read_device", C.c_int, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_hc_add_device", C.c_int, vp, sz, sz, vp, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_moe_forward_hc_device", C.c_int, vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp)
+        bind("pf_hip_hc_read_host", C.c_int, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, u32p)
+        bind("pf_hip_hc_add_host", C.c_int, vp, sz, sz, vp, sz, vp, sz, sz, sz, sz, u32p)
         bind("pf_hip_hc_time_step", C.c_int, C.c_int, vp, vp, vp, vp, sz, sz, sz, sz, vp, P(C.c_float))
         bind("pf_hip_moe_time_forwards_hc", C.c_int, vp, vp, vp, vp, sz, vp, vp, sz, sz, sz, C.c_int, P(C.c_float))
 

@@ -120,3 +120,27 @@ def test_product_fails_loudly_without_a_device():
     from helpers import call_route
     st, p, ids, w, _ = call_route(api, cfg, np.zeros((1, 4), dtype=np.float32))
     assert st in (abi.QW4_GPU_ERROR, abi.QW4_UNSUPPORTED) and (p == -99).all()
+
+
+def test_shim_entry_points_refuse_bad_arguments_before_touching_a_device():
+    """Null handles, zero dimensions and pitches narrower than a row are refused by the C-ABI shim itself
+    (PF_HIP_E_ARGUMENT = 1): no device is needed to find that out."""
+    hip = pf.load_product().hip
+    word = C.c_uint32()
+    ms = C.c_float()
+    buf = (C.c_float * 64)()
+    p = C.cast(buf, C.c_void_p)
+    assert hip.hc_read_device(None, 8, 4, p, 8, 4, p, 4, 1, 2, 4, p, None) == 1
+    assert hip.hc_read_device(p, 8, 4, p, 8, 4, p, 4, 1, 0, 4, p, None) == 1          # no streams
+    assert hip.hc_read_device(p, 8, 2, p, 8, 4, p, 4, 1, 2, 4, p, None) == 1          # stream pitch below hidden
+    assert hip.hc_read_device(p, 8, 4, p, 8, 4, p, 4, 1, 2, 4, None, None) == 1       # no error word
+    assert hip.hc_read_device(p, 8, 4, p, 8, 4, p, 4, 0, 2, 4, p, None) == 0          # no tokens: nothing to do
+    assert hip.hc_add_device(p, 8, 4, None, 4, p, 2, 1, 2, 4, p, None) == 1
+    assert hip.hc_add_device(p, 8, 4, p, 4, p, 1, 1, 2, 4, p, None) == 1              # inject pitch below streams
+    assert hip.hc_add_device(p, 8, 4, p, 4, p, 2, 0, 2, 4, p, None) == 0
+    assert hip.moe_forward_hc_device(None, None, p, 8, 4, p, 8, 4, p, 8, 4, p, 2, 1, None) == 1
+    assert hip.moe_forward_device(None, None, p, 4, p, 4, 1, None) == 1
+    assert hip.moe_kernel_family(None, None, 1) == 0
+    assert hip.hc_time_step(0, None, p, p, p, 1, 2, 4, 1, p, C.byref(ms)) == 1
+    assert hip.hc_read_host(None, 32, 16, p, 32, 16, p, 16, 1, 2, 4, C.byref(word)) == 1
+    assert hip.hc_read_host(p, 32, 16, p, 32, 16, p, 16, 0, 2, 4, C.byref(word)) == 0
