@@ -150,3 +150,26 @@ def test_prefill_kernels_on_checkpoint_profiles(product, oracle, h, e, k, i, s, 
         layer.force_general()
         _, y, ids, w = layer.forward(x)
         assert_parity(y, ids, w, *want, label="general kernels on the same layer")
+
+
+@pytest.mark.parametrize("profile", ["q2", "q4"])
+def test_full_size_profile_layers(product, oracle, profile):
+    """The measured shape (hidden 2048, 512 experts, top-10, intermediate 512, shared 512) in the checkpoint
+    profiles: one to four decode tokens and the first rows of a 640-token chunk against the oracle, the whole
+    chunk against the general kernels of the same library."""
+    print(f"case full-size profile {profile}", flush=True)
+    cfg = abi.moe_config(2048, 512, 10, 512, 512)
+    weights, x = make_layer_inputs(cfg, profile, 640, seed=9)
+    want = forward_with(oracle, cfg, weights, x[:6])
+    with pf.MoeLayer(product, cfg, weights, 640) as layer:
+        moe, work = layer.device_handles()
+        assert product.hip.moe_kernel_family(moe, work, 4) == 1 and product.hip.moe_kernel_family(moe, work, 640) == 2
+        for tokens in (1, 4):
+            _, y, ids, w = layer.forward(x[:tokens])
+            assert_parity(y, ids, w, want[0][:tokens], want[1][:tokens], want[2][:tokens], label=f"decode T={tokens}")
+        _, y, ids, w = layer.forward(x)
+        worst = assert_parity(y[:6], ids[:6], w[:6], *want, label="chunk, first rows against the oracle")
+        layer.force_general()
+        _, yg, idsg, wg = layer.forward(x)
+        assert_parity(y, ids, w, yg, idsg, wg, label="chunk against the general kernels")
+    print(f"  max abs err {worst:.2e}", flush=True)
