@@ -840,22 +840,32 @@ __device__ __forceinline__ PlainRow plain_row(const PfKernelArgs &a, int t, size
 }
 
 // acc0 / acc1 += staged activation columns [c0, c0 + cols) x the same columns of weight rows r0 / r1.
-// ahi / alo: this lane's activation row in LDS (high and low parts of the staged columns).  The
-// weight bytes of several groups are requested before the first product of the batch.
+// ahi / alo: this lane's activation row in LDS (high and low parts of the staged columns); sums: the
+// row's sums over every 16 staged columns (high parts, low parts sums_low further on; Q2_K only).
+// The weight bytes of several groups are requested before the first product of the batch.
 // A wave takes every `parts`-th batch (256-block for Q2_K) starting with batch `part`: with parts > 1 the
 // waves of a workgroup share one pair of rows and their partial sums are added afterwards.
 template <int FMT>
 __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow &r1, const half_t *ahi, const half_t *alo,
-                                              int c0, int cols, int h, int part, int parts, float16v &acc0, float16v &acc1) {
+                                              const half_t *sums, int sums_low, int c0, int cols, int h, int part, int parts,
+                                              float16v &acc0, float16v &acc1) {
     const float16v zero = {0};
     if (FMT == PF_Q2_K) {
         for (int b = part; b < cols / 256; b += parts) {
             const uint8_t *blk0 = r0.payload + 84 * (size_t)(c0 / 256 + b), *blk1 = r1.payload + 84 * (size_t)(c0 / 256 + b);
             const uint32_t dd0 = *reinterpret_cast<const uint32_t *>(blk0 + 80), dd1 = *reinterpret_cast<const uint32_t *>(blk1 + 80);
-            float16v part0 = zero, part1 = zero, low0 = zero, low1 = zero;
+            float16v part0 = zero, part1 = zero;
+            const uint32_t *sw0 = reinterpret_cast<const uint32_t *>(blk0), *sw1 = reinterpret_cast<const uint32_t *>(blk1);   // 4-byte aligned
+            // Q: the 16 groups' minima (scale bytes 8h..8h+7, high nibbles) against the rows' sums over the same groups
+            const half8v sh = *reinterpret_cast<const half8v *>(sums + 16 * b + 8 * h), sl = *reinterpret_cast<const half8v *>(sums + sums_low + 16 * b + 8 * h);
+            const half8v mv0 = half8_of_bytes((sw0[2 * h] >> 4) & 0x0F0F0F0Fu, (sw0[2 * h + 1] >> 4) & 0x0F0F0F0Fu, (half_t)1024.0f);
+            const half8v mv1 = half8_of_bytes((sw1[2 * h] >> 4) & 0x0F0F0F0Fu, (sw1[2 * h + 1] >> 4) & 0x0F0F0F0Fu, (half_t)1024.0f);
+            float16v low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(sh, mv0, zero, 0, 0, 0);
+            float16v low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(sh, mv1, zero, 0, 0, 0);
+            low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(sl, mv0, low0, 0, 0, 0);
+            low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(sl, mv1, low1, 0, 0, 0);
 #pragma unroll
             for (int half = 0; half < 2; half++) {   // eight groups of 16 weights per batch: one 32-byte half of the codes
-                const uint32_t *sw0 = reinterpret_cast<const uint32_t *>(blk0), *sw1 = reinterpret_cast<const uint32_t *>(blk1);   // 4-byte aligned
                 const uint32_t *q0 = reinterpret_cast<const uint32_t *>(blk0 + 16 + 32 * half + 8 * h);
                 const uint32_t *q1 = reinterpret_cast<const uint32_t *>(blk1 + 16 + 32 * half + 8 * h);
                 // bytes 8h..8h+7 and 16 + 8h..: the groups at l % 32 = 0 and 16, each at four bit planes
@@ -870,16 +880,10 @@ __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow
                     // byte-wise scale * code: at most 15 * 3, no carry between bytes
                     const half8v w0 = half8_of_bytes(((w0c[0] >> shift) & 0x03030303u) * (s0 & 15u), ((w0c[1] >> shift) & 0x03030303u) * (s0 & 15u), (half_t)1024.0f);
                     const half8v w1 = half8_of_bytes(((w1c[0] >> shift) & 0x03030303u) * (s1 & 15u), ((w1c[1] >> shift) & 0x03030303u) * (s1 & 15u), (half_t)1024.0f);
-                    const half_t m0 = (half_t)(int)(s0 >> 4), m1 = (half_t)(int)(s1 >> 4);
-                    const half8v mv0 = {m0, m0, m0, m0, m0, m0, m0, m0}, mv1 = {m1, m1, m1, m1, m1, m1, m1, m1};
                     part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
                     part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
                     part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w0, part0, 0, 0, 0);
                     part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, w1, part1, 0, 0, 0);
-                    low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv0, low0, 0, 0, 0);
-                    low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, mv1, low1, 0, 0, 0);
-                    low0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv0, low0, 0, 0, 0);
-                    low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xl, mv1, low1, 0, 0, 0);
                 }
             }
             const half2v h0 = __builtin_bit_cast(half2v, dd0), h1 = __builtin_bit_cast(half2v, dd1);
@@ -946,7 +950,9 @@ __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow
 
 #define PLAIN_CHUNK 512                     // activation columns staged per pass
 #define PLAIN_PITCH (PLAIN_CHUNK + 8)       // halfs between staged rows: 16 bytes of padding spread the rows over the banks
-#define PLAIN_LDS (2 * 32 * PLAIN_PITCH * 2)
+#define PLAIN_SUMS (PLAIN_CHUNK / 16 + 8)   // halfs between the rows' sums over 16 columns
+#define PLAIN_TILE_BYTES (2 * 32 * PLAIN_PITCH * 2)
+#define PLAIN_LDS (PLAIN_TILE_BYTES + 2 * 32 * PLAIN_SUMS * 2)
 
 // grid: (row tiles the list can hold) x slabs; 4 waves.  Items whose tensors are in a format of the ring
 // kernel are skipped here, as the ring kernel skips these.  Per pass the workgroup stages 512 columns
@@ -959,7 +965,7 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int to
     extern __shared__ __align__(16) unsigned char plain_lds[];
     __shared__ uint32_t src_row[32];
     __shared__ float src_scale[32];
-    half_t *tile = reinterpret_cast<half_t *>(plain_lds);
+    half_t *tile = reinterpret_cast<half_t *>(plain_lds), *sums = reinterpret_cast<half_t *>(plain_lds + PLAIN_TILE_BYTES);
     const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
     const int E = a.experts, K = a.top_k, P = tokens * K;
     const uint32_t item_tile = blockIdx.x / slabs, slab = blockIdx.x % slabs;
@@ -1020,20 +1026,41 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int to
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        if (fmt == PF_Q2_K) {
+            // sums of the staged rows over every 16 columns, as two-part halfs like the values themselves:
+            // thread = (row, four neighbouring groups)
+            const int row = threadIdx.x >> 3, g0 = 4 * (threadIdx.x & 7);
+#pragma unroll
+            for (int g = g0; g < g0 + 4; g++) {
+                float total = 0.0f;
+                if (16 * g < cols) {
+                    const half_t *hi = tile + (size_t)row * PLAIN_PITCH + 16 * g, *lo = hi + 32 * PLAIN_PITCH;
+                    const half8v a0 = *reinterpret_cast<const half8v *>(hi), a1 = *reinterpret_cast<const half8v *>(hi + 8);
+                    const half8v b0 = *reinterpret_cast<const half8v *>(lo), b1 = *reinterpret_cast<const half8v *>(lo + 8);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) total += ((float)a0[i] + (float)b0[i]) + ((float)a1[i] + (float)b1[i]);
+                }
+                const half_t top = (half_t)total;
+                sums[(size_t)row * PLAIN_SUMS + g] = top;
+                sums[(size_t)(32 + row) * PLAIN_SUMS + g] = (half_t)(total - (float)top);
+            }
+            __syncthreads();
+        }
         if (active) {
-            if (fmt == PF_Q8_0) plain_product<PF_Q8_0>(r0, r1, ahi, alo, c0, cols, h, part, parts, acc0, acc1);
-            else if (fmt == PF_MXFP4) plain_product<PF_MXFP4>(r0, r1, ahi, alo, c0, cols, h, part, parts, acc0, acc1);
-            else plain_product<PF_Q2_K>(r0, r1, ahi, alo, c0, cols, h, part, parts, acc0, acc1);
+            const half_t *mine = sums + (size_t)n * PLAIN_SUMS;
+            if (fmt == PF_Q8_0) plain_product<PF_Q8_0>(r0, r1, ahi, alo, mine, 32 * PLAIN_SUMS, c0, cols, h, part, parts, acc0, acc1);
+            else if (fmt == PF_MXFP4) plain_product<PF_MXFP4>(r0, r1, ahi, alo, mine, 32 * PLAIN_SUMS, c0, cols, h, part, parts, acc0, acc1);
+            else plain_product<PF_Q2_K>(r0, r1, ahi, alo, mine, 32 * PLAIN_SUMS, c0, cols, h, part, parts, acc0, acc1);
         }
     }
     if (split) {   // every wave is active here: the partial sums of waves 1..3 go through LDS (over the staged columns)
         __syncthreads();
-        float *sums = reinterpret_cast<float *>(plain_lds);
+        float *partial = reinterpret_cast<float *>(plain_lds);
         if (wave) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                sums[((wave - 1) * 32 + r) * 64 + lane] = acc0[r];
-                sums[((wave - 1) * 32 + 16 + r) * 64 + lane] = acc1[r];
+                partial[((wave - 1) * 32 + r) * 64 + lane] = acc0[r];
+                partial[((wave - 1) * 32 + 16 + r) * 64 + lane] = acc1[r];
             }
         }
         __syncthreads();
@@ -1042,8 +1069,8 @@ __global__ void __launch_bounds__(256) pf_k_pf_gemm_plain(PfKernelArgs a, int to
         for (int w = 0; w < 3; w++) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                acc0[r] += sums[(w * 32 + r) * 64 + lane];
-                acc1[r] += sums[(w * 32 + 16 + r) * 64 + lane];
+                acc0[r] += partial[(w * 32 + r) * 64 + lane];
+                acc1[r] += partial[(w * 32 + 16 + r) * 64 + lane];
             }
         }
     }
