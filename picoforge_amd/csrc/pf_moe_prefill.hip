@@ -817,13 +817,21 @@ __device__ __forceinline__ half8v half8_of_signed_bytes(uint32_t b0, uint32_t b1
     return half8_of_bytes(b0 ^ 0x80808080u, b1 ^ 0x80808080u, (half_t)1152.0f);
 }
 
-// four E2M1 codes (one per byte, low nibble) as signed bytes holding twice their value
-__device__ __forceinline__ uint32_t plain_e2m1_twice4(uint32_t nibbles) {
-    const uint32_t sel = nibbles & 0x07070707u;
-    const uint32_t pos = __builtin_amdgcn_perm(0x0C080604u, 0x03020100u, sel);
-    const uint32_t neg = __builtin_amdgcn_perm(0xF4F8FAFCu, 0xFDFEFF00u, sel);
-    const uint32_t mask = ((nibbles >> 3) & 0x01010101u) * 0xFFu;
-    return (neg & mask) | (pos & ~mask);
+// Eight E2M1 codes (one per byte of two dwords, in the low nibble) as halfs holding twice their value:
+// 0, 1, 2, 3, 4, 6, 8, 12 are 0x0000, 0x3C00, 0x4000, 0x4200, 0x4400, 0x4600, 0x4800, 0x4A00, so a byte
+// permute looks up the halfs' high bytes, bit 3 of the code becomes the sign bit, and two more permutes
+// spread the four bytes over two pairs of halfs (selector 0x0C writes a zero byte).
+__device__ __forceinline__ half8v half8_of_e2m1(uint32_t n0, uint32_t n1) {
+    auto pairs = [](uint32_t n, uint32_t &lo, uint32_t &hi) {
+        uint32_t top = __builtin_amdgcn_perm(0x4A484644u, 0x42403C00u, n & 0x07070707u);
+        top |= (n << 4) & 0x80808080u;
+        lo = __builtin_amdgcn_perm(0u, top, 0x010C000Cu);
+        hi = __builtin_amdgcn_perm(0u, top, 0x030C020Cu);
+    };
+    uint4 bits;
+    pairs(n0, bits.x, bits.y);
+    pairs(n1, bits.z, bits.w);
+    return __builtin_bit_cast(half8v, bits);
 }
 
 struct PlainRow {            // one weight row as the kernel reads it
@@ -931,8 +939,8 @@ __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow
                     w0 = half8_of_signed_bytes(q0[j][t].x, q0[j][t].y);
                     w1 = half8_of_signed_bytes(q1[j][t].x, q1[j][t].y);
                 } else {
-                    w0 = half8_of_signed_bytes(plain_e2m1_twice4(q0[j][t].x & 0x0F0F0F0Fu), plain_e2m1_twice4(q0[j][t].y & 0x0F0F0F0Fu));
-                    w1 = half8_of_signed_bytes(plain_e2m1_twice4(q1[j][t].x & 0x0F0F0F0Fu), plain_e2m1_twice4(q1[j][t].y & 0x0F0F0F0Fu));
+                    w0 = half8_of_e2m1(q0[j][t].x & 0x0F0F0F0Fu, q0[j][t].y & 0x0F0F0F0Fu);
+                    w1 = half8_of_e2m1(q1[j][t].x & 0x0F0F0F0Fu, q1[j][t].y & 0x0F0F0F0Fu);
                 }
                 part0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w0, part0, 0, 0, 0);
                 part1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xh, w1, part1, 0, 0, 0);
