@@ -83,10 +83,10 @@ WORKLOADS = {
 # HBM bytes per launch of each workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE scaled by the same counters on a plain 256 MiB copy (profiles/*.txt hold the runs).
 # A counter result cannot be read live; None where no such run exists for the workload.
-MEASURED_TRAFFIC = {"iq2xxs_decode": 9907723, "q4k_decode": 19881663, "q4k_verify4": None,
-                    "q4k_prefill1024": 816829197, "iq2xxs_prefill1024": 459296841,
+MEASURED_TRAFFIC = {"iq2xxs_decode": 9907760, "q4k_decode": 19881668, "q4k_verify4": None,
+                    "q4k_prefill1024": 816800329, "iq2xxs_prefill1024": 450023382,
                     # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
-                    "q4k_prefill1024_hc": 75633480, "iq2xxs_decode_hc": 117102, "q4k_decode_hc": None,
+                    "q4k_prefill1024_hc": 75633614, "iq2xxs_decode_hc": 117059, "q4k_decode_hc": None,
                     "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None,
                     "q4profile_prefill1024": None}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
