@@ -2,10 +2,10 @@
  *
  * Layout-compatible with the host-visible part of the reference's
  * src/qwen4_packed.h:6-19 and the two GGUF descriptor types it takes from
- * src/gguf.h:20-25.  Formats this build executes: F32 (type 0), Q4_K (type 12)
- * and IQ2_XXS (type 16).  The reference's other formats (F16, Q8_0, Q2_K, BF16,
- * MXFP4) are refused with QW4_UNSUPPORTED; unknown type ids with QW4_FORMAT as
- * in the reference (src/qwen4_packed_internal.h:57-63). */
+ * src/gguf.h:20-25.  Every format the reference registers is executed: F32 (type
+ * 0), F16 (1), Q8_0 (8), Q2_K (10), Q4_K (12), IQ2_XXS (16), BF16 (30) and MXFP4
+ * (39); unknown type ids are refused with QW4_FORMAT as in the reference
+ * (src/qwen4_packed_internal.h:57-63). */
 #ifndef PF_QWEN4_PACKED_H
 #define PF_QWEN4_PACKED_H
 #include "qwen4_types.h"

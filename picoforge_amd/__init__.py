@@ -7,3 +7,4 @@ if the library is missing, loading it raises.
 from . import abi  # noqa: F401
 from .binding import LibraryMissing, Synth, load_oracle, load_product, load_reference  # noqa: F401
 from .layer import LayerWeights, MoeError, MoeLayer, rms_normalise  # noqa: F401
+from .gguf import GgufError, GgufFile  # noqa: F401

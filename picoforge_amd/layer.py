@@ -81,12 +81,14 @@ class MoeError(RuntimeError):
 
 
 class MoeLayer:
-    def __init__(self, api, cfg, weights, token_cap):
+    def __init__(self, api, cfg, weights, token_cap, handle=None):
+        """handle: a Qwen4Moe the library already created from these weights (the layer then owns it)."""
         self.api, self.cfg, self.weights, self.cap = api, cfg, weights, token_cap
         self.err = abi.Qwen4Error()
-        self.handle, self.work = C.c_void_p(), C.c_void_p()
-        st = api.create(C.byref(cfg), C.byref(weights.struct), C.byref(self.handle), C.byref(self.err))
-        self._raise(st)
+        self.handle, self.work = handle or C.c_void_p(), C.c_void_p()
+        if handle is None:
+            st = api.create(C.byref(cfg), C.byref(weights.struct), C.byref(self.handle), C.byref(self.err))
+            self._raise(st)
         size = C.c_size_t()
         self._raise(api.work_size(self.handle, token_cap, C.byref(size), C.byref(self.err)))
         self.work_bytes = size.value

@@ -12,7 +12,7 @@ import picoforge_amd as pf
 from picoforge_amd import abi, binding
 
 ROOT = Path(__file__).resolve().parents[1]
-HEADERS = ["qwen4_packed.h", "qwen4_moe.h", "qwen4_hc.h", "pf_moe_hip.h"]
+HEADERS = ["qwen4_packed.h", "qwen4_moe.h", "qwen4_hc.h", "pf_gguf.h", "pf_moe_hip.h"]
 
 
 def declared_functions(header):
@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported():
         total += len(names)
         missing += [f"{header}:{n}" for n in names if not hasattr(lib, n)]
     assert not missing, missing
-    assert total >= 45
+    assert total >= 57
 
 
 def test_product_never_links_the_oracle():

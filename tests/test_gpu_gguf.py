@@ -1,0 +1,73 @@
+"""GPU parity of the MoE block on weights that come out of a GGUF file.
+
+The library opens the file, finds and checks a layer's eight tensors and uploads them
+(pf_gguf_moe_create); the CPU oracle runs on views of the very same file bytes.  Small whole models
+of both checkpoint profiles (every layer, the multi-token-prediction layer with its own formats
+included) and one layer at the size of the benchmarks, where the decode and matrix-core kernels run.
+"""
+import numpy as np
+import pytest
+
+import picoforge_amd as pf
+from picoforge_amd.gguf import GgufFile
+
+import gguf_files as gf
+from helpers import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def tokens_for(hidden, count, seed):
+    return pf.rms_normalise(pf.Synth().normal((count, hidden), seed))
+
+
+@pytest.mark.parametrize("profile", ["q2", "q4"])
+def test_every_layer_of_a_small_model(tmp_path, product, oracle, profile):
+    print(f"case small model, profile {profile}", flush=True)
+    mf = gf.ModelFile(profile=profile, kinds=("gdn", 4), mtp=1, dims=dict(experts=8, top_k=3), seed=3)
+    mf.write(tmp_path / "small.gguf")
+    with GgufFile(product, mf.path) as f:
+        model = f.moe_model()
+        assert (model.blocks, model.mtp_blocks, model.moe.experts) == (3, 1, 8)
+        for layer in range(model.blocks):
+            for count in (1, 3, 40):
+                x = tokens_for(mf.d["hidden"], count, 100 * layer + count)
+                with f.moe_layer(layer, count) as mine, f.moe_layer(layer, count, api=oracle) as cpu:
+                    _, y, ids, w = mine.forward(x)
+                    _, y_ref, ids_ref, w_ref = cpu.forward(x)
+                assert_parity(y, ids, w, y_ref, ids_ref, w_ref, f"{profile} layer {layer} tokens {count}")
+                assert np.abs(y_ref).max() > 1e-3
+
+
+def test_a_layer_outlives_its_file(tmp_path, product, oracle):
+    print("case layer used after the file is closed", flush=True)
+    mf = gf.ModelFile(profile="q4", kinds=("gdn",), mtp=0, moe_only=True, seed=5)
+    mf.write(tmp_path / "one.gguf")
+    x = tokens_for(mf.d["hidden"], 2, 7)
+    f = GgufFile(product, mf.path)
+    with f.moe_layer(0, 2, api=oracle) as cpu:
+        _, y_ref, ids_ref, w_ref = cpu.forward(x)
+    layer = f.moe_layer(0, 2)
+    f.close()                                   # the device copy stays; the mapping is gone
+    _, y, ids, w = layer.forward(x)
+    layer.close()
+    assert_parity(y, ids, w, y_ref, ids_ref, w_ref, "after close")
+
+
+def test_a_layer_of_benchmark_size_from_a_file(tmp_path, product, oracle):
+    """Hidden 2048, 512 experts, top-10, intermediate 512, shared 512, 460 MB of tensors: the
+    decode kernels at 1 and 4 tokens and the matrix-core kernels at 48 tokens must be the ones that run."""
+    print("case benchmark-size layer from a file, profile q2", flush=True)
+    dims = dict(hidden=2048, experts=512, top_k=10, inter=512, shared=512, streams=4)
+    mf = gf.ModelFile(profile="q2", kinds=("gdn",), mtp=0, dims=dims, moe_only=True, seed=9, std=0.02)
+    mf.write(tmp_path / "layer.gguf")
+    with GgufFile(product, mf.path) as f:
+        assert f.moe_model().moe.down_physical == 512 and f.moe_weights(0).nbytes > 400e6
+        for count, family in ((1, 1), (4, 1), (48, 2)):
+            x = tokens_for(2048, count, 40 + count)
+            with f.moe_layer(0, count) as mine, f.moe_layer(0, count, api=oracle) as cpu:
+                moe, work = mine.device_handles()
+                assert product.hip.moe_kernel_family(moe, work, count) == family
+                _, y, ids, w = mine.forward(x)
+                _, y_ref, ids_ref, w_ref = cpu.forward(x[:8])
+            assert_parity(y[:8], ids[:8], w[:8], y_ref, ids_ref, w_ref, f"tokens {count}")
