@@ -4,6 +4,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <mutex>
 
 static thread_local char g_error[256] = "";
 
@@ -92,6 +93,49 @@ static size_t split_header_bytes(uint32_t type) {
     return type == PF_IQ2_XXS || type == PF_Q8_0 ? 2 : type == PF_MXFP4 ? 1 : 0;
 }
 
+// Host bytes into device memory through a page-locked buffer of the library's own (32 MB, allocated
+// at the first upload and kept until the process ends), two halves in turn so that the CPU fills
+// one while the other is on its way.  The caller's memory (for a checkpoint: a read-only mapping of
+// the file) is read by the CPU only and never handed to the runtime, which would otherwise
+// page-lock it for the transfer.  Uploads of one process take turns.
+struct Bounce {
+    static constexpr size_t HALF = (size_t)16 << 20;
+    uint8_t *base = nullptr;
+    hipEvent_t sent[2] = {nullptr, nullptr};
+    bool open() {
+        if (base) return true;
+        const bool ok = hipHostMalloc((void **)&base, 2 * HALF, hipHostMallocDefault) == hipSuccess &&
+                        hipEventCreate(&sent[0]) == hipSuccess && hipEventCreate(&sent[1]) == hipSuccess;
+        if (!ok) base = nullptr;
+        return ok;
+    }
+    hipError_t upload(void *d_dst, const void *src, size_t bytes) {
+        hipError_t e = hipSuccess;
+        bool busy[2] = {false, false};
+        int k = 0;
+        for (size_t at = 0; at < bytes && e == hipSuccess; k ^= 1) {
+            const size_t n = bytes - at < HALF ? bytes - at : HALF;
+            if (busy[k]) e = hipEventSynchronize(sent[k]);
+            if (e != hipSuccess) break;
+            memcpy(base + k * HALF, static_cast<const uint8_t *>(src) + at, n);
+            e = hipMemcpyAsync(static_cast<uint8_t *>(d_dst) + at, base + k * HALF, n, hipMemcpyHostToDevice, nullptr);
+            if (e == hipSuccess) e = hipEventRecord(sent[k], nullptr);
+            busy[k] = true;
+            at += n;
+        }
+        const hipError_t done = hipStreamSynchronize(nullptr);   // the buffer is free again when this returns
+        return e != hipSuccess ? e : done;
+    }
+};
+
+static hipError_t upload_from_host(void *d_dst, const void *src, size_t bytes) {
+    static std::mutex turn;
+    static Bounce *bounce = new Bounce();   // never freed: the runtime may be gone when statics are destroyed
+    std::lock_guard<std::mutex> hold(turn);
+    if (!bounce->open()) return hipErrorOutOfMemory;
+    return bounce->upload(d_dst, src, bytes);
+}
+
 extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const host_weights[8], const size_t bytes[8],
                                  PfHipMoe **out) {
     if (out) *out = nullptr;
@@ -145,7 +189,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             size_t block, size;
             block_geometry(desc->type[a], &block, &size);
             e = hipMalloc((void **)&staging, gguf_bytes[a]);
-            if (e == hipSuccess) e = hipMemcpy(staging, host_weights[a], gguf_bytes[a], hipMemcpyHostToDevice);
+            if (e == hipSuccess) e = upload_from_host(staging, host_weights[a], gguf_bytes[a]);
             if (e == hipSuccess) {
                 if (desc->type[a] == PF_IQ2_XXS)
                     pf_launch_iq2_split(staging, m->w[a], reinterpret_cast<uint16_t *>(m->w[a] + m->scale_offset[a]),
@@ -157,7 +201,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             }
             if (staging) (void)hipFree(staging);
         } else if (e == hipSuccess) {
-            e = hipMemcpy(m->w[a], host_weights[a], m->bytes[a], hipMemcpyHostToDevice);
+            e = upload_from_host(m->w[a], host_weights[a], m->bytes[a]);
         }
         if (e != hipSuccess) {
             pf_set_error("weight upload", e);
@@ -762,7 +806,7 @@ extern "C" int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_
                  yb = (rows * n_out * 4 + 255) & ~(size_t)255;
     DeviceBlock blk;
     HIP_TRY(hipMalloc((void **)&blk.p, wb + xb + yb + 256));
-    HIP_TRY(hipMemcpy(blk.p, expert_bytes, row_bytes * n_out, hipMemcpyHostToDevice));
+    HIP_TRY(upload_from_host(blk.p, expert_bytes, row_bytes * n_out));
     HIP_TRY(hipMemcpy(blk.p + wb, x, rows * k_logical * 4, hipMemcpyHostToDevice));
     HIP_TRY(hipMemset(blk.p + wb + xb + yb, 0, 256));
     pf_launch_exact_matmul(gguf_type, blk.p, row_bytes, (int)n_out, (int)k_logical, (const float *)(blk.p + wb),
@@ -787,7 +831,7 @@ extern "C" int pf_hip_packed_decode_row_host(uint32_t gguf_type, const void *row
     const size_t wb = (row_bytes + 255) & ~(size_t)255, ob = (k_storage * 4 + 255) & ~(size_t)255;
     DeviceBlock blk;
     HIP_TRY(hipMalloc((void **)&blk.p, wb + ob + 256));
-    HIP_TRY(hipMemcpy(blk.p, row, row_bytes, hipMemcpyHostToDevice));
+    HIP_TRY(upload_from_host(blk.p, row, row_bytes));
     HIP_TRY(hipMemset(blk.p + wb + ob, 0, 256));
     pf_launch_exact_decode(gguf_type, blk.p, (int)k_storage, (float *)(blk.p + wb), (uint32_t *)(blk.p + wb + ob),
                            grid, nullptr);
