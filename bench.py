@@ -76,6 +76,11 @@ WORKLOADS = {
     "q4profile_prefill1024": dict(type="q4", tokens=1024, steps=50, warmup=5,
                                   label="checkpoint profile Q4 (Q4_K gate/up, MXFP4 down, Q8_0 shared expert), 1024-token "
                                         "prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
+    # the checkpoints' own widths (hidden 2560, intermediate 640, shared 640; the Q2_K down projection stored 768 wide)
+    "q2ckpt_decode": dict(type="q2", tokens=1, steps=5000, warmup=100, dims=(2560, 512, 10, 640, 640, 768),
+                          label="checkpoint profile Q2 at the checkpoints' widths, decode batch 1"),
+    "q4ckpt_decode": dict(type="q4", tokens=1, steps=5000, warmup=100, dims=(2560, 512, 10, 640, 640, 640),
+                          label="checkpoint profile Q4 at the checkpoints' widths, decode batch 1"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),
@@ -87,7 +92,7 @@ MEASURED_TRAFFIC = {"iq2xxs_decode": 9907760, "q4k_decode": 19881668, "q4k_verif
                     "q4k_prefill1024": 816800329, "iq2xxs_prefill1024": 450023382,
                     # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
                     "q4k_prefill1024_hc": 75633614, "iq2xxs_decode_hc": 117059, "q4k_decode_hc": None,
-                    "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None,
+                    "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None, "q2ckpt_decode": None, "q4ckpt_decode": None,
                     "q4profile_prefill1024": None}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
@@ -341,6 +346,9 @@ def main():
     if hip.device_count() < 1:
         sys.exit("no HIP device: the benchmark runs the HIP path only")
     cfg = workloads.measured_config()
+    if wl.get("dims"):
+        h, e, k, i, s_i, phys = wl["dims"]
+        cfg = abi.moe_config(h, e, k, i, s_i, down_physical=phys)
     if args.workload == "q4k_stack48":
         return run_stack(args, api, hip, cfg, steps, warmup)
     if wl.get("hc"):
@@ -422,7 +430,7 @@ def main():
                                   for j in (0, 2, 3)},
                  "binding_roofline": "hbm: about 80 flop per weight byte at this chunk size, below the MFMA ridge"}
     else:
-        alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique)
+        alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique, cfg=cfg)
         stage_bytes = [lb["routers"], unique * lb["gate_up"] + lb["shared_gate_up"],
                        unique * lb["down"] + lb["shared_down"]]
         if family == 0:
@@ -471,7 +479,8 @@ def main():
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if not prefill else "f16 products, f32 accumulation",
         "data": "synthetic",
-        "config": {"workload": f"one MoE layer, hidden 2048, 512 experts, top-10, intermediate 512, shared 512; "
+        "config": {"workload": f"one MoE layer, hidden {cfg.hidden_size}, {cfg.experts} experts, top-{cfg.top_k}, "
+                               f"intermediate {cfg.intermediate}, shared {cfg.shared_intermediate}; "
                                f"{wl['label']}; {n_inputs} seeded inputs{margins}",
                    "tokens_per_step": tokens, "expert_format": FORMAT_LABEL[wl["type"]],
                    "unique_experts_per_step": unique, "inputs": info},

@@ -37,6 +37,24 @@
 // steps (float), then K/32 group sums of the integer values.
 __host__ __device__ constexpr int image_words(int K) { return 3 * SEG_STRIDE * (K / 64) + 2 * (K / 32); }
 
+// Lanes that share one row of K values: the largest power of two that is at most K / 64 and at
+// most 32.  A lane takes the 64-value segment `seg` of the row and, where K / 64 is not that power
+// of two (K = 2560: 40 segments on 32 lanes, K = 640: 10 on 8), also segment seg + lanes if the
+// row has one (kernels instantiated with SPL = 2).
+__host__ __device__ inline int row_lanes(int K) {
+    int l = 1;
+    while (2 * l <= K / 64 && l < 32) l *= 2;
+    return l;
+}
+__host__ __device__ inline int row_passes(int K) { return (K / 64 + row_lanes(K) - 1) / row_lanes(K); }
+// Rows of the down projection per workgroup of kernel 3: what one wave covers in a step, doubled until
+// the row blocks of one token fit the 256 compute units (hidden 2560, intermediate 640: 16 rows, 160 blocks).
+__host__ __device__ inline int down_block_rows(int H, int I) {
+    int rows = 64 / row_lanes(I);
+    while ((H + rows - 1) / rows > 256 && rows < 64) rows *= 2;
+    return rows;
+}
+
 struct XSeg {          // one lane's 64 activations
     int d0[16], d1[16], d2[16];
     float step[2];
@@ -368,6 +386,7 @@ template <int FMT> __host__ __device__ constexpr int table_words() { return FMT 
 // ---- kernel 1: router logits -----------------------------------------------------------------
 // One F32 row per wave, all tokens: blocks [0, router_blocks) take the experts' rows, the
 // last block's first wave the shared router row (its sigmoid scales the shared expert).
+#define ROUTER_CHUNKS 10   // 16-byte pieces of a router row per lane: hidden <= 2560
 template <int NT>
 __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks) {
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
@@ -379,24 +398,24 @@ __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int route
     bool bad = false;
 #pragma unroll
     for (int t = 0; t < NT; t++) acc[t] = sq[t] = 0.0f;
-    // the whole row (hidden <= 2048: eight 16-byte chunks per lane) is requested before any use
-    float4 wv[8];
+    // the whole row (hidden <= 2560: ten 16-byte chunks per lane) is requested before any use
+    float4 wv[ROUTER_CHUNKS];
 #pragma unroll
-    for (int c = 0; c < 8; c++) {
+    for (int c = 0; c < ROUTER_CHUNKS; c++) {
         const int i = lane + PF_WAVE * c;
         wv[c] = i < H / 4 ? w[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        float4 xv[8];
+        float4 xv[ROUTER_CHUNKS];
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
+        for (int c = 0; c < ROUTER_CHUNKS; c++) {
             const int i = lane + PF_WAVE * c;
             xv[c] = i < H / 4 ? reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch)[i]
                               : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
+        for (int c = 0; c < ROUTER_CHUNKS; c++) {
             const float p0 = wv[c].x * xv[c].x, p1 = wv[c].y * xv[c].y, p2 = wv[c].z * xv[c].z, p3 = wv[c].w * xv[c].w;
             acc[t] += (p0 + p1) + (p2 + p3);
             sq[t] = fmaf(p0, p0, fmaf(p1, p1, fmaf(p2, p2, fmaf(p3, p3, sq[t]))));
@@ -521,29 +540,42 @@ __device__ __forceinline__ void route_finish(const PfKernelArgs &a, RouteLds *R,
 // activations itself, so no wave waits for another after the routing.  Waves 0..parts*NT-1 first reduce
 // the logits to candidates, waves 12..15 turn the token rows into digit images.
 // One tile's rows against the tokens' images: the part of kernel 2 that depends on the tensors' format.
-template <int FMT, int NT>
+template <int FMT, int NT, int SPL>
 __device__ __forceinline__ void gate_up_tile(const PfKernelArgs &a, const int *images, const uint32_t *tables, int W, int H,
                                              int I, int gate_tensor, uint32_t e, uint32_t mask, int u, int n0, int tile,
                                              bool shared) {
     const int lane = pf_lane(), wave = threadIdx.x >> 6;
-    const int LPR = H / 64, RPH = 32 / LPR;
+    const int LPR = row_lanes(H), RPH = 32 / LPR;
     const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
+    const bool second = SPL > 1 && seg + LPR < H / 64;   // this lane also holds segment seg + LPR of its row
     // the tile's units over 16 waves: RPH per wave step, one or two steps
     const int per_wave = max(RPH, tile / 16), steps = per_wave / RPH, unit0 = wave * per_wave;
     if (unit0 >= tile) return;
-    WSeg<FMT> w[2];
+    WSeg<FMT> w[2][SPL];
 #pragma unroll
-    for (int st = 0; st < 2; st++)
-        if (st < steps) wseg_load<FMT>(w[st], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg);
+    for (int st = 0; st < 2; st++) {
+        if (st >= steps) break;
+        wseg_load<FMT>(w[st][0], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg);
+        if (SPL > 1 && second) wseg_load<FMT>(w[st][SPL - 1], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg + LPR);
+    }
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         if (!((mask >> t) & 1u)) continue;
         XSeg x;
         xseg_load(x, images + t * W, H, seg);
+        float dot[2];
+#pragma unroll
+        for (int st = 0; st < 2; st++) dot[st] = st < steps ? wseg_dot<FMT>(w[st][0], x, seg, tables) : 0.0f;
+        if (SPL > 1 && second) {
+            xseg_load(x, images + t * W, H, seg + LPR);
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+                if (st < steps) dot[st] += wseg_dot<FMT>(w[st][SPL - 1], x, seg + LPR, tables);
+        }
 #pragma unroll
         for (int st = 0; st < 2; st++) {
             if (st >= steps) break;
-            const float v = span_sum(wseg_dot<FMT>(w[st], x, seg, tables), LPR);
+            const float v = span_sum(dot[st], LPR);
             const float up = __shfl(v, (lane & 31) + 32);
             if (half == 0 && seg == 0) {
                 const float act = pf_silu(v) * up;
@@ -557,7 +589,7 @@ __device__ __forceinline__ void gate_up_tile(const PfKernelArgs &a, const int *i
 }
 
 // FMT: format of the routed gate and up tensors; FMTS: of the shared expert's.
-template <int FMT, int FMTS, int NT, int NPL>
+template <int FMT, int FMTS, int NT, int NPL, int SPL>
 __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int routed_blocks, int shared_blocks, int parts, int chunk, int tile,
                                                          int mode) {
     extern __shared__ int lds[];
@@ -626,7 +658,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
         }
         if (mode == 1) return;
         if (prefetcher) {
-            const int rows_next = 64 / (a.inter / 64), first = routed_blocks + shared_blocks;
+            const int rows_next = down_block_rows(H, a.inter), first = routed_blocks + shared_blocks;
             prefetch_down(a, R.uniq, U, ((int)blockIdx.x - first) / 8, ((int)gridDim.x - first) / 8, rows_next,
                                (H + rows_next - 1) / rows_next);
             return;
@@ -642,8 +674,8 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
         }
     }
     STAMP(4);
-    if (shared) gate_up_tile<FMTS, NT>(a, images, tables, W, H, I, gate_tensor, e, mask, u, n0, tile, true);
-    else gate_up_tile<FMT, NT>(a, images, tables, W, H, I, gate_tensor, e, mask, u, n0, tile, false);
+    if (shared) gate_up_tile<FMTS, NT, SPL>(a, images, tables, W, H, I, gate_tensor, e, mask, u, n0, tile, true);
+    else gate_up_tile<FMT, NT, SPL>(a, images, tables, W, H, I, gate_tensor, e, mask, u, n0, tile, false);
     STAMP(5);
 }
 
@@ -652,31 +684,58 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
 // wave covers the block's rows in one step.  Every wave turns its slot's activation row into a
 // digit image in LDS while its weight bytes are on their way.
 // One wave's products of kernel 3: its slot's rows of the block against its activation image.
-template <int FMT>
+template <int FMT, int SPL>
 __device__ __forceinline__ void down_rows(const PfKernelArgs &a, float *partial_row, int *image, const uint32_t *tables,
                                           const float *act_row, bool block_sync, int tensor, uint32_t e, int I, int H,
                                           int n_base, int rows_per_block, int s) {
     const int lane = pf_lane();
-    const int LPR = I / 64, rows = 64 / LPR, steps = rows >= rows_per_block ? 1 : rows_per_block / rows;
+    const int LPR = row_lanes(I), rows = 64 / LPR, steps = rows >= rows_per_block ? 1 : rows_per_block / rows;
     const int seg = lane & (LPR - 1), r = lane / LPR;
-    WSeg<FMT> w;   // further steps (a shared expert wider than the routed ones) load as they go
-    wseg_load<FMT>(w, a, tensor, e, min(n_base + r, H - 1), seg);
+    const bool second = SPL > 1 && seg + LPR < I / 64;   // this lane also holds segment seg + LPR of its row
+    WSeg<FMT> w[SPL];   // further steps (a shared expert wider than the routed ones) load as they go
+    wseg_load<FMT>(w[0], a, tensor, e, min(n_base + r, H - 1), seg);
+    if (SPL > 1 && second) wseg_load<FMT>(w[SPL - 1], a, tensor, e, min(n_base + r, H - 1), seg + LPR);
     build_image(image, act_row, I, 64 * s, 64);
     if (block_sync) __syncthreads();   // the tables staged by the whole workgroup
     else pf_wave_lds_fence();
-    XSeg x;
+    XSeg x;   // one segment's digits at a time: with two segments they are read from LDS again at every step
     xseg_load(x, image, I, seg);
+    if (SPL == 1) {
+        for (int st = 0; st < steps; st++) {
+            const float v = span_sum(wseg_dot<FMT>(w[0], x, seg, tables), LPR);
+            const int row = st * rows + r;
+            if (seg == 0 && row < rows_per_block) partial_row[row] = v;
+            if (st + 1 < steps) wseg_load<FMT>(w[0], a, tensor, e, min(n_base + (st + 1) * rows + r, H - 1), seg);
+        }
+        return;
+    }
     for (int st = 0; st < steps; st++) {
-        const float v = span_sum(wseg_dot<FMT>(w, x, seg, tables), LPR);
+        WSeg<FMT> next[SPL];   // the following step's weights, on their way during this step's products
+        if (st + 1 < steps) {
+            wseg_load<FMT>(next[0], a, tensor, e, min(n_base + (st + 1) * rows + r, H - 1), seg);
+            if (second) wseg_load<FMT>(next[SPL - 1], a, tensor, e, min(n_base + (st + 1) * rows + r, H - 1), seg + LPR);
+        }
+        if (st > 0) xseg_load(x, image, I, seg);
+        float dot = wseg_dot<FMT>(w[0], x, seg, tables);
+        if (second) {
+            xseg_load(x, image, I, seg + LPR);
+            dot += wseg_dot<FMT>(w[SPL - 1], x, seg + LPR, tables);
+        }
+        const float v = span_sum(dot, LPR);
         const int row = st * rows + r;
         if (seg == 0 && row < rows_per_block) partial_row[row] = v;
-        if (st + 1 < steps) wseg_load<FMT>(w, a, tensor, e, min(n_base + (st + 1) * rows + r, H - 1), seg);
+        if (st + 1 < steps) {
+            w[0] = next[0];
+            if (second) w[SPL - 1] = next[SPL - 1];
+        }
     }
 }
 
 // FMT: format of the routed down tensor; FMTS: of the shared expert's.
-template <int FMT, int FMTS, int NT>
-__global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_blocks, int rows_per_block, int image_pitch) {
+// MAXT: the largest workgroup the instantiation is launched with (64 threads per slot and the shared
+// expert): 768 leaves room for the second segment's registers when top_k <= 11.
+template <int FMT, int FMTS, int NT, int SPL, int MAXT>
+__global__ void __launch_bounds__(MAXT) pf_k_dec_down(PfKernelArgs a, int row_blocks, int rows_per_block, int image_pitch) {
     __shared__ float partial[17][64];
     extern __shared__ int lds[];
     constexpr bool TABLES = FMT == PF_IQ2_XXS || FMTS == PF_IQ2_XXS;
@@ -707,10 +766,10 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down(PfKernelArgs a, int row_bl
     if ((int)threadIdx.x < rows_per_block && n_base + (int)threadIdx.x < H)
         pf_output_prefetch(a, t, n_base + threadIdx.x, out_regs);
     if (shared)
-        down_rows<FMTS>(a, partial[s], image, tables, a.shared_act + (size_t)t * I, TABLES, 6, 0, I, H, n_base,
+        down_rows<FMTS, SPL>(a, partial[s], image, tables, a.shared_act + (size_t)t * I, TABLES, 6, 0, I, H, n_base,
                         rows_per_block, s);
     else
-        down_rows<FMT>(a, partial[s], image, tables, a.act + ((size_t)u * NT + t) * I, TABLES, 3, e, I, H, n_base,
+        down_rows<FMT, SPL>(a, partial[s], image, tables, a.act + ((size_t)u * NT + t) * I, TABLES, 3, e, I, H, n_base,
                        rows_per_block, s);
     __syncthreads();
     const int n = n_base + threadIdx.x;
@@ -779,11 +838,25 @@ static int decode_combination(const uint32_t type[8]) {
     return 0;
 }
 
+// A row of k values in a format: whole blocks, and whole 64-value segments for the lanes.
+static bool row_width_ok(uint32_t type, uint32_t k) {
+    const bool big = type == PF_Q4_K || type == PF_IQ2_XXS || type == PF_Q2_K;
+    return k && k % (big ? 256 : 64) == 0;
+}
+
+// Widths: hidden 512..2560 in whole 256-blocks (2560 is the checkpoints' width), intermediate widths
+// 256..2048 in whole 64-value segments (640 in the checkpoints); the routed down projection may be
+// stored wider than its logical width only as Q2_K (640 padded to 768): the padding is never read.
 bool pf_decode_supported(const PfHipMoeDesc &d) {
     if (!decode_combination(d.type)) return false;
-    if (!pow2_between(d.hidden, 512, 2048) || !pow2_between(d.inter, 256, 2048) ||
-        !pow2_between(d.shared_inter, 256, 2048) || d.down_physical != d.inter || d.shared_inter > 4 * d.inter)
+    if (d.hidden < 512 || d.hidden > 64 * 4 * ROUTER_CHUNKS || d.hidden % 256) return false;
+    if (d.inter < 256 || d.inter > 2048 || d.shared_inter < 256 || d.shared_inter > 2048 || d.inter % 64 || d.shared_inter % 64)
         return false;
+    if (d.shared_inter > 4 * d.inter) return false;
+    if (!row_width_ok(d.type[1], d.hidden) || !row_width_ok(d.type[4], d.hidden) || !row_width_ok(d.type[6], d.shared_inter) ||
+        !row_width_ok(d.type[3], d.down_physical))
+        return false;
+    if (d.down_physical < d.inter || (d.down_physical != d.inter && d.type[3] != PF_Q2_K)) return false;
     if (d.experts > 1024 || d.top_k > 15 || d.top_k * PF_DECODE_MAX_TOKENS > 64 || d.top_k >= d.experts) return false;
     // the down kernel keeps one digit image per slot (and the IQ2_XXS tables) in LDS
     const uint32_t widest = d.inter > d.shared_inter ? d.inter : d.shared_inter;
@@ -791,27 +864,50 @@ bool pf_decode_supported(const PfHipMoeDesc &d) {
     return true;
 }
 
-template <int FG, int FS, int NT, int NPL>
+template <int FG, int FS, int NT, int NPL, int SPL>
 static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks,
                            int shared_blocks, int parts, int chunk, int tile) {
     // more workgroups than compute units: routing once, in a launch of its own, beats every workgroup repeating it
     const bool split = grid.x > 256;
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FG, FS, NT, NPL>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up<FG, FS, NT, NPL, SPL>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
         configured = true;
     }
     if (split)
-        hipLaunchKernelGGL((pf_k_dec_gate_up<FG, FS, NT, NPL>), dim3(1), dim3(1024), lds, stream, a, routed_blocks,
+        hipLaunchKernelGGL((pf_k_dec_gate_up<FG, FS, NT, NPL, SPL>), dim3(1), dim3(1024), lds, stream, a, routed_blocks,
                            shared_blocks, parts, chunk, tile, 1);
-    hipLaunchKernelGGL((pf_k_dec_gate_up<FG, FS, NT, NPL>), grid, dim3(1024), lds, stream, a, routed_blocks, shared_blocks,
+    hipLaunchKernelGGL((pf_k_dec_gate_up<FG, FS, NT, NPL, SPL>), grid, dim3(1024), lds, stream, a, routed_blocks, shared_blocks,
                        parts, chunk, tile, split ? 2 : 0);
 }
 
+template <int FD, int FS, int NT, int SPL, int MAXT>
+static void launch_down_bounded(const PfKernelArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t stream, int row_blocks,
+                                int rows_per_block, int image_pitch) {
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down<FD, FS, NT, SPL, MAXT>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL((pf_k_dec_down<FD, FS, NT, SPL, MAXT>), grid, block, lds, stream, a, row_blocks, rows_per_block,
+                       image_pitch);
+}
+
+template <int FD, int FS, int NT, int SPL>
+static void launch_down(const PfKernelArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t stream, int row_blocks,
+                        int rows_per_block, int image_pitch) {
+    constexpr int TIGHT = (SPL > 1) ? 768 : 1024;
+    if (SPL > 1 && block.x <= 768)
+        launch_down_bounded<FD, FS, NT, SPL, TIGHT>(a, grid, block, lds, stream, row_blocks, rows_per_block, image_pitch);
+    else
+        launch_down_bounded<FD, FS, NT, SPL, 1024>(a, grid, block, lds, stream, row_blocks, rows_per_block, image_pitch);
+}
+
 // FG: format of the routed gate and up tensors, FD: of the routed down tensor, FS: of the shared expert
-template <int FG, int FD, int FS, int NT>
-static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_limit) {
+template <int FG, int FD, int FS, int NT, int SPL2>
+static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int stage_limit) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
     const size_t tab2 = (FG == PF_IQ2_XXS || FS == PF_IQ2_XXS) ? 8192 * 4 : 0;
     const size_t tab3 = (FD == PF_IQ2_XXS || FS == PF_IQ2_XXS) ? 8192 * 4 : 0;
@@ -830,27 +926,30 @@ static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_l
     const int chunk = (E + parts - 1) / parts, npl = (chunk + 63) / 64;
     // compute units left over by the tiles (256 on this GPU) warm the L2 for the down kernel, whose
     // row blocks must then spread evenly over the eight XCDs
-    const int rows_next = 64 / (I / 64), row_blocks_next = (H + rows_next - 1) / rows_next;
+    const int rows_next = down_block_rows(H, I), row_blocks_next = (H + rows_next - 1) / rows_next;
     int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
     if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
     dim3 g2(routed_blocks + shared_blocks + prefetch_blocks);
-    if (npl <= 1) launch_gate_up<FG, FS, NT, 1>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
-    else if (npl <= 2) launch_gate_up<FG, FS, NT, 2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
-    else if (npl <= 4) launch_gate_up<FG, FS, NT, 4>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
-    else launch_gate_up<FG, FS, NT, 8>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024
+    if (npl <= 1) launch_gate_up<FG, FS, NT, 1, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else if (npl <= 2) launch_gate_up<FG, FS, NT, 2, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else if (npl <= 4) launch_gate_up<FG, FS, NT, 4, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    else launch_gate_up<FG, FS, NT, 8, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024
     if (last < 3) return;
     // kernel 3
-    const int rows_per_block = 64 / (I / 64), row_blocks = (H + rows_per_block - 1) / rows_per_block;
+    const int rows_per_block = down_block_rows(H, I), row_blocks = (H + rows_per_block - 1) / rows_per_block;
     const int image_pitch = image_words(I > Is ? I : Is);
     const size_t lds3 = tab3 + (size_t)(K + 1) * image_pitch * 4;
-    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down<FD, FS, NT>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
-        configured = true;
-    }
-    hipLaunchKernelGGL((pf_k_dec_down<FD, FS, NT>), dim3(NT * row_blocks), dim3(64 * (K + 1)), lds3, stream, a, row_blocks,
-                       rows_per_block, image_pitch);
+    if (row_passes(I) > 1 || row_passes(Is) > 1)
+        launch_down<FD, FS, NT, 2>(a, dim3(NT * row_blocks), dim3(64 * (K + 1)), lds3, stream, row_blocks, rows_per_block, image_pitch);
+    else
+        launch_down<FD, FS, NT, 1>(a, dim3(NT * row_blocks), dim3(64 * (K + 1)), lds3, stream, row_blocks, rows_per_block, image_pitch);
+}
+
+// SPL2: passes over a row of `hidden` values in kernel 2 (2 only for widths such as 2560)
+template <int FG, int FD, int FS, int NT>
+static void launch_decode(const PfKernelArgs &a, hipStream_t stream, int stage_limit) {
+    if (row_passes(a.hidden) > 1) launch_decode_passes<FG, FD, FS, NT, 2>(a, stream, stage_limit);
+    else launch_decode_passes<FG, FD, FS, NT, 1>(a, stream, stage_limit);
 }
 
 template <int FG, int FD, int FS>

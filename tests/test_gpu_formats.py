@@ -96,16 +96,20 @@ def test_uniform_layers_of_the_plain_formats(product, oracle, gtype):
 
 # shapes the decode kernels cover, on the two checkpoint profiles, 1..4 tokens per call
 DECODE_PROFILES = [
-    (512, 32, 6, 256, 256, "q2"), (512, 32, 6, 256, 256, "q4"),
-    (1024, 96, 5, 512, 256, "q2"), (1024, 96, 5, 256, 1024, "q4"),     # a shared expert wider than the routed ones
-    (2048, 64, 10, 512, 512, "q2"), (2048, 64, 10, 512, 512, "q4"),    # the measured widths
+    (512, 32, 6, 256, 256, "q2", None), (512, 32, 6, 256, 256, "q4", None),
+    (1024, 96, 5, 512, 256, "q2", None), (1024, 96, 5, 256, 1024, "q4", None),   # a shared expert wider than the routed ones
+    (2048, 64, 10, 512, 512, "q2", None), (2048, 64, 10, 512, 512, "q4", None),  # the measured widths
+    # the checkpoints' own widths (tests/fixtures/qwen4/text/config.json: hidden 2560, intermediate 640, shared 640;
+    # the Q2_K down projection stored 768 wide): rows of 40 and 10 segments, two passes on some lanes
+    (2560, 64, 10, 640, 640, "q2", 768), (2560, 64, 10, 640, 640, "q4", None), (2560, 512, 10, 640, 640, "q2", 768),
+    (1280, 48, 4, 320, 320, "q2", 512), (768, 24, 3, 384, 448, "q4", None),
 ]
 
 
-@pytest.mark.parametrize("h,e,k,i,s,profile", DECODE_PROFILES)
-def test_decode_kernels_on_checkpoint_profiles(product, oracle, h, e, k, i, s, profile):
-    print(f"case decode profile {profile} h={h} e={e} k={k} i={i} s={s}", flush=True)
-    cfg = abi.moe_config(h, e, k, i, s)
+@pytest.mark.parametrize("h,e,k,i,s,profile,down_physical", DECODE_PROFILES)
+def test_decode_kernels_on_checkpoint_profiles(product, oracle, h, e, k, i, s, profile, down_physical):
+    print(f"case decode profile {profile} h={h} e={e} k={k} i={i} s={s} down stored {down_physical or i} wide", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s, down_physical=down_physical)
     weights, x = make_layer_inputs(cfg, profile, 4, seed=h + e + len(profile))
     x[3] = x[2]                                   # two identical tokens share every expert
     want = forward_with(oracle, cfg, weights, x)

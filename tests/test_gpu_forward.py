@@ -34,11 +34,13 @@ def test_small_layers_match_oracle(product, oracle, h, e, k, i, s, gtype, tokens
     assert_parity(*got, *want, label=f"h{h} e{e} type{gtype}")
 
 
-# shapes the specialised decode kernels cover (power-of-two widths), 1..4 tokens per call
+# shapes the specialised decode kernels cover, 1..4 tokens per call; the last ones have rows whose 64-value
+# segments are not a power of two in number (40, 12, 20), so some lanes take two segments
 DECODE = [
     (512, 32, 6, 256, 256, abi.GGUF_Q4_K), (512, 32, 6, 256, 256, abi.GGUF_IQ2_XXS),
     (1024, 96, 5, 512, 256, abi.GGUF_Q4_K), (1024, 96, 5, 256, 1024, abi.GGUF_IQ2_XXS),
     (2048, 64, 10, 1024, 512, abi.GGUF_Q4_K),
+    (2560, 64, 10, 768, 768, abi.GGUF_Q4_K), (2560, 64, 10, 768, 256, abi.GGUF_IQ2_XXS), (1280, 40, 4, 256, 768, abi.GGUF_Q4_K),
 ]
 
 
@@ -50,6 +52,7 @@ def test_decode_kernels_match_oracle_and_general_kernels(product, oracle, h, e, 
     x[3] = x[2]                                   # two identical tokens share every expert
     want = forward_with(oracle, cfg, weights, x)
     with pf.MoeLayer(product, cfg, weights, 4) as layer:
+        assert product.hip.moe_kernel_family(*layer.device_handles(), 1) == 1, "the decode kernels do not cover this layer"
         for tokens in (1, 2, 3, 4):
             print(f"  tokens={tokens}", flush=True)
             _, y, ids, w = layer.forward(x[:tokens])
