@@ -81,6 +81,12 @@ WORKLOADS = {
                           label="checkpoint profile Q2 at the checkpoints' widths, decode batch 1"),
     "q4ckpt_decode": dict(type="q4", tokens=1, steps=5000, warmup=100, dims=(2560, 512, 10, 640, 640, 640),
                           label="checkpoint profile Q4 at the checkpoints' widths, decode batch 1"),
+    "q2ckpt_prefill1024": dict(type="q2", tokens=1024, steps=50, warmup=5, dims=(2560, 512, 10, 640, 640, 768),
+                               label="checkpoint profile Q2 at the checkpoints' widths, 1024-token prefill chunk, N(0,1) "
+                                     "activations, Zipf(1.1) expert popularity"),
+    "q4ckpt_prefill1024": dict(type="q4", tokens=1024, steps=50, warmup=5, dims=(2560, 512, 10, 640, 640, 640),
+                               label="checkpoint profile Q4 at the checkpoints' widths, 1024-token prefill chunk, N(0,1) "
+                                     "activations, Zipf(1.1) expert popularity"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),

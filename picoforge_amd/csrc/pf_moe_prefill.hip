@@ -29,7 +29,8 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 
 // halfs per row of a converted matrix: high parts, low parts, per 256-block the 16 group-sum halfs
 // [even groups: 4 high, 4 low][odd groups: 4 high, 4 low]
-__host__ __device__ constexpr size_t pf_half_row(int cols) { return 2 * (size_t)cols + (size_t)cols / 16; }
+// halfs per row of the fp16 form: high parts, low parts, 16 group-sum parts per (started) 256 columns
+__host__ __device__ constexpr size_t pf_half_row(int cols) { return 2 * (size_t)cols + 16 * (((size_t)cols + 255) / 256); }
 
 // ---- Q4_K tensors in tile order (once, at upload) ---------------------------------------------
 // The grouped product's loader moves one 32-row tile's share of a 256-block per instruction group.
@@ -59,7 +60,7 @@ void pf_launch_q4k_tile(const uint8_t *d_src, uint8_t *d_dst, size_t rows, int b
 }
 
 // ---- rows to scaled fp16 pairs ------------------------------------------------------------------
-// One workgroup per row (cols a multiple of 256).  scale = 2^e with max|row| / scale in
+// One workgroup per row (cols a multiple of 32).  scale = 2^e with max|row| / scale in
 // [0.5, 1) (1 for a zero row).  Thread j converts the eight values 8j..8j+7; four neighbouring
 // threads form one 32-group.
 __global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_t src_pitch, int cols, half_t *dst,
@@ -859,7 +860,9 @@ __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow
                                               float16v &acc0, float16v &acc1) {
     const float16v zero = {0};
     if (FMT == PF_Q2_K) {
-        for (int b = part; b < cols / 256; b += parts) {
+        // a row's last block may be half used (logical width 640 of 768 stored): its second half is skipped,
+        // and the sums of the groups beyond the width are zero
+        for (int b = part; b < (cols + 255) / 256; b += parts) {
             const uint8_t *blk0 = r0.payload + 84 * (size_t)(c0 / 256 + b), *blk1 = r1.payload + 84 * (size_t)(c0 / 256 + b);
             const uint32_t dd0 = *reinterpret_cast<const uint32_t *>(blk0 + 80), dd1 = *reinterpret_cast<const uint32_t *>(blk1 + 80);
             float16v part0 = zero, part1 = zero;
@@ -874,6 +877,7 @@ __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow
             low1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(sl, mv1, low1, 0, 0, 0);
 #pragma unroll
             for (int half = 0; half < 2; half++) {   // eight groups of 16 weights per batch: one 32-byte half of the codes
+                if (256 * b + 128 * half >= cols) break;
                 const uint32_t *q0 = reinterpret_cast<const uint32_t *>(blk0 + 16 + 32 * half + 8 * h);
                 const uint32_t *q1 = reinterpret_cast<const uint32_t *>(blk1 + 16 + 32 * half + 8 * h);
                 // bytes 8h..8h+7 and 16 + 8h..: the groups at l % 32 = 0 and 16, each at four bit planes
@@ -904,7 +908,7 @@ __device__ __forceinline__ void plain_product(const PlainRow &r0, const PlainRow
         }
         return;
     }
-    for (int g0 = 4 * part; g0 < cols / 32; g0 += 4 * parts) {   // batches of four groups of 32 weights (cols is a multiple of 256)
+    for (int g0 = 4 * part; g0 < cols / 32; g0 += 4 * parts) {   // batches of four groups of 32 weights (cols is a multiple of 128)
         const int first = c0 / 32 + g0;            // of the row's groups
         uint2 q0[4][2], q1[4][2];
         float s0[4], s1[4];
@@ -1138,7 +1142,14 @@ bool pf_prefill_supported(const PfHipMoeDesc &d) {
     auto covered = [&](uint32_t t) { return t == g || t == PF_Q8_0 || t == PF_Q2_K || t == PF_MXFP4; };
     if ((g != PF_Q4_K && g != PF_IQ2_XXS) || d.type[2] != g || !covered(d.type[3])) return false;
     if (d.type[5] != d.type[4] || !covered(d.type[4]) || !covered(d.type[6])) return false;
-    if (d.hidden % 256 || d.inter % 256 || d.shared_inter % 256 || d.down_physical != d.inter) return false;
+    // widths: whole 256-blocks where the ring kernel reads them; where the plain kernel takes a down projection, whole
+    // 128-column halves (the checkpoints' 640), and only Q2_K may be stored wider than its logical width
+    auto width_ok = [&](uint32_t type, uint32_t k) { return k % (type == g ? 256u : 128u) == 0; };
+    if (d.hidden % 256 || d.inter % 32 || d.shared_inter % 32 || !width_ok(d.type[3], d.inter) || !width_ok(d.type[6], d.shared_inter))
+        return false;
+    if (d.down_physical < d.inter || (d.down_physical != d.inter && d.type[3] != PF_Q2_K) ||
+        (d.type[3] == PF_Q2_K && d.down_physical % 256))
+        return false;
     if (d.top_k > 64 || d.top_k >= d.experts || d.experts >= 65535) return false;
     return true;
 }

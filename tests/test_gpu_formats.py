@@ -156,6 +156,29 @@ def test_prefill_kernels_on_checkpoint_profiles(product, oracle, h, e, k, i, s, 
         assert_parity(y, ids, w, *want, label="general kernels on the same layer")
 
 
+# chunks at widths that are not whole 256-blocks: the checkpoints' own (hidden 2560, intermediate and shared 640, the
+# Q2_K down projection stored 768 wide) and two smaller ones; (h, e, k, i, s, tokens)
+PREFILL_ODD_WIDTHS = [(2560, 32, 4, 640, 640, 70), (512, 16, 3, 384, 128, 40), (768, 24, 5, 128, 896, 300)]
+
+
+@pytest.mark.parametrize("profile", ["q2", "q4"])
+@pytest.mark.parametrize("h,e,k,i,s,tokens", PREFILL_ODD_WIDTHS)
+def test_prefill_kernels_at_checkpoint_widths(product, oracle, h, e, k, i, s, tokens, profile):
+    print(f"case prefill profile {profile} h={h} e={e} k={k} i={i} s={s} T={tokens}", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s, down_physical=(i + 255) // 256 * 256 if profile == "q2" else i)
+    weights, x = make_layer_inputs(cfg, profile, tokens, seed=h + i + tokens)
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, tokens) as layer:
+        moe, work = layer.device_handles()
+        assert product.hip.moe_kernel_family(moe, work, tokens) == 2, "the prefill kernels do not cover this layer"
+        _, y, ids, w = layer.forward(x)
+        worst = assert_parity(y, ids, w, *want, label=f"prefill {profile} T={tokens}")
+        print(f"  max abs err {worst:.2e}", flush=True)
+        layer.force_general()
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y, ids, w, *want, label="general kernels on the same layer")
+
+
 @pytest.mark.parametrize("profile", ["q2", "q4"])
 def test_full_size_profile_layers(product, oracle, profile):
     """The measured shape (hidden 2048, 512 experts, top-10, intermediate 512, shared 512) in the checkpoint
