@@ -566,6 +566,7 @@ __device__ __forceinline__ void gate_up_tile(const PfKernelArgs &a, const int *i
         float dot[2];
 #pragma unroll
         for (int st = 0; st < 2; st++) dot[st] = st < steps ? wseg_dot<FMT>(w[st][0], x, seg, tables) : 0.0f;
+        if (SPL > 1) __builtin_amdgcn_sched_barrier(0);   // the second segment's digits reuse the first's registers
         if (SPL > 1 && second) {
             xseg_load(x, images + t * W, H, seg + LPR);
 #pragma unroll
@@ -717,10 +718,12 @@ __device__ __forceinline__ void down_rows(const PfKernelArgs &a, float *partial_
         }
         if (st > 0) xseg_load(x, image, I, seg);
         float dot = wseg_dot<FMT>(w[0], x, seg, tables);
+        __builtin_amdgcn_sched_barrier(0);   // the second segment's digits reuse the first's registers: no hoisting above
         if (second) {
             xseg_load(x, image, I, seg + LPR);
             dot += wseg_dot<FMT>(w[SPL - 1], x, seg + LPR, tables);
         }
+        __builtin_amdgcn_sched_barrier(0);
         const float v = span_sum(dot, LPR);
         const int row = st * rows + r;
         if (seg == 0 && row < rows_per_block) partial_row[row] = v;
