@@ -54,17 +54,20 @@ def test_a_layer_outlives_its_file(tmp_path, product, oracle):
     assert_parity(y, ids, w, y_ref, ids_ref, w_ref, "after close")
 
 
-def test_a_layer_of_benchmark_size_from_a_file(tmp_path, product, oracle):
-    """Hidden 2048, 512 experts, top-10, intermediate 512, shared 512, 460 MB of tensors: the
-    decode kernels at 1 and 4 tokens and the matrix-core kernels at 48 tokens must be the ones that run."""
-    print("case benchmark-size layer from a file, profile q2", flush=True)
-    dims = dict(hidden=2048, experts=512, top_k=10, inter=512, shared=512, streams=4)
+@pytest.mark.parametrize("dims,physical", [
+    (dict(hidden=2048, experts=512, top_k=10, inter=512, shared=512, streams=4), 512),     # the benchmarks' layer, 460 MB
+    (dict(hidden=2560, experts=128, top_k=10, inter=640, shared=640, streams=4), 768),     # the checkpoints' widths
+], ids=["benchmark-size", "checkpoint-widths"])
+def test_a_full_width_layer_from_a_file(tmp_path, product, oracle, dims, physical):
+    """The decode kernels at 1 and 4 tokens and the matrix-core kernels at 48 tokens must be the ones that run
+    on a layer that came out of a file, at the benchmarks' widths and at the checkpoints' own (Q2_K down padded)."""
+    print(f"case layer from a file, profile q2, hidden {dims['hidden']}", flush=True)
     mf = gf.ModelFile(profile="q2", kinds=("gdn",), mtp=0, dims=dims, moe_only=True, seed=9, std=0.02)
     mf.write(tmp_path / "layer.gguf")
     with GgufFile(product, mf.path) as f:
-        assert f.moe_model().moe.down_physical == 512 and f.moe_weights(0).nbytes > 400e6
+        assert f.moe_model().moe.down_physical == physical and f.moe_weights(0).nbytes > 200e6
         for count, family in ((1, 1), (4, 1), (48, 2)):
-            x = tokens_for(2048, count, 40 + count)
+            x = tokens_for(dims["hidden"], count, 40 + count)
             with f.moe_layer(0, count) as mine, f.moe_layer(0, count, api=oracle) as cpu:
                 moe, work = mine.device_handles()
                 assert product.hip.moe_kernel_family(moe, work, count) == family
