@@ -65,7 +65,7 @@ def test_a_full_width_layer_from_a_file(tmp_path, product, oracle, dims, physica
     mf = gf.ModelFile(profile="q2", kinds=("gdn",), mtp=0, dims=dims, moe_only=True, seed=9, std=0.02)
     mf.write(tmp_path / "layer.gguf")
     with GgufFile(product, mf.path) as f:
-        assert f.moe_model().moe.down_physical == physical and f.moe_weights(0).nbytes > 200e6
+        assert f.moe_model().moe.down_physical == physical and f.moe_weights(0).nbytes > 150e6
         for count, family in ((1, 1), (4, 1), (48, 2)):
             x = tokens_for(dims["hidden"], count, 40 + count)
             with f.moe_layer(0, count) as mine, f.moe_layer(0, count, api=oracle) as cpu:
