@@ -144,6 +144,8 @@ CHAIN = [
     (256, 16, 4, 256, 256, abi.GGUF_IQ2_XXS, 33, 5),
     (512, 32, 6, 256, 256, "q2", 3, 4),                  # checkpoint profiles on the decode kernels
     (512, 32, 6, 256, 256, "q4", 9, 4),                  # ... a chunk, four tokens per launch
+    (2560, 48, 10, 640, 640, "q2", 1, 4),                # the checkpoints' widths (Q2_K down stored 768 wide): decode
+    (2560, 48, 10, 640, 640, "q4", 40, 4),               # ... and a chunk
 ]
 
 
@@ -161,7 +163,7 @@ def chain_inputs(cfg, tokens, streams, seed):
 @pytest.mark.parametrize("h,e,k,i,s,gtype,tokens,streams", CHAIN)
 def test_chained_forward_matches_oracle_stage_by_stage(product, oracle, h, e, k, i, s, gtype, tokens, streams):
     print(f"case chain h={h} e={e} k={k} type={gtype} T={tokens} streams={streams}", flush=True)
-    cfg = abi.moe_config(h, e, k, i, s)
+    cfg = abi.moe_config(h, e, k, i, s, down_physical=(i + 255) // 256 * 256 if gtype == "q2" else i)
     weights, _ = make_layer_inputs(cfg, gtype, 1, seed=3 * h + tokens, std=0.02 if gtype != abi.GGUF_F32 else 0.2)
     normed, logits, residual, inject = chain_inputs(cfg, tokens, streams, 900 + h + tokens)
     # the device's own mixed rows, so that every later stage is compared on identical inputs
