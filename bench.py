@@ -16,7 +16,9 @@ iq2xxs_prefill1024 (1024-token chunks, N(0,1) activations, Zipf(1.1) expert
 popularity), q4k_stack48 (48 resident layers, decode and 2048-token chunks), and
 q2profile_decode / q4profile_decode / q2profile_prefill1024 / q4profile_prefill1024 (the
 format mixes of real checkpoints: IQ2_XXS gate/up + Q2_K down, Q4_K gate/up + MXFP4 down,
-Q8_0 shared expert), and
+Q8_0 shared expert), q2ckpt_decode / q4ckpt_decode / q2ckpt_prefill1024 / q4ckpt_prefill1024 (those
+mixes at the checkpoints' own widths: hidden 2560, intermediate and shared 640, the Q2_K down
+projection stored 768 wide), and
 iq2xxs_decode_hc / q4k_decode_hc / q4k_prefill1024_hc: the same layer between its two
 hyper-connection steps (gated read of 4 residual streams before, injection into them
 after), with the injection folded into the block's last kernel and as a kernel of its own.

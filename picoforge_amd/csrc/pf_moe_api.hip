@@ -981,7 +981,8 @@ extern "C" int pf_hip_hc_time_step(int which, float *d_cube, const float *d_logi
 
 extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
                                         float *d_y, size_t tokens, size_t iters, float *elapsed_ms) {
-    if (!moe || !work || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
+    if (!moe || !work || work->moe != moe || tokens > work->cap || !d_x || !d_y || !n_inputs || !elapsed_ms)
+        return PF_HIP_E_ARGUMENT;
     return time_graph_replay(&moe, &work, 1, d_x, n_inputs, d_y, tokens, iters, 0, elapsed_ms);
 }
 
@@ -1002,7 +1003,8 @@ extern "C" int pf_hip_stack_time_forwards(const PfHipMoe *const *moes, PfHipWork
 // launches (the third being the routing pair); unused entries are zero.
 extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
                                          float *d_y, size_t tokens, size_t iters, float stage_ms[4]) {
-    if (!moe || !work || !d_x || !d_y || !n_inputs || !stage_ms || !iters) return PF_HIP_E_ARGUMENT;
+    if (!moe || !work || work->moe != moe || tokens > work->cap || !d_x || !d_y || !n_inputs || !stage_ms || !iters)
+        return PF_HIP_E_ARGUMENT;
     const int stages = pf_hip_moe_kernel_family(moe, work, tokens) == 1 ? 3 : 4;
     float previous = 0.0f;
     for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
