@@ -96,10 +96,10 @@ WORKLOADS = {
 # HBM bytes per launch of each workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE scaled by the same counters on a plain 256 MiB copy (profiles/*.txt hold the runs).
 # A counter result cannot be read live; None where no such run exists for the workload.
-MEASURED_TRAFFIC = {"iq2xxs_decode": 9907760, "q4k_decode": 19881668, "q4k_verify4": None,
-                    "q4k_prefill1024": 816800329, "iq2xxs_prefill1024": 450023382,
+MEASURED_TRAFFIC = {"iq2xxs_decode": 9892423, "q4k_decode": 19875557, "q4k_verify4": None,
+                    "q4k_prefill1024": 817391959, "iq2xxs_prefill1024": 460067641,
                     # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
-                    "q4k_prefill1024_hc": 75633614, "iq2xxs_decode_hc": 117059, "q4k_decode_hc": None,
+                    "q4k_prefill1024_hc": 75633928, "iq2xxs_decode_hc": 117050, "q4k_decode_hc": None,
                     "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None, "q2ckpt_decode": None, "q4ckpt_decode": None,
                     "q4profile_prefill1024": None}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
@@ -340,6 +340,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=None, help="tokens timed on the CPU path (default ~15 s of work)")
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--layers", type=int, default=48, help="layers of the q4k_stack48 workload")
+    ap.add_argument("--skip-stages", action="store_true",
+                    help="leave out the per-kernel timing by stage-limited graph replays (kernel_us is then meaningless): "
+                         "for runs under a profiler, which records the kernels' durations itself")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="also launch a plain copy kernel of this many MiB three times (byte-counter calibration)")
     args = ap.parse_args()
@@ -409,7 +412,8 @@ def main():
     # stage's duration is the difference between consecutive replays (it includes the dispatch
     # gap before it, as a profiler's start-to-end time of a dependent kernel does).
     stage = (C.c_float * 4)()
-    hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(steps, 2000), stage), "stages")
+    if not args.skip_stages:
+        hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(steps, 2000), stage), "stages")
     family = hip.moe_kernel_family(moe, work, tokens)
     names = {0: GENERAL_STAGES, 1: DECODE_STAGES, 2: PREFILL_STAGES}[family]
     stage_us = [max(float(stage[j]) * 1e3, 1e-3) for j in range(len(names))]
