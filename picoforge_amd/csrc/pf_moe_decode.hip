@@ -30,6 +30,12 @@
 #else
 #define STAMP(i) do {} while (0)
 #endif
+// The unit is compiled four times, once per format combination (PF_DECODE_PART 0..3, see the dispatch
+// at the end), so that the combinations' kernels build in parallel; part 0 also holds everything that
+// does not depend on the combination.
+#ifndef PF_DECODE_PART
+#define PF_DECODE_PART 0
+#endif
 #define SEG_STRIDE 20   // dwords per 64-value segment of a digit plane (16 used): spreads LDS banks
 
 // ---- digit images --------------------------------------------------------------------
@@ -786,6 +792,7 @@ __global__ void __launch_bounds__(MAXT) pf_k_dec_down(PfKernelArgs a, int row_bl
     }
 }
 
+#if PF_DECODE_PART == 0
 // ---- IQ2_XXS upload split -------------------------------------------------------------------------
 __global__ void pf_k_iq2_split(const uint8_t *gguf, uint8_t *payload, uint16_t *scales, size_t blocks) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;   // one 16-bit word of a block per thread
@@ -826,6 +833,8 @@ void pf_launch_block_split(const uint8_t *d_gguf, uint8_t *d_payload, uint8_t *d
 }
 
 // ---- dispatch ----------------------------------------------------------------------------------------
+#endif
+
 static bool pow2_between(uint32_t v, uint32_t lo, uint32_t hi) { return v >= lo && v <= hi && (v & (v - 1)) == 0; }
 
 // The format combinations with decode kernels: one format throughout (Q4_K or IQ2_XXS), and the two
@@ -847,6 +856,7 @@ static bool row_width_ok(uint32_t type, uint32_t k) {
     return k && k % (big ? 256 : 64) == 0;
 }
 
+#if PF_DECODE_PART == 0
 // Widths: hidden 512..2560 in whole 256-blocks (2560 is the checkpoints' width), intermediate widths
 // 256..2048 in whole 64-value segments (640 in the checkpoints); the routed down projection may be
 // stored wider than its logical width only as Q2_K (640 padded to 768): the padding is never read.
@@ -867,6 +877,8 @@ bool pf_decode_supported(const PfHipMoeDesc &d) {
     return true;
 }
 
+#endif
+
 template <int FG, int FS, int NT, int NPL, int SPL>
 static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks,
                            int shared_blocks, int parts, int chunk, int tile) {
@@ -884,6 +896,19 @@ static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStre
     hipLaunchKernelGGL((pf_k_dec_gate_up<FG, FS, NT, NPL, SPL>), grid, dim3(1024), lds, stream, a, routed_blocks, shared_blocks,
                        parts, chunk, tile, split ? 2 : 0);
 }
+
+void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
+#if PF_DECODE_PART == 0
+void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream) {
+    const dim3 grid(router_blocks + 1), block(256);
+    switch (tokens) {
+    case 1: hipLaunchKernelGGL((pf_k_dec_router<1>), grid, block, 0, stream, a, router_blocks); break;
+    case 2: hipLaunchKernelGGL((pf_k_dec_router<2>), grid, block, 0, stream, a, router_blocks); break;
+    case 3: hipLaunchKernelGGL((pf_k_dec_router<3>), grid, block, 0, stream, a, router_blocks); break;
+    default: hipLaunchKernelGGL((pf_k_dec_router<4>), grid, block, 0, stream, a, router_blocks); break;
+    }
+}
+#endif
 
 template <int FD, int FS, int NT, int SPL, int MAXT>
 static void launch_down_bounded(const PfKernelArgs &a, dim3 grid, dim3 block, size_t lds, hipStream_t stream, int row_blocks,
@@ -916,7 +941,7 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     const size_t tab3 = (FD == PF_IQ2_XXS || FS == PF_IQ2_XXS) ? 8192 * 4 : 0;
     // kernel 1 (stage_limit, profiling: launch only the first so many kernels; 0 = all)
     const int router_blocks = (E + 3) / 4, last = stage_limit ? stage_limit : 3;
-    hipLaunchKernelGGL((pf_k_dec_router<NT>), dim3(router_blocks + 1), dim3(256), 0, stream, a, router_blocks);
+    pf_launch_dec_router(a, NT, router_blocks, stream);
     if (last < 2) return;
     // kernel 2: the candidate stage uses up to 8 of waves 0..11 per token
     // 32 units per workgroup: every workgroup repeats the routing, and one workgroup per compute
@@ -965,12 +990,35 @@ static void launch_decode_tokens(const PfKernelArgs &a, int tokens, hipStream_t 
     }
 }
 
+void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_decode_iq2(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+
+#if PF_DECODE_PART == 0
+void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
+}
+
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     switch (decode_combination(a.type)) {
-    case 1: launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit); break;
-    case 2: launch_decode_tokens<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit); break;
-    case 3: launch_decode_tokens<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit); break;
-    case 4: launch_decode_tokens<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit); break;
+    case 1: pf_launch_decode_q4k(a, tokens, stream, stage_limit); break;
+    case 2: pf_launch_decode_iq2(a, tokens, stream, stage_limit); break;
+    case 3: pf_launch_decode_q2profile(a, tokens, stream, stage_limit); break;
+    case 4: pf_launch_decode_q4profile(a, tokens, stream, stage_limit); break;
     default: break;   // pf_decode_supported keeps other combinations away
     }
 }
+#elif PF_DECODE_PART == 1
+void pf_launch_decode_iq2(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    launch_decode_tokens<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit);
+}
+#elif PF_DECODE_PART == 2
+void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    launch_decode_tokens<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit);
+}
+#else
+void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    launch_decode_tokens<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit);
+}
+#endif
