@@ -832,11 +832,9 @@ void pf_launch_block_split(const uint8_t *d_gguf, uint8_t *d_payload, uint8_t *d
                        d_payload, d_scales, blocks, block_bytes, header_bytes);
 }
 
-// ---- dispatch ----------------------------------------------------------------------------------------
 #endif
 
-static bool pow2_between(uint32_t v, uint32_t lo, uint32_t hi) { return v >= lo && v <= hi && (v & (v - 1)) == 0; }
-
+// ---- dispatch ----------------------------------------------------------------------------------------
 // The format combinations with decode kernels: one format throughout (Q4_K or IQ2_XXS), and the two
 // profiles of real checkpoints (src/qwen4_config.c:197-216, src/qwen4_weights.c:91-99): IQ2_XXS gate/up
 // with Q2_K down, Q4_K gate/up with MXFP4 down, the shared expert in Q8_0.
