@@ -21,7 +21,8 @@ mixes at the checkpoints' own widths: hidden 2560, intermediate and shared 640, 
 projection stored 768 wide), and
 iq2xxs_decode_hc / q4k_decode_hc / q4k_prefill1024_hc: the same layer between its two
 hyper-connection steps (gated read of 4 residual streams before, injection into them
-after), with the injection folded into the block's last kernel and as a kernel of its own.
+after), with the injection folded into the block's last kernel and as a kernel of its own
+(q2ckpt_decode_hc / q2ckpt_prefill1024_hc: the same at the checkpoints' widths).
 
 Prints one JSON line.  `value` is microseconds per layer per token (lower is
 better).  `roofline` is for the kernel that moves the most bytes, timed live
@@ -89,6 +90,12 @@ WORKLOADS = {
     "q4ckpt_prefill1024": dict(type="q4", tokens=1024, steps=50, warmup=5, dims=(2560, 512, 10, 640, 640, 640),
                                label="checkpoint profile Q4 at the checkpoints' widths, 1024-token prefill chunk, N(0,1) "
                                      "activations, Zipf(1.1) expert popularity"),
+    "q2ckpt_decode_hc": dict(type="q2", tokens=1, steps=5000, warmup=100, hc=4, dims=(2560, 512, 10, 640, 640, 768),
+                             label="checkpoint profile Q2 at the checkpoints' widths, decode batch 1, between the HC read and "
+                                   "add of 4 residual streams"),
+    "q2ckpt_prefill1024_hc": dict(type="q2", tokens=1024, steps=50, warmup=5, hc=4, dims=(2560, 512, 10, 640, 640, 768),
+                                  label="checkpoint profile Q2 at the checkpoints' widths, 1024-token prefill chunk, between "
+                                        "the HC read and add of 4 residual streams, Zipf(1.1) expert popularity"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),
@@ -100,7 +107,7 @@ MEASURED_TRAFFIC = {"iq2xxs_decode": 9892423, "q4k_decode": 19875557, "q4k_verif
                     "q4k_prefill1024": 817391959, "iq2xxs_prefill1024": 460067641,
                     # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
                     "q4k_prefill1024_hc": 75633928, "iq2xxs_decode_hc": 117050, "q4k_decode_hc": None,
-                    "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None, "q2ckpt_decode": None, "q4ckpt_decode": None,
+                    "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None, "q2ckpt_decode": None, "q4ckpt_decode": None, "q2ckpt_decode_hc": None, "q2ckpt_prefill1024_hc": None,
                     "q4profile_prefill1024": None}
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
@@ -300,7 +307,8 @@ def run_hc(args, api, hip, cfg, wl, steps, warmup):
         "unit": "us/layer/token", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if tokens <= 4 else "f16 products, f32 accumulation", "data": "synthetic",
-        "config": {"workload": f"one MoE layer, hidden 2048, 512 experts, top-10, intermediate 512, shared 512; "
+        "config": {"workload": f"one MoE layer, hidden {cfg.hidden_size}, {cfg.experts} experts, top-{cfg.top_k}, "
+                               f"intermediate {cfg.intermediate}, shared {cfg.shared_intermediate}; "
                                f"{wl['label']}; {n_inputs} seeded inputs",
                    "tokens_per_step": tokens, "streams": streams,
                    "expert_format": FORMAT_LABEL[wl["type"]]},
