@@ -46,6 +46,7 @@ sys.path.insert(0, str(ROOT))
 
 import picoforge_amd as pf  # noqa: E402
 from picoforge_amd import abi, workloads  # noqa: E402
+from oracle.load import load_oracle, load_reference  # noqa: E402  (the cpu_baseline leg and its parity sample only)
 
 FORMAT_LABEL = {12: "Q4_K", 16: "IQ2_XXS", "q2": "IQ2_XXS gate/up, Q2_K down, Q8_0 shared expert",
                 "q4": "Q4_K gate/up, MXFP4 down, Q8_0 shared expert"}
@@ -166,8 +167,8 @@ def run_stack(args, api, hip, cfg, steps, warmup):
         hip.free(d_pre)
     errors = sum(int(hip.from_device(hip.work_error_word(w), (1,), np.uint32)[0]) for w in works)
     # parity and the CPU cost per layer-token on layer 0; the stack's CPU time is that times the layers
-    ref = pf.load_reference()
-    cpu_api, kind = (ref, "reference") if ref is not None else (pf.load_oracle(), "port")
+    ref = load_reference()
+    cpu_api, kind = (ref, "reference") if ref is not None else (load_oracle(), "port")
     n = args.cpu_sample or 16
     xs = dec[:n].copy()
     with pf.MoeLayer(cpu_api, cfg, sample, n) as cpu:
@@ -272,8 +273,8 @@ def run_hc(args, api, hip, cfg, wl, steps, warmup):
 
     # parity on a bounded sample, stage by stage on identical inputs: CPU read against the device's mixed rows,
     # CPU block on those rows, CPU add of its output; the device's chained call against that residual
-    ref = pf.load_reference()
-    cpu_api, kind = (ref, "reference") if ref is not None else (pf.load_oracle(), "port")
+    ref = load_reference()
+    cpu_api, kind = (ref, "reference") if ref is not None else (load_oracle(), "port")
     sample = min(tokens, args.cpu_sample or (24 if wl["type"] == abi.GGUF_IQ2_XXS else 40))
     steps_cpu = 1 if tokens > 1 else min(sample, n_inputs)
     rows = sample if tokens > 1 else 1
@@ -460,8 +461,8 @@ def main():
     achieved = stage_bytes[dom] / (stage_us[dom] * 1e-6) / 1e9
 
     # CPU baseline and parity on a bounded sample of the same inputs
-    ref = pf.load_reference()
-    cpu_api, kind = (ref, "reference") if ref is not None else (pf.load_oracle(), "port")
+    ref = load_reference()
+    cpu_api, kind = (ref, "reference") if ref is not None else (load_oracle(), "port")
     per_token_guess = 0.55 if wl["type"] in (abi.GGUF_IQ2_XXS, "q2") else 0.32
     if prefill:
         sample_tokens = min(tokens, args.cpu_sample or 48)

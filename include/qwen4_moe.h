@@ -105,6 +105,12 @@ void qw4_moe_observe(Qwen4MoeWork *work, QW4MoeObserver observer, void *ctx);
  * resident in HBM and enqueue forwards on their own stream.  Owned by the handles
  * they come from. */
 struct PfHipMoe *pf_moe_device_layer(const Qwen4Moe *moe);
+/* Extension: qwen4_moe_create copies the weight bytes to device memory, but like the reference
+ * (src/qwen4_moe.h:12, src/qwen4_moe.c:403-410) qwen4_moe_forward refuses views that overlap the
+ * host bytes the layer was created from, so those must stay allocated until destroy.  A caller
+ * that releases them earlier calls this first; forward then skips that comparison for the layer
+ * (pf_gguf_moe_create does so itself: its layers may outlive the file mapping). */
+void pf_moe_forget_host_weights(Qwen4Moe *moe);
 struct PfHipWork *pf_moe_device_work(Qwen4MoeWork *work);
 
 #ifdef __cplusplus

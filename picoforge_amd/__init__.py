@@ -5,6 +5,6 @@ host + hand-written HIP kernels for gfx950).  Nothing here computes on the CPU:
 if the library is missing, loading it raises.
 """
 from . import abi  # noqa: F401
-from .binding import LibraryMissing, Synth, load_oracle, load_product, load_reference  # noqa: F401
+from .binding import LibraryMissing, Synth, load_product  # noqa: F401
 from .layer import LayerWeights, MoeError, MoeLayer, rms_normalise  # noqa: F401
 from .gguf import GgufError, GgufFile  # noqa: F401

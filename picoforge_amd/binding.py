@@ -6,9 +6,8 @@ the HIP shim of include/pf_moe_hip.h.  It raises if the library is missing; no
 part of this package computes anything on the CPU in its place.
 
 `MoeApi` types the eight entry points (and the two tested private helpers) of a
-library that follows the reference's boundary.  The same class wraps the CPU
-oracle (functions prefixed orc_) and a build of the reference's own C path, so
-tests drive all three through identical code.
+library that follows the reference's boundary; the prefixes are parameters so
+that test code can type other libraries with the same boundary the same way.
 """
 import ctypes as C
 from pathlib import Path
@@ -62,6 +61,8 @@ class MoeApi:
         self.group_pairs = bind(private_prefix + "group_pairs", C.c_int, P(abi.Qwen4MoeConfig), abi.Qwen4U32Mut,
                                 abi.QW4MoeGrouping, P(E))
         self.observe = bind(private_prefix + "observe", None, vp, abi.OBSERVER, vp)
+        if hasattr(lib, "pf_moe_forget_host_weights"):
+            self.forget_host_weights = bind("pf_moe_forget_host_weights", None, vp)
         if hasattr(lib, "pf_moe_device_layer"):
             self.device_layer = bind("pf_moe_device_layer", vp, vp)
             self.device_work = bind("pf_moe_device_work", vp, vp)
@@ -93,25 +94,6 @@ def load_product():
     lib = _open(PRODUCT_LIB)
     api = MoeApi(lib)
     api.hip = HipShim(lib)
-    api.hc = HcApi(lib)
-    return api
-
-
-def load_oracle():
-    """CPU oracle: test infrastructure (oracle/), never part of the product path."""
-    lib = _open(REPO_DIR / "oracle" / "liborc.so")
-    api = MoeApi(lib, moe_prefix="orc_moe_", private_prefix="orc_moe_", packed_prefix="orc_packed_")
-    api.hc = HcApi(lib, prefix="orc_hc_")
-    return api
-
-
-def load_reference():
-    """The reference's own C path, if oracle/_ref was built where the reference tree is mounted."""
-    path = REPO_DIR / "oracle" / "_ref" / "libqwen4_ref.so"
-    if not path.exists():
-        return None
-    lib = _open(path)
-    api = MoeApi(lib)
     api.hc = HcApi(lib)
     return api
 

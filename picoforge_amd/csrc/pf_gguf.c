@@ -504,5 +504,8 @@ Qwen4Status pf_gguf_moe_create(const PfGguf *g, const PfGgufMoeModel *model, uin
     Qwen4Status s = pf_gguf_moe_weights(g, model, layer, &w, err);
     if (s != QW4_OK) return s;
     if ((s = pf_gguf_moe_layer_config(model, layer, &c, err)) != QW4_OK) return s;
-    return qwen4_moe_create(&c, &w, out, err);
+    s = qwen4_moe_create(&c, &w, out, err);
+    /* the layer may outlive the mapping: its views are not compared with the file's addresses later */
+    if (s == QW4_OK) pf_moe_forget_host_weights(*out);
+    return s;
 }

@@ -24,6 +24,7 @@ struct Qwen4Moe {
     bool alive;
     PfHipMoe *device;
     PfHipMoeDesc desc;
+    bool host_spans;   /* the caller still holds the weight bytes at w[].span (the reference's contract) */
 };
 
 struct Qwen4MoeWork {
@@ -99,6 +100,7 @@ Qwen4Status qwen4_moe_create(const Qwen4MoeConfig *c, const Qwen4MoeWeights *wei
     if (rc) { free(m); return pf_device_status(rc, err, "qwen4_moe"); }
     m->refs = 1;
     m->alive = true;
+    m->host_spans = true;
     *out = m;
     return moe_status(err, QW4_OK, "");
 }
@@ -156,6 +158,14 @@ Qwen4Status qwen4_moe_work_reset(Qwen4MoeWork *w, Qwen4Error *err) {
 
 void qwen4_moe_work_destroy(Qwen4MoeWork *w) {
     if (w && !w->busy) { pf_hip_work_destroy(w->device); moe_unref(w->owner); free(w); }
+}
+
+/* The weights live in device memory from create on.  A caller that frees or unmaps its host bytes
+ * before destroy (which the reference's borrowing contract, src/qwen4_moe.h:12, does not allow) says
+ * so here: forward then no longer compares its views with the addresses the bytes once had, which
+ * another allocation may own by then. */
+void pf_moe_forget_host_weights(Qwen4Moe *m) {
+    if (m) m->host_spans = false;
 }
 
 PfHipMoe *pf_moe_device_layer(const Qwen4Moe *m) { return m ? m->device : NULL; }
@@ -318,7 +328,7 @@ Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen
         nr = 4;
     }
     TRY(all_disjoint(r, nr, err));
-    for (size_t a = 0; a < 8; a++) {
+    for (size_t a = 0; a < 8 && m->host_spans; a++) {
         const Range wr = {(uintptr_t)m->w[a].span.data, (uintptr_t)m->w[a].span.data + m->w[a].layout.tensor_bytes};
         for (size_t b = 0; b < nr; b++) {
             const Range two[2] = {r[b], wr};

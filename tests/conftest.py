@@ -14,15 +14,15 @@ def pytest_configure(config):
 
 @pytest.fixture(scope="session")
 def oracle():
-    import picoforge_amd as pf
-    return pf.load_oracle()
+    from oracle.load import load_oracle
+    return load_oracle()
 
 
 @pytest.fixture(scope="session")
 def reference():
     """The reference's own C path (oracle/_ref), or None where it was not built."""
-    import picoforge_amd as pf
-    return pf.load_reference()
+    from oracle.load import load_reference
+    return load_reference()
 
 
 @pytest.fixture(scope="session")

@@ -52,7 +52,8 @@ def write_hc(ref):
 
 
 def main():
-    ref = pf.load_reference()
+    from oracle.load import load_reference
+    ref = load_reference()
     if ref is None:
         sys.exit("oracle/_ref/libqwen4_ref.so missing: run make -C oracle where the reference is mounted")
     write_hc(ref)

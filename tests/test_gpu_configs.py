@@ -1,0 +1,99 @@
+"""GPU parity on the benchmark configurations themselves, at their full shape
+(hidden 2048, 512 experts, top-10, intermediate 512, shared 512): the 1024-token Q4_K chunk under a
+Zipf(1.1) router, the 4-token verify batches with about half of the experts shared between
+neighbours, and a stack of independent layers."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import picoforge_amd as pf
+from picoforge_amd import abi, workloads
+
+from helpers import ATOL, RTOL, assert_parity, call_matmul, call_route
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_routes(oracle, cfg, weights, x):
+    """Router logits in the reference's serial order (the F32 packed product) and its routing, for every token."""
+    st, logits = call_matmul(oracle, weights.raw[0], abi.GGUF_F32, cfg.hidden_size, cfg.experts, 1, 0, x)
+    assert st == abi.QW4_OK
+    st, _, ids, w, _ = call_route(oracle, cfg, logits)
+    assert st == abi.QW4_OK
+    return ids, w
+
+
+def test_q4k_zipf_chunk_of_1024_tokens_at_full_shape(product, oracle):
+    cfg = workloads.measured_config()
+    weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=1)
+    workloads.zipf_router(weights, seed=1, temperature=0.18)
+    x = workloads.prefill_chunk(weights, 1024, seed=1)
+    print("zipf chunk: device forward", flush=True)
+    with pf.MoeLayer(product, cfg, weights, 1024) as layer:
+        assert product.hip.moe_kernel_family(*layer.device_handles(), 1024) == 2, "the prefill kernels do not cover this layer"
+        _, y, ids, w = layer.forward(x)
+        reroutes = layer.serial_order_reroutes()
+    print("zipf chunk: oracle routes of all 1024 tokens", flush=True)
+    ids0, w0 = oracle_routes(oracle, cfg, weights, x)
+    np.testing.assert_array_equal(ids, ids0, err_msg="expert ids of the 1024-token chunk")
+    np.testing.assert_allclose(w, w0, atol=2e-6, rtol=2e-5)
+    load = np.bincount(ids0.reshape(-1), minlength=cfg.experts)
+    assert load.max() > 96 and (load == 0).sum() < 64, (load.max(), (load == 0).sum())   # several 32-row tiles; most experts active
+    # rows of the busiest experts (first, middle and last of their row lists) and of the least loaded ones
+    picked = []
+    for e in np.argsort(-load)[:6]:
+        rows = np.nonzero((ids0 == e).any(axis=1))[0]
+        picked += [rows[0], rows[len(rows) // 2], rows[-1]]
+    for e in np.argsort(load)[:10]:                       # the least loaded experts (a few rows each)
+        if load[e]:
+            picked.append(np.nonzero((ids0 == e).any(axis=1))[0][0])
+    picked += [0, 511, 1023]
+    picked = np.unique(np.array(picked))
+    assert len(picked) >= 24
+    print(f"zipf chunk: oracle forward of {len(picked)} rows; max load {load.max()}, idle experts {(load == 0).sum()}, "
+          f"serial-order reroutes {reroutes}", flush=True)
+    with pf.MoeLayer(oracle, cfg, weights, len(picked)) as cpu:
+        _, y0, ids1, w1 = cpu.forward(x[picked])
+    np.testing.assert_array_equal(ids1, ids0[picked])       # the oracle's forward routes like its route call
+    worst = assert_parity(y[picked], ids[picked], w[picked], y0, ids1, w1, label="zipf chunk rows")
+    print(f"zipf chunk: max abs err {worst:.3e} on {len(picked)} rows", flush=True)
+
+
+def test_q4k_verify_batches_share_experts(product, oracle):
+    cfg = workloads.measured_config()
+    weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=1)
+    xs, info = workloads.verify_batches(weights, 4, seed=3)
+    print(f"verify batches: {info}", flush=True)
+    assert 0.3 <= info["mean_adjacent_overlap"] <= 0.7 and info["mean_unique_experts"] < 36
+    with pf.MoeLayer(product, cfg, weights, 4) as gpu, pf.MoeLayer(oracle, cfg, weights, 4) as cpu:
+        assert product.hip.moe_kernel_family(*gpu.device_handles(), 4) == 1
+        for b, x in enumerate(xs):
+            _, y, ids, w = gpu.forward(x)
+            _, y0, ids0, w0 = cpu.forward(x)
+            shared = len(set(ids0[0]) & set(ids0[1]))
+            worst = assert_parity(y, ids, w, y0, ids0, w0, label=f"verify batch {b}")
+            print(f"  batch {b}: {len(set(ids0.reshape(-1)))} unique experts, tokens 0/1 share {shared}, max abs err {worst:.2e}", flush=True)
+
+
+def test_views_over_released_weight_bytes(product, oracle):
+    """qwen4_moe_forward refuses views that overlap the bytes the layer was created from (the
+    reference's rule); after pf_moe_forget_host_weights the addresses are free for reuse."""
+    cfg = abi.moe_config(512, 32, 6, 256, 256)
+    weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=8)
+    x = pf.rms_normalise(pf.Synth().normal((2, 512), 12))
+    with pf.MoeLayer(oracle, cfg, weights, 2) as cpu:
+        _, y0, ids0, w0 = cpu.forward(x)
+    with pf.MoeLayer(product, cfg, weights, 2) as layer:
+        router = weights.raw[0].view(np.float32)                     # the layer's own router bytes, 64 KB
+        inside = router[:2 * 512].reshape(2, 512)
+        y = np.full((2, 512), -99.0, dtype=np.float32)
+        err = abi.Qwen4Error()
+        st = product.forward(layer.handle, abi.f32_view(inside), abi.f32_view(y), None, layer.work, C.byref(err))
+        assert st == abi.QW4_INVALID_ARGUMENT and (y == -99).all()
+        product.forget_host_weights(layer.handle)
+        inside[:] = x                                                # the bytes now belong to the caller again
+        st = product.forward(layer.handle, abi.f32_view(inside), abi.f32_view(y), None, layer.work, C.byref(err))
+        assert st == abi.QW4_OK, err.detail
+        err_abs = np.abs(y - y0)
+        assert (err_abs <= ATOL + RTOL * np.abs(y0)).all()
