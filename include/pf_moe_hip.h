@@ -67,6 +67,18 @@ void pf_hip_work_destroy(PfHipWork *work);
 int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
                               size_t x_pitch, float *d_y, size_t y_pitch, size_t tokens,
                               void *stream);
+/* No counterpart in the reference.  The same forward for callers that cannot allocate or hold a
+ * workspace: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Its scratch is a static device array of the library (1 MiB per GPU, held until the process
+ * ends), so the call allocates and frees nothing; at most 4 tokens, and PF_HIP_E_UNSUPPORTED
+ * (with pf_hip_last_error saying how much was needed) when the layer's scratch for `tokens`
+ * tokens exceeds the array.  Outputs are the caller's: d_y [tokens, hidden] (pitch in floats),
+ * optionally d_ids and d_route_weights (dense [tokens, top_k], NULL = not wanted), and
+ * d_error_word, one device uint32 the kernels OR PF_HIP_ERR_* bits into (the caller clears
+ * it).  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU race. */
+int pf_hip_moe_forward_static(const PfHipMoe *moe, const float *d_x, size_t x_pitch, float *d_y,
+                              size_t y_pitch, uint32_t *d_ids, float *d_route_weights,
+                              uint32_t *d_error_word, size_t tokens, void *stream);
 /* Which kernels a forward of `tokens` tokens runs on this layer and workspace: 1 the
  * decode kernels (1..4 tokens, supported shapes and formats), 2 the matrix-core
  * prefill kernels, 0 the general kernels (any shape and format mix). */

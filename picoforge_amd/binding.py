@@ -119,6 +119,7 @@ class HipShim:
         bind("pf_hip_work_create", C.c_int, vp, sz, P(vp))
         bind("pf_hip_work_destroy", None, vp)
         bind("pf_hip_moe_forward_device", C.c_int, vp, vp, vp, sz, vp, sz, sz, vp)
+        bind("pf_hip_moe_forward_static", C.c_int, vp, vp, sz, vp, sz, vp, vp, vp, sz, vp)
         bind("pf_hip_work_ids", vp, vp)
         bind("pf_hip_work_route_weights", vp, vp)
         bind("pf_hip_work_logits", vp, vp)

@@ -25,6 +25,31 @@ extern "C" int pf_hip_device_count(void) {
     return n;
 }
 
+// Scratch of the entry point that allocates nothing (pf_hip_moe_forward_static): one array per GPU,
+// held from the library's load until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress; kernels and copies use the address that call returns.
+#define PF_STATIC_SCRATCH_BYTES ((size_t)1 << 20)
+#define PF_MAX_DEVICES 16
+static __device__ __align__(256) unsigned char scratch[PF_STATIC_SCRATCH_BYTES];
+static uint8_t *g_scratch_ptr[PF_MAX_DEVICES];
+
+// The current device's copy of the array; looked up once per device, with that device current.
+static int static_scratch(uint8_t **out) {
+    int dev = -1;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= PF_MAX_DEVICES) {
+        snprintf(g_error, sizeof g_error, "device %d is beyond the %d devices the static scratch serves", dev, PF_MAX_DEVICES);
+        return PF_HIP_E_UNSUPPORTED;
+    }
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = static_cast<uint8_t *>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return PF_HIP_OK;
+}
+
 static int need_device(void) {
     if (pf_hip_device_count() >= 1) return PF_HIP_OK;
     snprintf(g_error, sizeof g_error, "no HIP device");
@@ -179,6 +204,11 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         m->expert_bytes[a] = m->row_bytes[a] * n_out[a];
     }
     if (!upload_constants()) { pf_hip_moe_destroy(m); return PF_HIP_E_MEMORY; }
+    {   // set-up: this device's address of the static scratch, so that the entry point that uses it calls nothing but launches
+        uint8_t *unused = nullptr;
+        const int rc = static_scratch(&unused);
+        if (rc != PF_HIP_OK) { pf_hip_moe_destroy(m); return rc; }
+    }
     m->iq2_grid = g_grid;
     m->iq2_signed = g_signed;
     for (int a = 0; a < 8; a++) {
@@ -327,6 +357,8 @@ extern "C" size_t pf_hip_work_bytes(const PfHipMoeDesc *desc, size_t token_cap) 
     return desc ? plan_work(desc, token_cap).total : 0;
 }
 
+static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base);
+
 extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWork **out) {
     if (out) *out = nullptr;
     if (!moe || !out) return PF_HIP_E_ARGUMENT;
@@ -343,6 +375,12 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
         return PF_HIP_E_MEMORY;
     }
     w->moe = moe; w->cap = token_cap; w->bytes = c.total;
+    carve_work(w, c, base);
+    *out = w;
+    return PF_HIP_OK;
+}
+
+static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base) {
     w->logits = (float *)(base + c.offset[W_LOGITS]);
     w->logit_ssq = (float *)(base + c.offset[W_SSQ]);
     w->route_weights = (float *)(base + c.offset[W_RW]);
@@ -372,8 +410,6 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
         w->group_bad = (uint32_t *)(base + c.offset[W_GROUPBAD]);
         w->tiles = (uint32_t *)(base + c.offset[W_TILES]);
     }
-    *out = w;
-    return PF_HIP_OK;
 }
 
 extern "C" void pf_hip_work_destroy(PfHipWork *w) {
@@ -498,6 +534,41 @@ extern "C" int pf_hip_moe_forward_device(const PfHipMoe *moe, PfHipWork *work, c
     if (tokens == 0) return PF_HIP_OK;
     if (!d_x || !d_y || x_pitch < moe->desc.hidden || y_pitch < moe->desc.hidden) return PF_HIP_E_ARGUMENT;
     return forward_enqueue(moe, work, d_x, x_pitch, d_y, y_pitch, tokens, nullptr, (hipStream_t)stream);
+}
+
+// The same forward for callers that cannot allocate (code under graph capture, tight serving loops):
+// the workspace is the library's static device array instead of a PfHipWork.  Calls nothing that
+// allocates or frees; every call on a GPU shares that GPU's array, so calls that overlap on one GPU race.
+// Nothing in the array has to start at zero: every buffer of it is written before it is read within a
+// forward (the re-route counter it also holds only ever accumulates and is not reported here).
+extern "C" int pf_hip_moe_forward_static(const PfHipMoe *moe, const float *d_x, size_t x_pitch, float *d_y,
+                                         size_t y_pitch, uint32_t *d_ids, float *d_route_weights,
+                                         uint32_t *d_error_word, size_t tokens, void *stream) {
+    if (!moe || !d_error_word) return PF_HIP_E_ARGUMENT;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!d_x || !d_y || x_pitch < moe->desc.hidden || y_pitch < moe->desc.hidden) return PF_HIP_E_ARGUMENT;
+    if (tokens > PF_DECODE_MAX_TOKENS) {
+        snprintf(g_error, sizeof g_error, "the static scratch serves batches of at most %d tokens, not %zu",
+                 PF_DECODE_MAX_TOKENS, tokens);
+        return PF_HIP_E_UNSUPPORTED;
+    }
+    const Carve c = plan_work(&moe->desc, tokens);
+    if (c.total > PF_STATIC_SCRATCH_BYTES) {
+        snprintf(g_error, sizeof g_error, "this layer needs %zu bytes of scratch for %zu tokens; the static scratch holds %zu",
+                 c.total, tokens, (size_t)PF_STATIC_SCRATCH_BYTES);
+        return PF_HIP_E_UNSUPPORTED;
+    }
+    uint8_t *base = nullptr;
+    const int rc = static_scratch(&base);
+    if (rc != PF_HIP_OK) return rc;
+    PfHipWork w;
+    memset(&w, 0, sizeof w);
+    w.moe = moe; w.cap = tokens; w.bytes = c.total;
+    carve_work(&w, c, base);
+    if (d_ids) w.ids = d_ids;
+    if (d_route_weights) w.route_weights = d_route_weights;
+    w.error_word = d_error_word;
+    return forward_enqueue(moe, &w, d_x, x_pitch, d_y, y_pitch, tokens, nullptr, (hipStream_t)stream);
 }
 
 // ---- hyper-connection read and add (src/qwen4_base.c:142-175) -----------------------------------
