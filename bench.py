@@ -1,39 +1,34 @@
 #!/usr/bin/env python3
 """Benchmark of the MoE feed-forward path on one MI355X.
 
-Default workload (the configuration the metric is quoted on): one MoE layer at
-hidden 2048 / 512 experts / top-10 / intermediate 512 with IQ2_XXS expert
-blocks, decode batch 1, seeded RMS-normalised tokens whose top-11 router logits
-are at least 1e-3 apart.  A step is one token batch through the layer; inputs and
-weights are resident in HBM before the timed region; every step uses another
-input, hence other experts.
-
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
-Workloads: iq2xxs_decode (default), q4k_decode, q4k_verify4 (4-token batches with
-about half of the experts shared between neighbours), q4k_prefill1024 and
-iq2xxs_prefill1024 (1024-token chunks, N(0,1) activations, Zipf(1.1) expert
-popularity), q4k_stack48 (48 resident layers, decode and 2048-token chunks), and
-q2profile_decode / q4profile_decode / q2profile_prefill1024 / q4profile_prefill1024 (the
-format mixes of real checkpoints: IQ2_XXS gate/up + Q2_K down, Q4_K gate/up + MXFP4 down,
-Q8_0 shared expert), q2ckpt_decode / q4ckpt_decode / q2ckpt_prefill1024 / q4ckpt_prefill1024 (those
-mixes at the checkpoints' own widths: hidden 2560, intermediate and shared 640, the Q2_K down
-projection stored 768 wide), and
-iq2xxs_decode_hc / q4k_decode_hc / q4k_prefill1024_hc: the same layer between its two
-hyper-connection steps (gated read of 4 residual streams before, injection into them
-after), with the injection folded into the block's last kernel and as a kernel of its own
-(q2ckpt_decode_hc / q2ckpt_prefill1024_hc: the same at the checkpoints' widths).
+Default (`--workload all`): one JSON line whose headline (`metric`, `value`, `roofline`,
+`cpu_baseline`) is the Q4_K decode layer -- one token through one MoE layer at hidden 2048 / 512
+experts / top-10 / intermediate 512 / shared 512 -- and whose `configs` object carries a record of
+the same form for each further benchmark configuration: IQ2_XXS decode, the 4-token Q4_K verify
+batch, the 1024-token Q4_K prefill chunk under a Zipf(1.1) router, and the 48-layer resident stack.
+`--workload NAME` runs one configuration alone and prints its record as the line.
 
-Prints one JSON line.  `value` is microseconds per layer per token (lower is
-better).  `roofline` is for the kernel that moves the most bytes, timed live
-with HIP events on the launch stream.  `cpu_baseline` times the CPU path (the
-reference's own compiled C when oracle/_ref is present, else the oracle port) on
-a bounded sample of the same tokens, single thread, and the same sample is used
-to check the GPU results (ids exact, outputs within 1e-3 + 1e-4 relative).
+A step is one token batch through the layer (or, for the stack, one token through all layers);
+inputs and weights are resident in HBM before the timed region; every step uses another seeded
+input, hence other experts.  K steps are captured once into HIP graphs and replayed until at least
+50 ms have been timed; `ms_per_step` is the median over the replays (p10 / p90 beside it), each
+replay bracketed by HIP events on the launch stream.  `roofline` is for the kernel that moves the
+most bytes: its duration is the difference between replays of the chain cut after it and before it
+(events on the launch stream).  `cpu_baseline` times the CPU path (the reference's own compiled C
+when oracle/_ref is present, else the oracle port) on a bounded sample of the same inputs, one
+thread, and the same sample checks the GPU results (ids exact, outputs within 1e-3 + 1e-4 relative).
+
+Further workloads: iq2xxs_prefill1024; q2profile_* / q4profile_* (the format mixes of real checkpoints)
+and q2ckpt_* / q4ckpt_* (those mixes at the checkpoints' own widths: hidden 2560, intermediate and shared
+640, the Q2_K down projection stored 768 wide); *_hc: the layer between its two hyper-connection steps.
 """
 import argparse
 import ctypes as C
+import hashlib
 import json
+import math
 import os
 import sys
 import time
@@ -52,64 +47,49 @@ FORMAT_LABEL = {12: "Q4_K", 16: "IQ2_XXS", "q2": "IQ2_XXS gate/up, Q2_K down, Q8
                 "q4": "Q4_K gate/up, MXFP4 down, Q8_0 shared expert"}
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+MIN_TIMED_MS = 50.0
+CKPT_Q2, CKPT_Q4 = (2560, 512, 10, 640, 640, 768), (2560, 512, 10, 640, 640, 640)
+PREFILL_LABEL = "1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"
 
 WORKLOADS = {
-    "iq2xxs_decode": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=10000, warmup=200,
-                          label="IQ2_XXS experts, decode batch 1"),
-    "q4k_decode": dict(type=abi.GGUF_Q4_K, tokens=1, steps=10000, warmup=200, label="Q4_K experts, decode batch 1"),
-    "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, steps=2000, warmup=100,
+    "q4k_decode": dict(type=abi.GGUF_Q4_K, tokens=1, steps=2000, warmup=200, label="Q4_K experts, decode batch 1"),
+    "iq2xxs_decode": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=2000, warmup=200, label="IQ2_XXS experts, decode batch 1"),
+    "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, steps=1000, warmup=100,
                         label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
-    "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10,
-                            label="Q4_K experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
-    "iq2xxs_prefill1024": dict(type=abi.GGUF_IQ2_XXS, tokens=1024, steps=100, warmup=10,
-                               label="IQ2_XXS experts, 1024-token prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
-    "iq2xxs_decode_hc": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=10000, warmup=200, hc=4,
+    "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=20, warmup=5, label="Q4_K experts, " + PREFILL_LABEL),
+    "iq2xxs_prefill1024": dict(type=abi.GGUF_IQ2_XXS, tokens=1024, steps=20, warmup=5, label="IQ2_XXS experts, " + PREFILL_LABEL),
+    "iq2xxs_decode_hc": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=2000, warmup=200, hc=4,
                              label="IQ2_XXS experts, decode batch 1, between the HC read and add of 4 residual streams"),
-    "q4k_decode_hc": dict(type=abi.GGUF_Q4_K, tokens=1, steps=10000, warmup=200, hc=4,
+    "q4k_decode_hc": dict(type=abi.GGUF_Q4_K, tokens=1, steps=2000, warmup=200, hc=4,
                           label="Q4_K experts, decode batch 1, between the HC read and add of 4 residual streams"),
-    "q4k_prefill1024_hc": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=100, warmup=10, hc=4,
+    "q4k_prefill1024_hc": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=20, warmup=5, hc=4,
                                label="Q4_K experts, 1024-token prefill chunk, between the HC read and add of 4 residual "
                                      "streams, Zipf(1.1) expert popularity"),
-    "q2profile_decode": dict(type="q2", tokens=1, steps=5000, warmup=100,
-                             label="checkpoint profile Q2 (IQ2_XXS gate/up, Q2_K down, Q8_0 shared expert), decode batch 1"),
-    "q4profile_decode": dict(type="q4", tokens=1, steps=5000, warmup=100,
-                             label="checkpoint profile Q4 (Q4_K gate/up, MXFP4 down, Q8_0 shared expert), decode batch 1"),
-    "q2profile_prefill1024": dict(type="q2", tokens=1024, steps=50, warmup=5,
-                                  label="checkpoint profile Q2 (IQ2_XXS gate/up, Q2_K down, Q8_0 shared expert), 1024-token "
-                                        "prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
-    "q4profile_prefill1024": dict(type="q4", tokens=1024, steps=50, warmup=5,
-                                  label="checkpoint profile Q4 (Q4_K gate/up, MXFP4 down, Q8_0 shared expert), 1024-token "
-                                        "prefill chunk, N(0,1) activations, Zipf(1.1) expert popularity"),
-    # the checkpoints' own widths (hidden 2560, intermediate 640, shared 640; the Q2_K down projection stored 768 wide)
-    "q2ckpt_decode": dict(type="q2", tokens=1, steps=5000, warmup=100, dims=(2560, 512, 10, 640, 640, 768),
+    "q2profile_decode": dict(type="q2", tokens=1, steps=2000, warmup=100, label="checkpoint profile Q2, decode batch 1"),
+    "q4profile_decode": dict(type="q4", tokens=1, steps=2000, warmup=100, label="checkpoint profile Q4, decode batch 1"),
+    "q2profile_prefill1024": dict(type="q2", tokens=1024, steps=20, warmup=5, label="checkpoint profile Q2, " + PREFILL_LABEL),
+    "q4profile_prefill1024": dict(type="q4", tokens=1024, steps=20, warmup=5, label="checkpoint profile Q4, " + PREFILL_LABEL),
+    "q2ckpt_decode": dict(type="q2", tokens=1, steps=2000, warmup=100, dims=CKPT_Q2,
                           label="checkpoint profile Q2 at the checkpoints' widths, decode batch 1"),
-    "q4ckpt_decode": dict(type="q4", tokens=1, steps=5000, warmup=100, dims=(2560, 512, 10, 640, 640, 640),
+    "q4ckpt_decode": dict(type="q4", tokens=1, steps=2000, warmup=100, dims=CKPT_Q4,
                           label="checkpoint profile Q4 at the checkpoints' widths, decode batch 1"),
-    "q2ckpt_prefill1024": dict(type="q2", tokens=1024, steps=50, warmup=5, dims=(2560, 512, 10, 640, 640, 768),
-                               label="checkpoint profile Q2 at the checkpoints' widths, 1024-token prefill chunk, N(0,1) "
-                                     "activations, Zipf(1.1) expert popularity"),
-    "q4ckpt_prefill1024": dict(type="q4", tokens=1024, steps=50, warmup=5, dims=(2560, 512, 10, 640, 640, 640),
-                               label="checkpoint profile Q4 at the checkpoints' widths, 1024-token prefill chunk, N(0,1) "
-                                     "activations, Zipf(1.1) expert popularity"),
-    "q2ckpt_decode_hc": dict(type="q2", tokens=1, steps=5000, warmup=100, hc=4, dims=(2560, 512, 10, 640, 640, 768),
+    "q2ckpt_prefill1024": dict(type="q2", tokens=1024, steps=20, warmup=5, dims=CKPT_Q2,
+                               label="checkpoint profile Q2 at the checkpoints' widths, " + PREFILL_LABEL),
+    "q4ckpt_prefill1024": dict(type="q4", tokens=1024, steps=20, warmup=5, dims=CKPT_Q4,
+                               label="checkpoint profile Q4 at the checkpoints' widths, " + PREFILL_LABEL),
+    "q2ckpt_decode_hc": dict(type="q2", tokens=1, steps=2000, warmup=100, hc=4, dims=CKPT_Q2,
                              label="checkpoint profile Q2 at the checkpoints' widths, decode batch 1, between the HC read and "
                                    "add of 4 residual streams"),
-    "q2ckpt_prefill1024_hc": dict(type="q2", tokens=1024, steps=50, warmup=5, hc=4, dims=(2560, 512, 10, 640, 640, 768),
+    "q2ckpt_prefill1024_hc": dict(type="q2", tokens=1024, steps=20, warmup=5, hc=4, dims=CKPT_Q2,
                                   label="checkpoint profile Q2 at the checkpoints' widths, 1024-token prefill chunk, between "
                                         "the HC read and add of 4 residual streams, Zipf(1.1) expert popularity"),
-    "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=200, warmup=20,
+    "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=100, warmup=10,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),
 }
-# HBM bytes per launch of each workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE scaled by the same counters on a plain 256 MiB copy (profiles/*.txt hold the runs).
-# A counter result cannot be read live; None where no such run exists for the workload.
-MEASURED_TRAFFIC = {"iq2xxs_decode": 9892423, "q4k_decode": 19875557, "q4k_verify4": None,
-                    "q4k_prefill1024": 817391959, "iq2xxs_prefill1024": 460067641,
-                    # the hyper-connection chains: traffic of pf_k_hc_read, their roofline kernel
-                    "q4k_prefill1024_hc": 75633928, "iq2xxs_decode_hc": 117050, "q4k_decode_hc": None,
-                    "q2profile_decode": None, "q4profile_decode": None, "q2profile_prefill1024": None, "q2ckpt_decode": None, "q4ckpt_decode": None, "q2ckpt_decode_hc": None, "q2ckpt_prefill1024_hc": None,
-                    "q4profile_prefill1024": None}
+HEADLINE = "q4k_decode"
+ALL_CONFIGS = ["iq2xxs_decode", "q4k_verify4", "q4k_prefill1024", "q4k_stack48"]
+
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
@@ -124,255 +104,105 @@ PREFILL_STAGES = ["pf_k_rows_to_half + pf_k_pf_router (fp16 copy of x, router lo
 # on the checkpoint profiles the Q8_0 / Q2_K / MXFP4 items of stages 3 and 4 run in pf_k_pf_gemm_plain
 
 
-def run_stack(args, api, hip, cfg, steps, warmup):
-    """A stack of independent layers, all resident: every token (or chunk) passes the layers in order, each
-    layer with its own seeded input, hence its own routing.  The popularity bias sits in router column 0
-    (workloads.zipf_router): inputs with coordinate 0 = 1 see Zipf(1.1) popularity, with 0 the plain router."""
-    layers_n, chunk = args.layers, 2048
-    t0 = time.time()
-    layers, sample = [], None
-    for l in range(layers_n):
-        weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=args.seed * 1000 + l)
-        workloads.zipf_router(weights, seed=args.seed * 1000 + l, temperature=0.18)
-        layers.append(pf.MoeLayer(api, cfg, weights, chunk))
-        if l == 0:
-            sample = weights
-        else:
-            layers[-1].weights = None      # the library copied the bytes into HBM at create
-    prep_s = time.time() - t0
-    moes = (C.c_void_p * layers_n)(*[l.device_handles()[0] for l in layers])
-    works = (C.c_void_p * layers_n)(*[l.device_handles()[1] for l in layers])
-    resident = sum(hip.moe_bytes(m) for m in moes)
-    synth = pf.Synth()
-    h = cfg.hidden_size
-    per_layer_tokens = 32
-    dec = pf.rms_normalise(synth.normal((per_layer_tokens * layers_n, h), 77 + args.seed))
-    pre = synth.normal((4 * chunk, h), 78 + args.seed)
-    d_y = hip.to_device(np.zeros((chunk, h), dtype=np.float32))
-    out = {}
-    ms = C.c_float()
-    for name, coord in (("uniform", 0.0), ("zipf", 1.0)):
-        dec[:, 0] = coord
-        pre[:, 0] = coord
-        d_dec, d_pre = hip.to_device(dec), hip.to_device(pre)
-        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_dec, len(dec), d_y, 1, warmup * layers_n, C.byref(ms)), "warmup")
-        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_dec, len(dec), d_y, 1, steps * layers_n, C.byref(ms)), "decode")
-        out[name + "_decode_us_per_token"] = ms.value * 1e3 / steps
-        chunks = max(2, steps // 50)
-        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_pre, 4, d_y, chunk, layers_n, C.byref(ms)), "warmup")
-        hip.check(hip.stack_time_forwards(moes, works, layers_n, d_pre, 4, d_y, chunk, chunks * layers_n, C.byref(ms)), "prefill")
-        out[name + "_prefill_ms_per_chunk"] = ms.value / chunks
-        out[name + "_prefill_tokens_per_s"] = chunk / (ms.value / chunks * 1e-3)
-        hip.free(d_dec)
-        hip.free(d_pre)
-    errors = sum(int(hip.from_device(hip.work_error_word(w), (1,), np.uint32)[0]) for w in works)
-    # parity and the CPU cost per layer-token on layer 0; the stack's CPU time is that times the layers
+class Tools:
+    """picoforge_amd/libpf_bench.so (csrc/pf_bench_tools.h): graph-replay timing on top of the shipped library."""
+
+    def __init__(self):
+        path = ROOT / "picoforge_amd" / "libpf_bench.so"
+        if not path.exists():
+            raise pf.LibraryMissing(f"{path} is not built: run make -C picoforge_amd/csrc")
+        lib = C.CDLL(str(path), mode=C.RTLD_GLOBAL)
+        vp, sz, P = C.c_void_p, C.c_size_t, C.POINTER
+        lib.pf_bench_last_error.restype = C.c_char_p
+        lib.pf_bench_plan_moe.argtypes = [P(vp), P(vp), sz, vp, sz, vp, sz, sz, sz, C.c_int, sz, P(vp)]
+        lib.pf_bench_plan_hc.argtypes = [vp, vp, vp, vp, sz, vp, vp, sz, sz, sz, C.c_int, sz, P(vp)]
+        lib.pf_bench_plan_run.argtypes = [vp, sz, P(C.c_float)]
+        lib.pf_bench_plan_destroy.argtypes = [vp]
+        lib.pf_bench_plan_destroy.restype = None
+        lib.pf_bench_hc_time_step.argtypes = [C.c_int, vp, vp, vp, vp, sz, sz, sz, sz, vp, P(C.c_float)]
+        lib.pf_bench_copy_probe.argtypes = [sz, sz]
+        self.lib = lib
+
+    def check(self, rc, what):
+        if rc != 0:
+            raise RuntimeError(f"{what}: status {rc}: {self.lib.pf_bench_last_error().decode()}")
+
+    def plan_moe(self, moes, works, d_x, n_inputs, d_y, y_blocks, tokens, forwards, hidden, kernel_limit=0):
+        n = len(moes)
+        plan = C.c_void_p()
+        self.check(self.lib.pf_bench_plan_moe((C.c_void_p * n)(*moes), (C.c_void_p * n)(*works), n, d_x, n_inputs, d_y,
+                                              y_blocks, tokens, forwards, kernel_limit, hidden, C.byref(plan)), "plan")
+        return plan
+
+    def plan_hc(self, moe, work, d_n, d_g, n_inputs, d_r, d_i, streams, tokens, forwards, fused, hidden):
+        plan = C.c_void_p()
+        self.check(self.lib.pf_bench_plan_hc(moe, work, d_n, d_g, n_inputs, d_r, d_i, streams, tokens, forwards, fused, hidden,
+                                             C.byref(plan)), "hc plan")
+        return plan
+
+    def run(self, plan, repeats):
+        ms = (C.c_float * repeats)()
+        self.check(self.lib.pf_bench_plan_run(plan, repeats, ms), "plan run")
+        return np.array(ms[:], dtype=np.float64)
+
+    def destroy(self, plan):
+        self.lib.pf_bench_plan_destroy(plan)
+
+    def timed(self, plan, forwards, warmup):
+        """Warm-up replays (at least `warmup` forwards), then replays until MIN_TIMED_MS are timed (at least 5).
+        Returns ms per forward: median, p10, p90, the number of timed replays and the total timed ms."""
+        self.run(plan, max(1, math.ceil(warmup / forwards)))
+        first = self.run(plan, 3)
+        est = max(float(np.median(first)), 1e-4)
+        repeats = int(min(5000, max(5, math.ceil(MIN_TIMED_MS / est))))
+        ms = self.run(plan, repeats)
+        per = ms / forwards
+        return {"median": float(np.median(per)), "p10": float(np.percentile(per, 10)), "p90": float(np.percentile(per, 90)),
+                "replays": repeats, "timed_ms": float(ms.sum())}
+
+
+def sources_digest():
+    """Digest of the kernel sources: a traffic figure from a profile is only quoted for the kernels it was taken on."""
+    h = hashlib.sha256()
+    for path in sorted((ROOT / "picoforge_amd" / "csrc").glob("*.h*")):
+        h.update(path.name.encode())
+        h.update(path.read_bytes())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the workload's dominant kernel from profiles/traffic.json (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE, scaled by the same counters on a plain copy of known size).  A counter cannot be
+    read live, so the figure is quoted only while the kernel sources are the ones it was measured on."""
+    path = ROOT / "profiles" / "traffic.json"
+    if not path.exists():
+        return None, None
+    entry = json.loads(path.read_text()).get(workload)
+    if not entry:
+        return None, None
+    source = {"profile": entry.get("profile"), "sources": entry.get("sources"), "kernel": entry.get("kernel")}
+    if entry.get("sources") != sources_digest():
+        return None, dict(source, stale=True)
+    return entry["bytes"], source
+
+
+def cpu_api_and_kind():
     ref = load_reference()
-    cpu_api, kind = (ref, "reference") if ref is not None else (load_oracle(), "port")
-    n = args.cpu_sample or 16
-    xs = dec[:n].copy()
-    with pf.MoeLayer(cpu_api, cfg, sample, n) as cpu:
-        c0 = time.perf_counter()
-        _, y0, ids0, _ = cpu.forward(xs)
-        cpu_s = time.perf_counter() - c0
-    _, y1, ids1, _ = layers[0].forward(xs)
-    ids_equal = bool((ids0 == ids1).all())
-    within = bool((np.abs(y1 - y0) <= 1e-3 + 1e-4 * np.abs(y0)).all())
-    for l in layers:
-        l.close()
-    us = out["uniform_decode_us_per_token"]
-    alg = layers_n * workloads.algorithmic_bytes_per_token(abi.GGUF_Q4_K)
-    result = {
-        "metric": "moe_stack_decode_us_per_token", "value": round(us, 2), "unit": "us/token (all layers)",
-        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(us * 1e-3, 6),
-        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{layers_n} independent MoE layers (hidden 2048, 512 experts, top-10, intermediate 512, "
-                               f"shared 512, Q4_K), {resident / 1e9:.1f} GB resident in HBM; decode batch 1 and "
-                               f"{chunk}-token prefill chunks; per-layer seeded inputs and routers",
-                   "layers": layers_n, "tokens_per_step": 1},
-        "us_per_layer_token": round(us / layers_n, 3),
-        "hbm_GBps_on_algorithmic_bytes": round(alg / (us * 1e-6) / 1e9, 1),
-        "algorithmic_bytes_per_step": int(alg),
-        "roofline": {"bound": "hbm", "kernel": "whole stack: three decode kernels per layer", "achieved":
-                     round(alg / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None},
-        "stack": {k: round(v, 3) for k, v in out.items()},
-        "cpu_baseline": {"value": round(cpu_s / n * 1e6 * layers_n, 1), "unit": "us/token (all layers)", "cores": 1,
-                         "kind": kind, "sample": f"{n} tokens through layer 0 ({cpu_s:.1f} s), times {layers_n} layers: "
-                                                 "an extrapolation, the CPU cost is linear in layers and tokens"},
-        "parity_on_sample": {"ids_equal": ids_equal, "within_1e-3_abs_1e-4_rel": within, "error_word": errors},
-        "prep_s": round(prep_s, 1),
-    }
-    print(json.dumps(result))
-    if not (ids_equal and within and errors == 0):
-        sys.exit("parity check failed on the sample")
+    return (ref, "reference") if ref is not None else (load_oracle(), "port")
 
 
-def run_hc(args, api, hip, cfg, wl, steps, warmup):
-    """One layer between its two hyper-connection steps (src/qwen4_forward.c:362-367): per step a gated read
-    of [tokens, streams, hidden] normed streams and gate logits, the MoE block, and the injection of the
-    block's output into the [tokens, streams, hidden] residual.  Timed three ways on resident buffers: the
-    chain with the injection folded into the block's last kernel (`value`), the chain with the injection as
-    a kernel of its own, and the block alone on the same mixed rows."""
-    tokens, streams, h = wl["tokens"], wl["hc"], cfg.hidden_size
-    t0 = time.time()
-    weights = pf.LayerWeights.synthetic(cfg, wl["type"], seed=args.seed)
-    if tokens > 4:
-        workloads.zipf_router(weights, seed=args.seed, temperature=0.18)
-    n_inputs = max(1, min(steps, 4 if tokens > 4 else 2000))
-    rng = np.random.default_rng(args.seed)
-    # streams whose gated mix has about unit RMS, as the block sees after the norm
-    normed = (rng.standard_normal((n_inputs, tokens, streams, h)) * (2.0 * streams ** 0.5 / 1.12)).astype(np.float32)
-    logits = rng.standard_normal((n_inputs, tokens, streams, h)).astype(np.float32)
-    residual = rng.standard_normal((tokens, streams, h)).astype(np.float32)
-    inject = rng.uniform(0.0, 2.0 / streams, (tokens, streams)).astype(np.float32)
-    # the timed loop adds into one residual thousands of times: weights scaled down so that it stays small
-    inject_timed = inject * np.float32(1e-3)
-    prep_s = time.time() - t0
-    layer = pf.MoeLayer(api, cfg, weights, tokens)
-    moe, work = layer.device_handles()
-    d_n, d_g, d_i = hip.to_device(normed), hip.to_device(logits), hip.to_device(inject_timed)
-    d_r = hip.to_device(residual)
-    ms = C.c_float()
-    timed = {}
-    for name, fused in (("fused", 1), ("separate_add", 0)):
-        hip.check(hip.memcpy_h2d(d_r, residual.ctypes.data, residual.nbytes), "residual")
-        hip.check(hip.moe_time_forwards_hc(moe, work, d_n, d_g, n_inputs, d_r, d_i, streams, tokens, warmup, fused,
-                                           C.byref(ms)), "warmup")
-        hip.check(hip.moe_time_forwards_hc(moe, work, d_n, d_g, n_inputs, d_r, d_i, streams, tokens, steps, fused,
-                                           C.byref(ms)), "timed loop")
-        timed[name] = ms.value / steps
-    err_word = int(hip.from_device(hip.work_error_word(work), (1,), np.uint32)[0])
-    # the block alone on the mixed rows the read produces
-    shape = abi.Qwen4HcShape(streams, h, 1, 1e-6)
-    mixed = np.empty((n_inputs, tokens, h), dtype=np.float32)
-    for b in range(n_inputs):
-        st = api.hc.read(C.byref(shape), abi.f32_cube(normed[b]), abi.f32_cube(logits[b]), abi.f32_view(mixed[b]), None)
-        assert st == abi.QW4_OK, st
-    d_x = hip.to_device(mixed)
-    d_y = hip.to_device(np.zeros((tokens, h), dtype=np.float32))
-    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, warmup, C.byref(ms)), "warmup")
-    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, steps, C.byref(ms)), "block alone")
-    block_ms = ms.value / steps
-
-    # the two hyper-connection kernels alone, HIP events on the launch stream around back-to-back launches
-    # (the add runs with zero weights so that the residual stays put over the launches)
-    d_zero = hip.to_device(np.zeros_like(inject))
-    d_err = hip.to_device(np.zeros(64, dtype=np.uint32))
-    kernel_us = {}
-    n_launch = max(50, min(steps, 1000))
-    for which, name in ((0, "pf_k_hc_read"), (1, "pf_k_hc_add")):
-        for count in (10, n_launch):
-            hip.check(hip.hc_time_step(which, d_n if which == 0 else d_r, d_g, d_x if which == 0 else d_y,
-                                       d_zero, tokens, streams, h, count, d_err, C.byref(ms)), name)
-        kernel_us[name] = ms.value * 1e3 / n_launch
-    read_bytes = tokens * h * 4 * (2 * streams + 1)
-    add_bytes = tokens * h * 4 * (2 * streams + 1) + tokens * streams * 4
-    if args.copy_probe:
-        hip.check(hip.copy_probe(args.copy_probe << 20, 3), "copy probe")
-
-    # parity on a bounded sample, stage by stage on identical inputs: CPU read against the device's mixed rows,
-    # CPU block on those rows, CPU add of its output; the device's chained call against that residual
-    ref = load_reference()
-    cpu_api, kind = (ref, "reference") if ref is not None else (load_oracle(), "port")
-    sample = min(tokens, args.cpu_sample or (24 if wl["type"] == abi.GGUF_IQ2_XXS else 40))
-    steps_cpu = 1 if tokens > 1 else min(sample, n_inputs)
-    rows = sample if tokens > 1 else 1
-    ids_equal = within = read_close = True
-    max_abs = 0.0
-    cpu_s = 0.0
-    with pf.MoeLayer(cpu_api, cfg, weights, rows) as cpu:
-        for b in range(steps_cpu):
-            n_b, g_b = normed[b][:rows], logits[b][:rows]
-            want = residual[:rows].copy()
-            c0 = time.perf_counter()
-            _, ids_c, _ = cpu.forward_hc(n_b, g_b, want, inject[:rows], fused=False)
-            cpu_s += time.perf_counter() - c0
-            # the same chain with the CPU block fed the device's mixed rows (identical inputs to every stage)
-            _, y_c, ids_m, _ = cpu.forward(mixed[b][:rows])
-            want_m = residual[:rows].copy()
-            cpu_api.hc.add(C.byref(shape), abi.f32_cube(want_m), abi.f32_view(y_c), abi.f32_view(inject[:rows]), None)
-            got = residual.copy()
-            _, ids_g, _ = layer.forward_hc(normed[b], logits[b], got, inject)
-            ids_equal &= bool((ids_g[:rows] == ids_m).all())
-            bound = np.abs(inject[:rows])[:, :, None] * (1e-3 + 1e-4 * np.abs(y_c)[:, None, :]) + 1e-6 * np.abs(want_m)
-            within &= bool((np.abs(got[:rows] - want_m) <= bound).all())
-            max_abs = max(max_abs, float(np.abs(got[:rows] - want_m).max()))
-            read_close &= bool(np.allclose(want, want_m, atol=1e-5, rtol=1e-5))
-    layer.close()
-    sample_tokens = steps_cpu * rows
-    ms_per_step = timed["fused"]
-    hc_bytes = tokens * h * 4 * (2 * streams + 1) + tokens * h * 4 * 2 * streams   # read in/out, residual in/out
-    result = {
-        "metric": "moe_hc_block_us_per_layer_token", "value": round(ms_per_step * 1e3 / tokens, 3),
-        "unit": "us/layer/token", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
-        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if tokens <= 4 else "f16 products, f32 accumulation", "data": "synthetic",
-        "config": {"workload": f"one MoE layer, hidden {cfg.hidden_size}, {cfg.experts} experts, top-{cfg.top_k}, "
-                               f"intermediate {cfg.intermediate}, shared {cfg.shared_intermediate}; "
-                               f"{wl['label']}; {n_inputs} seeded inputs",
-                   "tokens_per_step": tokens, "streams": streams,
-                   "expert_format": FORMAT_LABEL[wl["type"]]},
-        "chain_us_per_step": {"read + block with the add folded in": round(timed["fused"] * 1e3, 3),
-                              "read + block + add kernel": round(timed["separate_add"] * 1e3, 3),
-                              "block alone": round(block_ms * 1e3, 3)},
-        "hc_bytes_per_step": int(hc_bytes),
-        "kernel_us": {k: round(v, 3) for k, v in kernel_us.items()},
-        "kernel_bytes": {"pf_k_hc_read": int(read_bytes), "pf_k_hc_add": int(add_bytes)},
-        "kernel_GBps": {"pf_k_hc_read": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9, 1),
-                        "pf_k_hc_add": round(add_bytes / (kernel_us["pf_k_hc_add"] * 1e-6) / 1e9, 1)},
-        "roofline": {"bound": "hbm", "kernel": "pf_k_hc_read (gated mix of the residual streams)",
-                     "achieved": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(args.workload), "bytes_per_launch": int(read_bytes),
-                     "us_per_launch": round(kernel_us["pf_k_hc_read"], 3)},
-        "cpu_baseline": {"value": round(cpu_s / sample_tokens * 1e6, 1), "unit": "us/layer/token", "cores": 1,
-                         "kind": kind, "sample": f"{sample_tokens} tokens of the same inputs through read, block and add, "
-                                                 f"{cpu_s:.1f} s"},
-        "parity_on_sample": {"ids_equal": ids_equal, "residual_within_block_tolerance_times_inject": within,
-                             "cpu_read_vs_device_read_chain_close": read_close, "max_abs_err": max_abs,
-                             "error_word": err_word},
-        "prep_s": round(prep_s, 1),
-    }
-    print(json.dumps(result))
-    if not (ids_equal and within and err_word == 0):
-        sys.exit("parity check failed on the sample")
-
-
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None)
-    ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="iq2xxs_decode", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-sample", type=int, default=None, help="tokens timed on the CPU path (default ~15 s of work)")
-    ap.add_argument("--seed", type=int, default=1)
-    ap.add_argument("--layers", type=int, default=48, help="layers of the q4k_stack48 workload")
-    ap.add_argument("--skip-stages", action="store_true",
-                    help="leave out the per-kernel timing by stage-limited graph replays (kernel_us is then meaningless): "
-                         "for runs under a profiler, which records the kernels' durations itself")
-    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
-                    help="also launch a plain copy kernel of this many MiB three times (byte-counter calibration)")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); use --gpus 1")
-
-    wl = WORKLOADS[args.workload]
-    steps = args.steps if args.steps is not None else wl["steps"]
-    warmup = args.warmup if args.warmup is not None else wl["warmup"]
-    api = pf.load_product()
-    hip = api.hip
-    if hip.device_count() < 1:
-        sys.exit("no HIP device: the benchmark runs the HIP path only")
-    cfg = workloads.measured_config()
+def layer_config(wl):
     if wl.get("dims"):
         h, e, k, i, s_i, phys = wl["dims"]
-        cfg = abi.moe_config(h, e, k, i, s_i, down_physical=phys)
-    if args.workload == "q4k_stack48":
-        return run_stack(args, api, hip, cfg, steps, warmup)
-    if wl.get("hc"):
-        return run_hc(args, api, hip, cfg, wl, steps, warmup)
+        return abi.moe_config(h, e, k, i, s_i, down_physical=phys)
+    return workloads.measured_config()
+
+
+def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
+    """One MoE layer: decode batches or prefill chunks.  Returns the record."""
+    api, hip, tools = ctx
+    wl = WORKLOADS[name]
+    cfg = layer_config(wl)
     tokens = wl["tokens"]
     prefill = tokens > 4
     t0 = time.time()
@@ -388,47 +218,54 @@ def main():
         info = {"active_experts_chunk0": int(unique), "max_tokens_per_expert": int(load.max()),
                 "median_tokens_per_expert": float(np.median(load)), "chunks": n_inputs}
     elif tokens == 1:
-        n_inputs = max(1, min(steps, 10000))
+        n_inputs = max(1, min(steps, 2000))
         x, info = workloads.decode_tokens(weights, n_inputs, seed=args.seed)
         x = x.reshape(n_inputs, 1, cfg.hidden_size)
         unique = float(cfg.top_k)
     else:
-        n_inputs = max(1, min(steps, 2000))
+        n_inputs = max(1, min(steps, 1000))
         x, info = workloads.verify_batches(weights, n_inputs, seed=args.seed)
         unique = info["mean_unique_experts"]
     prep_s = time.time() - t0
 
     layer = pf.MoeLayer(api, cfg, weights, tokens)
     moe, work = layer.device_handles()     # the layer's HBM-resident tensors and scratch, for the timed loop
+    h = cfg.hidden_size
     d_x = hip.to_device(x)
-    d_y = hip.to_device(np.zeros((tokens, cfg.hidden_size), dtype=np.float32))
+    d_y = hip.to_device(np.zeros((tokens, h), dtype=np.float32))
 
-    ms = C.c_float()
-    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, warmup, C.byref(ms)), "warmup")
-    hip.check(hip.synchronize(), "sync")
     wall0 = time.perf_counter()
-    hip.check(hip.moe_time_forwards(moe, work, d_x, n_inputs, d_y, tokens, steps, C.byref(ms)), "timed loop")
-    hip.check(hip.synchronize(), "sync")
+    plan = tools.plan_moe([moe], [work], d_x, n_inputs, d_y, 1, tokens, steps, h)
+    timing = tools.timed(plan, steps, warmup)
+    tools.destroy(plan)
     wall_ms = (time.perf_counter() - wall0) * 1e3
-    ms_per_step = ms.value / steps
+    ms_per_step = timing["median"]
     us_per_token = ms_per_step * 1e3 / tokens
     err_word = hip.from_device(hip.work_error_word(work), (1,), np.uint32)[0]
     exact = C.c_uint32()
     hip.work_exact_rows(work, C.byref(exact))
 
-    # Per-kernel durations inside the dependent chain: graph replays of the first 1, 2, ...
-    # kernels (stages) of every forward, bracketed by HIP events on the launch stream; a
-    # stage's duration is the difference between consecutive replays (it includes the dispatch
-    # gap before it, as a profiler's start-to-end time of a dependent kernel does).
-    stage = (C.c_float * 4)()
-    if not args.skip_stages:
-        hip.check(hip.moe_profile_stages(moe, work, d_x, n_inputs, d_y, tokens, min(steps, 2000), stage), "stages")
+    # Per-kernel durations inside the dependent chain: the same plan with only the first 1, 2, ... kernel
+    # groups of every forward; a group's duration is the difference between consecutive plans (it includes
+    # the dispatch gap before it, as a profiler's start-to-end time of a dependent kernel does).
     family = hip.moe_kernel_family(moe, work, tokens)
     names = {0: GENERAL_STAGES, 1: DECODE_STAGES, 2: PREFILL_STAGES}[family]
-    stage_us = [max(float(stage[j]) * 1e3, 1e-3) for j in range(len(names))]
+    stage_us = [1e-3] * len(names)
+    if not args.skip_stages:
+        previous = 0.0
+        n_fw = min(steps, 512)
+        for j in range(len(names)):
+            if j + 1 < len(names):
+                plan = tools.plan_moe([moe], [work], d_x, n_inputs, d_y, 1, tokens, n_fw, h, kernel_limit=j + 1)
+                t = tools.timed(plan, n_fw, min(warmup, n_fw))["median"]
+                tools.destroy(plan)
+            else:
+                t = ms_per_step
+            stage_us[j] = max((t - previous) * 1e3, 1e-3)
+            previous = t
 
     lb = workloads.layer_bytes(wl["type"], cfg)
-    h, i, s_i, k = cfg.hidden_size, cfg.intermediate, cfg.shared_intermediate, cfg.top_k
+    i, s_i, k = cfg.intermediate, cfg.shared_intermediate, cfg.top_k
     extra = {}
     if prefill:
         # algorithmic bytes per launch: weights of the active experts once, activations once
@@ -461,11 +298,10 @@ def main():
     achieved = stage_bytes[dom] / (stage_us[dom] * 1e-6) / 1e9
 
     # CPU baseline and parity on a bounded sample of the same inputs
-    ref = load_reference()
-    cpu_api, kind = (ref, "reference") if ref is not None else (load_oracle(), "port")
-    per_token_guess = 0.55 if wl["type"] in (abi.GGUF_IQ2_XXS, "q2") else 0.32
+    cpu_api, kind = cpu_api_and_kind()
+    per_token_guess = 0.27 if wl["type"] in (abi.GGUF_IQ2_XXS, "q2") else 0.14
     if prefill:
-        sample_tokens = min(tokens, args.cpu_sample or 48)
+        sample_tokens = min(tokens, args.cpu_sample or max(4, int(cpu_seconds / per_token_guess)))
         with pf.MoeLayer(cpu_api, cfg, weights, sample_tokens) as cpu:
             c0 = time.perf_counter()
             cpu_out = [cpu.forward(x[0][:sample_tokens])[1:]]
@@ -474,7 +310,7 @@ def main():
         gpu_out = [(y[:sample_tokens], ids[:sample_tokens], w[:sample_tokens])]
         sample_text = f"first {sample_tokens} tokens of chunk 0 (the CPU cost is linear in tokens), {cpu_s:.1f} s"
     else:
-        sample = args.cpu_sample or max(1, int(15.0 / per_token_guess / tokens))
+        sample = args.cpu_sample or max(1, int(cpu_seconds / per_token_guess / tokens))
         sample = min(sample, n_inputs)
         sample_tokens = sample * tokens
         with pf.MoeLayer(cpu_api, cfg, weights, tokens) as cpu:
@@ -487,16 +323,22 @@ def main():
     max_abs = max(float(np.abs(g[0] - c[0]).max()) for g, c in zip(gpu_out, cpu_out))
     within = all((np.abs(g[0] - c[0]) <= 1e-3 + 1e-4 * np.abs(c[0])).all() for g, c in zip(gpu_out, cpu_out))
     layer.close()
+    hip.free(d_x)
+    hip.free(d_y)
     if args.copy_probe:
-        hip.check(hip.copy_probe(args.copy_probe << 20, 3), "copy probe")
+        tools.check(tools.lib.pf_bench_copy_probe(args.copy_probe << 20, 3), "copy probe")
 
+    traffic, traffic_from = measured_traffic(name)
     margins = "; top-11 logit margins >= 1e-3" if not prefill else ""
-    result = {
+    whole = alg_bytes / (ms_per_step * 1e-3) / 1e9
+    return {
         "metric": "moe_decode_us_per_layer_token" if not prefill else "moe_prefill_us_per_layer_token",
         "value": round(us_per_token, 3),
         "unit": "us/layer/token",
         "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 6),
+        "ms_per_step_p10_p90": [round(timing["p10"], 6), round(timing["p90"], 6)],
+        "timed_replays": timing["replays"], "timed_ms": round(timing["timed_ms"], 2),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32" if not prefill else "f16 products, f32 accumulation",
         "data": "synthetic",
@@ -505,12 +347,13 @@ def main():
                                f"{wl['label']}; {n_inputs} seeded inputs{margins}",
                    "tokens_per_step": tokens, "expert_format": FORMAT_LABEL[wl["type"]],
                    "unique_experts_per_step": unique, "inputs": info},
-        "hbm_GBps_on_algorithmic_bytes": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        "hbm_GBps_on_algorithmic_bytes": round(whole, 1),
+        "hbm_frac_whole_layer": round(whole / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": int(alg_bytes),
         "tokens_per_s": round(tokens / (ms_per_step * 1e-3), 1),
         "roofline": {"bound": "hbm", "kernel": names[dom], "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(args.workload),
+                     "traffic": traffic, "traffic_from": traffic_from,
                      "bytes_per_launch": int(stage_bytes[dom]), "us_per_launch": round(stage_us[dom], 3)},
         "kernel_us": dict(zip(names, [round(v, 3) for v in stage_us])),
         "kernel_bytes": dict(zip(names, [int(b) for b in stage_bytes])),
@@ -521,9 +364,283 @@ def main():
                              "max_abs_err": max_abs, "error_word": int(err_word), "serial_order_reroutes": int(exact.value)},
         "wall_ms_timed_loop": round(wall_ms, 2), "prep_s": round(prep_s, 1),
     }
-    print(json.dumps(result))
-    if not (ids_equal and within and err_word == 0):
-        sys.exit("parity check failed on the sample")
+
+
+def run_stack(args, ctx, steps, warmup, cpu_seconds):
+    """A stack of independent layers, all resident: every token (or chunk) passes the layers in order, each
+    layer with its own seeded input, hence its own routing.  The popularity bias sits in router column 0
+    (workloads.zipf_router): inputs with coordinate 0 = 1 see Zipf(1.1) popularity, with 0 the plain router."""
+    api, hip, tools = ctx
+    cfg = workloads.measured_config()
+    layers_n, chunk = args.layers, 2048
+    t0 = time.time()
+    layers, sample = [], None
+    for l in range(layers_n):
+        weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=args.seed * 1000 + l)
+        workloads.zipf_router(weights, seed=args.seed * 1000 + l, temperature=0.18)
+        layers.append(pf.MoeLayer(api, cfg, weights, chunk))
+        if l == 0:
+            sample = weights
+        else:
+            layers[-1].weights = None      # the library copied the bytes into HBM at create
+    prep_s = time.time() - t0
+    moes = [l.device_handles()[0] for l in layers]
+    works = [l.device_handles()[1] for l in layers]
+    resident = sum(hip.moe_bytes(m) for m in moes)
+    synth = pf.Synth()
+    h = cfg.hidden_size
+    per_layer_tokens = 8
+    dec = pf.rms_normalise(synth.normal((per_layer_tokens * layers_n, h), 77 + args.seed))
+    pre = synth.normal((4 * chunk, h), 78 + args.seed)
+    d_y = hip.to_device(np.zeros((chunk, h), dtype=np.float32))
+    out, spread = {}, {}
+    for name, coord in (("uniform", 0.0), ("zipf", 1.0)):
+        dec[:, 0] = coord
+        pre[:, 0] = coord
+        d_dec, d_pre = hip.to_device(dec), hip.to_device(pre)
+        plan = tools.plan_moe(moes, works, d_dec, len(dec), d_y, 1, 1, steps * layers_n, h)
+        t = tools.timed(plan, steps, warmup)        # per token through the stack
+        tools.destroy(plan)
+        out[name + "_decode_us_per_token"] = t["median"] * 1e3
+        spread[name + "_decode_us_p10_p90"] = [round(t["p10"] * 1e3, 2), round(t["p90"] * 1e3, 2)]
+        chunks = 2
+        plan = tools.plan_moe(moes, works, d_pre, 4, d_y, 1, chunk, chunks * layers_n, h)
+        t = tools.timed(plan, chunks, 1)
+        tools.destroy(plan)
+        out[name + "_prefill_ms_per_chunk"] = t["median"]
+        out[name + "_prefill_tokens_per_s"] = chunk / (t["median"] * 1e-3)
+        hip.free(d_dec)
+        hip.free(d_pre)
+    errors = sum(int(hip.from_device(hip.work_error_word(w), (1,), np.uint32)[0]) for w in works)
+    # parity and the CPU cost per layer-token on layer 0; the stack's CPU time is that times the layers
+    cpu_api, kind = cpu_api_and_kind()
+    n = args.cpu_sample or max(2, int(cpu_seconds / 0.14))
+    xs = dec[:n].copy()
+    with pf.MoeLayer(cpu_api, cfg, sample, n) as cpu:
+        c0 = time.perf_counter()
+        _, y0, ids0, _ = cpu.forward(xs)
+        cpu_s = time.perf_counter() - c0
+    _, y1, ids1, _ = layers[0].forward(xs)
+    ids_equal = bool((ids0 == ids1).all())
+    within = bool((np.abs(y1 - y0) <= 1e-3 + 1e-4 * np.abs(y0)).all())
+    for l in layers:
+        l.close()
+    hip.free(d_y)
+    us = out["uniform_decode_us_per_token"]
+    alg = layers_n * workloads.algorithmic_bytes_per_token(abi.GGUF_Q4_K)
+    return {
+        "metric": "moe_stack_decode_us_per_token", "value": round(us, 2), "unit": "us/token (all layers)",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(us * 1e-3, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{layers_n} independent MoE layers (hidden 2048, 512 experts, top-10, intermediate 512, "
+                               f"shared 512, Q4_K), {resident / 1e9:.1f} GB resident in HBM; decode batch 1 and "
+                               f"{chunk}-token prefill chunks; per-layer seeded inputs and routers",
+                   "layers": layers_n, "tokens_per_step": 1},
+        "us_per_layer_token": round(us / layers_n, 3),
+        "hbm_GBps_on_algorithmic_bytes": round(alg / (us * 1e-6) / 1e9, 1),
+        "algorithmic_bytes_per_step": int(alg),
+        "roofline": {"bound": "hbm", "kernel": "whole stack: three decode kernels per layer", "achieved":
+                     round(alg / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None},
+        "stack": {k: round(v, 3) for k, v in out.items()}, "stack_spread": spread,
+        "cpu_baseline": {"value": round(cpu_s / n * 1e6 * layers_n, 1), "unit": "us/token (all layers)", "cores": 1,
+                         "kind": kind, "sample": f"{n} tokens through layer 0 ({cpu_s:.1f} s), times {layers_n} layers: "
+                                                 "an extrapolation, the CPU cost is linear in layers and tokens"},
+        "parity_on_sample": {"ids_equal": ids_equal, "within_1e-3_abs_1e-4_rel": within, "error_word": errors},
+        "prep_s": round(prep_s, 1),
+    }
+
+
+def run_hc(args, ctx, name, steps, warmup, cpu_seconds):
+    """One layer between its two hyper-connection steps (src/qwen4_forward.c:362-367): per step a gated read
+    of [tokens, streams, hidden] normed streams and gate logits, the MoE block, and the injection of the
+    block's output into the [tokens, streams, hidden] residual.  Timed three ways on resident buffers: the
+    chain with the injection folded into the block's last kernel (`value`), the chain with the injection as
+    a kernel of its own, and the block alone on the same mixed rows."""
+    api, hip, tools = ctx
+    wl = WORKLOADS[name]
+    cfg = layer_config(wl)
+    tokens, streams, h = wl["tokens"], wl["hc"], cfg.hidden_size
+    t0 = time.time()
+    weights = pf.LayerWeights.synthetic(cfg, wl["type"], seed=args.seed)
+    if tokens > 4:
+        workloads.zipf_router(weights, seed=args.seed, temperature=0.18)
+    n_inputs = max(1, min(steps, 4 if tokens > 4 else 1000))
+    rng = np.random.default_rng(args.seed)
+    # streams whose gated mix has about unit RMS, as the block sees after the norm
+    normed = (rng.standard_normal((n_inputs, tokens, streams, h)) * (2.0 * streams ** 0.5 / 1.12)).astype(np.float32)
+    logits = rng.standard_normal((n_inputs, tokens, streams, h)).astype(np.float32)
+    residual = rng.standard_normal((tokens, streams, h)).astype(np.float32)
+    inject = rng.uniform(0.0, 2.0 / streams, (tokens, streams)).astype(np.float32)
+    # the timed loop adds into one residual many thousands of times: weights scaled down so that it stays small
+    inject_timed = inject * np.float32(1e-4)
+    prep_s = time.time() - t0
+    layer = pf.MoeLayer(api, cfg, weights, tokens)
+    moe, work = layer.device_handles()
+    d_n, d_g, d_i = hip.to_device(normed), hip.to_device(logits), hip.to_device(inject_timed)
+    d_r = hip.to_device(residual)
+    timed = {}
+    for label, fused in (("fused", 1), ("separate_add", 0)):
+        hip.check(hip.memcpy_h2d(d_r, residual.ctypes.data, residual.nbytes), "residual")
+        plan = tools.plan_hc(moe, work, d_n, d_g, n_inputs, d_r, d_i, streams, tokens, steps, fused, h)
+        timed[label] = tools.timed(plan, steps, warmup)
+        tools.destroy(plan)
+    err_word = int(hip.from_device(hip.work_error_word(work), (1,), np.uint32)[0])
+    # the block alone on the mixed rows the read produces
+    shape = abi.Qwen4HcShape(streams, h, 1, 1e-6)
+    mixed = np.empty((n_inputs, tokens, h), dtype=np.float32)
+    for b in range(n_inputs):
+        st = api.hc.read(C.byref(shape), abi.f32_cube(normed[b]), abi.f32_cube(logits[b]), abi.f32_view(mixed[b]), None)
+        assert st == abi.QW4_OK, st
+    d_x = hip.to_device(mixed)
+    d_y = hip.to_device(np.zeros((tokens, h), dtype=np.float32))
+    plan = tools.plan_moe([moe], [work], d_x, n_inputs, d_y, 1, tokens, steps, h)
+    block_ms = tools.timed(plan, steps, warmup)["median"]
+    tools.destroy(plan)
+
+    # the two hyper-connection kernels alone, HIP events on the launch stream around back-to-back launches
+    # (the add runs with zero weights so that the residual stays put over the launches)
+    d_zero = hip.to_device(np.zeros_like(inject))
+    d_err = hip.to_device(np.zeros(64, dtype=np.uint32))
+    kernel_us = {}
+    n_launch = max(50, min(steps, 1000))
+    ms = C.c_float()
+    for which, kname in ((0, "pf_k_hc_read"), (1, "pf_k_hc_add")):
+        for count in (10, n_launch):
+            tools.check(tools.lib.pf_bench_hc_time_step(which, d_n if which == 0 else d_r, d_g, d_x if which == 0 else d_y,
+                                                        d_zero, tokens, streams, h, count, d_err, C.byref(ms)), kname)
+        kernel_us[kname] = ms.value * 1e3 / n_launch
+    read_bytes = tokens * h * 4 * (2 * streams + 1)
+    add_bytes = tokens * h * 4 * (2 * streams + 1) + tokens * streams * 4
+    if args.copy_probe:
+        tools.check(tools.lib.pf_bench_copy_probe(args.copy_probe << 20, 3), "copy probe")
+
+    # parity on a bounded sample, stage by stage on identical inputs: CPU read against the device's mixed rows,
+    # CPU block on those rows, CPU add of its output; the device's chained call against that residual
+    cpu_api, kind = cpu_api_and_kind()
+    per_token = 0.27 if wl["type"] in (abi.GGUF_IQ2_XXS, "q2") else 0.14
+    sample = min(tokens, args.cpu_sample or max(2, int(cpu_seconds / per_token / 2)))
+    steps_cpu = 1 if tokens > 1 else min(sample, n_inputs)
+    rows = sample if tokens > 1 else 1
+    ids_equal = within = read_close = True
+    max_abs = 0.0
+    cpu_s = 0.0
+    with pf.MoeLayer(cpu_api, cfg, weights, rows) as cpu:
+        for b in range(steps_cpu):
+            n_b, g_b = normed[b][:rows], logits[b][:rows]
+            want = residual[:rows].copy()
+            c0 = time.perf_counter()
+            _, ids_c, _ = cpu.forward_hc(n_b, g_b, want, inject[:rows], fused=False)
+            cpu_s += time.perf_counter() - c0
+            # the same chain with the CPU block fed the device's mixed rows (identical inputs to every stage)
+            _, y_c, ids_m, _ = cpu.forward(mixed[b][:rows])
+            want_m = residual[:rows].copy()
+            cpu_api.hc.add(C.byref(shape), abi.f32_cube(want_m), abi.f32_view(y_c), abi.f32_view(inject[:rows]), None)
+            got = residual.copy()
+            _, ids_g, _ = layer.forward_hc(normed[b], logits[b], got, inject)
+            ids_equal &= bool((ids_g[:rows] == ids_m).all())
+            bound = np.abs(inject[:rows])[:, :, None] * (1e-3 + 1e-4 * np.abs(y_c)[:, None, :]) + 1e-6 * np.abs(want_m)
+            within &= bool((np.abs(got[:rows] - want_m) <= bound).all())
+            max_abs = max(max_abs, float(np.abs(got[:rows] - want_m).max()))
+            read_close &= bool(np.allclose(want, want_m, atol=1e-5, rtol=1e-5))
+    layer.close()
+    sample_tokens = steps_cpu * rows
+    ms_per_step = timed["fused"]["median"]
+    hc_bytes = tokens * h * 4 * (2 * streams + 1) + tokens * h * 4 * 2 * streams   # read in/out, residual in/out
+    traffic, traffic_from = measured_traffic(name)
+    return {
+        "metric": "moe_hc_block_us_per_layer_token", "value": round(ms_per_step * 1e3 / tokens, 3),
+        "unit": "us/layer/token", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
+        "ms_per_step_p10_p90": [round(timed["fused"]["p10"], 6), round(timed["fused"]["p90"], 6)],
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32" if tokens <= 4 else "f16 products, f32 accumulation", "data": "synthetic",
+        "config": {"workload": f"one MoE layer, hidden {cfg.hidden_size}, {cfg.experts} experts, top-{cfg.top_k}, "
+                               f"intermediate {cfg.intermediate}, shared {cfg.shared_intermediate}; "
+                               f"{wl['label']}; {n_inputs} seeded inputs",
+                   "tokens_per_step": tokens, "streams": streams,
+                   "expert_format": FORMAT_LABEL[wl["type"]]},
+        "chain_us_per_step": {"read + block with the add folded in": round(timed["fused"]["median"] * 1e3, 3),
+                              "read + block + add kernel": round(timed["separate_add"]["median"] * 1e3, 3),
+                              "block alone": round(block_ms * 1e3, 3)},
+        "hc_bytes_per_step": int(hc_bytes),
+        "kernel_us": {k: round(v, 3) for k, v in kernel_us.items()},
+        "kernel_bytes": {"pf_k_hc_read": int(read_bytes), "pf_k_hc_add": int(add_bytes)},
+        "kernel_GBps": {"pf_k_hc_read": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9, 1),
+                        "pf_k_hc_add": round(add_bytes / (kernel_us["pf_k_hc_add"] * 1e-6) / 1e9, 1)},
+        "roofline": {"bound": "hbm", "kernel": "pf_k_hc_read (gated mix of the residual streams)",
+                     "achieved": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(read_bytes / (kernel_us["pf_k_hc_read"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": traffic, "traffic_from": traffic_from, "bytes_per_launch": int(read_bytes),
+                     "us_per_launch": round(kernel_us["pf_k_hc_read"], 3)},
+        "cpu_baseline": {"value": round(cpu_s / sample_tokens * 1e6, 1), "unit": "us/layer/token", "cores": 1,
+                         "kind": kind, "sample": f"{sample_tokens} tokens of the same inputs through read, block and add, "
+                                                 f"{cpu_s:.1f} s"},
+        "parity_on_sample": {"ids_equal": ids_equal, "residual_within_block_tolerance_times_inject": within,
+                             "cpu_read_vs_device_read_chain_close": read_close, "max_abs_err": max_abs,
+                             "error_word": err_word},
+        "prep_s": round(prep_s, 1),
+    }
+
+
+def run_one(args, ctx, name, cpu_seconds):
+    wl = WORKLOADS[name]
+    steps = args.steps if args.steps is not None else wl["steps"]
+    warmup = args.warmup if args.warmup is not None else wl["warmup"]
+    if name == "q4k_stack48":
+        return run_stack(args, ctx, min(steps, 200), warmup, cpu_seconds)
+    if wl.get("hc"):
+        return run_hc(args, ctx, name, steps, warmup, cpu_seconds)
+    return run_layer(args, ctx, name, steps, warmup, cpu_seconds)
+
+
+def parity_ok(record):
+    p = record["parity_on_sample"]
+    return all(v for v in p.values() if isinstance(v, bool)) and p.get("error_word", 0) == 0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default="all", choices=["all"] + sorted(WORKLOADS))
+    ap.add_argument("--cpu-sample", type=int, default=None, help="tokens timed on the CPU path (default: 10 s of work for "
+                    "the headline, 3 s for each further configuration)")
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--layers", type=int, default=48, help="layers of the q4k_stack48 workload")
+    ap.add_argument("--no-stack", action="store_true", help="with --workload all: leave out the 48-layer stack")
+    ap.add_argument("--skip-stages", action="store_true",
+                    help="leave out the per-kernel timing by cut-off replays (kernel_us is then meaningless): for runs "
+                         "under a profiler, which records the kernels' durations itself")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="also launch a plain copy kernel of this many MiB three times (byte-counter calibration)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); use --gpus 1")
+
+    api = pf.load_product()
+    hip = api.hip
+    if hip.device_count() < 1:
+        sys.exit("no HIP device: the benchmark runs the HIP path only")
+    ctx = (api, hip, Tools())
+    if args.workload != "all":
+        record = run_one(args, ctx, args.workload, 12.0)
+        print(json.dumps(record))
+        if not parity_ok(record):
+            sys.exit("parity check failed on the sample")
+        return
+    record = run_one(args, ctx, HEADLINE, 10.0)
+    record["configs"] = {}
+    for name in ALL_CONFIGS:
+        if name == "q4k_stack48" and args.no_stack:
+            continue
+        print(f"[bench] {name} ...", file=sys.stderr, flush=True)
+        record["configs"][name] = run_one(args, ctx, name, 3.0)
+    print(json.dumps(record))
+    bad = [n for n, r in [(HEADLINE, record)] + list(record["configs"].items()) if not parity_ok(r)]
+    if bad:
+        sys.exit(f"parity check failed on the sample: {bad}")
 
 
 if __name__ == "__main__":

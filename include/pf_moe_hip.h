@@ -101,6 +101,12 @@ int pf_hip_work_clear_status(PfHipWork *work);
  * specialised decode kernels. */
 void pf_hip_work_force_general(PfHipWork *work, int on);
 
+/* Diagnostics: every later forward on this workspace enqueues only the first `count` of its
+ * dependent kernel groups (decode path: its three kernels; other paths: four groups; 0 = all;
+ * results are then incomplete).  A measuring program times the chain cut after 1, 2, ... groups
+ * and takes differences; nothing in the library calls it. */
+void pf_hip_work_limit_kernels(PfHipWork *work, int count);
+
 /* Host-buffer forward used by qwen4_moe_forward: copies x in, runs the forward,
  * copies y (and ids/weights when non-NULL) out, returns the error word.  Pitches
  * in bytes.  Outputs are written only when the error word is zero. */
@@ -181,59 +187,12 @@ int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_bytes, size
 int pf_hip_packed_decode_row_host(uint32_t gguf_type, const void *row_bytes_ptr, size_t row_bytes,
                                   size_t k_storage, float *out, uint32_t *error_word);
 
-/* Minimal device-memory and timing helpers so that a host program can keep
- * inputs resident and time launches with events on the launch stream. */
+/* Minimal device-memory helpers so that a host program can keep inputs resident. */
 int pf_hip_malloc(void **d_ptr, size_t bytes);
 void pf_hip_free(void *d_ptr);
 int pf_hip_memcpy_h2d(void *d_dst, const void *src, size_t bytes);
 int pf_hip_memcpy_d2h(void *dst, const void *d_src, size_t bytes);
 int pf_hip_synchronize(void);
-/* Runs `iters` forwards back to back on one stream, input row block i % n_inputs
- * of d_x each time, and returns the elapsed milliseconds between two events
- * recorded on that stream around the launches. */
-int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
-                             size_t n_inputs, float *d_y, size_t tokens, size_t iters,
-                             float *elapsed_ms);
-
-/* The block between its two hyper-connection steps, `iters` times: input block
- * i % n_inputs of d_normed / d_logits (dense [tokens, streams, hidden] each) and one
- * residual cube.  fused != 0 runs pf_hip_moe_forward_hc_device; fused == 0 runs the
- * read, a forward into the workspace and the add as three enqueues. */
-int pf_hip_moe_time_forwards_hc(const PfHipMoe *moe, PfHipWork *work, const float *d_normed,
-                                const float *d_logits, size_t n_inputs, float *d_residual,
-                                const float *d_inject, size_t streams, size_t tokens,
-                                size_t iters, int fused, float *elapsed_ms);
-
-/* One of the two hyper-connection kernels alone, `iters` launches back to back between
- * two events on the launch stream.  which 0: the read of d_cube (normed) and d_logits,
- * dense [tokens, streams, hidden], into d_rows [tokens, hidden]; which 1: the add of
- * d_rows into d_cube with weights d_inject [tokens, streams]. */
-int pf_hip_hc_time_step(int which, float *d_cube, const float *d_logits, float *d_rows,
-                        const float *d_inject, size_t tokens, size_t streams, size_t hidden,
-                        size_t iters, uint32_t *d_error_word, float *elapsed_ms);
-
-/* The same for a stack of layers of equal hidden size (works[l] belongs to moes[l]):
- * forward i runs through layer i % layers with input row block i % n_inputs, so
- * `iters` = tokens-through-the-stack x layers. */
-int pf_hip_stack_time_forwards(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers,
-                               const float *d_x, size_t n_inputs, float *d_y, size_t tokens,
-                               size_t iters, float *elapsed_ms);
-
-/* Average duration of each kernel inside the dependent chain: the same loop run
- * with only the first 1, 2, ... kernels of every forward launched; stage_ms[j] is
- * the difference between consecutive runs divided by iters.  Decode path (1..4
- * tokens, supported shapes): [0] router logits, [1] routing + gate/up, [2] down +
- * combine, [3] zero.  General path: [0] router + shared gate/up, [1] routing,
- * [2] routed gate/up, [3] down + combine. */
-int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x,
-                              size_t n_inputs, float *d_y, size_t tokens, size_t iters,
-                              float stage_ms[4]);
-
-/* Launches a plain device-to-device copy kernel (pf_k_copy_probe) of `bytes` bytes
- * `launches` times: a kernel of known traffic (bytes read, bytes written) against
- * which hardware byte counters read under a profiler can be scaled. */
-int pf_hip_copy_probe(size_t bytes, size_t launches);
-
 #ifdef __cplusplus
 }
 #endif

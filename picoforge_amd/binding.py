@@ -127,6 +127,7 @@ class HipShim:
         bind("pf_hip_work_exact_rows", C.c_int, vp, u32p)
         bind("pf_hip_work_clear_status", C.c_int, vp)
         bind("pf_hip_work_force_general", None, vp, C.c_int)
+        bind("pf_hip_work_limit_kernels", None, vp, C.c_int)
         bind("pf_hip_moe_forward_host", C.c_int, vp, vp, vp, sz, vp, sz, vp, sz, vp, sz, sz, u32p)
         bind("pf_hip_route_host", C.c_int, vp, sz, sz, sz, C.c_int, vp, vp, vp, u32p, P(C.c_uint64))
         bind("pf_hip_group_pairs_host", C.c_int, vp, sz, sz, sz, vp, vp, vp, u32p, P(C.c_int))
@@ -137,18 +138,12 @@ class HipShim:
         bind("pf_hip_memcpy_h2d", C.c_int, vp, vp, sz)
         bind("pf_hip_memcpy_d2h", C.c_int, vp, vp, sz)
         bind("pf_hip_synchronize", C.c_int)
-        bind("pf_hip_moe_time_forwards", C.c_int, vp, vp, vp, sz, vp, sz, sz, P(C.c_float))
-        bind("pf_hip_moe_profile_stages", C.c_int, vp, vp, vp, sz, vp, sz, sz, P(C.c_float))
-        bind("pf_hip_stack_time_forwards", C.c_int, P(vp), P(vp), sz, vp, sz, vp, sz, sz, P(C.c_float))
-        bind("pf_hip_copy_probe", C.c_int, sz, sz)
         bind("pf_hip_moe_kernel_family", C.c_int, vp, vp, sz)
         bind("pf_hip_hc_read_device", C.c_int, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_hc_add_device", C.c_int, vp, sz, sz, vp, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_moe_forward_hc_device", C.c_int, vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp)
         bind("pf_hip_hc_read_host", C.c_int, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, u32p)
         bind("pf_hip_hc_add_host", C.c_int, vp, sz, sz, vp, sz, vp, sz, sz, sz, sz, u32p)
-        bind("pf_hip_hc_time_step", C.c_int, C.c_int, vp, vp, vp, vp, sz, sz, sz, sz, vp, P(C.c_float))
-        bind("pf_hip_moe_time_forwards_hc", C.c_int, vp, vp, vp, vp, sz, vp, vp, sz, sz, sz, C.c_int, P(C.c_float))
 
     def check(self, rc, what):
         if rc != 0:

@@ -436,17 +436,8 @@ extern "C" int pf_hip_work_clear_status(PfHipWork *w) {
     return PF_HIP_OK;
 }
 
-// Instrumented builds only (-DPF_TIMING=<workgroup>): the decode kernels leave wall_clock64
-// stamps of their phases behind the re-route counter; this reads them back.
-#ifdef PF_TIMING
-extern "C" int pf_hip_debug_read(PfHipWork *w, void *out, size_t bytes) {
-    HIP_TRY(hipDeviceSynchronize());
-    HIP_TRY(hipMemcpy(out, w->exact_rows, bytes, hipMemcpyDeviceToHost));
-    return PF_HIP_OK;
-}
-#endif
-
 extern "C" void pf_hip_work_force_general(PfHipWork *w, int on) { if (w) w->force_general = on; }
+extern "C" void pf_hip_work_limit_kernels(PfHipWork *w, int count) { if (w) w->stage_limit = count > 0 ? count : 0; }
 
 static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x, size_t x_pitch, float *d_y,
                               size_t y_pitch) {
@@ -933,184 +924,4 @@ extern "C" int pf_hip_memcpy_d2h(void *dst, const void *d_src, size_t bytes) {
 extern "C" int pf_hip_synchronize(void) {
     HIP_TRY(hipDeviceSynchronize());
     return PF_HIP_OK;
-}
-
-// `iters` forwards back to back on one stream.  The launches are captured into graphs of
-// up to 256 forwards (each with its own input block) and the graphs are replayed in order,
-// so the measured gap between dependent kernels is the device's, not the host's enqueue rate.
-// Forward i goes through layer i % layers (a stack of layers in order, token after token).
-template <typename Enqueue>
-static int time_graph_replay_of(PfHipWork *const *works, size_t layers, size_t iters, int stage_limit,
-                                float *elapsed_ms, Enqueue enqueue) {
-    *elapsed_ms = 0.0f;
-    if (!iters) return PF_HIP_OK;
-    const size_t chunk = 256, n_graphs = (iters + chunk - 1) / chunk;
-    hipStream_t s = nullptr;
-    hipEvent_t t0 = nullptr, t1 = nullptr;
-    HIP_TRY(hipStreamCreate(&s));
-    hipGraphExec_t *execs = (hipGraphExec_t *)calloc(n_graphs, sizeof *execs);
-    int rc = execs ? PF_HIP_OK : PF_HIP_E_MEMORY;
-    for (size_t l = 0; l < layers; l++) works[l]->stage_limit = stage_limit;
-    for (size_t g = 0; g < n_graphs && rc == PF_HIP_OK; g++) {
-        hipGraph_t graph = nullptr;
-        if (hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal) != hipSuccess) { rc = PF_HIP_E_RUNTIME; break; }
-        for (size_t i = g * chunk; i < iters && i < (g + 1) * chunk && rc == PF_HIP_OK; i++)
-            rc = enqueue(i, s);
-        hipError_t e = hipStreamEndCapture(s, &graph);
-        if (e != hipSuccess && rc == PF_HIP_OK) { pf_set_error("hipStreamEndCapture", e); rc = PF_HIP_E_RUNTIME; }
-        if (rc == PF_HIP_OK && hipGraphInstantiate(&execs[g], graph, nullptr, nullptr, 0) != hipSuccess)
-            rc = PF_HIP_E_RUNTIME;
-        if (graph) (void)hipGraphDestroy(graph);
-    }
-    for (size_t l = 0; l < layers; l++) works[l]->stage_limit = 0;
-    if (rc == PF_HIP_OK && (hipEventCreate(&t0) != hipSuccess || hipEventCreate(&t1) != hipSuccess)) rc = PF_HIP_E_RUNTIME;
-    if (rc == PF_HIP_OK) {
-        hipError_t e = hipEventRecord(t0, s);
-        for (size_t g = 0; g < n_graphs && e == hipSuccess; g++) e = hipGraphLaunch(execs[g], s);
-        if (e == hipSuccess) e = hipEventRecord(t1, s);
-        if (e == hipSuccess) e = hipStreamSynchronize(s);
-        if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
-        if (e != hipSuccess) { pf_set_error("timed graph replay", e); rc = PF_HIP_E_RUNTIME; }
-    }
-    for (size_t g = 0; execs && g < n_graphs; g++) if (execs[g]) (void)hipGraphExecDestroy(execs[g]);
-    free(execs);
-    if (t0) (void)hipEventDestroy(t0);
-    if (t1) (void)hipEventDestroy(t1);
-    (void)hipStreamDestroy(s);
-    return rc;
-}
-
-static int time_graph_replay(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers, const float *d_x,
-                             size_t n_inputs, float *d_y, size_t tokens, size_t iters, int stage_limit, float *elapsed_ms) {
-    const size_t H = moes[0]->desc.hidden;
-    return time_graph_replay_of(works, layers, iters, stage_limit, elapsed_ms, [&](size_t i, hipStream_t s) {
-        return pf_hip_moe_forward_device(moes[i % layers], works[i % layers], d_x + (i % n_inputs) * tokens * H, H, d_y, H,
-                                         tokens, s);
-    });
-}
-
-// The block between its two hyper-connection steps, `iters` times back to back: input block
-// i % n_inputs of d_normed / d_logits (dense [tokens, streams, hidden] each), one residual cube.
-// fused != 0: read, then a forward whose last kernel adds into the residual.  fused == 0: read,
-// forward into the workspace's output rows, then the add as a kernel of its own.
-extern "C" int pf_hip_moe_time_forwards_hc(const PfHipMoe *moe, PfHipWork *work, const float *d_normed,
-                                           const float *d_logits, size_t n_inputs, float *d_residual,
-                                           const float *d_inject, size_t streams, size_t tokens, size_t iters,
-                                           int fused, float *elapsed_ms) {
-    if (!moe || !work || work->moe != moe || !d_normed || !d_logits || !d_residual || !d_inject || !n_inputs ||
-        !elapsed_ms || !streams || tokens > work->cap)
-        return PF_HIP_E_ARGUMENT;
-    const size_t H = moe->desc.hidden, cube = tokens * streams * H;
-    return time_graph_replay_of(&work, 1, iters, 0, elapsed_ms, [&](size_t i, hipStream_t s) {
-        const float *n = d_normed + (i % n_inputs) * cube, *g = d_logits + (i % n_inputs) * cube;
-        if (fused)
-            return pf_hip_moe_forward_hc_device(moe, work, n, streams * H, H, g, streams * H, H, d_residual,
-                                                streams * H, H, d_inject, streams, tokens, s);
-        int rc = pf_hip_hc_read_device(n, streams * H, H, g, streams * H, H, work->x, H, tokens, streams, H,
-                                       work->error_word, s);
-        if (rc == PF_HIP_OK) rc = pf_hip_moe_forward_device(moe, work, work->x, H, work->y, H, tokens, s);
-        if (rc == PF_HIP_OK)
-            rc = pf_hip_hc_add_device(d_residual, streams * H, H, work->y, H, d_inject, streams, tokens, streams, H,
-                                      work->error_word, s);
-        return rc;
-    });
-}
-
-// One of the two hyper-connection kernels alone, `iters` launches back to back on a stream of its own,
-// bracketed by two events on that stream.  which 0: the read (dense inputs, output into d_rows);
-// which 1: the add of d_rows into d_cube (dense), weights d_inject.
-extern "C" int pf_hip_hc_time_step(int which, float *d_cube, const float *d_logits, float *d_rows,
-                                   const float *d_inject, size_t tokens, size_t streams, size_t hidden, size_t iters,
-                                   uint32_t *d_error_word, float *elapsed_ms) {
-    if (!d_cube || !d_rows || !elapsed_ms || !d_error_word || !hc_dims_ok(tokens, streams, hidden) || !tokens ||
-        (which == 0 ? !d_logits : !d_inject))
-        return PF_HIP_E_ARGUMENT;
-    hipStream_t s = nullptr;
-    hipEvent_t t0 = nullptr, t1 = nullptr;
-    HIP_TRY(hipStreamCreate(&s));
-    hipError_t e = hipEventCreate(&t0);
-    if (e == hipSuccess) e = hipEventCreate(&t1);
-    if (e == hipSuccess) e = hipEventRecord(t0, s);
-    for (size_t i = 0; i < iters && e == hipSuccess; i++) {
-        if (which == 0)
-            pf_launch_hc_read(d_cube, streams * hidden, hidden, d_logits, streams * hidden, hidden, d_rows, hidden,
-                              (int)tokens, (int)streams, (int)hidden, d_error_word, s);
-        else
-            pf_launch_hc_add(d_cube, streams * hidden, hidden, d_rows, hidden, d_inject, streams, (int)tokens,
-                             (int)streams, (int)hidden, d_error_word, s);
-        e = hipGetLastError();
-    }
-    if (e == hipSuccess) e = hipEventRecord(t1, s);
-    if (e == hipSuccess) e = hipStreamSynchronize(s);
-    if (e == hipSuccess) e = hipEventElapsedTime(elapsed_ms, t0, t1);
-    if (t0) (void)hipEventDestroy(t0);
-    if (t1) (void)hipEventDestroy(t1);
-    (void)hipStreamDestroy(s);
-    if (e != hipSuccess) { pf_set_error("timed hyper-connection kernel", e); return PF_HIP_E_RUNTIME; }
-    return PF_HIP_OK;
-}
-
-extern "C" int pf_hip_moe_time_forwards(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
-                                        float *d_y, size_t tokens, size_t iters, float *elapsed_ms) {
-    if (!moe || !work || work->moe != moe || tokens > work->cap || !d_x || !d_y || !n_inputs || !elapsed_ms)
-        return PF_HIP_E_ARGUMENT;
-    return time_graph_replay(&moe, &work, 1, d_x, n_inputs, d_y, tokens, iters, 0, elapsed_ms);
-}
-
-extern "C" int pf_hip_stack_time_forwards(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers,
-                                          const float *d_x, size_t n_inputs, float *d_y, size_t tokens, size_t iters,
-                                          float *elapsed_ms) {
-    if (!moes || !works || !layers || !d_x || !d_y || !n_inputs || !elapsed_ms) return PF_HIP_E_ARGUMENT;
-    for (size_t l = 0; l < layers; l++)
-        if (!moes[l] || !works[l] || works[l]->moe != moes[l] || moes[l]->desc.hidden != moes[0]->desc.hidden)
-            return PF_HIP_E_ARGUMENT;
-    return time_graph_replay(moes, works, layers, d_x, n_inputs, d_y, tokens, iters, 0, elapsed_ms);
-}
-
-// Kernel durations inside the dependent chain: the same graph replay with only the first
-// 1, 2, ... kernels of every forward launched; stage j's time is the difference between
-// the runs with j + 1 and with j kernels, divided by the forwards.  HIP events on the launch
-// stream bracket each replay.  The decode path has three kernels, the general path four
-// launches (the third being the routing pair); unused entries are zero.
-extern "C" int pf_hip_moe_profile_stages(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t n_inputs,
-                                         float *d_y, size_t tokens, size_t iters, float stage_ms[4]) {
-    if (!moe || !work || work->moe != moe || tokens > work->cap || !d_x || !d_y || !n_inputs || !stage_ms || !iters)
-        return PF_HIP_E_ARGUMENT;
-    const int stages = pf_hip_moe_kernel_family(moe, work, tokens) == 1 ? 3 : 4;
-    float previous = 0.0f;
-    for (int j = 0; j < 4; j++) stage_ms[j] = 0.0f;
-    for (int j = 0; j < stages; j++) {
-        float warm = 0.0f, ms = 0.0f;
-        int rc = time_graph_replay(&moe, &work, 1, d_x, n_inputs, d_y, tokens, iters < 64 ? iters : 64, j + 1, &warm);
-        if (rc == PF_HIP_OK) rc = time_graph_replay(&moe, &work, 1, d_x, n_inputs, d_y, tokens, iters, j + 1, &ms);
-        if (rc != PF_HIP_OK) return rc;
-        stage_ms[j] = (ms - previous) / (float)iters;
-        previous = ms;
-    }
-    return PF_HIP_OK;
-}
-
-
-
-// A plain copy of a known size: the reference point for hardware byte counters, which a
-// profiler reads in units that are easiest to pin against a kernel whose traffic is known.
-__global__ void pf_k_copy_probe(const uint4 *src, uint4 *dst, size_t count) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
-        dst[i] = src[i];
-}
-
-extern "C" int pf_hip_copy_probe(size_t bytes, size_t launches) {
-    if (need_device()) return PF_HIP_E_NO_DEVICE;
-    bytes &= ~(size_t)15;
-    if (!bytes || !launches) return PF_HIP_E_ARGUMENT;
-    uint4 *src = nullptr, *dst = nullptr;
-    int rc = PF_HIP_OK;
-    if (hipMalloc((void **)&src, bytes) != hipSuccess || hipMalloc((void **)&dst, bytes) != hipSuccess) rc = PF_HIP_E_MEMORY;
-    if (rc == PF_HIP_OK && hipMemset(src, 1, bytes) != hipSuccess) rc = PF_HIP_E_RUNTIME;
-    for (size_t i = 0; i < launches && rc == PF_HIP_OK; i++)
-        hipLaunchKernelGGL(pf_k_copy_probe, dim3(2048), dim3(256), 0, nullptr, src, dst, bytes / 16);
-    if (rc == PF_HIP_OK && hipDeviceSynchronize() != hipSuccess) rc = PF_HIP_E_RUNTIME;
-    if (src) (void)hipFree(src);
-    if (dst) (void)hipFree(dst);
-    return rc;
 }

@@ -141,6 +141,5 @@ def test_shim_entry_points_refuse_bad_arguments_before_touching_a_device():
     assert hip.moe_forward_hc_device(None, None, p, 8, 4, p, 8, 4, p, 8, 4, p, 2, 1, None) == 1
     assert hip.moe_forward_device(None, None, p, 4, p, 4, 1, None) == 1
     assert hip.moe_kernel_family(None, None, 1) == 0
-    assert hip.hc_time_step(0, None, p, p, p, 1, 2, 4, 1, p, C.byref(ms)) == 1
     assert hip.hc_read_host(None, 32, 16, p, 32, 16, p, 16, 1, 2, 4, C.byref(word)) == 1
     assert hip.hc_read_host(p, 32, 16, p, 32, 16, p, 16, 0, 2, 4, C.byref(word)) == 0

@@ -76,6 +76,45 @@ def test_q4k_verify_batches_share_experts(product, oracle):
             print(f"  batch {b}: {len(set(ids0.reshape(-1)))} unique experts, tokens 0/1 share {shared}, max abs err {worst:.2e}", flush=True)
 
 
+def test_stack_of_independent_layers(product, oracle):
+    """Four resident Q4_K layers driven like the 48-layer benchmark: one captured sequence of forwards,
+    forward i through layer i % 4 with its own seeded input; every layer's last output against the oracle."""
+    from bench import Tools
+    tools, hip = Tools(), product.hip
+    cfg = workloads.measured_config()
+    n_layers, rounds = 4, 2
+    layers, all_weights = [], []
+    for l in range(n_layers):
+        weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=1000 + l)
+        workloads.zipf_router(weights, seed=1000 + l, temperature=0.18)
+        layers.append(pf.MoeLayer(product, cfg, weights, 4))
+        all_weights.append(weights)
+    h = cfg.hidden_size
+    x = pf.rms_normalise(pf.Synth().normal((rounds * n_layers, h), 79))
+    x[:, 0] = 1.0                                             # the Zipf bias input
+    moes = [l.device_handles()[0] for l in layers]
+    works = [l.device_handles()[1] for l in layers]
+    d_x = hip.to_device(x)
+    d_y = hip.to_device(np.full((n_layers, h), -99.0, dtype=np.float32))
+    plan = tools.plan_moe(moes, works, d_x, len(x), d_y, n_layers, 1, rounds * n_layers, h)
+    tools.run(plan, 2)
+    tools.destroy(plan)
+    y = hip.from_device(d_y, (n_layers, h), np.float32)
+    for l in (0, n_layers - 1):                               # forward i = layer i % 4; the last round's input stays
+        token = x[(rounds - 1) * n_layers + l][None, :]
+        ids = hip.from_device(hip.work_ids(works[l]), (1, cfg.top_k), np.uint32)
+        w = hip.from_device(hip.work_route_weights(works[l]), (1, cfg.top_k), np.float32)
+        assert int(hip.from_device(hip.work_error_word(works[l]), (1,), np.uint32)[0]) == 0
+        with pf.MoeLayer(oracle, cfg, all_weights[l], 1) as cpu:
+            _, y0, ids0, w0 = cpu.forward(token)
+        worst = assert_parity(y[l][None, :], ids, w, y0, ids0, w0, label=f"stack layer {l}")
+        print(f"  layer {l}: max abs err {worst:.2e}", flush=True)
+    hip.free(d_x)
+    hip.free(d_y)
+    for l in layers:
+        l.close()
+
+
 def test_views_over_released_weight_bytes(product, oracle):
     """qwen4_moe_forward refuses views that overlap the bytes the layer was created from (the
     reference's rule); after pf_moe_forget_host_weights the addresses are free for reuse."""

@@ -221,8 +221,10 @@ def test_chained_forward_validation_and_errors(product):
 
 
 def test_device_resident_chain_accumulates_like_the_host_calls(product):
-    """pf_hip_moe_forward_hc_device enqueued three times on device buffers (through the timing entry
-    point, which replays it in a graph) adds the same bits as three host-buffer calls, fused or not."""
+    """pf_hip_moe_forward_hc_device enqueued three times on device buffers (through the benchmark's plan,
+    which replays it from a HIP graph) adds the same bits as three host-buffer calls, fused or not."""
+    from bench import Tools
+    tools = Tools()
     cfg = abi.moe_config(512, 32, 6, 256, 256)
     weights, _ = make_layer_inputs(cfg, abi.GGUF_Q4_K, 1, seed=8)
     hip = product.hip
@@ -236,9 +238,9 @@ def test_device_resident_chain_accumulates_like_the_host_calls(product):
             d_n, d_g, d_i = hip.to_device(normed), hip.to_device(logits), hip.to_device(inject)
             for fused in (1, 0):
                 d_r = hip.to_device(residual)
-                ms = C.c_float()
-                hip.check(hip.moe_time_forwards_hc(moe, work, d_n, d_g, 1, d_r, d_i, 4, tokens, 3, fused, C.byref(ms)),
-                          "time_forwards_hc")
+                plan = tools.plan_hc(moe, work, d_n, d_g, 1, d_r, d_i, 4, tokens, 3, fused, cfg.hidden_size)
+                tools.run(plan, 1)
+                tools.destroy(plan)
                 got = hip.from_device(d_r, residual.shape, np.float32)
                 hip.free(d_r)
                 np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32),
