@@ -305,7 +305,7 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
 extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_bytes : 0; }
 
 // workspace layout: buffers carved from one allocation, each 256-byte aligned
-enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS,
+enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS, W_XIMG, W_AIMG,
        W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
        W_P2R, W_R2P, W_GROUPBAD, W_TILES, W_COUNT };
 struct Carve { size_t offset[W_COUNT], total; };
@@ -328,6 +328,11 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_ERR] = 256;
     want[W_EXACT] = 256;
     want[W_FLAGS] = (T + 1) * 4;
+    {   // digit images of the decode path: the token rows; the activation rows of every (unique expert, token) and the shared expert's
+        const size_t widest = I > d->shared_inter ? I : d->shared_inter;
+        want[W_XIMG] = Td * pf_image2_words(H) * 4;
+        want[W_AIMG] = (Td * K * Td + Td) * pf_image2_words(widest) * 4;
+    }
     // prefill path: fp16 copies, per-row scales, down products in expert order, grouping tables
     const bool prefill = T > PF_DECODE_MAX_TOKENS && pf_prefill_supported(*d);
     const size_t Tp = prefill ? T : 0, Is = d->shared_inter;
@@ -394,6 +399,8 @@ static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base) {
     w->error_word = (uint32_t *)(base + c.offset[W_ERR]);
     w->exact_rows = (uint32_t *)(base + c.offset[W_EXACT]);
     w->route_flags = (uint32_t *)(base + c.offset[W_FLAGS]);
+    w->ximg = (uint32_t *)(base + c.offset[W_XIMG]);
+    w->aimg = (uint32_t *)(base + c.offset[W_AIMG]);
     if (c.offset[W_GROUPBAD] != c.offset[W_X16]) {   // the prefill buffers were planned
         w->x16 = (uint16_t *)(base + c.offset[W_X16]);
         w->act16 = (uint16_t *)(base + c.offset[W_ACT16]);
@@ -462,6 +469,7 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.logits = w->logits; a.logit_ssq = w->logit_ssq; a.ids = w->ids; a.route_weights = w->route_weights;
     a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale;
     a.uniq = w->uniq;
+    a.ximg = w->ximg; a.aimg = w->aimg;
     a.error_word = w->error_word; a.exact_rows = w->exact_rows; a.route_flags = w->route_flags;
     a.x16 = w->x16; a.act16 = w->act16; a.sact16 = w->sact16;
     a.x_scale = w->x_scale; a.act_scale = w->act_scale; a.sact_scale = w->sact_scale; a.x_max2 = w->x_max2;

@@ -103,46 +103,96 @@ __device__ __forceinline__ void split_digits(int q, int &d0, int &d1, int &d2) {
     d2 = (r - d1) >> 7;
 }
 
-// All threads of the workgroup: image of src[0..K) (K % 32 == 0).  Thread j takes the
-// eight values 8j..8j+7; four neighbouring threads form one 32-group.
+// The eight values 8j..8j+7 of a K-vector (a, b) into its image; four neighbouring threads form one
+// 32-group, so the four threads of a group must all be here.  Returns whether a value is not finite.
+__device__ __forceinline__ bool image_chunk(int *img, const float4 a, const float4 b, int j, int K) {
+    const int plane = SEG_STRIDE * (K / 64);
+    bool bad = false;
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    float m = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 8; c++) { m = fmaxf(m, fabsf(v[c])); bad |= !pf_finite(v[c]); }
+    m = fmaxf(m, __int_as_float(dpp_quad_xor1(__float_as_int(m))));
+    m = fmaxf(m, __int_as_float(dpp_quad_xor2(__float_as_int(m))));
+    float step, inv;
+    group_step(m, step, inv);
+    int w0[2] = {0, 0}, w1[2] = {0, 0}, w2[2] = {0, 0}, sum = 0;
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        const int q = __float2int_rn(v[c] * inv);
+        sum += q;
+        int d0, d1, d2;
+        split_digits(q, d0, d1, d2);
+        w0[c >> 2] |= (d0 & 255) << (8 * (c & 3));
+        w1[c >> 2] |= (d1 & 255) << (8 * (c & 3));
+        w2[c >> 2] |= (d2 & 255) << (8 * (c & 3));
+    }
+    sum += dpp_quad_xor1(sum);
+    sum += dpp_quad_xor2(sum);
+    const int at = SEG_STRIDE * (j >> 3) + 2 * (j & 7);
+    img[at] = w0[0]; img[at + 1] = w0[1];
+    img[plane + at] = w1[0]; img[plane + at + 1] = w1[1];
+    img[2 * plane + at] = w2[0]; img[2 * plane + at + 1] = w2[1];
+    if ((j & 3) == 0) {
+        reinterpret_cast<float *>(img + 3 * plane)[j >> 2] = step;
+        img[3 * plane + K / 32 + (j >> 2)] = sum;
+    }
+    return bad;
+}
+
+// Threads [first_thread, first_thread + thread_count) of the workgroup: image of src[0..K) (K % 32 == 0).
+// Thread j takes the eight values 8j..8j+7, then 8(j + count).. and so on.
 __device__ __forceinline__ bool build_image(int *img, const float *src, int K, int first_thread = 0,
                                             int thread_count = 1 << 30) {
-    const int plane = SEG_STRIDE * (K / 64);
     bool bad = false;
     const int j0 = (int)threadIdx.x - first_thread, stride = min(thread_count, (int)blockDim.x - first_thread);
     if (j0 < 0 || j0 >= stride) return false;
-    for (int j = j0; j < K / 8; j += stride) {
-        const float4 a = reinterpret_cast<const float4 *>(src)[2 * j];
-        const float4 b = reinterpret_cast<const float4 *>(src)[2 * j + 1];
-        const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-        float m = 0.0f;
+    for (int j = j0; j < K / 8; j += stride)
+        bad |= image_chunk(img, reinterpret_cast<const float4 *>(src)[2 * j], reinterpret_cast<const float4 *>(src)[2 * j + 1], j, K);
+    return bad;
+}
+
+// ---- two-digit images in global memory (kernels whose lanes are weight rows) --------------------
+// Where every lane of a wave is a weight row, the activation digits are the same for the whole wave and
+// travel through scalar registers: the image lives in global memory (pf_image2_words), written by the
+// kernel before.  Two balanced base-256 digits (signed bytes): the values as 16-bit integers relative
+// to a step per 32-group that puts the group's largest magnitude at 127 * 256; the rounding error is at
+// most 2^-16 of that magnitude.
+__device__ __forceinline__ void group_step2(float m, float &step, float &inv) {
+    const bool none = !(m > 1e-30f);   // an all-zero (or vanishing) group
+    inv = none ? 0.0f : 32512.0f / m;
+    step = none ? 0.0f : m * (1.0f / 32512.0f);
+}
+
+// Thread j of a group of four neighbouring lanes: the eight values 8j..8j+7 of a K-vector into its image.
+__device__ __forceinline__ bool image2_chunk(uint32_t *img, const float4 a, const float4 b, int j, int K) {
+    bool bad = false;
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    float m = 0.0f;
 #pragma unroll
-        for (int c = 0; c < 8; c++) { m = fmaxf(m, fabsf(v[c])); bad |= !pf_finite(v[c]); }
-        m = fmaxf(m, __int_as_float(dpp_quad_xor1(__float_as_int(m))));
-        m = fmaxf(m, __int_as_float(dpp_quad_xor2(__float_as_int(m))));
-        float step, inv;
-        group_step(m, step, inv);
-        int w0[2] = {0, 0}, w1[2] = {0, 0}, w2[2] = {0, 0}, sum = 0;
+    for (int c = 0; c < 8; c++) { m = fmaxf(m, fabsf(v[c])); bad |= !pf_finite(v[c]); }
+    m = fmaxf(m, __int_as_float(dpp_quad_xor1(__float_as_int(m))));
+    m = fmaxf(m, __int_as_float(dpp_quad_xor2(__float_as_int(m))));
+    float step, inv;
+    group_step2(m, step, inv);
+    uint32_t w0[2] = {0, 0}, w1[2] = {0, 0};
+    int sum = 0;
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            const int q = __float2int_rn(v[c] * inv);
-            sum += q;
-            int d0, d1, d2;
-            split_digits(q, d0, d1, d2);
-            w0[c >> 2] |= (d0 & 255) << (8 * (c & 3));
-            w1[c >> 2] |= (d1 & 255) << (8 * (c & 3));
-            w2[c >> 2] |= (d2 & 255) << (8 * (c & 3));
-        }
-        sum += dpp_quad_xor1(sum);
-        sum += dpp_quad_xor2(sum);
-        const int at = SEG_STRIDE * (j >> 3) + 2 * (j & 7);
-        img[at] = w0[0]; img[at + 1] = w0[1];
-        img[plane + at] = w1[0]; img[plane + at + 1] = w1[1];
-        img[2 * plane + at] = w2[0]; img[2 * plane + at + 1] = w2[1];
-        if ((j & 3) == 0) {
-            reinterpret_cast<float *>(img + 3 * plane)[j >> 2] = step;
-            img[3 * plane + K / 32 + (j >> 2)] = sum;
-        }
+    for (int c = 0; c < 8; c++) {
+        const int q = __float2int_rn(v[c] * inv);
+        sum += q;
+        const int d0 = ((q + 128) & 255) - 128, d1 = (q - d0) >> 8;
+        w0[c >> 2] |= (uint32_t)(d0 & 255) << (8 * (c & 3));
+        w1[c >> 2] |= (uint32_t)(d1 & 255) << (8 * (c & 3));
+    }
+    sum += dpp_quad_xor1(sum);
+    sum += dpp_quad_xor2(sum);
+    const int g = j >> 2, at = 16 * g + 2 * (j & 3);
+    img[at] = w0[0]; img[at + 1] = w0[1];
+    img[at + 8] = w1[0]; img[at + 9] = w1[1];
+    if ((j & 3) == 0) {
+        img[16 * (K / 32) + g] = __float_as_uint(step);
+        img[17 * (K / 32) + g] = (uint32_t)sum;
     }
     return bad;
 }
@@ -396,6 +446,17 @@ template <int FMT> __host__ __device__ constexpr int table_words() { return FMT 
 template <int NT>
 __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks) {
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
+    if ((int)blockIdx.x > router_blocks) {
+        // workgroups beyond the router's (launched where the next kernel reads them): the tokens' two-digit images,
+        // 2048 values per workgroup
+        const int per_token = (H + 2047) / 2048, q = (int)blockIdx.x - router_blocks - 1;
+        const int t = q / per_token, j = (q % per_token) * 256 + (int)threadIdx.x;
+        if (t < NT && j < H / 8) {
+            const float4 *row = reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch);
+            image2_chunk(a.ximg + (size_t)t * pf_image2_words(H), row[2 * j], row[2 * j + 1], j, H);
+        }
+        return;
+    }
     const bool gate_row = (int)blockIdx.x == router_blocks;
     const int e = blockIdx.x * 4 + wave;
     if (gate_row ? wave != 0 : e >= E) return;
@@ -490,6 +551,8 @@ struct RouteLds {
     PfRouteCands cands[PF_DECODE_MAX_TOKENS];
 };
 
+__device__ __forceinline__ float *scratch_of(int *images, int words) { return reinterpret_cast<float *>(images + words); }
+
 // Entered by the whole block after the fast routing: reference-order routing of the
 // ambiguous tokens (rare), then the union of the tokens' experts.  Ends with a block barrier.
 template <int NT>
@@ -543,56 +606,106 @@ __device__ __forceinline__ void route_finish(const PfKernelArgs &a, RouteLds *R,
 // 1024 threads.  Routed block b: unique slot b / tiles, units [tile * (b % tiles), +tile) of
 // that expert (tile = 16 or 32); shared blocks follow.  A wave owns tile / 16 units (a unit =
 // gate row + up row: lower half-wave the gate rows, upper half-wave the up rows) and writes its
-// activations itself, so no wave waits for another after the routing.  Waves 0..parts*NT-1 first reduce
-// the logits to candidates, waves 12..15 turn the token rows into digit images.
-// One tile's rows against the tokens' images: the part of kernel 2 that depends on the tensors' format.
+// activations itself, so no wave waits for another after the routing.
+// One tile's rows against the tokens' images, the part of kernel 2 that depends on the tensors'
+// format, in three steps: the weights requested, the products, the activations stored.
+struct TilePlace {       // where this lane's rows sit in the tile
+    int LPR, RPH, half, seg, r, steps, unit0;
+    bool second, idle;
+};
+
+__device__ __forceinline__ TilePlace tile_place(int H, int tile, int spl) {
+    TilePlace p;
+    const int lane = pf_lane(), wave = threadIdx.x >> 6;
+    p.LPR = row_lanes(H);
+    p.RPH = 32 / p.LPR;
+    p.half = lane >> 5;
+    p.seg = lane & (p.LPR - 1);
+    p.r = (lane & 31) / p.LPR;
+    p.second = spl > 1 && p.seg + p.LPR < H / 64;   // this lane also holds segment seg + LPR of its row
+    // the tile's units over 16 waves: RPH per wave step, one or two steps
+    const int per_wave = max(p.RPH, tile / 16);
+    p.steps = per_wave / p.RPH;
+    p.unit0 = wave * per_wave;
+    p.idle = p.unit0 >= tile;
+    return p;
+}
+
+template <int FMT, int SPL> struct TileRows { WSeg<FMT> w[2][SPL]; };
+
+template <int FMT, int SPL>
+__device__ __forceinline__ void tile_load(TileRows<FMT, SPL> &rows, const TilePlace &p, const PfKernelArgs &a, int gate_tensor,
+                                          uint32_t e, int n0) {
+    if (p.idle) return;
+#pragma unroll
+    for (int st = 0; st < 2; st++) {
+        if (st >= p.steps) break;
+        wseg_load<FMT>(rows.w[st][0], a, gate_tensor + p.half, e, n0 + p.unit0 + st * p.RPH + p.r, p.seg);
+        if (SPL > 1 && p.second)
+            wseg_load<FMT>(rows.w[st][SPL - 1], a, gate_tensor + p.half, e, n0 + p.unit0 + st * p.RPH + p.r, p.seg + p.LPR);
+    }
+}
+
+// act[t][st]: SwiGLU of unit unit0 + st * RPH + r for token t, valid in the lanes with half == 0 and seg == 0
+template <int FMT, int NT, int SPL>
+__device__ __forceinline__ void tile_dot(const TileRows<FMT, SPL> &rows, const TilePlace &p, const int *images,
+                                         const uint32_t *tables, int W, int H, uint32_t mask, float (&act)[NT][2]) {
+    const int lane = pf_lane();
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        act[t][0] = act[t][1] = 0.0f;
+        if (p.idle || !((mask >> t) & 1u)) continue;
+        XSeg x;
+        xseg_load(x, images + t * W, H, p.seg);
+        float dot[2];
+#pragma unroll
+        for (int st = 0; st < 2; st++) dot[st] = st < p.steps ? wseg_dot<FMT>(rows.w[st][0], x, p.seg, tables) : 0.0f;
+        if (SPL > 1) __builtin_amdgcn_sched_barrier(0);   // the second segment's digits reuse the first's registers
+        if (SPL > 1 && p.second) {
+            xseg_load(x, images + t * W, H, p.seg + p.LPR);
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+                if (st < p.steps) dot[st] += wseg_dot<FMT>(rows.w[st][SPL - 1], x, p.seg + p.LPR, tables);
+        }
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            if (st >= p.steps) break;
+            const float v = span_sum(dot[st], p.LPR);
+            const float up = __shfl(v, (lane & 31) + 32);
+            act[t][st] = pf_silu(v) * up;
+        }
+    }
+}
+
+template <int NT>
+__device__ __forceinline__ void tile_store(const float (&act)[NT][2], const TilePlace &p, const PfKernelArgs &a, int I, uint32_t mask,
+                                           int u, int n0, bool shared) {
+    if (p.idle || p.half != 0 || p.seg != 0) return;
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        if (!((mask >> t) & 1u)) continue;
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            if (st >= p.steps) break;
+            const int unit = p.unit0 + st * p.RPH + p.r;
+            if (!pf_finite(act[t][st])) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+            if (shared) a.shared_act[(size_t)t * I + n0 + unit] = act[t][st];
+            else a.act[((size_t)u * NT + t) * I + n0 + unit] = act[t][st];
+        }
+    }
+}
+
 template <int FMT, int NT, int SPL>
 __device__ __forceinline__ void gate_up_tile(const PfKernelArgs &a, const int *images, const uint32_t *tables, int W, int H,
                                              int I, int gate_tensor, uint32_t e, uint32_t mask, int u, int n0, int tile,
                                              bool shared) {
-    const int lane = pf_lane(), wave = threadIdx.x >> 6;
-    const int LPR = row_lanes(H), RPH = 32 / LPR;
-    const int half = lane >> 5, seg = lane & (LPR - 1), r = (lane & 31) / LPR;
-    const bool second = SPL > 1 && seg + LPR < H / 64;   // this lane also holds segment seg + LPR of its row
-    // the tile's units over 16 waves: RPH per wave step, one or two steps
-    const int per_wave = max(RPH, tile / 16), steps = per_wave / RPH, unit0 = wave * per_wave;
-    if (unit0 >= tile) return;
-    WSeg<FMT> w[2][SPL];
-#pragma unroll
-    for (int st = 0; st < 2; st++) {
-        if (st >= steps) break;
-        wseg_load<FMT>(w[st][0], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg);
-        if (SPL > 1 && second) wseg_load<FMT>(w[st][SPL - 1], a, gate_tensor + half, e, n0 + unit0 + st * RPH + r, seg + LPR);
-    }
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        if (!((mask >> t) & 1u)) continue;
-        XSeg x;
-        xseg_load(x, images + t * W, H, seg);
-        float dot[2];
-#pragma unroll
-        for (int st = 0; st < 2; st++) dot[st] = st < steps ? wseg_dot<FMT>(w[st][0], x, seg, tables) : 0.0f;
-        if (SPL > 1) __builtin_amdgcn_sched_barrier(0);   // the second segment's digits reuse the first's registers
-        if (SPL > 1 && second) {
-            xseg_load(x, images + t * W, H, seg + LPR);
-#pragma unroll
-            for (int st = 0; st < 2; st++)
-                if (st < steps) dot[st] += wseg_dot<FMT>(w[st][SPL - 1], x, seg + LPR, tables);
-        }
-#pragma unroll
-        for (int st = 0; st < 2; st++) {
-            if (st >= steps) break;
-            const float v = span_sum(dot[st], LPR);
-            const float up = __shfl(v, (lane & 31) + 32);
-            if (half == 0 && seg == 0) {
-                const float act = pf_silu(v) * up;
-                const int unit = unit0 + st * RPH + r;
-                if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-                if (shared) a.shared_act[(size_t)t * I + n0 + unit] = act;
-                else a.act[((size_t)u * NT + t) * I + n0 + unit] = act;
-            }
-        }
-    }
+    const TilePlace p = tile_place(H, tile, SPL);
+    if (p.idle) return;
+    TileRows<FMT, SPL> rows;
+    tile_load<FMT, SPL>(rows, p, a, gate_tensor, e, n0);
+    float act[NT][2];
+    tile_dot<FMT, NT, SPL>(rows, p, images, tables, W, H, mask, act);
+    tile_store<NT>(act, p, a, I, mask, u, n0, shared);
 }
 
 // FMT: format of the routed gate and up tensors; FMTS: of the shared expert's.
@@ -686,6 +799,340 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
     STAMP(5);
 }
 
+// ---- kernel 2, one token ---------------------------------------------------------------------------
+// With one token the unique experts are the token's slots, so the workgroups of slot u need to know
+// only the u + 1 best logits before they can ask for their weights: wave 0 holds the logits in
+// registers, extracts maxima up to its workgroup's slot, hands the expert to the other waves, and
+// only then -- with the weight bytes on their way -- extracts the remaining slots, tests how close the
+// k + 1 best are and forms the route weights.  Activations are held back until that test is known:
+// a token whose candidates are too close is re-routed in the reference's serial order and, should its
+// slot then name another expert, the tile is done again with that expert's rows (rare).
+template <int FMT, int FMTS, int NPL, int SPL>
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up1(PfKernelArgs a, int routed_blocks, int tile) {
+    extern __shared__ int lds[];
+    __shared__ RouteLds R;
+    __shared__ uint32_t early_expert;
+    const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
+    constexpr bool TABLES = FMT == PF_IQ2_XXS || FMTS == PF_IQ2_XXS;
+    int *images = lds + (TABLES ? 8192 : 0);
+    const int W = image_words(H);
+    const bool shared = (int)blockIdx.x >= routed_blocks;
+    const int tiles = a.inter / tile;
+    const int u = shared ? K : (int)blockIdx.x / tiles;
+    const int n0 = tile * (shared ? (int)blockIdx.x - routed_blocks : (int)blockIdx.x % tiles);
+    const bool norm = a.norm_topk != 0;
+    const int rounds = K + 1;   // top_k < experts on this path
+    if (TABLES) stage_tables(tables, a.iq2_signed);
+    // wave 0 of a routed workgroup: the token's logits, expert lane * NPL + j in register j, and the maxima up to slot u
+    float v[NPL], s2[NPL], total = 0.0f, top_all = 0.0f;
+    PfTopk<NPL> top;
+    uint32_t my_key = 0;
+    bool bad = false;
+    if (wave == 0 && !shared) {
+#pragma unroll
+        for (int j = 0; j < NPL; j++) {
+            const int e = lane * NPL + j;
+            v[j] = e < E ? a.logits[e] : -INFINITY;
+            s2[j] = e < E ? a.logit_ssq[e] : 0.0f;
+            bad |= e < E && !pf_finite(v[j]);
+        }
+        bad = __any(bad);
+        if (!norm) {   // unnormalised weights need the full softmax denominator
+            float m = v[0];
+#pragma unroll
+            for (int j = 1; j < NPL; j++) m = fmaxf(m, v[j]);
+            top_all = pf_wave_max_fast(m);
+#pragma unroll
+            for (int j = 0; j < NPL; j++) total += expf(v[j] - top_all);   // exp(-inf) = 0 for padding
+            total = pf_wave_sum(total);
+        }
+        top.setup(v, E, lane);
+        for (int r = 0; r <= u; r++) {
+            const uint32_t best = top.pop();
+            if (lane == r) my_key = best;
+        }
+        const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)my_key, u);
+        if (lane == 0) early_expert = mine ? pf_key_id(mine) : 0xffffffffu;
+    }
+    build_image(images, a.x, H, 768, 256);
+    __syncthreads();
+    const uint32_t early = shared ? 0u : early_expert;
+    const TilePlace p = tile_place(H, tile, SPL);
+    const int I = shared ? a.shared_inter : a.inter, gate_tensor = shared ? 4 : 1;
+    if (shared) {
+        TileRows<FMTS, SPL> rows;
+        tile_load<FMTS, SPL>(rows, p, a, gate_tensor, 0, n0);
+        float act[1][2];
+        tile_dot<FMTS, 1, SPL>(rows, p, images, tables, W, H, 1u, act);
+        tile_store<1>(act, p, a, I, 1u, u, n0, true);
+        return;
+    }
+    TileRows<FMT, SPL> rows;
+    const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
+    tile_load<FMT, SPL>(rows, p, a, gate_tensor, early_ok ? early : 0u, n0);
+    if (wave == 0) {
+        // the remaining slots, the candidate beyond them and one more key, with this wave's weight bytes on their way
+        for (int r = u + 1; r <= rounds; r++) {
+            const uint32_t best = top.pop();
+            if (lane == r) my_key = best;
+        }
+        uint32_t my_id;
+        float my_z, my_s2, weight;
+        bool close;
+        const bool ambiguous = pf_topk_exact_order<NPL>(my_key, rounds + 1, v, s2, lane, my_id, my_z, my_s2);
+        pf_route_finish_wave(my_z, my_s2, K, rounds, norm, H, total, top_all, lane, weight, close);
+        close |= ambiguous;
+        if (lane < K) { R.ids[lane] = my_id; R.weights[lane] = weight; }
+        if (lane == 0) { R.close[0] = close ? 1u : 0u; R.nonfinite[0] = bad ? 1u : 0u; }
+    }
+    float act[1][2];
+    tile_dot<FMT, 1, SPL>(rows, p, images, tables, W, H, 1u, act);
+    __syncthreads();
+    if (R.close[0]) {   // the same for every thread of every workgroup: the inputs are the same
+        route_finish<1>(a, &R, scratch_of(images, W));
+    } else if (threadIdx.x == 0) {
+        R.close_mask = 0;
+        R.bad = R.nonfinite[0];
+    }
+    // the slot's expert in the final order: the early guess came from truncated keys, so two experts whose logits
+    // agree in their leading bits can have changed places, and the serial-order routing can name another one
+    const uint32_t e = R.ids[u];
+    if (e != early && e < (uint32_t)E) {
+        tile_load<FMT, SPL>(rows, p, a, gate_tensor, e, n0);
+        tile_dot<FMT, 1, SPL>(rows, p, images, tables, W, H, 1u, act);
+    }
+    if (blockIdx.x == 0) {
+        // publish the routes for the next kernel and the caller (one token: slot = pair = unique expert)
+        if (R.close[0] == 0) __syncthreads();   // R.bad above; route_finish ends with a barrier of its own
+        for (int q = threadIdx.x; q < K; q += blockDim.x) {
+            a.ids[q] = R.ids[q];
+            a.route_weights[q] = R.weights[q];
+            a.uniq[1 + q] = R.ids[q];
+            a.uniq[1 + K + q] = q;
+            a.uniq[1 + 2 * K + q] = 1u;
+        }
+        if (threadIdx.x == 0) {
+            a.uniq[0] = K;
+            if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+            if (R.close_mask) atomicAdd(a.exact_rows, 1u);
+        }
+    }
+    if (e >= (uint32_t)E) {   // only reachable with nonfinite logits
+        if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+        return;
+    }
+    tile_store<1>(act, p, a, I, 1u, u, n0, false);
+}
+
+// ---- kernel 2, one token, Q4_K tensors in tile order ---------------------------------------------
+// The tile-ordered copy of a Q4_K tensor (pf_k_q4k_tile: per 32-row tile and 256-block the 32 headers,
+// then per 64-weight run the 16-byte halves 0 of the 32 rows and the halves 1) puts the same piece of
+// 32 consecutive rows into 512 consecutive bytes, so here a lane is a weight row: lanes 0..31 the
+// tile's gate rows, 32..63 its up rows, and a wave takes half a 256-block (four 32-groups) of all of
+// them.  Every lane of the wave then meets the same activations: their digits come from the token's
+// two-digit image in global memory through scalar loads and enter the dot products as scalar
+// operands -- no LDS image, no reduction across lanes.  The waves' partial sums meet in LDS and are
+// added in a fixed order.  Routing as in pf_k_dec_gate_up1.
+typedef const __attribute__((address_space(4))) uint32_t *PfScalarWords;   // read through the scalar cache
+
+struct Q4TileItem { uint4 hdr, piece[2][2]; };   // a row's header and its halves of two runs
+
+__device__ __forceinline__ void q4t_load(Q4TileItem &w, const uint8_t *chunk, int row, int half_block) {
+    w.hdr = *reinterpret_cast<const uint4 *>(chunk + 16 * row);
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++)
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            w.piece[rr][h] = *reinterpret_cast<const uint4 *>(chunk + 512 + (2 * half_block + rr) * 1024 + h * 512 + 16 * row);
+}
+
+// groups 4 * half_block .. + 3 of the row's block against the image's digits of the same groups (uniform pointer)
+__device__ __forceinline__ float q4t_dot(const Q4TileItem &w, PfScalarWords digits, PfScalarWords steps, PfScalarWords sums,
+                                         int half_block) {
+    // the four groups' 6-bit scales and minima as bytes (src/qwen4_packed.c:89-90)
+    uint32_t sc4, mn4;
+    if (half_block == 0) {
+        sc4 = w.hdr.y & 0x3F3F3F3Fu;
+        mn4 = w.hdr.z & 0x3F3F3F3Fu;
+    } else {
+        sc4 = (w.hdr.w & 0x0F0F0F0Fu) | ((w.hdr.y >> 2) & 0x30303030u);
+        mn4 = ((w.hdr.w >> 4) & 0x0F0F0F0Fu) | ((w.hdr.z >> 2) & 0x30303030u);
+    }
+    const float d = half_bits(w.hdr.x & 0xffffu), dmin = half_bits(w.hdr.x >> 16);
+    float total = 0.0f;
+#pragma unroll
+    for (int rr = 0; rr < 2; rr++) {
+        int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
+        PfScalarWords even = digits + 32 * rr, odd = even + 16;   // the run's two groups: low nibbles, high nibbles
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t q[4] = {w.piece[rr][h].x, w.piece[rr][h].y, w.piece[rr][h].z, w.piece[rr][h].w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+                lo0 = __builtin_amdgcn_sdot4(lo, (int)even[4 * h + i], lo0, false);
+                lo1 = __builtin_amdgcn_sdot4(lo, (int)even[8 + 4 * h + i], lo1, false);
+                hi0 = __builtin_amdgcn_sdot4(hi, (int)odd[4 * h + i], hi0, false);
+                hi1 = __builtin_amdgcn_sdot4(hi, (int)odd[8 + 4 * h + i], hi1, false);
+            }
+        }
+        const int g0 = 2 * rr, g1 = 2 * rr + 1;
+        const float s0 = (float)((sc4 >> (8 * g0)) & 255u), m0 = (float)((mn4 >> (8 * g0)) & 255u);
+        const float s1 = (float)((sc4 >> (8 * g1)) & 255u), m1 = (float)((mn4 >> (8 * g1)) & 255u);
+        const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sums[g0]);
+        const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sums[g1]);
+        total = fmaf(__uint_as_float(steps[g0]), t0, total);
+        total = fmaf(__uint_as_float(steps[g1]), t1, total);
+    }
+    return total;
+}
+
+// The tile's rows of expert e against the token: every wave its half-blocks, partial sums into LDS.
+// partial: [items][64] floats.  Requests first, products after `between` has run (wave 0: the rest of the routing).
+template <typename Between>
+__device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, float *partial, int gate_tensor, uint32_t e, int n0, int wave,
+                                         Between between) {
+    const int lane = pf_lane(), kblocks = a.hidden / 256, items = 2 * kblocks;
+    const int tensor = gate_tensor + (lane >> 5), row = lane & 31;
+    const uint8_t *tile = a.wt[tensor] + (size_t)e * a.expert_bytes[tensor] + (size_t)(n0 / 32) * kblocks * 4608;
+    const PfScalarWords image = (PfScalarWords)(uintptr_t)a.ximg;
+    const int groups = a.hidden / 32;
+    Q4TileItem w[2];
+    // at most two items a wave (hidden <= 2560): both requested before the first product
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int it = wave + 16 * k;
+        if (it < items) q4t_load(w[k], tile + (size_t)(it >> 1) * 4608, row, it & 1);
+    }
+    between();
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int it = wave + 16 * k;
+        if (it < items) {
+            const int g = 8 * (it >> 1) + 4 * (it & 1);
+            partial[it * 64 + lane] = q4t_dot(w[k], image + 16 * g, image + 16 * groups + g, image + 17 * groups + g, it & 1);
+        }
+    }
+}
+
+template <int NPL>
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) {
+    extern __shared__ int lds[];
+    __shared__ RouteLds R;
+    __shared__ uint32_t early_expert;
+    const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    float *partial = reinterpret_cast<float *>(lds);
+    const int items = 2 * (H / 256);
+    float *scratch = partial + items * 64;   // the serial-order routing's arrays
+    const bool shared = (int)blockIdx.x >= routed_blocks;
+    const int tiles = a.inter / 32;
+    const int u = shared ? K : (int)blockIdx.x / tiles;
+    const int n0 = 32 * (shared ? (int)blockIdx.x - routed_blocks : (int)blockIdx.x % tiles);
+    const bool norm = a.norm_topk != 0;
+    const int rounds = K + 1;   // top_k < experts on this path
+    float v[NPL], s2[NPL], total = 0.0f, top_all = 0.0f;
+    PfTopk<NPL> top;
+    uint32_t my_key = 0;
+    bool bad = false;
+    if (wave == 0 && !shared) {
+#pragma unroll
+        for (int j = 0; j < NPL; j++) {
+            const int e = lane * NPL + j;
+            v[j] = e < E ? a.logits[e] : -INFINITY;
+            s2[j] = e < E ? a.logit_ssq[e] : 0.0f;
+            bad |= e < E && !pf_finite(v[j]);
+        }
+        bad = __any(bad);
+        if (!norm) {   // unnormalised weights need the full softmax denominator
+            float m = v[0];
+#pragma unroll
+            for (int j = 1; j < NPL; j++) m = fmaxf(m, v[j]);
+            top_all = pf_wave_max_fast(m);
+#pragma unroll
+            for (int j = 0; j < NPL; j++) total += expf(v[j] - top_all);   // exp(-inf) = 0 for padding
+            total = pf_wave_sum(total);
+        }
+        top.setup(v, E, lane);
+        for (int r = 0; r <= u; r++) {
+            const uint32_t best = top.pop();
+            if (lane == r) my_key = best;
+        }
+        const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)my_key, u);
+        if (lane == 0) early_expert = mine ? pf_key_id(mine) : 0xffffffffu;
+    }
+    if (!shared) __syncthreads();
+    const uint32_t early = shared ? 0u : early_expert;
+    const int I = shared ? a.shared_inter : a.inter, gate_tensor = shared ? 4 : 1;
+    const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
+    q4t_tile(a, partial, gate_tensor, early_ok ? early : 0u, n0, wave, [&]() {
+        if (wave != 0 || shared) return;
+        // the remaining slots, the candidate beyond them and one more key, with this wave's weight bytes on their way
+        for (int r = u + 1; r <= rounds; r++) {
+            const uint32_t best = top.pop();
+            if (lane == r) my_key = best;
+        }
+        uint32_t my_id;
+        float my_z, my_s2, weight;
+        bool close;
+        const bool ambiguous = pf_topk_exact_order<NPL>(my_key, rounds + 1, v, s2, lane, my_id, my_z, my_s2);
+        pf_route_finish_wave(my_z, my_s2, K, rounds, norm, H, total, top_all, lane, weight, close);
+        close |= ambiguous;
+        if (lane < K) { R.ids[lane] = my_id; R.weights[lane] = weight; }
+        if (lane == 0) { R.close[0] = close ? 1u : 0u; R.nonfinite[0] = bad ? 1u : 0u; }
+    });
+    __syncthreads();
+    uint32_t e = early;
+    if (!shared) {
+        if (R.close[0]) {   // the same for every thread of every workgroup: the inputs are the same
+            route_finish<1>(a, &R, scratch);
+        } else if (threadIdx.x == 0) {
+            R.close_mask = 0;
+            R.bad = R.nonfinite[0];
+        }
+        // the slot's expert in the final order (the early guess came from truncated keys; the serial-order routing
+        // can name another expert)
+        e = R.ids[u];
+        if (e != early && e < (uint32_t)E) {
+            __syncthreads();
+            q4t_tile(a, partial, gate_tensor, e, n0, wave, []() {});
+            __syncthreads();
+        }
+        if (blockIdx.x == 0) {
+            // publish the routes for the next kernel and the caller (one token: slot = pair = unique expert)
+            if (R.close[0] == 0) __syncthreads();   // R.bad above; route_finish ends with a barrier of its own
+            for (int q = threadIdx.x; q < K; q += blockDim.x) {
+                a.ids[q] = R.ids[q];
+                a.route_weights[q] = R.weights[q];
+                a.uniq[1 + q] = R.ids[q];
+                a.uniq[1 + K + q] = q;
+                a.uniq[1 + 2 * K + q] = 1u;
+            }
+            if (threadIdx.x == 0) {
+                a.uniq[0] = K;
+                if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+                if (R.close_mask) atomicAdd(a.exact_rows, 1u);
+            }
+        }
+        if (e >= (uint32_t)E) {   // only reachable with nonfinite logits
+            if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+            return;
+        }
+    }
+    // thread t < 32: unit n0 + t; the items' partial sums in item order, SwiGLU, the activation and its digits
+    if (threadIdx.x < 32) {
+        float g = 0.0f, up = 0.0f;
+        for (int it = 0; it < items; it++) {
+            g += partial[it * 64 + lane];
+            up += partial[it * 64 + 32 + lane];
+        }
+        const float act = pf_silu(g) * up;
+        if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        (shared ? a.shared_act : a.act + (size_t)u * I)[n0 + lane] = act;
+    }
+}
+
 // ---- kernel 3: down products and the combine ---------------------------------------------------
 // blockIdx.x = t * row_blocks + nb; one wave per slot plus one for the shared expert; a routed
 // wave covers the block's rows in one step.  Every wave turns its slot's activation row into a
@@ -699,10 +1146,20 @@ __device__ __forceinline__ void down_rows(const PfKernelArgs &a, float *partial_
     const int LPR = row_lanes(I), rows = 64 / LPR, steps = rows >= rows_per_block ? 1 : rows_per_block / rows;
     const int seg = lane & (LPR - 1), r = lane / LPR;
     const bool second = SPL > 1 && seg + LPR < I / 64;   // this lane also holds segment seg + LPR of its row
+    // the wave's first activations are requested before its weights: loads of a wave return in order, and the
+    // image can then be built while the weight bytes are still on their way
+    const bool first_chunk = lane < I / 8;
+    float4 a0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), a1 = a0;
+    if (first_chunk) {
+        a0 = reinterpret_cast<const float4 *>(act_row)[2 * lane];
+        a1 = reinterpret_cast<const float4 *>(act_row)[2 * lane + 1];
+    }
     WSeg<FMT> w[SPL];   // further steps (a shared expert wider than the routed ones) load as they go
     wseg_load<FMT>(w[0], a, tensor, e, min(n_base + r, H - 1), seg);
     if (SPL > 1 && second) wseg_load<FMT>(w[SPL - 1], a, tensor, e, min(n_base + r, H - 1), seg + LPR);
-    build_image(image, act_row, I, 64 * s, 64);
+    if (first_chunk) image_chunk(image, a0, a1, lane, I);
+    for (int j = lane + 64; j < I / 8; j += 64)
+        image_chunk(image, reinterpret_cast<const float4 *>(act_row)[2 * j], reinterpret_cast<const float4 *>(act_row)[2 * j + 1], j, I);
     if (block_sync) __syncthreads();   // the tables staged by the whole workgroup
     else pf_wave_lds_fence();
     XSeg x;   // one segment's digits at a time: with two segments they are read from LDS again at every step
@@ -895,10 +1352,22 @@ static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStre
                        parts, chunk, tile, split ? 2 : 0);
 }
 
+template <int FG, int FS, int NPL, int SPL>
+static void launch_gate_up1(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks, int tile) {
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up1<FG, FS, NPL, SPL>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL((pf_k_dec_gate_up1<FG, FS, NPL, SPL>), grid, dim3(1024), lds, stream, a, routed_blocks, tile);
+}
+
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
 #if PF_DECODE_PART == 0
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream) {
-    const dim3 grid(router_blocks + 1), block(256);
+    // the router's rows, the shared router's row, then the tokens' two-digit images (2048 values per workgroup)
+    const dim3 grid(router_blocks + 1 + tokens * ((a.hidden + 2047) / 2048)), block(256);
     switch (tokens) {
     case 1: hipLaunchKernelGGL((pf_k_dec_router<1>), grid, block, 0, stream, a, router_blocks); break;
     case 2: hipLaunchKernelGGL((pf_k_dec_router<2>), grid, block, 0, stream, a, router_blocks); break;
@@ -955,11 +1424,31 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     const int rows_next = down_block_rows(H, I), row_blocks_next = (H + rows_next - 1) / rows_next;
     int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
     if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
+    if constexpr (NT == 1) {
+        // one token: every workgroup extracts the maxima up to its own slot from all the logits
+        const dim3 g1(routed_blocks + shared_blocks);
+        const int all = (E + 63) / 64;
+        if (FG == PF_Q4_K && FS == PF_Q4_K && a.wt[1] && a.wt[2] && a.wt[4] && a.wt[5] && I % 32 == 0 && Is % 32 == 0) {
+            // the tile-ordered copy is there: lanes are weight rows
+            const size_t lds = (size_t)(2 * (H / 256)) * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+            if (all <= 1) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<1>, g1, dim3(1024), lds, stream, a, routed_blocks);
+            else if (all <= 2) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<2>, g1, dim3(1024), lds, stream, a, routed_blocks);
+            else if (all <= 4) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<4>, g1, dim3(1024), lds, stream, a, routed_blocks);
+            else if (all <= 8) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<8>, g1, dim3(1024), lds, stream, a, routed_blocks);
+            else hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<16>, g1, dim3(1024), lds, stream, a, routed_blocks);
+        } else
+        if (all <= 1) launch_gate_up1<FG, FS, 1, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
+        else if (all <= 2) launch_gate_up1<FG, FS, 2, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
+        else if (all <= 4) launch_gate_up1<FG, FS, 4, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
+        else if (all <= 8) launch_gate_up1<FG, FS, 8, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
+        else launch_gate_up1<FG, FS, 16, SPL2>(a, g1, lds2, stream, routed_blocks, tile);   // experts <= 1024
+    } else {
     dim3 g2(routed_blocks + shared_blocks + prefetch_blocks);
     if (npl <= 1) launch_gate_up<FG, FS, NT, 1, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else if (npl <= 2) launch_gate_up<FG, FS, NT, 2, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else if (npl <= 4) launch_gate_up<FG, FS, NT, 4, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else launch_gate_up<FG, FS, NT, 8, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024
+    }
     if (last < 3) return;
     // kernel 3
     const int rows_per_block = down_block_rows(H, I), row_blocks = (H + rows_per_block - 1) / rows_per_block;

@@ -28,6 +28,8 @@ struct PfKernelArgs {
     float *act;                      // general path [tokens * top_k, inter]; decode path [unique, tokens, inter]
     float *shared_act;               // [tokens, shared_inter]
     float *shared_scale;             // [tokens] sigmoid of the shared router logit
+    uint32_t *ximg, *aimg;           // decode path, tile-ordered Q4_K: digit images (pf_image2_words) of the token rows, written
+                                     // by kernel 1, and of the activation rows [unique, tokens] then [tokens] shared, by kernel 2
     uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
     uint32_t *error_word;
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
@@ -103,9 +105,14 @@ struct PfHipMoe {
     uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
 };
 
+// Two-digit image of a K-vector for wave-uniform (scalar) reads: per 32-group 16 dwords (the values' low base-256
+// digits as 32 signed bytes, then their high digits), then K/32 group steps (float), then K/32 sums of the integers.
+__host__ __device__ constexpr size_t pf_image2_words(size_t K) { return (K / 32) * 18; }
+
 struct PfHipWork {
     const PfHipMoe *moe;
     size_t cap, bytes;
+    uint32_t *ximg, *aimg;
     float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
     uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags;
     uint16_t *x16, *act16, *sact16;  // prefill buffers (allocated when cap exceeds the decode path's batch)

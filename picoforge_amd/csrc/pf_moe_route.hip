@@ -157,7 +157,7 @@ __global__ void pf_k_flag_all(uint32_t *list, int n) {
 
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     const int npl = (a.experts + PF_WAVE - 1) / PF_WAVE;
-    if (a.experts > ROUTE_MAX_FAST_EXPERTS || a.top_k >= PF_WAVE)
+    if (a.experts > ROUTE_MAX_FAST_EXPERTS || a.top_k >= PF_WAVE - 1)   // the fast routing keeps top_k + 2 keys, one per lane
         hipLaunchKernelGGL(pf_k_flag_all, dim3((tokens + 255) / 256), dim3(256), 0, stream, a.route_flags, tokens);
     else if (npl <= 1) hipLaunchKernelGGL(pf_k_route_fast<1>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 2) hipLaunchKernelGGL(pf_k_route_fast<2>, dim3(tokens), dim3(64), 0, stream, a);

@@ -82,15 +82,133 @@ __device__ __forceinline__ void pf_route_finish_wave(float my_z, float my_s2, in
     else weight = e * expf(top - top_all) / total;
 }
 
+// ---- selection by packed keys -------------------------------------------------------------
+// The extraction above costs about a hundred instructions a round.  This one costs a quarter of
+// that: every logit becomes one 32-bit key, the order-preserving integer of the float with its low
+// ten bits replaced by 1023 - id, so that a plain unsigned maximum names value and expert at once
+// and keys are unique.  Each lane sorts its keys once (maxima and minima of a sorting network);
+// a round then is the wave's maximum over the lanes' heads and a shift of the winner's list.
+// Ten mantissa bits are lost, so the order among the extracted is only approximate: the exact
+// logits of the extracted are fetched back from the registers they came from (lane id / NPL,
+// register id % NPL) and ranked again exactly (value descending, then id ascending), and one
+// more key than needed is extracted: if it has the same truncated value as the last one needed,
+// an expert that was not extracted could belong in front of it, and the token is reported as
+// close (it is then routed in the reference's serial order).
+#define PF_KEY_ID_BITS 10
+#define PF_KEY_ID_MASK 1023u
+
+__device__ __forceinline__ uint32_t pf_order_bits(float z) {
+    uint32_t u = __float_as_uint(z + 0.0f);   // -0 counted as +0
+    return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+}
+
+__device__ __forceinline__ uint32_t pf_dpp_umax_step(uint32_t v, const int which) {
+    int moved;
+    const int bits = (int)v;
+    switch (which) {
+    case 0: moved = __builtin_amdgcn_update_dpp(bits, bits, 0xB1, 0xF, 0xF, false); break;   // quad_perm [1,0,3,2]
+    case 1: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x4E, 0xF, 0xF, false); break;   // quad_perm [2,3,0,1]
+    case 2: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x141, 0xF, 0xF, false); break;  // row_half_mirror
+    case 3: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x140, 0xF, 0xF, false); break;  // row_mirror
+    case 4: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x142, 0xA, 0xF, false); break;  // row_bcast:15 into rows 1,3
+    default: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x143, 0xC, 0xF, false); break; // row_bcast:31 into rows 2,3
+    }
+    return max(v, (uint32_t)moved);
+}
+
+template <int NPL> struct PfTopk {
+    uint32_t key[NPL];   // this lane's keys, largest first; 0 = none left
+
+    // v[j]: logit of expert lane * NPL + j (experts beyond E: any value)
+    __device__ __forceinline__ void setup(const float (&v)[NPL], int E, int lane) {
+#pragma unroll
+        for (int j = 0; j < NPL; j++) {
+            const uint32_t id = (uint32_t)(lane * NPL + j);
+            key[j] = id < (uint32_t)E ? ((pf_order_bits(v[j]) & ~PF_KEY_ID_MASK) | (PF_KEY_ID_MASK - id)) : 0u;
+        }
+        // bitonic sorting network, descending
+#pragma unroll
+        for (int size = 2; size <= NPL; size *= 2) {
+#pragma unroll
+            for (int stride = size / 2; stride > 0; stride /= 2) {
+#pragma unroll
+                for (int i = 0; i < NPL; i++) {
+                    const int partner = i ^ stride;
+                    if (partner > i) {
+                        const bool descending = (i & size) == 0;
+                        const uint32_t hi = max(key[i], key[partner]), lo = min(key[i], key[partner]);
+                        key[i] = descending ? hi : lo;
+                        key[partner] = descending ? lo : hi;
+                    }
+                }
+            }
+        }
+    }
+
+    // the largest key left in the wave, removed from its lane's list; 0 when nothing is left
+    __device__ __forceinline__ uint32_t pop() {
+        uint32_t m = key[0];
+        m = pf_dpp_umax_step(m, 0);
+        m = pf_dpp_umax_step(m, 1);
+        m = pf_dpp_umax_step(m, 2);
+        m = pf_dpp_umax_step(m, 3);
+        m = pf_dpp_umax_step(m, 4);
+        m = pf_dpp_umax_step(m, 5);
+        const uint32_t best = (uint32_t)__builtin_amdgcn_readlane((int)m, 63);
+        const bool mine = key[0] == best && best != 0u;
+#pragma unroll
+        for (int j = 0; j + 1 < NPL; j++) key[j] = mine ? key[j + 1] : key[j];
+        key[NPL - 1] = mine ? 0u : key[NPL - 1];
+        return best;
+    }
+};
+
+__device__ __forceinline__ uint32_t pf_key_id(uint32_t key) { return PF_KEY_ID_MASK - (key & PF_KEY_ID_MASK); }
+
+// Lane r < count holds the r-th popped key in my_key (count <= 64: the k + 1 best and one more).  Fetches the
+// exact logit and sum of squares of the first count - 1 and ranks them exactly; afterwards lane r < count - 1
+// holds the r-th best (id, z, s2).  Returns (uniformly) whether the extra key ties the last one needed.
+template <int NPL>
+__device__ __forceinline__ bool pf_topk_exact_order(uint32_t my_key, int count, const float (&v)[NPL], const float (&s2)[NPL],
+                                                    int lane, uint32_t &id, float &z, float &ssq) {
+    const int need = count - 1;
+    const bool have = lane < need && my_key != 0u;
+    id = have ? pf_key_id(my_key) : 0xffffffffu;
+    const int at = have ? (int)id : 0;
+    z = -INFINITY;
+    ssq = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NPL; j++) {
+        const float vz = __shfl(v[j], at / NPL), vs = __shfl(s2[j], at / NPL);
+        if (have && at % NPL == j) { z = vz; ssq = vs; }
+    }
+    const uint32_t last = (uint32_t)__builtin_amdgcn_readlane((int)my_key, need - 1);
+    const uint32_t extra = (uint32_t)__builtin_amdgcn_readlane((int)my_key, need);
+    const bool ambiguous = extra != 0u && (extra >> PF_KEY_ID_BITS) == (last >> PF_KEY_ID_BITS);
+    // exact rank among the needed ones: how many come before this lane's
+    int rank = 0;
+    for (int q = 0; q < need; q++) {
+        const float zq = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(z), q));
+        const uint32_t idq = (uint32_t)__builtin_amdgcn_readlane((int)id, q);
+        rank += (zq > z || (zq == z && idq < id)) ? 1 : 0;
+    }
+    const int to = lane < need ? rank : lane;   // a permutation of the lanes
+    id = (uint32_t)__builtin_amdgcn_ds_permute(to * 4, (int)id);
+    z = __int_as_float(__builtin_amdgcn_ds_permute(to * 4, __float_as_int(z)));
+    ssq = __int_as_float(__builtin_amdgcn_ds_permute(to * 4, __float_as_int(ssq)));
+    return ambiguous;
+}
+
 template <int NPL>
 __device__ __forceinline__ PfRouteResult pf_route_fast_wave(const float *z_row, const float *ssq_row, int E, int K,
                                                             bool norm, int hidden, int lane) {
-    float v[NPL];
+    float v[NPL], s2[NPL];
     bool bad = false;
 #pragma unroll
     for (int j = 0; j < NPL; j++) {
         const int e = lane * NPL + j;
         v[j] = e < E ? z_row[e] : -INFINITY;
+        s2[j] = e < E ? ssq_row[e] : 0.0f;
         bad |= e < E && !pf_finite(v[j]);
     }
     bad = __any(bad);
@@ -105,21 +223,18 @@ __device__ __forceinline__ PfRouteResult pf_route_fast_wave(const float *z_row, 
         total = pf_wave_sum(total);
     }
     const int rounds = K < E ? K + 1 : K;
-    uint32_t my_id = 0;
-    float my_z = 0.0f, my_s2 = 0.0f;
-    for (int r = 0; r < rounds; r++) {
-        float wm;
-        int owner, jsel;
-        pf_extract_max<NPL>(v, lane, wm, owner, jsel);
-        if (lane == r) {
-            my_id = (uint32_t)(owner * NPL + jsel);
-            my_z = wm;
-        }
+    PfTopk<NPL> top;
+    top.setup(v, E, lane);
+    uint32_t my_key = 0;
+    for (int r = 0; r <= rounds; r++) {   // one more than needed: see pf_topk_exact_order
+        const uint32_t best = top.pop();
+        if (lane == r) my_key = best;
     }
-    if (lane < rounds && my_id < (uint32_t)E) my_s2 = ssq_row[my_id];
     PfRouteResult out;
+    float my_z, my_s2;
+    const bool ambiguous = pf_topk_exact_order<NPL>(my_key, rounds + 1, v, s2, lane, out.id, my_z, my_s2);
     pf_route_finish_wave(my_z, my_s2, K, rounds, norm, hidden, total, top_all, lane, out.weight, out.close);
-    out.id = my_id;
+    out.close |= ambiguous;
     out.bad = bad;
     return out;
 }
