@@ -197,6 +197,40 @@ __device__ __forceinline__ bool image2_chunk(uint32_t *img, const float4 a, cons
     return bad;
 }
 
+// Lanes 0..31 of a wave, one value each: group g of a K-vector's image.
+__device__ __forceinline__ int dpp_row_step(int v, const int which) {
+    switch (which) {
+    case 0: return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);    // quad_perm [1,0,3,2]
+    case 1: return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);    // quad_perm [2,3,0,1]
+    case 2: return __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);   // row_half_mirror
+    default: return __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true);  // row_mirror
+    }
+}
+
+__device__ __forceinline__ void image2_group(uint32_t *img, float v, int g, int K, int lane) {   // lanes 32..63 idle along
+    float m = fabsf(v);
+#pragma unroll
+    for (int k = 0; k < 4; k++) m = fmaxf(m, __int_as_float(dpp_row_step(__float_as_int(m), k)));
+    m = fmaxf(m, __shfl_xor(m, 16));
+    float step, inv;
+    group_step2(m, step, inv);
+    const int q = __float2int_rn(v * inv);
+    int sum = q;
+#pragma unroll
+    for (int k = 0; k < 4; k++) sum += dpp_row_step(sum, k);
+    sum += __shfl_xor(sum, 16);
+    const int d0 = ((q + 128) & 255) - 128, d1 = (q - d0) >> 8;
+    uint8_t *bytes = reinterpret_cast<uint8_t *>(img + 16 * g);
+    if (lane < 32) {
+        bytes[lane] = (uint8_t)d0;
+        bytes[32 + lane] = (uint8_t)d1;
+    }
+    if (lane == 0) {
+        img[16 * (K / 32) + g] = __float_as_uint(step);
+        img[17 * (K / 32) + g] = (uint32_t)sum;
+    }
+}
+
 // ---- one lane's 64 weights of a row --------------------------------------------------
 template <int FMT> struct WSeg;
 template <> struct WSeg<PF_Q4_K> { uint4 hdr, q0, q1; };
@@ -799,132 +833,6 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
     STAMP(5);
 }
 
-// ---- kernel 2, one token ---------------------------------------------------------------------------
-// With one token the unique experts are the token's slots, so the workgroups of slot u need to know
-// only the u + 1 best logits before they can ask for their weights: wave 0 holds the logits in
-// registers, extracts maxima up to its workgroup's slot, hands the expert to the other waves, and
-// only then -- with the weight bytes on their way -- extracts the remaining slots, tests how close the
-// k + 1 best are and forms the route weights.  Activations are held back until that test is known:
-// a token whose candidates are too close is re-routed in the reference's serial order and, should its
-// slot then name another expert, the tile is done again with that expert's rows (rare).
-template <int FMT, int FMTS, int NPL, int SPL>
-__global__ void __launch_bounds__(1024) pf_k_dec_gate_up1(PfKernelArgs a, int routed_blocks, int tile) {
-    extern __shared__ int lds[];
-    __shared__ RouteLds R;
-    __shared__ uint32_t early_expert;
-    const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
-    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
-    constexpr bool TABLES = FMT == PF_IQ2_XXS || FMTS == PF_IQ2_XXS;
-    int *images = lds + (TABLES ? 8192 : 0);
-    const int W = image_words(H);
-    const bool shared = (int)blockIdx.x >= routed_blocks;
-    const int tiles = a.inter / tile;
-    const int u = shared ? K : (int)blockIdx.x / tiles;
-    const int n0 = tile * (shared ? (int)blockIdx.x - routed_blocks : (int)blockIdx.x % tiles);
-    const bool norm = a.norm_topk != 0;
-    const int rounds = K + 1;   // top_k < experts on this path
-    if (TABLES) stage_tables(tables, a.iq2_signed);
-    // wave 0 of a routed workgroup: the token's logits, expert lane * NPL + j in register j, and the maxima up to slot u
-    float v[NPL], s2[NPL], total = 0.0f, top_all = 0.0f;
-    PfTopk<NPL> top;
-    uint32_t my_key = 0;
-    bool bad = false;
-    if (wave == 0 && !shared) {
-#pragma unroll
-        for (int j = 0; j < NPL; j++) {
-            const int e = lane * NPL + j;
-            v[j] = e < E ? a.logits[e] : -INFINITY;
-            s2[j] = e < E ? a.logit_ssq[e] : 0.0f;
-            bad |= e < E && !pf_finite(v[j]);
-        }
-        bad = __any(bad);
-        if (!norm) {   // unnormalised weights need the full softmax denominator
-            float m = v[0];
-#pragma unroll
-            for (int j = 1; j < NPL; j++) m = fmaxf(m, v[j]);
-            top_all = pf_wave_max_fast(m);
-#pragma unroll
-            for (int j = 0; j < NPL; j++) total += expf(v[j] - top_all);   // exp(-inf) = 0 for padding
-            total = pf_wave_sum(total);
-        }
-        top.setup(v, E, lane);
-        for (int r = 0; r <= u; r++) {
-            const uint32_t best = top.pop();
-            if (lane == r) my_key = best;
-        }
-        const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)my_key, u);
-        if (lane == 0) early_expert = mine ? pf_key_id(mine) : 0xffffffffu;
-    }
-    build_image(images, a.x, H, 768, 256);
-    __syncthreads();
-    const uint32_t early = shared ? 0u : early_expert;
-    const TilePlace p = tile_place(H, tile, SPL);
-    const int I = shared ? a.shared_inter : a.inter, gate_tensor = shared ? 4 : 1;
-    if (shared) {
-        TileRows<FMTS, SPL> rows;
-        tile_load<FMTS, SPL>(rows, p, a, gate_tensor, 0, n0);
-        float act[1][2];
-        tile_dot<FMTS, 1, SPL>(rows, p, images, tables, W, H, 1u, act);
-        tile_store<1>(act, p, a, I, 1u, u, n0, true);
-        return;
-    }
-    TileRows<FMT, SPL> rows;
-    const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
-    tile_load<FMT, SPL>(rows, p, a, gate_tensor, early_ok ? early : 0u, n0);
-    if (wave == 0) {
-        // the remaining slots, the candidate beyond them and one more key, with this wave's weight bytes on their way
-        for (int r = u + 1; r <= rounds; r++) {
-            const uint32_t best = top.pop();
-            if (lane == r) my_key = best;
-        }
-        uint32_t my_id;
-        float my_z, my_s2, weight;
-        bool close;
-        const bool ambiguous = pf_topk_exact_order<NPL>(my_key, rounds + 1, v, s2, lane, my_id, my_z, my_s2);
-        pf_route_finish_wave(my_z, my_s2, K, rounds, norm, H, total, top_all, lane, weight, close);
-        close |= ambiguous;
-        if (lane < K) { R.ids[lane] = my_id; R.weights[lane] = weight; }
-        if (lane == 0) { R.close[0] = close ? 1u : 0u; R.nonfinite[0] = bad ? 1u : 0u; }
-    }
-    float act[1][2];
-    tile_dot<FMT, 1, SPL>(rows, p, images, tables, W, H, 1u, act);
-    __syncthreads();
-    if (R.close[0]) {   // the same for every thread of every workgroup: the inputs are the same
-        route_finish<1>(a, &R, scratch_of(images, W));
-    } else if (threadIdx.x == 0) {
-        R.close_mask = 0;
-        R.bad = R.nonfinite[0];
-    }
-    // the slot's expert in the final order: the early guess came from truncated keys, so two experts whose logits
-    // agree in their leading bits can have changed places, and the serial-order routing can name another one
-    const uint32_t e = R.ids[u];
-    if (e != early && e < (uint32_t)E) {
-        tile_load<FMT, SPL>(rows, p, a, gate_tensor, e, n0);
-        tile_dot<FMT, 1, SPL>(rows, p, images, tables, W, H, 1u, act);
-    }
-    if (blockIdx.x == 0) {
-        // publish the routes for the next kernel and the caller (one token: slot = pair = unique expert)
-        if (R.close[0] == 0) __syncthreads();   // R.bad above; route_finish ends with a barrier of its own
-        for (int q = threadIdx.x; q < K; q += blockDim.x) {
-            a.ids[q] = R.ids[q];
-            a.route_weights[q] = R.weights[q];
-            a.uniq[1 + q] = R.ids[q];
-            a.uniq[1 + K + q] = q;
-            a.uniq[1 + 2 * K + q] = 1u;
-        }
-        if (threadIdx.x == 0) {
-            a.uniq[0] = K;
-            if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-            if (R.close_mask) atomicAdd(a.exact_rows, 1u);
-        }
-    }
-    if (e >= (uint32_t)E) {   // only reachable with nonfinite logits
-        if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
-        return;
-    }
-    tile_store<1>(act, p, a, I, 1u, u, n0, false);
-}
-
 // ---- kernel 2, one token, Q4_K tensors in tile order ---------------------------------------------
 // The tile-ordered copy of a Q4_K tensor (pf_k_q4k_tile: per 32-row tile and 256-block the 32 headers,
 // then per 64-weight run the 16-byte halves 0 of the 32 rows and the halves 1) puts the same piece of
@@ -936,84 +844,95 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up1(PfKernelArgs a, int ro
 // added in a fixed order.  Routing as in pf_k_dec_gate_up1.
 typedef const __attribute__((address_space(4))) uint32_t *PfScalarWords;   // read through the scalar cache
 
-struct Q4TileItem { uint4 hdr, piece[2][2]; };   // a row's header and its halves of two runs
+struct Q4TileItem { uint4 hdr, piece[2]; };   // a row's header and the two halves of one 64-weight run
 
-__device__ __forceinline__ void q4t_load(Q4TileItem &w, const uint8_t *chunk, int row, int half_block) {
+__device__ __forceinline__ void q4t_load(Q4TileItem &w, const uint8_t *chunk, int row, int run) {
     w.hdr = *reinterpret_cast<const uint4 *>(chunk + 16 * row);
-#pragma unroll
-    for (int rr = 0; rr < 2; rr++)
-#pragma unroll
-        for (int h = 0; h < 2; h++)
-            w.piece[rr][h] = *reinterpret_cast<const uint4 *>(chunk + 512 + (2 * half_block + rr) * 1024 + h * 512 + 16 * row);
+    w.piece[0] = *reinterpret_cast<const uint4 *>(chunk + 512 + run * 1024 + 16 * row);
+    w.piece[1] = *reinterpret_cast<const uint4 *>(chunk + 512 + run * 1024 + 512 + 16 * row);
 }
 
-// groups 4 * half_block .. + 3 of the row's block against the image's digits of the same groups (uniform pointer)
-__device__ __forceinline__ float q4t_dot(const Q4TileItem &w, PfScalarWords digits, PfScalarWords steps, PfScalarWords sums,
-                                         int half_block) {
-    // the four groups' 6-bit scales and minima as bytes (src/qwen4_packed.c:89-90)
-    uint32_t sc4, mn4;
-    if (half_block == 0) {
-        sc4 = w.hdr.y & 0x3F3F3F3Fu;
-        mn4 = w.hdr.z & 0x3F3F3F3Fu;
+// groups 2 * run, 2 * run + 1 of the row's block (low and high nibbles of the run's bytes) against the image's digits,
+// steps and sums of the same two groups (uniform pointers)
+__device__ __forceinline__ float q4t_dot(const Q4TileItem &w, PfScalarWords digits, PfScalarWords steps, PfScalarWords sums, int run) {
+    // the two groups' 6-bit scales and minima (src/qwen4_packed.c:89-90): bytes 2 * run, 2 * run + 1 of the packed twelve
+    uint32_t sc2, mn2;
+    if (run < 2) {
+        sc2 = (w.hdr.y >> (16 * run)) & 0x3F3Fu;
+        mn2 = (w.hdr.z >> (16 * run)) & 0x3F3Fu;
     } else {
-        sc4 = (w.hdr.w & 0x0F0F0F0Fu) | ((w.hdr.y >> 2) & 0x30303030u);
-        mn4 = ((w.hdr.w >> 4) & 0x0F0F0F0Fu) | ((w.hdr.z >> 2) & 0x30303030u);
+        const int sh = 16 * (run - 2);
+        sc2 = ((w.hdr.w >> sh) & 0x0F0Fu) | (((w.hdr.y >> sh) >> 2) & 0x3030u);
+        mn2 = (((w.hdr.w >> sh) >> 4) & 0x0F0Fu) | (((w.hdr.z >> sh) >> 2) & 0x3030u);
     }
     const float d = half_bits(w.hdr.x & 0xffffu), dmin = half_bits(w.hdr.x >> 16);
-    float total = 0.0f;
+    int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
+    PfScalarWords even = digits, odd = digits + 16;
 #pragma unroll
-    for (int rr = 0; rr < 2; rr++) {
-        int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
-        PfScalarWords even = digits + 32 * rr, odd = even + 16;   // the run's two groups: low nibbles, high nibbles
+    for (int h = 0; h < 2; h++) {
+        const uint32_t q[4] = {w.piece[h].x, w.piece[h].y, w.piece[h].z, w.piece[h].w};
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const uint32_t q[4] = {w.piece[rr][h].x, w.piece[rr][h].y, w.piece[rr][h].z, w.piece[rr][h].w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
-                lo0 = __builtin_amdgcn_sdot4(lo, (int)even[4 * h + i], lo0, false);
-                lo1 = __builtin_amdgcn_sdot4(lo, (int)even[8 + 4 * h + i], lo1, false);
-                hi0 = __builtin_amdgcn_sdot4(hi, (int)odd[4 * h + i], hi0, false);
-                hi1 = __builtin_amdgcn_sdot4(hi, (int)odd[8 + 4 * h + i], hi1, false);
-            }
+        for (int i = 0; i < 4; i++) {
+            const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+            lo0 = __builtin_amdgcn_sdot4(lo, (int)even[4 * h + i], lo0, false);
+            lo1 = __builtin_amdgcn_sdot4(lo, (int)even[8 + 4 * h + i], lo1, false);
+            hi0 = __builtin_amdgcn_sdot4(hi, (int)odd[4 * h + i], hi0, false);
+            hi1 = __builtin_amdgcn_sdot4(hi, (int)odd[8 + 4 * h + i], hi1, false);
         }
-        const int g0 = 2 * rr, g1 = 2 * rr + 1;
-        const float s0 = (float)((sc4 >> (8 * g0)) & 255u), m0 = (float)((mn4 >> (8 * g0)) & 255u);
-        const float s1 = (float)((sc4 >> (8 * g1)) & 255u), m1 = (float)((mn4 >> (8 * g1)) & 255u);
-        const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sums[g0]);
-        const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sums[g1]);
-        total = fmaf(__uint_as_float(steps[g0]), t0, total);
-        total = fmaf(__uint_as_float(steps[g1]), t1, total);
     }
-    return total;
+    const float s0 = (float)(sc2 & 255u), m0 = (float)(mn2 & 255u), s1 = (float)(sc2 >> 8), m1 = (float)(mn2 >> 8);
+    const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sums[0]);
+    const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sums[1]);
+    return fmaf(__uint_as_float(steps[0]), t0, __uint_as_float(steps[1]) * t1);
 }
 
-// The tile's rows of expert e against the token: every wave its half-blocks, partial sums into LDS.
-// partial: [items][64] floats.  Requests first, products after `between` has run (wave 0: the rest of the routing).
-template <typename Between>
-__device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, float *partial, int gate_tensor, uint32_t e, int n0, int wave,
-                                         Between between) {
-    const int lane = pf_lane(), kblocks = a.hidden / 256, items = 2 * kblocks;
-    const int tensor = gate_tensor + (lane >> 5), row = lane & 31;
-    const uint8_t *tile = a.wt[tensor] + (size_t)e * a.expert_bytes[tensor] + (size_t)(n0 / 32) * kblocks * 4608;
+// The tile's rows against the token: the 64-weight runs of all the rows go round the waves 1..15 (wave 0
+// routes); a wave adds up its runs and leaves one partial sum per lane in LDS: partial[wave - 1][64].
+#define Q4T_ITEMS 3   // run items a wave can hold: hidden <= 2816
+struct Q4TilePlan {   // what does not depend on the expert: set up before the expert is known
+    const uint8_t *base;    // this lane's tensor (gate or up) at the tile's first 256-block, expert 0
+    size_t expert_bytes;
+    int row, kblocks, items, groups;
+};
+
+__device__ __forceinline__ Q4TilePlan q4t_plan(const PfKernelArgs &a, bool shared, int n0) {
+    Q4TilePlan p;
+    const int lane = pf_lane();
+    p.row = lane & 31;
+    p.kblocks = a.hidden / 256;
+    p.items = 4 * p.kblocks;
+    p.groups = a.hidden / 32;
+    // the two tensors by scalar selects and one per-lane choice (an index computed per lane would fetch the pointer
+    // from the argument block through the vector memory path, a round trip before the first weight request)
+    const bool up = lane >= 32;
+    const uint8_t *gate_w = shared ? a.wt[4] : a.wt[1], *up_w = shared ? a.wt[5] : a.wt[2];
+    const size_t gate_bytes = shared ? a.expert_bytes[4] : a.expert_bytes[1], up_bytes = shared ? a.expert_bytes[5] : a.expert_bytes[2];
+    p.base = (up ? up_w : gate_w) + (size_t)(n0 / 32) * p.kblocks * 4608;
+    p.expert_bytes = up ? up_bytes : gate_bytes;
+    return p;
+}
+
+__device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, const Q4TilePlan &p, float *partial, uint32_t e, int wave) {
+    if (wave == 0) return;
+    const int lane = pf_lane();
+    const uint8_t *tile = p.base + (size_t)e * p.expert_bytes;
     const PfScalarWords image = (PfScalarWords)(uintptr_t)a.ximg;
-    const int groups = a.hidden / 32;
-    Q4TileItem w[2];
-    // at most two items a wave (hidden <= 2560): both requested before the first product
+    Q4TileItem w[Q4T_ITEMS];
 #pragma unroll
-    for (int k = 0; k < 2; k++) {
-        const int it = wave + 16 * k;
-        if (it < items) q4t_load(w[k], tile + (size_t)(it >> 1) * 4608, row, it & 1);
+    for (int k = 0; k < Q4T_ITEMS; k++) {
+        const int it = wave - 1 + 15 * k;
+        if (it < p.items) q4t_load(w[k], tile + (size_t)(it >> 2) * 4608, p.row, it & 3);
     }
-    between();
+    float total = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 2; k++) {
-        const int it = wave + 16 * k;
-        if (it < items) {
-            const int g = 8 * (it >> 1) + 4 * (it & 1);
-            partial[it * 64 + lane] = q4t_dot(w[k], image + 16 * g, image + 16 * groups + g, image + 17 * groups + g, it & 1);
+    for (int k = 0; k < Q4T_ITEMS; k++) {
+        const int it = wave - 1 + 15 * k;
+        if (it < p.items) {
+            const int g = 2 * it;   // the run's first group within the row
+            total += q4t_dot(w[k], image + 16 * g, image + 16 * p.groups + g, image + 17 * p.groups + g, it & 3);
         }
     }
+    partial[(wave - 1) * 64 + lane] = total;
 }
 
 template <int NPL>
@@ -1023,9 +942,8 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
     __shared__ uint32_t early_expert;
     const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    float *partial = reinterpret_cast<float *>(lds);
-    const int items = 2 * (H / 256);
-    float *scratch = partial + items * 64;   // the serial-order routing's arrays
+    float *partial = reinterpret_cast<float *>(lds);   // [15 waves][64 lanes]
+    float *scratch = partial + 15 * 64;   // the serial-order routing's arrays
     const bool shared = (int)blockIdx.x >= routed_blocks;
     const int tiles = a.inter / 32;
     const int u = shared ? K : (int)blockIdx.x / tiles;
@@ -1037,13 +955,10 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
     uint32_t my_key = 0;
     bool bad = false;
     if (wave == 0 && !shared) {
+        pf_load_row<NPL>(a.logits, E, lane, -INFINITY, v);
+        pf_load_row<NPL>(a.logit_ssq, E, lane, 0.0f, s2);
 #pragma unroll
-        for (int j = 0; j < NPL; j++) {
-            const int e = lane * NPL + j;
-            v[j] = e < E ? a.logits[e] : -INFINITY;
-            s2[j] = e < E ? a.logit_ssq[e] : 0.0f;
-            bad |= e < E && !pf_finite(v[j]);
-        }
+        for (int j = 0; j < NPL; j++) bad |= lane * NPL + j < E && !pf_finite(v[j]);
         bad = __any(bad);
         if (!norm) {   // unnormalised weights need the full softmax denominator
             float m = v[0];
@@ -1062,13 +977,14 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
         const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)my_key, u);
         if (lane == 0) early_expert = mine ? pf_key_id(mine) : 0xffffffffu;
     }
+    const Q4TilePlan plan = q4t_plan(a, shared, n0);
+    const int I = shared ? a.shared_inter : a.inter;
     if (!shared) __syncthreads();
     const uint32_t early = shared ? 0u : early_expert;
-    const int I = shared ? a.shared_inter : a.inter, gate_tensor = shared ? 4 : 1;
     const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
-    q4t_tile(a, partial, gate_tensor, early_ok ? early : 0u, n0, wave, [&]() {
-        if (wave != 0 || shared) return;
-        // the remaining slots, the candidate beyond them and one more key, with this wave's weight bytes on their way
+    q4t_tile(a, plan, partial, early_ok ? early : 0u, wave);
+    if (wave == 0 && !shared) {
+        // the remaining slots, the candidate beyond them and one more key, while the other waves' weight bytes travel
         for (int r = u + 1; r <= rounds; r++) {
             const uint32_t best = top.pop();
             if (lane == r) my_key = best;
@@ -1081,7 +997,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
         close |= ambiguous;
         if (lane < K) { R.ids[lane] = my_id; R.weights[lane] = weight; }
         if (lane == 0) { R.close[0] = close ? 1u : 0u; R.nonfinite[0] = bad ? 1u : 0u; }
-    });
+    }
     __syncthreads();
     uint32_t e = early;
     if (!shared) {
@@ -1096,7 +1012,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
         e = R.ids[u];
         if (e != early && e < (uint32_t)E) {
             __syncthreads();
-            q4t_tile(a, partial, gate_tensor, e, n0, wave, []() {});
+            q4t_tile(a, plan, partial, e, wave);
             __syncthreads();
         }
         if (blockIdx.x == 0) {
@@ -1120,16 +1036,21 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
             return;
         }
     }
-    // thread t < 32: unit n0 + t; the items' partial sums in item order, SwiGLU, the activation and its digits
-    if (threadIdx.x < 32) {
-        float g = 0.0f, up = 0.0f;
-        for (int it = 0; it < items; it++) {
-            g += partial[it * 64 + lane];
-            up += partial[it * 64 + 32 + lane];
-        }
+    // the second wave: lane t < 32 adds up the gate row of unit n0 + t over the waves in wave order, lane 32 + t its
+    // up row; then SwiGLU, the activation and its digits
+    if (wave == 1) {
+        float sum = 0.0f;
+        for (int w = 0; w < 15; w++) sum += partial[w * 64 + lane];
+        const float g = sum, up = __shfl(sum, (lane & 31) + 32);
         const float act = pf_silu(g) * up;
-        if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-        (shared ? a.shared_act : a.act + (size_t)u * I)[n0 + lane] = act;
+        // the 32 units are one 32-group of the activation row: its two-digit image for the down kernel
+        // (vector u of the activation images; the shared expert's follows the top_k routed ones)
+        const size_t widest = a.inter > a.shared_inter ? a.inter : a.shared_inter;
+        if (lane < 32) {
+            if (!pf_finite(act)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+            (shared ? a.shared_act : a.act + (size_t)u * I)[n0 + lane] = act;
+        }
+        image2_group(a.aimg + (size_t)u * pf_image2_words(widest), act, n0 / 32, I, lane);
     }
 }
 
@@ -1249,6 +1170,107 @@ __global__ void __launch_bounds__(MAXT) pf_k_dec_down(PfKernelArgs a, int row_bl
     }
 }
 
+// ---- kernel 3, one token, Q4_K tensors in tile order ------------------------------------------------
+// Eight output rows per workgroup, one wave per slot and one for the shared expert, as above; a lane is
+// (row, 64-weight run): lanes 0..7 the rows' run 0, 8..15 run 1 and so on (further runs in turn), so the
+// eight rows' pieces of a run are one 128-byte line of the tile-ordered copy.  The activation digits come
+// from the two-digit images kernel 2 left in global memory (nothing is built here); the lanes of a row add
+// up across the wave, the slots meet in LDS and are combined in slot order.
+__global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a);
+#if PF_DECODE_PART == 0
+__global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
+    __shared__ float partial[17][8];
+    extern __shared__ int images[];   // [slot][image words of the widest activation row]
+    const int H = a.hidden, K = a.top_k, lane = pf_lane();
+    const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const bool shared = s == K;
+    const int I = shared ? a.shared_inter : a.inter;
+    const int n_base = 8 * (int)blockIdx.x, r = lane & 7, part = lane >> 3;
+    const size_t widest = a.inter > a.shared_inter ? a.inter : a.shared_inter;
+    // the slot's expert and the combine's operands through the scalar cache
+    const PfScalarWords ids = (PfScalarWords)(uintptr_t)a.ids, rws = (PfScalarWords)(uintptr_t)a.route_weights;
+    uint32_t e = shared ? 0u : ids[s];
+    float rw[16];
+#pragma unroll
+    for (int slot = 0; slot < 16; slot++) rw[slot] = slot < K ? __uint_as_float(rws[slot]) : 0.0f;
+    const float shared_scale = __uint_as_float(((PfScalarWords)(uintptr_t)a.shared_scale)[0]);
+    if (e >= (uint32_t)a.experts) {   // only reachable with nonfinite logits
+        if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
+        e = 0;
+    }
+    PfOutputRegs out_regs;
+    if ((int)threadIdx.x < 8) pf_output_prefetch(a, 0, n_base + threadIdx.x, out_regs);
+    const uint8_t *w = (shared ? a.wt[6] : a.wt[3]) + (size_t)e * (shared ? a.expert_bytes[6] : a.expert_bytes[3]);
+    const int kblocks = (shared ? a.shared_inter : a.down_physical) / 256, runs = I / 64, groups = I / 32;
+    const uint32_t *image = a.aimg + (size_t)s * pf_image2_words(widest);   // slot = unique expert with one token; the shared expert's follows
+    const uint8_t *tile = w + (size_t)(n_base / 32) * kblocks * 4608 + 16 * ((n_base & 31) + r);
+    // the slot's image into this wave's part of LDS (each lane needs the digits of its own run; fetched per lane they
+    // would cost eight requests a lane)
+    uint32_t *mine = reinterpret_cast<uint32_t *>(images) + (size_t)s * pf_image2_words(widest);
+    const int words = (int)pf_image2_words(I);
+    for (int i = 4 * lane; i < words; i += 256) *reinterpret_cast<uint4 *>(mine + i) = *reinterpret_cast<const uint4 *>(image + i);
+    float total = 0.0f;
+    bool fenced = false;
+    for (int run = part; run < runs; run += 8) {
+        const uint8_t *chunk = tile + (size_t)(run >> 2) * 4608;
+        const int rr = run & 3;
+        const uint4 hdr = *reinterpret_cast<const uint4 *>(chunk);
+        const uint4 p0 = *reinterpret_cast<const uint4 *>(chunk + 512 + rr * 1024);
+        const uint4 p1 = *reinterpret_cast<const uint4 *>(chunk + 512 + rr * 1024 + 512);
+        if (!fenced) { pf_wave_lds_fence(); fenced = true; }   // the image's stores of this wave before its reads
+        uint4 dg[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) dg[i] = reinterpret_cast<const uint4 *>(mine + 32 * run)[i];
+        const uint2 st = *reinterpret_cast<const uint2 *>(mine + 16 * groups + 2 * run);
+        const uint2 sm = *reinterpret_cast<const uint2 *>(mine + 17 * groups + 2 * run);
+        uint32_t sc2, mn2;
+        if (rr < 2) {
+            sc2 = (hdr.y >> (16 * rr)) & 0x3F3Fu;
+            mn2 = (hdr.z >> (16 * rr)) & 0x3F3Fu;
+        } else {
+            const int sh = 16 * (rr - 2);
+            sc2 = ((hdr.w >> sh) & 0x0F0Fu) | (((hdr.y >> sh) >> 2) & 0x3030u);
+            mn2 = (((hdr.w >> sh) >> 4) & 0x0F0Fu) | (((hdr.z >> sh) >> 2) & 0x3030u);
+        }
+        const float d = half_bits(hdr.x & 0xffffu), dmin = half_bits(hdr.x >> 16);
+        // dg[0..1]: low digits of the even group, dg[2..3] its high digits, dg[4..7] the odd group's
+        const uint32_t e0[8] = {dg[0].x, dg[0].y, dg[0].z, dg[0].w, dg[1].x, dg[1].y, dg[1].z, dg[1].w};
+        const uint32_t e1[8] = {dg[2].x, dg[2].y, dg[2].z, dg[2].w, dg[3].x, dg[3].y, dg[3].z, dg[3].w};
+        const uint32_t o0[8] = {dg[4].x, dg[4].y, dg[4].z, dg[4].w, dg[5].x, dg[5].y, dg[5].z, dg[5].w};
+        const uint32_t o1[8] = {dg[6].x, dg[6].y, dg[6].z, dg[6].w, dg[7].x, dg[7].y, dg[7].z, dg[7].w};
+        const uint32_t q[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+        int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+            lo0 = __builtin_amdgcn_sdot4(lo, (int)e0[i], lo0, false);
+            lo1 = __builtin_amdgcn_sdot4(lo, (int)e1[i], lo1, false);
+            hi0 = __builtin_amdgcn_sdot4(hi, (int)o0[i], hi0, false);
+            hi1 = __builtin_amdgcn_sdot4(hi, (int)o1[i], hi1, false);
+        }
+        const float s0 = (float)(sc2 & 255u), m0 = (float)(mn2 & 255u), s1 = (float)(sc2 >> 8), m1 = (float)(mn2 >> 8);
+        const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sm.x);
+        const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sm.y);
+        total += fmaf(__uint_as_float(st.x), t0, __uint_as_float(st.y) * t1);
+    }
+    // the row's runs: lanes r, r + 8, ..., r + 56
+    total += __shfl_xor(total, 8);
+    total += __shfl_xor(total, 16);
+    total += __shfl_xor(total, 32);
+    if (lane < 8) partial[s][lane] = total;
+    __syncthreads();
+    const int n = n_base + threadIdx.x;
+    if ((int)threadIdx.x < 8 && n < H) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int slot = 0; slot < 16; slot++)   // slot order, as src/qwen4_moe.c:362-372
+            if (slot < K) sum += rw[slot] * partial[slot][threadIdx.x];
+        const float y = sum + shared_scale * partial[K][threadIdx.x];
+        if (!pf_output_commit(a, 0, n, y, out_regs)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+    }
+}
+#endif
+
 #if PF_DECODE_PART == 0
 // ---- IQ2_XXS upload split -------------------------------------------------------------------------
 __global__ void pf_k_iq2_split(const uint8_t *gguf, uint8_t *payload, uint16_t *scales, size_t blocks) {
@@ -1352,17 +1374,6 @@ static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStre
                        parts, chunk, tile, split ? 2 : 0);
 }
 
-template <int FG, int FS, int NPL, int SPL>
-static void launch_gate_up1(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks, int tile) {
-    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up1<FG, FS, NPL, SPL>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-        configured = true;
-    }
-    hipLaunchKernelGGL((pf_k_dec_gate_up1<FG, FS, NPL, SPL>), grid, dim3(1024), lds, stream, a, routed_blocks, tile);
-}
-
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
 #if PF_DECODE_PART == 0
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream) {
@@ -1424,25 +1435,22 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     const int rows_next = down_block_rows(H, I), row_blocks_next = (H + rows_next - 1) / rows_next;
     int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
     if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
-    if constexpr (NT == 1) {
-        // one token: every workgroup extracts the maxima up to its own slot from all the logits
+    bool rows_as_lanes = false;
+    if constexpr (NT == 1 && FG == PF_Q4_K && FS == PF_Q4_K)
+        rows_as_lanes = a.wt[1] && a.wt[2] && a.wt[4] && a.wt[5] && I % 32 == 0 && Is % 32 == 0 && 4 * (H / 256) <= 15 * Q4T_ITEMS;
+    if constexpr (NT == 1 && FG == PF_Q4_K && FS == PF_Q4_K) if (rows_as_lanes) {
+        // one token, the tile-ordered copy is there: lanes are weight rows, every workgroup extracts the maxima up to
+        // its own slot from all the logits
         const dim3 g1(routed_blocks + shared_blocks);
         const int all = (E + 63) / 64;
-        if (FG == PF_Q4_K && FS == PF_Q4_K && a.wt[1] && a.wt[2] && a.wt[4] && a.wt[5] && I % 32 == 0 && Is % 32 == 0) {
-            // the tile-ordered copy is there: lanes are weight rows
-            const size_t lds = (size_t)(2 * (H / 256)) * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
-            if (all <= 1) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<1>, g1, dim3(1024), lds, stream, a, routed_blocks);
-            else if (all <= 2) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<2>, g1, dim3(1024), lds, stream, a, routed_blocks);
-            else if (all <= 4) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<4>, g1, dim3(1024), lds, stream, a, routed_blocks);
-            else if (all <= 8) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<8>, g1, dim3(1024), lds, stream, a, routed_blocks);
-            else hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<16>, g1, dim3(1024), lds, stream, a, routed_blocks);
-        } else
-        if (all <= 1) launch_gate_up1<FG, FS, 1, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
-        else if (all <= 2) launch_gate_up1<FG, FS, 2, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
-        else if (all <= 4) launch_gate_up1<FG, FS, 4, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
-        else if (all <= 8) launch_gate_up1<FG, FS, 8, SPL2>(a, g1, lds2, stream, routed_blocks, tile);
-        else launch_gate_up1<FG, FS, 16, SPL2>(a, g1, lds2, stream, routed_blocks, tile);   // experts <= 1024
-    } else {
+        const size_t lds = (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+        if (all <= 1) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<1>, g1, dim3(1024), lds, stream, a, routed_blocks);
+        else if (all <= 2) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<2>, g1, dim3(1024), lds, stream, a, routed_blocks);
+        else if (all <= 4) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<4>, g1, dim3(1024), lds, stream, a, routed_blocks);
+        else if (all <= 8) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<8>, g1, dim3(1024), lds, stream, a, routed_blocks);
+        else hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<16>, g1, dim3(1024), lds, stream, a, routed_blocks);
+    }
+    if (!rows_as_lanes) {
     dim3 g2(routed_blocks + shared_blocks + prefetch_blocks);
     if (npl <= 1) launch_gate_up<FG, FS, NT, 1, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else if (npl <= 2) launch_gate_up<FG, FS, NT, 2, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
@@ -1451,6 +1459,12 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     }
     if (last < 3) return;
     // kernel 3
+    if constexpr (NT == 1 && FG == PF_Q4_K && FD == PF_Q4_K && FS == PF_Q4_K)
+        if (rows_as_lanes && a.wt[3] && a.wt[6] && H % 32 == 0 && I % 64 == 0 && Is % 64 == 0 && a.down_physical == I) {
+            const size_t widest = I > Is ? I : Is;
+            hipLaunchKernelGGL(pf_k_dec_down_q4t, dim3(H / 8), dim3(64 * (K + 1)), (size_t)(K + 1) * pf_image2_words(widest) * 4, stream, a);
+            return;
+        }
     const int rows_per_block = down_block_rows(H, I), row_blocks = (H + rows_per_block - 1) / rows_per_block;
     const int image_pitch = image_words(I > Is ? I : Is);
     const size_t lds3 = tab3 + (size_t)(K + 1) * image_pitch * 4;

@@ -39,6 +39,28 @@ __device__ __forceinline__ float pf_wave_max_fast(float v) {
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
+// Expert lane * NPL + j of a row of E values into register j (fill beyond E).  The registers of a lane are
+// consecutive in memory: requested as 16-byte pieces where the row allows it, and all before the first is used
+// (a bounds test per element would make every element a round trip of its own).
+template <int NPL>
+__device__ __forceinline__ void pf_load_row(const float *row, int E, int lane, float fill, float (&v)[NPL]) {
+    const int base = lane * NPL;
+    if (NPL % 4 == 0 && E % 4 == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+#pragma unroll
+        for (int j = 0; j < NPL; j += 4) {
+            float4 q = make_float4(fill, fill, fill, fill);
+            if (base + j < E) q = *reinterpret_cast<const float4 *>(row + base + j);
+            v[j] = q.x; v[j + 1] = q.y; v[j + 2] = q.z; v[j + 3] = q.w;
+        }
+        return;
+    }
+    float got[NPL];
+#pragma unroll
+    for (int j = 0; j < NPL; j++) got[j] = row[min(base + j, E - 1)];
+#pragma unroll
+    for (int j = 0; j < NPL; j++) v[j] = base + j < E ? got[j] : fill;
+}
+
 struct PfRouteResult {
     uint32_t id;     // lane r < top_k: expert of slot r
     float weight;    // lane r < top_k: route weight of slot r
@@ -98,20 +120,21 @@ __device__ __forceinline__ void pf_route_finish_wave(float my_z, float my_s2, in
 #define PF_KEY_ID_MASK 1023u
 
 __device__ __forceinline__ uint32_t pf_order_bits(float z) {
-    uint32_t u = __float_as_uint(z + 0.0f);   // -0 counted as +0
-    return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+    const uint32_t u = __float_as_uint(z);   // -0 sorts just below +0: the exact ranking afterwards treats them as equal
+    return u ^ ((uint32_t)((int32_t)u >> 31) | 0x80000000u);
 }
 
 __device__ __forceinline__ uint32_t pf_dpp_umax_step(uint32_t v, const int which) {
     int moved;
     const int bits = (int)v;
+    // lanes a step does not reach receive 0, the identity of the unsigned maximum (so the move can merge into it)
     switch (which) {
-    case 0: moved = __builtin_amdgcn_update_dpp(bits, bits, 0xB1, 0xF, 0xF, false); break;   // quad_perm [1,0,3,2]
-    case 1: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x4E, 0xF, 0xF, false); break;   // quad_perm [2,3,0,1]
-    case 2: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x141, 0xF, 0xF, false); break;  // row_half_mirror
-    case 3: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x140, 0xF, 0xF, false); break;  // row_mirror
-    case 4: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x142, 0xA, 0xF, false); break;  // row_bcast:15 into rows 1,3
-    default: moved = __builtin_amdgcn_update_dpp(bits, bits, 0x143, 0xC, 0xF, false); break; // row_bcast:31 into rows 2,3
+    case 0: moved = __builtin_amdgcn_update_dpp(0, bits, 0xB1, 0xF, 0xF, true); break;   // quad_perm [1,0,3,2]
+    case 1: moved = __builtin_amdgcn_update_dpp(0, bits, 0x4E, 0xF, 0xF, true); break;   // quad_perm [2,3,0,1]
+    case 2: moved = __builtin_amdgcn_update_dpp(0, bits, 0x141, 0xF, 0xF, true); break;  // row_half_mirror
+    case 3: moved = __builtin_amdgcn_update_dpp(0, bits, 0x140, 0xF, 0xF, true); break;  // row_mirror
+    case 4: moved = __builtin_amdgcn_update_dpp(0, bits, 0x142, 0xA, 0xF, false); break;  // row_bcast:15 into rows 1,3
+    default: moved = __builtin_amdgcn_update_dpp(0, bits, 0x143, 0xC, 0xF, false); break; // row_bcast:31 into rows 2,3
     }
     return max(v, (uint32_t)moved);
 }
@@ -204,13 +227,10 @@ __device__ __forceinline__ PfRouteResult pf_route_fast_wave(const float *z_row, 
                                                             bool norm, int hidden, int lane) {
     float v[NPL], s2[NPL];
     bool bad = false;
+    pf_load_row<NPL>(z_row, E, lane, -INFINITY, v);
+    pf_load_row<NPL>(ssq_row, E, lane, 0.0f, s2);
 #pragma unroll
-    for (int j = 0; j < NPL; j++) {
-        const int e = lane * NPL + j;
-        v[j] = e < E ? z_row[e] : -INFINITY;
-        s2[j] = e < E ? ssq_row[e] : 0.0f;
-        bad |= e < E && !pf_finite(v[j]);
-    }
+    for (int j = 0; j < NPL; j++) bad |= lane * NPL + j < E && !pf_finite(v[j]);
     bad = __any(bad);
     float total = 0.0f, top_all = 0.0f;
     if (!norm) {   // unnormalised weights need the full softmax denominator
