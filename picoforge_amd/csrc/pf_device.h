@@ -6,8 +6,7 @@
 
 #define PF_WAVE 64
 
-// GGUF type ids and block geometry (src/gguf.c:12-16 of the reference).
-enum { PF_F32 = 0, PF_F16 = 1, PF_Q8_0 = 8, PF_Q2_K = 10, PF_Q4_K = 12, PF_IQ2_XXS = 16, PF_BF16 = 30, PF_MXFP4 = 39 };
+#include "pf_decode_addr.h"   // GGUF type ids, device layout of the tensors, the decode kernels' offsets
 
 __device__ __forceinline__ int pf_lane() { return threadIdx.x & (PF_WAVE - 1); }
 

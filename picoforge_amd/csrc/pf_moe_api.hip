@@ -100,23 +100,8 @@ static bool upload_constants(void) {
 const uint64_t *pf_device_iq2_grid(void) { return upload_constants() ? g_grid : nullptr; }
 const uint32_t *pf_device_iq2_signed(void) { return upload_constants() ? g_signed : nullptr; }
 
-static bool block_geometry(uint32_t type, size_t *block, size_t *bytes) {
-    switch (type) {
-    case PF_F32: *block = 1; *bytes = 4; return true;
-    case PF_F16: case PF_BF16: *block = 1; *bytes = 2; return true;
-    case PF_Q8_0: *block = 32; *bytes = 34; return true;
-    case PF_Q2_K: *block = 256; *bytes = 84; return true;
-    case PF_Q4_K: *block = 256; *bytes = 144; return true;
-    case PF_IQ2_XXS: *block = 256; *bytes = 66; return true;
-    case PF_MXFP4: *block = 32; *bytes = 17; return true;
-    default: return false;
-    }
-}
-
-// Formats stored split on the device (payloads, then scales): bytes of a block's leading scale, else 0.
-static size_t split_header_bytes(uint32_t type) {
-    return type == PF_IQ2_XXS || type == PF_Q8_0 ? 2 : type == PF_MXFP4 ? 1 : 0;
-}
+static bool block_geometry(uint32_t type, size_t *block, size_t *bytes) { return pf_block_geometry(type, block, bytes); }
+static size_t split_header_bytes(uint32_t type) { return pf_split_header_bytes(type); }
 
 // Host bytes into device memory through a page-locked buffer of the library's own (32 MB, allocated
 // at the first upload and kept until the process ends), two halves in turn so that the CPU fills
@@ -178,30 +163,21 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
     m->desc = *desc;
     size_t gguf_bytes[8];
     for (int a = 0; a < 8; a++) {
-        size_t block, size;
-        if (!block_geometry(desc->type[a], &block, &size) || k_storage[a] % block || k_storage[a] > 0x7fffffffu ||
-            n_out[a] > 0x7fffffffu) {
+        PfTensorPlace place;
+        if (k_storage[a] > 0x7fffffffu || n_out[a] > 0x7fffffffu ||
+            !pf_tensor_place(desc->type[a], k_storage[a], n_out[a], experts[a], &place)) {
             pf_hip_moe_destroy(m);
             return PF_HIP_E_UNSUPPORTED;
         }
-        const size_t blocks_per_row = k_storage[a] / block, rows = n_out[a] * experts[a];
-        gguf_bytes[a] = blocks_per_row * size * rows;
+        gguf_bytes[a] = place.gguf_bytes;
         if (bytes[a] < gguf_bytes[a] || !host_weights[a]) { pf_hip_moe_destroy(m); return PF_HIP_E_ARGUMENT; }
         m->k_logical[a] = (int)k_logical[a];
-        m->n_out[a] = (int)n_out[a];
-        m->blocks_per_row[a] = (int)blocks_per_row;
-        const size_t head = split_header_bytes(desc->type[a]);
-        if (head) {
-            // device layout: every block's payload (64, 32 or 16 bytes), then every block's scale
-            const size_t payload = size - head;
-            m->row_bytes[a] = blocks_per_row * payload;
-            m->scale_offset[a] = (blocks_per_row * rows * payload + 255) & ~(size_t)255;
-            m->bytes[a] = m->scale_offset[a] + blocks_per_row * rows * head + 4;   // the prefill loader reads the dword around a scale
-        } else {
-            m->row_bytes[a] = blocks_per_row * size;
-            m->bytes[a] = gguf_bytes[a];
-        }
-        m->expert_bytes[a] = m->row_bytes[a] * n_out[a];
+        m->n_out[a] = place.n_out;
+        m->blocks_per_row[a] = place.blocks_per_row;
+        m->row_bytes[a] = place.row_bytes;
+        m->scale_offset[a] = place.scale_offset;
+        m->bytes[a] = place.bytes;
+        m->expert_bytes[a] = place.expert_bytes;
     }
     if (!upload_constants()) { pf_hip_moe_destroy(m); return PF_HIP_E_MEMORY; }
     {   // set-up: this device's address of the static scratch, so that the entry point that uses it calls nothing but launches

@@ -43,24 +43,6 @@
 // steps (float), then K/32 group sums of the integer values.
 __host__ __device__ constexpr int image_words(int K) { return 3 * SEG_STRIDE * (K / 64) + 2 * (K / 32); }
 
-// Lanes that share one row of K values: the largest power of two that is at most K / 64 and at
-// most 32.  A lane takes the 64-value segment `seg` of the row and, where K / 64 is not that power
-// of two (K = 2560: 40 segments on 32 lanes, K = 640: 10 on 8), also segment seg + lanes if the
-// row has one (kernels instantiated with SPL = 2).
-__host__ __device__ inline int row_lanes(int K) {
-    int l = 1;
-    while (2 * l <= K / 64 && l < 32) l *= 2;
-    return l;
-}
-__host__ __device__ inline int row_passes(int K) { return (K / 64 + row_lanes(K) - 1) / row_lanes(K); }
-// Rows of the down projection per workgroup of kernel 3: what one wave covers in a step, doubled until
-// the row blocks of one token fit the 256 compute units (hidden 2560, intermediate 640: 16 rows, 160 blocks).
-__host__ __device__ inline int down_block_rows(int H, int I) {
-    int rows = 64 / row_lanes(I);
-    while ((H + rows - 1) / rows > 256 && rows < 64) rows *= 2;
-    return rows;
-}
-
 struct XSeg {          // one lane's 64 activations
     int d0[16], d1[16], d2[16];
     float step[2];
@@ -239,12 +221,23 @@ template <> struct WSeg<PF_IQ2_XXS> { uint4 p; uint32_t dbits; };
 template <int FMT>
 __device__ __forceinline__ void wseg_load(WSeg<FMT> &w, const PfKernelArgs &a, int t, size_t e, size_t n, int seg);
 
+// Every loader takes its offsets from pf_segment_spans (pf_decode_addr.h), the function the host-side bounds
+// test walks.
+__device__ __forceinline__ PfTensorPlace tensor_place(const PfKernelArgs &a, int t) {
+    PfTensorPlace p;
+    p.row_bytes = a.row_bytes[t]; p.expert_bytes = a.expert_bytes[t]; p.scale_offset = a.scale_offset[t];
+    p.bytes = p.gguf_bytes = 0;
+    p.n_out = a.n_out[t]; p.blocks_per_row = a.blocks_per_row[t];
+    return p;
+}
+
 template <>
 __device__ __forceinline__ void wseg_load<PF_Q4_K>(WSeg<PF_Q4_K> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
                                                    int seg) {
-    const uint8_t *blk = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + (size_t)(seg >> 2) * 144;
-    w.hdr = *reinterpret_cast<const uint4 *>(blk);
-    const uint4 *q = reinterpret_cast<const uint4 *>(blk + 16 + 32 * (seg & 3));
+    PfSpan sp[4];
+    pf_segment_spans(PF_Q4_K, tensor_place(a, t), e, n, seg, sp);
+    w.hdr = *reinterpret_cast<const uint4 *>(a.w[t] + sp[0].at);
+    const uint4 *q = reinterpret_cast<const uint4 *>(a.w[t] + sp[1].at);
     w.q0 = q[0];
     w.q1 = q[1];
 }
@@ -252,10 +245,10 @@ __device__ __forceinline__ void wseg_load<PF_Q4_K>(WSeg<PF_Q4_K> &w, const PfKer
 template <>
 __device__ __forceinline__ void wseg_load<PF_IQ2_XXS>(WSeg<PF_IQ2_XXS> &w, const PfKernelArgs &a, int t, size_t e,
                                                       size_t n, int seg) {
-    const uint8_t *row = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t];
-    w.p = *reinterpret_cast<const uint4 *>(row + 16 * seg);
-    const uint16_t *scales = reinterpret_cast<const uint16_t *>(a.w[t] + a.scale_offset[t]);
-    w.dbits = scales[(e * a.n_out[t] + n) * a.blocks_per_row[t] + (seg >> 2)];
+    PfSpan sp[4];
+    pf_segment_spans(PF_IQ2_XXS, tensor_place(a, t), e, n, seg, sp);
+    w.p = *reinterpret_cast<const uint4 *>(a.w[t] + sp[0].at);
+    w.dbits = *reinterpret_cast<const uint16_t *>(a.w[t] + sp[1].at);
 }
 
 // Q8_0, device layout (32 code bytes per block, half scales apart): a segment is two blocks
@@ -263,11 +256,12 @@ template <> struct WSeg<PF_Q8_0> { uint4 q[4]; uint32_t d2; };
 template <>
 __device__ __forceinline__ void wseg_load<PF_Q8_0>(WSeg<PF_Q8_0> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
                                                    int seg) {
-    const uint4 *row = reinterpret_cast<const uint4 *>(a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + 64 * (size_t)seg);
+    PfSpan sp[4];
+    pf_segment_spans(PF_Q8_0, tensor_place(a, t), e, n, seg, sp);
+    const uint4 *row = reinterpret_cast<const uint4 *>(a.w[t] + sp[0].at);
 #pragma unroll
     for (int i = 0; i < 4; i++) w.q[i] = row[i];
-    const uint16_t *scales = reinterpret_cast<const uint16_t *>(a.w[t] + a.scale_offset[t]);
-    w.d2 = *reinterpret_cast<const uint32_t *>(scales + (e * a.n_out[t] + n) * a.blocks_per_row[t] + 2 * seg);
+    w.d2 = *reinterpret_cast<const uint32_t *>(a.w[t] + sp[1].at);
 }
 
 // MXFP4, device layout (16 nibble bytes per block, scale bytes apart): a segment is two blocks
@@ -275,11 +269,12 @@ template <> struct WSeg<PF_MXFP4> { uint4 q[2]; uint32_t e2; };
 template <>
 __device__ __forceinline__ void wseg_load<PF_MXFP4>(WSeg<PF_MXFP4> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
                                                     int seg) {
-    const uint4 *row = reinterpret_cast<const uint4 *>(a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + 32 * (size_t)seg);
+    PfSpan sp[4];
+    pf_segment_spans(PF_MXFP4, tensor_place(a, t), e, n, seg, sp);
+    const uint4 *row = reinterpret_cast<const uint4 *>(a.w[t] + sp[0].at);
     w.q[0] = row[0];
     w.q[1] = row[1];
-    const uint8_t *scales = a.w[t] + a.scale_offset[t] + (e * a.n_out[t] + n) * a.blocks_per_row[t] + 2 * seg;
-    w.e2 = *reinterpret_cast<const uint16_t *>(scales);
+    w.e2 = *reinterpret_cast<const uint16_t *>(a.w[t] + sp[1].at);
 }
 
 // Q2_K, GGUF bytes (84-byte blocks, 4-byte aligned): a segment is a quarter of a block: 32 code
@@ -288,12 +283,13 @@ template <> struct WSeg<PF_Q2_K> { uint32_t q[8], sm, dd; };
 template <>
 __device__ __forceinline__ void wseg_load<PF_Q2_K>(WSeg<PF_Q2_K> &w, const PfKernelArgs &a, int t, size_t e, size_t n,
                                                    int seg) {
-    const uint8_t *blk = a.w[t] + e * a.expert_bytes[t] + n * a.row_bytes[t] + (size_t)(seg >> 2) * 84;
-    const uint32_t *codes = reinterpret_cast<const uint32_t *>(blk + 16 + 32 * ((seg & 3) >> 1));
+    PfSpan sp[4];
+    pf_segment_spans(PF_Q2_K, tensor_place(a, t), e, n, seg, sp);
+    const uint32_t *codes = reinterpret_cast<const uint32_t *>(a.w[t] + sp[0].at);
 #pragma unroll
     for (int i = 0; i < 8; i++) w.q[i] = codes[i];
-    w.sm = *reinterpret_cast<const uint32_t *>(blk + 4 * (seg & 3));
-    w.dd = *reinterpret_cast<const uint32_t *>(blk + 80);
+    w.sm = *reinterpret_cast<const uint32_t *>(a.w[t] + sp[1].at);
+    w.dd = *reinterpret_cast<const uint32_t *>(a.w[t] + sp[2].at);
 }
 
 __device__ __forceinline__ float half_bits(uint32_t h) {
@@ -559,16 +555,9 @@ __device__ __forceinline__ void prefetch_down(const PfKernelArgs &a, const uint3
         const int tensor = slot == uniques ? 6 : 3;
         const size_t e = slot == uniques ? 0 : uniq[slot], row0 = (size_t)nb * rows_per_block;
         if (e >= (size_t)a.experts) continue;
-        const size_t bytes = (size_t)rows_per_block * a.row_bytes[tensor];
-        const uint8_t *p = a.w[tensor] + e * a.expert_bytes[tensor] + row0 * a.row_bytes[tensor];
-        if (l == lines - 1) {
-            if (!a.scale_offset[tensor]) continue;
-            const size_t each = a.type[tensor] == PF_MXFP4 ? 1 : 2;
-            p = a.w[tensor] + a.scale_offset[tensor] + (e * a.n_out[tensor] + row0) * a.blocks_per_row[tensor] * each;
-        } else {
-            p += min((size_t)l * 128, bytes - 4);
-        }
-        sink |= *reinterpret_cast<const volatile uint32_t *>((uintptr_t)p & ~(uintptr_t)3);
+        PfSpan sp;
+        if (!pf_warm_span(a.type[tensor], tensor_place(a, tensor), e, row0, rows_per_block, l, lines, &sp)) continue;
+        sink |= *reinterpret_cast<const volatile uint32_t *>(a.w[tensor] + sp.at);
     }
     if (sink == 0x9e3779b9u && a.hidden < 0) atomicOr(a.error_word, 0u);   // keeps the loads; never true
 }
@@ -847,9 +836,9 @@ typedef const __attribute__((address_space(4))) uint32_t *PfScalarWords;   // re
 struct Q4TileItem { uint4 hdr, piece[2]; };   // a row's header and the two halves of one 64-weight run
 
 __device__ __forceinline__ void q4t_load(Q4TileItem &w, const uint8_t *chunk, int row, int run) {
-    w.hdr = *reinterpret_cast<const uint4 *>(chunk + 16 * row);
-    w.piece[0] = *reinterpret_cast<const uint4 *>(chunk + 512 + run * 1024 + 16 * row);
-    w.piece[1] = *reinterpret_cast<const uint4 *>(chunk + 512 + run * 1024 + 512 + 16 * row);
+    w.hdr = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_header_at(row));
+    w.piece[0] = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(run, 0, row));
+    w.piece[1] = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(run, 1, row));
 }
 
 // groups 2 * run, 2 * run + 1 of the row's block (low and high nibbles of the run's bytes) against the image's digits,
@@ -907,7 +896,7 @@ __device__ __forceinline__ Q4TilePlan q4t_plan(const PfKernelArgs &a, bool share
     const bool up = lane >= 32;
     const uint8_t *gate_w = shared ? a.wt[4] : a.wt[1], *up_w = shared ? a.wt[5] : a.wt[2];
     const size_t gate_bytes = shared ? a.expert_bytes[4] : a.expert_bytes[1], up_bytes = shared ? a.expert_bytes[5] : a.expert_bytes[2];
-    p.base = (up ? up_w : gate_w) + (size_t)(n0 / 32) * p.kblocks * 4608;
+    p.base = (up ? up_w : gate_w) + pf_q4t_chunk_at(0, 0, n0 / 32, p.kblocks, 0);
     p.expert_bytes = up ? up_bytes : gate_bytes;
     return p;
 }
@@ -921,7 +910,7 @@ __device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, const Q4TilePlan
 #pragma unroll
     for (int k = 0; k < Q4T_ITEMS; k++) {
         const int it = wave - 1 + 15 * k;
-        if (it < p.items) q4t_load(w[k], tile + (size_t)(it >> 2) * 4608, p.row, it & 3);
+        if (it < p.items) q4t_load(w[k], tile + pf_q4t_chunk_at(0, 0, 0, p.kblocks, it >> 2), p.row, it & 3);
     }
     float total = 0.0f;
 #pragma unroll
@@ -1203,7 +1192,8 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
     const uint8_t *w = (shared ? a.wt[6] : a.wt[3]) + (size_t)e * (shared ? a.expert_bytes[6] : a.expert_bytes[3]);
     const int kblocks = (shared ? a.shared_inter : a.down_physical) / 256, runs = I / 64, groups = I / 32;
     const uint32_t *image = a.aimg + (size_t)s * pf_image2_words(widest);   // slot = unique expert with one token; the shared expert's follows
-    const uint8_t *tile = w + (size_t)(n_base / 32) * kblocks * 4608 + 16 * ((n_base & 31) + r);
+    const uint8_t *tile = w + pf_q4t_chunk_at(0, 0, n_base / 32, kblocks, 0);
+    const int row_in_tile = (n_base & 31) + r;
     // the slot's image into this wave's part of LDS (each lane needs the digits of its own run; fetched per lane they
     // would cost eight requests a lane)
     uint32_t *mine = reinterpret_cast<uint32_t *>(images) + (size_t)s * pf_image2_words(widest);
@@ -1212,11 +1202,11 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
     float total = 0.0f;
     bool fenced = false;
     for (int run = part; run < runs; run += 8) {
-        const uint8_t *chunk = tile + (size_t)(run >> 2) * 4608;
+        const uint8_t *chunk = tile + pf_q4t_chunk_at(0, 0, 0, kblocks, run >> 2);
         const int rr = run & 3;
-        const uint4 hdr = *reinterpret_cast<const uint4 *>(chunk);
-        const uint4 p0 = *reinterpret_cast<const uint4 *>(chunk + 512 + rr * 1024);
-        const uint4 p1 = *reinterpret_cast<const uint4 *>(chunk + 512 + rr * 1024 + 512);
+        const uint4 hdr = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_header_at(row_in_tile));
+        const uint4 p0 = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(rr, 0, row_in_tile));
+        const uint4 p1 = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(rr, 1, row_in_tile));
         if (!fenced) { pf_wave_lds_fence(); fenced = true; }   // the image's stores of this wave before its reads
         uint4 dg[8];
 #pragma unroll
