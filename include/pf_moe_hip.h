@@ -187,6 +187,20 @@ int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_bytes, size
 int pf_hip_packed_decode_row_host(uint32_t gguf_type, const void *row_bytes_ptr, size_t row_bytes,
                                   size_t k_storage, float *out, uint32_t *error_word);
 
+/* The block's elementwise steps in the reference's evaluation order, bit-identical on hosts whose C
+ * library computes expf as glibc 2.27+ does.  op 0: SiLU, op 1: sigmoid (qwen4_activate,
+ * src/qwen4_base.c:76-99), op 2: out[j] = a[j] * b[j] (src/qwen4_moe.c:327-330).  A nonfinite input
+ * or result sets PF_HIP_ERR_NONFINITE and leaves out untouched. */
+int pf_hip_exact_elementwise_host(int op, const float *a, const float *b, size_t n, float *out,
+                                  uint32_t *error_word);
+
+/* src/qwen4_moe.c:350-368: routed[t, c] = the slot-order sum of weights[t, s] * down[pair_to_row[t*k+s], c],
+ * y = routed + shared_gate[t] * shared[t, c].  Dense host arrays.  Both outputs are written even when
+ * the error word is set. */
+int pf_hip_exact_combine_host(const float *down, const uint64_t *pair_to_row, const float *weights,
+                              const float *shared_gate, const float *shared, size_t tokens, size_t top_k,
+                              size_t hidden, float *routed, float *y, uint32_t *error_word);
+
 /* Minimal device-memory helpers so that a host program can keep inputs resident. */
 int pf_hip_malloc(void **d_ptr, size_t bytes);
 void pf_hip_free(void *d_ptr);

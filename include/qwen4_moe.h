@@ -92,10 +92,12 @@ Qwen4Status qw4_moe_group_pairs(const Qwen4MoeConfig *config, Qwen4U32Mut ids,
 
 /* Replaces qw4_moe_observe (src/qwen4_moe.c:130-132).  Stage numbers follow
  * src/qwen4_moe_internal.h:9-12: 0..7 projections in weight order, 8 SiLU,
- * 9 product, 10 sigmoid, 11 routed, 12 y.  The intermediate stages stay on the
- * device and are not copied out: this path reports stage 12 only (x as input,
- * y as output, once per forward); views are the caller's, valid during the
- * callback. */
+ * 9 product, 10 sigmoid, 11 routed, 12 y; the (stage, expert, token, input, output) sequence is the
+ * reference's (src/qwen4_moe.c:305-382), per microbatch of at most 32 tokens.  While an observer is
+ * set, forward runs the block as that sequence of operators, one device call each in the reference's
+ * evaluation order (slow; outputs bit-identical to the reference's), and reads the weights from the
+ * caller's host views: QW4_BAD_STATE after pf_moe_forget_host_weights.  Views passed to the observer
+ * are host staging memory, valid during the callback. */
 typedef void (*QW4MoeObserver)(void *ctx, size_t stage, size_t expert, size_t token,
                                Qwen4F32 input, Qwen4F32 output);
 void qw4_moe_observe(Qwen4MoeWork *work, QW4MoeObserver observer, void *ctx);

@@ -61,4 +61,14 @@ PF_EXPF_FN float pf_expf_libm(float x) {
     y = y * s;
     return (float)y;
 }
+
+/* The reference's sigmoid (src/qwen4_cpu_internal.h:103-106): both of its branches need expf(-|x|),
+ * 1 / (1 + e) for x >= 0 and e / (1 + e) below. */
+PF_EXPF_FN float pf_sigmoid_libm(float x) {
+#ifdef __clang__
+#pragma clang fp contract(off)
+#endif
+    const float e = pf_expf_libm(x < 0.0f ? x : -x);
+    return (x >= 0.0f ? 1.0f : e) / (1.0f + e);
+}
 #endif

@@ -864,6 +864,73 @@ extern "C" int pf_hip_packed_matmul_host(uint32_t gguf_type, const void *expert_
     return PF_HIP_OK;
 }
 
+extern "C" int pf_hip_exact_elementwise_host(int op, const float *a, const float *b, size_t n, float *out,
+                                            uint32_t *error_word) {
+    if (!error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (op < 0 || op > 2) return PF_HIP_E_UNSUPPORTED;
+    if (n == 0) return PF_HIP_OK;
+    if (!a || !out || (op == 2 && !b)) return PF_HIP_E_ARGUMENT;
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
+    const size_t nb = (n * 4 + 255) & ~(size_t)255;
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, 3 * nb + 256));
+    float *d_a = (float *)blk.p, *d_b = (float *)(blk.p + nb), *d_out = (float *)(blk.p + 2 * nb);
+    uint32_t *d_err = (uint32_t *)(blk.p + 3 * nb);
+    HIP_TRY(hipMemcpy(d_a, a, n * 4, hipMemcpyHostToDevice));
+    if (op == 2) HIP_TRY(hipMemcpy(d_b, b, n * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(d_err, 0, 256));
+    pf_launch_exact_elementwise(op, d_a, d_b, d_out, n, d_err, nullptr);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, d_err, 4, hipMemcpyDeviceToHost));
+    if (*error_word) return PF_HIP_OK;
+    HIP_TRY(hipMemcpy(out, d_out, n * 4, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_exact_combine_host(const float *down, const uint64_t *pair_to_row, const float *weights,
+                                         const float *shared_gate, const float *shared, size_t tokens, size_t top_k,
+                                         size_t hidden, float *routed, float *y, uint32_t *error_word) {
+    if (!error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!down || !pair_to_row || !weights || !shared_gate || !shared || !routed || !y || !top_k || !hidden)
+        return PF_HIP_E_ARGUMENT;
+    if (tokens * hidden > 0x7fffffffu || tokens * top_k > 0x7fffffffu) return PF_HIP_E_UNSUPPORTED;
+    if (need_device()) return PF_HIP_E_NO_DEVICE;
+    const size_t pairs = tokens * top_k;
+    for (size_t j = 0; j < pairs; j++)
+        if (pair_to_row[j] >= pairs) return PF_HIP_E_ARGUMENT;
+    auto pad = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t db = pad(pairs * hidden * 4), pb = pad(pairs * 8), wb = pad(pairs * 4), gb = pad(tokens * 4),
+                 hb = pad(tokens * hidden * 4);
+    DeviceBlock blk;
+    HIP_TRY(hipMalloc((void **)&blk.p, db + pb + wb + gb + 3 * hb + 256));
+    uint8_t *at = blk.p;
+    float *d_down = (float *)at; at += db;
+    uint64_t *d_p2r = (uint64_t *)at; at += pb;
+    float *d_w = (float *)at; at += wb;
+    float *d_sa = (float *)at; at += gb;
+    float *d_shared = (float *)at; at += hb;
+    float *d_routed = (float *)at; at += hb;
+    float *d_y = (float *)at; at += hb;
+    uint32_t *d_err = (uint32_t *)at;
+    HIP_TRY(hipMemcpy(d_down, down, pairs * hidden * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(d_p2r, pair_to_row, pairs * 8, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(d_w, weights, pairs * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(d_sa, shared_gate, tokens * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemcpy(d_shared, shared, tokens * hidden * 4, hipMemcpyHostToDevice));
+    HIP_TRY(hipMemset(d_err, 0, 256));
+    pf_launch_exact_combine(d_down, d_p2r, d_w, d_sa, d_shared, d_routed, d_y, (int)tokens, (int)top_k, (int)hidden, d_err,
+                            nullptr);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, d_err, 4, hipMemcpyDeviceToHost));
+    // the sums are returned even when flagged: the caller decides which of the two stages failed
+    HIP_TRY(hipMemcpy(routed, d_routed, tokens * hidden * 4, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(y, d_y, tokens * hidden * 4, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
 extern "C" int pf_hip_packed_decode_row_host(uint32_t gguf_type, const void *row, size_t row_bytes, size_t k_storage,
                                              float *out, uint32_t *error_word) {
     if (!error_word) return PF_HIP_E_ARGUMENT;

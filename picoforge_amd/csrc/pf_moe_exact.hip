@@ -122,3 +122,59 @@ void pf_launch_exact_decode(uint32_t type, const uint8_t *d_row, int k_storage, 
     hipLaunchKernelGGL(pf_k_exact_decode, dim3((k_storage + 255) / 256), dim3(256), 0, stream, type, d_row, k_storage,
                        d_out, d_error, grid);
 }
+
+// ---- the block's elementwise steps in the reference's order --------------------------------------
+// op 0: SiLU (src/qwen4_base.c:76-91 with divisor and multiplier 1), op 1: sigmoid, op 2: a[j] *= b[j]
+// (src/qwen4_moe.c:327-330).  A nonfinite input or result sets the error word.
+__global__ void pf_k_exact_elementwise(int op, const float *a, const float *b, float *out, size_t n, uint32_t *error) {
+    const size_t j = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    const float v = a[j];
+    float r;
+    if (op == 2) r = mul_rn(v, b[j]);
+    else {
+        r = pf_sigmoid_libm(div_rn(v, 1.0f));
+        if (op == 0) r = mul_rn(v, r);
+        r = mul_rn(r, 1.0f);
+    }
+    out[j] = r;
+    if (!pf_finite(r) || (op != 2 && !pf_finite(v))) atomicOr(error, PF_HIP_ERR_NONFINITE);
+}
+
+// src/qwen4_moe.c:350-368: per (row, col) the slot-order sum of weight * down row, then the gated shared
+// row added.  routed receives the first sum (the observer's stage 11), y the finished value.
+__global__ void pf_k_exact_combine(const float *down, const uint64_t *pair_to_row, const float *weights, const float *sa,
+                                   const float *shared, float *routed, float *y, int tokens, int top_k, int hidden,
+                                   uint32_t *error) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)tokens * hidden) return;
+    const size_t row = i / hidden, col = i % hidden;
+    float sum = 0.0f;
+    bool bad = false;
+    for (int slot = 0; slot < top_k; slot++) {
+        const size_t pair = row * top_k + slot;
+        const float term = mul_rn(weights[pair], down[pair_to_row[pair] * hidden + col]);
+        sum = add_rn(sum, term);
+        bad |= !pf_finite(term) || !pf_finite(sum);
+    }
+    routed[i] = sum;
+    const float term = mul_rn(sa[row], shared[i]);
+    const float out = add_rn(sum, term);
+    bad |= !pf_finite(term) || !pf_finite(out);
+    y[i] = out;
+    if (bad) atomicOr(error, PF_HIP_ERR_NONFINITE);
+}
+
+void pf_launch_exact_elementwise(int op, const float *d_a, const float *d_b, float *d_out, size_t n, uint32_t *d_error,
+                                 hipStream_t stream) {
+    if (n) hipLaunchKernelGGL(pf_k_exact_elementwise, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, op, d_a, d_b,
+                              d_out, n, d_error);
+}
+
+void pf_launch_exact_combine(const float *d_down, const uint64_t *d_pair_to_row, const float *d_weights, const float *d_sa,
+                             const float *d_shared, float *d_routed, float *d_y, int tokens, int top_k, int hidden,
+                             uint32_t *d_error, hipStream_t stream) {
+    const size_t n = (size_t)tokens * hidden;
+    if (n) hipLaunchKernelGGL(pf_k_exact_combine, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, d_down,
+                              d_pair_to_row, d_weights, d_sa, d_shared, d_routed, d_y, tokens, top_k, hidden, d_error);
+}

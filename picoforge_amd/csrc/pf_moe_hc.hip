@@ -14,12 +14,7 @@
 #include <math.h>
 
 // src/qwen4_cpu_internal.h:103-106 with the C library's expf reproduced bit for bit
-__device__ __forceinline__ float hc_sigmoid(float x) {
-#pragma clang fp contract(off)
-    // both branches of the CPU form need expf(-|x|): 1 / (1 + e) for x >= 0, e / (1 + e) below
-    const float e = pf_expf_libm(-fabsf(x));
-    return (x >= 0.0f ? 1.0f : e) / (1.0f + e);
-}
+__device__ __forceinline__ float hc_sigmoid(float x) { return pf_sigmoid_libm(x); }
 
 template <int V> struct HcVec;
 template <> struct HcVec<1> { typedef float type; };

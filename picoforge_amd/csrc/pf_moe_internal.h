@@ -143,6 +143,11 @@ void pf_launch_exact_matmul(uint32_t type, const uint8_t *d_w, size_t row_bytes,
                             hipStream_t stream);
 void pf_launch_exact_decode(uint32_t type, const uint8_t *d_row, int k_storage, float *d_out, uint32_t *d_error,
                             const uint64_t *grid, hipStream_t stream);
+void pf_launch_exact_elementwise(int op, const float *d_a, const float *d_b, float *d_out, size_t n, uint32_t *d_error,
+                                 hipStream_t stream);
+void pf_launch_exact_combine(const float *d_down, const uint64_t *d_pair_to_row, const float *d_weights, const float *d_sa,
+                             const float *d_shared, float *d_routed, float *d_y, int tokens, int top_k, int hidden,
+                             uint32_t *d_error, hipStream_t stream);
 // pf_moe_decode.hip
 bool pf_decode_supported(const PfHipMoeDesc &d);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);

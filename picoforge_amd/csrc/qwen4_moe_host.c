@@ -25,6 +25,8 @@ struct Qwen4Moe {
     PfHipMoe *device;
     PfHipMoeDesc desc;
     bool host_spans;   /* the caller still holds the weight bytes at w[].span (the reference's contract) */
+    FILE *route_log;   /* PF_ROUTE_LOG: this layer's routed ids, one record per forward */
+    uint64_t route_pos;
 };
 
 struct Qwen4MoeWork {
@@ -55,6 +57,33 @@ static Qwen4Status admit_config(const Qwen4MoeConfig *c, Qwen4Error *err) {
         !c->shared_intermediate || c->down_physical < c->intermediate)
         return moe_status(err, QW4_RANGE, "invalid MoE dimensions");
     return QW4_OK;
+}
+
+/* ---- routing trace (the per-layer part of QW4_ROUTE_LOG, src/qwen4_forward_gpu.m:62-65,369-376,894-900) ----
+ * Off unless PF_ROUTE_LOG is set.  The n-th layer this process creates (n from 0) appends to the new
+ * file "<PF_ROUTE_LOG>.<n>" one record per forward in the reference's record format with one layer:
+ * uint32 pos, count, layers = 1, top_k, then uint32 ids [count][top_k]; pos is the number of tokens
+ * the layer has been given before the call.  Never read by the forward itself. */
+static unsigned route_log_layers;
+
+static Qwen4Status route_log_open(Qwen4Moe *m, Qwen4Error *err) {
+    const char *prefix = getenv("PF_ROUTE_LOG");
+    if (!prefix || !*prefix) return QW4_OK;
+    char path[4096];
+    if (snprintf(path, sizeof path, "%s.%u", prefix, route_log_layers) >= (int)sizeof path)
+        return moe_status(err, QW4_INVALID_ARGUMENT, "PF_ROUTE_LOG path too long");
+    m->route_log = fopen(path, "wbx");
+    if (!m->route_log) return moe_status(err, QW4_IO, "route log (PF_ROUTE_LOG.<layer> must name a new file)");
+    route_log_layers++;
+    return QW4_OK;
+}
+
+static void route_log_append(Qwen4Moe *m, const uint32_t *ids, size_t pitch_words, size_t tokens) {
+    const uint32_t head[4] = {(uint32_t)m->route_pos, (uint32_t)tokens, 1u, m->cfg.top_k};
+    fwrite(head, 4, 4, m->route_log);
+    for (size_t t = 0; t < tokens; t++) fwrite(ids + t * pitch_words, 4, m->cfg.top_k, m->route_log);
+    fflush(m->route_log);
+    m->route_pos += tokens;
 }
 
 /* ---- create / destroy ------------------------------------------------------ */
@@ -101,12 +130,18 @@ Qwen4Status qwen4_moe_create(const Qwen4MoeConfig *c, const Qwen4MoeWeights *wei
     m->refs = 1;
     m->alive = true;
     m->host_spans = true;
+    Qwen4Status st = route_log_open(m, err);
+    if (st) { pf_hip_moe_destroy(m->device); free(m); return st; }
     *out = m;
     return moe_status(err, QW4_OK, "");
 }
 
 static void moe_unref(Qwen4Moe *m) {
-    if (m && --m->refs == 0) { pf_hip_moe_destroy(m->device); free(m); }
+    if (m && --m->refs == 0) {
+        if (m->route_log) fclose(m->route_log);
+        pf_hip_moe_destroy(m->device);
+        free(m);
+    }
 }
 void qwen4_moe_destroy(Qwen4Moe *m) {
     if (m && m->alive) { m->alive = false; moe_unref(m); }
@@ -307,6 +342,143 @@ Qwen4Status qw4_moe_group_pairs(const Qwen4MoeConfig *c, Qwen4U32Mut ids, QW4Moe
     return st;
 }
 
+/* ---- the observed forward (src/qwen4_moe.c:305-382) -------------------------------------------
+ * With an observer set the block runs as the reference's sequence of operators, one device call each
+ * in the reference's evaluation order, in microbatches of at most 32 tokens, and every stage's input
+ * and output rows are handed to the observer from host staging memory.  This is the slow, bit-identical
+ * mode: it reads each expert's bytes from the caller's host views on every call, so it needs them. */
+typedef struct {
+    float *z, *p, *scores, *gather, *down, *gate, *up, *act, *shared, *sg, *sa, *routed, *yd;
+    uint32_t *ids;
+    size_t *offsets, *cursors, *p2r, *r2p;
+} Stage;
+
+static Qwen4F32Mut rows_of(float *data, size_t rows, size_t cols) {
+    return (Qwen4F32Mut){.data = data, .capacity_bytes = rows * cols * 4, .rank = 2, .dim = {rows, cols},
+                         .stride_bytes = {cols * 4, 4}};
+}
+static Qwen4F32 ro(Qwen4F32Mut v) {
+    Qwen4F32 r = {.data = v.data, .capacity_bytes = v.capacity_bytes, .rank = v.rank};
+    memcpy(r.dim, v.dim, sizeof r.dim);
+    memcpy(r.stride_bytes, v.stride_bytes, sizeof r.stride_bytes);
+    return r;
+}
+static void trace(Qwen4MoeWork *w, size_t stage, size_t expert, size_t token, Qwen4F32 in, Qwen4F32Mut out) {
+    w->observer(w->observer_ctx, stage, expert, token, in, ro(out));
+}
+static Qwen4Status linear(Qwen4MoeWork *w, size_t stage, size_t expert, size_t token, Qwen4F32 x, Qwen4F32Mut y,
+                          Qwen4Error *err) {
+    TRY(qw4_packed_matmul(&w->owner->w[stage], expert, x, y, err));
+    trace(w, stage, expert, token, x, y);
+    return QW4_OK;
+}
+static Qwen4Status elementwise(int op, const float *a, const float *b, size_t n, float *out, const char *what,
+                               Qwen4Error *err) {
+    uint32_t word = 0;
+    int rc = pf_hip_exact_elementwise_host(op, a, b, n, out, &word);
+    if (rc) return pf_device_status(rc, err, "qwen4_moe");
+    if (word & PF_HIP_ERR_NONFINITE) return moe_status(err, QW4_NONFINITE, what);
+    return word ? moe_status(err, QW4_GPU_ERROR, "device error word") : QW4_OK;
+}
+
+static Qwen4Status observed_expert(Qwen4MoeWork *w, Stage *b, size_t expert, size_t token, Qwen4F32 x, Qwen4F32Mut y,
+                                   bool shared, Qwen4Error *err) {
+    const Qwen4MoeConfig *c = &w->owner->cfg;
+    const size_t n = x.dim[0], i = shared ? c->shared_intermediate : c->intermediate;
+    const size_t who = shared ? SIZE_MAX : expert;
+    Qwen4F32Mut g = rows_of(b->gate, n, i), u = rows_of(b->up, n, i), a = rows_of(b->act, n, i);
+    TRY(linear(w, shared ? 4 : 1, expert, token, x, g, err));
+    TRY(linear(w, shared ? 5 : 2, expert, token, x, u, err));
+    TRY(elementwise(0, g.data, NULL, n * i, a.data, "activation overflow", err));
+    trace(w, 8, who, token, ro(g), a);
+    TRY(elementwise(2, a.data, u.data, n * i, a.data, "gate/up overflow", err));
+    trace(w, 9, who, token, ro(u), a);
+    return linear(w, shared ? 6 : 3, expert, token, ro(a), y, err);
+}
+
+static Qwen4Status observed_batch(Qwen4MoeWork *w, Stage *b, Qwen4F32 x, Qwen4F32Mut y, size_t token, Qwen4Error *err) {
+    const Qwen4MoeConfig *c = &w->owner->cfg;
+    const size_t t = x.dim[0], e = c->experts, k = c->top_k, h = c->hidden_size, pairs = t * k;
+    Qwen4F32Mut z = rows_of(b->z, t, e), p = rows_of(b->p, t, e);
+    Qwen4MoeRoutes routes = {{b->ids, pairs * 4, t, k, k * 4}, rows_of(b->scores, t, k)};
+    TRY(linear(w, 0, 0, token, x, z, err));
+    TRY(qwen4_moe_route(c, ro(z), routes, p, err));
+    QW4MoeGrouping g = {b->offsets, (e + 1) * sizeof(size_t), b->cursors, e * sizeof(size_t), b->p2r, b->r2p,
+                        pairs * sizeof(size_t), pairs * sizeof(size_t)};
+    TRY(qw4_moe_group_pairs(c, routes.ids, g, err));
+    for (size_t row = 0; row < pairs; row++)
+        memcpy(b->gather + row * h, x.data + (g.row_to_pair[row] / k) * (x.stride_bytes[0] / 4), h * 4);
+    for (size_t expert = 0; expert < e; expert++) {
+        const size_t first = g.offsets[expert], n = g.offsets[expert + 1] - first;
+        if (!n) continue;
+        TRY(observed_expert(w, b, expert, token, ro(rows_of(b->gather + first * h, n, h)), rows_of(b->down + first * h, n, h),
+                            false, err));
+    }
+    Qwen4F32Mut shared = rows_of(b->shared, t, h), sg = rows_of(b->sg, t, 1), sa = rows_of(b->sa, t, 1);
+    TRY(observed_expert(w, b, 0, token, x, shared, true, err));
+    TRY(linear(w, 7, 0, token, x, sg, err));
+    TRY(elementwise(1, sg.data, NULL, t, sa.data, "activation overflow", err));
+    trace(w, 10, SIZE_MAX, token, ro(sg), sa);
+    uint32_t word = 0;
+    _Static_assert(sizeof(size_t) == sizeof(uint64_t), "the shim exchanges 64-bit indices");
+    int rc = pf_hip_exact_combine_host(b->down, (const uint64_t *)g.pair_to_row, b->scores, b->sa, b->shared, t, k, h,
+                                       b->routed, b->yd, &word);
+    if (rc) return pf_device_status(rc, err, "qwen4_moe");
+    if (word & ~PF_HIP_ERR_NONFINITE) return moe_status(err, QW4_GPU_ERROR, "device error word");
+    const size_t ys = y.stride_bytes[0] / 4;
+    if (word)   /* a nonfinite routed sum fails before stage 11, anything later after it */
+        for (size_t j = 0; j < t * h; j++)
+            if (!isfinite(b->routed[j])) return moe_status(err, QW4_NONFINITE, "routed reduction overflow");
+    for (size_t row = 0; row < t; row++) memcpy(y.data + row * ys, b->routed + row * h, h * 4);
+    trace(w, 11, SIZE_MAX, token, x, y);
+    if (word) return moe_status(err, QW4_NONFINITE, "shared sum overflow");
+    for (size_t row = 0; row < t; row++) memcpy(y.data + row * ys, b->yd + row * h, h * 4);
+    trace(w, 12, SIZE_MAX, token, x, y);
+    return QW4_OK;
+}
+
+static Qwen4Status observed_forward(Qwen4MoeWork *w, Qwen4F32 x, Qwen4F32Mut y, Qwen4MoeRoutes *routes, Qwen4Error *err) {
+    const Qwen4MoeConfig *c = &w->owner->cfg;
+    if (!w->owner->host_spans) return moe_status(err, QW4_BAD_STATE, "the observer needs the host weight bytes");
+    const size_t T = x.dim[0], micro = w->cap < 32 ? w->cap : 32, e = c->experts, k = c->top_k, h = c->hidden_size;
+    const size_t i = c->intermediate > c->shared_intermediate ? c->intermediate : c->shared_intermediate;
+    const size_t pairs = micro * k;
+    const size_t floats[13] = {micro * e, micro * e, pairs, pairs * h, pairs * h, micro * i, micro * i, micro * i,
+                               micro * h, micro, micro, micro * h, micro * h};
+    size_t total = 0;
+    for (size_t j = 0; j < 13; j++) total += floats[j];
+    float *arena = malloc((total ? total : 1) * 4);
+    uint32_t *ids = malloc((pairs ? pairs : 1) * 4);
+    size_t *index = malloc((2 * e + 1 + 2 * pairs) * sizeof(size_t));
+    Qwen4Status st = QW4_OK;
+    if (!arena || !ids || !index) st = moe_status(err, QW4_OOM, "observer staging");
+    if (!st) {
+        float *at = arena;
+        Stage b = {.ids = ids, .offsets = index, .cursors = index + e + 1, .p2r = index + 2 * e + 1,
+                   .r2p = index + 2 * e + 1 + pairs};
+        float **fields[13] = {&b.z, &b.p, &b.scores, &b.gather, &b.down, &b.gate, &b.up, &b.act, &b.shared, &b.sg, &b.sa,
+                              &b.routed, &b.yd};
+        for (size_t j = 0; j < 13; j++) { *fields[j] = at; at += floats[j]; }
+        for (size_t start = 0; start < T && !st;) {
+            const size_t n = T - start < micro ? T - start : micro;
+            Qwen4F32 bx = x;
+            Qwen4F32Mut by = y;
+            bx.data += start * (x.stride_bytes[0] / 4); bx.capacity_bytes -= start * x.stride_bytes[0]; bx.dim[0] = n;
+            by.data += start * (y.stride_bytes[0] / 4); by.capacity_bytes -= start * y.stride_bytes[0]; by.dim[0] = n;
+            st = observed_batch(w, &b, bx, by, start, err);
+            if (!st && routes)
+                for (size_t row = 0; row < n; row++) {
+                    memcpy(routes->ids.data + (start + row) * (routes->ids.row_stride_bytes / 4), b.ids + row * k, k * 4);
+                    memcpy(routes->weights.data + (start + row) * (routes->weights.stride_bytes[0] / 4), b.scores + row * k,
+                           k * 4);
+                }
+            start += n;
+        }
+    }
+    free(arena); free(ids); free(index);
+    return st ? st : moe_status(err, QW4_OK, "");
+}
+
 /* ---- forward (src/qwen4_moe.c:384-431) -------------------------------------------------- */
 Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen4MoeRoutes *routes, Qwen4MoeWork *w,
                               Qwen4Error *err) {
@@ -340,27 +512,34 @@ Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen
         for (size_t col = 0; col < H; col++)
             if (!isfinite(x.data[row * xs + col])) return moe_status(err, QW4_NONFINITE, "nonfinite input");
     if (!T) return moe_status(err, QW4_OK, "");
+    /* the routing trace needs the ids also when the caller did not ask for them */
+    Qwen4MoeRoutes traced;
+    void *trace_memory = NULL;
+    if (m->route_log && !routes) {
+        trace_memory = malloc(T * K * 8);
+        if (!trace_memory) return moe_status(err, QW4_OOM, "route log staging");
+        traced = (Qwen4MoeRoutes){{trace_memory, T * K * 4, T, K, K * 4}, rows_of((float *)trace_memory + T * K, T, K)};
+        routes = &traced;
+    }
     w->busy = true;
-    uint32_t word = 0;
-    int rc = pf_hip_moe_forward_host(m->device, w->device, x.data, x.stride_bytes[0], y.data, y.stride_bytes[0],
-                                     routes ? routes->ids.data : NULL, routes ? routes->ids.row_stride_bytes : 0,
-                                     routes ? routes->weights.data : NULL,
-                                     routes ? routes->weights.stride_bytes[0] : 0, T, &word);
+    Qwen4Status st;
+    if (w->observer) st = observed_forward(w, x, y, routes, err);
+    else {
+        uint32_t word = 0;
+        int rc = pf_hip_moe_forward_host(m->device, w->device, x.data, x.stride_bytes[0], y.data, y.stride_bytes[0],
+                                         routes ? routes->ids.data : NULL, routes ? routes->ids.row_stride_bytes : 0,
+                                         routes ? routes->weights.data : NULL,
+                                         routes ? routes->weights.stride_bytes[0] : 0, T, &word);
+        if (rc) st = pf_device_status(rc, err, "qwen4_moe");
+        else if (word & PF_HIP_ERR_NONFINITE) st = moe_status(err, QW4_NONFINITE, "nonfinite value in the MoE block");
+        else if (word) st = moe_status(err, QW4_GPU_ERROR, "device error word");
+        else st = moe_status(err, QW4_OK, "");
+    }
     w->busy = false;
-    if (rc || word) {
-        w->failed = true;
-        if (rc) return pf_device_status(rc, err, "qwen4_moe");
-        if (word & PF_HIP_ERR_NONFINITE) return moe_status(err, QW4_NONFINITE, "nonfinite value in the MoE block");
-        return moe_status(err, QW4_GPU_ERROR, "device error word");
-    }
-    if (w->observer) {
-        /* stage 12 of src/qwen4_moe_internal.h:9-12: the finished block output */
-        Qwen4F32 out = {.data = y.data, .capacity_bytes = y.capacity_bytes, .rank = 2};
-        memcpy(out.dim, y.dim, sizeof out.dim);
-        memcpy(out.stride_bytes, y.stride_bytes, sizeof out.stride_bytes);
-        w->observer(w->observer_ctx, 12, SIZE_MAX, 0, x, out);
-    }
-    return moe_status(err, QW4_OK, "");
+    if (st) w->failed = true;
+    else if (m->route_log) route_log_append((Qwen4Moe *)m, routes->ids.data, routes->ids.row_stride_bytes / 4, T);
+    free(trace_memory);
+    return st;
 }
 
 /* ---- the block between its two hyper-connection steps (src/qwen4_forward.c:362-367) ------------
@@ -401,6 +580,14 @@ Qwen4Status pf_moe_forward_hc(const Qwen4Moe *m, const Qwen4HcShape *s, Qwen4F32
             if (r[i].lo < r[j].hi && r[j].lo < r[i].hi)
                 return moe_status(err, QW4_INVALID_ARGUMENT, "overlapping views");
     if (!T) return moe_status(err, QW4_OK, "");
+    Qwen4MoeRoutes traced;
+    void *trace_memory = NULL;
+    if (m->route_log && !routes) {
+        trace_memory = malloc(T * K * 8);
+        if (!trace_memory) return moe_status(err, QW4_OOM, "route log staging");
+        traced = (Qwen4MoeRoutes){{trace_memory, T * K * 4, T, K, K * 4}, rows_of((float *)trace_memory + T * K, T, K)};
+        routes = &traced;
+    }
     w->busy = true;
     uint32_t word = 0;
     int rc = pf_hip_moe_forward_hc_host(m->device, w->device, normed.data, normed.stride_bytes[0],
@@ -411,6 +598,8 @@ Qwen4Status pf_moe_forward_hc(const Qwen4Moe *m, const Qwen4HcShape *s, Qwen4F32
                                         routes ? routes->weights.data : NULL,
                                         routes ? routes->weights.stride_bytes[0] : 0, &word);
     w->busy = false;
+    if (!rc && !word && m->route_log) route_log_append((Qwen4Moe *)m, routes->ids.data, routes->ids.row_stride_bytes / 4, T);
+    free(trace_memory);
     if (rc || word) {
         w->failed = true;
         if (rc) return pf_device_status(rc, err, "qwen4_moe");

@@ -145,6 +145,23 @@ class MoeLayer:
             self._raise(st)
         return st, ids, w
 
+    def observe(self, record=None):
+        """Set (record: a list to append to) or clear the forward's observer.  Each entry is
+        (stage, expert, token, input rows, output rows) with the rows copied out during the callback;
+        expert is -1 where the library reports SIZE_MAX."""
+        def view(v):
+            rows, cols, pitch = v.dim[0], v.dim[1], v.stride_bytes[0] // 4
+            if not rows or not cols:
+                return np.zeros((rows, cols), np.float32)
+            flat = np.frombuffer((C.c_float * ((rows - 1) * pitch + cols)).from_address(v.data), dtype=np.float32)
+            return np.stack([flat[r * pitch:r * pitch + cols].copy() for r in range(rows)])
+
+        def callback(_ctx, stage, expert, token, a, b):
+            record.append((stage, -1 if expert == C.c_size_t(-1).value else expert, token, view(a), view(b)))
+
+        self._observer = abi.OBSERVER(callback) if record is not None else C.cast(None, abi.OBSERVER)
+        self.api.observe(self.work, self._observer, None)
+
     def device_handles(self):
         """(PfHipMoe*, PfHipWork*) behind this layer: shipped library only."""
         return self.api.device_layer(self.handle), self.api.device_work(self.work)
