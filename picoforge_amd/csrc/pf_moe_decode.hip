@@ -924,11 +924,28 @@ __device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, const Q4TilePlan
     partial[(wave - 1) * 64 + lane] = total;
 }
 
+// The kernels below take one token per value of blockIdx.y: the argument block's per-token pointers moved to token t
+// (the output row stays indexed by the token: the output helpers take it as an argument).
+__device__ __forceinline__ void q4t_at_token(PfKernelArgs &a, int t) {
+    const size_t widest = a.inter > a.shared_inter ? a.inter : a.shared_inter;
+    a.x += (size_t)t * a.x_pitch;
+    a.logits += (size_t)t * a.experts;
+    a.logit_ssq += (size_t)t * a.experts;
+    a.ids += (size_t)t * a.top_k;
+    a.route_weights += (size_t)t * a.top_k;
+    a.act += (size_t)t * a.top_k * a.inter;
+    a.shared_act += (size_t)t * a.shared_inter;
+    a.shared_scale += t;
+    a.ximg += (size_t)t * pf_image2_words(a.hidden);
+    a.aimg += (size_t)t * (a.top_k + 1) * pf_image2_words(widest);
+}
+
 template <int NPL>
 __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
     __shared__ uint32_t early_expert;
+    q4t_at_token(a, (int)blockIdx.y);
     const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     float *partial = reinterpret_cast<float *>(lds);   // [15 waves][64 lanes]
@@ -1010,12 +1027,14 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
             for (int q = threadIdx.x; q < K; q += blockDim.x) {
                 a.ids[q] = R.ids[q];
                 a.route_weights[q] = R.weights[q];
-                a.uniq[1 + q] = R.ids[q];
-                a.uniq[1 + K + q] = q;
-                a.uniq[1 + 2 * K + q] = 1u;
+                if (gridDim.y == 1) {   // the table of unique experts: read by the other down kernel, which runs after this one only for one token
+                    a.uniq[1 + q] = R.ids[q];
+                    a.uniq[1 + K + q] = q;
+                    a.uniq[1 + 2 * K + q] = 1u;
+                }
             }
             if (threadIdx.x == 0) {
-                a.uniq[0] = K;
+                if (gridDim.y == 1) a.uniq[0] = K;
                 if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
                 if (R.close_mask) atomicAdd(a.exact_rows, 1u);
             }
@@ -1170,6 +1189,8 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a);
 __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
     __shared__ float partial[17][8];
     extern __shared__ int images[];   // [slot][image words of the widest activation row]
+    const int token = (int)blockIdx.y;
+    q4t_at_token(a, token);
     const int H = a.hidden, K = a.top_k, lane = pf_lane();
     const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const bool shared = s == K;
@@ -1188,7 +1209,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
         e = 0;
     }
     PfOutputRegs out_regs;
-    if ((int)threadIdx.x < 8) pf_output_prefetch(a, 0, n_base + threadIdx.x, out_regs);
+    if ((int)threadIdx.x < 8) pf_output_prefetch(a, token, n_base + threadIdx.x, out_regs);
     const uint8_t *w = (shared ? a.wt[6] : a.wt[3]) + (size_t)e * (shared ? a.expert_bytes[6] : a.expert_bytes[3]);
     const int kblocks = (shared ? a.shared_inter : a.down_physical) / 256, runs = I / 64, groups = I / 32;
     const uint32_t *image = a.aimg + (size_t)s * pf_image2_words(widest);   // slot = unique expert with one token; the shared expert's follows
@@ -1256,7 +1277,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
         for (int slot = 0; slot < 16; slot++)   // slot order, as src/qwen4_moe.c:362-372
             if (slot < K) sum += rw[slot] * partial[slot][threadIdx.x];
         const float y = sum + shared_scale * partial[K][threadIdx.x];
-        if (!pf_output_commit(a, 0, n, y, out_regs)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+        if (!pf_output_commit(a, token, n, y, out_regs)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
 }
 #endif
@@ -1425,13 +1446,19 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     const int rows_next = down_block_rows(H, I), row_blocks_next = (H + rows_next - 1) / rows_next;
     int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
     if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
-    bool rows_as_lanes = false;
-    if constexpr (NT == 1 && FG == PF_Q4_K && FS == PF_Q4_K)
+    bool rows_as_lanes = false, down_as_lanes = false;
+    if constexpr (FG == PF_Q4_K && FS == PF_Q4_K)
         rows_as_lanes = a.wt[1] && a.wt[2] && a.wt[4] && a.wt[5] && I % 32 == 0 && Is % 32 == 0 && 4 * (H / 256) <= 15 * Q4T_ITEMS;
-    if constexpr (NT == 1 && FG == PF_Q4_K && FS == PF_Q4_K) if (rows_as_lanes) {
-        // one token, the tile-ordered copy is there: lanes are weight rows, every workgroup extracts the maxima up to
-        // its own slot from all the logits
-        const dim3 g1(routed_blocks + shared_blocks);
+    if constexpr (FG == PF_Q4_K && FD == PF_Q4_K && FS == PF_Q4_K)
+        down_as_lanes = rows_as_lanes && a.wt[3] && a.wt[6] && H % 32 == 0 && I % 64 == 0 && Is % 64 == 0 && a.down_physical == I;
+    // several tokens: one token per blockIdx.y in both kernels, or neither (the other down kernel reads a table of the
+    // tokens' unique experts that this gate/up kernel does not build)
+    if (NT > 1 && !down_as_lanes) rows_as_lanes = false;
+    if constexpr (FG == PF_Q4_K && FS == PF_Q4_K) if (rows_as_lanes) {
+        // the tile-ordered copy is there: lanes are weight rows, every workgroup extracts the maxima up to
+        // its own slot from all of its token's logits
+        const dim3 g1(K * (I / tile) + shared_blocks, NT);
+        const int routed_blocks = K * (I / tile);
         const int all = (E + 63) / 64;
         const size_t lds = (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
         if (all <= 1) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<1>, g1, dim3(1024), lds, stream, a, routed_blocks);
@@ -1449,10 +1476,10 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     }
     if (last < 3) return;
     // kernel 3
-    if constexpr (NT == 1 && FG == PF_Q4_K && FD == PF_Q4_K && FS == PF_Q4_K)
-        if (rows_as_lanes && a.wt[3] && a.wt[6] && H % 32 == 0 && I % 64 == 0 && Is % 64 == 0 && a.down_physical == I) {
+    if constexpr (FG == PF_Q4_K && FD == PF_Q4_K && FS == PF_Q4_K)
+        if (down_as_lanes) {
             const size_t widest = I > Is ? I : Is;
-            hipLaunchKernelGGL(pf_k_dec_down_q4t, dim3(H / 8), dim3(64 * (K + 1)), (size_t)(K + 1) * pf_image2_words(widest) * 4, stream, a);
+            hipLaunchKernelGGL(pf_k_dec_down_q4t, dim3(H / 8, NT), dim3(64 * (K + 1)), (size_t)(K + 1) * pf_image2_words(widest) * 4, stream, a);
             return;
         }
     const int rows_per_block = down_block_rows(H, I), row_blocks = (H + rows_per_block - 1) / rows_per_block;

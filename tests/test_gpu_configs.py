@@ -10,7 +10,7 @@ import pytest
 import picoforge_amd as pf
 from picoforge_amd import abi, workloads
 
-from helpers import ATOL, RTOL, assert_parity, call_matmul, call_route
+from helpers import ATOL, RTOL, assert_parity, call_matmul, call_route, forward_with, make_layer_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -136,3 +136,16 @@ def test_views_over_released_weight_bytes(product, oracle):
         assert st == abi.QW4_OK, err.detail
         err_abs = np.abs(y - y0)
         assert (err_abs <= ATOL + RTOL * np.abs(y0)).all()
+
+
+@pytest.mark.parametrize("gtype", [abi.GGUF_Q4_K, abi.GGUF_IQ2_XXS])
+@pytest.mark.parametrize("tokens", [8, 32])
+def test_batches_between_decode_and_prefill_match_oracle(product, oracle, gtype, tokens):
+    """5 to 32 rows at the measured shape (a long verify batch, a short prompt): more rows than the decode kernels
+    take, few enough that nearly every routed expert sees one row.  Every row against the CPU path."""
+    cfg = workloads.measured_config()
+    weights, x = make_layer_inputs(cfg, gtype, tokens, seed=40 + tokens)
+    print(f"full shape, {tokens} rows, type={gtype}", flush=True)
+    want = forward_with(oracle, cfg, weights, x)
+    y, ids, w = forward_with(product, cfg, weights, x)
+    assert_parity(y, ids, w, *want, label=f"{tokens} rows")
