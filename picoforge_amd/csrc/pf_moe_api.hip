@@ -290,6 +290,10 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     memset(&c, 0, sizeof c);
     const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden, I = d->inter;
     const size_t Td = T < PF_DECODE_MAX_TOKENS ? T : PF_DECODE_MAX_TOKENS;   // tokens per decode launch
+    // ... and per launch of the kernels for tile-ordered Q4_K (whether the copies are kept is not known here)
+    bool q4k = true;
+    for (int t = 1; t <= 6; t++) q4k &= d->type[t] == PF_Q4_K;
+    const size_t Tt = !q4k ? Td : T < PF_TILE_DECODE_MAX_TOKENS ? T : PF_TILE_DECODE_MAX_TOKENS;
     size_t want[W_COUNT];
     want[W_LOGITS] = T * E * 4;
     want[W_SSQ] = T * E * 4;
@@ -306,8 +310,9 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_FLAGS] = (T + 1) * 4;
     {   // digit images of the decode path: the token rows; the activation rows of every (unique expert, token) and the shared expert's
         const size_t widest = I > d->shared_inter ? I : d->shared_inter;
-        want[W_XIMG] = Td * pf_image2_words(H) * 4;
-        want[W_AIMG] = (Td * K * Td + Td) * pf_image2_words(widest) * 4;
+        const size_t rows = Td * K * Td + Td > Tt * (K + 1) ? Td * K * Td + Td : Tt * (K + 1);
+        want[W_XIMG] = Tt * pf_image2_words(H) * 4;
+        want[W_AIMG] = rows * pf_image2_words(widest) * 4;
     }
     // prefill path: fp16 copies, per-row scales, down products in expert order, grouping tables
     const bool prefill = T > PF_DECODE_MAX_TOKENS && pf_prefill_supported(*d);
@@ -465,6 +470,11 @@ struct HcTarget {   // residual streams to inject into instead of writing y
     int streams;
 };
 
+// Most tokens the decode kernels take in one forward of this layer.
+static size_t decode_limit(const PfHipMoe *moe) {
+    return pf_decode_tile_layer(moe->desc, moe->w_tiled) ? PF_TILE_DECODE_MAX_TOKENS : PF_DECODE_MAX_TOKENS;
+}
+
 static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch, float *d_y,
                            size_t y_pitch, size_t tokens, const HcTarget *hc, hipStream_t s) {
     const PfHipMoeDesc *d = &moe->desc;
@@ -475,7 +485,7 @@ static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_
         a.hc_token_pitch = hc->token_pitch; a.hc_stream_pitch = hc->stream_pitch;
     }
     const bool aligned = (x_pitch % 4 == 0) && ((uintptr_t)d_x % 16 == 0);
-    if (moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS && aligned && !work->force_general) {
+    if (moe->decode_ready && tokens <= decode_limit(moe) && aligned && !work->force_general) {
         pf_launch_decode(a, (int)tokens, s, work->stage_limit);
     } else if (moe->prefill_ready && work->down && tokens > PF_DECODE_MAX_TOKENS && aligned && !work->force_general) {
         pf_launch_prefill(a, (int)tokens, s, work->stage_limit);
@@ -496,7 +506,7 @@ static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_
 // 2 the matrix-core prefill kernels, 0 the general kernels.
 extern "C" int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t tokens) {
     if (!moe || !work || work->force_general) return 0;
-    if (moe->decode_ready && tokens <= PF_DECODE_MAX_TOKENS) return 1;
+    if (moe->decode_ready && tokens <= decode_limit(moe)) return 1;
     if (moe->prefill_ready && work->down && tokens > PF_DECODE_MAX_TOKENS) return 2;
     return 0;
 }

@@ -474,19 +474,25 @@ template <int FMT> __host__ __device__ constexpr int table_words() { return FMT 
 // last block's first wave the shared router row (its sigmoid scales the shared expert).
 #define ROUTER_CHUNKS 10   // 16-byte pieces of a router row per lane: hidden <= 2560
 template <int NT>
-__global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks) {
+__global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks, int tokens) {
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     if ((int)blockIdx.x > router_blocks) {
         // workgroups beyond the router's (launched where the next kernel reads them): the tokens' two-digit images,
         // 2048 values per workgroup
         const int per_token = (H + 2047) / 2048, q = (int)blockIdx.x - router_blocks - 1;
         const int t = q / per_token, j = (q % per_token) * 256 + (int)threadIdx.x;
-        if (t < NT && j < H / 8) {
+        if (blockIdx.y == 0 && t < tokens && j < H / 8) {
             const float4 *row = reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch);
             image2_chunk(a.ximg + (size_t)t * pf_image2_words(H), row[2 * j], row[2 * j + 1], j, H);
         }
         return;
     }
+    // blockIdx.y: the group of NT tokens (more than NT tokens only with the tile-ordered kernels behind this one)
+    const int t0 = NT * (int)blockIdx.y, nt = tokens - t0 < NT ? tokens - t0 : NT;
+    a.x += (size_t)t0 * a.x_pitch;
+    a.logits += (size_t)t0 * E;
+    a.logit_ssq += (size_t)t0 * E;
+    a.shared_scale += t0;
     const bool gate_row = (int)blockIdx.x == router_blocks;
     const int e = blockIdx.x * 4 + wave;
     if (gate_row ? wave != 0 : e >= E) return;
@@ -508,8 +514,8 @@ __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int route
 #pragma unroll
         for (int c = 0; c < ROUTER_CHUNKS; c++) {
             const int i = lane + PF_WAVE * c;
-            xv[c] = i < H / 4 ? reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch)[i]
-                              : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            xv[c] = i < H / 4 && t < nt ? reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch)[i]
+                                        : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
         for (int c = 0; c < ROUTER_CHUNKS; c++) {
@@ -522,7 +528,7 @@ __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int route
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const float z = pf_wave_sum(acc[t]), s2 = pf_wave_sum(sq[t]);
-        if (lane == 0) {
+        if (lane == 0 && t < nt) {
             if (gate_row) {
                 a.shared_scale[t] = pf_sigmoid(z);
                 if (!pf_finite(z)) bad = true;
@@ -941,7 +947,7 @@ __device__ __forceinline__ void q4t_at_token(PfKernelArgs &a, int t) {
 }
 
 template <int NPL>
-__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) {
+__device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
     __shared__ uint32_t early_expert;
@@ -1061,6 +1067,11 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int
         image2_group(a.aimg + (size_t)u * pf_image2_words(widest), act, n0 / 32, I, lane);
     }
 }
+
+// With several tokens there are more workgroups than compute units; two workgroups per compute unit (64 registers a
+// lane) measured slower than one after the other: the products are bound by the vector units, not by waiting.
+template <int NPL>
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) { q4t_gate_up<NPL>(a, routed_blocks); }
 
 // ---- kernel 3: down products and the combine ---------------------------------------------------
 // blockIdx.x = t * row_blocks + nb; one wave per slot plus one for the shared expert; a routed
@@ -1388,13 +1399,14 @@ static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStre
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
 #if PF_DECODE_PART == 0
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream) {
-    // the router's rows, the shared router's row, then the tokens' two-digit images (2048 values per workgroup)
-    const dim3 grid(router_blocks + 1 + tokens * ((a.hidden + 2047) / 2048)), block(256);
+    // the router's rows, the shared router's row, then the tokens' two-digit images (2048 values per workgroup);
+    // beyond four tokens: groups of four along the grid's second dimension
+    const dim3 grid(router_blocks + 1 + tokens * ((a.hidden + 2047) / 2048), (tokens + 3) / 4), block(256);
     switch (tokens) {
-    case 1: hipLaunchKernelGGL((pf_k_dec_router<1>), grid, block, 0, stream, a, router_blocks); break;
-    case 2: hipLaunchKernelGGL((pf_k_dec_router<2>), grid, block, 0, stream, a, router_blocks); break;
-    case 3: hipLaunchKernelGGL((pf_k_dec_router<3>), grid, block, 0, stream, a, router_blocks); break;
-    default: hipLaunchKernelGGL((pf_k_dec_router<4>), grid, block, 0, stream, a, router_blocks); break;
+    case 1: hipLaunchKernelGGL((pf_k_dec_router<1>), grid, block, 0, stream, a, router_blocks, tokens); break;
+    case 2: hipLaunchKernelGGL((pf_k_dec_router<2>), grid, block, 0, stream, a, router_blocks, tokens); break;
+    case 3: hipLaunchKernelGGL((pf_k_dec_router<3>), grid, block, 0, stream, a, router_blocks, tokens); break;
+    default: hipLaunchKernelGGL((pf_k_dec_router<4>), grid, block, 0, stream, a, router_blocks, tokens); break;
     }
 }
 #endif
@@ -1422,6 +1434,39 @@ static void launch_down(const PfKernelArgs &a, dim3 grid, dim3 block, size_t lds
         launch_down_bounded<FD, FS, NT, SPL, 1024>(a, grid, block, lds, stream, row_blocks, rows_per_block, image_pitch);
 }
 
+// Every expert tensor Q4_K with its tile-ordered copy kept, and widths the kernels whose lanes are weight rows
+// cover: those take the layer, one token per grid row, for up to PF_TILE_DECODE_MAX_TOKENS tokens.
+bool pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const tiled[8]);
+#if PF_DECODE_PART == 0
+bool pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const tiled[8]) {
+    for (int t = 1; t <= 6; t++)
+        if (d.type[t] != PF_Q4_K || !tiled[t]) return false;
+    return d.hidden % 256 == 0 && 4 * (d.hidden / 256) <= 15 * Q4T_ITEMS && d.inter % 64 == 0 && d.shared_inter % 64 == 0 &&
+           d.down_physical == d.inter && d.top_k < d.experts && d.top_k <= 15;
+}
+
+static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
+    const int router_blocks = (E + 3) / 4, last = stage_limit ? stage_limit : 3;
+    pf_launch_dec_router(a, tokens, router_blocks, stream);
+    if (last < 2) return;
+    // kernel 2: every workgroup extracts the maxima up to its own slot from all of its token's logits
+    const int routed_blocks = K * (I / 32);
+    const dim3 g1(routed_blocks + Is / 32, tokens);
+    const int all = (E + 63) / 64;
+    const size_t lds = (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+    if (all <= 1) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<1>, g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 2) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<2>, g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 4) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<4>, g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 8) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<8>, g1, dim3(1024), lds, stream, a, routed_blocks);
+    else hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<16>, g1, dim3(1024), lds, stream, a, routed_blocks);
+    if (last < 3) return;
+    const size_t widest = I > Is ? I : Is;
+    hipLaunchKernelGGL(pf_k_dec_down_q4t, dim3(H / 8, tokens), dim3(64 * (K + 1)), (size_t)(K + 1) * pf_image2_words(widest) * 4,
+                       stream, a);
+}
+#endif
+
 // FG: format of the routed gate and up tensors, FD: of the routed down tensor, FS: of the shared expert
 template <int FG, int FD, int FS, int NT, int SPL2>
 static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int stage_limit) {
@@ -1446,42 +1491,13 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     const int rows_next = down_block_rows(H, I), row_blocks_next = (H + rows_next - 1) / rows_next;
     int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
     if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
-    bool rows_as_lanes = false, down_as_lanes = false;
-    if constexpr (FG == PF_Q4_K && FS == PF_Q4_K)
-        rows_as_lanes = a.wt[1] && a.wt[2] && a.wt[4] && a.wt[5] && I % 32 == 0 && Is % 32 == 0 && 4 * (H / 256) <= 15 * Q4T_ITEMS;
-    if constexpr (FG == PF_Q4_K && FD == PF_Q4_K && FS == PF_Q4_K)
-        down_as_lanes = rows_as_lanes && a.wt[3] && a.wt[6] && H % 32 == 0 && I % 64 == 0 && Is % 64 == 0 && a.down_physical == I;
-    // several tokens: one token per blockIdx.y in both kernels, or neither (the other down kernel reads a table of the
-    // tokens' unique experts that this gate/up kernel does not build)
-    if (NT > 1 && !down_as_lanes) rows_as_lanes = false;
-    if constexpr (FG == PF_Q4_K && FS == PF_Q4_K) if (rows_as_lanes) {
-        // the tile-ordered copy is there: lanes are weight rows, every workgroup extracts the maxima up to
-        // its own slot from all of its token's logits
-        const dim3 g1(K * (I / tile) + shared_blocks, NT);
-        const int routed_blocks = K * (I / tile);
-        const int all = (E + 63) / 64;
-        const size_t lds = (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
-        if (all <= 1) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<1>, g1, dim3(1024), lds, stream, a, routed_blocks);
-        else if (all <= 2) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<2>, g1, dim3(1024), lds, stream, a, routed_blocks);
-        else if (all <= 4) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<4>, g1, dim3(1024), lds, stream, a, routed_blocks);
-        else if (all <= 8) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<8>, g1, dim3(1024), lds, stream, a, routed_blocks);
-        else hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<16>, g1, dim3(1024), lds, stream, a, routed_blocks);
-    }
-    if (!rows_as_lanes) {
     dim3 g2(routed_blocks + shared_blocks + prefetch_blocks);
     if (npl <= 1) launch_gate_up<FG, FS, NT, 1, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else if (npl <= 2) launch_gate_up<FG, FS, NT, 2, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else if (npl <= 4) launch_gate_up<FG, FS, NT, 4, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else launch_gate_up<FG, FS, NT, 8, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024
-    }
     if (last < 3) return;
     // kernel 3
-    if constexpr (FG == PF_Q4_K && FD == PF_Q4_K && FS == PF_Q4_K)
-        if (down_as_lanes) {
-            const size_t widest = I > Is ? I : Is;
-            hipLaunchKernelGGL(pf_k_dec_down_q4t, dim3(H / 8, NT), dim3(64 * (K + 1)), (size_t)(K + 1) * pf_image2_words(widest) * 4, stream, a);
-            return;
-        }
     const int rows_per_block = down_block_rows(H, I), row_blocks = (H + rows_per_block - 1) / rows_per_block;
     const int image_pitch = image_words(I > Is ? I : Is);
     const size_t lds3 = tab3 + (size_t)(K + 1) * image_pitch * 4;
@@ -1515,7 +1531,12 @@ void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t s
 
 #if PF_DECODE_PART == 0
 void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
+    PfHipMoeDesc d = {};
+    d.hidden = a.hidden; d.experts = a.experts; d.top_k = a.top_k; d.inter = a.inter; d.shared_inter = a.shared_inter;
+    d.down_physical = a.down_physical;
+    for (int t = 0; t < 8; t++) d.type[t] = a.type[t];
+    if (pf_decode_tile_layer(d, a.wt)) launch_decode_q4t(a, tokens, stream, stage_limit);
+    else launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {

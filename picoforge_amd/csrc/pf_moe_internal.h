@@ -4,6 +4,7 @@
 #include "../../include/pf_moe_hip.h"
 
 #define PF_DECODE_MAX_TOKENS 4
+#define PF_TILE_DECODE_MAX_TOKENS 16   // Q4_K layers whose tile-ordered copies are kept: one token per grid row
 
 // Everything a kernel needs, passed by value.  Weight index order is
 // Qwen4MoeWeights': router, gate, up, down, shared gate/up/down, shared router.
@@ -150,6 +151,7 @@ void pf_launch_exact_combine(const float *d_down, const uint64_t *d_pair_to_row,
                              uint32_t *d_error, hipStream_t stream);
 // pf_moe_decode.hip
 bool pf_decode_supported(const PfHipMoeDesc &d);
+bool pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const tiled[8]);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);

@@ -139,7 +139,7 @@ def test_views_over_released_weight_bytes(product, oracle):
 
 
 @pytest.mark.parametrize("gtype", [abi.GGUF_Q4_K, abi.GGUF_IQ2_XXS])
-@pytest.mark.parametrize("tokens", [8, 32])
+@pytest.mark.parametrize("tokens", [8, 13, 16, 17, 32])
 def test_batches_between_decode_and_prefill_match_oracle(product, oracle, gtype, tokens):
     """5 to 32 rows at the measured shape (a long verify batch, a short prompt): more rows than the decode kernels
     take, few enough that nearly every routed expert sees one row.  Every row against the CPU path."""

@@ -138,6 +138,7 @@ CHAIN = [
     (512, 32, 6, 256, 256, abi.GGUF_IQ2_XXS, 4, 4),
     (1024, 96, 5, 512, 256, abi.GGUF_Q4_K, 3, 1),
     (256, 16, 4, 256, 256, abi.GGUF_Q4_K, 33, 4),        # prefill kernels
+    (512, 32, 6, 256, 256, abi.GGUF_Q4_K, 11, 4),        # Q4_K decode kernels, one token per grid row
     (512, 8, 3, 256, 512, abi.GGUF_IQ2_XXS, 70, 4),
     (768, 40, 5, 256, 256, abi.GGUF_Q4_K, 129, 2),
     (512, 32, 6, 256, 256, abi.GGUF_Q4_K, 2, 6),         # more streams than the last kernel folds in: separate add
