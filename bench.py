@@ -218,12 +218,12 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
         info = {"active_experts_chunk0": int(unique), "max_tokens_per_expert": int(load.max()),
                 "median_tokens_per_expert": float(np.median(load)), "chunks": n_inputs}
     elif tokens == 1:
-        n_inputs = max(1, min(steps, 2000))
+        n_inputs = max(1, min(steps, 64))       # a plan replays one graph of 64 forwards: 64 inputs = 1.5 GB of weights touched, far beyond the caches
         x, info = workloads.decode_tokens(weights, n_inputs, seed=args.seed)
         x = x.reshape(n_inputs, 1, cfg.hidden_size)
         unique = float(cfg.top_k)
     else:
-        n_inputs = max(1, min(steps, 1000))
+        n_inputs = max(1, min(steps, 64))
         x, info = workloads.verify_batches(weights, n_inputs, seed=args.seed)
         unique = info["mean_unique_experts"]
     prep_s = time.time() - t0
@@ -465,7 +465,7 @@ def run_hc(args, ctx, name, steps, warmup, cpu_seconds):
     weights = pf.LayerWeights.synthetic(cfg, wl["type"], seed=args.seed)
     if tokens > 4:
         workloads.zipf_router(weights, seed=args.seed, temperature=0.18)
-    n_inputs = max(1, min(steps, 4 if tokens > 4 else 1000))
+    n_inputs = max(1, min(steps, 4 if tokens > 4 else 64))
     rng = np.random.default_rng(args.seed)
     # streams whose gated mix has about unit RMS, as the block sees after the norm
     normed = (rng.standard_normal((n_inputs, tokens, streams, h)) * (2.0 * streams ** 0.5 / 1.12)).astype(np.float32)

@@ -11,9 +11,11 @@ extern "C" {
 typedef struct PfBenchPlan PfBenchPlan;
 const char *pf_bench_last_error(void);
 
-/* `forwards` forwards captured once: forward i runs layer i % layers on input block i % n_inputs of
- * d_x ([tokens, hidden] blocks, dense) into output block i % y_blocks of d_y.  kernel_limit > 0
- * captures only the first so many kernel launches of every forward. */
+/* A replay of `forwards` forwards.  They are captured as one graph of u forwards (u = the largest
+ * multiple of `layers` up to 64, at least `layers`) launched forwards / u times and one graph of the
+ * remaining forwards; forward i of a graph runs layer i % layers on input block i % n_inputs of d_x
+ * ([tokens, hidden] blocks, dense) into output block i % y_blocks of d_y.  kernel_limit > 0 captures
+ * only the first so many kernel launches of every forward. */
 int pf_bench_plan_moe(const PfHipMoe *const *moes, PfHipWork *const *works, size_t layers, const float *d_x,
                       size_t n_inputs, float *d_y, size_t y_blocks, size_t tokens, size_t forwards,
                       int kernel_limit, size_t hidden, PfBenchPlan **out);

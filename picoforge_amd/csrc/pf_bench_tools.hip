@@ -2,9 +2,13 @@
 // shipped one.  It drives libpicoforge_moe.so through its public entry points only
 // (include/pf_moe_hip.h) and times with HIP events on the stream the kernels are launched on.
 //
-// A plan is a sequence of forwards captured once into HIP graphs (at most 64 forwards per graph) and
-// replayed as often as wanted: the gap between dependent kernels is then the device's, not the
-// host's enqueue rate, and nothing is instantiated or destroyed between two timed replays.
+// A plan is a sequence of forwards captured once into HIP graphs and replayed as often as wanted: the
+// gap between dependent kernels is then the device's, not the host's enqueue rate, and nothing is
+// instantiated or destroyed between two timed replays.  A plan of many forwards is one graph of about
+// 64 forwards (a whole number of passes over the layers) launched as often as it fits, then one graph
+// for the remainder: every kernel node holds its 808-byte argument block, and rocprofv3's kernel trace
+// crashed in a graph launch once the nodes of a process added up to more than 1 MiB of them (6144
+// nodes did, 960 did not), so a plan keeps to a few hundred nodes whatever its length.
 #include <hip/hip_runtime.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -28,7 +32,8 @@ static int fail(const char *what, hipError_t e) {
 struct PfBenchPlan {
     hipStream_t stream = nullptr;
     hipEvent_t t0 = nullptr, t1 = nullptr;
-    std::vector<hipGraphExec_t> graphs;
+    std::vector<hipGraphExec_t> graphs;   // owned
+    std::vector<hipGraphExec_t> launches; // one replay: the graphs in launch order
     void *owned = nullptr;   // device memory the plan's launches use
 };
 
@@ -44,21 +49,26 @@ extern "C" void pf_bench_plan_destroy(PfBenchPlan *p) {
 
 static const size_t FORWARDS_PER_GRAPH = 64;
 
+// enqueue(i, stream): forward i of a graph (i counts from 0 in each graph).  period: forwards after which the
+// sequence of layers repeats; a graph holds a whole number of periods.
 template <typename Enqueue>
-static int build_plan(size_t forwards, PfBenchPlan **out, Enqueue enqueue) {
+static int build_plan(size_t forwards, size_t period, PfBenchPlan **out, Enqueue enqueue) {
     *out = nullptr;
     PfBenchPlan *p = new PfBenchPlan();
     hipError_t e = hipStreamCreate(&p->stream);
     if (e == hipSuccess) e = hipEventCreate(&p->t0);
     if (e == hipSuccess) e = hipEventCreate(&p->t1);
     if (e != hipSuccess) { pf_bench_plan_destroy(p); return fail("plan set-up", e); }
+    const size_t unit = period * (FORWARDS_PER_GRAPH / period ? FORWARDS_PER_GRAPH / period : 1);
+    const size_t sizes[2] = {forwards >= unit ? unit : 0, forwards % unit}, copies[2] = {forwards / unit, 1};
     int rc = PF_HIP_OK;
-    for (size_t first = 0; first < forwards && rc == PF_HIP_OK; first += FORWARDS_PER_GRAPH) {
+    for (int which = 0; which < 2 && rc == PF_HIP_OK; which++) {
+        if (!sizes[which]) continue;
         hipGraph_t graph = nullptr;
         hipGraphExec_t exec = nullptr;
         e = hipStreamBeginCapture(p->stream, hipStreamCaptureModeThreadLocal);
         if (e != hipSuccess) { rc = fail("hipStreamBeginCapture", e); break; }
-        for (size_t i = first; i < forwards && i < first + FORWARDS_PER_GRAPH && rc == PF_HIP_OK; i++) {
+        for (size_t i = 0; i < sizes[which] && rc == PF_HIP_OK; i++) {
             rc = enqueue(i, p->stream);
             if (rc != PF_HIP_OK) snprintf(g_error, sizeof g_error, "forward %zu: shim status %d: %s", i, rc, pf_hip_last_error());
         }
@@ -67,7 +77,10 @@ static int build_plan(size_t forwards, PfBenchPlan **out, Enqueue enqueue) {
         if (rc == PF_HIP_OK) {
             e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
             if (e != hipSuccess) rc = fail("hipGraphInstantiate", e);
-            else p->graphs.push_back(exec);
+            else {
+                p->graphs.push_back(exec);
+                for (size_t c = 0; c < copies[which]; c++) p->launches.push_back(exec);
+            }
         }
         if (graph) {
             e = hipGraphDestroy(graph);
@@ -90,7 +103,7 @@ extern "C" int pf_bench_plan_moe(const PfHipMoe *const *moes, PfHipWork *const *
         pf_hip_work_limit_kernels(works[l], kernel_limit);
     }
     const size_t block = tokens * hidden;
-    const int rc = build_plan(forwards, out, [&](size_t i, hipStream_t s) {
+    const int rc = build_plan(forwards, layers, out, [&](size_t i, hipStream_t s) {
         return pf_hip_moe_forward_device(moes[i % layers], works[i % layers], d_x + (i % n_inputs) * block, hidden,
                                          d_y + (i % y_blocks) * block, hidden, tokens, s);
     });
@@ -109,7 +122,7 @@ extern "C" int pf_bench_plan_hc(const PfHipMoe *moe, PfHipWork *work, const floa
     // the unfused chain needs rows for the mixed input and the block's output between its three enqueues
     float *rows = nullptr;
     if (!fused) HIP_TRY(hipMalloc((void **)&rows, 2 * tokens * H * sizeof(float)));
-    const int rc = build_plan(forwards, out, [&](size_t i, hipStream_t s) {
+    const int rc = build_plan(forwards, 1, out, [&](size_t i, hipStream_t s) {
         const float *n = d_normed + (i % n_inputs) * cube, *g = d_logits + (i % n_inputs) * cube;
         if (fused)
             return pf_hip_moe_forward_hc_device(moe, work, n, streams * H, H, g, streams * H, H, d_residual, streams * H, H,
@@ -130,7 +143,7 @@ extern "C" int pf_bench_plan_run(PfBenchPlan *p, size_t repeats, float *ms_each)
     if (!p || !repeats || !ms_each) return PF_HIP_E_ARGUMENT;
     for (size_t r = 0; r < repeats; r++) {
         HIP_TRY(hipEventRecord(p->t0, p->stream));
-        for (hipGraphExec_t g : p->graphs) HIP_TRY(hipGraphLaunch(g, p->stream));
+        for (hipGraphExec_t g : p->launches) HIP_TRY(hipGraphLaunch(g, p->stream));
         HIP_TRY(hipEventRecord(p->t1, p->stream));
         HIP_TRY(hipStreamSynchronize(p->stream));
         HIP_TRY(hipEventElapsedTime(&ms_each[r], p->t0, p->t1));
