@@ -113,6 +113,21 @@ struct PfHipMoe *pf_moe_device_layer(const Qwen4Moe *moe);
  * that releases them earlier calls this first; forward then skips that comparison for the layer
  * (pf_gguf_moe_create does so itself: its layers may outlive the file mapping). */
 void pf_moe_forget_host_weights(Qwen4Moe *moe);
+
+/* Extension for models larger than device memory, the counterpart of the reference's expert streaming
+ * (src/qwen4_expert_pool.h; the remap hook of src/qwen4_moe_internal.h:49-54; its caller in
+ * src/qwen4_forward_gpu.m).  pf_moe_create_streamed takes the same arguments as qwen4_moe_create with
+ * the gate, up and down views carrying their layouts and a NULL span: those tensors stay in the model
+ * file (formats stored as the file stores them: Q4_K, Q2_K, F32, F16, BF16).  pf_moe_forward_streamed is
+ * qwen4_moe_forward for such a layer: after the routing it acquires the batch's experts from `pool` as
+ * layer `layer` (tokens * top_k pins: the pool needs that many slots), runs the expert products on the
+ * pool's slots and releases them.  QW4_IO when the pool cannot take the batch or a read fails;
+ * qwen4_moe_forward on a streamed layer, or a pool with a resident one: QW4_BAD_STATE. */
+struct QW4ExpertPool;
+Qwen4Status pf_moe_create_streamed(const Qwen4MoeConfig *config, const Qwen4MoeWeights *weights, Qwen4Moe **out,
+                                   Qwen4Error *err);
+Qwen4Status pf_moe_forward_streamed(const Qwen4Moe *moe, struct QW4ExpertPool *pool, uint32_t layer, Qwen4F32 x,
+                                    Qwen4F32Mut y, Qwen4MoeRoutes *optional_routes, Qwen4MoeWork *work, Qwen4Error *err);
 struct PfHipWork *pf_moe_device_work(Qwen4MoeWork *work);
 
 #ifdef __cplusplus

@@ -89,6 +89,15 @@ class QW4MoeGrouping(C.Structure):
                 ("row_to_pair_capacity_bytes", C.c_size_t)]
 
 
+class QW4ExpertLayer(C.Structure):   # include/qwen4_expert_pool.h
+    _fields_ = [("offset", C.c_uint64 * 3)]
+
+
+class QW4PoolStats(C.Structure):
+    _fields_ = [("hits", C.c_uint64), ("misses", C.c_uint64), ("evictions", C.c_uint64), ("bytes_read", C.c_uint64),
+                ("acquire_ns", C.c_uint64)]
+
+
 OBSERVER = C.CFUNCTYPE(None, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, Qwen4F32, Qwen4F32)
 
 

@@ -66,6 +66,19 @@ class MoeApi:
         if hasattr(lib, "pf_moe_device_layer"):
             self.device_layer = bind("pf_moe_device_layer", vp, vp)
             self.device_work = bind("pf_moe_device_work", vp, vp)
+        if hasattr(lib, "pf_moe_create_streamed"):   # expert streaming (include/qwen4_expert_pool.h, include/qwen4_moe.h)
+            u32 = C.c_uint32
+            self.create_streamed = bind("pf_moe_create_streamed", C.c_int, P(abi.Qwen4MoeConfig), P(abi.Qwen4MoeWeights),
+                                        P(vp), P(E))
+            self.forward_streamed = bind("pf_moe_forward_streamed", C.c_int, vp, vp, u32, abi.Qwen4F32, abi.Qwen4F32Mut,
+                                         P(abi.Qwen4MoeRoutes), vp, P(E))
+            self.pool_create = bind("qw4_pool_create", vp, C.c_int, P(abi.QW4ExpertLayer), u32, u32, P(sz), u32)
+            self.pool_destroy = bind("qw4_pool_destroy", None, vp)
+            self.pool_acquire = bind("qw4_pool_acquire", C.c_int, vp, u32, P(u32), sz, P(u32))
+            self.pool_release = bind("qw4_pool_release", None, vp, P(u32), sz)
+            self.pool_set_readers = bind("qw4_pool_set_readers", None, vp, u32)
+            self.pool_region = bind("qw4_pool_region", vp, vp, C.c_int, P(sz))
+            self.pool_stats = bind("qw4_pool_stats", abi.QW4PoolStats, vp)
         self.layout_init = bind(packed_prefix + "layout_init", C.c_int, P(abi.GgufTensor), sz,
                                 P(abi.QW4PackedLayout), P(E))
         self.decode_row = bind(packed_prefix + "decode_row", C.c_int, P(abi.QW4PackedCpuView), sz, sz, vp, sz, P(E))

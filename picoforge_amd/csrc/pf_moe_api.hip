@@ -170,7 +170,14 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             return PF_HIP_E_UNSUPPORTED;
         }
         gguf_bytes[a] = place.gguf_bytes;
-        if (bytes[a] < gguf_bytes[a] || !host_weights[a]) { pf_hip_moe_destroy(m); return PF_HIP_E_ARGUMENT; }
+        // a layer whose routed tensors stay on disk (forwards then read them from an expert pool): all three absent
+        const bool routed = a >= 1 && a <= 3;
+        if (routed && !host_weights[1] && !host_weights[2] && !host_weights[3]) m->streamed = true;
+        else if (bytes[a] < gguf_bytes[a] || !host_weights[a]) { pf_hip_moe_destroy(m); return PF_HIP_E_ARGUMENT; }
+        if (m->streamed && routed && split_header_bytes(desc->type[a])) {
+            pf_hip_moe_destroy(m);   // pool slots hold experts as the file stores them: formats stored split on the device are not streamed
+            return PF_HIP_E_UNSUPPORTED;
+        }
         m->k_logical[a] = (int)k_logical[a];
         m->n_out[a] = place.n_out;
         m->blocks_per_row[a] = place.blocks_per_row;
@@ -188,6 +195,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
     m->iq2_grid = g_grid;
     m->iq2_signed = g_signed;
     for (int a = 0; a < 8; a++) {
+        if (m->streamed && a >= 1 && a <= 3) continue;
         hipError_t e = hipMalloc((void **)&m->w[a], m->bytes[a]);
         const size_t head = split_header_bytes(desc->type[a]);
         if (e == hipSuccess && head) {
@@ -230,9 +238,9 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         }
         m->total_bytes += slab_floats * sizeof(float);
     }
-    m->decode_ready = pf_decode_supported(*desc);
+    m->decode_ready = !m->streamed && pf_decode_supported(*desc);
     // prefill path: squared norms of the router rows (the routing tolerance's bound)
-    m->prefill_ready = pf_prefill_supported(*desc);
+    m->prefill_ready = !m->streamed && pf_prefill_supported(*desc);
     if (m->prefill_ready) {
         hipError_t e = hipMalloc((void **)&m->w_norm2, E * sizeof(float));
         if (e == hipSuccess) {
@@ -281,7 +289,7 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
 extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_bytes : 0; }
 
 // workspace layout: buffers carved from one allocation, each 256-byte aligned
-enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_IDS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS, W_XIMG, W_AIMG,
+enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_IDS, W_SLOTS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS, W_XIMG, W_AIMG,
        W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
        W_P2R, W_R2P, W_GROUPBAD, W_TILES, W_COUNT };
 struct Carve { size_t offset[W_COUNT], total; };
@@ -304,6 +312,7 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_X] = T * H * 4;
     want[W_Y] = T * H * 4;
     want[W_IDS] = T * K * 4;
+    want[W_SLOTS] = T * K * 4;   // expert streaming: the pairs' pool slots
     want[W_UNIQ] = (1 + 3 * Td * K) * 4;
     want[W_ERR] = 256;
     want[W_EXACT] = 256;
@@ -377,6 +386,7 @@ static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base) {
     w->y = (float *)(base + c.offset[W_Y]);
     w->ids = (uint32_t *)(base + c.offset[W_IDS]);
     w->uniq = (uint32_t *)(base + c.offset[W_UNIQ]);
+    w->slots = (uint32_t *)(base + c.offset[W_SLOTS]);
     w->error_word = (uint32_t *)(base + c.offset[W_ERR]);
     w->exact_rows = (uint32_t *)(base + c.offset[W_EXACT]);
     w->route_flags = (uint32_t *)(base + c.offset[W_FLAGS]);
@@ -483,6 +493,10 @@ static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_
     if (hc) {
         a.hc_residual = hc->residual; a.hc_inject = hc->inject; a.hc_streams = hc->streams;
         a.hc_token_pitch = hc->token_pitch; a.hc_stream_pitch = hc->stream_pitch;
+    }
+    if (moe->streamed) {
+        snprintf(g_error, sizeof g_error, "the layer's routed experts are not resident: forward it through an expert pool");
+        return PF_HIP_E_UNSUPPORTED;
     }
     const bool aligned = (x_pitch % 4 == 0) && ((uintptr_t)d_x % 16 == 0);
     if (moe->decode_ready && tokens <= decode_limit(moe) && aligned && !work->force_general) {
@@ -635,6 +649,69 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
     HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
     if (*error_word) {
         HIP_TRY(hipMemset(work->error_word, 0, 4));   // the word is sticky on the device; reading it clears it
+        return PF_HIP_OK;
+    }
+    HIP_TRY(hipMemcpy2D(y, y_pitch_bytes, work->y, H * 4, H * 4, tokens, hipMemcpyDeviceToHost));
+    if (ids) HIP_TRY(hipMemcpy2D(ids, ids_pitch_bytes, work->ids, K * 4, K * 4, tokens, hipMemcpyDeviceToHost));
+    if (weights)
+        HIP_TRY(hipMemcpy2D(weights, weights_pitch_bytes, work->route_weights, K * 4, K * 4, tokens,
+                            hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+// ---- a layer whose routed experts are streamed (src/qwen4_moe_internal.h:49-54, the remap hook) -----------------
+// Two calls with the caller's pool in between.  The first runs the router and the routing and returns the pairs'
+// expert ids; the caller makes those experts resident (qw4_pool_acquire) and passes the pool's device regions and
+// the pairs' slots to the second, which runs the expert products and the combine reading rows at
+// region + slot * expert_bytes.  The general kernels serve both: streaming is bound by the reads that fill the pool.
+extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
+                                              size_t tokens, uint32_t *ids, uint32_t *error_word) {
+    if (!moe || !work || work->moe != moe || !error_word) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!x || !ids || tokens > work->cap) return PF_HIP_E_ARGUMENT;
+    const size_t H = moe->desc.hidden, K = moe->desc.top_k;
+    if (tokens * K > 0x7fffffffu / 4) return PF_HIP_E_UNSUPPORTED;
+    HIP_TRY(hipMemcpy2D(work->x, H * 4, x, x_pitch_bytes, H * 4, tokens, hipMemcpyHostToDevice));
+    PfKernelArgs a = make_args(moe, work, work->x, H, work->y, H);
+    const size_t lds_route = (H + 3 * (size_t)moe->desc.experts) * 4;
+    if (pf_general_lds_bytes(a) > 64 * 1024 || lds_route > 64 * 1024) {
+        snprintf(g_error, sizeof g_error, "dimensions exceed the LDS staging of the general kernels");
+        return PF_HIP_E_UNSUPPORTED;
+    }
+    pf_launch_general(a, (int)tokens, nullptr, 2);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
+    if (*error_word) {
+        HIP_TRY(hipMemset(work->error_word, 0, 4));
+        return PF_HIP_OK;
+    }
+    HIP_TRY(hipMemcpy(ids, work->ids, tokens * K * 4, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const void *const regions[3],
+                                                const size_t expert_bytes[3], uint32_t pool_slots, const uint32_t *slots,
+                                                float *y, size_t y_pitch_bytes, uint32_t *ids, size_t ids_pitch_bytes,
+                                                float *weights, size_t weights_pitch_bytes, size_t tokens,
+                                                uint32_t *error_word) {
+    if (!moe || !work || work->moe != moe || !error_word || !regions || !expert_bytes) return PF_HIP_E_ARGUMENT;
+    *error_word = 0;
+    if (tokens == 0) return PF_HIP_OK;
+    if (!y || !slots || !pool_slots || tokens > work->cap) return PF_HIP_E_ARGUMENT;
+    const size_t H = moe->desc.hidden, K = moe->desc.top_k;
+    for (int j = 0; j < 3; j++)   // a slot holds one expert of each tensor as the file stores it
+        if (!regions[j] || expert_bytes[j] != moe->expert_bytes[1 + j]) return PF_HIP_E_ARGUMENT;
+    HIP_TRY(hipMemcpy(work->slots, slots, tokens * K * 4, hipMemcpyHostToDevice));
+    PfKernelArgs a = make_args(moe, work, work->x, H, work->y, H);
+    for (int j = 0; j < 3; j++) a.w[1 + j] = static_cast<const uint8_t *>(regions[j]);
+    a.slots = work->slots;
+    a.pool_slots = pool_slots;
+    pf_launch_general(a, (int)tokens, nullptr, 0, 3);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
+    if (*error_word) {
+        HIP_TRY(hipMemset(work->error_word, 0, 4));
         return PF_HIP_OK;
     }
     HIP_TRY(hipMemcpy2D(y, y_pitch_bytes, work->y, H * 4, H * 4, tokens, hipMemcpyDeviceToHost));

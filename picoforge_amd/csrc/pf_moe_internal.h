@@ -32,6 +32,10 @@ struct PfKernelArgs {
     uint32_t *ximg, *aimg;           // decode path, tile-ordered Q4_K: digit images (pf_image2_words) of the token rows, written
                                      // by kernel 1, and of the activation rows [unique, tokens] then [tokens] shared, by kernel 2
     uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
+    // expert streaming (general kernels only): w[1..3] are pool regions of pool_slots experts each and the routed
+    // tensors are addressed by slots[pair] instead of ids[pair] (null: every expert resident, addressed by id)
+    const uint32_t *slots;
+    uint32_t pool_slots;
     uint32_t *error_word;
     uint32_t *exact_rows;            // count of tokens re-routed in serial order
     uint32_t *route_flags;           // tokens to route again in serial order: [0] their number, then the tokens; the kernel
@@ -104,6 +108,7 @@ struct PfHipMoe {
     float *w_norm2;                  // [experts] squared norm of each router row
     float *router_t;                 // [slab of 64 experts][hidden / 4][64][4] copy of the router
     uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
+    bool streamed;                   // the routed tensors are not resident: forwards read them from an expert pool
 };
 
 // Two-digit image of a K-vector for wave-uniform (scalar) reads: per 32-group 16 dwords (the values' low base-256
@@ -115,7 +120,7 @@ struct PfHipWork {
     size_t cap, bytes;
     uint32_t *ximg, *aimg;
     float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
-    uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags;
+    uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags, *slots;
     uint16_t *x16, *act16, *sact16;  // prefill buffers (allocated when cap exceeds the decode path's batch)
     float *x_scale, *act_scale, *sact_scale, *x_max2, *down;
     uint32_t *counts, *offsets, *pair_to_row, *row_to_pair, *group_bad, *tiles;
@@ -124,7 +129,7 @@ struct PfHipWork {
 };
 
 // pf_moe_kernels.hip
-void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit, int first_stage = 1);
 size_t pf_general_lds_bytes(const PfKernelArgs &a);
 // pf_moe_route.hip
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream);

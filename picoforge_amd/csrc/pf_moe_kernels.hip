@@ -270,13 +270,13 @@ __global__ void __launch_bounds__(256) pf_k_gate_up(PfKernelArgs a) {
     __syncthreads();
     const int n = blockIdx.x * 4 + wave;
     if (n >= a.inter) return;
-    const uint32_t e = a.ids[pair];
-    if (e >= (uint32_t)a.experts) {
+    const uint32_t e = a.ids[pair], at = a.slots ? a.slots[pair] : e;   // where the expert's rows are
+    if (e >= (uint32_t)a.experts || (a.slots && at >= a.pool_slots)) {
         if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
         return;
     }
-    float g = dot_tensor_row(a, 1, e, n, lds, lane, grid);
-    float u = dot_tensor_row(a, 2, e, n, lds, lane, grid);
+    float g = dot_tensor_row(a, 1, at, n, lds, lane, grid);
+    float u = dot_tensor_row(a, 2, at, n, lds, lane, grid);
     float v = pf_silu(g) * u;
     if (lane == 0) {
         a.act[(size_t)pair * a.inter + n] = v;
@@ -301,12 +301,12 @@ __global__ void __launch_bounds__(256) pf_k_down_combine(PfKernelArgs a) {
     if (n >= a.hidden) return;
     float sum = 0.0f;
     for (int s = 0; s < K; s++) {
-        const uint32_t e = a.ids[(size_t)t * K + s];
-        if (e >= (uint32_t)a.experts) {
+        const uint32_t e = a.ids[(size_t)t * K + s], at = a.slots ? a.slots[(size_t)t * K + s] : e;
+        if (e >= (uint32_t)a.experts || (a.slots && at >= a.pool_slots)) {
             if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
             return;
         }
-        float dsum = dot_tensor_row(a, 3, e, n, lds + s * Ip, lane, grid);
+        float dsum = dot_tensor_row(a, 3, at, n, lds + s * Ip, lane, grid);
         sum += a.route_weights[(size_t)t * K + s] * dsum;   // slot order, as src/qwen4_moe.c:362-372
     }
     float sh = dot_tensor_row(a, 6, 0, n, sact, lane, grid);
@@ -324,15 +324,15 @@ size_t pf_general_lds_bytes(const PfKernelArgs &a) {
     return down > x ? down : x;
 }
 
-void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    // stage_limit (profiling): launch only the first so many of the four stages; 0 = all
+void pf_launch_general(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit, int first_stage) {
+    // stage_limit (profiling, expert streaming): launch only the first so many of the four stages; 0 = all.
+    // first_stage: the stage to start at (expert streaming resumes at 3 once the routed experts are resident).
     const int units = a.experts + a.shared_inter + 1, last = stage_limit ? stage_limit : 4;
     const size_t x_lds = (size_t)a.hidden * sizeof(float);
-    hipLaunchKernelGGL(pf_k_pre, dim3((units + 3) / 4, tokens), dim3(256), x_lds, stream, a);
-    if (last < 2) return;
-    pf_launch_route(a, tokens, stream);
-    if (last < 3) return;
-    hipLaunchKernelGGL(pf_k_gate_up, dim3((a.inter + 3) / 4, tokens * a.top_k), dim3(256), x_lds, stream, a);
+    if (first_stage <= 1 && last >= 1) hipLaunchKernelGGL(pf_k_pre, dim3((units + 3) / 4, tokens), dim3(256), x_lds, stream, a);
+    if (first_stage <= 2 && last >= 2) pf_launch_route(a, tokens, stream);
+    if (first_stage <= 3 && last >= 3)
+        hipLaunchKernelGGL(pf_k_gate_up, dim3((a.inter + 3) / 4, tokens * a.top_k), dim3(256), x_lds, stream, a);
     if (last < 4) return;
     const size_t act_lds = ((size_t)a.top_k * a.down_physical + a.shared_inter) * sizeof(float);
     hipLaunchKernelGGL(pf_k_down_combine, dim3((a.hidden + 3) / 4, tokens), dim3(256), act_lds, stream, a);

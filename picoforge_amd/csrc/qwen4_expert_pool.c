@@ -1,0 +1,197 @@
+/* Expert pool in device memory (include/qwen4_expert_pool.h): the bookkeeping of
+ * src/qwen4_expert_pool.c of the reference restated for HBM-resident slots.
+ *
+ * Recency is a counter stamped on a slot whenever it is acquired; the victim of a miss is the slot
+ * with the oldest stamp among those nobody pins (fresh pools stamp slot s with s, so slot 0 goes first,
+ * as in the reference).  A scan over the slots per miss is enough: pools hold a few thousand slots and
+ * a miss costs a file read of megabytes.  Reads go through one staging buffer per reader thread:
+ * pread into it, then one copy to the slot's place in the matrix region. */
+#define _GNU_SOURCE
+#include "../../include/qwen4_expert_pool.h"
+#include "../../include/pf_moe_hip.h"
+#include <pthread.h>
+#include <stdatomic.h>
+#include <stdlib.h>
+#include <time.h>
+#include <unistd.h>
+
+#define NO_SLOT UINT32_MAX
+
+struct QW4ExpertPool {
+    int fd;
+    uint32_t n_layers, experts, slots, readers;
+    size_t bytes[3], region_bytes[3];
+    QW4ExpertLayer *layers;
+    void *region[3];        /* device memory: slots * bytes[m] each */
+    uint32_t *where;        /* [layer * experts + expert] -> slot or NO_SLOT */
+    uint32_t *holds;        /* [slot] -> layer * experts + expert or NO_SLOT */
+    uint32_t *pins;         /* [slot] */
+    uint64_t *stamp, clock; /* [slot] recency */
+    uint32_t *new_slot, *new_expert;   /* the misses of the acquire in progress */
+    QW4PoolStats stats;
+};
+
+QW4ExpertPool *qw4_pool_create(int fd, const QW4ExpertLayer *layers, uint32_t n_layers, uint32_t experts,
+                               const size_t bytes[3], uint32_t slots) {
+    if (fd < 0 || !layers || !bytes || !n_layers || !experts || !slots || slots == NO_SLOT) return NULL;
+    if (!bytes[0] || !bytes[1] || !bytes[2] || (uint64_t)n_layers * experts >= NO_SLOT) return NULL;
+    QW4ExpertPool *p = calloc(1, sizeof *p);
+    if (!p) return NULL;
+    p->fd = fd; p->n_layers = n_layers; p->experts = experts; p->slots = slots; p->readers = 8;
+    const size_t keys = (size_t)n_layers * experts;
+    p->layers = malloc(n_layers * sizeof *p->layers);
+    p->where = malloc(keys * sizeof *p->where);
+    p->holds = malloc(slots * sizeof *p->holds);
+    p->pins = calloc(slots, sizeof *p->pins);
+    p->stamp = malloc(slots * sizeof *p->stamp);
+    p->new_slot = malloc(slots * sizeof *p->new_slot);
+    p->new_expert = malloc(slots * sizeof *p->new_expert);
+    if (!p->layers || !p->where || !p->holds || !p->pins || !p->stamp || !p->new_slot || !p->new_expert) {
+        qw4_pool_destroy(p);
+        return NULL;
+    }
+    for (uint32_t l = 0; l < n_layers; l++) p->layers[l] = layers[l];
+    for (size_t k = 0; k < keys; k++) p->where[k] = NO_SLOT;
+    for (uint32_t s = 0; s < slots; s++) { p->holds[s] = NO_SLOT; p->stamp[s] = s; }
+    p->clock = slots;
+    for (int m = 0; m < 3; m++) {
+        p->bytes[m] = bytes[m];
+        p->region_bytes[m] = (size_t)slots * bytes[m];
+        if (pf_hip_malloc(&p->region[m], p->region_bytes[m]) != PF_HIP_OK) {
+            p->region[m] = NULL;
+            qw4_pool_destroy(p);
+            return NULL;
+        }
+    }
+    return p;
+}
+
+void qw4_pool_destroy(QW4ExpertPool *p) {
+    if (!p) return;
+    for (int m = 0; m < 3; m++)
+        if (p->region[m]) pf_hip_free(p->region[m]);
+    free(p->layers); free(p->where); free(p->holds); free(p->pins); free(p->stamp); free(p->new_slot); free(p->new_expert);
+    free(p);
+}
+
+void qw4_pool_set_readers(QW4ExpertPool *p, uint32_t readers) {
+    if (p) p->readers = readers ? readers : 1;
+}
+
+void qw4_pool_release(QW4ExpertPool *p, const uint32_t *slots, size_t n) {
+    if (!p || !slots) return;
+    for (size_t i = 0; i < n; i++)
+        if (slots[i] < p->slots && p->pins[slots[i]]) p->pins[slots[i]]--;
+}
+
+void *qw4_pool_region(const QW4ExpertPool *p, int matrix, size_t *bytes) {
+    if (!p || matrix < 0 || matrix > 2) return NULL;
+    if (bytes) *bytes = p->region_bytes[matrix];
+    return p->region[matrix];
+}
+
+QW4PoolStats qw4_pool_stats(const QW4ExpertPool *p) {
+    QW4PoolStats none = {0, 0, 0, 0, 0};
+    return p ? p->stats : none;
+}
+
+/* ---- the reads of one acquire ------------------------------------------------------------------
+ * A job is one matrix of one missed expert; the readers take jobs from a shared counter until none
+ * is left.  (The reference hands reader g the jobs g, g + width, ...; which reader reads what does
+ * not show in the result.) */
+typedef struct {
+    QW4ExpertPool *p;
+    uint32_t layer, misses;
+    atomic_size_t next;
+    atomic_int failed;
+} Reads;
+
+static int read_exactly(int fd, unsigned char *dst, size_t bytes, uint64_t offset) {
+    size_t done = 0;
+    while (done < bytes) {
+        const ssize_t got = pread(fd, dst + done, bytes - done, (off_t)(offset + done));
+        if (got <= 0) return -1;
+        done += (size_t)got;
+    }
+    return 0;
+}
+
+static void *reader(void *arg) {
+    Reads *r = arg;
+    QW4ExpertPool *p = r->p;
+    size_t widest = p->bytes[0];
+    for (int m = 1; m < 3; m++) widest = p->bytes[m] > widest ? p->bytes[m] : widest;
+    unsigned char *staging = malloc(widest);
+    if (!staging) { atomic_store(&r->failed, 1); return NULL; }
+    for (;;) {
+        const size_t job = atomic_fetch_add(&r->next, 1);
+        if (job >= (size_t)r->misses * 3 || atomic_load(&r->failed)) break;
+        const size_t miss = job / 3;
+        const int m = (int)(job % 3);
+        const uint64_t from = p->layers[r->layer].offset[m] + (uint64_t)p->new_expert[miss] * p->bytes[m];
+        unsigned char *to = (unsigned char *)p->region[m] + (size_t)p->new_slot[miss] * p->bytes[m];
+        if (read_exactly(p->fd, staging, p->bytes[m], from) || pf_hip_memcpy_h2d(to, staging, p->bytes[m]) != PF_HIP_OK)
+            atomic_store(&r->failed, 1);
+    }
+    free(staging);
+    return NULL;
+}
+
+static uint64_t now_ns(void) {
+    struct timespec t;
+    clock_gettime(CLOCK_MONOTONIC, &t);
+    return (uint64_t)t.tv_sec * 1000000000ull + (uint64_t)t.tv_nsec;
+}
+
+int qw4_pool_acquire(QW4ExpertPool *p, uint32_t layer, const uint32_t *experts, size_t n, uint32_t *slots) {
+    if (!p || layer >= p->n_layers || (n && (!experts || !slots))) return -1;
+    const uint64_t t0 = now_ns();
+    uint32_t misses = 0;
+    int rc = 0;
+    /* pass 1: slots and victims, in list order */
+    for (size_t i = 0; i < n && !rc; i++) {
+        if (experts[i] >= p->experts) { qw4_pool_release(p, slots, i); rc = -1; break; }
+        const uint32_t key = layer * p->experts + experts[i];
+        uint32_t s = p->where[key];
+        if (s != NO_SLOT) {
+            p->stats.hits++;
+        } else {
+            for (uint32_t c = 0; c < p->slots; c++)   /* oldest stamp among the unpinned */
+                if (!p->pins[c] && (s == NO_SLOT || p->stamp[c] < p->stamp[s])) s = c;
+            if (s == NO_SLOT) { qw4_pool_release(p, slots, i); rc = -1; break; }
+            if (p->holds[s] != NO_SLOT) { p->where[p->holds[s]] = NO_SLOT; p->stats.evictions++; }
+            p->holds[s] = key;
+            p->where[key] = s;
+            p->stats.misses++;
+            p->stats.bytes_read += p->bytes[0] + p->bytes[1] + p->bytes[2];
+            p->new_slot[misses] = s;
+            p->new_expert[misses] = experts[i];
+            misses++;
+        }
+        p->pins[s]++;
+        p->stamp[s] = p->clock++;
+        slots[i] = s;
+    }
+    /* pass 2: the misses, read together */
+    if (!rc && misses) {
+        Reads reads = {.p = p, .layer = layer, .misses = misses};
+        atomic_init(&reads.next, 0);
+        atomic_init(&reads.failed, 0);
+        uint32_t width = p->readers < misses * 3 ? p->readers : misses * 3;
+        if (width > 64) width = 64;
+        pthread_t thread[64];
+        uint32_t started = 0;
+        for (; started + 1 < width; started++)
+            if (pthread_create(&thread[started], NULL, reader, &reads)) break;
+        reader(&reads);   /* this thread reads too; alone when no other could be started */
+        for (uint32_t j = 0; j < started; j++) pthread_join(thread[j], NULL);
+        if (atomic_load(&reads.failed)) { qw4_pool_release(p, slots, n); rc = -1; }
+    }
+    if (rc)   /* the slots this call took hold nothing usable: forget them (their recency stays) */
+        for (uint32_t j = 0; j < misses; j++) {
+            p->where[p->holds[p->new_slot[j]]] = NO_SLOT;
+            p->holds[p->new_slot[j]] = NO_SLOT;
+        }
+    p->stats.acquire_ns += now_ns() - t0;
+    return rc;
+}

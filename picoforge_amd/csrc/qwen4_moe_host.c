@@ -5,6 +5,7 @@
  * CPU fallback: without a device every compute entry point fails. */
 #include "../../include/qwen4_moe.h"
 #include "../../include/qwen4_hc.h"
+#include "../../include/qwen4_expert_pool.h"
 #include "../../include/pf_moe_hip.h"
 #include "pf_hc_host.h"
 #include <math.h>
@@ -13,6 +14,7 @@
 #include <string.h>
 
 Qwen4Status pf_packed_admit(const QW4PackedCpuView *w, size_t expert);              /* qwen4_packed_host.c */
+Qwen4Status pf_layout_admit(const QW4PackedLayout *l);
 Qwen4Status pf_device_status(int rc, Qwen4Error *err, const char *subject);
 
 typedef struct { uintptr_t lo, hi; } Range;
@@ -25,6 +27,7 @@ struct Qwen4Moe {
     PfHipMoe *device;
     PfHipMoeDesc desc;
     bool host_spans;   /* the caller still holds the weight bytes at w[].span (the reference's contract) */
+    bool streamed;     /* the routed tensors are read from an expert pool, forward by forward */
     FILE *route_log;   /* PF_ROUTE_LOG: this layer's routed ids, one record per forward */
     uint64_t route_pos;
 };
@@ -87,8 +90,8 @@ static void route_log_append(Qwen4Moe *m, const uint32_t *ids, size_t pitch_word
 }
 
 /* ---- create / destroy ------------------------------------------------------ */
-Qwen4Status qwen4_moe_create(const Qwen4MoeConfig *c, const Qwen4MoeWeights *weights, Qwen4Moe **out,
-                             Qwen4Error *err) {
+static Qwen4Status create_layer(const Qwen4MoeConfig *c, const Qwen4MoeWeights *weights, bool streamed, Qwen4Moe **out,
+                                Qwen4Error *err) {
     if (out) *out = NULL;
     if (!out || !weights) return moe_status(err, QW4_INVALID_ARGUMENT, "null create argument");
     TRY(admit_config(c, err));
@@ -104,7 +107,9 @@ Qwen4Status qwen4_moe_create(const Qwen4MoeConfig *c, const Qwen4MoeWeights *wei
             l->k_storage != (a == 3 ? c->down_physical : k_in[a]))
             return moe_status(err, QW4_SHAPE, "MoE weight shape mismatch");
         if ((a == 0 || a == 7) && l->gguf_type != 0) return moe_status(err, QW4_FORMAT, "router must be F32");
-        Qwen4Status st = pf_packed_admit(&w[a], 0);
+        const bool on_disk = streamed && a >= 1 && a <= 3;
+        if (on_disk && w[a].span.data) return moe_status(err, QW4_INVALID_ARGUMENT, "a streamed layer takes no routed bytes");
+        Qwen4Status st = on_disk ? pf_layout_admit(l) : pf_packed_admit(&w[a], 0);
         if (st) {
             moe_status(err, st, "invalid weight view");
             if (err) snprintf(err->subject, sizeof err->subject, "packed weights");
@@ -130,10 +135,23 @@ Qwen4Status qwen4_moe_create(const Qwen4MoeConfig *c, const Qwen4MoeWeights *wei
     m->refs = 1;
     m->alive = true;
     m->host_spans = true;
+    m->streamed = streamed;
     Qwen4Status st = route_log_open(m, err);
     if (st) { pf_hip_moe_destroy(m->device); free(m); return st; }
     *out = m;
     return moe_status(err, QW4_OK, "");
+}
+
+Qwen4Status qwen4_moe_create(const Qwen4MoeConfig *c, const Qwen4MoeWeights *weights, Qwen4Moe **out,
+                             Qwen4Error *err) {
+    return create_layer(c, weights, false, out, err);
+}
+
+/* A layer for models larger than device memory: router, shared expert and shared router resident, the
+ * routed gate, up and down tensors left in the model file (their views carry layouts and no bytes). */
+Qwen4Status pf_moe_create_streamed(const Qwen4MoeConfig *c, const Qwen4MoeWeights *weights, Qwen4Moe **out,
+                                   Qwen4Error *err) {
+    return create_layer(c, weights, true, out, err);
 }
 
 static void moe_unref(Qwen4Moe *m) {
@@ -480,12 +498,56 @@ static Qwen4Status observed_forward(Qwen4MoeWork *w, Qwen4F32 x, Qwen4F32Mut y, 
 }
 
 /* ---- forward (src/qwen4_moe.c:384-431) -------------------------------------------------- */
-Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen4MoeRoutes *routes, Qwen4MoeWork *w,
-                              Qwen4Error *err) {
+/* The two device calls of a streamed layer with the pool between them (the reference's remap hook,
+ * src/qwen4_moe_internal.h:49-54, and its caller's acquire/release, src/qwen4_forward_gpu.m). */
+static Qwen4Status streamed_forward(const Qwen4Moe *m, Qwen4MoeWork *w, QW4ExpertPool *pool, uint32_t layer, Qwen4F32 x,
+                                    Qwen4F32Mut y, Qwen4MoeRoutes *routes, Qwen4Error *err) {
+    const size_t T = x.dim[0], K = m->cfg.top_k, pairs = T * K;
+    const void *regions[3];
+    size_t expert_bytes[3], pool_slots = 0;
+    for (int j = 0; j < 3; j++) {
+        size_t region_bytes = 0;
+        regions[j] = qw4_pool_region(pool, j, &region_bytes);
+        expert_bytes[j] = m->w[1 + j].layout.expert_bytes;
+        if (!regions[j] || region_bytes % expert_bytes[j] || (j && region_bytes / expert_bytes[j] != pool_slots))
+            return moe_status(err, QW4_SHAPE, "the pool's slots do not hold this layer's experts");
+        pool_slots = region_bytes / expert_bytes[j];
+    }
+    uint32_t *ids = malloc(pairs * 2 * sizeof *ids), *slots = ids ? ids + pairs : NULL, word = 0;
+    if (!ids) return moe_status(err, QW4_OOM, "streaming staging");
+    Qwen4Status st = QW4_OK;
+    int rc = pf_hip_moe_route_streamed_host(m->device, w->device, x.data, x.stride_bytes[0], T, ids, &word);
+    if (rc) st = pf_device_status(rc, err, "qwen4_moe");
+    else if (word & PF_HIP_ERR_NONFINITE) st = moe_status(err, QW4_NONFINITE, "nonfinite value in the MoE block");
+    else if (word) st = moe_status(err, QW4_GPU_ERROR, "device error word");
+    else if (qw4_pool_acquire(pool, layer, ids, pairs, slots))
+        st = moe_status(err, QW4_IO, "expert pool: every slot pinned, or a read of the model file failed");
+    if (!st) {
+        rc = pf_hip_moe_experts_streamed_host(m->device, w->device, regions, expert_bytes, (uint32_t)pool_slots, slots, y.data,
+                                              y.stride_bytes[0], routes ? routes->ids.data : NULL,
+                                              routes ? routes->ids.row_stride_bytes : 0,
+                                              routes ? routes->weights.data : NULL,
+                                              routes ? routes->weights.stride_bytes[0] : 0, T, &word);
+        qw4_pool_release(pool, slots, pairs);
+        if (rc) st = pf_device_status(rc, err, "qwen4_moe");
+        else if (word & PF_HIP_ERR_NONFINITE) st = moe_status(err, QW4_NONFINITE, "nonfinite value in the MoE block");
+        else if (word) st = moe_status(err, QW4_GPU_ERROR, "device error word");
+        else st = moe_status(err, QW4_OK, "");
+    }
+    free(ids);
+    return st;
+}
+
+static Qwen4Status forward_checked(const Qwen4Moe *m, QW4ExpertPool *pool, uint32_t layer, Qwen4F32 x, Qwen4F32Mut y,
+                                   Qwen4MoeRoutes *routes, Qwen4MoeWork *w, Qwen4Error *err) {
     if (!m || !w) return moe_status(err, QW4_INVALID_ARGUMENT, "null forward handle");
     if (w->owner != m) return moe_status(err, QW4_OWNER, "workspace belongs to another MoE");
     if (!m->alive || w->failed) return moe_status(err, QW4_BAD_STATE, "inactive MoE/workspace; reset required");
     if (w->busy) return moe_status(err, QW4_BUSY, "workspace executing");
+    if (m->streamed != (pool != NULL))
+        return moe_status(err, QW4_BAD_STATE, m->streamed ? "a streamed layer forwards through an expert pool"
+                                                           : "the layer's experts are resident: no pool applies");
+    if (m->streamed && w->observer) return moe_status(err, QW4_BAD_STATE, "the observer needs the host weight bytes");
     const size_t T = x.dim[0], H = m->cfg.hidden_size, K = m->cfg.top_k;
     if (T > w->cap) return moe_status(err, QW4_CAPACITY, "batch exceeds token capacity");
     Range r[4];
@@ -524,6 +586,7 @@ Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen
     w->busy = true;
     Qwen4Status st;
     if (w->observer) st = observed_forward(w, x, y, routes, err);
+    else if (pool) st = streamed_forward(m, w, pool, layer, x, y, routes, err);
     else {
         uint32_t word = 0;
         int rc = pf_hip_moe_forward_host(m->device, w->device, x.data, x.stride_bytes[0], y.data, y.stride_bytes[0],
@@ -540,6 +603,17 @@ Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen
     else if (m->route_log) route_log_append((Qwen4Moe *)m, routes->ids.data, routes->ids.row_stride_bytes / 4, T);
     free(trace_memory);
     return st;
+}
+
+Qwen4Status qwen4_moe_forward(const Qwen4Moe *m, Qwen4F32 x, Qwen4F32Mut y, Qwen4MoeRoutes *routes, Qwen4MoeWork *w,
+                              Qwen4Error *err) {
+    return forward_checked(m, NULL, 0, x, y, routes, w, err);
+}
+
+Qwen4Status pf_moe_forward_streamed(const Qwen4Moe *m, QW4ExpertPool *pool, uint32_t layer, Qwen4F32 x, Qwen4F32Mut y,
+                                    Qwen4MoeRoutes *routes, Qwen4MoeWork *w, Qwen4Error *err) {
+    if (!pool) return moe_status(err, QW4_INVALID_ARGUMENT, "null expert pool");
+    return forward_checked(m, pool, layer, x, y, routes, w, err);
 }
 
 /* ---- the block between its two hyper-connection steps (src/qwen4_forward.c:362-367) ------------

@@ -71,9 +71,9 @@ Qwen4Status qw4_packed_layout_init(const GgufTensor *t, size_t logical, QW4Packe
 }
 
 /* Same admission as the reference's packed_view (src/qwen4_packed.c:35-50). */
-Qwen4Status pf_packed_admit(const QW4PackedCpuView *w, size_t expert) {
-    if (!w) return QW4_INVALID_ARGUMENT;
-    const QW4PackedLayout *l = &w->layout;
+/* The layout alone: a view of a tensor whose bytes are not in host memory (a streamed layer's routed tensors). */
+Qwen4Status pf_layout_admit(const QW4PackedLayout *l) {
+    if (!l) return QW4_INVALID_ARGUMENT;
     GgufTensor t;
     memset(&t, 0, sizeof t);
     t.type = l->gguf_type;
@@ -86,6 +86,14 @@ Qwen4Status pf_packed_admit(const QW4PackedCpuView *w, size_t expert) {
     if (memcmp(&want.k_storage, &l->k_storage, sizeof want - offsetof(QW4PackedLayout, k_storage)) ||
         want.gguf_type != l->gguf_type)
         return QW4_FORMAT;
+    return QW4_OK;
+}
+
+Qwen4Status pf_packed_admit(const QW4PackedCpuView *w, size_t expert) {
+    if (!w) return QW4_INVALID_ARGUMENT;
+    const QW4PackedLayout *l = &w->layout;
+    Qwen4Status st = pf_layout_admit(l);
+    if (st) return st;
     if (expert >= l->n_experts) return QW4_RANGE;
     if (w->span.bytes < l->tensor_bytes) return QW4_CAPACITY;
     if (!has_extent(w->span.data, l->tensor_bytes)) return QW4_INVALID_ARGUMENT;
