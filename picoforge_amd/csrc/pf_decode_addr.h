@@ -143,3 +143,14 @@ PF_HD size_t pf_q4t_chunk_at(size_t expert_bytes, size_t e, int row_tile, int kb
 }
 PF_HD size_t pf_q4t_header_at(int row_in_tile) { return 16 * (size_t)row_in_tile; }
 PF_HD size_t pf_q4t_piece_at(int run, int half, int row_in_tile) { return 512 + (size_t)run * 1024 + (size_t)half * 512 + 16 * (size_t)row_in_tile; }
+
+// ---- tile-ordered IQ2_XXS (32 rows x one 256-block = 2176 bytes: per 64-weight run the rows' 16-byte pieces -- two
+// 32-groups of four grid indices and a sign/scale word each -- then the rows' 32 half scales and 64 bytes of padding
+// that keep every piece group on whole 128-byte lines) ----
+#define PF_I2T_CHUNK 2176
+PF_HD size_t pf_i2t_expert_bytes(int n_out, int kblocks) { return (size_t)(n_out / 32) * kblocks * PF_I2T_CHUNK; }
+PF_HD size_t pf_i2t_chunk_at(size_t expert_bytes, size_t e, int row_tile, int kblocks, int kb) {
+    return e * expert_bytes + ((size_t)row_tile * kblocks + kb) * PF_I2T_CHUNK;
+}
+PF_HD size_t pf_i2t_scale_at(int row_in_tile) { return 2048 + 2 * (size_t)row_in_tile; }
+PF_HD size_t pf_i2t_piece_at(int run, int row_in_tile) { return (size_t)run * 512 + 16 * (size_t)row_in_tile; }

@@ -273,6 +273,30 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             }
         }
     }
+    {   // IQ2_XXS layers: a tile-ordered second copy of the expert tensors for the decode kernels whose lanes are weight
+        // rows (doubles the expert bytes; PF_MOE_PREFILL_COPY=0 does without it, as for Q4_K)
+        const char *copy = getenv("PF_MOE_PREFILL_COPY");
+        bool all_iq2 = m->decode_ready;
+        for (int a = 1; a <= 6; a++) all_iq2 &= desc->type[a] == PF_IQ2_XXS && n_out[a] % 32 == 0;
+        hipError_t e = hipSuccess;
+        if (all_iq2 && (!copy || strcmp(copy, "0") != 0)) {
+            for (int a = 1; a <= 6 && e == hipSuccess; a++) {
+                const size_t bytes = pf_i2t_expert_bytes((int)n_out[a], m->blocks_per_row[a]) * experts[a];
+                e = hipMalloc((void **)&m->w_itile[a], bytes);
+                if (e == hipSuccess) {
+                    pf_launch_iq2_tile(m->w[a], reinterpret_cast<const uint16_t *>(m->w[a] + m->scale_offset[a]), m->w_itile[a],
+                                       (size_t)n_out[a] * experts[a], m->blocks_per_row[a], nullptr);
+                    m->total_bytes += bytes;
+                }
+            }
+            if (e == hipSuccess) e = hipDeviceSynchronize();
+            if (e != hipSuccess) {
+                pf_set_error("tile-ordered weights", e);
+                pf_hip_moe_destroy(m);
+                return e == hipErrorOutOfMemory ? PF_HIP_E_MEMORY : PF_HIP_E_RUNTIME;
+            }
+        }
+    }
     *out = m;
     return PF_HIP_OK;
 }
@@ -283,6 +307,7 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
     if (m->w_norm2) (void)hipFree(m->w_norm2);
     if (m->router_t) (void)hipFree(m->router_t);
     for (int a = 0; a < 8; a++) if (m->w_tiled[a]) (void)hipFree(m->w_tiled[a]);
+    for (int a = 0; a < 8; a++) if (m->w_itile[a]) (void)hipFree(m->w_itile[a]);
     free(m);
 }
 
@@ -299,9 +324,9 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden, I = d->inter;
     const size_t Td = T < PF_DECODE_MAX_TOKENS ? T : PF_DECODE_MAX_TOKENS;   // tokens per decode launch
     // ... and per launch of the kernels for tile-ordered Q4_K (whether the copies are kept is not known here)
-    bool q4k = true;
-    for (int t = 1; t <= 6; t++) q4k &= d->type[t] == PF_Q4_K;
-    const size_t Tt = !q4k ? Td : T < PF_TILE_DECODE_MAX_TOKENS ? T : PF_TILE_DECODE_MAX_TOKENS;
+    bool one_format = d->type[1] == PF_Q4_K || d->type[1] == PF_IQ2_XXS;
+    for (int t = 2; t <= 6; t++) one_format &= d->type[t] == d->type[1];
+    const size_t Tt = !one_format ? Td : T < PF_TILE_DECODE_MAX_TOKENS ? T : PF_TILE_DECODE_MAX_TOKENS;
     size_t want[W_COUNT];
     want[W_LOGITS] = T * E * 4;
     want[W_SSQ] = T * E * 4;
@@ -469,7 +494,7 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.group_bad = w->group_bad; a.tiles = w->tiles;
     a.token_cap = (uint32_t)w->cap;
     a.router_t = m->router_t;
-    for (int j = 0; j < 8; j++) a.wt[j] = m->w_tiled[j];
+    for (int j = 0; j < 8; j++) { a.wt[j] = m->w_tiled[j]; a.wi[j] = m->w_itile[j]; }
     return a;
 }
 
@@ -482,7 +507,7 @@ struct HcTarget {   // residual streams to inject into instead of writing y
 
 // Most tokens the decode kernels take in one forward of this layer.
 static size_t decode_limit(const PfHipMoe *moe) {
-    return pf_decode_tile_layer(moe->desc, moe->w_tiled) ? PF_TILE_DECODE_MAX_TOKENS : PF_DECODE_MAX_TOKENS;
+    return pf_decode_tile_layer(moe->desc, moe->w_tiled, moe->w_itile) ? PF_TILE_DECODE_MAX_TOKENS : PF_DECODE_MAX_TOKENS;
 }
 
 static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch, float *d_y,

@@ -839,17 +839,37 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
 // added in a fixed order.  Routing as in pf_k_dec_gate_up1.
 typedef const __attribute__((address_space(4))) uint32_t *PfScalarWords;   // read through the scalar cache
 
-struct Q4TileItem { uint4 hdr, piece[2]; };   // a row's header and the two halves of one 64-weight run
+template <int FMT> struct TileItem;
+template <> struct TileItem<PF_Q4_K> { uint4 hdr, piece[2]; };   // a row's header and the two halves of one 64-weight run
+template <> struct TileItem<PF_IQ2_XXS> { uint4 piece; uint32_t dbits; };   // two 32-groups (indices, sign/scale word) and the block's half scale
+typedef TileItem<PF_Q4_K> Q4TileItem;
 
-__device__ __forceinline__ void q4t_load(Q4TileItem &w, const uint8_t *chunk, int row, int run) {
+template <int FMT> struct TileGeometry;
+template <> struct TileGeometry<PF_Q4_K> {
+    static __device__ __forceinline__ size_t expert_bytes(const PfKernelArgs &a, int t) { return a.expert_bytes[t]; }
+    static __device__ __forceinline__ size_t chunk_at(int row_tile, int kblocks, int kb) { return pf_q4t_chunk_at(0, 0, row_tile, kblocks, kb); }
+    static __device__ __forceinline__ const uint8_t *tensor(const PfKernelArgs &a, int t) { return a.wt[t]; }
+};
+template <> struct TileGeometry<PF_IQ2_XXS> {
+    static __device__ __forceinline__ size_t expert_bytes(const PfKernelArgs &a, int t) { return pf_i2t_expert_bytes(a.n_out[t], a.blocks_per_row[t]); }
+    static __device__ __forceinline__ size_t chunk_at(int row_tile, int kblocks, int kb) { return pf_i2t_chunk_at(0, 0, row_tile, kblocks, kb); }
+    static __device__ __forceinline__ const uint8_t *tensor(const PfKernelArgs &a, int t) { return a.wi[t]; }
+};
+
+__device__ __forceinline__ void q4t_load(TileItem<PF_Q4_K> &w, const uint8_t *chunk, int row, int run) {
     w.hdr = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_header_at(row));
     w.piece[0] = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(run, 0, row));
     w.piece[1] = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(run, 1, row));
 }
+__device__ __forceinline__ void q4t_load(TileItem<PF_IQ2_XXS> &w, const uint8_t *chunk, int row, int run) {
+    w.piece = *reinterpret_cast<const uint4 *>(chunk + pf_i2t_piece_at(run, row));
+    w.dbits = *reinterpret_cast<const uint16_t *>(chunk + pf_i2t_scale_at(row));
+}
 
 // groups 2 * run, 2 * run + 1 of the row's block (low and high nibbles of the run's bytes) against the image's digits,
 // steps and sums of the same two groups (uniform pointers)
-__device__ __forceinline__ float q4t_dot(const Q4TileItem &w, PfScalarWords digits, PfScalarWords steps, PfScalarWords sums, int run) {
+__device__ __forceinline__ float q4t_dot(const Q4TileItem &w, PfScalarWords digits, PfScalarWords steps, PfScalarWords sums, int run,
+                                         const uint32_t *) {
     // the two groups' 6-bit scales and minima (src/qwen4_packed.c:89-90): bytes 2 * run, 2 * run + 1 of the packed twelve
     uint32_t sc2, mn2;
     if (run < 2) {
@@ -881,6 +901,33 @@ __device__ __forceinline__ float q4t_dot(const Q4TileItem &w, PfScalarWords digi
     return fmaf(__uint_as_float(steps[0]), t0, __uint_as_float(steps[1]) * t1);
 }
 
+// IQ2_XXS: the run's two 32-groups; tables as in wseg_dot<PF_IQ2_XXS> (LDS: four signed magnitudes per grid entry and
+// sign nibble); the digits as scalar operands
+__device__ __forceinline__ float q4t_dot(const TileItem<PF_IQ2_XXS> &w, PfScalarWords digits, PfScalarWords steps, PfScalarWords sums, int,
+                                         const uint32_t *tables) {
+    (void)sums;
+    float acc[2];
+#pragma unroll
+    for (int gg = 0; gg < 2; gg++) {
+        const uint32_t idx = gg ? w.piece.z : w.piece.x, word = gg ? w.piece.w : w.piece.y;
+        PfScalarWords dg = digits + 16 * gg;
+        int lo = 0, hi = 0;
+#pragma unroll
+        for (int slot = 0; slot < 4; slot++) {
+            const uint32_t g = (idx >> (8 * slot)) & 255u, s7 = (word >> (7 * slot)) & 127u;
+            const uint32_t par = __popc(s7) & 1u;
+            const int ml = (int)tables[(g << 4) | (s7 & 15u)];
+            const int mh = (int)tables[4096u + ((g << 4) | (s7 >> 4) | (par << 3))];
+            lo = __builtin_amdgcn_sdot4(ml, (int)dg[2 * slot], lo, false);
+            hi = __builtin_amdgcn_sdot4(ml, (int)dg[8 + 2 * slot], hi, false);
+            lo = __builtin_amdgcn_sdot4(mh, (int)dg[2 * slot + 1], lo, false);
+            hi = __builtin_amdgcn_sdot4(mh, (int)dg[8 + 2 * slot + 1], hi, false);
+        }
+        acc[gg] = __uint_as_float(steps[gg]) * (float)(2u * (word >> 28) + 1u) * (float)(lo + (hi << 8));
+    }
+    return half_bits(w.dbits) * 0.125f * (acc[0] + acc[1]);
+}
+
 // The tile's rows against the token: the 64-weight runs of all the rows go round the waves 1..15 (wave 0
 // routes); a wave adds up its runs and leaves one partial sum per lane in LDS: partial[wave - 1][64].
 #define Q4T_ITEMS 3   // run items a wave can hold: hidden <= 2816
@@ -890,6 +937,7 @@ struct Q4TilePlan {   // what does not depend on the expert: set up before the e
     int row, kblocks, items, groups;
 };
 
+template <int FMT>
 __device__ __forceinline__ Q4TilePlan q4t_plan(const PfKernelArgs &a, bool shared, int n0) {
     Q4TilePlan p;
     const int lane = pf_lane();
@@ -899,24 +947,28 @@ __device__ __forceinline__ Q4TilePlan q4t_plan(const PfKernelArgs &a, bool share
     p.groups = a.hidden / 32;
     // the two tensors by scalar selects and one per-lane choice (an index computed per lane would fetch the pointer
     // from the argument block through the vector memory path, a round trip before the first weight request)
+    typedef TileGeometry<FMT> G;
     const bool up = lane >= 32;
-    const uint8_t *gate_w = shared ? a.wt[4] : a.wt[1], *up_w = shared ? a.wt[5] : a.wt[2];
-    const size_t gate_bytes = shared ? a.expert_bytes[4] : a.expert_bytes[1], up_bytes = shared ? a.expert_bytes[5] : a.expert_bytes[2];
-    p.base = (up ? up_w : gate_w) + pf_q4t_chunk_at(0, 0, n0 / 32, p.kblocks, 0);
+    const uint8_t *gate_w = shared ? G::tensor(a, 4) : G::tensor(a, 1), *up_w = shared ? G::tensor(a, 5) : G::tensor(a, 2);
+    const size_t gate_bytes = shared ? G::expert_bytes(a, 4) : G::expert_bytes(a, 1);
+    const size_t up_bytes = shared ? G::expert_bytes(a, 5) : G::expert_bytes(a, 2);
+    p.base = (up ? up_w : gate_w) + G::chunk_at(n0 / 32, p.kblocks, 0);
     p.expert_bytes = up ? up_bytes : gate_bytes;
     return p;
 }
 
-__device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, const Q4TilePlan &p, float *partial, uint32_t e, int wave) {
+template <int FMT>
+__device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, const Q4TilePlan &p, float *partial, const uint32_t *tables,
+                                         uint32_t e, int wave) {
     if (wave == 0) return;
     const int lane = pf_lane();
     const uint8_t *tile = p.base + (size_t)e * p.expert_bytes;
     const PfScalarWords image = (PfScalarWords)(uintptr_t)a.ximg;
-    Q4TileItem w[Q4T_ITEMS];
+    TileItem<FMT> w[Q4T_ITEMS];
 #pragma unroll
     for (int k = 0; k < Q4T_ITEMS; k++) {
         const int it = wave - 1 + 15 * k;
-        if (it < p.items) q4t_load(w[k], tile + pf_q4t_chunk_at(0, 0, 0, p.kblocks, it >> 2), p.row, it & 3);
+        if (it < p.items) q4t_load(w[k], tile + TileGeometry<FMT>::chunk_at(0, p.kblocks, it >> 2), p.row, it & 3);
     }
     float total = 0.0f;
 #pragma unroll
@@ -924,7 +976,7 @@ __device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, const Q4TilePlan
         const int it = wave - 1 + 15 * k;
         if (it < p.items) {
             const int g = 2 * it;   // the run's first group within the row
-            total += q4t_dot(w[k], image + 16 * g, image + 16 * p.groups + g, image + 17 * p.groups + g, it & 3);
+            total += q4t_dot(w[k], image + 16 * g, image + 16 * p.groups + g, image + 17 * p.groups + g, it & 3, tables);
         }
     }
     partial[(wave - 1) * 64 + lane] = total;
@@ -946,7 +998,7 @@ __device__ __forceinline__ void q4t_at_token(PfKernelArgs &a, int t) {
     a.aimg += (size_t)t * (a.top_k + 1) * pf_image2_words(widest);
 }
 
-template <int NPL>
+template <int NPL, int FMT>
 __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
@@ -954,7 +1006,13 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
     q4t_at_token(a, (int)blockIdx.y);
     const int H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    float *partial = reinterpret_cast<float *>(lds);   // [15 waves][64 lanes]
+    // IQ2_XXS: the signed-magnitude tables first (32 KB, staged by every wave but the routing one)
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
+    if (FMT == PF_IQ2_XXS && wave != 0) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.iq2_signed);
+        for (int i = (int)threadIdx.x - 64; i < 2048; i += 960) reinterpret_cast<uint4 *>(tables)[i] = src[i];
+    }
+    float *partial = reinterpret_cast<float *>(lds + table_words<FMT>());   // [15 waves][64 lanes]
     float *scratch = partial + 15 * 64;   // the serial-order routing's arrays
     const bool shared = (int)blockIdx.x >= routed_blocks;
     const int tiles = a.inter / 32;
@@ -989,12 +1047,12 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
         const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)my_key, u);
         if (lane == 0) early_expert = mine ? pf_key_id(mine) : 0xffffffffu;
     }
-    const Q4TilePlan plan = q4t_plan(a, shared, n0);
+    const Q4TilePlan plan = q4t_plan<FMT>(a, shared, n0);
     const int I = shared ? a.shared_inter : a.inter;
-    if (!shared) __syncthreads();
+    if (!shared || FMT == PF_IQ2_XXS) __syncthreads();   // the early expert; the tables
     const uint32_t early = shared ? 0u : early_expert;
     const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
-    q4t_tile(a, plan, partial, early_ok ? early : 0u, wave);
+    q4t_tile<FMT>(a, plan, partial, tables, early_ok ? early : 0u, wave);
     if (wave == 0 && !shared) {
         // the remaining slots, the candidate beyond them and one more key, while the other waves' weight bytes travel
         for (int r = u + 1; r <= rounds; r++) {
@@ -1024,7 +1082,7 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
         e = R.ids[u];
         if (e != early && e < (uint32_t)E) {
             __syncthreads();
-            q4t_tile(a, plan, partial, e, wave);
+            q4t_tile<FMT>(a, plan, partial, tables, e, wave);
             __syncthreads();
         }
         if (blockIdx.x == 0) {
@@ -1070,8 +1128,8 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
 
 // With several tokens there are more workgroups than compute units; two workgroups per compute unit (64 registers a
 // lane) measured slower than one after the other: the products are bound by the vector units, not by waiting.
-template <int NPL>
-__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) { q4t_gate_up<NPL>(a, routed_blocks); }
+template <int NPL, int FMT>
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) { q4t_gate_up<NPL, FMT>(a, routed_blocks); }
 
 // ---- kernel 3: down products and the combine ---------------------------------------------------
 // blockIdx.x = t * row_blocks + nb; one wave per slot plus one for the shared expert; a routed
@@ -1195,15 +1253,94 @@ __global__ void __launch_bounds__(MAXT) pf_k_dec_down(PfKernelArgs a, int row_bl
 // eight rows' pieces of a run are one 128-byte line of the tile-ordered copy.  The activation digits come
 // from the two-digit images kernel 2 left in global memory (nothing is built here); the lanes of a row add
 // up across the wave, the slots meet in LDS and are combined in slot order.
-__global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a);
-#if PF_DECODE_PART == 0
+// One run of one row (its item loaded by q4t_load) against the slot's digits in LDS (mine: the slot's image).  Q4_K: header
+// and two halves; IQ2_XXS: one 16-byte piece and the block's half scale, magnitudes from the tables.
+__device__ __forceinline__ float down_dot(const TileItem<PF_Q4_K> &w, int rr, const uint32_t *mine, int run, int groups, const uint32_t *) {
+    const uint4 hdr = w.hdr, p0 = w.piece[0], p1 = w.piece[1];
+    uint4 dg[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) dg[i] = reinterpret_cast<const uint4 *>(mine + 32 * run)[i];
+    const uint2 st = *reinterpret_cast<const uint2 *>(mine + 16 * groups + 2 * run);
+    const uint2 sm = *reinterpret_cast<const uint2 *>(mine + 17 * groups + 2 * run);
+    uint32_t sc2, mn2;
+    if (rr < 2) {
+        sc2 = (hdr.y >> (16 * rr)) & 0x3F3Fu;
+        mn2 = (hdr.z >> (16 * rr)) & 0x3F3Fu;
+    } else {
+        const int sh = 16 * (rr - 2);
+        sc2 = ((hdr.w >> sh) & 0x0F0Fu) | (((hdr.y >> sh) >> 2) & 0x3030u);
+        mn2 = (((hdr.w >> sh) >> 4) & 0x0F0Fu) | (((hdr.z >> sh) >> 2) & 0x3030u);
+    }
+    const float d = half_bits(hdr.x & 0xffffu), dmin = half_bits(hdr.x >> 16);
+    // dg[0..1]: low digits of the even group, dg[2..3] its high digits, dg[4..7] the odd group's
+    const uint32_t e0[8] = {dg[0].x, dg[0].y, dg[0].z, dg[0].w, dg[1].x, dg[1].y, dg[1].z, dg[1].w};
+    const uint32_t e1[8] = {dg[2].x, dg[2].y, dg[2].z, dg[2].w, dg[3].x, dg[3].y, dg[3].z, dg[3].w};
+    const uint32_t o0[8] = {dg[4].x, dg[4].y, dg[4].z, dg[4].w, dg[5].x, dg[5].y, dg[5].z, dg[5].w};
+    const uint32_t o1[8] = {dg[6].x, dg[6].y, dg[6].z, dg[6].w, dg[7].x, dg[7].y, dg[7].z, dg[7].w};
+    const uint32_t q[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+    int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+        lo0 = __builtin_amdgcn_sdot4(lo, (int)e0[i], lo0, false);
+        lo1 = __builtin_amdgcn_sdot4(lo, (int)e1[i], lo1, false);
+        hi0 = __builtin_amdgcn_sdot4(hi, (int)o0[i], hi0, false);
+        hi1 = __builtin_amdgcn_sdot4(hi, (int)o1[i], hi1, false);
+    }
+    const float s0 = (float)(sc2 & 255u), m0 = (float)(mn2 & 255u), s1 = (float)(sc2 >> 8), m1 = (float)(mn2 >> 8);
+    const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sm.x);
+    const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sm.y);
+    return fmaf(__uint_as_float(st.x), t0, __uint_as_float(st.y) * t1);
+}
+
+// (tables: here the 256-entry magnitude grid, 2 KB, not the signed tables: staging 32 KB per workgroup cost this
+// kernel more than the sign arithmetic does)
+__device__ __forceinline__ float down_dot(const TileItem<PF_IQ2_XXS> &w, int, const uint32_t *mine, int run, int groups,
+                                          const uint32_t *tables) {
+    const uint4 piece = w.piece;
+    const uint32_t dbits = w.dbits;
+    uint4 dg[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) dg[i] = reinterpret_cast<const uint4 *>(mine + 32 * run)[i];
+    const uint2 st = *reinterpret_cast<const uint2 *>(mine + 16 * groups + 2 * run);
+    const uint32_t d32[32] = {dg[0].x, dg[0].y, dg[0].z, dg[0].w, dg[1].x, dg[1].y, dg[1].z, dg[1].w,
+                              dg[2].x, dg[2].y, dg[2].z, dg[2].w, dg[3].x, dg[3].y, dg[3].z, dg[3].w,
+                              dg[4].x, dg[4].y, dg[4].z, dg[4].w, dg[5].x, dg[5].y, dg[5].z, dg[5].w,
+                              dg[6].x, dg[6].y, dg[6].z, dg[6].w, dg[7].x, dg[7].y, dg[7].z, dg[7].w};
+    float acc[2];
+#pragma unroll
+    for (int gg = 0; gg < 2; gg++) {
+        const uint32_t idx = gg ? piece.z : piece.x, word = gg ? piece.w : piece.y;
+        int lo = 0, hi = 0;
+#pragma unroll
+        for (int slot = 0; slot < 4; slot++) {
+            const uint32_t g = (idx >> (8 * slot)) & 255u, s7 = (word >> (7 * slot)) & 127u;
+            const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);   // the eighth sign is the parity of the seven
+            // the grid entry's eight magnitudes (8, 25 or 43: never zero) with the signs applied byte by byte: sign bit i
+            // of a nibble moved to bit 8i, widened to a byte mask, then ~m + 1 in every flagged byte (no byte overflows)
+            const uint2 mag = reinterpret_cast<const uint2 *>(tables)[g];
+            const uint32_t tl = ((s8 & 15u) * 0x00204081u) & 0x01010101u, th = ((s8 >> 4) * 0x00204081u) & 0x01010101u;
+            const int ml = (int)((mag.x ^ (tl * 0xFFu)) + tl), mh = (int)((mag.y ^ (th * 0xFFu)) + th);
+            lo = __builtin_amdgcn_sdot4(ml, (int)d32[16 * gg + 2 * slot], lo, false);
+            hi = __builtin_amdgcn_sdot4(ml, (int)d32[16 * gg + 8 + 2 * slot], hi, false);
+            lo = __builtin_amdgcn_sdot4(mh, (int)d32[16 * gg + 2 * slot + 1], lo, false);
+            hi = __builtin_amdgcn_sdot4(mh, (int)d32[16 * gg + 8 + 2 * slot + 1], hi, false);
+        }
+        acc[gg] = __uint_as_float(gg ? st.y : st.x) * (float)(2u * (word >> 28) + 1u) * (float)(lo + (hi << 8));
+    }
+    return half_bits(dbits) * 0.125f * (acc[0] + acc[1]);
+}
+
+template <int FMT>
 __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
     __shared__ float partial[17][8];
-    extern __shared__ int images[];   // [slot][image words of the widest activation row]
+    extern __shared__ int lds[];   // IQ2_XXS: the magnitude grid; then [slot][image words of the widest activation row]
     const int token = (int)blockIdx.y;
     q4t_at_token(a, token);
     const int H = a.hidden, K = a.top_k, lane = pf_lane();
     const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
+    int *images = lds + (FMT == PF_IQ2_XXS ? 512 * (K + 1) : 0);   // IQ2_XXS: the waves' copies of the magnitude grid first
     const bool shared = s == K;
     const int I = shared ? a.shared_inter : a.inter;
     const int n_base = 8 * (int)blockIdx.x, r = lane & 7, part = lane >> 3;
@@ -1221,11 +1358,22 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
     }
     PfOutputRegs out_regs;
     if ((int)threadIdx.x < 8) pf_output_prefetch(a, token, n_base + threadIdx.x, out_regs);
-    const uint8_t *w = (shared ? a.wt[6] : a.wt[3]) + (size_t)e * (shared ? a.expert_bytes[6] : a.expert_bytes[3]);
+    typedef TileGeometry<FMT> G;
+    const int tensor = shared ? 6 : 3;
+    const uint8_t *w = (shared ? G::tensor(a, 6) : G::tensor(a, 3)) + (size_t)e * (shared ? G::expert_bytes(a, 6) : G::expert_bytes(a, 3));
+    (void)tensor;
     const int kblocks = (shared ? a.shared_inter : a.down_physical) / 256, runs = I / 64, groups = I / 32;
     const uint32_t *image = a.aimg + (size_t)s * pf_image2_words(widest);   // slot = unique expert with one token; the shared expert's follows
-    const uint8_t *tile = w + pf_q4t_chunk_at(0, 0, n_base / 32, kblocks, 0);
+    const uint8_t *tile = w + G::chunk_at(n_base / 32, kblocks, 0);
     const int row_in_tile = (n_base & 31) + r;
+    // IQ2_XXS: every wave keeps its own copy of the 2 KB magnitude grid, so that no wave waits for another before the
+    // final sums (a shared copy needs a workgroup barrier between its staging and its first use)
+    if (FMT == PF_IQ2_XXS) {
+        tables += 512 * s;
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.iq2_grid);
+        reinterpret_cast<uint4 *>(tables)[lane] = src[lane];
+        reinterpret_cast<uint4 *>(tables)[64 + lane] = src[64 + lane];
+    }
     // the slot's image into this wave's part of LDS (each lane needs the digits of its own run; fetched per lane they
     // would cost eight requests a lane)
     uint32_t *mine = reinterpret_cast<uint32_t *>(images) + (size_t)s * pf_image2_words(widest);
@@ -1234,46 +1382,10 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
     float total = 0.0f;
     bool fenced = false;
     for (int run = part; run < runs; run += 8) {
-        const uint8_t *chunk = tile + pf_q4t_chunk_at(0, 0, 0, kblocks, run >> 2);
-        const int rr = run & 3;
-        const uint4 hdr = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_header_at(row_in_tile));
-        const uint4 p0 = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(rr, 0, row_in_tile));
-        const uint4 p1 = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(rr, 1, row_in_tile));
-        if (!fenced) { pf_wave_lds_fence(); fenced = true; }   // the image's stores of this wave before its reads
-        uint4 dg[8];
-#pragma unroll
-        for (int i = 0; i < 8; i++) dg[i] = reinterpret_cast<const uint4 *>(mine + 32 * run)[i];
-        const uint2 st = *reinterpret_cast<const uint2 *>(mine + 16 * groups + 2 * run);
-        const uint2 sm = *reinterpret_cast<const uint2 *>(mine + 17 * groups + 2 * run);
-        uint32_t sc2, mn2;
-        if (rr < 2) {
-            sc2 = (hdr.y >> (16 * rr)) & 0x3F3Fu;
-            mn2 = (hdr.z >> (16 * rr)) & 0x3F3Fu;
-        } else {
-            const int sh = 16 * (rr - 2);
-            sc2 = ((hdr.w >> sh) & 0x0F0Fu) | (((hdr.y >> sh) >> 2) & 0x3030u);
-            mn2 = (((hdr.w >> sh) >> 4) & 0x0F0Fu) | (((hdr.z >> sh) >> 2) & 0x3030u);
-        }
-        const float d = half_bits(hdr.x & 0xffffu), dmin = half_bits(hdr.x >> 16);
-        // dg[0..1]: low digits of the even group, dg[2..3] its high digits, dg[4..7] the odd group's
-        const uint32_t e0[8] = {dg[0].x, dg[0].y, dg[0].z, dg[0].w, dg[1].x, dg[1].y, dg[1].z, dg[1].w};
-        const uint32_t e1[8] = {dg[2].x, dg[2].y, dg[2].z, dg[2].w, dg[3].x, dg[3].y, dg[3].z, dg[3].w};
-        const uint32_t o0[8] = {dg[4].x, dg[4].y, dg[4].z, dg[4].w, dg[5].x, dg[5].y, dg[5].z, dg[5].w};
-        const uint32_t o1[8] = {dg[6].x, dg[6].y, dg[6].z, dg[6].w, dg[7].x, dg[7].y, dg[7].z, dg[7].w};
-        const uint32_t q[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-        int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
-            lo0 = __builtin_amdgcn_sdot4(lo, (int)e0[i], lo0, false);
-            lo1 = __builtin_amdgcn_sdot4(lo, (int)e1[i], lo1, false);
-            hi0 = __builtin_amdgcn_sdot4(hi, (int)o0[i], hi0, false);
-            hi1 = __builtin_amdgcn_sdot4(hi, (int)o1[i], hi1, false);
-        }
-        const float s0 = (float)(sc2 & 255u), m0 = (float)(mn2 & 255u), s1 = (float)(sc2 >> 8), m1 = (float)(mn2 >> 8);
-        const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sm.x);
-        const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sm.y);
-        total += fmaf(__uint_as_float(st.x), t0, __uint_as_float(st.y) * t1);
+        TileItem<FMT> item;
+        q4t_load(item, tile + G::chunk_at(0, kblocks, run >> 2), row_in_tile, run & 3);
+        if (!fenced) { pf_wave_lds_fence(); fenced = true; }   // the image's (and grid's) stores of this wave before its reads
+        total += down_dot(item, run & 3, mine, run, groups, tables);
     }
     // the row's runs: lanes r, r + 8, ..., r + 56
     total += __shfl_xor(total, 8);
@@ -1291,9 +1403,37 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
         if (!pf_output_commit(a, token, n, y, out_regs)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
     }
 }
-#endif
 
 #if PF_DECODE_PART == 0
+// ---- IQ2_XXS in tile order ---------------------------------------------------------------------------
+// From the split device layout (64-byte payloads row by row, half scales apart) to the chunks of pf_decode_addr.h per
+// (32-row tile, 256-block): per 64-weight run the rows' 16-byte pieces, then the 32 rows' scales.  One thread per 16-byte piece or
+// per scale; rows is a multiple of 32.
+__global__ void pf_k_iq2_tile(const uint8_t *payload, const uint16_t *scales, uint8_t *dst, size_t rows, int blocks_per_row) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, per_chunk = 128 + 32;
+    const size_t chunk = i / per_chunk, tile = chunk / blocks_per_row, kb = chunk % blocks_per_row;
+    if (chunk >= rows / 32 * (size_t)blocks_per_row) return;
+    const int p = (int)(i % per_chunk);
+    uint8_t *out = dst + chunk * PF_I2T_CHUNK;
+    if (p < 128) {
+        const int run = p >> 5, row = p & 31;
+        const size_t n = 32 * tile + row;
+        *reinterpret_cast<uint4 *>(out + pf_i2t_piece_at(run, row)) =
+            *reinterpret_cast<const uint4 *>(payload + (n * blocks_per_row + kb) * 64 + 16 * run);
+    } else {
+        const int row = p - 128;
+        const size_t n = 32 * tile + row;
+        *reinterpret_cast<uint16_t *>(out + pf_i2t_scale_at(row)) = scales[n * blocks_per_row + kb];
+    }
+}
+
+void pf_launch_iq2_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8_t *d_dst, size_t rows, int blocks_per_row,
+                        hipStream_t stream) {
+    const size_t threads = rows / 32 * (size_t)blocks_per_row * 160;
+    hipLaunchKernelGGL(pf_k_iq2_tile, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, d_payload, d_scales, d_dst, rows,
+                       blocks_per_row);
+}
+
 // ---- IQ2_XXS upload split -------------------------------------------------------------------------
 __global__ void pf_k_iq2_split(const uint8_t *gguf, uint8_t *payload, uint16_t *scales, size_t blocks) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;   // one 16-bit word of a block per thread
@@ -1434,17 +1574,22 @@ static void launch_down(const PfKernelArgs &a, dim3 grid, dim3 block, size_t lds
         launch_down_bounded<FD, FS, NT, SPL, 1024>(a, grid, block, lds, stream, row_blocks, rows_per_block, image_pitch);
 }
 
-// Every expert tensor Q4_K with its tile-ordered copy kept, and widths the kernels whose lanes are weight rows
-// cover: those take the layer, one token per grid row, for up to PF_TILE_DECODE_MAX_TOKENS tokens.
-bool pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const tiled[8]);
+// Every expert tensor Q4_K, or every one IQ2_XXS, with its tile-ordered copy kept, and widths the kernels whose lanes
+// are weight rows cover: those take the layer, one token per grid row, for up to PF_TILE_DECODE_MAX_TOKENS tokens.
+// Returns the format, 0 for other layers.
 #if PF_DECODE_PART == 0
-bool pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const tiled[8]) {
+uint32_t pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const q4k_tiled[8], const uint8_t *const iq2_tiled[8]) {
+    const uint32_t format = d.type[1];
+    if (format != PF_Q4_K && format != PF_IQ2_XXS) return 0;
     for (int t = 1; t <= 6; t++)
-        if (d.type[t] != PF_Q4_K || !tiled[t]) return false;
-    return d.hidden % 256 == 0 && 4 * (d.hidden / 256) <= 15 * Q4T_ITEMS && d.inter % 64 == 0 && d.shared_inter % 64 == 0 &&
-           d.down_physical == d.inter && d.top_k < d.experts && d.top_k <= 15;
+        if (d.type[t] != format || !(format == PF_Q4_K ? q4k_tiled[t] : iq2_tiled[t])) return 0;
+    const bool fits = d.hidden % 256 == 0 && 4 * (d.hidden / 256) <= 15 * Q4T_ITEMS && d.inter % 256 == 0 &&
+                      d.shared_inter % 256 == 0 && d.down_physical == d.inter && d.top_k < d.experts && d.top_k <= 15 &&
+                      d.experts <= 1024;
+    return fits ? format : 0;
 }
 
+template <int FMT>
 static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
     const int router_blocks = (E + 3) / 4, last = stage_limit ? stage_limit : 3;
@@ -1454,16 +1599,16 @@ static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t str
     const int routed_blocks = K * (I / 32);
     const dim3 g1(routed_blocks + Is / 32, tokens);
     const int all = (E + 63) / 64;
-    const size_t lds = (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
-    if (all <= 1) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<1>, g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 2) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<2>, g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 4) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<4>, g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 8) hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<8>, g1, dim3(1024), lds, stream, a, routed_blocks);
-    else hipLaunchKernelGGL(pf_k_dec_gate_up_q4t<16>, g1, dim3(1024), lds, stream, a, routed_blocks);
+    const size_t lds = (size_t)table_words<FMT>() * 4 + (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+    if (all <= 1) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<1, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 2) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<2, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 4) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<4, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 8) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<8, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<16, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
     if (last < 3) return;
     const size_t widest = I > Is ? I : Is;
-    hipLaunchKernelGGL(pf_k_dec_down_q4t, dim3(H / 8, tokens), dim3(64 * (K + 1)), (size_t)(K + 1) * pf_image2_words(widest) * 4,
-                       stream, a);
+    hipLaunchKernelGGL((pf_k_dec_down_q4t<FMT>), dim3(H / 8, tokens), dim3(64 * (K + 1)),
+                       (FMT == PF_IQ2_XXS ? 2048 * (size_t)(K + 1) : 0) + (size_t)(K + 1) * pf_image2_words(widest) * 4, stream, a);
 }
 #endif
 
@@ -1530,19 +1675,26 @@ void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t s
 void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 
 #if PF_DECODE_PART == 0
-void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+static PfHipMoeDesc desc_of(const PfKernelArgs &a) {
     PfHipMoeDesc d = {};
     d.hidden = a.hidden; d.experts = a.experts; d.top_k = a.top_k; d.inter = a.inter; d.shared_inter = a.shared_inter;
     d.down_physical = a.down_physical;
     for (int t = 0; t < 8; t++) d.type[t] = a.type[t];
-    if (pf_decode_tile_layer(d, a.wt)) launch_decode_q4t(a, tokens, stream, stage_limit);
+    return d;
+}
+
+void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi) == PF_Q4_K) launch_decode_q4t<PF_Q4_K>(a, tokens, stream, stage_limit);
     else launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     switch (decode_combination(a.type)) {
     case 1: pf_launch_decode_q4k(a, tokens, stream, stage_limit); break;
-    case 2: pf_launch_decode_iq2(a, tokens, stream, stage_limit); break;
+    case 2:
+        if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi) == PF_IQ2_XXS) launch_decode_q4t<PF_IQ2_XXS>(a, tokens, stream, stage_limit);
+        else pf_launch_decode_iq2(a, tokens, stream, stage_limit);
+        break;
     case 3: pf_launch_decode_q2profile(a, tokens, stream, stage_limit); break;
     case 4: pf_launch_decode_q4profile(a, tokens, stream, stage_limit); break;
     default: break;   // pf_decode_supported keeps other combinations away

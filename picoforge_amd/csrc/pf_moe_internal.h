@@ -16,6 +16,7 @@ struct PfKernelArgs {
     size_t scale_offset[8];                 // IQ2_XXS: byte offset of the half scales in the tensor buffer
     int k_logical[8], blocks_per_row[8], n_out[8];
     const uint8_t *wt[8];            // Q4_K expert tensors in tile order for the grouped product (null: not kept)
+    const uint8_t *wi[8];            // IQ2_XXS expert tensors in tile order for the decode kernels (null: not kept)
     const float *router_t;           // router as [slab of 64 experts][hidden / 4][64][4] (serial-order re-routing)
     const uint64_t *iq2_grid;        // 256 x 8 magnitudes, device memory
     const uint32_t *iq2_signed;      // 2 x 4096 words: four signed magnitudes per (grid entry, sign nibble)
@@ -108,6 +109,7 @@ struct PfHipMoe {
     float *w_norm2;                  // [experts] squared norm of each router row
     float *router_t;                 // [slab of 64 experts][hidden / 4][64][4] copy of the router
     uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
+    uint8_t *w_itile[8];             // tile-ordered second copy of IQ2_XXS expert tensors for the decode path (or null)
     bool streamed;                   // the routed tensors are not resident: forwards read them from an expert pool
 };
 
@@ -156,7 +158,9 @@ void pf_launch_exact_combine(const float *d_down, const uint64_t *d_pair_to_row,
                              uint32_t *d_error, hipStream_t stream);
 // pf_moe_decode.hip
 bool pf_decode_supported(const PfHipMoeDesc &d);
-bool pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const tiled[8]);
+uint32_t pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const q4k_tiled[8], const uint8_t *const iq2_tiled[8]);
+void pf_launch_iq2_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8_t *d_dst, size_t rows, int blocks_per_row,
+                        hipStream_t stream);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);

@@ -123,6 +123,26 @@ int main(int argc, char **argv) {
             }
         }
     }
+    // the tile-ordered IQ2_XXS copies (their own size: PF_I2T_CHUNK bytes per 32 rows and 256-block)
+    if (type[1] == PF_IQ2_XXS && type[2] == PF_IQ2_XXS && type[3] == PF_IQ2_XXS && type[4] == PF_IQ2_XXS && type[5] == PF_IQ2_XXS &&
+        type[6] == PF_IQ2_XXS && H % 256 == 0 && phys == I && I % 256 == 0 && Is % 256 == 0) {
+        for (int a = 1; a <= 6; a++) {
+            const int rows = (int)n_out[a], kblocks = (int)k_storage[a] / 256;
+            PfTensorPlace copy = place[a];
+            copy.expert_bytes = pf_i2t_expert_bytes(rows, kblocks);
+            copy.bytes = copy.expert_bytes * experts[a];
+            for (size_t e : some_experts) {
+                if (experts[a] == 1 && e) continue;
+                for (int n = 0; n < rows; n++)
+                    for (int kb = 0; kb < kblocks; kb++) {
+                        const size_t chunk = pf_i2t_chunk_at(copy.expert_bytes, e, n / 32, kblocks, kb);
+                        check("tile scale", a, copy, {chunk + pf_i2t_scale_at(n & 31), 2}, 2, e, n, kb);
+                        for (int run = 0; run < 4; run++)
+                            check("tile piece", a, copy, {chunk + pf_i2t_piece_at(run, n & 31), 16}, 16, e, n, 4 * kb + run);
+                    }
+            }
+        }
+    }
     printf("%lld spans checked, %lld outside or misaligned\n", checked, bad);
     return bad ? 1 : 0;
 }
