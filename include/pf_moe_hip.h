@@ -201,20 +201,33 @@ int pf_hip_exact_combine_host(const float *down, const uint64_t *pair_to_row, co
                               const float *shared_gate, const float *shared, size_t tokens, size_t top_k,
                               size_t hidden, float *routed, float *y, uint32_t *error_word);
 
-/* A layer created with its three routed tensors absent (host_weights[1..3] all NULL; formats stored as
- * the file stores them only: Q4_K, Q2_K, F32, F16, BF16) keeps none of them in device memory.  Its
+/* A layer created with its three routed tensors absent (host_weights[1..3] all NULL) keeps none of them
+ * in device memory.  Its
  * forward is two calls with an expert pool in between, the shape of the reference's remap hook
  * (src/qwen4_moe_internal.h:49-54): the first runs the router and the routing and returns the pairs'
  * expert ids (dense [tokens, top_k]); the caller makes them resident and passes the pool's three device
- * regions, the bytes of one expert in each, the pool's slot count and the pairs' slots to the second,
- * which runs the expert products and the combine.  pf_hip_moe_forward_* refuse such a layer. */
+ * regions, the payload bytes of one expert and the offset of the scales in each (pf_hip_pool_region_plan's
+ * layout for the pool's slot count), the slot count and the pairs' slots to the second, which runs the
+ * expert products and the combine.  pf_hip_moe_forward_* refuse such a layer. */
 int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
                                    size_t tokens, uint32_t *ids, uint32_t *error_word);
 int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const void *const regions[3],
-                                     const size_t expert_bytes[3], uint32_t pool_slots, const uint32_t *slots,
+                                     const size_t expert_bytes[3], const size_t scale_offsets[3],
+                                     uint32_t pool_slots, const uint32_t *slots,
                                      float *y, size_t y_pitch_bytes, uint32_t *ids, size_t ids_pitch_bytes,
                                      float *weights, size_t weights_pitch_bytes, size_t tokens,
                                      uint32_t *error_word);
+
+/* Pool regions in the device layout: a region of `slots` experts of one matrix is laid out as a resident
+ * tensor of `slots` experts (formats stored as the file stores them slot after slot; IQ2_XXS, Q8_0 and
+ * MXFP4 as all payloads, then all scales).  pf_hip_pool_region_plan gives the region's size, the bytes
+ * of one expert in the file, the bytes of its payload in a slot and the offset of the scales (0: not split); pf_hip_pool_store copies one
+ * expert's file bytes from host memory into a slot, splitting on the device where the format needs it,
+ * and returns when the slot is readable. */
+int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, size_t *region_bytes,
+                            size_t *file_expert_bytes, size_t *payload_expert_bytes, size_t *scale_offset);
+int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, void *region, size_t slot,
+                      const void *file_bytes);
 
 /* Minimal device-memory helpers so that a host program can keep inputs resident. */
 int pf_hip_malloc(void **d_ptr, size_t bytes);

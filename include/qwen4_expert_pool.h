@@ -43,6 +43,17 @@ void qw4_pool_release(QW4ExpertPool *pool, const uint32_t *slots, size_t n);
 void *qw4_pool_region(const QW4ExpertPool *pool, int matrix, size_t *bytes);
 QW4PoolStats qw4_pool_stats(const QW4ExpertPool *pool);
 
+/* Extensions without a counterpart in the reference (its pool holds file bytes and its kernels read them).
+ * pf_pool_set_formats tells the pool the three matrices' GGUF types and shapes (rows of k_storage[m] weights,
+ * n_out[m] rows per expert; bytes[m] of qw4_pool_create must be one expert's file bytes of that shape) so that
+ * every slot holds its expert in the layout this library's kernels read: IQ2_XXS, Q8_0 and MXFP4 are split into
+ * payloads and scales on arrival, the other formats stay as the file stores them.  Needed for layers whose routed
+ * tensors are in one of those three formats (both checkpoint profiles); before the first acquire only.  0 or -1. */
+int pf_pool_set_formats(QW4ExpertPool *pool, const uint32_t gguf_type[3], const size_t k_storage[3], const size_t n_out[3]);
+uint32_t pf_pool_slots(const QW4ExpertPool *pool);
+size_t pf_pool_scale_offset(const QW4ExpertPool *pool, int matrix);   /* where matrix m's scales start in its region; 0: not split */
+uint32_t pf_pool_format(const QW4ExpertPool *pool, int matrix);      /* UINT32_MAX: slots as the file stores them */
+
 #ifdef __cplusplus
 }
 #endif

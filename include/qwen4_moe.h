@@ -118,7 +118,8 @@ void pf_moe_forget_host_weights(Qwen4Moe *moe);
  * (src/qwen4_expert_pool.h; the remap hook of src/qwen4_moe_internal.h:49-54; its caller in
  * src/qwen4_forward_gpu.m).  pf_moe_create_streamed takes the same arguments as qwen4_moe_create with
  * the gate, up and down views carrying their layouts and a NULL span: those tensors stay in the model
- * file (formats stored as the file stores them: Q4_K, Q2_K, F32, F16, BF16).  pf_moe_forward_streamed is
+ * file (where they are IQ2_XXS, Q8_0 or MXFP4 the pool must know its formats: pf_pool_set_formats, else
+ * QW4_SHAPE from the forward).  pf_moe_forward_streamed is
  * qwen4_moe_forward for such a layer: after the routing it acquires the batch's experts from `pool` as
  * layer `layer` (tokens * top_k pins: the pool needs that many slots), runs the expert products on the
  * pool's slots and releases them.  QW4_IO when the pool cannot take the batch or a read fails;

@@ -79,6 +79,9 @@ class MoeApi:
             self.pool_set_readers = bind("qw4_pool_set_readers", None, vp, u32)
             self.pool_region = bind("qw4_pool_region", vp, vp, C.c_int, P(sz))
             self.pool_stats = bind("qw4_pool_stats", abi.QW4PoolStats, vp)
+            self.pool_set_formats = bind("pf_pool_set_formats", C.c_int, vp, P(u32), P(sz), P(sz))
+            self.pool_slots = bind("pf_pool_slots", u32, vp)
+            self.pool_format = bind("pf_pool_format", u32, vp, C.c_int)
         self.layout_init = bind(packed_prefix + "layout_init", C.c_int, P(abi.GgufTensor), sz,
                                 P(abi.QW4PackedLayout), P(E))
         self.decode_row = bind(packed_prefix + "decode_row", C.c_int, P(abi.QW4PackedCpuView), sz, sz, vp, sz, P(E))

@@ -174,10 +174,6 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         const bool routed = a >= 1 && a <= 3;
         if (routed && !host_weights[1] && !host_weights[2] && !host_weights[3]) m->streamed = true;
         else if (bytes[a] < gguf_bytes[a] || !host_weights[a]) { pf_hip_moe_destroy(m); return PF_HIP_E_ARGUMENT; }
-        if (m->streamed && routed && split_header_bytes(desc->type[a])) {
-            pf_hip_moe_destroy(m);   // pool slots hold experts as the file stores them: formats stored split on the device are not streamed
-            return PF_HIP_E_UNSUPPORTED;
-        }
         m->k_logical[a] = (int)k_logical[a];
         m->n_out[a] = place.n_out;
         m->blocks_per_row[a] = place.blocks_per_row;
@@ -716,7 +712,8 @@ extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *wo
 }
 
 extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const void *const regions[3],
-                                                const size_t expert_bytes[3], uint32_t pool_slots, const uint32_t *slots,
+                                                const size_t expert_bytes[3], const size_t scale_offsets[3],
+                                                uint32_t pool_slots, const uint32_t *slots,
                                                 float *y, size_t y_pitch_bytes, uint32_t *ids, size_t ids_pitch_bytes,
                                                 float *weights, size_t weights_pitch_bytes, size_t tokens,
                                                 uint32_t *error_word) {
@@ -725,11 +722,20 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
     if (tokens == 0) return PF_HIP_OK;
     if (!y || !slots || !pool_slots || tokens > work->cap) return PF_HIP_E_ARGUMENT;
     const size_t H = moe->desc.hidden, K = moe->desc.top_k;
-    for (int j = 0; j < 3; j++)   // a slot holds one expert of each tensor as the file stores it
-        if (!regions[j] || expert_bytes[j] != moe->expert_bytes[1 + j]) return PF_HIP_E_ARGUMENT;
+    for (int j = 0; j < 3; j++) {   // a slot holds one expert of each tensor in the device layout of `pool_slots` experts
+        PfTensorPlace place;
+        const int t = 1 + j;
+        const size_t k_storage = t == 3 ? moe->desc.down_physical : moe->desc.hidden;
+        if (!regions[j] || !scale_offsets || !pf_tensor_place(moe->desc.type[t], k_storage, (size_t)moe->n_out[t], pool_slots, &place) ||
+            expert_bytes[j] != place.expert_bytes || scale_offsets[j] != place.scale_offset)
+            return PF_HIP_E_ARGUMENT;
+    }
     HIP_TRY(hipMemcpy(work->slots, slots, tokens * K * 4, hipMemcpyHostToDevice));
     PfKernelArgs a = make_args(moe, work, work->x, H, work->y, H);
-    for (int j = 0; j < 3; j++) a.w[1 + j] = static_cast<const uint8_t *>(regions[j]);
+    for (int j = 0; j < 3; j++) {
+        a.w[1 + j] = static_cast<const uint8_t *>(regions[j]);
+        a.scale_offset[1 + j] = scale_offsets[j];
+    }
     a.slots = work->slots;
     a.pool_slots = pool_slots;
     pf_launch_general(a, (int)tokens, nullptr, 0, 3);
@@ -747,11 +753,54 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
     return PF_HIP_OK;
 }
 
-// ---- stand-alone operators on host buffers ---------------------------------------
 struct DeviceBlock {   // one allocation, freed on scope exit
     uint8_t *p = nullptr;
     ~DeviceBlock() { if (p) (void)hipFree(p); }
 };
+
+// Pool slots in the device layout (the pool itself is C11 and knows no layouts).  A region holds `slots` experts of one
+// matrix exactly as a resident tensor of `slots` experts would be laid out (pf_tensor_place): formats stored as the file
+// stores them slot after slot; formats stored split as all payloads, then (256-aligned) all scales.
+extern "C" int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, size_t *region_bytes,
+                                       size_t *file_expert_bytes, size_t *payload_expert_bytes, size_t *scale_offset) {
+    PfTensorPlace place;
+    if (!region_bytes || !file_expert_bytes || !payload_expert_bytes || !scale_offset || !slots || !n_out ||
+        !pf_tensor_place(gguf_type, k_storage, n_out, slots, &place))
+        return PF_HIP_E_ARGUMENT;
+    *region_bytes = place.bytes;
+    *file_expert_bytes = place.gguf_bytes / slots;
+    *payload_expert_bytes = place.expert_bytes;
+    *scale_offset = place.scale_offset;
+    return PF_HIP_OK;
+}
+
+// One expert's slice of one matrix, as the file stores it, into slot `slot` of the matrix's region.
+extern "C" int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, void *region, size_t slot,
+                                 const void *file_bytes) {
+    PfTensorPlace place;
+    if (!region || !file_bytes || slot >= slots || !pf_tensor_place(gguf_type, k_storage, n_out, slots, &place))
+        return PF_HIP_E_ARGUMENT;
+    uint8_t *base = static_cast<uint8_t *>(region);
+    const size_t head = split_header_bytes(gguf_type), file_expert = place.gguf_bytes / slots;
+    if (!head) {
+        HIP_TRY(hipMemcpy(base + slot * place.expert_bytes, file_bytes, file_expert, hipMemcpyHostToDevice));
+        return PF_HIP_OK;
+    }
+    size_t block, size;
+    block_geometry(gguf_type, &block, &size);
+    DeviceBlock staging;
+    HIP_TRY(hipMalloc((void **)&staging.p, file_expert));
+    HIP_TRY(hipMemcpy(staging.p, file_bytes, file_expert, hipMemcpyHostToDevice));
+    const size_t blocks = (size_t)place.blocks_per_row * n_out;
+    uint8_t *payload = base + slot * place.expert_bytes, *scales = base + place.scale_offset + slot * blocks * head;
+    if (gguf_type == PF_IQ2_XXS) pf_launch_iq2_split(staging.p, payload, reinterpret_cast<uint16_t *>(scales), blocks, nullptr);
+    else pf_launch_block_split(staging.p, payload, scales, blocks, (int)size, (int)head, nullptr);
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipStreamSynchronize(nullptr));
+    return PF_HIP_OK;
+}
+
+// ---- stand-alone operators on host buffers ---------------------------------------
 
 // A [tokens, streams, hidden] cube between host memory (byte pitches) and a dense device array.
 static hipError_t copy_cube(void *dense, void *host, size_t token_pitch, size_t stream_pitch, size_t T, size_t S,

@@ -11,6 +11,7 @@
 #include "../../include/pf_moe_hip.h"
 #include <pthread.h>
 #include <stdatomic.h>
+#include <stdbool.h>
 #include <stdlib.h>
 #include <time.h>
 #include <unistd.h>
@@ -29,6 +30,10 @@ struct QW4ExpertPool {
     uint64_t *stamp, clock; /* [slot] recency */
     uint32_t *new_slot, *new_expert;   /* the misses of the acquire in progress */
     QW4PoolStats stats;
+    /* pf_pool_set_formats: slots in the device layout */
+    bool formatted, used;
+    uint32_t type[3];
+    size_t k_storage[3], n_out[3], scale_offset[3];
 };
 
 QW4ExpertPool *qw4_pool_create(int fd, const QW4ExpertLayer *layers, uint32_t n_layers, uint32_t experts,
@@ -72,6 +77,36 @@ void qw4_pool_destroy(QW4ExpertPool *p) {
         if (p->region[m]) pf_hip_free(p->region[m]);
     free(p->layers); free(p->where); free(p->holds); free(p->pins); free(p->stamp); free(p->new_slot); free(p->new_expert);
     free(p);
+}
+
+/* Extension: the matrices' formats, so that a slot holds its expert in the layout the kernels read (formats the
+ * device stores split are split on arrival).  Before the first acquire only; the regions are allocated again. */
+int pf_pool_set_formats(QW4ExpertPool *p, const uint32_t gguf_type[3], const size_t k_storage[3], const size_t n_out[3]) {
+    if (!p || p->used || !gguf_type || !k_storage || !n_out) return -1;
+    size_t region_bytes[3], file_bytes, payload_bytes, scale_offset[3];
+    for (int m = 0; m < 3; m++)
+        if (pf_hip_pool_region_plan(gguf_type[m], k_storage[m], n_out[m], p->slots, &region_bytes[m], &file_bytes,
+                                    &payload_bytes, &scale_offset[m]) != PF_HIP_OK || file_bytes != p->bytes[m])
+            return -1;
+    for (int m = 0; m < 3; m++) {
+        void *region = NULL;
+        if (pf_hip_malloc(&region, region_bytes[m]) != PF_HIP_OK) return -1;   /* earlier matrices keep their new regions: sizes only grow */
+        pf_hip_free(p->region[m]);
+        p->region[m] = region;
+        p->region_bytes[m] = region_bytes[m];
+        p->type[m] = gguf_type[m]; p->k_storage[m] = k_storage[m]; p->n_out[m] = n_out[m]; p->scale_offset[m] = scale_offset[m];
+    }
+    p->formatted = true;
+    return 0;
+}
+
+uint32_t pf_pool_slots(const QW4ExpertPool *p) { return p ? p->slots : 0; }
+size_t pf_pool_scale_offset(const QW4ExpertPool *p, int matrix) {
+    return p && p->formatted && matrix >= 0 && matrix < 3 ? p->scale_offset[matrix] : 0;
+}
+/* The format matrix m's slots are laid out for; UINT32_MAX: as the file stores it, whatever the format. */
+uint32_t pf_pool_format(const QW4ExpertPool *p, int matrix) {
+    return p && p->formatted && matrix >= 0 && matrix < 3 ? p->type[matrix] : UINT32_MAX;
 }
 
 void qw4_pool_set_readers(QW4ExpertPool *p, uint32_t readers) {
@@ -130,8 +165,12 @@ static void *reader(void *arg) {
         const int m = (int)(job % 3);
         const uint64_t from = p->layers[r->layer].offset[m] + (uint64_t)p->new_expert[miss] * p->bytes[m];
         unsigned char *to = (unsigned char *)p->region[m] + (size_t)p->new_slot[miss] * p->bytes[m];
-        if (read_exactly(p->fd, staging, p->bytes[m], from) || pf_hip_memcpy_h2d(to, staging, p->bytes[m]) != PF_HIP_OK)
-            atomic_store(&r->failed, 1);
+        int rc = read_exactly(p->fd, staging, p->bytes[m], from);
+        if (!rc && p->formatted)
+            rc = pf_hip_pool_store(p->type[m], p->k_storage[m], p->n_out[m], p->slots, p->region[m], p->new_slot[miss], staging);
+        else if (!rc)
+            rc = pf_hip_memcpy_h2d(to, staging, p->bytes[m]);
+        if (rc) atomic_store(&r->failed, 1);
     }
     free(staging);
     return NULL;
@@ -146,6 +185,7 @@ static uint64_t now_ns(void) {
 int qw4_pool_acquire(QW4ExpertPool *p, uint32_t layer, const uint32_t *experts, size_t n, uint32_t *slots) {
     if (!p || layer >= p->n_layers || (n && (!experts || !slots))) return -1;
     const uint64_t t0 = now_ns();
+    p->used = true;
     uint32_t misses = 0;
     int rc = 0;
     /* pass 1: slots and victims, in list order */

@@ -504,14 +504,20 @@ static Qwen4Status streamed_forward(const Qwen4Moe *m, Qwen4MoeWork *w, QW4Exper
                                     Qwen4F32Mut y, Qwen4MoeRoutes *routes, Qwen4Error *err) {
     const size_t T = x.dim[0], K = m->cfg.top_k, pairs = T * K;
     const void *regions[3];
-    size_t expert_bytes[3], pool_slots = 0;
+    size_t expert_bytes[3], scale_offsets[3];
+    const size_t pool_slots = pf_pool_slots(pool);
     for (int j = 0; j < 3; j++) {
-        size_t region_bytes = 0;
+        const QW4PackedLayout *l = &m->w[1 + j].layout;
+        const uint32_t format = pf_pool_format(pool, j);
+        size_t region_bytes = 0, want_bytes = 0, file_bytes = 0;
         regions[j] = qw4_pool_region(pool, j, &region_bytes);
-        expert_bytes[j] = m->w[1 + j].layout.expert_bytes;
-        if (!regions[j] || region_bytes % expert_bytes[j] || (j && region_bytes / expert_bytes[j] != pool_slots))
+        if (!regions[j] || !pool_slots ||
+            pf_hip_pool_region_plan(l->gguf_type, l->k_storage, l->n_out, pool_slots, &want_bytes, &file_bytes, &expert_bytes[j],
+                                    &scale_offsets[j]) ||
+            /* a pool that was not told its formats holds file bytes: right only where the kernels read those */
+            (format == UINT32_MAX ? scale_offsets[j] != 0 : format != l->gguf_type) || file_bytes != l->expert_bytes ||
+            region_bytes < want_bytes)
             return moe_status(err, QW4_SHAPE, "the pool's slots do not hold this layer's experts");
-        pool_slots = region_bytes / expert_bytes[j];
     }
     uint32_t *ids = malloc(pairs * 2 * sizeof *ids), *slots = ids ? ids + pairs : NULL, word = 0;
     if (!ids) return moe_status(err, QW4_OOM, "streaming staging");
@@ -523,7 +529,7 @@ static Qwen4Status streamed_forward(const Qwen4Moe *m, Qwen4MoeWork *w, QW4Exper
     else if (qw4_pool_acquire(pool, layer, ids, pairs, slots))
         st = moe_status(err, QW4_IO, "expert pool: every slot pinned, or a read of the model file failed");
     if (!st) {
-        rc = pf_hip_moe_experts_streamed_host(m->device, w->device, regions, expert_bytes, (uint32_t)pool_slots, slots, y.data,
+        rc = pf_hip_moe_experts_streamed_host(m->device, w->device, regions, expert_bytes, scale_offsets, (uint32_t)pool_slots, slots, y.data,
                                               y.stride_bytes[0], routes ? routes->ids.data : NULL,
                                               routes ? routes->ids.row_stride_bytes : 0,
                                               routes ? routes->weights.data : NULL,

@@ -128,8 +128,11 @@ def streamed_weights(weights):
     return struct
 
 
-@pytest.mark.parametrize("gtype", [abi.GGUF_Q4_K, abi.GGUF_F16])
-def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype):
+@pytest.mark.parametrize("gtype,formatted", [(abi.GGUF_Q4_K, False), (abi.GGUF_F16, False), (abi.GGUF_Q4_K, True),
+                                             (abi.GGUF_IQ2_XXS, True), ("q2", True), ("q4", True)])
+def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype, formatted):
+    """formatted: the pool is told the matrices' formats and keeps its slots in the device layout (needed where that
+    differs from the file's: IQ2_XXS, Q8_0, MXFP4 -- both checkpoint profiles, "q2" and "q4")."""
     cfg = abi.moe_config(256, 16, 4, 256, 256)
     weights, x = make_layer_inputs(cfg, gtype, 9, seed=61)
     # the model file: two layers' worth of tensors, this layer second, at page-aligned offsets
@@ -151,6 +154,14 @@ def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype):
     pool = product.pool_create(fd, table, 2, cfg.experts, (C.c_size_t * 3)(*sizes), 12)   # 12 slots for 16 experts
     assert pool
     product.pool_set_readers(pool, 3)
+    def tell_formats(which):
+        h, i = cfg.hidden_size, cfg.intermediate
+        assert product.pool_set_formats(which, (C.c_uint32 * 3)(*weights.types[1:4]), (C.c_size_t * 3)(h, h, cfg.down_physical),
+                                        (C.c_size_t * 3)(i, i, h)) == 0
+
+    if formatted:
+        tell_formats(pool)
+        assert product.pool_format(pool, 2) == weights.types[3] and product.pool_slots(pool) == 12
     err, handle = abi.Qwen4Error(), C.c_void_p()
     struct = streamed_weights(weights)
     assert product.create_streamed(C.byref(cfg), C.byref(struct), C.byref(handle), C.byref(err)) == abi.QW4_OK, err.detail
@@ -175,6 +186,8 @@ def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype):
         assert stats.bytes_read == stats.misses * sum(sizes)
         # a pool with fewer slots than one token routes to cannot make the batch resident
         tiny = product.pool_create(fd, table, 2, cfg.experts, (C.c_size_t * 3)(*sizes), cfg.top_k - 1)
+        if formatted:
+            tell_formats(tiny)
         rows = np.ascontiguousarray(x[:2])
         y = np.full((2, cfg.hidden_size), -99.0, np.float32)
         st = product.forward_streamed(layer.handle, tiny, 1, abi.f32_view(rows), abi.f32_view(y), None, layer.work,
@@ -193,11 +206,29 @@ def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype):
     os.close(fd)
 
 
-def test_streaming_refuses_what_it_cannot_hold(product):
+def test_streaming_refuses_what_it_cannot_hold(product, tmp_path):
     cfg = abi.moe_config(256, 16, 4, 256, 256)
-    weights, _ = make_layer_inputs(cfg, abi.GGUF_IQ2_XXS, 1, seed=3)   # stored split on the device
+    weights, x = make_layer_inputs(cfg, abi.GGUF_IQ2_XXS, 1, seed=3)   # stored split on the device
     err, handle = abi.Qwen4Error(), C.c_void_p()
-    struct = streamed_weights(weights)
-    assert product.create_streamed(C.byref(cfg), C.byref(struct), C.byref(handle), C.byref(err)) == abi.QW4_UNSUPPORTED
-    assert not handle
+    # routed bytes handed to a streamed layer
     assert product.create_streamed(C.byref(cfg), C.byref(weights.struct), C.byref(handle), C.byref(err)) == abi.QW4_INVALID_ARGUMENT
+    assert not handle
+    # a pool of file bytes under a layer whose kernels read another layout; a pool told another format
+    sizes = [weights.raw[j].size // cfg.experts for j in (1, 2, 3)]
+    path = tmp_path / "model.bin"
+    np.concatenate([weights.raw[j] for j in (1, 2, 3)]).tofile(path)
+    fd = os.open(path, os.O_RDONLY)
+    table = (abi.QW4ExpertLayer * 1)(abi.QW4ExpertLayer((C.c_uint64 * 3)(0, weights.raw[1].size, weights.raw[1].size + weights.raw[2].size)))
+    struct = streamed_weights(weights)
+    assert product.create_streamed(C.byref(cfg), C.byref(struct), C.byref(handle), C.byref(err)) == abi.QW4_OK
+    with pf.MoeLayer(product, cfg, weights, 1, handle=handle) as layer:
+        y = np.full((1, cfg.hidden_size), -99.0, np.float32)
+        plain = product.pool_create(fd, table, 1, cfg.experts, (C.c_size_t * 3)(*sizes), 8)
+        st = product.forward_streamed(layer.handle, plain, 0, abi.f32_view(x), abi.f32_view(y), None, layer.work, C.byref(layer.err))
+        assert st == abi.QW4_SHAPE and (y == -99.0).all()
+        h, i = cfg.hidden_size, cfg.intermediate
+        # the formats cannot change once the pool was used, and must match the slices' sizes
+        wrong = (C.c_uint32 * 3)(abi.GGUF_Q4_K, abi.GGUF_Q4_K, abi.GGUF_Q4_K)
+        assert product.pool_set_formats(plain, wrong, (C.c_size_t * 3)(h, h, i), (C.c_size_t * 3)(i, i, h)) == -1
+        product.pool_destroy(plain)
+    os.close(fd)
