@@ -293,6 +293,16 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             }
         }
     }
+    // A Q4_K layer that every kernel family can read through the tile-ordered copy alone (the decode kernels whose lanes
+    // are weight rows, the grouped product, the general kernels' tile reader) gives its row-ordered expert tensors
+    // back: one copy of the experts in device memory, not two.
+    if (pf_decode_tile_layer(m->desc, m->w_tiled, m->w_itile) == PF_Q4_K) {
+        for (int a = 1; a <= 6; a++) {
+            (void)hipFree(m->w[a]);
+            m->w[a] = nullptr;
+            m->total_bytes -= m->bytes[a];
+        }
+    }
     *out = m;
     return PF_HIP_OK;
 }

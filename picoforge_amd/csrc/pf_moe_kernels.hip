@@ -65,6 +65,42 @@ __device__ __forceinline__ float dot_row_q4k(const uint8_t *row, const float *x,
     return acc;
 }
 
+// The same product on the tile-ordered copy (pf_decode_addr.h: per 32-row tile and 256-block the 32 headers, then per
+// 64-weight run the rows' halves): row n of the expert whose tiles start at `expert`.  Layers that keep only this
+// copy of their Q4_K tensors are read through it.
+__device__ __forceinline__ float dot_row_q4k_tiled(const uint8_t *expert, int n, const float *x, int nblk, int lane) {
+    const int r = lane & 7, j = r >> 1, half = r & 1, row_in_tile = n & 31;
+    float acc = 0.0f;
+    for (int b = lane >> 3; b < nblk; b += 8) {
+        const uint8_t *chunk = expert + pf_q4t_chunk_at(0, 0, n >> 5, nblk, b);
+        const uint4 hdr = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_header_at(row_in_tile));
+        const uint4 q = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(j, half, row_in_tile));
+        const float d = pf_half_bits_to_float(hdr.x & 0xffffu);
+        const float dmin = pf_half_bits_to_float(hdr.x >> 16);
+        const uint32_t sc[3] = {hdr.y, hdr.z, hdr.w};
+        uint32_t s0, m0, s1, m1;
+        pf_q4k_scale_min(sc, 2 * j, s0, m0);
+        pf_q4k_scale_min(sc, 2 * j + 1, s1, m1);
+        const float *xl = x + 256 * b + 64 * j + 16 * half, *xh = xl + 32;
+        const uint32_t qw[4] = {q.x, q.y, q.z, q.w};
+        float ql = 0.0f, qh = 0.0f, sl = 0.0f, sh = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const uint32_t byte = (qw[w] >> (8 * c)) & 255u;
+                const float a = xl[4 * w + c], bb = xh[4 * w + c];
+                ql = fmaf((float)(byte & 15u), a, ql);
+                qh = fmaf((float)(byte >> 4), bb, qh);
+                sl += a;
+                sh += bb;
+            }
+        }
+        acc += d * ((float)s0 * ql + (float)s1 * qh) - dmin * ((float)m0 * sl + (float)m1 * sh);
+    }
+    return acc;
+}
+
 // Lane l takes group l (32 weights, one aligned 8-byte payload word) per pass.
 __device__ __forceinline__ float dot_row_iq2(const uint8_t *payload, const uint16_t *scales, const float *x, int nblk,
                                              int lane, const uint64_t *grid) {
@@ -185,7 +221,10 @@ __device__ __forceinline__ float dot_tensor_row(const PfKernelArgs &a, int t, si
     case PF_F32: v = dot_row_f32(row, x, a.k_logical[t], lane); break;
     case PF_F16: v = dot_row_16<false>(row, x, a.k_logical[t], lane); break;
     case PF_BF16: v = dot_row_16<true>(row, x, a.k_logical[t], lane); break;
-    case PF_Q4_K: v = dot_row_q4k(row, x, a.blocks_per_row[t], lane); break;
+    case PF_Q4_K:
+        v = a.w[t] ? dot_row_q4k(row, x, a.blocks_per_row[t], lane)
+                   : dot_row_q4k_tiled(a.wt[t] + e * a.expert_bytes[t], (int)n, x, a.blocks_per_row[t], lane);
+        break;
     case PF_Q2_K: v = dot_row_q2k(row, x, a.blocks_per_row[t], lane); break;
     case PF_Q8_0:
         v = dot_row_q8(row, reinterpret_cast<const uint16_t *>(scales) + first_block, x, a.blocks_per_row[t], lane);

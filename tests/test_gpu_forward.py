@@ -89,7 +89,8 @@ def test_prefill_kernels_match_oracle_and_general_kernels(product, oracle, h, e,
 
 
 def test_prefill_from_row_order_when_the_tile_ordered_copy_is_switched_off(product, oracle, monkeypatch):
-    """PF_MOE_PREFILL_COPY=0 at create: the grouped product reads the GGUF row order, same results bit for bit."""
+    """PF_MOE_PREFILL_COPY=0 at create: the grouped product reads the GGUF row order, same results bit for bit.  A Q4_K
+    layer keeps one copy of its experts either way: the tile-ordered one alone serves every kernel family."""
     cfg = abi.moe_config(512, 8, 3, 256, 512)
     weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 70, seed=590)
     want = forward_with(oracle, cfg, weights, x)
@@ -104,7 +105,7 @@ def test_prefill_from_row_order_when_the_tile_ordered_copy_is_switched_off(produ
         bytes_with = product.hip.moe_bytes(layer.device_handles()[0])
     assert_parity(y, ids, w, *want, label="prefill from the row order")
     np.testing.assert_array_equal(y, y_tiled, err_msg="the two weight orders give different results")
-    assert bytes_with > bytes_without
+    assert bytes_with == bytes_without
 
 
 def test_prefill_rows_of_very_different_magnitude(product, oracle):
