@@ -154,3 +154,12 @@ PF_HD size_t pf_i2t_chunk_at(size_t expert_bytes, size_t e, int row_tile, int kb
 }
 PF_HD size_t pf_i2t_scale_at(int row_in_tile) { return 2048 + 2 * (size_t)row_in_tile; }
 PF_HD size_t pf_i2t_piece_at(int run, int row_in_tile) { return (size_t)run * 512 + 16 * (size_t)row_in_tile; }
+
+// ---- tile-ordered Q8_0 (the shared expert of the checkpoint profiles; 32 rows x one 64-weight run = 2176 bytes: the
+// rows' 64 code bytes as four 16-byte pieces, piece by piece, then the rows' two half scales each, then padding) ----
+PF_HD size_t pf_q8t_expert_bytes(int n_out, int runs) { return (size_t)(n_out / 32) * runs * PF_I2T_CHUNK; }
+PF_HD size_t pf_q8t_chunk_at(size_t expert_bytes, size_t e, int row_tile, int runs, int run) {
+    return e * expert_bytes + ((size_t)row_tile * runs + run) * PF_I2T_CHUNK;
+}
+PF_HD size_t pf_q8t_piece_at(int piece, int row_in_tile) { return (size_t)piece * 512 + 16 * (size_t)row_in_tile; }
+PF_HD size_t pf_q8t_scales_at(int row_in_tile) { return 2048 + 4 * (size_t)row_in_tile; }

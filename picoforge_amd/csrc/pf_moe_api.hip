@@ -269,20 +269,33 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             }
         }
     }
-    {   // IQ2_XXS layers: a tile-ordered second copy of the expert tensors for the decode kernels whose lanes are weight
-        // rows (doubles the expert bytes; PF_MOE_PREFILL_COPY=0 does without it, as for Q4_K)
+    {   // Tile-ordered second copies for the decode kernels whose lanes are weight rows: the IQ2_XXS expert tensors (all
+        // six of a layer that is IQ2_XXS throughout; the routed gate and up of the q2 checkpoint profile) and the Q8_0
+        // shared gate and up of both profiles.  PF_MOE_PREFILL_COPY=0 does without them, as for Q4_K.
         const char *copy = getenv("PF_MOE_PREFILL_COPY");
-        bool all_iq2 = m->decode_ready;
-        for (int a = 1; a <= 6; a++) all_iq2 &= desc->type[a] == PF_IQ2_XXS && n_out[a] % 32 == 0;
+        bool all_iq2 = true;
+        for (int a = 1; a <= 6; a++) all_iq2 &= desc->type[a] == PF_IQ2_XXS;
         hipError_t e = hipSuccess;
-        if (all_iq2 && (!copy || strcmp(copy, "0") != 0)) {
+        if (m->decode_ready && (!copy || strcmp(copy, "0") != 0)) {
             for (int a = 1; a <= 6 && e == hipSuccess; a++) {
-                const size_t bytes = pf_i2t_expert_bytes((int)n_out[a], m->blocks_per_row[a]) * experts[a];
-                e = hipMalloc((void **)&m->w_itile[a], bytes);
-                if (e == hipSuccess) {
-                    pf_launch_iq2_tile(m->w[a], reinterpret_cast<const uint16_t *>(m->w[a] + m->scale_offset[a]), m->w_itile[a],
-                                       (size_t)n_out[a] * experts[a], m->blocks_per_row[a], nullptr);
-                    m->total_bytes += bytes;
+                const bool gate_or_up = a == 1 || a == 2 || a == 4 || a == 5;
+                if (n_out[a] % 32) continue;
+                if (desc->type[a] == PF_IQ2_XXS && (all_iq2 || a == 1 || a == 2)) {
+                    const size_t bytes = pf_i2t_expert_bytes((int)n_out[a], m->blocks_per_row[a]) * experts[a];
+                    e = hipMalloc((void **)&m->w_itile[a], bytes);
+                    if (e == hipSuccess) {
+                        pf_launch_iq2_tile(m->w[a], reinterpret_cast<const uint16_t *>(m->w[a] + m->scale_offset[a]), m->w_itile[a],
+                                           (size_t)n_out[a] * experts[a], m->blocks_per_row[a], nullptr);
+                        m->total_bytes += bytes;
+                    }
+                } else if (desc->type[a] == PF_Q8_0 && gate_or_up && experts[a] == 1 && k_storage[a] % 64 == 0) {
+                    const size_t bytes = pf_q8t_expert_bytes((int)n_out[a], (int)(k_storage[a] / 64));
+                    e = hipMalloc((void **)&m->w_qtile[a], bytes);
+                    if (e == hipSuccess) {
+                        pf_launch_q8_tile(m->w[a], reinterpret_cast<const uint16_t *>(m->w[a] + m->scale_offset[a]), m->w_qtile[a],
+                                          n_out[a], m->blocks_per_row[a], nullptr);
+                        m->total_bytes += bytes;
+                    }
                 }
             }
             if (e == hipSuccess) e = hipDeviceSynchronize();
@@ -314,6 +327,7 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
     if (m->router_t) (void)hipFree(m->router_t);
     for (int a = 0; a < 8; a++) if (m->w_tiled[a]) (void)hipFree(m->w_tiled[a]);
     for (int a = 0; a < 8; a++) if (m->w_itile[a]) (void)hipFree(m->w_itile[a]);
+    for (int a = 0; a < 8; a++) if (m->w_qtile[a]) (void)hipFree(m->w_qtile[a]);
     free(m);
 }
 
@@ -500,7 +514,7 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.group_bad = w->group_bad; a.tiles = w->tiles;
     a.token_cap = (uint32_t)w->cap;
     a.router_t = m->router_t;
-    for (int j = 0; j < 8; j++) { a.wt[j] = m->w_tiled[j]; a.wi[j] = m->w_itile[j]; }
+    for (int j = 0; j < 8; j++) { a.wt[j] = m->w_tiled[j]; a.wi[j] = m->w_itile[j]; a.wq[j] = m->w_qtile[j]; }
     return a;
 }
 

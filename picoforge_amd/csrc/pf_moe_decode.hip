@@ -134,16 +134,33 @@ __device__ __forceinline__ bool build_image(int *img, const float *src, int K, i
     return bad;
 }
 
-// ---- two-digit images in global memory (kernels whose lanes are weight rows) --------------------
+// ---- digit images in global memory (kernels whose lanes are weight rows) ------------------------
 // Where every lane of a wave is a weight row, the activation digits are the same for the whole wave and
 // travel through scalar registers: the image lives in global memory (pf_image2_words), written by the
-// kernel before.  Two balanced base-256 digits (signed bytes): the values as 16-bit integers relative
-// to a step per 32-group that puts the group's largest magnitude at 127 * 256; the rounding error is at
-// most 2^-16 of that magnitude.
+// kernel before.  PF_IMG_PLANES balanced base-256 digits (signed bytes): the values as integers relative
+// to a step per 32-group that puts the group's largest magnitude at 127 * 256^(planes - 1); the rounding
+// error is at most 2^-24 of that magnitude with three planes.
+#define PF_IMG_TOP (PF_IMG_PLANES == 3 ? 8323072.0f : 32512.0f)   // the integer the group's largest magnitude becomes: 127 * 256^(planes - 1)
 __device__ __forceinline__ void group_step2(float m, float &step, float &inv) {
     const bool none = !(m > 1e-30f);   // an all-zero (or vanishing) group
-    inv = none ? 0.0f : 32512.0f / m;
-    step = none ? 0.0f : m * (1.0f / 32512.0f);
+    inv = none ? 0.0f : PF_IMG_TOP / m;
+    step = none ? 0.0f : m * (1.0f / PF_IMG_TOP);
+}
+// balanced base-256 digits of q, lowest first (each in -128..127)
+__device__ __forceinline__ void image_digits(int q, int (&d)[PF_IMG_PLANES]) {
+#pragma unroll
+    for (int p = 0; p + 1 < PF_IMG_PLANES; p++) {
+        d[p] = ((q + 128) & 255) - 128;
+        q = (q - d[p]) >> 8;
+    }
+    d[PF_IMG_PLANES - 1] = q;
+}
+// the integer dot product from its per-plane parts (float: three planes leave 32 bits)
+__device__ __forceinline__ float image_value(const int (&part)[PF_IMG_PLANES]) {
+    float v = (float)part[PF_IMG_PLANES - 1];
+#pragma unroll
+    for (int p = PF_IMG_PLANES - 2; p >= 0; p--) v = fmaf(256.0f, v, (float)part[p]);
+    return v;
 }
 
 // Thread j of a group of four neighbouring lanes: the eight values 8j..8j+7 of a K-vector into its image.
@@ -157,24 +174,25 @@ __device__ __forceinline__ bool image2_chunk(uint32_t *img, const float4 a, cons
     m = fmaxf(m, __int_as_float(dpp_quad_xor2(__float_as_int(m))));
     float step, inv;
     group_step2(m, step, inv);
-    uint32_t w0[2] = {0, 0}, w1[2] = {0, 0};
+    uint32_t w[PF_IMG_PLANES][2] = {};
     int sum = 0;
 #pragma unroll
     for (int c = 0; c < 8; c++) {
         const int q = __float2int_rn(v[c] * inv);
         sum += q;
-        const int d0 = ((q + 128) & 255) - 128, d1 = (q - d0) >> 8;
-        w0[c >> 2] |= (uint32_t)(d0 & 255) << (8 * (c & 3));
-        w1[c >> 2] |= (uint32_t)(d1 & 255) << (8 * (c & 3));
+        int d[PF_IMG_PLANES];
+        image_digits(q, d);
+#pragma unroll
+        for (int p = 0; p < PF_IMG_PLANES; p++) w[p][c >> 2] |= (uint32_t)(d[p] & 255) << (8 * (c & 3));
     }
     sum += dpp_quad_xor1(sum);
     sum += dpp_quad_xor2(sum);
-    const int g = j >> 2, at = 16 * g + 2 * (j & 3);
-    img[at] = w0[0]; img[at + 1] = w0[1];
-    img[at + 8] = w1[0]; img[at + 9] = w1[1];
+    const int g = j >> 2, at = PF_IMG_GROUP * g + 2 * (j & 3);
+#pragma unroll
+    for (int p = 0; p < PF_IMG_PLANES; p++) { img[at + 8 * p] = w[p][0]; img[at + 8 * p + 1] = w[p][1]; }
     if ((j & 3) == 0) {
-        img[16 * (K / 32) + g] = __float_as_uint(step);
-        img[17 * (K / 32) + g] = (uint32_t)sum;
+        img[PF_IMG_GROUP * (K / 32) + g] = __float_as_uint(step);
+        img[(PF_IMG_GROUP + 1) * (K / 32) + g] = (uint32_t)sum;
     }
     return bad;
 }
@@ -201,15 +219,16 @@ __device__ __forceinline__ void image2_group(uint32_t *img, float v, int g, int 
 #pragma unroll
     for (int k = 0; k < 4; k++) sum += dpp_row_step(sum, k);
     sum += __shfl_xor(sum, 16);
-    const int d0 = ((q + 128) & 255) - 128, d1 = (q - d0) >> 8;
-    uint8_t *bytes = reinterpret_cast<uint8_t *>(img + 16 * g);
+    int d[PF_IMG_PLANES];
+    image_digits(q, d);
+    uint8_t *bytes = reinterpret_cast<uint8_t *>(img + PF_IMG_GROUP * g);
     if (lane < 32) {
-        bytes[lane] = (uint8_t)d0;
-        bytes[32 + lane] = (uint8_t)d1;
+#pragma unroll
+        for (int p = 0; p < PF_IMG_PLANES; p++) bytes[32 * p + lane] = (uint8_t)d[p];
     }
     if (lane == 0) {
-        img[16 * (K / 32) + g] = __float_as_uint(step);
-        img[17 * (K / 32) + g] = (uint32_t)sum;
+        img[PF_IMG_GROUP * (K / 32) + g] = __float_as_uint(step);
+        img[(PF_IMG_GROUP + 1) * (K / 32) + g] = (uint32_t)sum;
     }
 }
 
@@ -477,7 +496,7 @@ template <int NT>
 __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks, int tokens) {
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     if ((int)blockIdx.x > router_blocks) {
-        // workgroups beyond the router's (launched where the next kernel reads them): the tokens' two-digit images,
+        // workgroups beyond the router's (launched where the next kernel reads them): the tokens' digit images,
         // 2048 values per workgroup
         const int per_token = (H + 2047) / 2048, q = (int)blockIdx.x - router_blocks - 1;
         const int t = q / per_token, j = (q % per_token) * 256 + (int)threadIdx.x;
@@ -834,7 +853,7 @@ __global__ void __launch_bounds__(1024) pf_k_dec_gate_up(PfKernelArgs a, int rou
 // 32 consecutive rows into 512 consecutive bytes, so here a lane is a weight row: lanes 0..31 the
 // tile's gate rows, 32..63 its up rows, and a wave takes half a 256-block (four 32-groups) of all of
 // them.  Every lane of the wave then meets the same activations: their digits come from the token's
-// two-digit image in global memory through scalar loads and enter the dot products as scalar
+// digit image in global memory through scalar loads and enter the dot products as scalar
 // operands -- no LDS image, no reduction across lanes.  The waves' partial sums meet in LDS and are
 // added in a fixed order.  Routing as in pf_k_dec_gate_up1.
 typedef const __attribute__((address_space(4))) uint32_t *PfScalarWords;   // read through the scalar cache
@@ -842,8 +861,13 @@ typedef const __attribute__((address_space(4))) uint32_t *PfScalarWords;   // re
 template <int FMT> struct TileItem;
 template <> struct TileItem<PF_Q4_K> { uint4 hdr, piece[2]; };   // a row's header and the two halves of one 64-weight run
 template <> struct TileItem<PF_IQ2_XXS> { uint4 piece; uint32_t dbits; };   // two 32-groups (indices, sign/scale word) and the block's half scale
+template <> struct TileItem<PF_Q8_0> { uint4 q[4]; uint32_t d2; };   // two blocks: 64 code bytes and their two half scales
 typedef TileItem<PF_Q4_K> Q4TileItem;
 
+template <int FMT> struct TileGeometryHost { static const uint8_t *tensor(const PfKernelArgs &, int) { return nullptr; } };
+template <> struct TileGeometryHost<PF_Q4_K> { static const uint8_t *tensor(const PfKernelArgs &a, int t) { return a.wt[t]; } };
+template <> struct TileGeometryHost<PF_IQ2_XXS> { static const uint8_t *tensor(const PfKernelArgs &a, int t) { return a.wi[t]; } };
+template <> struct TileGeometryHost<PF_Q8_0> { static const uint8_t *tensor(const PfKernelArgs &a, int t) { return a.wq[t]; } };
 template <int FMT> struct TileGeometry;
 template <> struct TileGeometry<PF_Q4_K> {
     static __device__ __forceinline__ size_t expert_bytes(const PfKernelArgs &a, int t) { return a.expert_bytes[t]; }
@@ -856,6 +880,18 @@ template <> struct TileGeometry<PF_IQ2_XXS> {
     static __device__ __forceinline__ const uint8_t *tensor(const PfKernelArgs &a, int t) { return a.wi[t]; }
 };
 
+template <> struct TileGeometry<PF_Q8_0> {   // one chunk per 64-weight run: a 256-block is four of them
+    static __device__ __forceinline__ size_t expert_bytes(const PfKernelArgs &a, int t) { return pf_q8t_expert_bytes(a.n_out[t], a.blocks_per_row[t] / 2); }
+    static __device__ __forceinline__ size_t chunk_at(int row_tile, int kblocks, int kb) { return pf_q8t_chunk_at(0, 0, row_tile, 4 * kblocks, 4 * kb); }
+    static __device__ __forceinline__ const uint8_t *tensor(const PfKernelArgs &a, int t) { return a.wq[t]; }
+};
+
+__device__ __forceinline__ void q4t_load(TileItem<PF_Q8_0> &w, const uint8_t *chunk, int row, int run) {
+    const uint8_t *mine = chunk + (size_t)run * PF_I2T_CHUNK;
+#pragma unroll
+    for (int p = 0; p < 4; p++) w.q[p] = *reinterpret_cast<const uint4 *>(mine + pf_q8t_piece_at(p, row));
+    w.d2 = *reinterpret_cast<const uint32_t *>(mine + pf_q8t_scales_at(row));
+}
 __device__ __forceinline__ void q4t_load(TileItem<PF_Q4_K> &w, const uint8_t *chunk, int row, int run) {
     w.hdr = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_header_at(row));
     w.piece[0] = *reinterpret_cast<const uint4 *>(chunk + pf_q4t_piece_at(run, 0, row));
@@ -881,23 +917,24 @@ __device__ __forceinline__ float q4t_dot(const Q4TileItem &w, PfScalarWords digi
         mn2 = (((w.hdr.w >> sh) >> 4) & 0x0F0Fu) | (((w.hdr.z >> sh) >> 2) & 0x3030u);
     }
     const float d = half_bits(w.hdr.x & 0xffffu), dmin = half_bits(w.hdr.x >> 16);
-    int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
-    PfScalarWords even = digits, odd = digits + 16;
+    int lo_part[PF_IMG_PLANES] = {}, hi_part[PF_IMG_PLANES] = {};
+    PfScalarWords even = digits, odd = digits + PF_IMG_GROUP;
 #pragma unroll
     for (int h = 0; h < 2; h++) {
         const uint32_t q[4] = {w.piece[h].x, w.piece[h].y, w.piece[h].z, w.piece[h].w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
-            lo0 = __builtin_amdgcn_sdot4(lo, (int)even[4 * h + i], lo0, false);
-            lo1 = __builtin_amdgcn_sdot4(lo, (int)even[8 + 4 * h + i], lo1, false);
-            hi0 = __builtin_amdgcn_sdot4(hi, (int)odd[4 * h + i], hi0, false);
-            hi1 = __builtin_amdgcn_sdot4(hi, (int)odd[8 + 4 * h + i], hi1, false);
+#pragma unroll
+            for (int p = 0; p < PF_IMG_PLANES; p++) {
+                lo_part[p] = __builtin_amdgcn_sdot4(lo, (int)even[8 * p + 4 * h + i], lo_part[p], false);
+                hi_part[p] = __builtin_amdgcn_sdot4(hi, (int)odd[8 * p + 4 * h + i], hi_part[p], false);
+            }
         }
     }
     const float s0 = (float)(sc2 & 255u), m0 = (float)(mn2 & 255u), s1 = (float)(sc2 >> 8), m1 = (float)(mn2 >> 8);
-    const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sums[0]);
-    const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sums[1]);
+    const float t0 = fmaf(d * s0, image_value(lo_part), -(dmin * m0) * (float)(int)sums[0]);
+    const float t1 = fmaf(d * s1, image_value(hi_part), -(dmin * m1) * (float)(int)sums[1]);
     return fmaf(__uint_as_float(steps[0]), t0, __uint_as_float(steps[1]) * t1);
 }
 
@@ -910,22 +947,45 @@ __device__ __forceinline__ float q4t_dot(const TileItem<PF_IQ2_XXS> &w, PfScalar
 #pragma unroll
     for (int gg = 0; gg < 2; gg++) {
         const uint32_t idx = gg ? w.piece.z : w.piece.x, word = gg ? w.piece.w : w.piece.y;
-        PfScalarWords dg = digits + 16 * gg;
-        int lo = 0, hi = 0;
+        PfScalarWords dg = digits + PF_IMG_GROUP * gg;
+        int part[PF_IMG_PLANES] = {};
 #pragma unroll
         for (int slot = 0; slot < 4; slot++) {
             const uint32_t g = (idx >> (8 * slot)) & 255u, s7 = (word >> (7 * slot)) & 127u;
             const uint32_t par = __popc(s7) & 1u;
             const int ml = (int)tables[(g << 4) | (s7 & 15u)];
             const int mh = (int)tables[4096u + ((g << 4) | (s7 >> 4) | (par << 3))];
-            lo = __builtin_amdgcn_sdot4(ml, (int)dg[2 * slot], lo, false);
-            hi = __builtin_amdgcn_sdot4(ml, (int)dg[8 + 2 * slot], hi, false);
-            lo = __builtin_amdgcn_sdot4(mh, (int)dg[2 * slot + 1], lo, false);
-            hi = __builtin_amdgcn_sdot4(mh, (int)dg[8 + 2 * slot + 1], hi, false);
+#pragma unroll
+            for (int p = 0; p < PF_IMG_PLANES; p++) {
+                part[p] = __builtin_amdgcn_sdot4(ml, (int)dg[8 * p + 2 * slot], part[p], false);
+                part[p] = __builtin_amdgcn_sdot4(mh, (int)dg[8 * p + 2 * slot + 1], part[p], false);
+            }
         }
-        acc[gg] = __uint_as_float(steps[gg]) * (float)(2u * (word >> 28) + 1u) * (float)(lo + (hi << 8));
+        acc[gg] = __uint_as_float(steps[gg]) * (float)(2u * (word >> 28) + 1u) * image_value(part);
     }
     return half_bits(w.dbits) * 0.125f * (acc[0] + acc[1]);
+}
+
+// Q8_0: the run's two blocks of 32 signed codes against the digit planes
+__device__ __forceinline__ float q4t_dot(const TileItem<PF_Q8_0> &w, PfScalarWords digits, PfScalarWords steps, PfScalarWords sums, int,
+                                         const uint32_t *) {
+    (void)sums;
+    float acc[2];
+#pragma unroll
+    for (int gg = 0; gg < 2; gg++) {
+        const uint32_t q[8] = {w.q[2 * gg].x, w.q[2 * gg].y, w.q[2 * gg].z, w.q[2 * gg].w,
+                               w.q[2 * gg + 1].x, w.q[2 * gg + 1].y, w.q[2 * gg + 1].z, w.q[2 * gg + 1].w};
+        PfScalarWords dg = digits + PF_IMG_GROUP * gg;
+        int part[PF_IMG_PLANES] = {};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+#pragma unroll
+            for (int p = 0; p < PF_IMG_PLANES; p++) part[p] = __builtin_amdgcn_sdot4((int)q[i], (int)dg[8 * p + i], part[p], false);
+        }
+        const float d = half_bits(gg ? w.d2 >> 16 : w.d2 & 0xffffu);
+        acc[gg] = __uint_as_float(steps[gg]) * d * image_value(part);
+    }
+    return acc[0] + acc[1];
 }
 
 // The tile's rows against the token: the 64-weight runs of all the rows go round the waves 1..15 (wave 0
@@ -976,7 +1036,8 @@ __device__ __forceinline__ void q4t_tile(const PfKernelArgs &a, const Q4TilePlan
         const int it = wave - 1 + 15 * k;
         if (it < p.items) {
             const int g = 2 * it;   // the run's first group within the row
-            total += q4t_dot(w[k], image + 16 * g, image + 16 * p.groups + g, image + 17 * p.groups + g, it & 3, tables);
+            total += q4t_dot(w[k], image + PF_IMG_GROUP * g, image + PF_IMG_GROUP * p.groups + g, image + (PF_IMG_GROUP + 1) * p.groups + g,
+                             it & 3, tables);
         }
     }
     partial[(wave - 1) * 64 + lane] = total;
@@ -998,7 +1059,8 @@ __device__ __forceinline__ void q4t_at_token(PfKernelArgs &a, int t) {
     a.aimg += (size_t)t * (a.top_k + 1) * pf_image2_words(widest);
 }
 
-template <int NPL, int FMT>
+// FMT: format of the routed gate and up tensors, FMTS: of the shared expert's (the same, or the profiles' Q8_0)
+template <int NPL, int FMT, int FMTS>
 __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
@@ -1047,12 +1109,13 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
         const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)my_key, u);
         if (lane == 0) early_expert = mine ? pf_key_id(mine) : 0xffffffffu;
     }
-    const Q4TilePlan plan = q4t_plan<FMT>(a, shared, n0);
+    const Q4TilePlan plan = shared ? q4t_plan<FMTS>(a, true, n0) : q4t_plan<FMT>(a, false, n0);
     const int I = shared ? a.shared_inter : a.inter;
     if (!shared || FMT == PF_IQ2_XXS) __syncthreads();   // the early expert; the tables
     const uint32_t early = shared ? 0u : early_expert;
     const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
-    q4t_tile<FMT>(a, plan, partial, tables, early_ok ? early : 0u, wave);
+    if (shared) q4t_tile<FMTS>(a, plan, partial, tables, 0u, wave);
+    else q4t_tile<FMT>(a, plan, partial, tables, early_ok ? early : 0u, wave);
     if (wave == 0 && !shared) {
         // the remaining slots, the candidate beyond them and one more key, while the other waves' weight bytes travel
         for (int r = u + 1; r <= rounds; r++) {
@@ -1115,7 +1178,7 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
         for (int w = 0; w < 15; w++) sum += partial[w * 64 + lane];
         const float g = sum, up = __shfl(sum, (lane & 31) + 32);
         const float act = pf_silu(g) * up;
-        // the 32 units are one 32-group of the activation row: its two-digit image for the down kernel
+        // the 32 units are one 32-group of the activation row: its digit image for the down kernel
         // (vector u of the activation images; the shared expert's follows the top_k routed ones)
         const size_t widest = a.inter > a.shared_inter ? a.inter : a.shared_inter;
         if (lane < 32) {
@@ -1128,8 +1191,34 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
 
 // With several tokens there are more workgroups than compute units; two workgroups per compute unit (64 registers a
 // lane) measured slower than one after the other: the products are bound by the vector units, not by waiting.
-template <int NPL, int FMT>
-__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) { q4t_gate_up<NPL, FMT>(a, routed_blocks); }
+template <int NPL, int FMT, int FMTS>
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) { q4t_gate_up<NPL, FMT, FMTS>(a, routed_blocks); }
+
+// Kernel 2 alone on the tile order (one token; the down kernel stays the segment one): layers whose routed gate and up
+// tensors are Q4_K or IQ2_XXS with the copy kept and whose shared expert is in the same format or, as in the checkpoint
+// profiles, Q8_0 with its copy kept.
+template <int FMT, int FMTS>
+static bool q4t_gate_up_applies(const PfKernelArgs &a) {
+    if (!((FMT == PF_Q4_K || FMT == PF_IQ2_XXS) && (FMTS == FMT || FMTS == PF_Q8_0))) return false;
+    for (int t : {1, 2}) if (!TileGeometryHost<FMT>::tensor(a, t)) return false;
+    for (int t : {4, 5}) if (!TileGeometryHost<FMTS>::tensor(a, t)) return false;
+    return a.hidden % 256 == 0 && 4 * (a.hidden / 256) <= 15 * Q4T_ITEMS && a.inter % 32 == 0 && a.shared_inter % 32 == 0 &&
+           a.top_k < a.experts && a.top_k <= 15 && a.experts <= 1024;
+}
+
+template <int FMT, int FMTS>
+static void launch_gate_up_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream) {
+    const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
+    const int routed_blocks = K * (I / 32);
+    const dim3 g1(routed_blocks + Is / 32, tokens);
+    const int all = (E + 63) / 64;
+    const size_t lds = (size_t)table_words<FMT>() * 4 + (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+    if (all <= 1) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<1, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 2) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<2, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 4) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<4, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else if (all <= 8) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<8, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    else hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<16, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
+}
 
 // ---- kernel 3: down products and the combine ---------------------------------------------------
 // blockIdx.x = t * row_blocks + nb; one wave per slot plus one for the shared expert; a routed
@@ -1251,17 +1340,21 @@ __global__ void __launch_bounds__(MAXT) pf_k_dec_down(PfKernelArgs a, int row_bl
 // Eight output rows per workgroup, one wave per slot and one for the shared expert, as above; a lane is
 // (row, 64-weight run): lanes 0..7 the rows' run 0, 8..15 run 1 and so on (further runs in turn), so the
 // eight rows' pieces of a run are one 128-byte line of the tile-ordered copy.  The activation digits come
-// from the two-digit images kernel 2 left in global memory (nothing is built here); the lanes of a row add
+// from the digit images kernel 2 left in global memory (nothing is built here); the lanes of a row add
 // up across the wave, the slots meet in LDS and are combined in slot order.
 // One run of one row (its item loaded by q4t_load) against the slot's digits in LDS (mine: the slot's image).  Q4_K: header
 // and two halves; IQ2_XXS: one 16-byte piece and the block's half scale, magnitudes from the tables.
 __device__ __forceinline__ float down_dot(const TileItem<PF_Q4_K> &w, int rr, const uint32_t *mine, int run, int groups, const uint32_t *) {
     const uint4 hdr = w.hdr, p0 = w.piece[0], p1 = w.piece[1];
-    uint4 dg[8];
+    // the run's two groups: PF_IMG_GROUP dwords each, plane by plane
+    uint32_t dg[2 * PF_IMG_GROUP];
 #pragma unroll
-    for (int i = 0; i < 8; i++) dg[i] = reinterpret_cast<const uint4 *>(mine + 32 * run)[i];
-    const uint2 st = *reinterpret_cast<const uint2 *>(mine + 16 * groups + 2 * run);
-    const uint2 sm = *reinterpret_cast<const uint2 *>(mine + 17 * groups + 2 * run);
+    for (int i = 0; i < 2 * PF_IMG_GROUP / 4; i++) {
+        const uint4 v = reinterpret_cast<const uint4 *>(mine + 2 * PF_IMG_GROUP * run)[i];
+        dg[4 * i] = v.x; dg[4 * i + 1] = v.y; dg[4 * i + 2] = v.z; dg[4 * i + 3] = v.w;
+    }
+    const uint2 st = *reinterpret_cast<const uint2 *>(mine + PF_IMG_GROUP * groups + 2 * run);
+    const uint2 sm = *reinterpret_cast<const uint2 *>(mine + (PF_IMG_GROUP + 1) * groups + 2 * run);
     uint32_t sc2, mn2;
     if (rr < 2) {
         sc2 = (hdr.y >> (16 * rr)) & 0x3F3Fu;
@@ -1272,24 +1365,20 @@ __device__ __forceinline__ float down_dot(const TileItem<PF_Q4_K> &w, int rr, co
         mn2 = (((hdr.w >> sh) >> 4) & 0x0F0Fu) | (((hdr.z >> sh) >> 2) & 0x3030u);
     }
     const float d = half_bits(hdr.x & 0xffffu), dmin = half_bits(hdr.x >> 16);
-    // dg[0..1]: low digits of the even group, dg[2..3] its high digits, dg[4..7] the odd group's
-    const uint32_t e0[8] = {dg[0].x, dg[0].y, dg[0].z, dg[0].w, dg[1].x, dg[1].y, dg[1].z, dg[1].w};
-    const uint32_t e1[8] = {dg[2].x, dg[2].y, dg[2].z, dg[2].w, dg[3].x, dg[3].y, dg[3].z, dg[3].w};
-    const uint32_t o0[8] = {dg[4].x, dg[4].y, dg[4].z, dg[4].w, dg[5].x, dg[5].y, dg[5].z, dg[5].w};
-    const uint32_t o1[8] = {dg[6].x, dg[6].y, dg[6].z, dg[6].w, dg[7].x, dg[7].y, dg[7].z, dg[7].w};
     const uint32_t q[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-    int lo0 = 0, lo1 = 0, hi0 = 0, hi1 = 0;
+    int lo_part[PF_IMG_PLANES] = {}, hi_part[PF_IMG_PLANES] = {};
 #pragma unroll
     for (int i = 0; i < 8; i++) {
         const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
-        lo0 = __builtin_amdgcn_sdot4(lo, (int)e0[i], lo0, false);
-        lo1 = __builtin_amdgcn_sdot4(lo, (int)e1[i], lo1, false);
-        hi0 = __builtin_amdgcn_sdot4(hi, (int)o0[i], hi0, false);
-        hi1 = __builtin_amdgcn_sdot4(hi, (int)o1[i], hi1, false);
+#pragma unroll
+        for (int p = 0; p < PF_IMG_PLANES; p++) {
+            lo_part[p] = __builtin_amdgcn_sdot4(lo, (int)dg[8 * p + i], lo_part[p], false);
+            hi_part[p] = __builtin_amdgcn_sdot4(hi, (int)dg[PF_IMG_GROUP + 8 * p + i], hi_part[p], false);
+        }
     }
     const float s0 = (float)(sc2 & 255u), m0 = (float)(mn2 & 255u), s1 = (float)(sc2 >> 8), m1 = (float)(mn2 >> 8);
-    const float t0 = fmaf(d * s0, (float)(lo0 + (lo1 << 8)), -(dmin * m0) * (float)(int)sm.x);
-    const float t1 = fmaf(d * s1, (float)(hi0 + (hi1 << 8)), -(dmin * m1) * (float)(int)sm.y);
+    const float t0 = fmaf(d * s0, image_value(lo_part), -(dmin * m0) * (float)(int)sm.x);
+    const float t1 = fmaf(d * s1, image_value(hi_part), -(dmin * m1) * (float)(int)sm.y);
     return fmaf(__uint_as_float(st.x), t0, __uint_as_float(st.y) * t1);
 }
 
@@ -1299,19 +1388,18 @@ __device__ __forceinline__ float down_dot(const TileItem<PF_IQ2_XXS> &w, int, co
                                           const uint32_t *tables) {
     const uint4 piece = w.piece;
     const uint32_t dbits = w.dbits;
-    uint4 dg[8];
+    uint32_t d32[2 * PF_IMG_GROUP];
 #pragma unroll
-    for (int i = 0; i < 8; i++) dg[i] = reinterpret_cast<const uint4 *>(mine + 32 * run)[i];
-    const uint2 st = *reinterpret_cast<const uint2 *>(mine + 16 * groups + 2 * run);
-    const uint32_t d32[32] = {dg[0].x, dg[0].y, dg[0].z, dg[0].w, dg[1].x, dg[1].y, dg[1].z, dg[1].w,
-                              dg[2].x, dg[2].y, dg[2].z, dg[2].w, dg[3].x, dg[3].y, dg[3].z, dg[3].w,
-                              dg[4].x, dg[4].y, dg[4].z, dg[4].w, dg[5].x, dg[5].y, dg[5].z, dg[5].w,
-                              dg[6].x, dg[6].y, dg[6].z, dg[6].w, dg[7].x, dg[7].y, dg[7].z, dg[7].w};
+    for (int i = 0; i < 2 * PF_IMG_GROUP / 4; i++) {
+        const uint4 v = reinterpret_cast<const uint4 *>(mine + 2 * PF_IMG_GROUP * run)[i];
+        d32[4 * i] = v.x; d32[4 * i + 1] = v.y; d32[4 * i + 2] = v.z; d32[4 * i + 3] = v.w;
+    }
+    const uint2 st = *reinterpret_cast<const uint2 *>(mine + PF_IMG_GROUP * groups + 2 * run);
     float acc[2];
 #pragma unroll
     for (int gg = 0; gg < 2; gg++) {
         const uint32_t idx = gg ? piece.z : piece.x, word = gg ? piece.w : piece.y;
-        int lo = 0, hi = 0;
+        int part[PF_IMG_PLANES] = {};
 #pragma unroll
         for (int slot = 0; slot < 4; slot++) {
             const uint32_t g = (idx >> (8 * slot)) & 255u, s7 = (word >> (7 * slot)) & 127u;
@@ -1321,12 +1409,13 @@ __device__ __forceinline__ float down_dot(const TileItem<PF_IQ2_XXS> &w, int, co
             const uint2 mag = reinterpret_cast<const uint2 *>(tables)[g];
             const uint32_t tl = ((s8 & 15u) * 0x00204081u) & 0x01010101u, th = ((s8 >> 4) * 0x00204081u) & 0x01010101u;
             const int ml = (int)((mag.x ^ (tl * 0xFFu)) + tl), mh = (int)((mag.y ^ (th * 0xFFu)) + th);
-            lo = __builtin_amdgcn_sdot4(ml, (int)d32[16 * gg + 2 * slot], lo, false);
-            hi = __builtin_amdgcn_sdot4(ml, (int)d32[16 * gg + 8 + 2 * slot], hi, false);
-            lo = __builtin_amdgcn_sdot4(mh, (int)d32[16 * gg + 2 * slot + 1], lo, false);
-            hi = __builtin_amdgcn_sdot4(mh, (int)d32[16 * gg + 8 + 2 * slot + 1], hi, false);
+#pragma unroll
+            for (int p = 0; p < PF_IMG_PLANES; p++) {
+                part[p] = __builtin_amdgcn_sdot4(ml, (int)d32[PF_IMG_GROUP * gg + 8 * p + 2 * slot], part[p], false);
+                part[p] = __builtin_amdgcn_sdot4(mh, (int)d32[PF_IMG_GROUP * gg + 8 * p + 2 * slot + 1], part[p], false);
+            }
         }
-        acc[gg] = __uint_as_float(gg ? st.y : st.x) * (float)(2u * (word >> 28) + 1u) * (float)(lo + (hi << 8));
+        acc[gg] = __uint_as_float(gg ? st.y : st.x) * (float)(2u * (word >> 28) + 1u) * image_value(part);
     }
     return half_bits(dbits) * 0.125f * (acc[0] + acc[1]);
 }
@@ -1431,6 +1520,35 @@ void pf_launch_iq2_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint
                         hipStream_t stream) {
     const size_t threads = rows / 32 * (size_t)blocks_per_row * 160;
     hipLaunchKernelGGL(pf_k_iq2_tile, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, d_payload, d_scales, d_dst, rows,
+                       blocks_per_row);
+}
+
+// ---- Q8_0 in tile order (the profiles' shared gate and up) ------------------------------------------------
+// From the split device layout (32 code bytes per block row by row, half scales apart) to the chunks of
+// pf_decode_addr.h per (32-row tile, 64-weight run).  One thread per 16-byte piece or per pair of scales.
+__global__ void pf_k_q8_tile(const uint8_t *payload, const uint16_t *scales, uint8_t *dst, size_t rows, int blocks_per_row) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x, per_chunk = 128 + 32;
+    const int runs = blocks_per_row / 2;
+    const size_t chunk = i / per_chunk, tile = chunk / runs, run = chunk % runs;
+    if (chunk >= rows / 32 * (size_t)runs) return;
+    const int p = (int)(i % per_chunk);
+    uint8_t *out = dst + chunk * PF_I2T_CHUNK;
+    if (p < 128) {
+        const int piece = p >> 5, row = p & 31;
+        const size_t n = 32 * tile + row;
+        *reinterpret_cast<uint4 *>(out + pf_q8t_piece_at(piece, row)) =
+            *reinterpret_cast<const uint4 *>(payload + (n * blocks_per_row + 2 * run) * 32 + 16 * piece);
+    } else {
+        const int row = p - 128;
+        const size_t n = 32 * tile + row, b = n * blocks_per_row + 2 * run;
+        *reinterpret_cast<uint32_t *>(out + pf_q8t_scales_at(row)) = (uint32_t)scales[b] | ((uint32_t)scales[b + 1] << 16);
+    }
+}
+
+void pf_launch_q8_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8_t *d_dst, size_t rows, int blocks_per_row,
+                       hipStream_t stream) {
+    const size_t threads = rows / 32 * (size_t)(blocks_per_row / 2) * 160;
+    hipLaunchKernelGGL(pf_k_q8_tile, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, d_payload, d_scales, d_dst, rows,
                        blocks_per_row);
 }
 
@@ -1539,7 +1657,7 @@ static void launch_gate_up(const PfKernelArgs &a, dim3 grid, size_t lds, hipStre
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
 #if PF_DECODE_PART == 0
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream) {
-    // the router's rows, the shared router's row, then the tokens' two-digit images (2048 values per workgroup);
+    // the router's rows, the shared router's row, then the tokens' digit images (2048 values per workgroup);
     // beyond four tokens: groups of four along the grid's second dimension
     const dim3 grid(router_blocks + 1 + tokens * ((a.hidden + 2047) / 2048), (tokens + 3) / 4), block(256);
     switch (tokens) {
@@ -1596,15 +1714,7 @@ static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t str
     pf_launch_dec_router(a, tokens, router_blocks, stream);
     if (last < 2) return;
     // kernel 2: every workgroup extracts the maxima up to its own slot from all of its token's logits
-    const int routed_blocks = K * (I / 32);
-    const dim3 g1(routed_blocks + Is / 32, tokens);
-    const int all = (E + 63) / 64;
-    const size_t lds = (size_t)table_words<FMT>() * 4 + (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
-    if (all <= 1) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<1, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 2) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<2, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 4) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<4, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 8) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<8, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<16, FMT>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    launch_gate_up_q4t<FMT, FMT>(a, tokens, stream);
     if (last < 3) return;
     const size_t widest = I > Is ? I : Is;
     hipLaunchKernelGGL((pf_k_dec_down_q4t<FMT>), dim3(H / 8, tokens), dim3(64 * (K + 1)),
@@ -1637,7 +1747,13 @@ static void launch_decode_passes(const PfKernelArgs &a, hipStream_t stream, int 
     int prefetch_blocks = (256 - routed_blocks - shared_blocks) / 8 * 8;
     if (prefetch_blocks < 8 || row_blocks_next % 8) prefetch_blocks = 0;
     dim3 g2(routed_blocks + shared_blocks + prefetch_blocks);
-    if (npl <= 1) launch_gate_up<FG, FS, NT, 1, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
+    bool tile_order = false;
+    if constexpr (NT == 1 && (FG == PF_Q4_K || FG == PF_IQ2_XXS) && (FS == FG || FS == PF_Q8_0)) tile_order = q4t_gate_up_applies<FG, FS>(a);
+    if constexpr (NT == 1 && (FG == PF_Q4_K || FG == PF_IQ2_XXS) && (FS == FG || FS == PF_Q8_0)) {
+        if (tile_order) launch_gate_up_q4t<FG, FS>(a, 1, stream);   // it publishes the unique-expert table kernel 3 below reads
+    }
+    if (tile_order) {}
+    else if (npl <= 1) launch_gate_up<FG, FS, NT, 1, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else if (npl <= 2) launch_gate_up<FG, FS, NT, 2, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else if (npl <= 4) launch_gate_up<FG, FS, NT, 4, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);
     else launch_gate_up<FG, FS, NT, 8, SPL2>(a, g2, lds2, stream, routed_blocks, shared_blocks, parts, chunk, tile);   // experts <= 1024

@@ -17,6 +17,7 @@ struct PfKernelArgs {
     int k_logical[8], blocks_per_row[8], n_out[8];
     const uint8_t *wt[8];            // Q4_K expert tensors in tile order for the grouped product (null: not kept)
     const uint8_t *wi[8];            // IQ2_XXS expert tensors in tile order for the decode kernels (null: not kept)
+    const uint8_t *wq[8];            // Q8_0 tensors (the profiles' shared gate and up) in tile order (null: not kept)
     const float *router_t;           // router as [slab of 64 experts][hidden / 4][64][4] (serial-order re-routing)
     const uint64_t *iq2_grid;        // 256 x 8 magnitudes, device memory
     const uint32_t *iq2_signed;      // 2 x 4096 words: four signed magnitudes per (grid entry, sign nibble)
@@ -110,12 +111,17 @@ struct PfHipMoe {
     float *router_t;                 // [slab of 64 experts][hidden / 4][64][4] copy of the router
     uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
     uint8_t *w_itile[8];             // tile-ordered second copy of IQ2_XXS expert tensors for the decode path (or null)
+    uint8_t *w_qtile[8];             // tile-ordered second copy of the Q8_0 shared gate and up tensors (or null)
     bool streamed;                   // the routed tensors are not resident: forwards read them from an expert pool
 };
 
-// Two-digit image of a K-vector for wave-uniform (scalar) reads: per 32-group 16 dwords (the values' low base-256
-// digits as 32 signed bytes, then their high digits), then K/32 group steps (float), then K/32 sums of the integers.
-__host__ __device__ constexpr size_t pf_image2_words(size_t K) { return (K / 32) * 18; }
+// Digit image of a K-vector for wave-uniform (scalar) reads: per 32-group PF_IMG_GROUP dwords (the values' lowest
+// base-256 digits as 32 signed bytes, then the next digits, then the highest), then K/32 group steps (float), then K/32
+// sums of the integers.  Two digits (16 bits) held the benchmark's tolerance but not that of layers with eight times
+// larger weights (1.6 times the bound on the smallest outputs of a row); three leave a margin of 2^8 more.
+#define PF_IMG_PLANES 3                       // signed byte digits per value: 24 bits
+#define PF_IMG_GROUP (8 * PF_IMG_PLANES)      // dwords of one 32-group's digits
+__host__ __device__ constexpr size_t pf_image2_words(size_t K) { return (K / 32) * (PF_IMG_GROUP + 2); }
 
 struct PfHipWork {
     const PfHipMoe *moe;
@@ -161,6 +167,8 @@ bool pf_decode_supported(const PfHipMoeDesc &d);
 uint32_t pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const q4k_tiled[8], const uint8_t *const iq2_tiled[8]);
 void pf_launch_iq2_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8_t *d_dst, size_t rows, int blocks_per_row,
                         hipStream_t stream);
+void pf_launch_q8_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8_t *d_dst, size_t rows, int blocks_per_row,
+                       hipStream_t stream);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);

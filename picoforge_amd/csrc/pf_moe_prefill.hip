@@ -116,6 +116,70 @@ __global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_
     }
 }
 
+// The same for rows of at most 512 values (the activation rows): one wave per row, four rows per workgroup, the row
+// read once -- a lane keeps its eight values between the maximum and the conversion.  With a workgroup per row three
+// of its four waves only took part in the maximum.
+__global__ void __launch_bounds__(256) pf_k_rows_to_half_short(const float *src, size_t src_pitch, int cols, size_t rows, half_t *dst,
+                                                               float *scale_out, float *max2_out, uint32_t *error_word) {
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int j = pf_lane();
+    const bool mine = j < cols / 8;
+    const float *s = src + row * src_pitch;
+    float4 a = make_float4(0.0f, 0.0f, 0.0f, 0.0f), b = a;
+    if (mine) { a = reinterpret_cast<const float4 *>(s)[2 * j]; b = reinterpret_cast<const float4 *>(s)[2 * j + 1]; }
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    float m = 0.0f;
+    bool bad = false;
+#pragma unroll
+    for (int c = 0; c < 8; c++) { bad |= !pf_finite(v[c]); m = fmaxf(m, fabsf(v[c])); }
+    m = pf_wave_max(m);
+    if (__any(bad) && j == 0) atomicOr(error_word, PF_HIP_ERR_NONFINITE);
+    int e = (__float_as_int(m) >> 23) & 255;                  // m in [2^(e-127), 2^(e-126))
+    e = (e == 0 || e == 255) ? 126 : min(e, 252);             // zero, subnormal or nonfinite row: scale 1
+    const float scale = __int_as_float((e + 1) << 23);        // 2^(e-126)
+    const float inv = __int_as_float((253 - e) << 23);        // 2^(126-e)
+    half_t *out = dst + row * pf_half_row(cols);
+    half8v hi, lo;
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        const float x = v[c] * inv;
+        const half_t h = (half_t)x, l = (half_t)(x - (float)h);
+        hi[c] = h;
+        lo[c] = l;
+        sum += (float)h + (float)l;
+    }
+    if (mine) {
+        *reinterpret_cast<half8v *>(out + 8 * j) = hi;
+        *reinterpret_cast<half8v *>(out + cols + 8 * j) = lo;
+    }
+    sum += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sum), 0xB1, 0xF, 0xF, true));   // quad xor 1
+    sum += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(sum), 0x4E, 0xF, 0xF, true));   // quad xor 2
+    if (mine && (j & 3) == 0) {
+        const int g = j >> 2;
+        const half_t sh = (half_t)sum, sl = (half_t)(sum - (float)sh);
+        half_t *sums = out + 2 * cols + 16 * (g >> 3) + 8 * (g & 1) + ((g & 7) >> 1);
+        sums[0] = sh;
+        sums[4] = sl;
+    }
+    if (j == 0) {
+        scale_out[row] = scale;
+        if (max2_out) max2_out[row] = m * m;
+    }
+}
+
+static void launch_rows_to_half(const float *src, size_t src_pitch, int cols, size_t rows, half_t *dst, float *scale_out,
+                                float *max2_out, uint32_t *error_word, hipStream_t stream) {
+    if (rows == 0) return;
+    if (cols <= 512)
+        hipLaunchKernelGGL(pf_k_rows_to_half_short, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, src, src_pitch, cols, rows,
+                           dst, scale_out, max2_out, error_word);
+    else
+        hipLaunchKernelGGL(pf_k_rows_to_half, dim3((unsigned)rows), dim3(256), 0, stream, src, src_pitch, cols, dst, scale_out,
+                           max2_out, error_word);
+}
+
 // squared norm of every router row (once, at upload)
 __global__ void __launch_bounds__(64) pf_k_row_norm2(const float *w, int cols, float *out) {
     const float *r = w + (size_t)blockIdx.x * cols;
@@ -1213,10 +1277,8 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     else launch_gemm<PF_GEMM_GATE_UP, PF_Q4_K>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
     // only the shared expert's tiles (tokens / 32 of them) are left for this launch: columns split over the waves
     if (a.type[4] != ring_fmt) launch_gemm_plain<PF_GEMM_GATE_UP>(a, tokens, tile_cap, (gi + 31) / 32, 1, stream);
-    hipLaunchKernelGGL(pf_k_rows_to_half, dim3(P), dim3(256), 0, stream, a.act, (size_t)I, I, (half_t *)a.act16, a.act_scale,
-                       (float *)nullptr, a.error_word);
-    hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.shared_act, (size_t)Is, Is,
-                       (half_t *)a.sact16, a.sact_scale, (float *)nullptr, a.error_word);
+    launch_rows_to_half(a.act, (size_t)I, I, (size_t)P, (half_t *)a.act16, a.act_scale, nullptr, a.error_word, stream);
+    launch_rows_to_half(a.shared_act, (size_t)Is, Is, (size_t)tokens, (half_t *)a.sact16, a.sact_scale, nullptr, a.error_word, stream);
     if (last < 4) return;
     // stage 4: down and combine
     if (a.type[3] == ring_fmt || a.type[6] == ring_fmt) {

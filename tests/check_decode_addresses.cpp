@@ -123,25 +123,41 @@ int main(int argc, char **argv) {
             }
         }
     }
-    // the tile-ordered IQ2_XXS copies (their own size: PF_I2T_CHUNK bytes per 32 rows and 256-block)
-    if (type[1] == PF_IQ2_XXS && type[2] == PF_IQ2_XXS && type[3] == PF_IQ2_XXS && type[4] == PF_IQ2_XXS && type[5] == PF_IQ2_XXS &&
-        type[6] == PF_IQ2_XXS && H % 256 == 0 && phys == I && I % 256 == 0 && Is % 256 == 0) {
-        for (int a = 1; a <= 6; a++) {
-            const int rows = (int)n_out[a], kblocks = (int)k_storage[a] / 256;
-            PfTensorPlace copy = place[a];
-            copy.expert_bytes = pf_i2t_expert_bytes(rows, kblocks);
-            copy.bytes = copy.expert_bytes * experts[a];
-            for (size_t e : some_experts) {
-                if (experts[a] == 1 && e) continue;
-                for (int n = 0; n < rows; n++)
-                    for (int kb = 0; kb < kblocks; kb++) {
-                        const size_t chunk = pf_i2t_chunk_at(copy.expert_bytes, e, n / 32, kblocks, kb);
-                        check("tile scale", a, copy, {chunk + pf_i2t_scale_at(n & 31), 2}, 2, e, n, kb);
-                        for (int run = 0; run < 4; run++)
-                            check("tile piece", a, copy, {chunk + pf_i2t_piece_at(run, n & 31), 16}, 16, e, n, 4 * kb + run);
-                    }
-            }
+    // the tile-ordered IQ2_XXS copies (their own size: PF_I2T_CHUNK bytes per 32 rows and 256-block): every IQ2_XXS
+    // expert tensor of a layer that is IQ2_XXS throughout, the routed gate and up tensors of the q2 profile
+    for (int a = 1; a <= 6; a++) {
+        if (type[a] != PF_IQ2_XXS || n_out[a] % 32 || k_storage[a] % 256) continue;
+        const int rows = (int)n_out[a], kblocks = (int)k_storage[a] / 256;
+        PfTensorPlace copy = place[a];
+        copy.expert_bytes = pf_i2t_expert_bytes(rows, kblocks);
+        copy.bytes = copy.expert_bytes * experts[a];
+        for (size_t e : some_experts) {
+            if (experts[a] == 1 && e) continue;
+            for (int n = 0; n < rows; n++)
+                for (int kb = 0; kb < kblocks; kb++) {
+                    const size_t chunk = pf_i2t_chunk_at(copy.expert_bytes, e, n / 32, kblocks, kb);
+                    check("tile scale", a, copy, {chunk + pf_i2t_scale_at(n & 31), 2}, 2, e, n, kb);
+                    for (int run = 0; run < 4; run++)
+                        check("tile piece", a, copy, {chunk + pf_i2t_piece_at(run, n & 31), 16}, 16, e, n, 4 * kb + run);
+                }
         }
+    }
+    // the tile-ordered Q8_0 copies of the profiles' shared gate and up tensors: one chunk per 64-weight run, addressed by
+    // the gate/up kernel as four chunks per 256-block
+    for (int a : {4, 5}) {
+        if (type[a] != PF_Q8_0 || n_out[a] % 32 || k_storage[a] % 256) continue;
+        const int rows = (int)n_out[a], kblocks = (int)k_storage[a] / 256, runs = 4 * kblocks;
+        PfTensorPlace copy = place[a];
+        copy.expert_bytes = pf_q8t_expert_bytes(rows, runs);
+        copy.bytes = copy.expert_bytes;
+        for (int n = 0; n < rows; n++)
+            for (int kb = 0; kb < kblocks; kb++)
+                for (int run = 0; run < 4; run++) {
+                    const size_t chunk = pf_q8t_chunk_at(0, 0, n / 32, runs, 4 * kb) + (size_t)run * PF_I2T_CHUNK;
+                    check("tile scales", a, copy, {chunk + pf_q8t_scales_at(n & 31), 4}, 4, 0, n, 4 * kb + run);
+                    for (int p = 0; p < 4; p++)
+                        check("tile piece", a, copy, {chunk + pf_q8t_piece_at(p, n & 31), 16}, 16, 0, n, 4 * kb + run);
+                }
     }
     printf("%lld spans checked, %lld outside or misaligned\n", checked, bad);
     return bad ? 1 : 0;
