@@ -178,7 +178,7 @@ def measured_traffic(workload):
     if not path.exists():
         return None, None
     entry = json.loads(path.read_text()).get(workload)
-    if not entry:
+    if not entry or WORKLOADS.get(workload, {}).get("custom_shape"):   # --dims: the table holds the workload's own shape
         return None, None
     source = {"profile": entry.get("profile"), "sources": entry.get("sources"), "kernel": entry.get("kernel")}
     if entry.get("sources") != sources_digest():
@@ -615,7 +615,18 @@ def main():
                          "under a profiler, which records the kernels' durations itself")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="also launch a plain copy kernel of this many MiB three times (byte-counter calibration)")
+    ap.add_argument("--dims", default=None, metavar="H,E,K,I,S,P",
+                    help="with --workload NAME: the layer's shape instead of the workload's own (hidden, experts, top_k, "
+                         "intermediate, shared intermediate, stored width of the down projection)")
     args = ap.parse_args()
+    if args.dims:
+        if args.workload == "all":
+            sys.exit("--dims needs --workload NAME")
+        dims = tuple(int(v) for v in args.dims.split(","))
+        if len(dims) != 6:
+            sys.exit("--dims takes six numbers: H,E,K,I,S,P")
+        wl = WORKLOADS[args.workload]
+        WORKLOADS[args.workload] = dict(wl, dims=dims, custom_shape=True, label=wl["label"] + " at the shape " + args.dims)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); use --gpus 1")
 

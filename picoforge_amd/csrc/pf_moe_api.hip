@@ -309,7 +309,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
     // A Q4_K layer that every kernel family can read through the tile-ordered copy alone (the decode kernels whose lanes
     // are weight rows, the grouped product, the general kernels' tile reader) gives its row-ordered expert tensors
     // back: one copy of the experts in device memory, not two.
-    if (pf_decode_tile_layer(m->desc, m->w_tiled, m->w_itile) == PF_Q4_K) {
+    if (pf_decode_tile_layer(m->desc, m->w_tiled, m->w_itile, m->w_qtile) == 1) {
         for (int a = 1; a <= 6; a++) {
             (void)hipFree(m->w[a]);
             m->w[a] = nullptr;
@@ -344,8 +344,9 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden, I = d->inter;
     const size_t Td = T < PF_DECODE_MAX_TOKENS ? T : PF_DECODE_MAX_TOKENS;   // tokens per decode launch
     // ... and per launch of the kernels for tile-ordered Q4_K (whether the copies are kept is not known here)
-    bool one_format = d->type[1] == PF_Q4_K || d->type[1] == PF_IQ2_XXS;
-    for (int t = 2; t <= 6; t++) one_format &= d->type[t] == d->type[1];
+    // (one format throughout, or a checkpoint profile: Q8_0 shared expert)
+    bool one_format = (d->type[1] == PF_Q4_K || d->type[1] == PF_IQ2_XXS) && d->type[2] == d->type[1];
+    for (int t = 4; t <= 6; t++) one_format &= d->type[t] == d->type[1] || d->type[t] == PF_Q8_0;
     const size_t Tt = !one_format ? Td : T < PF_TILE_DECODE_MAX_TOKENS ? T : PF_TILE_DECODE_MAX_TOKENS;
     size_t want[W_COUNT];
     want[W_LOGITS] = T * E * 4;
@@ -527,7 +528,7 @@ struct HcTarget {   // residual streams to inject into instead of writing y
 
 // Most tokens the decode kernels take in one forward of this layer.
 static size_t decode_limit(const PfHipMoe *moe) {
-    return pf_decode_tile_layer(moe->desc, moe->w_tiled, moe->w_itile) ? PF_TILE_DECODE_MAX_TOKENS : PF_DECODE_MAX_TOKENS;
+    return pf_decode_tile_layer(moe->desc, moe->w_tiled, moe->w_itile, moe->w_qtile) ? PF_TILE_DECODE_MAX_TOKENS : PF_DECODE_MAX_TOKENS;
 }
 
 static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_x, size_t x_pitch, float *d_y,

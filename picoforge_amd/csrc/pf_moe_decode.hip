@@ -1346,13 +1346,6 @@ __global__ void __launch_bounds__(MAXT) pf_k_dec_down(PfKernelArgs a, int row_bl
 // and two halves; IQ2_XXS: one 16-byte piece and the block's half scale, magnitudes from the tables.
 __device__ __forceinline__ float down_dot(const TileItem<PF_Q4_K> &w, int rr, const uint32_t *mine, int run, int groups, const uint32_t *) {
     const uint4 hdr = w.hdr, p0 = w.piece[0], p1 = w.piece[1];
-    // the run's two groups: PF_IMG_GROUP dwords each, plane by plane
-    uint32_t dg[2 * PF_IMG_GROUP];
-#pragma unroll
-    for (int i = 0; i < 2 * PF_IMG_GROUP / 4; i++) {
-        const uint4 v = reinterpret_cast<const uint4 *>(mine + 2 * PF_IMG_GROUP * run)[i];
-        dg[4 * i] = v.x; dg[4 * i + 1] = v.y; dg[4 * i + 2] = v.z; dg[4 * i + 3] = v.w;
-    }
     const uint2 st = *reinterpret_cast<const uint2 *>(mine + PF_IMG_GROUP * groups + 2 * run);
     const uint2 sm = *reinterpret_cast<const uint2 *>(mine + (PF_IMG_GROUP + 1) * groups + 2 * run);
     uint32_t sc2, mn2;
@@ -1366,19 +1359,28 @@ __device__ __forceinline__ float down_dot(const TileItem<PF_Q4_K> &w, int rr, co
     }
     const float d = half_bits(hdr.x & 0xffffu), dmin = half_bits(hdr.x >> 16);
     const uint32_t q[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-    int lo_part[PF_IMG_PLANES] = {}, hi_part[PF_IMG_PLANES] = {};
+    float value[2];
+    // the run's two groups, PF_IMG_GROUP dwords each, plane by plane: the low nibbles against the first, the high against the second
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const int lo = (int)(q[i] & 0x0F0F0F0Fu), hi = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+    for (int g = 0; g < 2; g++) {
+        uint32_t dg[PF_IMG_GROUP];
 #pragma unroll
-        for (int p = 0; p < PF_IMG_PLANES; p++) {
-            lo_part[p] = __builtin_amdgcn_sdot4(lo, (int)dg[8 * p + i], lo_part[p], false);
-            hi_part[p] = __builtin_amdgcn_sdot4(hi, (int)dg[PF_IMG_GROUP + 8 * p + i], hi_part[p], false);
+        for (int i = 0; i < PF_IMG_GROUP / 4; i++) {
+            const uint4 v = reinterpret_cast<const uint4 *>(mine + PF_IMG_GROUP * (2 * run + g))[i];
+            dg[4 * i] = v.x; dg[4 * i + 1] = v.y; dg[4 * i + 2] = v.z; dg[4 * i + 3] = v.w;
         }
+        int part[PF_IMG_PLANES] = {};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int nib = (int)((q[i] >> (4 * g)) & 0x0F0F0F0Fu);
+#pragma unroll
+            for (int p = 0; p < PF_IMG_PLANES; p++) part[p] = __builtin_amdgcn_sdot4(nib, (int)dg[8 * p + i], part[p], false);
+        }
+        value[g] = image_value(part);
     }
     const float s0 = (float)(sc2 & 255u), m0 = (float)(mn2 & 255u), s1 = (float)(sc2 >> 8), m1 = (float)(mn2 >> 8);
-    const float t0 = fmaf(d * s0, image_value(lo_part), -(dmin * m0) * (float)(int)sm.x);
-    const float t1 = fmaf(d * s1, image_value(hi_part), -(dmin * m1) * (float)(int)sm.y);
+    const float t0 = fmaf(d * s0, value[0], -(dmin * m0) * (float)(int)sm.x);
+    const float t1 = fmaf(d * s1, value[1], -(dmin * m1) * (float)(int)sm.y);
     return fmaf(__uint_as_float(st.x), t0, __uint_as_float(st.y) * t1);
 }
 
@@ -1388,16 +1390,16 @@ __device__ __forceinline__ float down_dot(const TileItem<PF_IQ2_XXS> &w, int, co
                                           const uint32_t *tables) {
     const uint4 piece = w.piece;
     const uint32_t dbits = w.dbits;
-    uint32_t d32[2 * PF_IMG_GROUP];
-#pragma unroll
-    for (int i = 0; i < 2 * PF_IMG_GROUP / 4; i++) {
-        const uint4 v = reinterpret_cast<const uint4 *>(mine + 2 * PF_IMG_GROUP * run)[i];
-        d32[4 * i] = v.x; d32[4 * i + 1] = v.y; d32[4 * i + 2] = v.z; d32[4 * i + 3] = v.w;
-    }
     const uint2 st = *reinterpret_cast<const uint2 *>(mine + PF_IMG_GROUP * groups + 2 * run);
     float acc[2];
 #pragma unroll
     for (int gg = 0; gg < 2; gg++) {
+        uint32_t d32[PF_IMG_GROUP];
+#pragma unroll
+        for (int i = 0; i < PF_IMG_GROUP / 4; i++) {
+            const uint4 v = reinterpret_cast<const uint4 *>(mine + PF_IMG_GROUP * (2 * run + gg))[i];
+            d32[4 * i] = v.x; d32[4 * i + 1] = v.y; d32[4 * i + 2] = v.z; d32[4 * i + 3] = v.w;
+        }
         const uint32_t idx = gg ? piece.z : piece.x, word = gg ? piece.w : piece.y;
         int part[PF_IMG_PLANES] = {};
 #pragma unroll
@@ -1411,8 +1413,8 @@ __device__ __forceinline__ float down_dot(const TileItem<PF_IQ2_XXS> &w, int, co
             const int ml = (int)((mag.x ^ (tl * 0xFFu)) + tl), mh = (int)((mag.y ^ (th * 0xFFu)) + th);
 #pragma unroll
             for (int p = 0; p < PF_IMG_PLANES; p++) {
-                part[p] = __builtin_amdgcn_sdot4(ml, (int)d32[PF_IMG_GROUP * gg + 8 * p + 2 * slot], part[p], false);
-                part[p] = __builtin_amdgcn_sdot4(mh, (int)d32[PF_IMG_GROUP * gg + 8 * p + 2 * slot + 1], part[p], false);
+                part[p] = __builtin_amdgcn_sdot4(ml, (int)d32[8 * p + 2 * slot], part[p], false);
+                part[p] = __builtin_amdgcn_sdot4(mh, (int)d32[8 * p + 2 * slot + 1], part[p], false);
             }
         }
         acc[gg] = __uint_as_float(gg ? st.y : st.x) * (float)(2u * (word >> 28) + 1u) * image_value(part);
@@ -1420,20 +1422,169 @@ __device__ __forceinline__ float down_dot(const TileItem<PF_IQ2_XXS> &w, int, co
     return half_bits(dbits) * 0.125f * (acc[0] + acc[1]);
 }
 
-template <int FMT>
-__global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
-    __shared__ float partial[17][8];
-    extern __shared__ int lds[];   // IQ2_XXS: the magnitude grid; then [slot][image words of the widest activation row]
+// The formats kept row by row (the profiles' down tensors): a lane's run is the segment the loaders above fetch; lanes
+// r * 8 + part, so that the eight runs of a row are neighbouring lanes and neighbouring bytes.
+struct GroupDigits {   // one 32-group from the slot's image in LDS
+    uint32_t dg[PF_IMG_GROUP];
+    float step;
+};
+__device__ __forceinline__ void group_digits(GroupDigits &x, const uint32_t *mine, int group, int groups) {
+#pragma unroll
+    for (int i = 0; i < PF_IMG_GROUP / 4; i++) {
+        const uint4 v = reinterpret_cast<const uint4 *>(mine + PF_IMG_GROUP * group)[i];
+        x.dg[4 * i] = v.x; x.dg[4 * i + 1] = v.y; x.dg[4 * i + 2] = v.z; x.dg[4 * i + 3] = v.w;
+    }
+    x.step = __uint_as_float(mine[PF_IMG_GROUP * groups + group]);
+}
+
+__device__ __forceinline__ float down_dot(const WSeg<PF_Q8_0> &w, const uint32_t *mine, int run, int groups) {
+    float out = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        GroupDigits x;
+        group_digits(x, mine, 2 * run + g, groups);
+        const uint32_t q[8] = {w.q[2 * g].x, w.q[2 * g].y, w.q[2 * g].z, w.q[2 * g].w,
+                               w.q[2 * g + 1].x, w.q[2 * g + 1].y, w.q[2 * g + 1].z, w.q[2 * g + 1].w};
+        int part[PF_IMG_PLANES] = {};
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int p = 0; p < PF_IMG_PLANES; p++) part[p] = __builtin_amdgcn_sdot4((int)q[i], (int)x.dg[8 * p + i], part[p], false);
+        out = fmaf(x.step * half_bits((w.d2 >> (16 * g)) & 0xffffu), image_value(part), out);
+    }
+    return out;
+}
+
+__device__ __forceinline__ float down_dot(const WSeg<PF_MXFP4> &w, const uint32_t *mine, int run, int groups) {
+    float out = 0.0f;
+#pragma unroll
+    for (int g = 0; g < 2; g++) {
+        GroupDigits x;
+        group_digits(x, mine, 2 * run + g, groups);
+        const uint32_t q[4] = {w.q[g].x, w.q[g].y, w.q[g].z, w.q[g].w};
+        int part[PF_IMG_PLANES] = {};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {   // a byte's low nibble is weight j of the block, its high nibble weight j + 16
+            const int lo = e2m1_twice4(q[i] & 0x0F0F0F0Fu), hi = e2m1_twice4((q[i] >> 4) & 0x0F0F0F0Fu);
+#pragma unroll
+            for (int p = 0; p < PF_IMG_PLANES; p++) {
+                part[p] = __builtin_amdgcn_sdot4(lo, (int)x.dg[8 * p + i], part[p], false);
+                part[p] = __builtin_amdgcn_sdot4(hi, (int)x.dg[8 * p + 4 + i], part[p], false);
+            }
+        }
+        const float scale = 0.5f * pf_e8m0_scale((w.e2 >> (8 * g)) & 255u);   // the integers are twice the values
+        out = fmaf(x.step * scale, image_value(part), out);
+    }
+    return out;
+}
+
+// Q2_K: the sums of the activation integers per sub-group of 16 come from dot products with ones, as in wseg_dot.
+__device__ __forceinline__ float down_dot(const WSeg<PF_Q2_K> &w, const uint32_t *mine, int run, int groups) {
+    const float d = half_bits(w.dd & 0xffffu), dmin = half_bits(w.dd >> 16);
+    float out = 0.0f;
+#pragma unroll
+    for (int gg = 0; gg < 2; gg++) {
+        GroupDigits x;
+        group_digits(x, mine, 2 * run + gg, groups);
+        const int shift = 2 * (2 * (run & 1) + gg);
+        float group = 0.0f;
+#pragma unroll
+        for (int sub = 0; sub < 2; sub++) {
+            int c[PF_IMG_PLANES] = {}, ones[PF_IMG_PLANES] = {};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int codes = (int)((w.q[4 * sub + i] >> shift) & 0x03030303u);
+#pragma unroll
+                for (int p = 0; p < PF_IMG_PLANES; p++) {
+                    const int digits = (int)x.dg[8 * p + 4 * sub + i];
+                    c[p] = __builtin_amdgcn_sdot4(codes, digits, c[p], false);
+                    ones[p] = __builtin_amdgcn_sdot4(0x01010101, digits, ones[p], false);
+                }
+            }
+            const uint32_t sm = (w.sm >> (8 * (2 * gg + sub))) & 255u;
+            group += fmaf(d * (float)(sm & 15u), image_value(c), -(dmin * (float)(sm >> 4)) * image_value(ones));
+        }
+        out = fmaf(x.step, group, out);
+    }
+    return out;
+}
+
+constexpr size_t Q4T_DOWN_LDS = 150 * 1024;   // dynamic LDS kernel 3 on the tile order may ask for
+template <int F> __host__ __device__ constexpr bool tile_ordered() { return F == PF_Q4_K || F == PF_IQ2_XXS; }
+
+// One wave's rows of its slot (eight in the tile order): partial_row[0..rows).  tensor: 3 (the slot's expert e) or 6 (the
+// shared expert); I: the logical width, k_stored: the stored one; dots: rows * I / 64 floats of LDS of the wave's own.
+template <int F>
+__device__ __forceinline__ void down_wave(const PfKernelArgs &a, int tensor, uint32_t e, int I, int k_stored, int n_base, int rows,
+                                          const uint32_t *image, uint32_t *mine, uint32_t *tables, float *dots, float *partial_row) {
+    const int lane = pf_lane(), runs = I / 64, groups = I / 32;
+    // IQ2_XXS: every wave keeps its own copy of the 2 KB magnitude grid, so that no wave waits for another before the
+    // final sums (a shared copy needs a workgroup barrier between its staging and its first use)
+    if (F == PF_IQ2_XXS) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.iq2_grid);
+        reinterpret_cast<uint4 *>(tables)[lane] = src[lane];
+        reinterpret_cast<uint4 *>(tables)[64 + lane] = src[64 + lane];
+    }
+    // the slot's image into this wave's part of LDS (each lane needs the digits of its own run; fetched per lane they
+    // would cost eight requests a lane).  Sending the first weights' loads ahead of the image's, or two steps' weights
+    // at once, measured the same or slower.
+    const int words = (int)pf_image2_words(I);
+    for (int i = 4 * lane; i < words; i += 256) *reinterpret_cast<uint4 *>(mine + i) = *reinterpret_cast<const uint4 *>(image + i);
+    float total = 0.0f;
+    bool fenced = false;
+    if constexpr (tile_ordered<F>()) {
+        typedef TileGeometry<F> G;
+        const int r = lane & 7, part = lane >> 3, kblocks = k_stored / 256;
+        const uint8_t *tile = G::tensor(a, tensor) + (size_t)e * G::expert_bytes(a, tensor) + G::chunk_at(n_base / 32, kblocks, 0);
+        const int row_in_tile = (n_base & 31) + r;
+        for (int run = part; run < runs; run += 8) {
+            TileItem<F> item;
+            q4t_load(item, tile + G::chunk_at(0, kblocks, run >> 2), row_in_tile, run & 3);
+            if (!fenced) { pf_wave_lds_fence(); fenced = true; }   // the image's (and grid's) stores of this wave before its reads
+            total += down_dot(item, run & 3, mine, run, groups, tables);
+        }
+        // the row's runs: lanes r, r + 8, ..., r + 56
+        total += __shfl_xor(total, 8);
+        total += __shfl_xor(total, 16);
+        total += __shfl_xor(total, 32);
+        if (lane < 8) partial_row[lane] = total;
+    } else {
+        // the (row, run) pairs of the wave's rows in turn over the lanes: neighbouring lanes are neighbouring runs of a
+        // row, neighbouring bytes, and a row count that does not divide 64 (ten for a hidden width of 2560) leaves no
+        // lane idle but in the last step.  The products meet in LDS; a lane per row adds its runs in order.
+        const int items = rows * runs;
+        for (int item = lane; item < items; item += 64) {
+            const int r = item / runs, run = item - r * runs;
+            WSeg<F> w;
+            wseg_load<F>(w, a, tensor, e, (size_t)(n_base + r), run);
+            if (!fenced) { pf_wave_lds_fence(); fenced = true; }
+            dots[item] = down_dot(w, mine, run, groups);
+        }
+        pf_wave_lds_fence();
+        if (lane < rows) {
+            for (int run = 0; run < runs; run++) total += dots[lane * runs + run];
+            partial_row[lane] = total;
+        }
+    }
+}
+
+// (at most 80 registers a lane: two workgroups of eleven waves then share a compute unit, which a hidden width of 2560,
+// 320 workgroups on 256 compute units, needs to finish in one round)
+template <int FMT, int FMTS>
+__global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT == PF_IQ2_XXS ? 4 : 6))) pf_k_dec_down_q4t(PfKernelArgs a, int rows) {
+    __shared__ float partial[17][16];
+    extern __shared__ int lds[];   // IQ2_XXS: the waves' magnitude grids; [slot][image words of the widest activation row]; [slot][rows * runs] products
+    constexpr bool GRID = FMT == PF_IQ2_XXS || FMTS == PF_IQ2_XXS;
     const int token = (int)blockIdx.y;
     q4t_at_token(a, token);
     const int H = a.hidden, K = a.top_k, lane = pf_lane();
     const int s = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
-    int *images = lds + (FMT == PF_IQ2_XXS ? 512 * (K + 1) : 0);   // IQ2_XXS: the waves' copies of the magnitude grid first
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds) + (GRID ? 512 * s : 0);
+    int *images = lds + (GRID ? 512 * (K + 1) : 0);
     const bool shared = s == K;
-    const int I = shared ? a.shared_inter : a.inter;
-    const int n_base = 8 * (int)blockIdx.x, r = lane & 7, part = lane >> 3;
+    const int n_base = rows * (int)blockIdx.x;
     const size_t widest = a.inter > a.shared_inter ? a.inter : a.shared_inter;
+    float *dots = reinterpret_cast<float *>(images + (size_t)(K + 1) * pf_image2_words(widest)) + (size_t)s * rows * (widest / 64);
     // the slot's expert and the combine's operands through the scalar cache
     const PfScalarWords ids = (PfScalarWords)(uintptr_t)a.ids, rws = (PfScalarWords)(uintptr_t)a.route_weights;
     uint32_t e = shared ? 0u : ids[s];
@@ -1446,44 +1597,14 @@ __global__ void __launch_bounds__(1024) pf_k_dec_down_q4t(PfKernelArgs a) {
         e = 0;
     }
     PfOutputRegs out_regs;
-    if ((int)threadIdx.x < 8) pf_output_prefetch(a, token, n_base + threadIdx.x, out_regs);
-    typedef TileGeometry<FMT> G;
-    const int tensor = shared ? 6 : 3;
-    const uint8_t *w = (shared ? G::tensor(a, 6) : G::tensor(a, 3)) + (size_t)e * (shared ? G::expert_bytes(a, 6) : G::expert_bytes(a, 3));
-    (void)tensor;
-    const int kblocks = (shared ? a.shared_inter : a.down_physical) / 256, runs = I / 64, groups = I / 32;
+    if ((int)threadIdx.x < rows) pf_output_prefetch(a, token, n_base + threadIdx.x, out_regs);
     const uint32_t *image = a.aimg + (size_t)s * pf_image2_words(widest);   // slot = unique expert with one token; the shared expert's follows
-    const uint8_t *tile = w + G::chunk_at(n_base / 32, kblocks, 0);
-    const int row_in_tile = (n_base & 31) + r;
-    // IQ2_XXS: every wave keeps its own copy of the 2 KB magnitude grid, so that no wave waits for another before the
-    // final sums (a shared copy needs a workgroup barrier between its staging and its first use)
-    if (FMT == PF_IQ2_XXS) {
-        tables += 512 * s;
-        const uint4 *src = reinterpret_cast<const uint4 *>(a.iq2_grid);
-        reinterpret_cast<uint4 *>(tables)[lane] = src[lane];
-        reinterpret_cast<uint4 *>(tables)[64 + lane] = src[64 + lane];
-    }
-    // the slot's image into this wave's part of LDS (each lane needs the digits of its own run; fetched per lane they
-    // would cost eight requests a lane)
     uint32_t *mine = reinterpret_cast<uint32_t *>(images) + (size_t)s * pf_image2_words(widest);
-    const int words = (int)pf_image2_words(I);
-    for (int i = 4 * lane; i < words; i += 256) *reinterpret_cast<uint4 *>(mine + i) = *reinterpret_cast<const uint4 *>(image + i);
-    float total = 0.0f;
-    bool fenced = false;
-    for (int run = part; run < runs; run += 8) {
-        TileItem<FMT> item;
-        q4t_load(item, tile + G::chunk_at(0, kblocks, run >> 2), row_in_tile, run & 3);
-        if (!fenced) { pf_wave_lds_fence(); fenced = true; }   // the image's (and grid's) stores of this wave before its reads
-        total += down_dot(item, run & 3, mine, run, groups, tables);
-    }
-    // the row's runs: lanes r, r + 8, ..., r + 56
-    total += __shfl_xor(total, 8);
-    total += __shfl_xor(total, 16);
-    total += __shfl_xor(total, 32);
-    if (lane < 8) partial[s][lane] = total;
+    if (shared) down_wave<FMTS>(a, 6, 0u, a.shared_inter, a.shared_inter, n_base, rows, image, mine, tables, dots, partial[s]);
+    else down_wave<FMT>(a, 3, e, a.inter, a.down_physical, n_base, rows, image, mine, tables, dots, partial[s]);
     __syncthreads();
     const int n = n_base + threadIdx.x;
-    if ((int)threadIdx.x < 8 && n < H) {
+    if ((int)threadIdx.x < rows && n < H) {
         float sum = 0.0f;
 #pragma unroll
         for (int slot = 0; slot < 16; slot++)   // slot order, as src/qwen4_moe.c:362-372
@@ -1692,35 +1813,70 @@ static void launch_down(const PfKernelArgs &a, dim3 grid, dim3 block, size_t lds
         launch_down_bounded<FD, FS, NT, SPL, 1024>(a, grid, block, lds, stream, row_blocks, rows_per_block, image_pitch);
 }
 
-// Every expert tensor Q4_K, or every one IQ2_XXS, with its tile-ordered copy kept, and widths the kernels whose lanes
-// are weight rows cover: those take the layer, one token per grid row, for up to PF_TILE_DECODE_MAX_TOKENS tokens.
-// Returns the format, 0 for other layers.
+// Layers the kernels whose lanes are weight rows take, one token per grid row, for up to PF_TILE_DECODE_MAX_TOKENS
+// tokens: every expert tensor Q4_K, or every one IQ2_XXS, with its tile-ordered copy kept; the two checkpoint profiles
+// with the tile-ordered copies of their routed gate and up tensors and of the shared expert's Q8_0 gate and up (their
+// down tensors are read row by row).  Returns the combination as decode_combination numbers it, 0 for other layers.
 #if PF_DECODE_PART == 0
-uint32_t pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const q4k_tiled[8], const uint8_t *const iq2_tiled[8]) {
+int pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const q4k_tiled[8], const uint8_t *const iq2_tiled[8],
+                         const uint8_t *const q8_tiled[8]) {
+    const int combination = decode_combination(d.type);
+    if (!combination) return 0;
     const uint32_t format = d.type[1];
-    if (format != PF_Q4_K && format != PF_IQ2_XXS) return 0;
-    for (int t = 1; t <= 6; t++)
-        if (d.type[t] != format || !(format == PF_Q4_K ? q4k_tiled[t] : iq2_tiled[t])) return 0;
-    const bool fits = d.hidden % 256 == 0 && 4 * (d.hidden / 256) <= 15 * Q4T_ITEMS && d.inter % 256 == 0 &&
-                      d.shared_inter % 256 == 0 && d.down_physical == d.inter && d.top_k < d.experts && d.top_k <= 15 &&
-                      d.experts <= 1024;
-    return fits ? format : 0;
+    const uint8_t *const *tiled = format == PF_Q4_K ? q4k_tiled : iq2_tiled;
+    bool fits = d.hidden % 256 == 0 && 4 * (d.hidden / 256) <= 15 * Q4T_ITEMS && d.top_k < d.experts && d.top_k <= 15 &&
+                d.experts <= 1024;
+    if (combination <= 2) {
+        for (int t = 1; t <= 6; t++) fits &= tiled[t] != nullptr;
+        fits &= d.inter % 256 == 0 && d.shared_inter % 256 == 0 && d.down_physical == d.inter;
+    } else {
+        fits &= tiled[1] && tiled[2] && q8_tiled[4] && q8_tiled[5];
+        fits &= d.inter % 64 == 0 && d.shared_inter % 64 == 0 && row_width_ok(d.type[3], d.down_physical) &&
+                row_width_ok(d.type[6], d.shared_inter) && d.down_physical >= d.inter;
+    }
+    // kernel 3's LDS: per slot the activation row's image and the products of up to 16 rows, and the IQ2_XXS grids
+    const size_t widest = d.inter > d.shared_inter ? d.inter : d.shared_inter;
+    fits &= (size_t)(d.top_k + 1) * ((pf_image2_words(widest) + 16 * (widest / 64)) * 4 + 2048) <= Q4T_DOWN_LDS;
+    return fits ? combination : 0;
+}
+#endif
+
+static PfHipMoeDesc desc_of(const PfKernelArgs &a) {
+    PfHipMoeDesc d = {};
+    d.hidden = a.hidden; d.experts = a.experts; d.top_k = a.top_k; d.inter = a.inter; d.shared_inter = a.shared_inter;
+    d.down_physical = a.down_physical;
+    for (int t = 0; t < 8; t++) d.type[t] = a.type[t];
+    return d;
 }
 
-template <int FMT>
+template <int FG, int FD, int FS>
 static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
     const int router_blocks = (E + 3) / 4, last = stage_limit ? stage_limit : 3;
     pf_launch_dec_router(a, tokens, router_blocks, stream);
     if (last < 2) return;
     // kernel 2: every workgroup extracts the maxima up to its own slot from all of its token's logits
-    launch_gate_up_q4t<FMT, FMT>(a, tokens, stream);
+    launch_gate_up_q4t<FG, FS>(a, tokens, stream);
     if (last < 3) return;
     const size_t widest = I > Is ? I : Is;
-    hipLaunchKernelGGL((pf_k_dec_down_q4t<FMT>), dim3(H / 8, tokens), dim3(64 * (K + 1)),
-                       (FMT == PF_IQ2_XXS ? 2048 * (size_t)(K + 1) : 0) + (size_t)(K + 1) * pf_image2_words(widest) * 4, stream, a);
+    constexpr bool GRID = FD == PF_IQ2_XXS || FS == PF_IQ2_XXS;
+    // rows per workgroup: eight in the tile order; for down tensors kept row by row the fewest that leave no more
+    // workgroups than compute units (256 on this GPU), so that a hidden width of 2560 runs ten rows in one round
+    int rows = 8;
+    if (!tile_ordered<FD>() && !tile_ordered<FS>()) {
+        rows = (H + 255) / 256;
+        while (rows < 16 && H % rows) rows++;
+        if (H % rows || rows > 16) rows = 8;
+    }
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down_q4t<FD, FS>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)Q4T_DOWN_LDS);
+        configured = true;
+    }
+    hipLaunchKernelGGL((pf_k_dec_down_q4t<FD, FS>), dim3(H / rows, tokens), dim3(64 * (K + 1)),
+                       (GRID ? 2048 * (size_t)(K + 1) : 0) + (size_t)(K + 1) * (pf_image2_words(widest) + rows * (widest / 64)) * 4, stream, a, rows);
 }
-#endif
 
 // FG: format of the routed gate and up tensors, FD: of the routed down tensor, FS: of the shared expert
 template <int FG, int FD, int FS, int NT, int SPL2>
@@ -1791,26 +1947,15 @@ void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t s
 void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 
 #if PF_DECODE_PART == 0
-static PfHipMoeDesc desc_of(const PfKernelArgs &a) {
-    PfHipMoeDesc d = {};
-    d.hidden = a.hidden; d.experts = a.experts; d.top_k = a.top_k; d.inter = a.inter; d.shared_inter = a.shared_inter;
-    d.down_physical = a.down_physical;
-    for (int t = 0; t < 8; t++) d.type[t] = a.type[t];
-    return d;
-}
-
 void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi) == PF_Q4_K) launch_decode_q4t<PF_Q4_K>(a, tokens, stream, stage_limit);
+    if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq) == 1) launch_decode_q4t<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
     else launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     switch (decode_combination(a.type)) {
     case 1: pf_launch_decode_q4k(a, tokens, stream, stage_limit); break;
-    case 2:
-        if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi) == PF_IQ2_XXS) launch_decode_q4t<PF_IQ2_XXS>(a, tokens, stream, stage_limit);
-        else pf_launch_decode_iq2(a, tokens, stream, stage_limit);
-        break;
+    case 2: pf_launch_decode_iq2(a, tokens, stream, stage_limit); break;
     case 3: pf_launch_decode_q2profile(a, tokens, stream, stage_limit); break;
     case 4: pf_launch_decode_q4profile(a, tokens, stream, stage_limit); break;
     default: break;   // pf_decode_supported keeps other combinations away
@@ -1818,14 +1963,20 @@ void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int
 }
 #elif PF_DECODE_PART == 1
 void pf_launch_decode_iq2(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    launch_decode_tokens<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit);
+    if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq) == 2)
+        launch_decode_q4t<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit);
+    else launch_decode_tokens<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit);
 }
 #elif PF_DECODE_PART == 2
 void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    launch_decode_tokens<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit);
+    if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq) == 3)
+        launch_decode_q4t<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit);
+    else launch_decode_tokens<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit);
 }
 #else
 void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    launch_decode_tokens<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit);
+    if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq) == 4)
+        launch_decode_q4t<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit);
+    else launch_decode_tokens<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit);
 }
 #endif

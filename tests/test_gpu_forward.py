@@ -40,6 +40,7 @@ DECODE = [
     (512, 32, 6, 256, 256, abi.GGUF_Q4_K), (512, 32, 6, 256, 256, abi.GGUF_IQ2_XXS),
     (1024, 96, 5, 512, 256, abi.GGUF_Q4_K), (1024, 96, 5, 256, 1024, abi.GGUF_IQ2_XXS),
     (2048, 64, 10, 1024, 512, abi.GGUF_Q4_K),
+    (512, 32, 14, 1536, 512, abi.GGUF_Q4_K),      # the widest activation rows: more than 64 KB of LDS in the down kernel
     (2560, 64, 10, 768, 768, abi.GGUF_Q4_K), (2560, 64, 10, 768, 256, abi.GGUF_IQ2_XXS), (1280, 40, 4, 256, 768, abi.GGUF_Q4_K),
 ]
 
@@ -57,9 +58,10 @@ def test_decode_kernels_match_oracle_and_general_kernels(product, oracle, h, e, 
             print(f"  tokens={tokens}", flush=True)
             _, y, ids, w = layer.forward(x[:tokens])
             assert_parity(y, ids, w, want[0][:tokens], want[1][:tokens], want[2][:tokens], label=f"decode T={tokens}")
-        layer.force_general()
-        _, y, ids, w = layer.forward(x)
-        assert_parity(y, ids, w, *want, label="general kernels on a decode shape")
+        if (k * cfg.down_physical + s) * 4 <= 64 * 1024:   # the general kernels stage a token's activation rows in LDS
+            layer.force_general()
+            _, y, ids, w = layer.forward(x)
+            assert_parity(y, ids, w, *want, label="general kernels on a decode shape")
 
 
 # shapes the matrix-core prefill kernels cover (Q4_K or IQ2_XXS experts, widths in whole 256-blocks), more than 4 tokens
