@@ -242,8 +242,9 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
     ms_per_step = timing["median"]
     us_per_token = ms_per_step * 1e3 / tokens
     err_word = hip.from_device(hip.work_error_word(work), (1,), np.uint32)[0]
-    exact = C.c_uint32()
+    exact, exact_full = C.c_uint32(), C.c_uint32()
     hip.work_exact_rows(work, C.byref(exact))
+    hip.work_full_reroutes(work, C.byref(exact_full))
 
     # Per-kernel durations inside the dependent chain: the same plan with only the first 1, 2, ... kernel
     # groups of every forward; a group's duration is the difference between consecutive plans (it includes
@@ -361,7 +362,8 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
         "cpu_baseline": {"value": round(cpu_s / sample_tokens * 1e6, 1), "unit": "us/layer/token", "cores": 1,
                          "kind": kind, "sample": sample_text},
         "parity_on_sample": {"ids_equal": bool(ids_equal), "within_1e-3_abs_1e-4_rel": bool(within),
-                             "max_abs_err": max_abs, "error_word": int(err_word), "serial_order_reroutes": int(exact.value)},
+                             "max_abs_err": max_abs, "error_word": int(err_word), "serial_order_reroutes": int(exact.value),
+                             "of_those_all_logits_serially": int(exact_full.value)},
         "wall_ms_timed_loop": round(wall_ms, 2), "prep_s": round(prep_s, 1),
     }
 

@@ -93,6 +93,11 @@ const uint32_t *pf_hip_work_error_word(const PfHipWork *work);
 /* Number of tokens of the last forward whose routing was re-evaluated in the
  * reference's serial order because two candidate logits were too close. */
 int pf_hip_work_exact_rows(PfHipWork *work, uint32_t *count);
+/* Of those, the tokens that summing only the doubtful experts again did not settle (two of their
+ * probabilities within a few ulps without being equal, more than 64 doubtful experts, probabilities near the
+ * subnormals): all their logits were summed serially.  Kernels that re-route every flagged token that way
+ * (more than 1024 experts, the segment decode kernels) do not count here. */
+int pf_hip_work_full_reroutes(PfHipWork *work, uint32_t *count);
 
 /* The error word and the re-route counter accumulate over forwards (a forward only
  * enqueues kernels, so it can be captured into a graph); this clears both. */

@@ -141,6 +141,7 @@ class HipShim:
         bind("pf_hip_work_logits", vp, vp)
         bind("pf_hip_work_error_word", vp, vp)
         bind("pf_hip_work_exact_rows", C.c_int, vp, u32p)
+        bind("pf_hip_work_full_reroutes", C.c_int, vp, u32p)
         bind("pf_hip_work_clear_status", C.c_int, vp)
         bind("pf_hip_work_force_general", None, vp, C.c_int)
         bind("pf_hip_work_limit_kernels", None, vp, C.c_int)

@@ -473,10 +473,16 @@ extern "C" int pf_hip_work_exact_rows(PfHipWork *w, uint32_t *count) {
     return PF_HIP_OK;
 }
 
+extern "C" int pf_hip_work_full_reroutes(PfHipWork *w, uint32_t *count) {
+    if (!w || !count) return PF_HIP_E_ARGUMENT;
+    HIP_TRY(hipMemcpy(count, w->exact_rows + 1, 4, hipMemcpyDeviceToHost));
+    return PF_HIP_OK;
+}
+
 extern "C" int pf_hip_work_clear_status(PfHipWork *w) {
     if (!w) return PF_HIP_E_ARGUMENT;
     HIP_TRY(hipMemset(w->error_word, 0, 4));
-    HIP_TRY(hipMemset(w->exact_rows, 0, 4));
+    HIP_TRY(hipMemset(w->exact_rows, 0, 8));
     return PF_HIP_OK;
 }
 

@@ -24,6 +24,7 @@
 #include "pf_moe_internal.h"
 #include "pf_route_device.h"
 #include "pf_route_fast.h"
+#include "pf_route_fix.h"
 
 #ifdef PF_TIMING
 #define STAMP(i) do { if (blockIdx.x == PF_TIMING && threadIdx.x == 0) reinterpret_cast<unsigned long long *>(a.exact_rows + 2)[i] = wall_clock64(); } while (0)
@@ -1059,6 +1060,20 @@ __device__ __forceinline__ void q4t_at_token(PfKernelArgs &a, int t) {
     a.aimg += (size_t)t * (a.top_k + 1) * pf_image2_words(widest);
 }
 
+// The routing wave sums the doubtful experts again in the reference's order, a second wave fetches their rows ahead,
+// the others wait (pf_route_fix.h).  Not inlined: the rare path's registers (the rows' pieces on their way) must not
+// weigh on the kernel's; the LDS is named here again so that its accesses stay LDS instructions.
+template <int NPL>
+__device__ __attribute__((noinline)) void q4t_route_fix(const float *router, const float *x, const float *logits, const float *ssq, int E,
+                                                        int K, bool norm, int H, int scratch_at, RouteLds *R) {
+    extern __shared__ int lds[];
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = pf_lane();
+    const int how = pf_route_fix_block<NPL, 2, false>(router, x, logits, ssq, E, K, norm, H, reinterpret_cast<float *>(lds) + scratch_at, R->ids,
+                                               R->weights, wave, lane);
+    if (threadIdx.x == 0) { R->close_mask = (uint32_t)how; R->bad = R->nonfinite[0]; }
+    __syncthreads();
+}
+
 // FMT: format of the routed gate and up tensors, FMTS: of the shared expert's (the same, or the profiles' Q8_0)
 template <int NPL, int FMT, int FMTS>
 __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) {
@@ -1135,7 +1150,8 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
     uint32_t e = early;
     if (!shared) {
         if (R.close[0]) {   // the same for every thread of every workgroup: the inputs are the same
-            route_finish<1>(a, &R, scratch);
+            q4t_route_fix<NPL>(reinterpret_cast<const float *>(a.w[0]), a.x, a.logits, a.logit_ssq, E, K, norm, H,
+                               (int)(scratch - reinterpret_cast<float *>(lds)), &R);
         } else if (threadIdx.x == 0) {
             R.close_mask = 0;
             R.bad = R.nonfinite[0];
@@ -1164,6 +1180,7 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
                 if (gridDim.y == 1) a.uniq[0] = K;
                 if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
                 if (R.close_mask) atomicAdd(a.exact_rows, 1u);
+                if (R.close_mask == 2u) atomicAdd(a.exact_rows + 1, 1u);   // settled the long way
             }
         }
         if (e >= (uint32_t)E) {   // only reachable with nonfinite logits
@@ -1212,7 +1229,7 @@ static void launch_gate_up_q4t(const PfKernelArgs &a, int tokens, hipStream_t st
     const int routed_blocks = K * (I / 32);
     const dim3 g1(routed_blocks + Is / 32, tokens);
     const int all = (E + 63) / 64;
-    const size_t lds = (size_t)table_words<FMT>() * 4 + (size_t)15 * 64 * 4 + ((size_t)H + 3 * (size_t)E) * 4;
+    const size_t lds = (size_t)table_words<FMT>() * 4 + (size_t)15 * 64 * 4 + pf_route_fix_lds_floats(H, E) * 4;
     if (all <= 1) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<1, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
     else if (all <= 2) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<2, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
     else if (all <= 4) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<4, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);

@@ -9,6 +9,7 @@
 #include "pf_moe_internal.h"
 #include "pf_route_device.h"
 #include "pf_route_fast.h"
+#include "pf_route_fix.h"
 
 #define ROUTE_MAX_FAST_EXPERTS 1024
 
@@ -148,6 +149,27 @@ __global__ void __launch_bounds__(64) pf_k_route_fix_select(PfKernelArgs a) {
     }
 }
 
+// The listed tokens, one wave each: only the experts whose order is in doubt are summed again in serial order
+// (pf_route_fix.h); a token that this does not settle is routed the long way by the same wave.  exact_rows[0]
+// counts the listed tokens, exact_rows[1] those that went the long way.
+template <int NPL>
+__global__ void __launch_bounds__(128) pf_k_route_fix(PfKernelArgs a) {
+    extern __shared__ float fix_floats[];
+    const int E = a.experts, K = a.top_k, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t listed = a.route_flags[0];
+    for (uint32_t item = blockIdx.x; item < listed; item += gridDim.x) {
+        const int t = (int)a.route_flags[1 + item];
+        const int how = pf_route_fix_block<NPL, 4, true>(reinterpret_cast<const float *>(a.w[0]), a.x + (size_t)t * a.x_pitch,
+                                                   a.logits + (size_t)t * E, a.logit_ssq + (size_t)t * E, E, K, a.norm_topk != 0,
+                                                   a.hidden, fix_floats, a.ids + (size_t)t * K, a.route_weights + (size_t)t * K,
+                                                   wave, lane);
+        if (threadIdx.x == 0) {
+            atomicAdd(a.exact_rows, 1u);
+            if (how == 2) atomicAdd(a.exact_rows + 1, 1u);
+        }
+    }
+}
+
 // Every token through the exact path (expert counts the fast kernel cannot hold): the full list.
 __global__ void pf_k_flag_all(uint32_t *list, int n) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -164,6 +186,18 @@ void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     else if (npl <= 4) hipLaunchKernelGGL(pf_k_route_fast<4>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 8) hipLaunchKernelGGL(pf_k_route_fast<8>, dim3(tokens), dim3(64), 0, stream, a);
     else hipLaunchKernelGGL(pf_k_route_fast<16>, dim3(tokens), dim3(64), 0, stream, a);
+    // the listed tokens are few: a fixed number of workgroups walks the list
+    const int workers = tokens < 256 ? tokens : 256;
+    if (a.experts <= ROUTE_MAX_FAST_EXPERTS && a.top_k < PF_WAVE - 1) {
+        const size_t lds = pf_route_fix_lds_floats(a.hidden, a.experts) * sizeof(float);
+        if (npl <= 1) hipLaunchKernelGGL(pf_k_route_fix<1>, dim3(workers), dim3(128), lds, stream, a);
+        else if (npl <= 2) hipLaunchKernelGGL(pf_k_route_fix<2>, dim3(workers), dim3(128), lds, stream, a);
+        else if (npl <= 4) hipLaunchKernelGGL(pf_k_route_fix<4>, dim3(workers), dim3(128), lds, stream, a);
+        else if (npl <= 8) hipLaunchKernelGGL(pf_k_route_fix<8>, dim3(workers), dim3(128), lds, stream, a);
+        else hipLaunchKernelGGL(pf_k_route_fix<16>, dim3(workers), dim3(128), lds, stream, a);
+        return;
+    }
+    // more experts than a wave's registers hold: every token is listed and all its logits are summed serially
     const size_t fix_lds = (size_t)FIX_RING * FIX_BATCH * 1024 + (size_t)a.hidden * sizeof(float);
     static bool configured = false;   // more than the default 64 KB of dynamic LDS
     if (!configured) {
@@ -171,8 +205,6 @@ void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         configured = true;
     }
-    // the listed tokens are few: a fixed number of workgroups walks the list
-    const int workers = tokens < 256 ? tokens : 256;
     hipLaunchKernelGGL(pf_k_route_fix_logits, dim3(workers, (a.experts + PF_WAVE - 1) / PF_WAVE), dim3(3 * PF_WAVE), fix_lds, stream, a);
     hipLaunchKernelGGL(pf_k_route_fix_select, dim3(workers), dim3(PF_WAVE), 3 * (size_t)a.experts * sizeof(float), stream,
                        a);

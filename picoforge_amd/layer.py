@@ -175,6 +175,12 @@ class MoeLayer:
         self.api.hip.work_exact_rows(self.api.device_work(self.work), C.byref(count))
         return count.value
 
+    def full_reroutes(self):
+        """Of the re-routed tokens, those whose every logit was summed serially (see pf_hip_work_full_reroutes)."""
+        count = C.c_uint32()
+        self.api.hip.work_full_reroutes(self.api.device_work(self.work), C.byref(count))
+        return count.value
+
     def reset(self):
         return self.api.work_reset(self.work, C.byref(self.err))
 

@@ -213,6 +213,46 @@ def test_close_logits_are_rerouted_in_serial_order(product, oracle):
             assert layer.serial_order_reroutes() >= 1
 
 
+@pytest.mark.parametrize("norm", [True, False])
+def test_many_near_ties_are_settled_by_the_doubtful_experts_alone(product, oracle, norm):
+    """Router rows in pairs that differ by a few ulps in a few places: nearly every token has logits closer than the
+    guard's tolerance among its best, some with equal probabilities (the lower id wins), some with probabilities a
+    few ulps apart (all logits are then summed serially).  Ids must match the CPU path bit for bit on the decode
+    kernels (1 and 16 tokens a call), the prefill kernels and the general ones."""
+    cfg = abi.moe_config(512, 64, 6, 256, 256, norm=norm)
+    tokens = 320
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, tokens, seed=2024)
+    router = weights.raw[0].view(np.float32).reshape(64, 512)
+    rng = np.random.default_rng(7)
+    for pair in range(32):
+        twin = router[2 * pair].copy()
+        for col in rng.choice(512, size=int(rng.integers(0, 4)), replace=False):   # 0 places: an exact twin
+            for _ in range(int(rng.integers(1, 4))):
+                twin[col] = np.nextafter(twin[col], np.float32(rng.choice([-10.0, 10.0])))
+        router[2 * pair + 1] = twin
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, tokens) as layer:
+        for first in range(0, 24):                          # one token a call
+            _, y, ids, w = layer.forward(x[first:first + 1])
+            assert_parity(y, ids, w, want[0][first:first + 1], want[1][first:first + 1], want[2][first:first + 1],
+                          label=f"near ties, token {first} alone")
+        for first in range(0, tokens, 16):                  # short batches on the decode kernels
+            _, y, ids, w = layer.forward(x[first:first + 16])
+            assert_parity(y, ids, w, want[0][first:first + 16], want[1][first:first + 16], want[2][first:first + 16],
+                          label=f"near ties, tokens {first}..{first + 15}")
+        decode_reroutes, decode_full = layer.serial_order_reroutes(), layer.full_reroutes()
+        _, y, ids, w = layer.forward(x)                      # one chunk on the prefill kernels
+        assert_parity(y, ids, w, *want, label="near ties, prefill chunk")
+        reroutes, full = layer.serial_order_reroutes() - decode_reroutes, layer.full_reroutes() - decode_full
+        print(f"  decode calls: {decode_reroutes} re-routed, {decode_full} the long way; chunk: {reroutes} of {tokens} "
+              f"re-routed, {full} the long way", flush=True)
+        assert reroutes > tokens // 2, "the case must be full of near ties"
+        assert full < reroutes, "the doubtful experts alone must settle some tokens"
+        layer.force_general()
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y, ids, w, *want, label="near ties, general kernels")
+
+
 def test_nonfinite_activation_is_reported_and_sticky_until_reset(product):
     cfg = abi.moe_config(512, 32, 6, 256, 256)
     weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 2, seed=6)
