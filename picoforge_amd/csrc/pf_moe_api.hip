@@ -220,7 +220,7 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
         }
         m->total_bytes += m->bytes[a];
     }
-    {   // router copy in 64-expert slabs for the serial-order re-routing
+    if (pf_route_needs_slabs((int)E, (int)desc->top_k)) {   // router copy in 64-expert slabs: only where every token is routed in serial order
         const size_t slab_floats = pf_router_slab_floats((int)E, (int)h);
         hipError_t e = hipMalloc((void **)&m->router_t, slab_floats * sizeof(float));
         if (e == hipSuccess) {

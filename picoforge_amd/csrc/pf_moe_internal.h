@@ -164,6 +164,9 @@ void pf_launch_exact_combine(const float *d_down, const uint64_t *d_pair_to_row,
                              uint32_t *d_error, hipStream_t stream);
 // pf_moe_decode.hip
 bool pf_decode_supported(const PfHipMoeDesc &d);
+// more experts (or slots) than the fast routing holds in a wave's registers: every token's logits are summed serially
+// from the router's slab copy (pf_moe_route.hip)
+bool pf_route_needs_slabs(int experts, int top_k);
 int pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const q4k_tiled[8], const uint8_t *const iq2_tiled[8],
                          const uint8_t *const q8_tiled[8]);
 void pf_launch_iq2_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8_t *d_dst, size_t rows, int blocks_per_row,

@@ -177,9 +177,11 @@ __global__ void pf_k_flag_all(uint32_t *list, int n) {
     if (i < n) list[1 + i] = (uint32_t)i;
 }
 
+bool pf_route_needs_slabs(int experts, int top_k) { return experts > ROUTE_MAX_FAST_EXPERTS || top_k >= PF_WAVE - 1; }
+
 void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     const int npl = (a.experts + PF_WAVE - 1) / PF_WAVE;
-    if (a.experts > ROUTE_MAX_FAST_EXPERTS || a.top_k >= PF_WAVE - 1)   // the fast routing keeps top_k + 2 keys, one per lane
+    if (pf_route_needs_slabs(a.experts, a.top_k))   // the fast routing keeps top_k + 2 keys, one per lane
         hipLaunchKernelGGL(pf_k_flag_all, dim3((tokens + 255) / 256), dim3(256), 0, stream, a.route_flags, tokens);
     else if (npl <= 1) hipLaunchKernelGGL(pf_k_route_fast<1>, dim3(tokens), dim3(64), 0, stream, a);
     else if (npl <= 2) hipLaunchKernelGGL(pf_k_route_fast<2>, dim3(tokens), dim3(64), 0, stream, a);
@@ -188,7 +190,7 @@ void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     else hipLaunchKernelGGL(pf_k_route_fast<16>, dim3(tokens), dim3(64), 0, stream, a);
     // the listed tokens are few: a fixed number of workgroups walks the list
     const int workers = tokens < 256 ? tokens : 256;
-    if (a.experts <= ROUTE_MAX_FAST_EXPERTS && a.top_k < PF_WAVE - 1) {
+    if (!pf_route_needs_slabs(a.experts, a.top_k)) {
         const size_t lds = pf_route_fix_lds_floats(a.hidden, a.experts) * sizeof(float);
         if (npl <= 1) hipLaunchKernelGGL(pf_k_route_fix<1>, dim3(workers), dim3(128), lds, stream, a);
         else if (npl <= 2) hipLaunchKernelGGL(pf_k_route_fix<2>, dim3(workers), dim3(128), lds, stream, a);

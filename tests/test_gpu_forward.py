@@ -20,6 +20,7 @@ SMALL = [
     (512, 32, 6, 256, 512, abi.GGUF_Q4_K, 5),
     (256, 16, 4, 256, 256, abi.GGUF_IQ2_XXS, 7),
     (768, 24, 3, 512, 256, abi.GGUF_IQ2_XXS, 4),
+    (64, 1088, 3, 24, 12, abi.GGUF_F32, 6),       # more experts than a wave's registers hold: every token routed in serial order
 ]
 
 
