@@ -219,7 +219,8 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
                 "median_tokens_per_expert": float(np.median(load)), "chunks": n_inputs}
     elif tokens == 1:
         n_inputs = max(1, min(steps, 64))       # a plan replays one graph of 64 forwards: 64 inputs = 1.5 GB of weights touched, far beyond the caches
-        x, info = workloads.decode_tokens(weights, n_inputs, seed=args.seed)
+        x, info = workloads.decode_tokens(weights, n_inputs, seed=args.seed, min_margin=args.margin_window[0],
+                                          max_margin=args.margin_window[1])
         x = x.reshape(n_inputs, 1, cfg.hidden_size)
         unique = float(cfg.top_k)
     else:
@@ -331,6 +332,9 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
 
     traffic, traffic_from = measured_traffic(name)
     margins = "; top-11 logit margins >= 1e-3" if not prefill else ""
+    if tokens == 1 and args.margin_window != (1e-3, None):
+        lo, hi = args.margin_window
+        margins = f"; top-11 logit margins in [{lo:g}, {'inf' if hi is None else format(hi, 'g')})"
     whole = alg_bytes / (ms_per_step * 1e-3) / 1e9
     return {
         "metric": "moe_decode_us_per_layer_token" if not prefill else "moe_prefill_us_per_layer_token",
@@ -617,10 +621,16 @@ def main():
                          "under a profiler, which records the kernels' durations itself")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="also launch a plain copy kernel of this many MiB three times (byte-counter calibration)")
+    ap.add_argument("--margin-window", default="1e-3,inf", metavar="LO,HI",
+                    help="one-token decode workloads: keep the seeded tokens whose closest pair among the top-(k+1) router "
+                         "logits is at least LO and less than HI apart (default 1e-3,inf: no token is routed again in "
+                         "serial order; 0,inf: every drawn token; 0,2e-5: only tokens that are)")
     ap.add_argument("--dims", default=None, metavar="H,E,K,I,S,P",
                     help="with --workload NAME: the layer's shape instead of the workload's own (hidden, experts, top_k, "
                          "intermediate, shared intermediate, stored width of the down projection)")
     args = ap.parse_args()
+    lo, hi = args.margin_window.split(",")
+    args.margin_window = (float(lo), None if hi.strip() in ("inf", "") else float(hi))
     if args.dims:
         if args.workload == "all":
             sys.exit("--dims needs --workload NAME")

@@ -1060,16 +1060,16 @@ __device__ __forceinline__ void q4t_at_token(PfKernelArgs &a, int t) {
     a.aimg += (size_t)t * (a.top_k + 1) * pf_image2_words(widest);
 }
 
-// The routing wave sums the doubtful experts again in the reference's order, a second wave fetches their rows ahead,
-// the others wait (pf_route_fix.h).  Not inlined: the rare path's registers (the rows' pieces on their way) must not
-// weigh on the kernel's; the LDS is named here again so that its accesses stay LDS instructions.
+// The workgroup sums the doubtful experts again in the reference's order, a wave each (pf_route_fix.h).  Not inlined:
+// the rare path's registers (a router row's products) must not weigh on the kernel's; the LDS is named here again so
+// that its accesses stay LDS instructions.
 template <int NPL>
-__device__ __attribute__((noinline)) void q4t_route_fix(const float *router, const float *x, const float *logits, const float *ssq, int E,
+__device__ __forceinline__ void q4t_route_fix(const float *router, const float *x, const float *logits, const float *ssq, int E,
                                                         int K, bool norm, int H, int scratch_at, RouteLds *R) {
     extern __shared__ int lds[];
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = pf_lane();
-    const int how = pf_route_fix_block<NPL, 2, false>(router, x, logits, ssq, E, K, norm, H, reinterpret_cast<float *>(lds) + scratch_at, R->ids,
-                                               R->weights, wave, lane);
+    const int how = pf_route_fix_block<NPL>(router, x, logits, ssq, E, K, norm, H, reinterpret_cast<float *>(lds) + scratch_at, R->ids,
+                                            R->weights, wave, lane);
     if (threadIdx.x == 0) { R->close_mask = (uint32_t)how; R->bad = R->nonfinite[0]; }
     __syncthreads();
 }
@@ -1223,6 +1223,17 @@ static bool q4t_gate_up_applies(const PfKernelArgs &a) {
            a.top_k < a.experts && a.top_k <= 15 && a.experts <= 1024;
 }
 
+template <int NPL, int FMT, int FMTS>
+static void launch_gate_up_q4t_lists(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks) {
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS (the re-route's chunk buffers)
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up_q4t<NPL, FMT, FMTS>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);   // the kernel has static LDS too
+        configured = true;
+    }
+    hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<NPL, FMT, FMTS>), grid, dim3(1024), lds, stream, a, routed_blocks);
+}
+
 template <int FMT, int FMTS>
 static void launch_gate_up_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
@@ -1230,11 +1241,11 @@ static void launch_gate_up_q4t(const PfKernelArgs &a, int tokens, hipStream_t st
     const dim3 g1(routed_blocks + Is / 32, tokens);
     const int all = (E + 63) / 64;
     const size_t lds = (size_t)table_words<FMT>() * 4 + (size_t)15 * 64 * 4 + pf_route_fix_lds_floats(H, E) * 4;
-    if (all <= 1) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<1, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 2) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<2, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 4) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<4, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else if (all <= 8) hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<8, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
-    else hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<16, FMT, FMTS>), g1, dim3(1024), lds, stream, a, routed_blocks);
+    if (all <= 1) launch_gate_up_q4t_lists<1, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
+    else if (all <= 2) launch_gate_up_q4t_lists<2, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
+    else if (all <= 4) launch_gate_up_q4t_lists<4, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
+    else if (all <= 8) launch_gate_up_q4t_lists<8, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
+    else launch_gate_up_q4t_lists<16, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
 }
 
 // ---- kernel 3: down products and the combine ---------------------------------------------------

@@ -153,16 +153,16 @@ __global__ void __launch_bounds__(64) pf_k_route_fix_select(PfKernelArgs a) {
 // (pf_route_fix.h); a token that this does not settle is routed the long way by the same wave.  exact_rows[0]
 // counts the listed tokens, exact_rows[1] those that went the long way.
 template <int NPL>
-__global__ void __launch_bounds__(128) pf_k_route_fix(PfKernelArgs a) {
+__global__ void __launch_bounds__(1024) pf_k_route_fix(PfKernelArgs a) {
     extern __shared__ float fix_floats[];
     const int E = a.experts, K = a.top_k, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t listed = a.route_flags[0];
     for (uint32_t item = blockIdx.x; item < listed; item += gridDim.x) {
         const int t = (int)a.route_flags[1 + item];
-        const int how = pf_route_fix_block<NPL, 4, true>(reinterpret_cast<const float *>(a.w[0]), a.x + (size_t)t * a.x_pitch,
-                                                   a.logits + (size_t)t * E, a.logit_ssq + (size_t)t * E, E, K, a.norm_topk != 0,
-                                                   a.hidden, fix_floats, a.ids + (size_t)t * K, a.route_weights + (size_t)t * K,
-                                                   wave, lane);
+        const int how = pf_route_fix_block<NPL>(reinterpret_cast<const float *>(a.w[0]), a.x + (size_t)t * a.x_pitch,
+                                                a.logits + (size_t)t * E, a.logit_ssq + (size_t)t * E, E, K, a.norm_topk != 0,
+                                                a.hidden, fix_floats, a.ids + (size_t)t * K, a.route_weights + (size_t)t * K,
+                                                wave, lane);
         if (threadIdx.x == 0) {
             atomicAdd(a.exact_rows, 1u);
             if (how == 2) atomicAdd(a.exact_rows + 1, 1u);
@@ -175,6 +175,17 @@ __global__ void pf_k_flag_all(uint32_t *list, int n) {
     int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i == 0) list[0] = (uint32_t)n;
     if (i < n) list[1 + i] = (uint32_t)i;
+}
+
+template <int NPL>
+static void launch_route_fix(const PfKernelArgs &a, int workers, size_t lds, hipStream_t stream) {
+    static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_route_fix<NPL>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  144 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL(pf_k_route_fix<NPL>, dim3(workers), dim3(1024), lds, stream, a);
 }
 
 bool pf_route_needs_slabs(int experts, int top_k) { return experts > ROUTE_MAX_FAST_EXPERTS || top_k >= PF_WAVE - 1; }
@@ -192,11 +203,11 @@ void pf_launch_route(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     const int workers = tokens < 256 ? tokens : 256;
     if (!pf_route_needs_slabs(a.experts, a.top_k)) {
         const size_t lds = pf_route_fix_lds_floats(a.hidden, a.experts) * sizeof(float);
-        if (npl <= 1) hipLaunchKernelGGL(pf_k_route_fix<1>, dim3(workers), dim3(128), lds, stream, a);
-        else if (npl <= 2) hipLaunchKernelGGL(pf_k_route_fix<2>, dim3(workers), dim3(128), lds, stream, a);
-        else if (npl <= 4) hipLaunchKernelGGL(pf_k_route_fix<4>, dim3(workers), dim3(128), lds, stream, a);
-        else if (npl <= 8) hipLaunchKernelGGL(pf_k_route_fix<8>, dim3(workers), dim3(128), lds, stream, a);
-        else hipLaunchKernelGGL(pf_k_route_fix<16>, dim3(workers), dim3(128), lds, stream, a);
+        if (npl <= 1) launch_route_fix<1>(a, workers, lds, stream);
+        else if (npl <= 2) launch_route_fix<2>(a, workers, lds, stream);
+        else if (npl <= 4) launch_route_fix<4>(a, workers, lds, stream);
+        else if (npl <= 8) launch_route_fix<8>(a, workers, lds, stream);
+        else launch_route_fix<16>(a, workers, lds, stream);
         return;
     }
     // more experts than a wave's registers hold: every token is listed and all its logits are summed serially

@@ -51,17 +51,21 @@ def top_margins(logits, k):
     return (top[:, :-1] - top[:, 1:]).min(axis=1)
 
 
-def decode_tokens(weights, count, seed, min_margin=1e-3):
+def decode_tokens(weights, count, seed, min_margin=1e-3, max_margin=None):
     """`count` RMS-normalised N(0,1) activations whose sorted top-(k+1) router logits are at
     least min_margin apart (drawn, then kept or rejected), so expert selection does not depend
-    on the order a logit is summed in."""
+    on the order a logit is summed in.  max_margin keeps only tokens with a closer pair than that
+    (tokens the kernels route again in the reference's order)."""
     synth, cfg = Synth(), weights.cfg
     kept, draw, drawn = [], 0, 0
     while sum(len(k) for k in kept) < count:
         x = rms_normalise(synth.normal((max(1024, count // 4), cfg.hidden_size), seed * 1000 + draw))
         draw += 1
         drawn += len(x)
-        ok = top_margins(router_logits64(weights, x), cfg.top_k) >= min_margin
+        margins = top_margins(router_logits64(weights, x), cfg.top_k)
+        ok = margins >= min_margin
+        if max_margin is not None:
+            ok &= margins < max_margin
         kept.append(x[ok])
     x = np.concatenate(kept)[:count]
     return np.ascontiguousarray(x), {"drawn": drawn, "kept_fraction": float(sum(len(k) for k in kept) / drawn)}
