@@ -119,9 +119,9 @@ __global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_
 // The same for rows of at most 512 values (the activation rows): one wave per row, four rows per workgroup, the row
 // read once -- a lane keeps its eight values between the maximum and the conversion.  With a workgroup per row three
 // of its four waves only took part in the maximum.
-__global__ void __launch_bounds__(256) pf_k_rows_to_half_short(const float *src, size_t src_pitch, int cols, size_t rows, half_t *dst,
-                                                               float *scale_out, float *max2_out, uint32_t *error_word) {
-    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+__device__ __forceinline__ void rows_to_half_short(size_t block, const float *src, size_t src_pitch, int cols, size_t rows, half_t *dst,
+                                                   float *scale_out, float *max2_out, uint32_t *error_word) {
+    const size_t row = block * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
     const int j = pf_lane();
     const bool mine = j < cols / 8;
@@ -167,6 +167,20 @@ __global__ void __launch_bounds__(256) pf_k_rows_to_half_short(const float *src,
         scale_out[row] = scale;
         if (max2_out) max2_out[row] = m * m;
     }
+}
+
+__global__ void __launch_bounds__(256) pf_k_rows_to_half_short(const float *src, size_t src_pitch, int cols, size_t rows, half_t *dst,
+                                                               float *scale_out, float *max2_out, uint32_t *error_word) {
+    rows_to_half_short(blockIdx.x, src, src_pitch, cols, rows, dst, scale_out, max2_out, error_word);
+}
+
+// Two matrices of short rows in one launch (the routed and the shared activation rows): workgroups [0, blocks_a) take
+// the first, the others the second.
+__global__ void __launch_bounds__(256) pf_k_rows_to_half_short2(const float *src_a, int cols_a, size_t rows_a, half_t *dst_a, float *scale_a,
+                                                                unsigned blocks_a, const float *src_b, int cols_b, size_t rows_b,
+                                                                half_t *dst_b, float *scale_b, uint32_t *error_word) {
+    if (blockIdx.x < blocks_a) rows_to_half_short(blockIdx.x, src_a, (size_t)cols_a, cols_a, rows_a, dst_a, scale_a, nullptr, error_word);
+    else rows_to_half_short(blockIdx.x - blocks_a, src_b, (size_t)cols_b, cols_b, rows_b, dst_b, scale_b, nullptr, error_word);
 }
 
 static void launch_rows_to_half(const float *src, size_t src_pitch, int cols, size_t rows, half_t *dst, float *scale_out,
@@ -1263,9 +1277,11 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     if (last < 2) return;
     // stage 2: routes and grouping
     pf_launch_route(a, tokens, stream);
-    hipLaunchKernelGGL(pf_k_pf_count, dim3((P + 255) / 256), dim3(256), 0, stream, a.ids, P, E, a.counts);
-    hipLaunchKernelGGL(pf_k_pf_scan_tiles, dim3(1), dim3(256), 0, stream, a.counts, E, tokens, a.offsets, a.tiles);
-    pf_launch_group_place(a.ids, P, E, a.offsets, a.pair_to_row, a.row_to_pair, stream);
+    if (!pf_launch_group_fused(a.ids, P, E, tokens, a.offsets, a.tiles, a.pair_to_row, a.row_to_pair, stream)) {
+        hipLaunchKernelGGL(pf_k_pf_count, dim3((P + 255) / 256), dim3(256), 0, stream, a.ids, P, E, a.counts);
+        hipLaunchKernelGGL(pf_k_pf_scan_tiles, dim3(1), dim3(256), 0, stream, a.counts, E, tokens, a.offsets, a.tiles);
+        pf_launch_group_place(a.ids, P, E, a.offsets, a.pair_to_row, a.row_to_pair, stream);
+    }
     if (last < 3) return;
     // stage 3: gate/up + SwiGLU, then fp16 parts of the activation rows
     // the ring kernel takes the items whose tensors are in the routed gate's format, the plain kernel the rest
@@ -1277,8 +1293,15 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     else launch_gemm<PF_GEMM_GATE_UP, PF_Q4_K>(a, tokens, (gi + 32 * NW - 1) / (32 * NW), stream);
     // only the shared expert's tiles (tokens / 32 of them) are left for this launch: columns split over the waves
     if (a.type[4] != ring_fmt) launch_gemm_plain<PF_GEMM_GATE_UP>(a, tokens, tile_cap, (gi + 31) / 32, 1, stream);
-    launch_rows_to_half(a.act, (size_t)I, I, (size_t)P, (half_t *)a.act16, a.act_scale, nullptr, a.error_word, stream);
-    launch_rows_to_half(a.shared_act, (size_t)Is, Is, (size_t)tokens, (half_t *)a.sact16, a.sact_scale, nullptr, a.error_word, stream);
+    if (I <= 512 && Is <= 512 && P > 0 && tokens > 0) {
+        const unsigned blocks_a = (unsigned)((P + 3) / 4), blocks_b = (unsigned)((tokens + 3) / 4);
+        hipLaunchKernelGGL(pf_k_rows_to_half_short2, dim3(blocks_a + blocks_b), dim3(256), 0, stream, a.act, I, (size_t)P,
+                           (half_t *)a.act16, a.act_scale, blocks_a, a.shared_act, Is, (size_t)tokens, (half_t *)a.sact16, a.sact_scale,
+                           a.error_word);
+    } else {
+        launch_rows_to_half(a.act, (size_t)I, I, (size_t)P, (half_t *)a.act16, a.act_scale, nullptr, a.error_word, stream);
+        launch_rows_to_half(a.shared_act, (size_t)Is, Is, (size_t)tokens, (half_t *)a.sact16, a.sact_scale, nullptr, a.error_word, stream);
+    }
     if (last < 4) return;
     // stage 4: down and combine
     if (a.type[3] == ring_fmt || a.type[6] == ring_fmt) {

@@ -375,6 +375,131 @@ void pf_launch_group_place(const uint32_t *d_ids, int pairs, int experts, const 
                        d_pair_to_row, d_row_to_pair);
 }
 
+// ---- grouping in one launch (the prefill path) ---------------------------------------------------------
+// Every workgroup stages all ids in LDS, counts them there (LDS atomics), scans the counts, and its four waves place
+// their four experts' pairs as pf_k_group_place does; workgroup 0 also writes offsets[E + 1] and the row tiles
+// (tiles[0] = count, tiles[1 + i] = expert | tile index << 16; the shared expert = expert E with every token), as
+// pf_k_pf_scan_tiles does.  The histogram and the scan are repeated by every workgroup: a few microseconds of LDS
+// work against two kernel boundaries.
+#define GROUP_FUSED_MAX_PAIRS 32768
+#define GROUP_FUSED_MAX_EXPERTS 2047
+__global__ void __launch_bounds__(256) pf_k_group_fused(const uint32_t *ids, int pairs, int E, int tokens, uint32_t *offsets,
+                                                        uint32_t *tiles, uint32_t *pair_to_row, uint32_t *row_to_pair) {
+    extern __shared__ __align__(16) uint32_t fused_lds[];
+    __shared__ uint32_t rows_before[256], tiles_before[256];
+    const int padded = (pairs + 511) & ~511, tid = threadIdx.x, lane = pf_lane();
+    uint32_t *staged = fused_lds, *counts = staged + padded, *starts = counts + (E + 1);
+    // all of a thread's loads are requested before the first is stored (pairs on a 16-byte boundary of ids; the
+    // ragged end is read id by id); beyond the pairs: no expert
+    for (int i0 = 4 * tid; i0 < padded; i0 += 4 * 256 * 8) {
+        uint4 held[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = i0 + 4 * 256 * j;
+            uint4 v = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+            if (i + 4 <= pairs) {
+                v = *reinterpret_cast<const uint4 *>(ids + i);
+            } else if (i < pairs) {
+                v.x = ids[i];
+                if (i + 1 < pairs) v.y = ids[i + 1];
+                if (i + 2 < pairs) v.z = ids[i + 2];
+            }
+            held[j] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int i = i0 + 4 * 256 * j;
+            if (i < padded) *reinterpret_cast<uint4 *>(staged + i) = held[j];
+        }
+    }
+    for (int e = tid; e <= E; e += 256) counts[e] = 0;
+    __syncthreads();
+    for (int i = tid; i < pairs; i += 256) {
+        const uint32_t id = staged[i];
+        if (id < (uint32_t)E) atomicAdd(&counts[id], 1u);
+    }
+    __syncthreads();
+    // exclusive scan of the counts (rows) and of the row-tile counts, thread t owning `per` consecutive experts
+    const int per = (E + 1 + 255) / 256, lo = tid * per, hi = min(E + 1, lo + per);
+    uint32_t rows = 0, ntiles = 0;
+    for (int e = lo; e < hi; e++) {
+        const uint32_t c = e < E ? counts[e] : (uint32_t)tokens;
+        if (e < E) rows += c;
+        ntiles += (c + 31u) / 32u;
+    }
+    rows_before[tid] = rows;
+    tiles_before[tid] = ntiles;
+    __syncthreads();
+    uint32_t run_rows = rows, run_tiles = ntiles;
+    for (int d = 1; d < 256; d <<= 1) {
+        const uint32_t add_rows = tid >= d ? rows_before[tid - d] : 0u, add_tiles = tid >= d ? tiles_before[tid - d] : 0u;
+        __syncthreads();
+        run_rows += add_rows;
+        run_tiles += add_tiles;
+        rows_before[tid] = run_rows;
+        tiles_before[tid] = run_tiles;
+        __syncthreads();
+    }
+    const bool writer = blockIdx.x == 0;
+    if (writer && tid == 255) {
+        offsets[E] = run_rows;
+        tiles[0] = run_tiles;
+    }
+    uint32_t row = run_rows - rows, at = run_tiles - ntiles;
+    for (int e = lo; e < hi; e++) {
+        const uint32_t c = e < E ? counts[e] : (uint32_t)tokens, n = (c + 31u) / 32u;
+        if (e < E) {
+            starts[e] = row;
+            if (writer) offsets[e] = row;
+            row += c;
+        }
+        if (writer)
+            for (uint32_t i = 0; i < n; i++) tiles[1 + at + i] = (uint32_t)e | (i << 16);
+        at += n;
+    }
+    __syncthreads();
+    // placement: one wave per expert walks the pairs in order (rank = earlier pairs of the same expert)
+    const int e = blockIdx.x * 4 + (tid >> 6);
+    if (e >= E || counts[e] == 0) return;
+    uint32_t base = starts[e];
+    const unsigned long long below = (1ull << lane) - 1ull;
+    auto place = [&](const uint4 &v, int p0) {   // 256 pairs, lane l holds pairs 4l .. 4l + 3 of them
+        const bool h0 = v.x == (uint32_t)e, h1 = v.y == (uint32_t)e, h2 = v.z == (uint32_t)e, h3 = v.w == (uint32_t)e;
+        const int mine = (int)h0 + (int)h1 + (int)h2 + (int)h3;
+        const unsigned long long any = __ballot(mine != 0);
+        if (!any) return;
+        // pairs of lower lanes come first, then this lane's own earlier ones
+        const unsigned long long m0 = __ballot(h0), m1 = __ballot(h1), m2 = __ballot(h2), m3 = __ballot(h3);
+        uint32_t r = base + __popcll(m0 & below) + __popcll(m1 & below) + __popcll(m2 & below) + __popcll(m3 & below);
+        const int p = p0 + 4 * lane;
+        if (h0) { pair_to_row[p] = r; row_to_pair[r] = (uint32_t)p; r++; }
+        if (h1) { pair_to_row[p + 1] = r; row_to_pair[r] = (uint32_t)(p + 1); r++; }
+        if (h2) { pair_to_row[p + 2] = r; row_to_pair[r] = (uint32_t)(p + 2); r++; }
+        if (h3) { pair_to_row[p + 3] = r; row_to_pair[r] = (uint32_t)(p + 3); }
+        base += __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
+    };
+    const uint4 *quads = reinterpret_cast<const uint4 *>(staged);
+    for (int p0 = 0; p0 < padded; p0 += 512) {
+        const uint4 va = quads[p0 / 4 + lane], vb = quads[p0 / 4 + 64 + lane];
+        place(va, p0);
+        place(vb, p0 + 256);
+    }
+}
+
+bool pf_launch_group_fused(const uint32_t *d_ids, int pairs, int experts, int tokens, uint32_t *d_offsets, uint32_t *d_tiles,
+                           uint32_t *d_pair_to_row, uint32_t *d_row_to_pair, hipStream_t stream) {
+    if (pairs <= 0 || pairs > GROUP_FUSED_MAX_PAIRS || experts > GROUP_FUSED_MAX_EXPERTS || (reinterpret_cast<uintptr_t>(d_ids) & 15)) return false;
+    const size_t lds = ((size_t)((pairs + 511) & ~511) + 2 * ((size_t)experts + 1)) * sizeof(uint32_t);
+    static bool configured = false;   // more than the default 64 KB of dynamic LDS for the longer chunks
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_group_fused), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL(pf_k_group_fused, dim3((experts + 3) / 4), dim3(256), lds, stream, d_ids, pairs, experts, tokens, d_offsets, d_tiles,
+                       d_pair_to_row, d_row_to_pair);
+    return true;
+}
+
 int pf_group_pairs_device(const uint32_t *d_ids, int tokens, int experts, int top_k, uint32_t *d_counts,
                           uint32_t *d_offsets, uint32_t *d_pair_to_row, uint32_t *d_row_to_pair, uint32_t *d_first_bad,
                           hipStream_t stream) {
