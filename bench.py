@@ -57,6 +57,8 @@ WORKLOADS = {
     "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, steps=1000, warmup=100,
                         label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
     "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=20, warmup=5, label="Q4_K experts, " + PREFILL_LABEL),
+    "q4k_prefill2048": dict(type=abi.GGUF_Q4_K, tokens=2048, steps=20, warmup=5,
+                            label="Q4_K experts, " + PREFILL_LABEL.replace("1024", "2048") + " (the chunk size of the 48-layer stack)"),
     "iq2xxs_prefill1024": dict(type=abi.GGUF_IQ2_XXS, tokens=1024, steps=20, warmup=5, label="IQ2_XXS experts, " + PREFILL_LABEL),
     "iq2xxs_decode_hc": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=2000, warmup=200, hc=4,
                              label="IQ2_XXS experts, decode batch 1, between the HC read and add of 4 residual streams"),

@@ -12,11 +12,13 @@
 //               reference's maximum (the largest logit is a candidate); p = expf(z - max) with the C
 //               library's expf reproduced bit for bit.
 //   order       by p descending, then id ascending.  The reference orders by fl(p / sum) with the same
-//               tie rule; dividing by a common sum keeps the order of two p that differ by two ulps or
-//               more strictly, and keeps equal p equal.  Two neighbours among the k + 1 first that are
-//               closer than that without being equal need the sum itself: then, or with more than 64
-//               candidates, or with probabilities near the subnormals, the workgroup routes the token the
-//               long way (all logits serially, a thread per expert, then pf_route_exact_wave).
+//               tie rule.  Two p four ulps or more apart give quotients that round to different values,
+//               equal p stay equal, and closer p can only tie, which goes to the lower id: no change
+//               when the larger p has the lower id already.  Two neighbours among the k + 1 first that
+//               are fewer than four ulps apart, not equal, with the larger p on the higher id need the
+//               sum itself: then, or with more than 64 candidates, or with probabilities near the
+//               subnormals, the workgroup routes the token the long way (all logits serially, 64 experts
+//               a pass through the same chains, then pf_route_exact_wave).
 //
 // Route weights need not be bit-exact: normalised ones are p / sum of the chosen p (the common sum
 // cancels), the others p over the fast logits' softmax denominator.
@@ -96,10 +98,8 @@ __device__ __forceinline__ float pf_serial_chunk(float sum, const float *w, cons
 }
 
 // LDS the workgroup needs: the candidates' ids (64 words), four words of hand-over, the token's row (H floats), then
-// the two chunk buffers, which the long way's 3 E floats share.
-__host__ __device__ constexpr size_t pf_route_fix_lds_floats(int H, int E) {
-    return 68 + (size_t)H + (2 * PF_FIX_CHUNK_FLOATS > 3 * (size_t)E ? 2 * PF_FIX_CHUNK_FLOATS : 3 * (size_t)E);
-}
+// the two chunk buffers and the long way's 3 E floats.
+__host__ __device__ constexpr size_t pf_route_fix_lds_floats(int H, int E) { return 68 + (size_t)H + 2 * PF_FIX_CHUNK_FLOATS + 3 * (size_t)E; }
 
 // Called by every wave of a workgroup of at least two waves (workgroup barriers inside); E <= 64 NPL, K < 63.
 // Wave 0 picks the candidates and runs their sums, the others feed it.  router: [E][H] f32 as the file stores it;
@@ -112,7 +112,7 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
                                                   int wave, int lane) {
 #pragma clang fp contract(off)
     uint32_t *cand = reinterpret_cast<uint32_t *>(lds), *hand = cand + 64;   // hand[0]: candidates (0: the long way), hand[1]: outcome
-    float *xs = lds + 68, *stage = xs + H, *z = stage, *p = z + E, *q = p + E;
+    float *xs = lds + 68, *stage = xs + H, *z = stage + 2 * PF_FIX_CHUNK_FLOATS, *p = z + E, *q = p + E;
     const int picks = K < E ? K : E;
     const int helpers = (int)blockDim.x - PF_WAVE, me = (int)threadIdx.x - PF_WAVE;   // the waves after the first
     float v[NPL];
@@ -165,12 +165,13 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
         if (lane == 0) hand[0] = (uint32_t)count;
     }
     __syncthreads();
-    const int n = (int)hand[0];
-    float zc = 0.0f;
-    if (n > 0) {
+    // Serial sums of n router rows, lane r of wave 0 the r-th: the listed candidates (base < 0) or rows base .. base + n.
+    // Every wave calls it (workgroup barriers inside).
+    auto staged_sums = [&](int n, int base) -> float {
+        float sum = 0.0f;
         const int rows = n <= 16 ? 16 : n <= 32 ? 32 : 64, chunk = 8192 / rows, pitch = chunk + 4;
         const int chunks = (H + chunk - 1) / chunk;
-        auto bring = [&](int c) {   // chunk c of every candidate's row into its buffer, by the waves after the first
+        auto bring = [&](int c) {   // chunk c of every row into its buffer, by the waves after the first
             const int first = c * chunk, pieces = min(chunk, H - first) / 4, total = n * pieces;
             float *buf = stage + (c & 1) * PF_FIX_CHUNK_FLOATS;
             for (int i0 = me; i0 >= 0 && i0 < total; i0 += 4 * helpers) {
@@ -180,7 +181,8 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
                 for (int j = 0; j < 4; j++) {
                     const int i = min(i0 + j * helpers, total - 1);
                     row[j] = i / pieces; piece[j] = i - row[j] * pieces;
-                    held[j] = reinterpret_cast<const float4 *>(router + (size_t)cand[row[j]] * H + first)[piece[j]];
+                    const size_t expert = base < 0 ? cand[row[j]] : (uint32_t)(base + row[j]);
+                    held[j] = reinterpret_cast<const float4 *>(router + expert * H + first)[piece[j]];
                 }
 #pragma unroll
                 for (int j = 0; j < 4; j++)
@@ -192,13 +194,17 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
         for (int c = 0; c < chunks; c++) {
             if (wave != 0) {
                 if (c + 1 < chunks) bring(c + 1);
-            } else {   // lanes beyond the candidates sum the last candidate's row again, unused
+            } else {   // lanes beyond the rows sum the last row again, unused
                 const int first = c * chunk, pieces = min(chunk, H - first) / 4;
-                zc = pf_serial_chunk(zc, stage + (c & 1) * PF_FIX_CHUNK_FLOATS + min(lane, n - 1) * pitch, xs + first, pieces);
+                sum = pf_serial_chunk(sum, stage + (c & 1) * PF_FIX_CHUNK_FLOATS + min(lane, n - 1) * pitch, xs + first, pieces);
             }
             __syncthreads();
         }
-    }
+        return sum;
+    };
+    const int n = (int)hand[0];
+    float zc = 0.0f;
+    if (n > 0) zc = staged_sums(n, -1);
     if (wave == 0) {
         bool long_way = n == 0;
         if (!long_way) {
@@ -218,11 +224,16 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
             const int to = active ? rank : lane;   // a permutation of the lanes
             const uint32_t sid = (uint32_t)__builtin_amdgcn_ds_permute(to * 4, (int)id);
             const float sp = __int_as_float(__builtin_amdgcn_ds_permute(to * 4, __float_as_int(pc)));
-            // neighbours among the first k + 1: equal, or apart by more than the division can close; nothing near the subnormals
+            // Neighbours among the first k + 1.  The reference orders by fl(p / sum): two p that are four ulps or more
+            // apart give quotients more than one ulp apart, which round to different values; closer p may tie after the
+            // division, and a tie goes to the lower id: that changes nothing when the larger p has the lower id already.
+            // So the doubt is a pair fewer than four ulps apart, not equal, whose larger p has the higher id; and
+            // nothing may be near the subnormals.
             const float next = __shfl_down(sp, 1);
+            const uint32_t next_id = (uint32_t)__shfl_down((int)sid, 1);
             const bool paired = lane < picks && lane + 1 < count;
-            const bool doubtful = (paired && !(sp == next || sp - next > 1e-6f * sp)) || (lane < picks && !(sp > 1e-30f)) ||
-                                  (paired && !(next > 1e-30f));
+            const bool near = sp != next && __float_as_uint(sp) - __float_as_uint(next) < 4u;
+            const bool doubtful = (paired && near && sid > next_id) || (lane < picks && !(sp > 1e-30f)) || (paired && !(next > 1e-30f));
             long_way = __any(doubtful);
             if (!long_way) {
                 const float chosen = pf_wave_sum(lane < picks ? sp : 0.0f);
@@ -243,8 +254,16 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
     }
     __syncthreads();
     const int how = (int)hand[1];
-    if (how == 2) {   // every logit in serial order, a thread per expert, then the reference's routing step by step
-        for (int e = threadIdx.x; e < E; e += blockDim.x) z[e] = pf_serial_logit(router + (size_t)e * H, xs, H);
+    if (how == 2) {   // every logit in serial order, 64 experts a pass, then the reference's routing step by step
+        if (H % 4 == 0 && (reinterpret_cast<uintptr_t>(router) & 15) == 0) {
+            for (int e0 = 0; e0 < E; e0 += PF_WAVE) {
+                const int rows = min(PF_WAVE, E - e0);
+                const float ze = staged_sums(rows, e0);
+                if (wave == 0 && lane < rows) z[e0 + lane] = ze;
+            }
+        } else {   // rows that cannot be fetched in 16-byte pieces: a thread per expert
+            for (int e = threadIdx.x; e < E; e += blockDim.x) z[e] = pf_serial_logit(router + (size_t)e * H, xs, H);
+        }
         __syncthreads();
         if (wave == 0) pf_route_exact_wave(z, p, q, E, K, norm, ids_out, w_out, lane);
     }
