@@ -254,6 +254,43 @@ def test_many_near_ties_are_settled_by_the_doubtful_experts_alone(product, oracl
         assert_parity(y, ids, w, *want, label="near ties, general kernels")
 
 
+@pytest.mark.parametrize("clones", [24, 40, 80])
+def test_crowds_of_near_equal_experts(product, oracle, clones):
+    """Many router rows that are copies of one row up to a few ulps, and tokens that point along that row: the crowd
+    fills the top of every token's logits, so the re-route sees 17..32, 33..64 or more than 64 doubtful experts (the
+    last go the long way).  Decode, prefill and general kernels against the CPU path, ids bit for bit."""
+    cfg = abi.moe_config(512, 128, 8, 256, 256)
+    tokens = 48
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, tokens, seed=77 + clones)
+    router = weights.raw[0].view(np.float32).reshape(128, 512)
+    rng = np.random.default_rng(clones)
+    for e in range(1, clones):
+        row = router[0].copy()
+        for col in rng.choice(512, size=int(rng.integers(0, 3)), replace=False):   # 0 places: an exact copy
+            row[col] = np.nextafter(row[col], np.float32(rng.choice([-10.0, 10.0])))
+        router[e] = row
+    x = (x * np.float32(0.3) + router[0][None, :] * np.float32(40.0)).astype(np.float32)   # the crowd's logit leads
+    want = forward_with(oracle, cfg, weights, x)
+    assert (want[1] < clones).all(), "every selected expert must come from the crowd"
+    with pf.MoeLayer(product, cfg, weights, tokens) as layer:
+        for first in range(0, 6):
+            _, y, ids, w = layer.forward(x[first:first + 1])
+            assert_parity(y, ids, w, want[0][first:first + 1], want[1][first:first + 1], want[2][first:first + 1],
+                          label=f"crowd of {clones}, token {first} alone")
+        _, y, ids, w = layer.forward(x[:16])
+        assert_parity(y, ids, w, want[0][:16], want[1][:16], want[2][:16], label=f"crowd of {clones}, 16 tokens")
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y, ids, w, *want, label=f"crowd of {clones}, chunk")
+        reroutes, full = layer.serial_order_reroutes(), layer.full_reroutes()
+        print(f"  crowd of {clones}: {reroutes} re-routed, {full} the long way", flush=True)
+        assert reroutes >= tokens
+        if clones > 64:
+            assert full > 0, "more than 64 doubtful experts must go the long way"
+        layer.force_general()
+        _, y, ids, w = layer.forward(x)
+        assert_parity(y, ids, w, *want, label=f"crowd of {clones}, general kernels")
+
+
 def test_nonfinite_activation_is_reported_and_sticky_until_reset(product):
     cfg = abi.moe_config(512, 32, 6, 256, 256)
     weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 2, seed=6)
