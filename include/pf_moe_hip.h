@@ -80,8 +80,9 @@ int pf_hip_moe_forward_static(const PfHipMoe *moe, const float *d_x, size_t x_pi
                               size_t y_pitch, uint32_t *d_ids, float *d_route_weights,
                               uint32_t *d_error_word, size_t tokens, void *stream);
 /* Which kernels a forward of `tokens` tokens runs on this layer and workspace: 1 the
- * decode kernels (1..4 tokens, supported shapes and formats), 2 the matrix-core
- * prefill kernels, 0 the general kernels (any shape and format mix). */
+ * decode kernels (1..4 tokens, 1..16 with the tile-ordered copies; supported shapes and formats),
+ * 2 the matrix-core prefill kernels, 0 the general kernels (any shape and format mix).  A streamed
+ * layer: 1 for the batches its decode kernels take when the pool keeps Q4_K slots in the tile order. */
 int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t tokens);
 /* Device pointers into the workspace, valid after a forward: expert ids
  * [tokens, top_k] uint32, route weights [tokens, top_k], router logits
@@ -213,12 +214,16 @@ int pf_hip_exact_combine_host(const float *down, const uint64_t *pair_to_row, co
  * expert ids (dense [tokens, top_k]); the caller makes them resident and passes the pool's three device
  * regions, the payload bytes of one expert and the offset of the scales in each (pf_hip_pool_region_plan's
  * layout for the pool's slot count), the slot count and the pairs' slots to the second, which runs the
- * expert products and the combine.  pf_hip_moe_forward_* refuse such a layer. */
+ * expert products and the combine.  pf_hip_moe_forward_* refuse such a layer.
+ * tiled_mask, the same in both calls: bit j set when region j holds Q4_K slots in the tile order (what
+ * pf_hip_pool_store writes where pf_hip_pool_slot_tiled says so).  With all three set, batches of up to 16
+ * tokens run the decode kernels on the slots (the first call the router kernel and the routing, the second
+ * the expert kernels); otherwise the general kernels. */
 int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
-                                   size_t tokens, uint32_t *ids, uint32_t *error_word);
+                                   size_t tokens, uint32_t tiled_mask, uint32_t *ids, uint32_t *error_word);
 int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const void *const regions[3],
                                      const size_t expert_bytes[3], const size_t scale_offsets[3],
-                                     uint32_t pool_slots, const uint32_t *slots,
+                                     uint32_t pool_slots, uint32_t tiled_mask, const uint32_t *slots,
                                      float *y, size_t y_pitch_bytes, uint32_t *ids, size_t ids_pitch_bytes,
                                      float *weights, size_t weights_pitch_bytes, size_t tokens,
                                      uint32_t *error_word);
@@ -227,12 +232,14 @@ int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const
  * tensor of `slots` experts (formats stored as the file stores them slot after slot; IQ2_XXS, Q8_0 and
  * MXFP4 as all payloads, then all scales).  pf_hip_pool_region_plan gives the region's size, the bytes
  * of one expert in the file, the bytes of its payload in a slot and the offset of the scales (0: not split); pf_hip_pool_store copies one
- * expert's file bytes from host memory into a slot, splitting on the device where the format needs it,
+ * expert's file bytes from host memory into a slot, splitting on the device where the format needs it
+ * (a Q4_K matrix whose row count is a multiple of 32 goes into the tile order: pf_hip_pool_slot_tiled),
  * and returns when the slot is readable. */
 int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, size_t *region_bytes,
                             size_t *file_expert_bytes, size_t *payload_expert_bytes, size_t *scale_offset);
 int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, void *region, size_t slot,
                       const void *file_bytes);
+int pf_hip_pool_slot_tiled(uint32_t gguf_type, size_t n_out);
 
 /* Minimal device-memory helpers so that a host program can keep inputs resident. */
 int pf_hip_malloc(void **d_ptr, size_t bytes);

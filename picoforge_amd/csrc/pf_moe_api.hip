@@ -306,6 +306,34 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             }
         }
     }
+    // A streamed layer that is Q4_K throughout: tile-ordered copies of its shared expert, so that short batches run the
+    // tile decode kernels on pool slots kept in tile order (the routed tensors are not here to be copied).
+    if (m->streamed) {
+        bool all_q4k = true;
+        for (int a = 1; a <= 6; a++) all_q4k &= desc->type[a] == PF_Q4_K;
+        const char *copy = getenv("PF_MOE_PREFILL_COPY");
+        if (all_q4k && pf_decode_supported(*desc) && (!copy || strcmp(copy, "0") != 0)) {
+            hipError_t e = hipSuccess;
+            for (int a = 4; a <= 6 && e == hipSuccess; a++) {
+                if (n_out[a] % 32) { e = hipErrorInvalidValue; break; }
+                e = hipMalloc((void **)&m->w_tiled[a], m->bytes[a]);
+                if (e == hipSuccess) {
+                    pf_launch_q4k_tile(m->w[a], m->w_tiled[a], (size_t)n_out[a], m->blocks_per_row[a], nullptr);
+                    m->total_bytes += m->bytes[a];
+                }
+            }
+            if (e == hipSuccess) e = hipDeviceSynchronize();
+            if (e == hipSuccess) {
+                const uint8_t *tiled[8];
+                for (int a = 0; a < 8; a++) tiled[a] = a >= 1 && a <= 3 ? m->w[0] : m->w_tiled[a];   // 1..3: any non-null address, the pool's at forward time
+                m->stream_decode_ready = n_out[1] % 32 == 0 && n_out[3] % 32 == 0 && pf_decode_tile_layer(m->desc, tiled, m->w_itile, m->w_qtile) == 1;
+            } else {
+                (void)hipGetLastError();   // without the copies the general kernels serve every batch
+                for (int a = 4; a <= 6; a++)
+                    if (m->w_tiled[a]) { (void)hipFree(m->w_tiled[a]); m->w_tiled[a] = nullptr; }
+            }
+        }
+    }
     // A Q4_K layer that every kernel family can read through the tile-ordered copy alone (the decode kernels whose lanes
     // are weight rows, the grouped product, the general kernels' tile reader) gives its row-ordered expert tensors
     // back: one copy of the experts in device memory, not two.
@@ -572,6 +600,7 @@ static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_
 // 2 the matrix-core prefill kernels, 0 the general kernels.
 extern "C" int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t tokens) {
     if (!moe || !work || work->force_general) return 0;
+    if (moe->streamed) return moe->stream_decode_ready && tokens <= PF_TILE_DECODE_MAX_TOKENS ? 1 : 0;   // given a pool with tile-ordered slots
     if (moe->decode_ready && tokens <= decode_limit(moe)) return 1;
     if (moe->prefill_ready && work->down && tokens > PF_DECODE_MAX_TOKENS) return 2;
     return 0;
@@ -716,8 +745,16 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
 // expert ids; the caller makes those experts resident (qw4_pool_acquire) and passes the pool's device regions and
 // the pairs' slots to the second, which runs the expert products and the combine reading rows at
 // region + slot * expert_bytes.  The general kernels serve both: streaming is bound by the reads that fill the pool.
+extern "C" int pf_hip_pool_slot_tiled(uint32_t gguf_type, size_t n_out) { return gguf_type == PF_Q4_K && n_out % 32 == 0; }
+
+// Short batches of a streamed Q4_K layer whose three pool regions hold tile-ordered slots run the tile decode kernels:
+// kernel 1 and the routing kernels in the first call, kernels 2 and 3 reading the pairs' slots in the second.
+static bool streamed_decode(const PfHipMoe *moe, const PfHipWork *work, size_t tokens, uint32_t tiled_mask) {
+    return moe->stream_decode_ready && tiled_mask == 7u && tokens <= PF_TILE_DECODE_MAX_TOKENS && !work->force_general;
+}
+
 extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
-                                              size_t tokens, uint32_t *ids, uint32_t *error_word) {
+                                              size_t tokens, uint32_t tiled_mask, uint32_t *ids, uint32_t *error_word) {
     if (!moe || !work || work->moe != moe || !error_word) return PF_HIP_E_ARGUMENT;
     *error_word = 0;
     if (tokens == 0) return PF_HIP_OK;
@@ -731,7 +768,13 @@ extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *wo
         snprintf(g_error, sizeof g_error, "dimensions exceed the LDS staging of the general kernels");
         return PF_HIP_E_UNSUPPORTED;
     }
-    pf_launch_general(a, (int)tokens, nullptr, 2);
+    if (streamed_decode(moe, work, tokens, tiled_mask)) {
+        HIP_TRY(hipMemsetAsync(work->route_flags, 0, 4, nullptr));   // the routing's list starts empty (the other router kernels clear it themselves)
+        pf_launch_dec_router(a, (int)tokens, (int)((moe->desc.experts + 3) / 4), nullptr);
+        pf_launch_route(a, (int)tokens, nullptr);
+    } else {
+        pf_launch_general(a, (int)tokens, nullptr, 2);
+    }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
     if (*error_word) {
@@ -744,7 +787,7 @@ extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *wo
 
 extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const void *const regions[3],
                                                 const size_t expert_bytes[3], const size_t scale_offsets[3],
-                                                uint32_t pool_slots, const uint32_t *slots,
+                                                uint32_t pool_slots, uint32_t tiled_mask, const uint32_t *slots,
                                                 float *y, size_t y_pitch_bytes, uint32_t *ids, size_t ids_pitch_bytes,
                                                 float *weights, size_t weights_pitch_bytes, size_t tokens,
                                                 uint32_t *error_word) {
@@ -764,12 +807,21 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
     HIP_TRY(hipMemcpy(work->slots, slots, tokens * K * 4, hipMemcpyHostToDevice));
     PfKernelArgs a = make_args(moe, work, work->x, H, work->y, H);
     for (int j = 0; j < 3; j++) {
-        a.w[1 + j] = static_cast<const uint8_t *>(regions[j]);
-        a.scale_offset[1 + j] = scale_offsets[j];
+        const int t = 1 + j;
+        const bool tiled = (tiled_mask >> j) & 1u;
+        if (tiled && !pf_hip_pool_slot_tiled(moe->desc.type[t], (size_t)moe->n_out[t])) return PF_HIP_E_ARGUMENT;
+        a.w[t] = tiled ? nullptr : static_cast<const uint8_t *>(regions[j]);    // Q4_K slots in tile order: every kernel's tile reader
+        a.wt[t] = tiled ? static_cast<const uint8_t *>(regions[j]) : nullptr;
+        a.scale_offset[t] = scale_offsets[j];
     }
     a.slots = work->slots;
     a.pool_slots = pool_slots;
-    pf_launch_general(a, (int)tokens, nullptr, 0, 3);
+    if (streamed_decode(moe, work, tokens, tiled_mask)) {
+        // kernel 1 ran in the first call (logits and the token rows' images are in the workspace): kernels 2 and 3 only
+        pf_launch_decode_q4k_experts(a, (int)tokens, nullptr);
+    } else {
+        pf_launch_general(a, (int)tokens, nullptr, 0, 3);
+    }
     HIP_TRY(hipGetLastError());
     HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
     if (*error_word) {
@@ -813,6 +865,15 @@ extern "C" int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_
         return PF_HIP_E_ARGUMENT;
     uint8_t *base = static_cast<uint8_t *>(region);
     const size_t head = split_header_bytes(gguf_type), file_expert = place.gguf_bytes / slots;
+    if (pf_hip_pool_slot_tiled(gguf_type, n_out)) {   // Q4_K: the slot in the tile order every kernel family reads
+        DeviceBlock staging;
+        HIP_TRY(hipMalloc((void **)&staging.p, file_expert));
+        HIP_TRY(hipMemcpy(staging.p, file_bytes, file_expert, hipMemcpyHostToDevice));
+        pf_launch_q4k_tile(staging.p, base + slot * place.expert_bytes, n_out, place.blocks_per_row, nullptr);
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipStreamSynchronize(nullptr));
+        return PF_HIP_OK;
+    }
     if (!head) {
         HIP_TRY(hipMemcpy(base + slot * place.expert_bytes, file_bytes, file_expert, hipMemcpyHostToDevice));
         return PF_HIP_OK;

@@ -1053,6 +1053,7 @@ __device__ __forceinline__ void q4t_at_token(PfKernelArgs &a, int t) {
     a.logit_ssq += (size_t)t * a.experts;
     a.ids += (size_t)t * a.top_k;
     a.route_weights += (size_t)t * a.top_k;
+    if (a.slots) a.slots += (size_t)t * a.top_k;
     a.act += (size_t)t * a.top_k * a.inter;
     a.shared_act += (size_t)t * a.shared_inter;
     a.shared_scale += t;
@@ -1129,8 +1130,19 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
     if (!shared || FMT == PF_IQ2_XXS) __syncthreads();   // the early expert; the tables
     const uint32_t early = shared ? 0u : early_expert;
     const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
+    // Expert streaming: the slot's expert was routed by an earlier launch and sits in pool slot slots[u]; the tile is
+    // read there, whatever the early guess says, and the routing below only has to agree with the ids it was fetched by.
+    const bool pooled = a.pool_slots != 0u;
+    uint32_t pooled_at = 0u;
+    if (pooled && !shared) {
+        pooled_at = a.slots[u];
+        if (pooled_at >= a.pool_slots) {
+            if (threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
+            pooled_at = 0u;
+        }
+    }
     if (shared) q4t_tile<FMTS>(a, plan, partial, tables, 0u, wave);
-    else q4t_tile<FMT>(a, plan, partial, tables, early_ok ? early : 0u, wave);
+    else q4t_tile<FMT>(a, plan, partial, tables, pooled ? pooled_at : early_ok ? early : 0u, wave);
     if (wave == 0 && !shared) {
         // the remaining slots, the candidate beyond them and one more key, while the other waves' weight bytes travel
         for (int r = u + 1; r <= rounds; r++) {
@@ -1159,7 +1171,7 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
         // the slot's expert in the final order (the early guess came from truncated keys; the serial-order routing
         // can name another expert)
         e = R.ids[u];
-        if (e != early && e < (uint32_t)E) {
+        if (!pooled && e != early && e < (uint32_t)E) {
             __syncthreads();
             q4t_tile<FMT>(a, plan, partial, tables, e, wave);
             __syncthreads();
@@ -1168,6 +1180,7 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
             // publish the routes for the next kernel and the caller (one token: slot = pair = unique expert)
             if (R.close[0] == 0) __syncthreads();   // R.bad above; route_finish ends with a barrier of its own
             for (int q = threadIdx.x; q < K; q += blockDim.x) {
+                if (pooled && a.ids[q] != R.ids[q]) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);   // not the experts that were fetched
                 a.ids[q] = R.ids[q];
                 a.route_weights[q] = R.weights[q];
                 if (gridDim.y == 1) {   // the table of unique experts: read by the other down kernel, which runs after this one only for one token
@@ -1624,6 +1637,13 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
         if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
         e = 0;
     }
+    if (a.pool_slots != 0u && !shared) {   // expert streaming: the expert's rows sit in its pool slot
+        e = ((PfScalarWords)(uintptr_t)a.slots)[s];
+        if (e >= a.pool_slots) {
+            if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
+            e = 0;
+        }
+    }
     PfOutputRegs out_regs;
     if ((int)threadIdx.x < rows) pf_output_prefetch(a, token, n_base + threadIdx.x, out_regs);
     const uint32_t *image = a.aimg + (size_t)s * pf_image2_words(widest);   // slot = unique expert with one token; the shared expert's follows
@@ -1878,11 +1898,8 @@ static PfHipMoeDesc desc_of(const PfKernelArgs &a) {
 }
 
 template <int FG, int FD, int FS>
-static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
-    const int router_blocks = (E + 3) / 4, last = stage_limit ? stage_limit : 3;
-    pf_launch_dec_router(a, tokens, router_blocks, stream);
-    if (last < 2) return;
+static void launch_q4t_experts(const PfKernelArgs &a, int tokens, hipStream_t stream, int last) {
+    const int H = a.hidden, I = a.inter, Is = a.shared_inter, K = a.top_k;
     // kernel 2: every workgroup extracts the maxima up to its own slot from all of its token's logits
     launch_gate_up_q4t<FG, FS>(a, tokens, stream);
     if (last < 3) return;
@@ -1904,6 +1921,14 @@ static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t str
     }
     hipLaunchKernelGGL((pf_k_dec_down_q4t<FD, FS>), dim3(H / rows, tokens), dim3(64 * (K + 1)),
                        (GRID ? 2048 * (size_t)(K + 1) : 0) + (size_t)(K + 1) * (pf_image2_words(widest) + rows * (widest / 64)) * 4, stream, a, rows);
+}
+
+template <int FG, int FD, int FS>
+static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
+    const int last = stage_limit ? stage_limit : 3;
+    pf_launch_dec_router(a, tokens, (a.experts + 3) / 4, stream);
+    if (last < 2) return;
+    launch_q4t_experts<FG, FD, FS>(a, tokens, stream, last);
 }
 
 // FG: format of the routed gate and up tensors, FD: of the routed down tensor, FS: of the shared expert
@@ -1978,6 +2003,10 @@ void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t s
 void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq) == 1) launch_decode_q4t<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
     else launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
+}
+
+void pf_launch_decode_q4k_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
+    launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, 3);
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {

@@ -34,7 +34,7 @@ struct PfKernelArgs {
     uint32_t *ximg, *aimg;           // decode path, tile-ordered Q4_K: digit images (pf_image2_words) of the token rows, written
                                      // by kernel 1, and of the activation rows [unique, tokens] then [tokens] shared, by kernel 2
     uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
-    // expert streaming (general kernels only): w[1..3] are pool regions of pool_slots experts each and the routed
+    // expert streaming: w[1..3] (wt[1..3] for Q4_K slots in tile order) are pool regions of pool_slots experts each and the routed
     // tensors are addressed by slots[pair] instead of ids[pair] (null: every expert resident, addressed by id)
     const uint32_t *slots;
     uint32_t pool_slots;
@@ -107,6 +107,7 @@ struct PfHipMoe {
     size_t total_bytes;
     bool decode_ready;               // shapes and formats the specialised decode kernels cover
     bool prefill_ready;              // shapes and formats the matrix-core prefill kernels cover
+    bool stream_decode_ready;        // a streamed layer whose short batches run the tile decode kernels on pool slots in tile order
     float *w_norm2;                  // [experts] squared norm of each router row
     float *router_t;                 // [slab of 64 experts][hidden / 4][64][4] copy of the router
     uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
@@ -177,6 +178,9 @@ void pf_launch_iq2_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint
 void pf_launch_q8_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8_t *d_dst, size_t rows, int blocks_per_row,
                        hipStream_t stream);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
+// kernels 2 and 3 of the tile decode path for a Q4_K layer (expert streaming: kernel 1 ran in an earlier call)
+void pf_launch_decode_q4k_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);
 void pf_launch_block_split(const uint8_t *d_gguf, uint8_t *d_payload, uint8_t *d_scales, size_t blocks,

@@ -506,9 +506,11 @@ static Qwen4Status streamed_forward(const Qwen4Moe *m, Qwen4MoeWork *w, QW4Exper
     const void *regions[3];
     size_t expert_bytes[3], scale_offsets[3];
     const size_t pool_slots = pf_pool_slots(pool);
+    uint32_t tiled_mask = 0;   /* regions whose slots the pool stored in the Q4_K tile order */
     for (int j = 0; j < 3; j++) {
         const QW4PackedLayout *l = &m->w[1 + j].layout;
         const uint32_t format = pf_pool_format(pool, j);
+        if (format != UINT32_MAX && pf_hip_pool_slot_tiled(l->gguf_type, l->n_out)) tiled_mask |= 1u << j;
         size_t region_bytes = 0, want_bytes = 0, file_bytes = 0;
         regions[j] = qw4_pool_region(pool, j, &region_bytes);
         if (!regions[j] || !pool_slots ||
@@ -522,14 +524,14 @@ static Qwen4Status streamed_forward(const Qwen4Moe *m, Qwen4MoeWork *w, QW4Exper
     uint32_t *ids = malloc(pairs * 2 * sizeof *ids), *slots = ids ? ids + pairs : NULL, word = 0;
     if (!ids) return moe_status(err, QW4_OOM, "streaming staging");
     Qwen4Status st = QW4_OK;
-    int rc = pf_hip_moe_route_streamed_host(m->device, w->device, x.data, x.stride_bytes[0], T, ids, &word);
+    int rc = pf_hip_moe_route_streamed_host(m->device, w->device, x.data, x.stride_bytes[0], T, tiled_mask, ids, &word);
     if (rc) st = pf_device_status(rc, err, "qwen4_moe");
     else if (word & PF_HIP_ERR_NONFINITE) st = moe_status(err, QW4_NONFINITE, "nonfinite value in the MoE block");
     else if (word) st = moe_status(err, QW4_GPU_ERROR, "device error word");
     else if (qw4_pool_acquire(pool, layer, ids, pairs, slots))
         st = moe_status(err, QW4_IO, "expert pool: every slot pinned, or a read of the model file failed");
     if (!st) {
-        rc = pf_hip_moe_experts_streamed_host(m->device, w->device, regions, expert_bytes, scale_offsets, (uint32_t)pool_slots, slots, y.data,
+        rc = pf_hip_moe_experts_streamed_host(m->device, w->device, regions, expert_bytes, scale_offsets, (uint32_t)pool_slots, tiled_mask, slots, y.data,
                                               y.stride_bytes[0], routes ? routes->ids.data : NULL,
                                               routes ? routes->ids.row_stride_bytes : 0,
                                               routes ? routes->weights.data : NULL,

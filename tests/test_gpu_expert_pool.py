@@ -206,6 +206,57 @@ def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype, f
     os.close(fd)
 
 
+def test_streamed_q4k_layer_on_the_decode_kernels(product, oracle, tmp_path):
+    """A Q4_K layer of a shape the decode kernels cover, streamed through a pool that was told its formats: the
+    slots are kept in the tile order and batches of up to 16 tokens run the decode kernels on them (the router kernel
+    and the routing in the first device call, the expert kernels on the pairs' slots in the second); longer batches
+    run the general kernels on the same slots.  56 slots for 64 experts: evictions on the way."""
+    cfg = abi.moe_config(512, 64, 4, 256, 256)
+    tokens = 40
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, tokens, seed=67)
+    x[5] = x[4]                                              # two tokens of a batch share every expert
+    sizes = [weights.raw[j].size // cfg.experts for j in (1, 2, 3)]
+    filler = np.zeros(4096, np.uint8)
+    pieces, offsets, at = [filler], [], filler.size
+    for j in (1, 2, 3):
+        offsets.append(at)
+        pieces.append(weights.raw[j])
+        at += weights.raw[j].size
+    path = tmp_path / "model.bin"
+    np.concatenate(pieces).tofile(path)
+    fd = os.open(path, os.O_RDONLY)
+    table = (abi.QW4ExpertLayer * 1)(abi.QW4ExpertLayer((C.c_uint64 * 3)(*offsets)))
+    pool = product.pool_create(fd, table, 1, cfg.experts, (C.c_size_t * 3)(*sizes), 56)
+    assert pool
+    h, i = cfg.hidden_size, cfg.intermediate
+    assert product.pool_set_formats(pool, (C.c_uint32 * 3)(*weights.types[1:4]), (C.c_size_t * 3)(h, h, cfg.down_physical),
+                                    (C.c_size_t * 3)(i, i, h)) == 0
+    err, handle = abi.Qwen4Error(), C.c_void_p()
+    struct = streamed_weights(weights)
+    assert product.create_streamed(C.byref(cfg), C.byref(struct), C.byref(handle), C.byref(err)) == abi.QW4_OK, err.detail
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, tokens, handle=handle) as layer:
+        moe, work = layer.device_handles()
+        assert product.hip.moe_kernel_family(moe, work, 1) == 1 and product.hip.moe_kernel_family(moe, work, 16) == 1
+        assert product.hip.moe_kernel_family(moe, work, 17) == 0
+        for first, count in ((0, 1), (1, 1), (2, 4), (6, 16), (22, 3), (0, 16), (20, 18), (25, 15)):
+            print(f"  streamed rows {first}..{first + count}", flush=True)
+            rows = np.ascontiguousarray(x[first:first + count])
+            y = np.full((count, cfg.hidden_size), -99.0, np.float32)
+            ids = np.full((count, cfg.top_k), 0xFFFFFFFF, np.uint32)
+            w = np.full((count, cfg.top_k), -99.0, np.float32)
+            routes = abi.Qwen4MoeRoutes(abi.u32_view(ids), abi.f32_view(w))
+            st = product.forward_streamed(layer.handle, pool, 0, abi.f32_view(rows), abi.f32_view(y), C.byref(routes),
+                                          layer.work, C.byref(layer.err))
+            assert st == abi.QW4_OK, layer.err.detail
+            assert_parity(y, ids, w, want[0][first:first + count], want[1][first:first + count],
+                          want[2][first:first + count], label=f"streamed rows {first}..{first + count}")
+        stats = product.pool_stats(pool)
+        assert stats.evictions > 0 and stats.hits > 0
+    product.pool_destroy(pool)
+    os.close(fd)
+
+
 def test_streaming_refuses_what_it_cannot_hold(product, tmp_path):
     cfg = abi.moe_config(256, 16, 4, 256, 256)
     weights, x = make_layer_inputs(cfg, abi.GGUF_IQ2_XXS, 1, seed=3)   # stored split on the device
