@@ -1075,8 +1075,9 @@ __device__ __forceinline__ void q4t_route_fix(const float *router, const float *
     __syncthreads();
 }
 
-// FMT: format of the routed gate and up tensors, FMTS: of the shared expert's (the same, or the profiles' Q8_0)
-template <int NPL, int FMT, int FMTS>
+// FMT: format of the routed gate and up tensors, FMTS: of the shared expert's (the same, or the profiles' Q8_0);
+// POOL: the routed tensors sit in pool slots (expert streaming)
+template <int NPL, int FMT, int FMTS, bool POOL>
 __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) {
     extern __shared__ int lds[];
     __shared__ RouteLds R;
@@ -1132,7 +1133,7 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
     const bool early_ok = early < (uint32_t)E;   // a nonfinite logit can leave no maximum: the error word says so below
     // Expert streaming: the slot's expert was routed by an earlier launch and sits in pool slot slots[u]; the tile is
     // read there, whatever the early guess says, and the routing below only has to agree with the ids it was fetched by.
-    const bool pooled = a.pool_slots != 0u;
+    constexpr bool pooled = POOL;
     uint32_t pooled_at = 0u;
     if (pooled && !shared) {
         pooled_at = a.slots[u];
@@ -1221,8 +1222,10 @@ __device__ __forceinline__ void q4t_gate_up(PfKernelArgs &a, int routed_blocks) 
 
 // With several tokens there are more workgroups than compute units; two workgroups per compute unit (64 registers a
 // lane) measured slower than one after the other: the products are bound by the vector units, not by waiting.
-template <int NPL, int FMT, int FMTS>
-__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) { q4t_gate_up<NPL, FMT, FMTS>(a, routed_blocks); }
+template <int NPL, int FMT, int FMTS, bool POOL>
+__global__ void __launch_bounds__(1024) pf_k_dec_gate_up_q4t(PfKernelArgs a, int routed_blocks) {
+    q4t_gate_up<NPL, FMT, FMTS, POOL>(a, routed_blocks);
+}
 
 // Kernel 2 alone on the tile order (one token; the down kernel stays the segment one): layers whose routed gate and up
 // tensors are Q4_K or IQ2_XXS with the copy kept and whose shared expert is in the same format or, as in the checkpoint
@@ -1236,29 +1239,29 @@ static bool q4t_gate_up_applies(const PfKernelArgs &a) {
            a.top_k < a.experts && a.top_k <= 15 && a.experts <= 1024;
 }
 
-template <int NPL, int FMT, int FMTS>
+template <int NPL, int FMT, int FMTS, bool POOL>
 static void launch_gate_up_q4t_lists(const PfKernelArgs &a, dim3 grid, size_t lds, hipStream_t stream, int routed_blocks) {
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS (the re-route's chunk buffers)
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up_q4t<NPL, FMT, FMTS>),
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_gate_up_q4t<NPL, FMT, FMTS, POOL>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);   // the kernel has static LDS too
         configured = true;
     }
-    hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<NPL, FMT, FMTS>), grid, dim3(1024), lds, stream, a, routed_blocks);
+    hipLaunchKernelGGL((pf_k_dec_gate_up_q4t<NPL, FMT, FMTS, POOL>), grid, dim3(1024), lds, stream, a, routed_blocks);
 }
 
-template <int FMT, int FMTS>
+template <int FMT, int FMTS, bool POOL = false>
 static void launch_gate_up_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, E = a.experts, K = a.top_k;
     const int routed_blocks = K * (I / 32);
     const dim3 g1(routed_blocks + Is / 32, tokens);
     const int all = (E + 63) / 64;
     const size_t lds = (size_t)table_words<FMT>() * 4 + (size_t)15 * 64 * 4 + pf_route_fix_lds_floats(H, E) * 4;
-    if (all <= 1) launch_gate_up_q4t_lists<1, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
-    else if (all <= 2) launch_gate_up_q4t_lists<2, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
-    else if (all <= 4) launch_gate_up_q4t_lists<4, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
-    else if (all <= 8) launch_gate_up_q4t_lists<8, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
-    else launch_gate_up_q4t_lists<16, FMT, FMTS>(a, g1, lds, stream, routed_blocks);
+    if (all <= 1) launch_gate_up_q4t_lists<1, FMT, FMTS, POOL>(a, g1, lds, stream, routed_blocks);
+    else if (all <= 2) launch_gate_up_q4t_lists<2, FMT, FMTS, POOL>(a, g1, lds, stream, routed_blocks);
+    else if (all <= 4) launch_gate_up_q4t_lists<4, FMT, FMTS, POOL>(a, g1, lds, stream, routed_blocks);
+    else if (all <= 8) launch_gate_up_q4t_lists<8, FMT, FMTS, POOL>(a, g1, lds, stream, routed_blocks);
+    else launch_gate_up_q4t_lists<16, FMT, FMTS, POOL>(a, g1, lds, stream, routed_blocks);
 }
 
 // ---- kernel 3: down products and the combine ---------------------------------------------------
@@ -1611,7 +1614,7 @@ __device__ __forceinline__ void down_wave(const PfKernelArgs &a, int tensor, uin
 
 // (at most 80 registers a lane: two workgroups of eleven waves then share a compute unit, which a hidden width of 2560,
 // 320 workgroups on 256 compute units, needs to finish in one round)
-template <int FMT, int FMTS>
+template <int FMT, int FMTS, bool POOL>
 __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT == PF_IQ2_XXS ? 4 : 6))) pf_k_dec_down_q4t(PfKernelArgs a, int rows) {
     __shared__ float partial[17][16];
     extern __shared__ int lds[];   // IQ2_XXS: the waves' magnitude grids; [slot][image words of the widest activation row]; [slot][rows * runs] products
@@ -1637,7 +1640,7 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
         if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);
         e = 0;
     }
-    if (a.pool_slots != 0u && !shared) {   // expert streaming: the expert's rows sit in its pool slot
+    if (POOL && !shared) {   // expert streaming: the expert's rows sit in its pool slot
         e = ((PfScalarWords)(uintptr_t)a.slots)[s];
         if (e >= a.pool_slots) {
             if (lane == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS);
@@ -1897,11 +1900,11 @@ static PfHipMoeDesc desc_of(const PfKernelArgs &a) {
     return d;
 }
 
-template <int FG, int FD, int FS>
+template <int FG, int FD, int FS, bool POOL = false>
 static void launch_q4t_experts(const PfKernelArgs &a, int tokens, hipStream_t stream, int last) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, K = a.top_k;
     // kernel 2: every workgroup extracts the maxima up to its own slot from all of its token's logits
-    launch_gate_up_q4t<FG, FS>(a, tokens, stream);
+    launch_gate_up_q4t<FG, FS, POOL>(a, tokens, stream);
     if (last < 3) return;
     const size_t widest = I > Is ? I : Is;
     constexpr bool GRID = FD == PF_IQ2_XXS || FS == PF_IQ2_XXS;
@@ -1915,11 +1918,11 @@ static void launch_q4t_experts(const PfKernelArgs &a, int tokens, hipStream_t st
     }
     static bool configured = false;   // once per instantiation: more than the default 64 KB of dynamic LDS
     if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down_q4t<FD, FS>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_down_q4t<FD, FS, POOL>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)Q4T_DOWN_LDS);
         configured = true;
     }
-    hipLaunchKernelGGL((pf_k_dec_down_q4t<FD, FS>), dim3(H / rows, tokens), dim3(64 * (K + 1)),
+    hipLaunchKernelGGL((pf_k_dec_down_q4t<FD, FS, POOL>), dim3(H / rows, tokens), dim3(64 * (K + 1)),
                        (GRID ? 2048 * (size_t)(K + 1) : 0) + (size_t)(K + 1) * (pf_image2_words(widest) + rows * (widest / 64)) * 4, stream, a, rows);
 }
 
@@ -2006,7 +2009,7 @@ void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream,
 }
 
 void pf_launch_decode_q4k_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
-    launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, 3);
+    launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K, true>(a, tokens, stream, 3);
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
