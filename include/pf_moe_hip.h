@@ -115,7 +115,10 @@ void pf_hip_work_limit_kernels(PfHipWork *work, int count);
 
 /* Host-buffer forward used by qwen4_moe_forward: copies x in, runs the forward,
  * copies y (and ids/weights when non-NULL) out, returns the error word.  Pitches
- * in bytes.  Outputs are written only when the error word is zero. */
+ * in bytes.  Outputs are written only when the error word is zero.  Batches of up
+ * to 16 tokens go through a pinned host block the workspace owns (one enqueued copy
+ * in, output rows written into the block by the kernels, one enqueued copy for the
+ * error word, ids and weights, one wait); longer ones use a blocking copy per buffer. */
 int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, const float *x,
                             size_t x_pitch_bytes, float *y, size_t y_pitch_bytes,
                             uint32_t *ids, size_t ids_pitch_bytes, float *weights,

@@ -362,7 +362,8 @@ extern "C" void pf_hip_moe_destroy(PfHipMoe *m) {
 extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_bytes : 0; }
 
 // workspace layout: buffers carved from one allocation, each 256-byte aligned
-enum { W_LOGITS, W_SSQ, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_IDS, W_SLOTS, W_UNIQ, W_ERR, W_EXACT, W_FLAGS, W_XIMG, W_AIMG,
+// (the error word, the ids and the route weights follow each other: a short batch's are fetched by one copy)
+enum { W_LOGITS, W_SSQ, W_ERR, W_IDS, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_SLOTS, W_UNIQ, W_EXACT, W_FLAGS, W_XIMG, W_AIMG,
        W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
        W_P2R, W_R2P, W_GROUPBAD, W_TILES, W_COUNT };
 struct Carve { size_t offset[W_COUNT], total; };
@@ -428,6 +429,66 @@ extern "C" size_t pf_hip_work_bytes(const PfHipMoeDesc *desc, size_t token_cap) 
 
 static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base);
 
+// The pinned block of a workspace: a head that mirrors the workspace from the error word to the route weights of a short
+// batch (one copy brings all three when that span is at most PF_HOST_HEAD_BYTES; ids and weights have places of their
+// own for workspaces of more tokens), then input rows, output rows and pool slots of up to PF_HOST_BLOCK_TOKENS
+// tokens, each part 256-byte aligned.  The kernels write the output rows straight into the block.
+#define PF_HOST_BLOCK_TOKENS PF_TILE_DECODE_MAX_TOKENS
+#define PF_HOST_HEAD_BYTES (32 * 1024)
+struct HostBlock {
+    uint8_t *head;
+    uint32_t *ids, *slots;
+    float *x, *y, *weights;
+    size_t y_offset, bytes;
+};
+static HostBlock host_block(const PfHipMoeDesc *d, uint8_t *base) {
+    const size_t T = PF_HOST_BLOCK_TOKENS, rows = (T * d->hidden * 4 + 255) & ~(size_t)255, pairs = (T * d->top_k * 4 + 255) & ~(size_t)255;
+    HostBlock b;
+    size_t at = 0;
+    b.head = base + at; at += PF_HOST_HEAD_BYTES;
+    b.x = (float *)(base + at); at += rows;
+    b.y_offset = at;
+    b.y = (float *)(base + at); at += rows;
+    b.ids = (uint32_t *)(base + at); at += pairs;
+    b.weights = (float *)(base + at); at += pairs;
+    b.slots = (uint32_t *)(base + at); at += pairs;
+    b.bytes = at;
+    return b;
+}
+static size_t host_block_bytes(const PfHipMoeDesc *d) { return host_block(d, nullptr).bytes; }
+static bool through_host_block(const PfHipWork *w, size_t tokens) { return w->host && tokens <= PF_HOST_BLOCK_TOKENS; }
+
+// Enqueues the copies that bring a short batch's error word, ids and route weights into the block; after the stream
+// has been waited for, host_results hands them out.
+struct HostResults { const uint32_t *error_word, *ids; const float *weights; };
+static hipError_t fetch_results(const PfHipWork *w, const HostBlock &b, size_t tokens, bool want_ids, bool want_weights,
+                                HostResults *r) {
+    const size_t pairs = tokens * w->moe->desc.top_k * 4;
+    const size_t ids_at = (size_t)((const uint8_t *)w->ids - (const uint8_t *)w->error_word);
+    const size_t rw_at = (size_t)((const uint8_t *)w->route_weights - (const uint8_t *)w->error_word);
+    r->error_word = (const uint32_t *)b.head;
+    if ((const uint8_t *)w->ids > (const uint8_t *)w->error_word && w->route_weights > (const float *)w->ids &&
+        rw_at + pairs <= PF_HOST_HEAD_BYTES) {
+        const size_t span = want_weights ? rw_at + pairs : want_ids ? ids_at + pairs : 4;
+        r->ids = (const uint32_t *)(b.head + ids_at);
+        r->weights = (const float *)(b.head + rw_at);
+        return hipMemcpyAsync(b.head, w->error_word, span, hipMemcpyDeviceToHost, nullptr);
+    }
+    r->ids = b.ids;
+    r->weights = b.weights;
+    hipError_t e = hipMemcpyAsync(b.head, w->error_word, 4, hipMemcpyDeviceToHost, nullptr);
+    if (e == hipSuccess && want_ids) e = hipMemcpyAsync(b.ids, w->ids, pairs, hipMemcpyDeviceToHost, nullptr);
+    if (e == hipSuccess && want_weights) e = hipMemcpyAsync(b.weights, w->route_weights, pairs, hipMemcpyDeviceToHost, nullptr);
+    return e;
+}
+
+static void rows_in(void *dst, const void *src, size_t src_pitch, size_t row_bytes, size_t rows) {
+    for (size_t r = 0; r < rows; r++) memcpy((uint8_t *)dst + r * row_bytes, (const uint8_t *)src + r * src_pitch, row_bytes);
+}
+static void rows_out(void *dst, size_t dst_pitch, const void *src, size_t row_bytes, size_t rows) {
+    for (size_t r = 0; r < rows; r++) memcpy((uint8_t *)dst + r * dst_pitch, (const uint8_t *)src + r * row_bytes, row_bytes);
+}
+
 extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWork **out) {
     if (out) *out = nullptr;
     if (!moe || !out) return PF_HIP_E_ARGUMENT;
@@ -445,6 +506,16 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     }
     w->moe = moe; w->cap = token_cap; w->bytes = c.total;
     carve_work(w, c, base);
+    // short batches through host pointers stage their rows in pinned memory: the copies are then enqueued and the call
+    // waits once, for the last of them (without the block the forwards fall back to one blocking copy per buffer)
+    if (hipHostMalloc((void **)&w->host, host_block_bytes(&moe->desc), hipHostMallocDefault) != hipSuccess) {
+        (void)hipGetLastError();
+        w->host = nullptr;
+    } else if (hipHostGetDevicePointer((void **)&w->host_device, w->host, 0) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipHostFree(w->host);
+        w->host = nullptr;
+    }
     *out = w;
     return PF_HIP_OK;
 }
@@ -487,6 +558,7 @@ static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base) {
 extern "C" void pf_hip_work_destroy(PfHipWork *w) {
     if (!w) return;
     if (w->logits) (void)hipFree(w->logits);   // base of the single allocation
+    if (w->host) (void)hipHostFree(w->host);
     free(w);
 }
 
@@ -723,6 +795,26 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
     if (tokens == 0) return PF_HIP_OK;
     if (!x || !y || tokens > work->cap) return PF_HIP_E_ARGUMENT;
     const size_t H = moe->desc.hidden, K = moe->desc.top_k;
+    if (through_host_block(work, tokens)) {
+        const HostBlock b = host_block(&moe->desc, work->host);
+        rows_in(b.x, x, x_pitch_bytes, H * 4, tokens);
+        HIP_TRY(hipMemcpyAsync(work->x, b.x, tokens * H * 4, hipMemcpyHostToDevice, nullptr));
+        // the last kernel writes the output rows into the pinned block itself
+        int rc = pf_hip_moe_forward_device(moe, work, work->x, H, (float *)(work->host_device + b.y_offset), H, tokens, nullptr);
+        if (rc != PF_HIP_OK) return rc;
+        HostResults r;
+        HIP_TRY(fetch_results(work, b, tokens, ids != nullptr, weights != nullptr, &r));
+        HIP_TRY(hipStreamSynchronize(nullptr));
+        *error_word = *r.error_word;
+        if (*error_word) {
+            HIP_TRY(hipMemset(work->error_word, 0, 4));   // the word is sticky on the device; reading it clears it
+            return PF_HIP_OK;
+        }
+        rows_out(y, y_pitch_bytes, b.y, H * 4, tokens);
+        if (ids) rows_out(ids, ids_pitch_bytes, r.ids, K * 4, tokens);
+        if (weights) rows_out(weights, weights_pitch_bytes, r.weights, K * 4, tokens);
+        return PF_HIP_OK;
+    }
     HIP_TRY(hipMemcpy2D(work->x, H * 4, x, x_pitch_bytes, H * 4, tokens, hipMemcpyHostToDevice));
     // prefill-sized batches go through whole; 2..4 tokens use the decode path in one launch
     int rc = pf_hip_moe_forward_device(moe, work, work->x, H, work->y, H, tokens, nullptr);
@@ -761,7 +853,14 @@ extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *wo
     if (!x || !ids || tokens > work->cap) return PF_HIP_E_ARGUMENT;
     const size_t H = moe->desc.hidden, K = moe->desc.top_k;
     if (tokens * K > 0x7fffffffu / 4) return PF_HIP_E_UNSUPPORTED;
-    HIP_TRY(hipMemcpy2D(work->x, H * 4, x, x_pitch_bytes, H * 4, tokens, hipMemcpyHostToDevice));
+    const bool staged = through_host_block(work, tokens);
+    const HostBlock b = host_block(&moe->desc, work->host);
+    if (staged) {
+        rows_in(b.x, x, x_pitch_bytes, H * 4, tokens);
+        HIP_TRY(hipMemcpyAsync(work->x, b.x, tokens * H * 4, hipMemcpyHostToDevice, nullptr));
+    } else {
+        HIP_TRY(hipMemcpy2D(work->x, H * 4, x, x_pitch_bytes, H * 4, tokens, hipMemcpyHostToDevice));
+    }
     PfKernelArgs a = make_args(moe, work, work->x, H, work->y, H);
     const size_t lds_route = (H + 3 * (size_t)moe->desc.experts) * 4;
     if (pf_general_lds_bytes(a) > 64 * 1024 || lds_route > 64 * 1024) {
@@ -776,12 +875,20 @@ extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *wo
         pf_launch_general(a, (int)tokens, nullptr, 2);
     }
     HIP_TRY(hipGetLastError());
-    HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
+    HostResults r = {nullptr, nullptr, nullptr};
+    if (staged) {
+        HIP_TRY(fetch_results(work, b, tokens, true, false, &r));
+        HIP_TRY(hipStreamSynchronize(nullptr));
+        *error_word = *r.error_word;
+    } else {
+        HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
+    }
     if (*error_word) {
         HIP_TRY(hipMemset(work->error_word, 0, 4));
         return PF_HIP_OK;
     }
-    HIP_TRY(hipMemcpy(ids, work->ids, tokens * K * 4, hipMemcpyDeviceToHost));
+    if (staged) memcpy(ids, r.ids, tokens * K * 4);
+    else HIP_TRY(hipMemcpy(ids, work->ids, tokens * K * 4, hipMemcpyDeviceToHost));
     return PF_HIP_OK;
 }
 
@@ -804,8 +911,15 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
             expert_bytes[j] != place.expert_bytes || scale_offsets[j] != place.scale_offset)
             return PF_HIP_E_ARGUMENT;
     }
-    HIP_TRY(hipMemcpy(work->slots, slots, tokens * K * 4, hipMemcpyHostToDevice));
-    PfKernelArgs a = make_args(moe, work, work->x, H, work->y, H);
+    const bool staged = through_host_block(work, tokens);
+    const HostBlock b = host_block(&moe->desc, work->host);
+    if (staged) {
+        memcpy(b.slots, slots, tokens * K * 4);
+        HIP_TRY(hipMemcpyAsync(work->slots, b.slots, tokens * K * 4, hipMemcpyHostToDevice, nullptr));
+    } else {
+        HIP_TRY(hipMemcpy(work->slots, slots, tokens * K * 4, hipMemcpyHostToDevice));
+    }
+    PfKernelArgs a = make_args(moe, work, work->x, H, staged ? (float *)(work->host_device + b.y_offset) : work->y, H);
     for (int j = 0; j < 3; j++) {
         const int t = 1 + j;
         const bool tiled = (tiled_mask >> j) & 1u;
@@ -823,6 +937,20 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
         pf_launch_general(a, (int)tokens, nullptr, 0, 3);
     }
     HIP_TRY(hipGetLastError());
+    if (staged) {
+        HostResults r;
+        HIP_TRY(fetch_results(work, b, tokens, ids != nullptr, weights != nullptr, &r));
+        HIP_TRY(hipStreamSynchronize(nullptr));
+        *error_word = *r.error_word;
+        if (*error_word) {
+            HIP_TRY(hipMemset(work->error_word, 0, 4));
+            return PF_HIP_OK;
+        }
+        rows_out(y, y_pitch_bytes, b.y, H * 4, tokens);
+        if (ids) rows_out(ids, ids_pitch_bytes, r.ids, K * 4, tokens);
+        if (weights) rows_out(weights, weights_pitch_bytes, r.weights, K * 4, tokens);
+        return PF_HIP_OK;
+    }
     HIP_TRY(hipMemcpy(error_word, work->error_word, 4, hipMemcpyDeviceToHost));
     if (*error_word) {
         HIP_TRY(hipMemset(work->error_word, 0, 4));

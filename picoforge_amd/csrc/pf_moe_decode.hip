@@ -489,12 +489,24 @@ __device__ __forceinline__ void stage_tables(uint32_t *lds, const uint32_t *glob
 
 template <int FMT> __host__ __device__ constexpr int table_words() { return FMT == PF_IQ2_XXS ? 8192 : 0; }
 
+// Requests fields of the kernel's argument block now, together.  Left to itself the compiler fetches a field where it
+// is first used, behind the wait for the fields before it: several turns to the scalar cache, one after the other,
+// before a kernel's first weight bytes are asked for.
+__device__ __forceinline__ void pf_args_now() {}
+template <typename T, typename... Rest>
+__device__ __forceinline__ void pf_args_now(T &field, Rest &...rest) {
+    asm volatile("" : "+s"(field));
+    pf_args_now(rest...);
+}
+
+
 // ---- kernel 1: router logits -----------------------------------------------------------------
 // One F32 row per wave, all tokens: blocks [0, router_blocks) take the experts' rows, the
 // last block's first wave the shared router row (its sigmoid scales the shared expert).
 #define ROUTER_CHUNKS 10   // 16-byte pieces of a router row per lane: hidden <= 2560
 template <int NT>
 __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks, int tokens) {
+    pf_args_now(a.w[0], a.w[7], a.x, a.x_pitch, a.logits, a.logit_ssq, a.shared_scale, a.ximg, router_blocks, tokens);
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     if ((int)blockIdx.x > router_blocks) {
         // workgroups beyond the router's (launched where the next kernel reads them): the tokens' digit images,
@@ -1619,6 +1631,8 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
     __shared__ float partial[17][16];
     extern __shared__ int lds[];   // IQ2_XXS: the waves' magnitude grids; [slot][image words of the widest activation row]; [slot][rows * runs] products
     constexpr bool GRID = FMT == PF_IQ2_XXS || FMTS == PF_IQ2_XXS;
+    pf_args_now(a.ids, a.route_weights, a.shared_scale, a.aimg, a.hc_residual, a.wt[3], a.wt[6], a.w[3], a.w[6], a.expert_bytes[3],
+                a.shared_inter, a.down_physical, a.hc_streams, a.error_word, rows);
     const int token = (int)blockIdx.y;
     q4t_at_token(a, token);
     const int H = a.hidden, K = a.top_k, lane = pf_lane();

@@ -133,6 +133,8 @@ struct PfHipWork {
     uint16_t *x16, *act16, *sact16;  // prefill buffers (allocated when cap exceeds the decode path's batch)
     float *x_scale, *act_scale, *sact_scale, *x_max2, *down;
     uint32_t *counts, *offsets, *pair_to_row, *row_to_pair, *group_bad, *tiles;
+    uint8_t *host;                  // pinned host block for the host-pointer forwards of short batches (null: not available)
+    uint8_t *host_device;           // the same block as the kernels address it (they write the output rows straight into it)
     int stage_limit;                // profiling: launch only the first so many kernels of a forward; 0 = all
     int force_general;               // tests: run the general kernels even where the decode path applies
 };

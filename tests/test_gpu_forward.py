@@ -1,4 +1,5 @@
 """GPU parity of qwen4_moe_forward: the HIP path through the C-ABI against the CPU oracle."""
+import ctypes as C
 import sys
 
 import numpy as np
@@ -191,6 +192,32 @@ def test_decode_unnormalised_weights_and_repeat_calls(product, oracle, norm):
         for _ in range(3):                        # the workspace is reused call after call
             _, y, ids, w = layer.forward(x)
             assert_parity(y, ids, w, *want, label=f"norm={norm}")
+
+
+@pytest.mark.parametrize("tokens", [1, 5, 16, 17])
+def test_host_pointer_forward_with_padded_rows_and_without_routes(product, tokens):
+    """Batches of up to 16 tokens pass through the workspace's pinned block (the output rows are written into it by the
+    kernels, ids and weights arrive in one copy), longer ones through one copy per buffer: both must place rows at the
+    caller's pitches, leave the padding alone and give the same rows with and without the routes asked for."""
+    cfg = abi.moe_config(512, 64, 4, 256, 256)
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, tokens, seed=31)
+    h, k = cfg.hidden_size, cfg.top_k
+    with pf.MoeLayer(product, cfg, weights, 32) as layer:
+        _, y0, ids0, w0 = layer.forward(x)
+        _, y1, _, _ = layer.forward(x, want_routes=False)
+        assert np.array_equal(y0, y1)
+        wide_x = np.full((tokens, h + 24), 7.0, dtype=np.float32)
+        wide_x[:, :h] = x
+        wide_y = np.full((tokens, h + 8), -5.0, dtype=np.float32)
+        wide_ids = np.full((tokens, k + 3), 0xABCDEF01, dtype=np.uint32)
+        wide_w = np.full((tokens, k + 1), -5.0, dtype=np.float32)
+        routes = abi.Qwen4MoeRoutes(abi.u32_view(wide_ids, cols=k), abi.f32_view(wide_w, cols=k))
+        st = product.forward(layer.handle, abi.f32_view(wide_x, cols=h), abi.f32_view(wide_y, cols=h), C.byref(routes),
+                             layer.work, C.byref(layer.err))
+        assert st == abi.QW4_OK, layer.err.detail
+        assert np.array_equal(wide_y[:, :h], y0) and (wide_y[:, h:] == -5.0).all()
+        assert np.array_equal(wide_ids[:, :k], ids0) and (wide_ids[:, k:] == 0xABCDEF01).all()
+        assert np.array_equal(wide_w[:, :k], w0) and (wide_w[:, k:] == -5.0).all()
 
 
 def test_close_logits_are_rerouted_in_serial_order(product, oracle):
