@@ -209,29 +209,70 @@ void pf_launch_row_norm2(const float *d_w, int rows, int cols, float *d_out, hip
 
 // ---- router logits by FP32 MFMA ----------------------------------------------------------------
 // Workgroup = one 32-token x 32-expert tile, its four waves a quarter of the columns each (the
-// partial tiles are added in wave order); operands straight from global memory (the lines a
-// lane touches are consumed over the following iterations from the vector cache).
-// Column E is the shared router.  Also writes the routing tolerance's bound on the sum of
-// squared products, max(x)^2 * |w_e|^2.
+// partial tiles are added in wave order).  Column E is the shared router.  Also writes the routing
+// tolerance's bound on the sum of squared products, max(x)^2 * |w_e|^2.
+//
+// Operands.  A product step wants, from lane (i, kk), element k = kk of row i: fetched like that
+// from global memory, every load instruction touches 32 rows, and the address unit, which takes a
+// cache line at a time, sets the pace (the kernel took 3.3 times the matrix cores' time at the
+// benchmark shape).
+// Instead a wave fetches a 32-column piece of its 32 + 32 rows as eight instructions of eight whole
+// 128-byte lines each (lane = 8 * row + 16-byte piece), stores it into LDS of its own at a row
+// pitch of 144 bytes, and reads its operands from there, 16 bytes a lane: columns
+// 4 (2 c + kk) .. + 3 for steps 4 c .. 4 c + 3, the same pairing for both operands.  The next
+// piece's global loads are on their way while the current one is multiplied; the LDS is the
+// wave's alone, so no barrier is needed before the partial tiles meet.
+typedef float float4v __attribute__((ext_vector_type(4)));
+#define PF_ROUTER_PITCH 36   // floats between rows of a staged piece: eight neighbouring lanes' 16-byte reads cover all banks
 __global__ void __launch_bounds__(256) pf_k_pf_router(PfKernelArgs a, int tokens) {
     __shared__ float partial[3][16][64];
+    __shared__ __align__(16) float staged[4][2][32 * PF_ROUTER_PITCH];   // [wave][x | w][row][column]
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     const int t0 = blockIdx.x * 32, e0 = blockIdx.y * 32;
     if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) a.route_flags[0] = 0;   // the routing's list starts empty
     const int i = lane & 31, kk = lane >> 5;
-    const int t = min(t0 + i, tokens - 1), e = min(e0 + i, E);
-    // the four waves share the tile and split the columns into quarters (hidden is a multiple of 32)
-    const int q0 = wave * (H / 32), q1 = q0 + H / 32;
-    const float4 *xp = reinterpret_cast<const float4 *>(a.x + (size_t)t * a.x_pitch) + kk;
-    const float4 *wp = reinterpret_cast<const float4 *>(e < E ? a.w[0] + (size_t)e * H * 4 : a.w[7]) + kk;
+    // the four waves split the rows' 128-byte lines (hidden is a multiple of 32)
+    const int lines = H / 32, l0 = lines * wave / 4, l1 = lines * (wave + 1) / 4;
+    const int lr = lane >> 3, piece = lane & 7;   // fetch: row within a group of eight, 16-byte piece of the line
+    const float4v *xsrc[4], *wsrc[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const int t = min(t0 + 8 * g + lr, tokens - 1), e = min(e0 + 8 * g + lr, E);
+        xsrc[g] = reinterpret_cast<const float4v *>(a.x + (size_t)t * a.x_pitch) + piece;
+        wsrc[g] = reinterpret_cast<const float4v *>(e < E ? a.w[0] + (size_t)e * H * 4 : a.w[7]) + piece;
+    }
+    float *xs = staged[wave][0], *ws = staged[wave][1];
     float16v acc = {0};
-#pragma unroll 4
-    for (int q = q0; q < q1; q++) {
-        const float4 xv = xp[2 * q], wv = wp[2 * q];
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.x, wv.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.y, wv.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.z, wv.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.w, wv.w, acc, 0, 0, 0);
+    if (l0 < l1) {
+        float4v xg[4], wg[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) { xg[g] = xsrc[g][8 * l0]; wg[g] = wsrc[g][8 * l0]; }
+        for (int l = l0; l < l1; l++) {
+            // the piece fetched last into LDS (after the reads of the piece before it, in the wave's program order),
+            // then the next one's loads on their way (the last step fetches its own piece again; two pieces ahead
+            // measured no faster)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                *reinterpret_cast<float4v *>(xs + (8 * g + lr) * PF_ROUTER_PITCH + 4 * piece) = xg[g];
+                *reinterpret_cast<float4v *>(ws + (8 * g + lr) * PF_ROUTER_PITCH + 4 * piece) = wg[g];
+            }
+            const int next = l + 1 < l1 ? l + 1 : l;
+#pragma unroll
+            for (int g = 0; g < 4; g++) { xg[g] = xsrc[g][8 * next]; wg[g] = wsrc[g][8 * next]; }
+            float4v xv[4], wv[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                xv[c] = *reinterpret_cast<const float4v *>(xs + i * PF_ROUTER_PITCH + 4 * (2 * c + kk));
+                wv[c] = *reinterpret_cast<const float4v *>(ws + i * PF_ROUTER_PITCH + 4 * (2 * c + kk));
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[c].x, wv[c].x, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[c].y, wv[c].y, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[c].z, wv[c].z, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[c].w, wv[c].w, acc, 0, 0, 0);
+            }
+        }
     }
     if (wave > 0) {
 #pragma unroll
@@ -1198,16 +1239,29 @@ __global__ void __launch_bounds__(256) pf_k_pf_combine(PfKernelArgs a, int token
     __syncthreads();
     const float ss = a.shared_scale[t];
     bool bad = false;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) {
-        PfOutputRegs out_regs;
-        pf_output_prefetch(a, t, c, out_regs);
-        float sum = 0.0f;
-        for (int s = 0; s < K; s++) {
-            const float term = weights[s] * a.down[(size_t)rows[s] * H + c];
-            sum += term;
+    // four columns a thread; the rows of sixteen slots at a time are all requested before the first of their sums
+    for (int c = 4 * threadIdx.x; c < H; c += 4 * blockDim.x) {
+        PfOutputRegs out_regs[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) pf_output_prefetch(a, t, c + j, out_regs[j]);
+        const float4 sh = *reinterpret_cast<const float4 *>(a.down + (size_t)(P + t) * H + c);
+        float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int s0 = 0; s0 < K; s0 += 16) {
+            float4 v[16];
+#pragma unroll
+            for (int s = 0; s < 16; s++)
+                if (s0 + s < K) v[s] = *reinterpret_cast<const float4 *>(a.down + (size_t)rows[s0 + s] * H + c);
+#pragma unroll
+            for (int s = 0; s < 16; s++) {
+                if (s0 + s < K) {
+                    const float w = weights[s0 + s];
+                    sum[0] += w * v[s].x; sum[1] += w * v[s].y; sum[2] += w * v[s].z; sum[3] += w * v[s].w;
+                }
+            }
         }
-        const float y = sum + ss * a.down[(size_t)(P + t) * H + c];
-        bad |= !pf_output_commit(a, t, c, y, out_regs);
+        const float y[4] = {sum[0] + ss * sh.x, sum[1] + ss * sh.y, sum[2] + ss * sh.z, sum[3] + ss * sh.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) bad |= !pf_output_commit(a, t, c + j, y[j], out_regs[j]);
     }
     if (__any(bad) && pf_lane() == 0) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
 }
