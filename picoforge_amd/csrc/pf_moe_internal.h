@@ -149,7 +149,8 @@ void pf_launch_router_slabs(const float *d_src, int experts, int hidden, float *
 int pf_route_exact_device(const float *d_logits, int tokens, int experts, int top_k, int norm,
                           float *d_probs, uint32_t *d_ids, float *d_weights, uint32_t *d_error,
                           unsigned long long *d_bad_row, hipStream_t stream);
-// histogram, scan, row tiles and stable placement in one launch; false (nothing launched) when the pairs do not fit its LDS
+// histogram, scan, row tiles and placement (an expert's rows in no particular order) in one launch; false (nothing
+// launched) for more pairs or experts than it takes
 bool pf_launch_group_fused(const uint32_t *d_ids, int pairs, int experts, int tokens, uint32_t *d_offsets, uint32_t *d_tiles,
                            uint32_t *d_pair_to_row, uint32_t *d_row_to_pair, hipStream_t stream);
 void pf_launch_group_place(const uint32_t *d_ids, int pairs, int experts, const uint32_t *d_offsets,

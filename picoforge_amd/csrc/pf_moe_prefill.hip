@@ -3,7 +3,7 @@
 //
 //   pf_k_rows_to_half   f32 rows -> power-of-two scaled fp16 pairs (high + low part) and the
 //                       per-32-group sums, the scale, max^2, finite check
-//   pf_k_pf_router      router logits [T, E] (+ the shared router as column E) by FP32 MFMA
+//   pf_k_pf_router      router logits [T, E] by FP32 MFMA
 //   routing, grouping   the kernels of pf_moe_route.hip (serial-order re-route of close tokens,
 //                       histogram / scan / stable placement)
 //   pf_k_pf_gemm        grouped product over the rows of each expert (the shared expert is
@@ -63,9 +63,14 @@ void pf_launch_q4k_tile(const uint8_t *d_src, uint8_t *d_dst, size_t rows, int b
 // One workgroup per row (cols a multiple of 32).  scale = 2^e with max|row| / scale in
 // [0.5, 1) (1 for a zero row).  Thread j converts the eight values 8j..8j+7; four neighbouring
 // threads form one 32-group.
+// gate (may be null): a row of `cols` weights; gate_out[row] = sigmoid(row . gate), the shared router's scale (four
+// partial sums a lane, lanes and waves added in a fixed order).
 __global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_t src_pitch, int cols, half_t *dst,
-                                                         float *scale_out, float *max2_out, uint32_t *error_word) {
+                                                         float *scale_out, float *max2_out, uint32_t *error_word,
+                                                         const float *gate, float *gate_out) {
     __shared__ float part[4];
+    __shared__ float dots[4];
+    float dot = 0.0f;
     const size_t row = blockIdx.x;
     const float *s = src + row * src_pitch;
     float m = 0.0f;
@@ -88,6 +93,10 @@ __global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_
     for (int j = threadIdx.x; j < cols / 8; j += blockDim.x) {
         const float4 a = reinterpret_cast<const float4 *>(s)[2 * j], b = reinterpret_cast<const float4 *>(s)[2 * j + 1];
         const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        if (gate) {
+            const float4 ga = reinterpret_cast<const float4 *>(gate)[2 * j], gb = reinterpret_cast<const float4 *>(gate)[2 * j + 1];
+            dot += ((a.x * ga.x + a.y * ga.y) + (a.z * ga.z + a.w * ga.w)) + ((b.x * gb.x + b.y * gb.y) + (b.z * gb.z + b.w * gb.w));
+        }
         half8v hi, lo;
         float sum = 0.0f;
 #pragma unroll
@@ -108,6 +117,16 @@ __global__ void __launch_bounds__(256) pf_k_rows_to_half(const float *src, size_
             half_t *sums = out + 2 * cols + 16 * (g >> 3) + 8 * (g & 1) + ((g & 7) >> 1);
             sums[0] = sh;
             sums[4] = sl;
+        }
+    }
+    if (gate) {   // uniform
+        dot = pf_wave_sum(dot);
+        if (pf_lane() == 0) dots[threadIdx.x >> 6] = dot;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const float z = (dots[0] + dots[1]) + (dots[2] + dots[3]);
+            gate_out[row] = pf_sigmoid(z);
+            if (!pf_finite(z)) atomicOr(error_word, PF_HIP_ERR_NONFINITE);
         }
     }
     if (threadIdx.x == 0) {
@@ -191,7 +210,7 @@ static void launch_rows_to_half(const float *src, size_t src_pitch, int cols, si
                            dst, scale_out, max2_out, error_word);
     else
         hipLaunchKernelGGL(pf_k_rows_to_half, dim3((unsigned)rows), dim3(256), 0, stream, src, src_pitch, cols, dst, scale_out,
-                           max2_out, error_word);
+                           max2_out, error_word, (const float *)nullptr, (float *)nullptr);
 }
 
 // squared norm of every router row (once, at upload)
@@ -209,8 +228,8 @@ void pf_launch_row_norm2(const float *d_w, int rows, int cols, float *d_out, hip
 
 // ---- router logits by FP32 MFMA ----------------------------------------------------------------
 // Workgroup = one 32-token x 32-expert tile, its four waves a quarter of the columns each (the
-// partial tiles are added in wave order).  Column E is the shared router.  Also writes the routing
-// tolerance's bound on the sum of squared products, max(x)^2 * |w_e|^2.
+// partial tiles are added in wave order).  Also writes the routing tolerance's bound on the sum of
+// squared products, max(x)^2 * |w_e|^2.  (The shared router's logit comes from pf_k_rows_to_half.)
 //
 // Operands.  A product step wants, from lane (i, kk), element k = kk of row i: fetched like that
 // from global memory, every load instruction touches 32 rows, and the address unit, which takes a
@@ -237,9 +256,9 @@ __global__ void __launch_bounds__(256) pf_k_pf_router(PfKernelArgs a, int tokens
     const float4v *xsrc[4], *wsrc[4];
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-        const int t = min(t0 + 8 * g + lr, tokens - 1), e = min(e0 + 8 * g + lr, E);
+        const int t = min(t0 + 8 * g + lr, tokens - 1), e = min(e0 + 8 * g + lr, E - 1);
         xsrc[g] = reinterpret_cast<const float4v *>(a.x + (size_t)t * a.x_pitch) + piece;
-        wsrc[g] = reinterpret_cast<const float4v *>(e < E ? a.w[0] + (size_t)e * H * 4 : a.w[7]) + piece;
+        wsrc[g] = reinterpret_cast<const float4v *>(a.w[0] + (size_t)e * H * 4) + piece;
     }
     float *xs = staged[wave][0], *ws = staged[wave][1];
     float16v acc = {0};
@@ -287,15 +306,9 @@ __global__ void __launch_bounds__(256) pf_k_pf_router(PfKernelArgs a, int tokens
 #pragma unroll
     for (int r = 0; r < 16; r++) {
         const int row = t0 + 8 * (r >> 2) + 4 * kk + (r & 3);
-        if (row >= tokens || col > E) continue;
-        const float z = acc[r];
-        if (col < E) {
-            a.logits[(size_t)row * E + col] = z;
-            a.logit_ssq[(size_t)row * E + col] = a.x_max2[row] * wn;
-        } else {
-            a.shared_scale[row] = pf_sigmoid(z);
-            if (!pf_finite(z)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
-        }
+        if (row >= tokens || col >= E) continue;
+        a.logits[(size_t)row * E + col] = acc[r];
+        a.logit_ssq[(size_t)row * E + col] = a.x_max2[row] * wn;
     }
 }
 
@@ -1325,9 +1338,11 @@ void pf_launch_prefill(const PfKernelArgs &a, int tokens, hipStream_t stream, in
     const int H = a.hidden, E = a.experts, K = a.top_k, I = a.inter, Is = a.shared_inter, P = tokens * K;
     const int last = stage_limit ? stage_limit : 4;
     // stage 1: fp16 parts of x, router logits
+    // (the shared router's column rides with the conversion: as a column of the router product it cost a 17th column
+    // tile of full depth, and 544 workgroups do not spread evenly over 256 compute units, 512 do)
     hipLaunchKernelGGL(pf_k_rows_to_half, dim3(tokens), dim3(256), 0, stream, a.x, a.x_pitch, H, (half_t *)a.x16, a.x_scale,
-                       a.x_max2, a.error_word);
-    hipLaunchKernelGGL(pf_k_pf_router, dim3((tokens + 31) / 32, (E + 1 + 31) / 32), dim3(256), 0, stream, a, tokens);
+                       a.x_max2, a.error_word, reinterpret_cast<const float *>(a.w[7]), a.shared_scale);
+    hipLaunchKernelGGL(pf_k_pf_router, dim3((tokens + 31) / 32, (E + 31) / 32), dim3(256), 0, stream, a, tokens);
     if (last < 2) return;
     // stage 2: routes and grouping
     pf_launch_route(a, tokens, stream);

@@ -376,72 +376,55 @@ void pf_launch_group_place(const uint32_t *d_ids, int pairs, int experts, const 
 }
 
 // ---- grouping in one launch (the prefill path) ---------------------------------------------------------
-// Every workgroup stages all ids in LDS, counts them there (LDS atomics), scans the counts, and its four waves place
-// their four experts' pairs as pf_k_group_place does; workgroup 0 also writes offsets[E + 1] and the row tiles
-// (tiles[0] = count, tiles[1 + i] = expert | tile index << 16; the shared expert = expert E with every token), as
-// pf_k_pf_scan_tiles does.  The histogram and the scan are repeated by every workgroup: a few microseconds of LDS
-// work against two kernel boundaries.
+// One workgroup of 1024 threads: counts the pairs per expert in LDS, scans the counts (offsets, and the row tiles:
+// tiles[0] = count, tiles[1 + i] = expert | tile index << 16; the shared expert = expert E with every token, as
+// pf_k_pf_scan_tiles lists them), and hands every pair the next free row of its expert through an LDS cursor.  The rows
+// of an expert are therefore in no particular order (pf_k_group_place keeps them in pair order): every row of the
+// grouped products is computed on its own and found again through pair_to_row, so the order changes no result, and a
+// walk over all pairs per expert, which the order costs, took three times as long as everything else here.
 #define GROUP_FUSED_MAX_PAIRS 32768
 #define GROUP_FUSED_MAX_EXPERTS 2047
-__global__ void __launch_bounds__(256) pf_k_group_fused(const uint32_t *ids, int pairs, int E, int tokens, uint32_t *offsets,
-                                                        uint32_t *tiles, uint32_t *pair_to_row, uint32_t *row_to_pair) {
+__global__ void __launch_bounds__(1024) pf_k_group_fused(const uint32_t *ids, int pairs, int E, int tokens, uint32_t *offsets,
+                                                         uint32_t *tiles, uint32_t *pair_to_row, uint32_t *row_to_pair) {
     extern __shared__ __align__(16) uint32_t fused_lds[];
-    __shared__ uint32_t rows_before[256], tiles_before[256];
-    const int padded = (pairs + 511) & ~511, tid = threadIdx.x, lane = pf_lane();
-    uint32_t *staged = fused_lds, *counts = staged + padded, *starts = counts + (E + 1);
-    // all of a thread's loads are requested before the first is stored (pairs on a 16-byte boundary of ids; the
-    // ragged end is read id by id); beyond the pairs: no expert
-    for (int i0 = 4 * tid; i0 < padded; i0 += 4 * 256 * 8) {
-        uint4 held[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int i = i0 + 4 * 256 * j;
-            uint4 v = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-            if (i + 4 <= pairs) {
-                v = *reinterpret_cast<const uint4 *>(ids + i);
-            } else if (i < pairs) {
-                v.x = ids[i];
-                if (i + 1 < pairs) v.y = ids[i + 1];
-                if (i + 2 < pairs) v.z = ids[i + 2];
-            }
-            held[j] = v;
-        }
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const int i = i0 + 4 * 256 * j;
-            if (i < padded) *reinterpret_cast<uint4 *>(staged + i) = held[j];
-        }
-    }
-    for (int e = tid; e <= E; e += 256) counts[e] = 0;
+    __shared__ uint32_t wave_rows[16], wave_tiles[16];
+    const int tid = threadIdx.x, quads = pairs / 4;
+    uint32_t *counts = fused_lds, *cursor = counts + (E + 1);
+    for (int e = tid; e <= E; e += 1024) counts[e] = 0;
     __syncthreads();
-    for (int i = tid; i < pairs; i += 256) {
-        const uint32_t id = staged[i];
+    // four pairs a thread and step (ids on a 16-byte boundary), the ragged end pair by pair
+    for (int q = tid; q < quads; q += 1024) {
+        const uint4 v = reinterpret_cast<const uint4 *>(ids)[q];
+        if (v.x < (uint32_t)E) atomicAdd(&counts[v.x], 1u);
+        if (v.y < (uint32_t)E) atomicAdd(&counts[v.y], 1u);
+        if (v.z < (uint32_t)E) atomicAdd(&counts[v.z], 1u);
+        if (v.w < (uint32_t)E) atomicAdd(&counts[v.w], 1u);
+    }
+    for (int p = 4 * quads + tid; p < pairs; p += 1024) {
+        const uint32_t id = ids[p];
         if (id < (uint32_t)E) atomicAdd(&counts[id], 1u);
     }
     __syncthreads();
     // exclusive scan of the counts (rows) and of the row-tile counts, thread t owning `per` consecutive experts
-    const int per = (E + 1 + 255) / 256, lo = tid * per, hi = min(E + 1, lo + per);
+    const int per = (E + 1 + 1023) / 1024, lo = tid * per, hi = min(E + 1, lo + per);
     uint32_t rows = 0, ntiles = 0;
     for (int e = lo; e < hi; e++) {
         const uint32_t c = e < E ? counts[e] : (uint32_t)tokens;
         if (e < E) rows += c;
         ntiles += (c + 31u) / 32u;
     }
-    rows_before[tid] = rows;
-    tiles_before[tid] = ntiles;
-    __syncthreads();
+    // inclusive scan over the 1024 threads: within a wave by shuffles, then the sixteen waves' totals through LDS
+    const int lane = pf_lane(), wave = tid >> 6;
     uint32_t run_rows = rows, run_tiles = ntiles;
-    for (int d = 1; d < 256; d <<= 1) {
-        const uint32_t add_rows = tid >= d ? rows_before[tid - d] : 0u, add_tiles = tid >= d ? tiles_before[tid - d] : 0u;
-        __syncthreads();
-        run_rows += add_rows;
-        run_tiles += add_tiles;
-        rows_before[tid] = run_rows;
-        tiles_before[tid] = run_tiles;
-        __syncthreads();
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t up_rows = __shfl_up(run_rows, d), up_tiles = __shfl_up(run_tiles, d);
+        if (lane >= d) { run_rows += up_rows; run_tiles += up_tiles; }
     }
-    const bool writer = blockIdx.x == 0;
-    if (writer && tid == 255) {
+    if (lane == 63) { wave_rows[wave] = run_rows; wave_tiles[wave] = run_tiles; }
+    __syncthreads();
+    for (int w = 0; w < wave; w++) { run_rows += wave_rows[w]; run_tiles += wave_tiles[w]; }
+    if (tid == 1023) {
         offsets[E] = run_rows;
         tiles[0] = run_tiles;
     }
@@ -449,53 +432,32 @@ __global__ void __launch_bounds__(256) pf_k_group_fused(const uint32_t *ids, int
     for (int e = lo; e < hi; e++) {
         const uint32_t c = e < E ? counts[e] : (uint32_t)tokens, n = (c + 31u) / 32u;
         if (e < E) {
-            starts[e] = row;
-            if (writer) offsets[e] = row;
+            cursor[e] = row;
+            offsets[e] = row;
             row += c;
         }
-        if (writer)
-            for (uint32_t i = 0; i < n; i++) tiles[1 + at + i] = (uint32_t)e | (i << 16);
+        for (uint32_t i = 0; i < n; i++) tiles[1 + at + i] = (uint32_t)e | (i << 16);
         at += n;
     }
     __syncthreads();
-    // placement: one wave per expert walks the pairs in order (rank = earlier pairs of the same expert)
-    const int e = blockIdx.x * 4 + (tid >> 6);
-    if (e >= E || counts[e] == 0) return;
-    uint32_t base = starts[e];
-    const unsigned long long below = (1ull << lane) - 1ull;
-    auto place = [&](const uint4 &v, int p0) {   // 256 pairs, lane l holds pairs 4l .. 4l + 3 of them
-        const bool h0 = v.x == (uint32_t)e, h1 = v.y == (uint32_t)e, h2 = v.z == (uint32_t)e, h3 = v.w == (uint32_t)e;
-        const int mine = (int)h0 + (int)h1 + (int)h2 + (int)h3;
-        const unsigned long long any = __ballot(mine != 0);
-        if (!any) return;
-        // pairs of lower lanes come first, then this lane's own earlier ones
-        const unsigned long long m0 = __ballot(h0), m1 = __ballot(h1), m2 = __ballot(h2), m3 = __ballot(h3);
-        uint32_t r = base + __popcll(m0 & below) + __popcll(m1 & below) + __popcll(m2 & below) + __popcll(m3 & below);
-        const int p = p0 + 4 * lane;
-        if (h0) { pair_to_row[p] = r; row_to_pair[r] = (uint32_t)p; r++; }
-        if (h1) { pair_to_row[p + 1] = r; row_to_pair[r] = (uint32_t)(p + 1); r++; }
-        if (h2) { pair_to_row[p + 2] = r; row_to_pair[r] = (uint32_t)(p + 2); r++; }
-        if (h3) { pair_to_row[p + 3] = r; row_to_pair[r] = (uint32_t)(p + 3); }
-        base += __popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3);
+    auto place = [&](uint32_t id, int p) {
+        if (id >= (uint32_t)E) return;
+        const uint32_t r = atomicAdd(&cursor[id], 1u);
+        pair_to_row[p] = r;
+        row_to_pair[r] = (uint32_t)p;
     };
-    const uint4 *quads = reinterpret_cast<const uint4 *>(staged);
-    for (int p0 = 0; p0 < padded; p0 += 512) {
-        const uint4 va = quads[p0 / 4 + lane], vb = quads[p0 / 4 + 64 + lane];
-        place(va, p0);
-        place(vb, p0 + 256);
+    for (int q = tid; q < quads; q += 1024) {
+        const uint4 v = reinterpret_cast<const uint4 *>(ids)[q];
+        place(v.x, 4 * q); place(v.y, 4 * q + 1); place(v.z, 4 * q + 2); place(v.w, 4 * q + 3);
     }
+    for (int p = 4 * quads + tid; p < pairs; p += 1024) place(ids[p], p);
 }
 
 bool pf_launch_group_fused(const uint32_t *d_ids, int pairs, int experts, int tokens, uint32_t *d_offsets, uint32_t *d_tiles,
                            uint32_t *d_pair_to_row, uint32_t *d_row_to_pair, hipStream_t stream) {
     if (pairs <= 0 || pairs > GROUP_FUSED_MAX_PAIRS || experts > GROUP_FUSED_MAX_EXPERTS || (reinterpret_cast<uintptr_t>(d_ids) & 15)) return false;
-    const size_t lds = ((size_t)((pairs + 511) & ~511) + 2 * ((size_t)experts + 1)) * sizeof(uint32_t);
-    static bool configured = false;   // more than the default 64 KB of dynamic LDS for the longer chunks
-    if (!configured) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_group_fused), hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-        configured = true;
-    }
-    hipLaunchKernelGGL(pf_k_group_fused, dim3((experts + 3) / 4), dim3(256), lds, stream, d_ids, pairs, experts, tokens, d_offsets, d_tiles,
+    const size_t lds = 2 * ((size_t)experts + 1) * sizeof(uint32_t);
+    hipLaunchKernelGGL(pf_k_group_fused, dim3(1), dim3(1024), lds, stream, d_ids, pairs, experts, tokens, d_offsets, d_tiles,
                        d_pair_to_row, d_row_to_pair);
     return true;
 }
