@@ -219,9 +219,10 @@ int pf_hip_exact_combine_host(const float *down, const uint64_t *pair_to_row, co
  * layout for the pool's slot count), the slot count and the pairs' slots to the second, which runs the
  * expert products and the combine.  pf_hip_moe_forward_* refuse such a layer.
  * tiled_mask, the same in both calls: bit j set when region j holds Q4_K slots in the tile order (what
- * pf_hip_pool_store writes where pf_hip_pool_slot_tiled says so).  With all three set, batches of up to 16
- * tokens run the decode kernels on the slots (the first call the router kernel and the routing, the second
- * the expert kernels); otherwise the general kernels. */
+ * pf_hip_pool_store writes where pf_hip_pool_slot_tiled says so).  With every Q4_K region set -- all three
+ * of a layer that is Q4_K throughout, gate and up of one in the q4 checkpoint profile (MXFP4 down, Q8_0
+ * shared expert) -- batches of up to 16 tokens run the decode kernels on the slots (the first call the router
+ * kernel and the routing, the second the expert kernels); otherwise the general kernels. */
 int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
                                    size_t tokens, uint32_t tiled_mask, uint32_t *ids, uint32_t *error_word);
 int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const void *const regions[3],

@@ -306,15 +306,18 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             }
         }
     }
-    // A streamed layer that is Q4_K throughout: tile-ordered copies of its shared expert, so that short batches run the
-    // tile decode kernels on pool slots kept in tile order (the routed tensors are not here to be copied).
+    // A streamed layer that is Q4_K throughout, or in the q4 checkpoint profile (Q4_K gate and up, MXFP4 down, Q8_0 shared
+    // expert): tile-ordered copies of its shared expert's tensors as the resident layer keeps them, so that short batches
+    // run the tile decode kernels on pool slots (Q4_K slots in tile order; the routed tensors are not here to be copied).
     if (m->streamed) {
-        bool all_q4k = true;
+        bool all_q4k = true, q4_profile = desc->type[1] == PF_Q4_K && desc->type[2] == PF_Q4_K && desc->type[3] == PF_MXFP4;
         for (int a = 1; a <= 6; a++) all_q4k &= desc->type[a] == PF_Q4_K;
+        for (int a = 4; a <= 6; a++) q4_profile &= desc->type[a] == PF_Q8_0;
+        const int combination = all_q4k ? 1 : q4_profile ? 4 : 0;
         const char *copy = getenv("PF_MOE_PREFILL_COPY");
-        if (all_q4k && pf_decode_supported(*desc) && (!copy || strcmp(copy, "0") != 0)) {
+        if (combination && pf_decode_supported(*desc) && (!copy || strcmp(copy, "0") != 0)) {
             hipError_t e = hipSuccess;
-            for (int a = 4; a <= 6 && e == hipSuccess; a++) {
+            for (int a = 4; a <= 6 && e == hipSuccess && combination == 1; a++) {
                 if (n_out[a] % 32) { e = hipErrorInvalidValue; break; }
                 e = hipMalloc((void **)&m->w_tiled[a], m->bytes[a]);
                 if (e == hipSuccess) {
@@ -322,15 +325,28 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
                     m->total_bytes += m->bytes[a];
                 }
             }
+            for (int a = 4; a <= 5 && e == hipSuccess && combination == 4; a++) {
+                if (n_out[a] % 32 || k_storage[a] % 64) { e = hipErrorInvalidValue; break; }
+                const size_t bytes = pf_q8t_expert_bytes((int)n_out[a], (int)(k_storage[a] / 64));
+                e = hipMalloc((void **)&m->w_qtile[a], bytes);
+                if (e == hipSuccess) {
+                    pf_launch_q8_tile(m->w[a], reinterpret_cast<const uint16_t *>(m->w[a] + m->scale_offset[a]), m->w_qtile[a],
+                                      n_out[a], m->blocks_per_row[a], nullptr);
+                    m->total_bytes += bytes;
+                }
+            }
             if (e == hipSuccess) e = hipDeviceSynchronize();
             if (e == hipSuccess) {
                 const uint8_t *tiled[8];
                 for (int a = 0; a < 8; a++) tiled[a] = a >= 1 && a <= 3 ? m->w[0] : m->w_tiled[a];   // 1..3: any non-null address, the pool's at forward time
-                m->stream_decode_ready = n_out[1] % 32 == 0 && n_out[3] % 32 == 0 && pf_decode_tile_layer(m->desc, tiled, m->w_itile, m->w_qtile) == 1;
+                const bool slots_tile = n_out[1] % 32 == 0 && (combination == 4 || n_out[3] % 32 == 0);
+                if (slots_tile && pf_decode_tile_layer(m->desc, tiled, m->w_itile, m->w_qtile) == combination) m->stream_decode = combination;
             } else {
                 (void)hipGetLastError();   // without the copies the general kernels serve every batch
-                for (int a = 4; a <= 6; a++)
+                for (int a = 4; a <= 6; a++) {
                     if (m->w_tiled[a]) { (void)hipFree(m->w_tiled[a]); m->w_tiled[a] = nullptr; }
+                    if (m->w_qtile[a]) { (void)hipFree(m->w_qtile[a]); m->w_qtile[a] = nullptr; }
+                }
             }
         }
     }
@@ -672,7 +688,7 @@ static int forward_enqueue(const PfHipMoe *moe, PfHipWork *work, const float *d_
 // 2 the matrix-core prefill kernels, 0 the general kernels.
 extern "C" int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t tokens) {
     if (!moe || !work || work->force_general) return 0;
-    if (moe->streamed) return moe->stream_decode_ready && tokens <= PF_TILE_DECODE_MAX_TOKENS ? 1 : 0;   // given a pool with tile-ordered slots
+    if (moe->streamed) return moe->stream_decode && tokens <= PF_TILE_DECODE_MAX_TOKENS ? 1 : 0;   // given a pool with tile-ordered slots
     if (moe->decode_ready && tokens <= decode_limit(moe)) return 1;
     if (moe->prefill_ready && work->down && tokens > PF_DECODE_MAX_TOKENS) return 2;
     return 0;
@@ -796,6 +812,8 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
     if (!x || !y || tokens > work->cap) return PF_HIP_E_ARGUMENT;
     const size_t H = moe->desc.hidden, K = moe->desc.top_k;
     if (through_host_block(work, tokens)) {
+        // (the whole sequence as one replayed graph measured slower, 50 us against 43: the copies become graph nodes
+        // of their own)
         const HostBlock b = host_block(&moe->desc, work->host);
         rows_in(b.x, x, x_pitch_bytes, H * 4, tokens);
         HIP_TRY(hipMemcpyAsync(work->x, b.x, tokens * H * 4, hipMemcpyHostToDevice, nullptr));
@@ -839,10 +857,12 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
 // region + slot * expert_bytes.  The general kernels serve both: streaming is bound by the reads that fill the pool.
 extern "C" int pf_hip_pool_slot_tiled(uint32_t gguf_type, size_t n_out) { return gguf_type == PF_Q4_K && n_out % 32 == 0; }
 
-// Short batches of a streamed Q4_K layer whose three pool regions hold tile-ordered slots run the tile decode kernels:
-// kernel 1 and the routing kernels in the first call, kernels 2 and 3 reading the pairs' slots in the second.
+// Short batches of a streamed layer whose Q4_K pool regions hold tile-ordered slots (all three of a Q4_K layer; gate and
+// up of the q4 checkpoint profile, whose MXFP4 down slots stay row by row) run the tile decode kernels: kernel 1 and the
+// routing kernels in the first call, kernels 2 and 3 reading the pairs' slots in the second.
 static bool streamed_decode(const PfHipMoe *moe, const PfHipWork *work, size_t tokens, uint32_t tiled_mask) {
-    return moe->stream_decode_ready && tiled_mask == 7u && tokens <= PF_TILE_DECODE_MAX_TOKENS && !work->force_general;
+    const uint32_t wanted = moe->stream_decode == 1 ? 7u : 3u;
+    return moe->stream_decode && tiled_mask == wanted && tokens <= PF_TILE_DECODE_MAX_TOKENS && !work->force_general;
 }
 
 extern "C" int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
@@ -932,7 +952,7 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
     a.pool_slots = pool_slots;
     if (streamed_decode(moe, work, tokens, tiled_mask)) {
         // kernel 1 ran in the first call (logits and the token rows' images are in the workspace): kernels 2 and 3 only
-        pf_launch_decode_q4k_experts(a, (int)tokens, nullptr);
+        pf_launch_decode_stream_experts(a, (int)tokens, nullptr);
     } else {
         pf_launch_general(a, (int)tokens, nullptr, 0, 3);
     }

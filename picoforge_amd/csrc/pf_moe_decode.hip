@@ -2015,6 +2015,7 @@ void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream,
 void pf_launch_decode_iq2(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
+void pf_launch_decode_q4profile_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);
 
 #if PF_DECODE_PART == 0
 void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
@@ -2022,8 +2023,9 @@ void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream,
     else launch_decode_tokens<PF_Q4_K, PF_Q4_K, PF_Q4_K>(a, tokens, stream, stage_limit);
 }
 
-void pf_launch_decode_q4k_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
-    launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K, true>(a, tokens, stream, 3);
+void pf_launch_decode_stream_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
+    if (decode_combination(a.type) == 4) pf_launch_decode_q4profile_experts(a, tokens, stream);
+    else launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K, true>(a, tokens, stream, 3);
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
@@ -2052,5 +2054,9 @@ void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t s
     if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq) == 4)
         launch_decode_q4t<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit);
     else launch_decode_tokens<PF_Q4_K, PF_MXFP4, PF_Q8_0>(a, tokens, stream, stage_limit);
+}
+
+void pf_launch_decode_q4profile_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
+    launch_q4t_experts<PF_Q4_K, PF_MXFP4, PF_Q8_0, true>(a, tokens, stream, 3);
 }
 #endif

@@ -107,7 +107,8 @@ struct PfHipMoe {
     size_t total_bytes;
     bool decode_ready;               // shapes and formats the specialised decode kernels cover
     bool prefill_ready;              // shapes and formats the matrix-core prefill kernels cover
-    bool stream_decode_ready;        // a streamed layer whose short batches run the tile decode kernels on pool slots in tile order
+    int stream_decode;               // a streamed layer whose short batches run the tile decode kernels on pool slots: 1 Q4_K
+                                     // throughout, 4 the q4 checkpoint profile (0: the general kernels serve every batch)
     float *w_norm2;                  // [experts] squared norm of each router row
     float *router_t;                 // [slab of 64 experts][hidden / 4][64][4] copy of the router
     uint8_t *w_tiled[8];             // tile-ordered second copy of the expert tensors for the prefill path (or null)
@@ -182,8 +183,9 @@ void pf_launch_q8_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8
                        hipStream_t stream);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
-// kernels 2 and 3 of the tile decode path for a Q4_K layer (expert streaming: kernel 1 ran in an earlier call)
-void pf_launch_decode_q4k_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);
+// kernels 2 and 3 of the tile decode path on pool slots, for a Q4_K layer or one in the q4 checkpoint profile (expert
+// streaming: kernel 1 ran in an earlier call)
+void pf_launch_decode_stream_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);
 void pf_launch_iq2_split(const uint8_t *d_gguf, uint8_t *d_payload, uint16_t *d_scales, size_t blocks,
                          hipStream_t stream);
 void pf_launch_block_split(const uint8_t *d_gguf, uint8_t *d_payload, uint8_t *d_scales, size_t blocks,

@@ -206,14 +206,16 @@ def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype, f
     os.close(fd)
 
 
-def test_streamed_q4k_layer_on_the_decode_kernels(product, oracle, tmp_path):
-    """A Q4_K layer of a shape the decode kernels cover, streamed through a pool that was told its formats: the
-    slots are kept in the tile order and batches of up to 16 tokens run the decode kernels on them (the router kernel
-    and the routing in the first device call, the expert kernels on the pairs' slots in the second); longer batches
-    run the general kernels on the same slots.  56 slots for 64 experts: evictions on the way."""
+@pytest.mark.parametrize("expert_type", [abi.GGUF_Q4_K, "q4"])
+def test_streamed_layer_on_the_decode_kernels(product, oracle, tmp_path, expert_type):
+    """A layer of a shape the decode kernels cover, Q4_K throughout or in the q4 checkpoint profile (Q4_K gate and up,
+    MXFP4 down, Q8_0 shared expert), streamed through a pool that was told its formats: the Q4_K slots are kept in the
+    tile order and batches of up to 16 tokens run the decode kernels on them (the router kernel and the routing in the
+    first device call, the expert kernels on the pairs' slots in the second); longer batches run the general kernels
+    on the same slots.  56 slots for 64 experts: evictions on the way."""
     cfg = abi.moe_config(512, 64, 4, 256, 256)
     tokens = 40
-    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, tokens, seed=67)
+    weights, x = make_layer_inputs(cfg, expert_type, tokens, seed=67)
     x[5] = x[4]                                              # two tokens of a batch share every expert
     sizes = [weights.raw[j].size // cfg.experts for j in (1, 2, 3)]
     filler = np.zeros(4096, np.uint8)

@@ -220,6 +220,33 @@ def test_host_pointer_forward_with_padded_rows_and_without_routes(product, token
         assert np.array_equal(wide_w[:, :k], w0) and (wide_w[:, k:] == -5.0).all()
 
 
+@pytest.mark.parametrize("tokens", [1, 4])
+def test_host_pointer_forwards_in_turn_share_one_pinned_block(product, oracle, tokens):
+    """Short batches stage their rows and results in one pinned block of the workspace: calls of different batch
+    sizes, with and without routes, and on the general kernels, one after the other, must not see each other's rows."""
+    cfg = abi.moe_config(512, 64, 4, 256, 256)
+    weights, x = make_layer_inputs(cfg, abi.GGUF_Q4_K, 2 * tokens + 3, seed=41)
+    xa, xb, xc = x[:tokens], x[tokens:2 * tokens], x[2 * tokens:]
+    want_a, want_b = forward_with(oracle, cfg, weights, xa), forward_with(oracle, cfg, weights, xb)
+    with pf.MoeLayer(product, cfg, weights, 8) as layer:
+        _, ya, ids_a, w_a = layer.forward(xa)
+        _, yb, _, _ = layer.forward(xb, want_routes=False)
+        assert_parity(ya, ids_a, w_a, *want_a, label="first call")
+        for turn in range(3):
+            _, y, ids, w = layer.forward(xb)
+            assert np.array_equal(y, yb), turn
+            assert_parity(y, ids, w, *want_b, label=f"turn {turn}, second input")
+            layer.forward(xc)                                       # another batch size in between
+            _, y, ids, w = layer.forward(xa)
+            assert np.array_equal(y, ya) and np.array_equal(ids, ids_a) and np.array_equal(w, w_a), turn
+            _, y, _, _ = layer.forward(xa, want_routes=False)
+            assert np.array_equal(y, ya), turn
+            layer.force_general()
+            _, yg, idsg, wg = layer.forward(xa)
+            assert_parity(yg, idsg, wg, *want_a, label=f"general kernels, turn {turn}")
+            layer.force_general(False)
+
+
 def test_close_logits_are_rerouted_in_serial_order(product, oracle):
     """Two router rows that differ in the last place give logits closer than the guard's
     tolerance: the token must go through the reference-order path and still match the oracle."""
