@@ -492,10 +492,15 @@ template <int FMT> __host__ __device__ constexpr int table_words() { return FMT 
 // Requests fields of the kernel's argument block now, together.  Left to itself the compiler fetches a field where it
 // is first used, behind the wait for the fields before it: several turns to the scalar cache, one after the other,
 // before a kernel's first weight bytes are asked for.
+// (The fields are inputs of the statement only: as in-out operands they would stay in their registers for certain, but a
+// pointer that has passed through the statement is no longer known to point to global memory, and its accesses become
+// flat ones.)
+template <typename T>
+__device__ __forceinline__ void pf_arg_now(const T &field) { asm volatile("" ::"s"(field)); }
 __device__ __forceinline__ void pf_args_now() {}
 template <typename T, typename... Rest>
-__device__ __forceinline__ void pf_args_now(T &field, Rest &...rest) {
-    asm volatile("" : "+s"(field));
+__device__ __forceinline__ void pf_args_now(const T &field, const Rest &...rest) {
+    pf_arg_now(field);
     pf_args_now(rest...);
 }
 
@@ -554,16 +559,17 @@ __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int route
             const float p0 = wv[c].x * xv[c].x, p1 = wv[c].y * xv[c].y, p2 = wv[c].z * xv[c].z, p3 = wv[c].w * xv[c].w;
             acc[t] += (p0 + p1) + (p2 + p3);
             sq[t] = fmaf(p0, p0, fmaf(p1, p1, fmaf(p2, p2, fmaf(p3, p3, sq[t]))));
-            bad |= !pf_finite(xv[c].x) || !pf_finite(xv[c].y) || !pf_finite(xv[c].z) || !pf_finite(xv[c].w);
         }
     }
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         const float z = pf_wave_sum(acc[t]), s2 = pf_wave_sum(sq[t]);
         if (lane == 0 && t < nt) {
+            // a nonfinite activation makes every product with it nonfinite (0 * inf is NaN), and a sum with a nonfinite
+            // term stays nonfinite: the rows are not looked through element by element
+            if (!pf_finite(z)) bad = true;
             if (gate_row) {
                 a.shared_scale[t] = pf_sigmoid(z);
-                if (!pf_finite(z)) bad = true;
             } else {
                 a.logits[(size_t)t * E + e] = z;
                 a.logit_ssq[(size_t)t * E + e] = s2;
