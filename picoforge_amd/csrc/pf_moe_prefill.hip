@@ -390,13 +390,18 @@ struct GemmTarget {   // one work item of the grouped product: a 32-row tile of 
 };
 
 // Work item q -> (row tile, slab).  Workgroups go to the eight XCDs round robin by index and a
-// workgroup's items are a multiple of eight apart, so the slabs of one row tile, which read the
-// same activation rows, are given item numbers eight apart: one XCD, one L2.  False: nothing to do
+// workgroup's items are a multiple of eight apart.  The tile list is cut into groups of GEMM_XCD_TILES
+// consecutive tiles and the groups dealt to the XCDs in turn; the items of a group (its tiles' slabs)
+// get numbers eight apart: neighbouring workgroups of one XCD, one L2, at the same time.  The slabs of
+// a row tile read the same activation rows, and the row tiles of one expert, neighbours in the list,
+// the same weights: fetched once from memory where they fall into one group.  False: nothing to do
 // for q.  Every wave of the workgroup evaluates this for itself, with the same result.
+#define GEMM_XCD_TILES 8
 template <int MODE, int FMT>
 __device__ __forceinline__ bool gemm_item(const PfKernelArgs &a, int tokens, int slabs, uint32_t q, GemmTarget &g) {
     const int E = a.experts, K = a.top_k;
-    const uint32_t xcd = q % 8, turn = q / 8, tile = (turn / slabs) * 8 + xcd;
+    const uint32_t xcd = q % 8, turn = q / 8, r = turn / slabs;
+    const uint32_t tile = GEMM_XCD_TILES * ((r / GEMM_XCD_TILES) * 8 + xcd) + r % GEMM_XCD_TILES;
     if (tile >= a.tiles[0]) return false;
     const uint32_t entry = a.tiles[1 + tile];
     const int expert = entry & 0xffffu;
@@ -866,7 +871,7 @@ __global__ void __launch_bounds__(64 * (NW + NL), 3) pf_k_pf_gemm(PfKernelArgs a
     extern __shared__ __align__(16) unsigned char ring[];
     __shared__ float row_scale[4][32];
     const int lane = pf_lane(), wave = threadIdx.x >> 6, n = lane & 31, h = lane >> 5;
-    const uint32_t items = (a.tiles[0] + 7u) / 8u * 8u * (uint32_t)slabs;
+    const uint32_t items = (a.tiles[0] + 8u * GEMM_XCD_TILES - 1u) / (8u * GEMM_XCD_TILES) * (8u * GEMM_XCD_TILES) * (uint32_t)slabs;
     if (FMT == PF_IQ2_XXS) {
         // grid magnitudes, and for every 7-bit sign field the fp16 sign bits of its eight weights
         // (the eighth sign makes the number of negative weights even)
