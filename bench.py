@@ -95,6 +95,8 @@ ALL_CONFIGS = ["iq2xxs_decode", "q4k_verify4", "q4k_prefill1024", "q4k_stack48"]
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
+FUSED_DECODE_STAGES = ["pf_k_dec_router (router logits)",
+                       "pf_k_dec_fused (routing, gate/up + SwiGLU, activation lines through memory, down products, combine)"]
 GENERAL_STAGES = ["pf_k_pre (router logits, shared gate/up + SwiGLU, shared gate)",
                   "routing (top-k, serial-order re-routes)",
                   "pf_k_gate_up (routed gate/up + SwiGLU)",
@@ -254,6 +256,8 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
     # the dispatch gap before it, as a profiler's start-to-end time of a dependent kernel does).
     family = hip.moe_kernel_family(moe, work, tokens)
     names = {0: GENERAL_STAGES, 1: DECODE_STAGES, 2: PREFILL_STAGES}[family]
+    if family == 1 and hip.moe_decode_launches(moe, work, tokens) == 2:
+        names = FUSED_DECODE_STAGES
     stage_us = [1e-3] * len(names)
     if not args.skip_stages:
         previous = 0.0
@@ -295,6 +299,8 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
         alg_bytes = workloads.algorithmic_bytes_per_token(wl["type"], unique_experts=unique, cfg=cfg)
         stage_bytes = [lb["routers"], unique * lb["gate_up"] + lb["shared_gate_up"],
                        unique * lb["down"] + lb["shared_down"]]
+        if len(names) == 2:
+            stage_bytes = [stage_bytes[0], stage_bytes[1] + stage_bytes[2]]
         if family == 0:
             stage_bytes = [lb["routers"] + lb["shared_gate_up"], tokens * cfg.experts * 8, unique * lb["gate_up"],
                            unique * lb["down"] + lb["shared_down"]]

@@ -33,6 +33,7 @@ enum {
  * src/qwen4_gpu.h:27-31: bit 1 nonfinite, bit 2 bounds). */
 #define PF_HIP_ERR_NONFINITE 2u
 #define PF_HIP_ERR_BOUNDS 4u
+#define PF_HIP_ERR_TIMEOUT 8u   /* a workgroup gave up waiting for another of its launch (build-defined bit) */
 
 typedef struct PfHipMoe PfHipMoe;    /* one layer's eight tensors, resident in HBM */
 typedef struct PfHipWork PfHipWork;  /* device scratch for up to token_cap tokens */
@@ -84,6 +85,12 @@ int pf_hip_moe_forward_static(const PfHipMoe *moe, const float *d_x, size_t x_pi
  * 2 the matrix-core prefill kernels, 0 the general kernels (any shape and format mix).  A streamed
  * layer: 1 for the batches its decode kernels take when the pool keeps Q4_K slots in the tile order. */
 int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t tokens);
+/* Dependent launches of such a forward on the decode kernels: 3 (router logits; routing, gate/up and
+ * SwiGLU; down products and combine), or 2 where one launch takes the whole expert stage (one token,
+ * Q4_K or IQ2_XXS throughout, a workspace created with PF_MOE_DECODE_FUSED=1 in the environment, a
+ * device with a compute unit per workgroup: an option, slower than the three kernels where it was
+ * measured).  0: the forward runs other kernels. */
+int pf_hip_moe_decode_launches(const PfHipMoe *moe, const PfHipWork *work, size_t tokens);
 /* Device pointers into the workspace, valid after a forward: expert ids
  * [tokens, top_k] uint32, route weights [tokens, top_k], router logits
  * [tokens, experts], the error word (one uint32). */

@@ -156,6 +156,7 @@ class HipShim:
         bind("pf_hip_memcpy_d2h", C.c_int, vp, vp, sz)
         bind("pf_hip_synchronize", C.c_int)
         bind("pf_hip_moe_kernel_family", C.c_int, vp, vp, sz)
+        bind("pf_hip_moe_decode_launches", C.c_int, vp, vp, sz)
         bind("pf_hip_hc_read_device", C.c_int, vp, sz, sz, vp, sz, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_hc_add_device", C.c_int, vp, sz, sz, vp, sz, vp, sz, sz, sz, sz, vp, vp)
         bind("pf_hip_moe_forward_hc_device", C.c_int, vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp, sz, sz, vp)

@@ -380,10 +380,12 @@ extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_byte
 // workspace layout: buffers carved from one allocation, each 256-byte aligned
 // (the error word, the ids and the route weights follow each other: a short batch's are fetched by one copy)
 enum { W_LOGITS, W_SSQ, W_ERR, W_IDS, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_SLOTS, W_UNIQ, W_EXACT, W_FLAGS, W_XIMG, W_AIMG,
-       W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
+       W_FLINES, W_FGEN, W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
        W_P2R, W_R2P, W_GROUPBAD, W_TILES, W_COUNT };
-struct Carve { size_t offset[W_COUNT], total; };
-static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
+struct Carve { size_t offset[W_COUNT], total; bool fused; };
+// fused: plan the activation lines of the decode path's one-launch expert stage (a workspace of the library's own;
+// the static scratch is too small for them and its forwards run the three kernels)
+static Carve plan_work(const PfHipMoeDesc *d, size_t cap, bool fused = false) {
     Carve c;
     memset(&c, 0, sizeof c);
     const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden, I = d->inter;
@@ -408,6 +410,13 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     want[W_ERR] = 256;
     want[W_EXACT] = 256;
     want[W_FLAGS] = (T + 1) * 4;
+    {
+        size_t lines = 0;
+        if (fused) pf_decode_fused_scratch(*d, &lines);
+        want[W_FLINES] = lines;
+        want[W_FGEN] = lines ? 256 : 0;
+        c.fused = lines != 0;
+    }
     {   // digit images of the decode path: the token rows; the activation rows of every (unique expert, token) and the shared expert's
         const size_t widest = I > d->shared_inter ? I : d->shared_inter;
         const size_t rows = Td * K * Td + Td > Tt * (K + 1) ? Td * K * Td + Td : Tt * (K + 1);
@@ -439,8 +448,15 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap) {
     return c;
 }
 
+// PF_MOE_DECODE_FUSED=1: one-token forwards of layers the fused launch takes run two launches instead of the three decode
+// kernels (measured slower on this GPU: the hand-off through memory inside the launch costs what the kernel boundary does)
+static bool fused_wanted() {
+    const char *v = getenv("PF_MOE_DECODE_FUSED");
+    return v && v[0] == '1';
+}
+
 extern "C" size_t pf_hip_work_bytes(const PfHipMoeDesc *desc, size_t token_cap) {
-    return desc ? plan_work(desc, token_cap).total : 0;
+    return desc ? plan_work(desc, token_cap, fused_wanted()).total : 0;
 }
 
 static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base);
@@ -510,7 +526,7 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     if (!moe || !out) return PF_HIP_E_ARGUMENT;
     PfHipWork *w = (PfHipWork *)calloc(1, sizeof *w);
     if (!w) return PF_HIP_E_MEMORY;
-    const Carve c = plan_work(&moe->desc, token_cap);
+    const Carve c = plan_work(&moe->desc, token_cap, fused_wanted());
     uint8_t *base = nullptr;
     hipError_t e = hipMalloc((void **)&base, c.total);
     if (e == hipSuccess) e = hipMemset(base, 0, c.total);
@@ -553,6 +569,10 @@ static void carve_work(PfHipWork *w, const Carve &c, uint8_t *base) {
     w->route_flags = (uint32_t *)(base + c.offset[W_FLAGS]);
     w->ximg = (uint32_t *)(base + c.offset[W_XIMG]);
     w->aimg = (uint32_t *)(base + c.offset[W_AIMG]);
+    if (c.fused) {
+        w->fuse_lines = (uint32_t *)(base + c.offset[W_FLINES]);
+        w->fuse_gen = (uint32_t *)(base + c.offset[W_FGEN]);
+    }
     if (c.offset[W_GROUPBAD] != c.offset[W_X16]) {   // the prefill buffers were planned
         w->x16 = (uint16_t *)(base + c.offset[W_X16]);
         w->act16 = (uint16_t *)(base + c.offset[W_ACT16]);
@@ -595,6 +615,17 @@ extern "C" int pf_hip_work_full_reroutes(PfHipWork *w, uint32_t *count) {
     return PF_HIP_OK;
 }
 
+#ifdef PF_TIMING
+// instrumented builds only: the router kernel's start and the fused launch's phase stamps (eight per workgroup, 256 workgroups)
+extern "C" int pf_debug_stamps(PfHipWork *w, unsigned long long *out) {
+    if (!w || !out) return PF_HIP_E_ARGUMENT;
+    HIP_TRY(hipMemcpy(out, w->exact_rows + 2, 8, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemcpy(out + 1, w->act, 256 * 8 * 8, hipMemcpyDeviceToHost));
+    HIP_TRY(hipMemset(w->act, 0, 256 * 8 * 8));
+    return PF_HIP_OK;
+}
+#endif
+
 extern "C" int pf_hip_work_clear_status(PfHipWork *w) {
     if (!w) return PF_HIP_E_ARGUMENT;
     HIP_TRY(hipMemset(w->error_word, 0, 4));
@@ -629,6 +660,7 @@ static PfKernelArgs make_args(const PfHipMoe *m, PfHipWork *w, const float *d_x,
     a.act = w->act; a.shared_act = w->shared_act; a.shared_scale = w->shared_scale;
     a.uniq = w->uniq;
     a.ximg = w->ximg; a.aimg = w->aimg;
+    a.fuse_lines = w->fuse_lines; a.fuse_gen = w->fuse_gen;
     a.error_word = w->error_word; a.exact_rows = w->exact_rows; a.route_flags = w->route_flags;
     a.x16 = w->x16; a.act16 = w->act16; a.sact16 = w->sact16;
     a.x_scale = w->x_scale; a.act_scale = w->act_scale; a.sact_scale = w->sact_scale; a.x_max2 = w->x_max2;
@@ -692,6 +724,12 @@ extern "C" int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *wo
     if (moe->decode_ready && tokens <= decode_limit(moe)) return 1;
     if (moe->prefill_ready && work->down && tokens > PF_DECODE_MAX_TOKENS) return 2;
     return 0;
+}
+
+extern "C" int pf_hip_moe_decode_launches(const PfHipMoe *moe, const PfHipWork *work, size_t tokens) {
+    if (pf_hip_moe_kernel_family(moe, work, tokens) != 1 || moe->streamed) return 0;
+    const PfKernelArgs a = make_args(moe, const_cast<PfHipWork *>(work), nullptr, 0, nullptr, 0);
+    return pf_decode_launches(a, (int)tokens);
 }
 
 // Enqueue only: no allocation, no synchronisation, no memset; safe under stream capture.

@@ -28,8 +28,13 @@
 
 #ifdef PF_TIMING
 #define STAMP(i) do { if (blockIdx.x == PF_TIMING && threadIdx.x == 0) reinterpret_cast<unsigned long long *>(a.exact_rows + 2)[i] = wall_clock64(); } while (0)
+// the fused launch: workgroup b's phase i (eight per workgroup) into the activation rows' buffer, which that launch leaves unused
+#define FSTAMP(i) do { if (threadIdx.x == 0) reinterpret_cast<unsigned long long *>(a.act)[8 * blockIdx.x + (i)] = wall_clock64(); } while (0)
+#define STAMP_FIRST(i) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y == 0) reinterpret_cast<unsigned long long *>(a.exact_rows + 2)[i] = wall_clock64(); } while (0)
 #else
 #define STAMP(i) do {} while (0)
+#define FSTAMP(i) do {} while (0)
+#define STAMP_FIRST(i) do {} while (0)
 #endif
 // The unit is compiled four times, once per format combination (PF_DECODE_PART 0..3, see the dispatch
 // at the end), so that the combinations' kernels build in parallel; part 0 also holds everything that
@@ -512,6 +517,7 @@ __device__ __forceinline__ void pf_args_now(const T &field, const Rest &...rest)
 template <int NT>
 __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int router_blocks, int tokens) {
     pf_args_now(a.w[0], a.w[7], a.x, a.x_pitch, a.logits, a.logit_ssq, a.shared_scale, a.ximg, router_blocks, tokens);
+    STAMP_FIRST(0);
     const int H = a.hidden, E = a.experts, lane = pf_lane(), wave = threadIdx.x >> 6;
     if ((int)blockIdx.x > router_blocks) {
         // workgroups beyond the router's (launched where the next kernel reads them): the tokens' digit images,
@@ -531,6 +537,8 @@ __global__ void __launch_bounds__(256) pf_k_dec_router(PfKernelArgs a, int route
     a.logit_ssq += (size_t)t0 * E;
     a.shared_scale += t0;
     const bool gate_row = (int)blockIdx.x == router_blocks;
+    // the tag of the forward's activation lines (the launch behind this one, where it takes the whole expert stage)
+    if (gate_row && blockIdx.y == 0 && threadIdx.x == 64 && a.fuse_gen) a.fuse_gen[0] = a.fuse_gen[0] + 1u;
     const int e = blockIdx.x * 4 + wave;
     if (gate_row ? wave != 0 : e >= E) return;
     const float4 *w = reinterpret_cast<const float4 *>(gate_row ? a.w[7] : a.w[0] + (size_t)e * H * 4);
@@ -1685,6 +1693,407 @@ __global__ void __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(FMT =
     }
 }
 
+// ---- one token: the whole expert stage in ONE launch ----------------------------------------------
+// Workgroup b computes the 32 activations of its (slot, tile) as kernel 2 does, publishes them -- one 128-byte line:
+// the group's digit image, step and sum, and the forward's tag -- and then takes eight output rows of the block as
+// kernel 3 does, a wave per slot.  Between the two halves every wave waits for the lines of its slot (they are written
+// by the sixteen workgroups of that slot), so the launch replaces a kernel boundary by one hand-off through memory:
+//   * the down rows of all slots are requested as soon as the routing is known, by the routing wave, into LDS
+//     (16 bytes a lane and instruction, lane l at base + 16 l): they travel while the gate and up products run;
+//   * a line is 26 pairs {word, tag}: every pair is written with one 64-bit agent-scope atomic store and read with one
+//     64-bit agent-scope atomic load (the XCDs' L2s are not coherent with one another), so a pair is never seen half
+//     written, a reader that finds the forward's tag in a pair has that word, and the read that polls is the read
+//     that fetches;
+//   * every line is written FUSE_REPLICAS times and a workgroup polls the replica of its index modulo that: a line that
+//     all 256 workgroups poll is a hot spot of the memory channel that holds it;
+//   * the tag is a counter in the workspace that the router kernel before this one increments, so nothing has to be
+//     cleared and a forward that was cut short leaves nothing a later one could mistake for its own.
+// Every workgroup waits for lines of other workgroups, so all of them must be resident at once: the launch is used
+// only where the device has a compute unit per workgroup, and the wait is bounded -- a wave that gives up sets
+// PF_HIP_ERR_TIMEOUT and goes on with what it has, so the launch ends whatever happens.
+#define FUSE_REPLICAS 8
+#define FUSE_SPIN_LIMIT (1 << 20)
+#define FUSE_DOWN_ROWS 8
+#define FUSE_PAIRS (PF_IMG_GROUP + 2)   // pairs of a line: the digit words, the step, the sum
+#define FUSE_LINE 64          // dwords of a line: FUSE_PAIRS pairs {word, tag}, padded to 256 bytes
+struct FuseGeometry {
+    int routed_blocks, expert_blocks;   // workgroups with a routed tile; with any tile (the shared expert's follow)
+    int down_blocks;                    // workgroups with output rows
+    int grid, lines;
+};
+__host__ __device__ inline FuseGeometry fuse_geometry(int H, int K, int I, int Is) {
+    FuseGeometry g;
+    g.routed_blocks = K * (I / 32);
+    g.expert_blocks = g.routed_blocks + Is / 32;
+    g.down_blocks = (H + FUSE_DOWN_ROWS - 1) / FUSE_DOWN_ROWS;
+    g.grid = g.expert_blocks > g.down_blocks ? g.expert_blocks : g.down_blocks;
+    g.lines = g.expert_blocks;
+    return g;
+}
+
+__device__ __forceinline__ unsigned long long ld_agent(const unsigned long long *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_agent(unsigned long long *p, unsigned long long v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// everything this wave has requested from memory has arrived (rows on their way into LDS included)
+__device__ __forceinline__ void memory_settled() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// The workgroup's 32 activations (lanes 0..31 of the calling wave) as a digit image in LDS: PF_IMG_GROUP dwords of
+// digits, the step, the sum of the integers (one group of image2_group's image).
+__device__ __forceinline__ void image_group_lds(uint32_t *img, float v, int lane) {
+    float m = fabsf(v);
+#pragma unroll
+    for (int k = 0; k < 4; k++) m = fmaxf(m, __int_as_float(dpp_row_step(__float_as_int(m), k)));
+    m = fmaxf(m, __shfl_xor(m, 16));
+    float step, inv;
+    group_step2(m, step, inv);
+    const int q = __float2int_rn(v * inv);
+    int sum = q;
+#pragma unroll
+    for (int k = 0; k < 4; k++) sum += dpp_row_step(sum, k);
+    sum += __shfl_xor(sum, 16);
+    int d[PF_IMG_PLANES];
+    image_digits(q, d);
+    uint8_t *bytes = reinterpret_cast<uint8_t *>(img);
+    if (lane < 32) {
+#pragma unroll
+        for (int p = 0; p < PF_IMG_PLANES; p++) bytes[32 * p + lane] = (uint8_t)d[p];
+    }
+    if (lane == 0) { img[PF_IMG_GROUP] = __float_as_uint(step); img[PF_IMG_GROUP + 1] = (uint32_t)sum; }
+}
+
+__device__ __forceinline__ void fuse_to_lds(const void *global, unsigned char *lds) {
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(global), reinterpret_cast<uint32_t *>(lds), 16, 0, 0);
+}
+__device__ __forceinline__ void fuse_to_lds_dword(const void *global, unsigned char *lds) {   // lane l at base + 4 l
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(global), reinterpret_cast<uint32_t *>(lds), 4, 0, 0);
+}
+template <int FMT> __host__ __device__ constexpr int fuse_stage_bytes() { return FMT == PF_Q4_K ? 3072 : 1280; }   // a wave's down items
+
+// One (row, run) item a lane into the stage: Q4_K the row's header and the run's two halves; IQ2_XXS the run's piece and
+// the dword around the block's scale.
+__device__ __forceinline__ void item_request(const TileItem<PF_Q4_K> *, const uint8_t *chunk, int row, int run, unsigned char *stage) {
+    fuse_to_lds(chunk + pf_q4t_header_at(row), stage);
+    fuse_to_lds(chunk + pf_q4t_piece_at(run, 0, row), stage + 1024);
+    fuse_to_lds(chunk + pf_q4t_piece_at(run, 1, row), stage + 2048);
+}
+__device__ __forceinline__ void item_request(const TileItem<PF_IQ2_XXS> *, const uint8_t *chunk, int row, int run, unsigned char *stage) {
+    fuse_to_lds(chunk + pf_i2t_piece_at(run, row), stage);
+    fuse_to_lds_dword(chunk + (pf_i2t_scale_at(row) & ~(size_t)3), stage + 1024);
+}
+__device__ __forceinline__ void item_take(TileItem<PF_Q4_K> &w, const unsigned char *stage, int lane, int) {
+    w.hdr = *reinterpret_cast<const uint4 *>(stage + 16 * lane);
+    w.piece[0] = *reinterpret_cast<const uint4 *>(stage + 1024 + 16 * lane);
+    w.piece[1] = *reinterpret_cast<const uint4 *>(stage + 2048 + 16 * lane);
+}
+__device__ __forceinline__ void item_take(TileItem<PF_IQ2_XXS> &w, const unsigned char *stage, int lane, int row) {
+    w.piece = *reinterpret_cast<const uint4 *>(stage + 16 * lane);
+    const uint32_t both = *reinterpret_cast<const uint32_t *>(stage + 1024 + 4 * lane);
+    w.dbits = row & 1 ? both >> 16 : both & 0xffffu;
+}
+
+// FMT: the format of every expert tensor (routed and shared)
+template <int NPL, int FMT>
+__global__ void __launch_bounds__(1024) pf_k_dec_fused(PfKernelArgs a, FuseGeometry geo) {
+    extern __shared__ __align__(16) int fuse_lds[];   // (16-byte aligned: rows land here 16 bytes a lane)
+    int *const lds = fuse_lds;
+    __shared__ RouteLds R;
+    __shared__ uint32_t early_expert;
+    __shared__ __attribute__((aligned(16))) uint32_t act_image[PF_IMG_GROUP + 4];
+    __shared__ float down_partial[17][FUSE_DOWN_ROWS];
+    typedef TileGeometry<FMT> G;
+    const int b = (int)blockIdx.x, H = a.hidden, K = a.top_k, E = a.experts, lane = pf_lane();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const bool has_tile = b < geo.expert_blocks, has_rows = b < geo.down_blocks;
+    const bool shared = has_tile && b >= geo.routed_blocks;
+    const bool routed = has_tile && !shared;
+    const int tiles = a.inter / 32, tiles_s = a.shared_inter / 32;
+    const int u = routed ? b / tiles : K;
+    const int tile = shared ? b - geo.routed_blocks : b % tiles, n0 = 32 * tile;
+    const uint32_t tag = a.fuse_gen[0];
+    const int n_base = FUSE_DOWN_ROWS * b;
+    PfOutputRegs out_regs;
+    if (has_rows && (int)threadIdx.x < FUSE_DOWN_ROWS && n_base + (int)threadIdx.x < H) pf_output_prefetch(a, 0, n_base + threadIdx.x, out_regs);
+    const float shared_scale = a.shared_scale[0];
+    FSTAMP(0);
+    // LDS: IQ2_XXS: the signed-magnitude tables (32 KB) and the magnitude grid (2 KB); the waves' partial sums; then the
+    // serial-order routing's arrays or, in their place, the slots' down items and the slots' activation images
+    uint32_t *tables = reinterpret_cast<uint32_t *>(lds);
+    uint32_t *grid = tables + table_words<FMT>();
+    constexpr int GRID_WORDS = FMT == PF_IQ2_XXS ? 512 : 0;
+    if (FMT == PF_IQ2_XXS && wave != 0) {
+        const uint4 *src = reinterpret_cast<const uint4 *>(a.iq2_signed);
+        for (int i = (int)threadIdx.x - 64; i < 2048; i += 960) reinterpret_cast<uint4 *>(tables)[i] = src[i];
+        if (wave == 1) {
+            const uint4 *g = reinterpret_cast<const uint4 *>(a.iq2_grid);
+            reinterpret_cast<uint4 *>(grid)[lane] = g[lane];
+            reinterpret_cast<uint4 *>(grid)[64 + lane] = g[64 + lane];
+        }
+    }
+    float *partial = reinterpret_cast<float *>(grid + GRID_WORDS);   // [15 waves][64 lanes]
+    float *scratch = partial + 15 * 64;
+    unsigned char *stages = reinterpret_cast<unsigned char *>(scratch);                     // [K + 1][fuse_stage_bytes]
+    const size_t widest = a.inter > a.shared_inter ? a.inter : a.shared_inter;
+    const int image_words = (int)pf_image2_words(widest);
+    uint32_t *images = reinterpret_cast<uint32_t *>(stages + (size_t)(K + 1) * fuse_stage_bytes<FMT>());   // [K + 1][image_words]
+    const bool norm = a.norm_topk != 0;
+    const int rounds = K + 1, first_rounds = routed ? u + 1 : 0;
+    float v[NPL], s2[NPL], total = 0.0f, top_all = 0.0f;
+    PfTopk<NPL> top;
+    uint32_t my_key = 0;
+    bool bad = false;
+    if (wave == 0) {
+        pf_load_row<NPL>(a.logits, E, lane, -INFINITY, v);
+        pf_load_row<NPL>(a.logit_ssq, E, lane, 0.0f, s2);
+#pragma unroll
+        for (int j = 0; j < NPL; j++) bad |= lane * NPL + j < E && !pf_finite(v[j]);
+        bad = __any(bad);
+        if (!norm) {
+            float m = v[0];
+#pragma unroll
+            for (int j = 1; j < NPL; j++) m = fmaxf(m, v[j]);
+            top_all = pf_wave_max_fast(m);
+#pragma unroll
+            for (int j = 0; j < NPL; j++) total += expf(v[j] - top_all);
+            total = pf_wave_sum(total);
+        }
+        top.setup(v, E, lane);
+        for (int r = 0; r < first_rounds; r++) {
+            const uint32_t best = top.pop();
+            if (lane == r) my_key = best;
+        }
+        if (routed) {
+            const uint32_t mine = (uint32_t)__builtin_amdgcn_readlane((int)my_key, u);
+            if (lane == 0) early_expert = mine ? pf_key_id(mine) : 0xffffffffu;
+        }
+    }
+    const Q4TilePlan plan = q4t_plan<FMT>(a, shared, has_tile ? n0 : 0);
+    if (routed || FMT == PF_IQ2_XXS) __syncthreads();   // the early expert; the tables
+    const uint32_t early = routed ? early_expert : 0u;
+    const bool early_ok = early < (uint32_t)E;
+    FSTAMP(1);
+    TileItem<FMT> gu[Q4T_ITEMS];
+    auto request_tile = [&](uint32_t e) {
+        if (wave == 0 || !has_tile) return;
+        const uint8_t *t = plan.base + (size_t)e * plan.expert_bytes;
+#pragma unroll
+        for (int k = 0; k < Q4T_ITEMS; k++) {
+            const int it = wave - 1 + 15 * k;
+            if (it < plan.items) q4t_load(gu[k], t + G::chunk_at(0, plan.kblocks, it >> 2), plan.row, it & 3);
+        }
+    };
+    auto tile_products = [&]() {
+        if (wave == 0 || !has_tile) return;
+        const PfScalarWords image = (PfScalarWords)(uintptr_t)a.ximg;
+        float sum = 0.0f;
+#pragma unroll
+        for (int k = 0; k < Q4T_ITEMS; k++) {
+            const int it = wave - 1 + 15 * k;
+            if (it < plan.items) {
+                const int g = 2 * it;
+                sum += q4t_dot(gu[k], image + PF_IMG_GROUP * g, image + PF_IMG_GROUP * plan.groups + g, image + (PF_IMG_GROUP + 1) * plan.groups + g,
+                               it & 3, tables);
+            }
+        }
+        partial[(wave - 1) * 64 + lane] = sum;
+    };
+    // The routing wave requests this workgroup's down rows of every slot: lane (row r of eight, run) fetches what the same
+    // lane of the slot's wave multiplies later.  id_of(s): the slot's expert.
+    const int row_in_tile = (n_base & 31) + (lane & 7), my_run = lane >> 3;
+    auto request_rows = [&](auto id_of) {
+        const int kb_r = a.inter / 256, kb_s = a.shared_inter / 256;
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            if (s > K) break;
+            const bool sh = s == K;
+            uint32_t e = sh ? 0u : id_of(s);
+            if (e >= (uint32_t)E) e = 0u;   // only reachable with nonfinite logits: the error word says so
+            const int kblocks = sh ? kb_s : kb_r, runs = 4 * kblocks;
+            const int run = my_run < runs ? my_run : 0;
+            const int tensor = sh ? 6 : 3;
+            const uint8_t *chunk = G::tensor(a, tensor) + (size_t)e * G::expert_bytes(a, tensor) + G::chunk_at(n_base / 32, kblocks, run >> 2);
+            item_request(static_cast<const TileItem<FMT> *>(nullptr), chunk, row_in_tile, run & 3, stages + (size_t)s * fuse_stage_bytes<FMT>());
+        }
+    };
+    request_tile(early_ok ? early : 0u);
+    tile_products();
+    if (wave == 0) {
+        for (int r = first_rounds; r <= rounds; r++) {
+            const uint32_t best = top.pop();
+            if (lane == r) my_key = best;
+        }
+        uint32_t my_id;
+        float my_z, my_s2, weight;
+        bool close;
+        const bool ambiguous = pf_topk_exact_order<NPL>(my_key, rounds + 1, v, s2, lane, my_id, my_z, my_s2);
+        pf_route_finish_wave(my_z, my_s2, K, rounds, norm, H, total, top_all, lane, weight, close);
+        close |= ambiguous;
+        if (lane < K) { R.ids[lane] = my_id; R.weights[lane] = weight; }
+        if (lane == 0) { R.close[0] = close ? 1u : 0u; R.nonfinite[0] = bad ? 1u : 0u; }
+        if (has_rows && !close) request_rows([&](int s) { return (uint32_t)__builtin_amdgcn_readlane((int)my_id, s); });
+    }
+    __syncthreads();
+    FSTAMP(2);
+    const bool again = R.close[0] != 0;
+    if (again) {
+        // a close call: the token is routed again in the reference's order (in the LDS the down rows land in: none were requested)
+        q4t_route_fix<NPL>(reinterpret_cast<const float *>(a.w[0]), a.x, a.logits, a.logit_ssq, E, K, norm, H,
+                           (int)(scratch - reinterpret_cast<float *>(lds)), &R);
+        if (wave == 0 && has_rows) request_rows([&](int s) { return R.ids[s]; });
+    } else if (threadIdx.x == 0) {
+        R.close_mask = 0;
+        R.bad = R.nonfinite[0];
+    }
+    uint32_t e = routed ? R.ids[u] : 0u;
+    if (routed && e != early && e < (uint32_t)E) {   // the early guess came from truncated keys, or the token was routed again
+        __syncthreads();
+        request_tile(e);
+        tile_products();
+        __syncthreads();
+    }
+    if (b == 0) {
+        if (!again) __syncthreads();   // R.bad above; the re-route ends with a barrier of its own
+        for (int q = threadIdx.x; q < K; q += blockDim.x) {
+            a.ids[q] = R.ids[q];
+            a.route_weights[q] = R.weights[q];
+        }
+        if (threadIdx.x == 0) {
+            if (R.bad) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+            if (R.close_mask) atomicAdd(a.exact_rows, 1u);
+            if (R.close_mask == 2u) atomicAdd(a.exact_rows + 1, 1u);
+        }
+    }
+    if (routed && e >= (uint32_t)E && threadIdx.x == 0) atomicOr(a.error_word, PF_HIP_ERR_BOUNDS | PF_HIP_ERR_NONFINITE);   // nonfinite logits
+    // wave 1: the gate and up rows' sums over the waves in wave order, SwiGLU, the 32 activations as one group's image,
+    // and the image as this workgroup's line, once per replica
+    if (wave == 1 && has_tile) {
+        float sum = 0.0f;
+        for (int w = 0; w < 15; w++) sum += partial[w * 64 + lane];
+        const float up = __shfl(sum, (lane & 31) + 32);
+        float act = pf_silu(sum) * up;
+        if (lane < 32 && !pf_finite(act)) { atomicOr(a.error_word, PF_HIP_ERR_NONFINITE); act = 0.0f; }
+        image_group_lds(act_image, act, lane);
+        pf_wave_lds_fence();
+        if (lane < FUSE_PAIRS) {
+            const unsigned long long pair = ((unsigned long long)tag << 32) | act_image[lane];
+            unsigned long long *line = reinterpret_cast<unsigned long long *>(a.fuse_lines + (size_t)b * FUSE_LINE) + lane;
+#pragma unroll
+            for (int r = 0; r < FUSE_REPLICAS; r++) st_agent(line + (size_t)r * geo.lines * (FUSE_LINE / 2), pair);
+        }
+    }
+    if (wave == 0) memory_settled();   // the down rows this wave requested have landed
+    __syncthreads();
+    FSTAMP(3);
+    if (!has_rows) return;
+    if (wave <= K) {
+        const int s = wave;
+        const bool sh = s == K;
+        const int groups = sh ? tiles_s : tiles, runs = groups / 2;
+        uint32_t *mine = images + (size_t)s * image_words;
+        // the slot's lines: its groups' pairs go round the lanes
+        const unsigned long long *src = reinterpret_cast<const unsigned long long *>(
+            a.fuse_lines + ((size_t)(b % FUSE_REPLICAS) * geo.lines + (size_t)s * tiles) * FUSE_LINE);
+        constexpr int TURNS = (16 * FUSE_PAIRS + 63) / 64;   // at most 16 groups a slot
+        const int wanted = groups * FUSE_PAIRS;
+        unsigned long long got[TURNS];
+        bool ok = false;
+        for (int spin = 0; spin < FUSE_SPIN_LIMIT && !ok; spin++) {
+            bool here = true;
+#pragma unroll
+            for (int j = 0; j < TURNS; j++) {
+                const int i = lane + 64 * j;
+                if (i < wanted) {
+                    const int group = i / FUSE_PAIRS, p = i - group * FUSE_PAIRS;
+                    got[j] = ld_agent(src + (size_t)group * (FUSE_LINE / 2) + p);
+                    here &= (uint32_t)(got[j] >> 32) == tag;
+                }
+            }
+            ok = __all(here);
+            if (!ok) __builtin_amdgcn_s_sleep(1);
+        }
+        if (!ok && lane == 0) atomicOr(a.error_word, PF_HIP_ERR_TIMEOUT);   // a workgroup never came: the launch still ends
+        FSTAMP(4);
+#pragma unroll
+        for (int j = 0; j < TURNS; j++) {
+            const int i = lane + 64 * j;
+            if (i < wanted) {
+                const int group = i / FUSE_PAIRS, p = i - group * FUSE_PAIRS;
+                const uint32_t word = (uint32_t)got[j];
+                if (p < PF_IMG_GROUP) mine[PF_IMG_GROUP * group + p] = word;
+                else if (p == PF_IMG_GROUP) mine[PF_IMG_GROUP * groups + group] = word;
+                else mine[(PF_IMG_GROUP + 1) * groups + group] = word;
+            }
+        }
+        pf_wave_lds_fence();
+        float dot = 0.0f;
+        if (my_run < runs) {
+            TileItem<FMT> item;
+            item_take(item, stages + (size_t)s * fuse_stage_bytes<FMT>(), lane, row_in_tile);
+            dot = down_dot(item, my_run & 3, mine, my_run, groups, grid);
+        }
+        // the row's runs: lanes r, r + 8, ..., r + 56
+        dot += __shfl_xor(dot, 8);
+        dot += __shfl_xor(dot, 16);
+        dot += __shfl_xor(dot, 32);
+        if (lane < FUSE_DOWN_ROWS) down_partial[s][lane] = dot;
+    }
+    __syncthreads();
+    const int n = n_base + threadIdx.x;
+    if ((int)threadIdx.x < FUSE_DOWN_ROWS && n < H) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int slot = 0; slot < 16; slot++)   // slot order, as src/qwen4_moe.c:362-372
+            if (slot < K) sum += R.weights[slot] * down_partial[slot][threadIdx.x];
+        const float y = sum + shared_scale * down_partial[K][threadIdx.x];
+        if (!pf_output_commit(a, 0, n, y, out_regs)) atomicOr(a.error_word, PF_HIP_ERR_NONFINITE);
+    }
+    FSTAMP(5);
+}
+
+// Layers the fused launch takes: one token, every expert tensor Q4_K or every one IQ2_XXS with the tile-ordered copies
+// kept, intermediate widths of at most 512 (a lane holds one run of a down row), whole groups of eight output rows,
+// the workspace's lines, and a device with a compute unit for every workgroup.
+static int device_compute_units() {
+    static int units = -1;
+    if (units < 0) {
+        int device = 0, count = 0;
+        if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) count = 0;
+        units = count;
+    }
+    return units;
+}
+
+template <int FMT>
+static bool fused_applies(const PfKernelArgs &a) {
+    if (!a.fuse_lines || !a.fuse_gen || a.slots) return false;
+    if (a.inter % 256 || a.shared_inter % 256 || a.inter > 512 || a.shared_inter > 512 || a.hidden % 32 || a.top_k > 15) return false;
+    const FuseGeometry g = fuse_geometry(a.hidden, a.top_k, a.inter, a.shared_inter);
+    return g.grid <= device_compute_units();
+}
+
+template <int NPL, int FMT>
+static void launch_fused_lists(const PfKernelArgs &a, const FuseGeometry &g, size_t lds, hipStream_t stream) {
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void *>(pf_k_dec_fused<NPL, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);
+        configured = true;
+    }
+    hipLaunchKernelGGL((pf_k_dec_fused<NPL, FMT>), dim3(g.grid), dim3(1024), lds, stream, a, g);
+}
+
+template <int FMT>
+static void launch_fused(const PfKernelArgs &a, hipStream_t stream) {
+    const FuseGeometry g = fuse_geometry(a.hidden, a.top_k, a.inter, a.shared_inter);
+    const size_t widest = a.inter > a.shared_inter ? a.inter : a.shared_inter;
+    const size_t fix = pf_route_fix_lds_floats(a.hidden, a.experts) * 4;
+    const size_t rows = (size_t)(a.top_k + 1) * (fuse_stage_bytes<FMT>() + pf_image2_words(widest) * 4);
+    const size_t lds = (size_t)table_words<FMT>() * 4 + (FMT == PF_IQ2_XXS ? 2048 : 0) + (size_t)15 * 64 * 4 + (fix > rows ? fix : rows);
+    const int all = (a.experts + 63) / 64;
+    if (all <= 1) launch_fused_lists<1, FMT>(a, g, lds, stream);
+    else if (all <= 2) launch_fused_lists<2, FMT>(a, g, lds, stream);
+    else if (all <= 4) launch_fused_lists<4, FMT>(a, g, lds, stream);
+    else if (all <= 8) launch_fused_lists<8, FMT>(a, g, lds, stream);
+    else launch_fused_lists<16, FMT>(a, g, lds, stream);
+}
+
 #if PF_DECODE_PART == 0
 // ---- IQ2_XXS in tile order ---------------------------------------------------------------------------
 // From the split device layout (64-byte payloads row by row, half scales apart) to the chunks of pf_decode_addr.h per
@@ -1912,6 +2321,17 @@ int pf_decode_tile_layer(const PfHipMoeDesc &d, const uint8_t *const q4k_tiled[8
 }
 #endif
 
+#if PF_DECODE_PART == 0
+void pf_decode_fused_scratch(const PfHipMoeDesc &d, size_t *line_bytes) {
+    *line_bytes = 0;
+    const int combination = decode_combination(d.type);
+    if (combination != 1 && combination != 2) return;
+    if (d.inter % 256 || d.shared_inter % 256 || d.inter > 512 || d.shared_inter > 512 || d.hidden % 32 || d.down_physical != d.inter || d.top_k > 15) return;
+    const FuseGeometry g = fuse_geometry((int)d.hidden, (int)d.top_k, (int)d.inter, (int)d.shared_inter);
+    *line_bytes = (size_t)FUSE_REPLICAS * g.lines * FUSE_LINE * 4;
+}
+#endif
+
 static PfHipMoeDesc desc_of(const PfKernelArgs &a) {
     PfHipMoeDesc d = {};
     d.hidden = a.hidden; d.experts = a.experts; d.top_k = a.top_k; d.inter = a.inter; d.shared_inter = a.shared_inter;
@@ -1951,6 +2371,12 @@ static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t str
     const int last = stage_limit ? stage_limit : 3;
     pf_launch_dec_router(a, tokens, (a.experts + 3) / 4, stream);
     if (last < 2) return;
+    if constexpr (FG == FD && FG == FS && (FG == PF_Q4_K || FG == PF_IQ2_XXS)) {
+        if (tokens == 1 && fused_applies<FG>(a)) {
+            launch_fused<FG>(a, stream);
+            return;
+        }
+    }
     launch_q4t_experts<FG, FD, FS>(a, tokens, stream, last);
 }
 
@@ -2032,6 +2458,14 @@ void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream,
 void pf_launch_decode_stream_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
     if (decode_combination(a.type) == 4) pf_launch_decode_q4profile_experts(a, tokens, stream);
     else launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K, true>(a, tokens, stream, 3);
+}
+
+int pf_decode_launches(const PfKernelArgs &a, int tokens) {
+    const int combination = pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq);
+    if (tokens != 1) return 3;
+    if (combination == 1) return fused_applies<PF_Q4_K>(a) ? 2 : 3;
+    if (combination == 2) return fused_applies<PF_IQ2_XXS>(a) ? 2 : 3;
+    return 3;
 }
 
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {

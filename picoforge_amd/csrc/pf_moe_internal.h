@@ -34,6 +34,9 @@ struct PfKernelArgs {
     uint32_t *ximg, *aimg;           // decode path, tile-ordered Q4_K: digit images (pf_image2_words) of the token rows, written
                                      // by kernel 1, and of the activation rows [unique, tokens] then [tokens] shared, by kernel 2
     uint32_t *uniq;                  // decode path: [0] count, then ids[P], then pair->unique[P], then token masks[P]
+    // decode path, one token, the expert stage in one launch (null: three kernels): the workgroups' activation lines
+    // (FUSE_REPLICAS copies) and the counter whose value tags a forward's lines, incremented by the router kernel
+    uint32_t *fuse_lines, *fuse_gen;
     // expert streaming: w[1..3] (wt[1..3] for Q4_K slots in tile order) are pool regions of pool_slots experts each and the routed
     // tensors are addressed by slots[pair] instead of ids[pair] (null: every expert resident, addressed by id)
     const uint32_t *slots;
@@ -130,7 +133,7 @@ struct PfHipWork {
     size_t cap, bytes;
     uint32_t *ximg, *aimg;
     float *logits, *logit_ssq, *route_weights, *act, *shared_act, *shared_scale, *x, *y;
-    uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags, *slots;
+    uint32_t *ids, *uniq, *error_word, *exact_rows, *route_flags, *slots, *fuse_lines, *fuse_gen;
     uint16_t *x16, *act16, *sact16;  // prefill buffers (allocated when cap exceeds the decode path's batch)
     float *x_scale, *act_scale, *sact_scale, *x_max2, *down;
     uint32_t *counts, *offsets, *pair_to_row, *row_to_pair, *group_bad, *tiles;
@@ -183,6 +186,11 @@ void pf_launch_q8_tile(const uint8_t *d_payload, const uint16_t *d_scales, uint8
                        hipStream_t stream);
 void pf_launch_decode(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, hipStream_t stream);
+// bytes of the activation lines a workspace needs for the one-launch expert stage of a one-token forward (0: the
+// layer's shape or formats are not taken)
+void pf_decode_fused_scratch(const PfHipMoeDesc &d, size_t *line_bytes);
+// launches per one-token forward on the decode path: 2 with the fused expert stage, else 3
+int pf_decode_launches(const PfKernelArgs &a, int tokens);
 // kernels 2 and 3 of the tile decode path on pool slots, for a Q4_K layer or one in the q4 checkpoint profile (expert
 // streaming: kernel 1 ran in an earlier call)
 void pf_launch_decode_stream_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);

@@ -1,6 +1,6 @@
 """GPU parity on the benchmark configurations themselves, at their full shape
-(hidden 2048, 512 experts, top-10, intermediate 512, shared 512): the 1024-token Q4_K chunk under a
-Zipf(1.1) router, the 4-token verify batches with about half of the experts shared between
+(hidden 2048, 512 experts, top-10, intermediate 512, shared 512): Q4_K chunks of 1024, 1777 and 2048 tokens
+under a Zipf(1.1) router, the 4-token verify batches with about half of the experts shared between
 neighbours, and a stack of independent layers."""
 import ctypes as C
 
@@ -24,23 +24,9 @@ def oracle_routes(oracle, cfg, weights, x):
     return ids, w
 
 
-def test_q4k_zipf_chunk_of_1024_tokens_at_full_shape(product, oracle):
-    cfg = workloads.measured_config()
-    weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=1)
-    workloads.zipf_router(weights, seed=1, temperature=0.18)
-    x = workloads.prefill_chunk(weights, 1024, seed=1)
-    print("zipf chunk: device forward", flush=True)
-    with pf.MoeLayer(product, cfg, weights, 1024) as layer:
-        assert product.hip.moe_kernel_family(*layer.device_handles(), 1024) == 2, "the prefill kernels do not cover this layer"
-        _, y, ids, w = layer.forward(x)
-        reroutes = layer.serial_order_reroutes()
-    print("zipf chunk: oracle routes of all 1024 tokens", flush=True)
-    ids0, w0 = oracle_routes(oracle, cfg, weights, x)
-    np.testing.assert_array_equal(ids, ids0, err_msg="expert ids of the 1024-token chunk")
-    np.testing.assert_allclose(w, w0, atol=2e-6, rtol=2e-5)
-    load = np.bincount(ids0.reshape(-1), minlength=cfg.experts)
-    assert load.max() > 96 and (load == 0).sum() < 64, (load.max(), (load == 0).sum())   # several 32-row tiles; most experts active
-    # rows of the busiest experts (first, middle and last of their row lists) and of the least loaded ones
+def pick_chunk_rows(ids0, load, tokens):
+    """Rows of the busiest experts (first, middle and last of their row lists), of the least loaded ones, and the
+    chunk's first, middle and last rows."""
     picked = []
     for e in np.argsort(-load)[:6]:
         rows = np.nonzero((ids0 == e).any(axis=1))[0]
@@ -48,16 +34,53 @@ def test_q4k_zipf_chunk_of_1024_tokens_at_full_shape(product, oracle):
     for e in np.argsort(load)[:10]:                       # the least loaded experts (a few rows each)
         if load[e]:
             picked.append(np.nonzero((ids0 == e).any(axis=1))[0][0])
-    picked += [0, 511, 1023]
-    picked = np.unique(np.array(picked))
+    picked += [0, tokens // 2 - 1, tokens - 1]
+    return np.unique(np.array(picked))
+
+
+def check_zipf_chunk(product, oracle, cfg, weights, layer, x, label, extra_rows=()):
+    """One chunk through a resident layer: every token's expert ids and route weights against the oracle's routing,
+    the outputs of picked rows against the oracle's forward (the oracle works token by token, so a subset of rows
+    is a valid check).  Returns the row-tile count of the chunk's grouped products."""
+    tokens = len(x)
+    print(f"{label}: device forward of {tokens} tokens", flush=True)
+    _, y, ids, w = layer.forward(x)
+    reroutes = layer.serial_order_reroutes()
+    print(f"{label}: oracle routes of all {tokens} tokens", flush=True)
+    ids0, w0 = oracle_routes(oracle, cfg, weights, x)
+    np.testing.assert_array_equal(ids, ids0, err_msg=f"expert ids of the {tokens}-token chunk")
+    np.testing.assert_allclose(w, w0, atol=2e-6, rtol=2e-5)
+    load = np.bincount(ids0.reshape(-1), minlength=cfg.experts)
+    tiles = int(((load + 31) // 32).sum()) + (tokens + 31) // 32       # the experts' 32-row tiles and the shared expert's
+    picked = np.unique(np.concatenate([pick_chunk_rows(ids0, load, tokens), np.array(extra_rows, dtype=np.int64)]))
     assert len(picked) >= 24
-    print(f"zipf chunk: oracle forward of {len(picked)} rows; max load {load.max()}, idle experts {(load == 0).sum()}, "
-          f"serial-order reroutes {reroutes}", flush=True)
+    print(f"{label}: oracle forward of {len(picked)} rows; max load {load.max()}, idle experts {(load == 0).sum()}, "
+          f"{tiles} row tiles, serial-order reroutes {reroutes}", flush=True)
     with pf.MoeLayer(oracle, cfg, weights, len(picked)) as cpu:
         _, y0, ids1, w1 = cpu.forward(x[picked])
     np.testing.assert_array_equal(ids1, ids0[picked])       # the oracle's forward routes like its route call
-    worst = assert_parity(y[picked], ids[picked], w[picked], y0, ids1, w1, label="zipf chunk rows")
-    print(f"zipf chunk: max abs err {worst:.3e} on {len(picked)} rows", flush=True)
+    worst = assert_parity(y[picked], ids[picked], w[picked], y0, ids1, w1, label=f"{label} rows")
+    print(f"{label}: max abs err {worst:.3e} on {len(picked)} rows", flush=True)
+    return tiles, load
+
+
+@pytest.mark.parametrize("tokens", [1024, 1777, 2048])
+def test_q4k_zipf_chunk_at_full_shape(product, oracle, tokens):
+    """The prefill chunk of the benchmark (1024 tokens), the stack's chunk (2048 tokens) and a ragged length
+    between them, Q4_K experts under the Zipf(1.1) router."""
+    cfg = workloads.measured_config()
+    weights = pf.LayerWeights.synthetic(cfg, abi.GGUF_Q4_K, seed=1)
+    workloads.zipf_router(weights, seed=1, temperature=0.18)
+    x = workloads.prefill_chunk(weights, tokens, seed=tokens // 1024)
+    with pf.MoeLayer(product, cfg, weights, tokens) as layer:
+        assert product.hip.moe_kernel_family(*layer.device_handles(), tokens) == 2, "the prefill kernels do not cover this layer"
+        tiles, load = check_zipf_chunk(product, oracle, cfg, weights, layer, x, f"zipf chunk {tokens}",
+                                       extra_rows=(31, 32, tokens - 33, tokens - 32))
+    assert load.max() > 96 and (load == 0).sum() < 64, (load.max(), (load == 0).sum())   # several 32-row tiles; most experts active
+    if tokens != 1024:
+        # the grouped products deal their row tiles to the XCDs in groups of 64: a count that is no multiple of 64
+        # has a last, partly filled group
+        assert tiles % 64 != 0, tiles
 
 
 def test_q4k_verify_batches_share_experts(product, oracle):
@@ -111,6 +134,12 @@ def test_stack_of_independent_layers(product, oracle):
         print(f"  layer {l}: max abs err {worst:.2e}", flush=True)
     hip.free(d_x)
     hip.free(d_y)
+    # the stack's other leg: a 2048-token chunk through the first and the last layer, each under its own router
+    for l in (0, n_layers - 1):
+        chunk = workloads.prefill_chunk(all_weights[l], 2048, seed=50 + l)
+        with pf.MoeLayer(product, cfg, all_weights[l], 2048) as wide:
+            assert product.hip.moe_kernel_family(*wide.device_handles(), 2048) == 2
+            check_zipf_chunk(product, oracle, cfg, all_weights[l], wide, chunk, f"stack layer {l}, chunk")
     for l in layers:
         l.close()
 
