@@ -110,16 +110,6 @@ int pf_hip_work_full_reroutes(PfHipWork *work, uint32_t *count);
 /* The error word and the re-route counter accumulate over forwards (a forward only
  * enqueues kernels, so it can be captured into a graph); this clears both. */
 int pf_hip_work_clear_status(PfHipWork *work);
-/* Tests: route every batch size through the general kernels (on != 0) instead of the
- * specialised decode kernels. */
-void pf_hip_work_force_general(PfHipWork *work, int on);
-
-/* Diagnostics: every later forward on this workspace enqueues only the first `count` of its
- * dependent kernel groups (decode path: its three kernels; other paths: four groups; 0 = all;
- * results are then incomplete).  A measuring program times the chain cut after 1, 2, ... groups
- * and takes differences; nothing in the library calls it. */
-void pf_hip_work_limit_kernels(PfHipWork *work, int count);
-
 /* Host-buffer forward used by qwen4_moe_forward: copies x in, runs the forward,
  * copies y (and ids/weights when non-NULL) out, returns the error word.  Pitches
  * in bytes.  Outputs are written only when the error word is zero.  Batches of up

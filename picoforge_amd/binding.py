@@ -145,6 +145,7 @@ class HipShim:
         bind("pf_hip_work_clear_status", C.c_int, vp)
         bind("pf_hip_work_force_general", None, vp, C.c_int)
         bind("pf_hip_work_limit_kernels", None, vp, C.c_int)
+        bind("pf_hip_work_check_guards", C.c_int, vp, P(C.c_int), P(C.c_int))
         bind("pf_hip_moe_forward_host", C.c_int, vp, vp, vp, sz, vp, sz, vp, sz, vp, sz, sz, u32p)
         bind("pf_hip_route_host", C.c_int, vp, sz, sz, sz, C.c_int, vp, vp, vp, u32p, P(C.c_uint64))
         bind("pf_hip_group_pairs_host", C.c_int, vp, sz, sz, sz, vp, vp, vp, u32p, P(C.c_int))

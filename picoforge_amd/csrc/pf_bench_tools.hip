@@ -15,6 +15,7 @@
 #include <string.h>
 #include <vector>
 #include "pf_bench_tools.h"
+#include "pf_moe_debug.h"
 
 static thread_local char g_error[256] = "";
 extern "C" const char *pf_bench_last_error(void) { return g_error; }

@@ -1,5 +1,6 @@
 // C-ABI entry points of the HIP side (include/pf_moe_hip.h).
 #include "pf_moe_internal.h"
+#include "pf_moe_debug.h"
 #include "../../include/pf_iq2_codes.h"
 #include <stdio.h>
 #include <stdlib.h>
@@ -382,10 +383,11 @@ extern "C" size_t pf_hip_moe_bytes(const PfHipMoe *m) { return m ? m->total_byte
 enum { W_LOGITS, W_SSQ, W_ERR, W_IDS, W_RW, W_ACT, W_SACT, W_SSCALE, W_X, W_Y, W_SLOTS, W_UNIQ, W_EXACT, W_FLAGS, W_XIMG, W_AIMG,
        W_FLINES, W_FGEN, W_X16, W_ACT16, W_SACT16, W_XSCALE, W_ACTSCALE, W_SACTSCALE, W_XMAX2, W_DOWN, W_COUNTS, W_OFFSETS,
        W_P2R, W_R2P, W_GROUPBAD, W_TILES, W_COUNT };
-struct Carve { size_t offset[W_COUNT], total; bool fused; };
+#define PF_GUARD_BYTES 4096
+struct Carve { size_t offset[W_COUNT], size[W_COUNT], total; bool fused; size_t guard; };
 // fused: plan the activation lines of the decode path's one-launch expert stage (a workspace of the library's own;
 // the static scratch is too small for them and its forwards run the three kernels)
-static Carve plan_work(const PfHipMoeDesc *d, size_t cap, bool fused = false) {
+static Carve plan_work(const PfHipMoeDesc *d, size_t cap, bool fused = false, size_t guard = 0) {
     Carve c;
     memset(&c, 0, sizeof c);
     const size_t T = cap ? cap : 1, E = d->experts, K = d->top_k, H = d->hidden, I = d->inter;
@@ -441,9 +443,11 @@ static Carve plan_work(const PfHipMoeDesc *d, size_t cap, bool fused = false) {
     want[W_R2P] = Tp * K * 4;
     want[W_GROUPBAD] = prefill ? 4 : 0;
     want[W_TILES] = prefill ? (1 + (size_t)pf_prefill_max_tiles((int)T, (int)E, (int)K)) * 4 : 0;
+    c.guard = guard;
     for (int j = 0; j < W_COUNT; j++) {
         c.offset[j] = c.total;
-        c.total += (want[j] + 255) & ~(size_t)255;
+        c.size[j] = (want[j] + 255) & ~(size_t)255;
+        c.total += c.size[j] + guard;   // (diagnostics: a guard of a fixed pattern behind every buffer)
     }
     return c;
 }
@@ -526,10 +530,12 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     if (!moe || !out) return PF_HIP_E_ARGUMENT;
     PfHipWork *w = (PfHipWork *)calloc(1, sizeof *w);
     if (!w) return PF_HIP_E_MEMORY;
-    const Carve c = plan_work(&moe->desc, token_cap, fused_wanted());
+    const char *guard_env = getenv("PF_WORK_GUARD");
+    const Carve c = plan_work(&moe->desc, token_cap, fused_wanted(), guard_env && guard_env[0] == '1' ? PF_GUARD_BYTES : 0);
     uint8_t *base = nullptr;
     hipError_t e = hipMalloc((void **)&base, c.total);
     if (e == hipSuccess) e = hipMemset(base, 0, c.total);
+    for (int j = 0; j < W_COUNT && c.guard && e == hipSuccess; j++) e = hipMemset(base + c.offset[j] + c.size[j], 0xA5, c.guard);
     if (e != hipSuccess) {
         pf_set_error("workspace allocation", e);
         if (base) (void)hipFree(base);
@@ -538,6 +544,8 @@ extern "C" int pf_hip_work_create(const PfHipMoe *moe, size_t token_cap, PfHipWo
     }
     w->moe = moe; w->cap = token_cap; w->bytes = c.total;
     carve_work(w, c, base);
+    w->guard = c.guard;
+    for (int j = 0; j < W_COUNT; j++) w->guard_at[j] = c.offset[j] + c.size[j];
     // short batches through host pointers stage their rows in pinned memory: the copies are then enqueued and the call
     // waits once, for the last of them (without the block the forwards fall back to one blocking copy per buffer)
     if (hipHostMalloc((void **)&w->host, host_block_bytes(&moe->desc), hipHostMallocDefault) != hipSuccess) {
@@ -630,6 +638,28 @@ extern "C" int pf_hip_work_clear_status(PfHipWork *w) {
     if (!w) return PF_HIP_E_ARGUMENT;
     HIP_TRY(hipMemset(w->error_word, 0, 4));
     HIP_TRY(hipMemset(w->exact_rows, 0, 8));
+    return PF_HIP_OK;
+}
+
+extern "C" int pf_hip_work_check_guards(PfHipWork *w, int *damaged, int *first) {
+    if (!w || !damaged || !first) return PF_HIP_E_ARGUMENT;
+    *damaged = 0;
+    *first = -1;
+    if (!w->guard) return PF_HIP_OK;
+    HIP_TRY(hipDeviceSynchronize());
+    uint8_t *host = (uint8_t *)malloc(w->guard);
+    if (!host) return PF_HIP_E_MEMORY;
+    const uint8_t *base = (const uint8_t *)w->logits;   // the single allocation starts with its first buffer
+    for (int j = 0; j < W_COUNT; j++) {
+        if (hipMemcpy(host, base + w->guard_at[j], w->guard, hipMemcpyDeviceToHost) != hipSuccess) { free(host); return PF_HIP_E_RUNTIME; }
+        bool intact = true;
+        for (size_t b = 0; b < w->guard; b++) intact &= host[b] == 0xA5;
+        if (!intact) {
+            if (*first < 0) *first = j;
+            ++*damaged;
+        }
+    }
+    free(host);
     return PF_HIP_OK;
 }
 
@@ -846,6 +876,8 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
                                        uint32_t *error_word) {
     if (!moe || !work || !error_word) return PF_HIP_E_ARGUMENT;
     *error_word = 0;
+    // before any row is copied: the pinned block and the workspace's rows are sized for the workspace's own layer
+    if (work->moe != moe) return PF_HIP_E_ARGUMENT;
     if (tokens == 0) return PF_HIP_OK;
     if (!x || !y || tokens > work->cap) return PF_HIP_E_ARGUMENT;
     const size_t H = moe->desc.hidden, K = moe->desc.top_k;

@@ -141,6 +141,7 @@ struct PfHipWork {
     uint8_t *host_device;           // the same block as the kernels address it (they write the output rows straight into it)
     int stage_limit;                // profiling: launch only the first so many kernels of a forward; 0 = all
     int force_general;               // tests: run the general kernels even where the decode path applies
+    size_t guard, guard_at[40];      // diagnostics (PF_WORK_GUARD=1): bytes of pattern behind each buffer, and where
 };
 
 // pf_moe_kernels.hip

@@ -21,6 +21,7 @@
 // accumulators, so the result differs from the reference's serial FP32 sum by accumulation
 // order and the 2^-22 activation rounding only.
 #include "pf_moe_internal.h"
+#include "pf_upload_addr.h"
 
 typedef _Float16 half_t;
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
@@ -38,24 +39,13 @@ __host__ __device__ constexpr size_t pf_half_row(int cols) { return 2 * (size_t)
 // it is 4608 consecutive bytes: [32 headers of 16 bytes][run 0..3: 16-byte halves 0 of the 32 rows,
 // then halves 1].  One thread per 16-byte piece; rows is a multiple of 32.
 __global__ void pf_k_q4k_tile(const uint8_t *src, uint8_t *dst, size_t rows, int blocks_per_row) {
-    const size_t piece = (size_t)blockIdx.x * blockDim.x + threadIdx.x, pieces = rows * (size_t)blocks_per_row * 9;
-    if (piece >= pieces) return;
-    const size_t chunk = piece / 288, tile = chunk / blocks_per_row, kb = chunk % blocks_per_row;
-    const int p = (int)(piece % 288);
-    size_t n, off;
-    if (p < 32) {
-        n = p; off = 0;
-    } else {
-        const int q = p - 32;
-        n = q & 31; off = 16 + 32 * (q >> 6) + 16 * ((q >> 5) & 1);
-    }
-    const size_t row_bytes = (size_t)blocks_per_row * 144;
-    reinterpret_cast<uint4 *>(dst)[piece] =
-        *reinterpret_cast<const uint4 *>(src + (32 * tile + n) * row_bytes + 144 * kb + off);
+    const PfMove m = pf_q4k_tile_move((size_t)blockIdx.x * blockDim.x + threadIdx.x, rows, blocks_per_row);
+    if (!m.active) return;
+    *reinterpret_cast<uint4 *>(dst + m.dst) = *reinterpret_cast<const uint4 *>(src + m.src);
 }
 
 void pf_launch_q4k_tile(const uint8_t *d_src, uint8_t *d_dst, size_t rows, int blocks_per_row, hipStream_t stream) {
-    const size_t pieces = rows * (size_t)blocks_per_row * 9;
+    const size_t pieces = pf_q4k_tile_threads(rows, blocks_per_row);
     hipLaunchKernelGGL(pf_k_q4k_tile, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, stream, d_src, d_dst, rows, blocks_per_row);
 }
 
