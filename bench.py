@@ -85,6 +85,9 @@ WORKLOADS = {
     "q2ckpt_prefill1024_hc": dict(type="q2", tokens=1024, steps=20, warmup=5, hc=4, dims=CKPT_Q2,
                                   label="checkpoint profile Q2 at the checkpoints' widths, 1024-token prefill chunk, between "
                                         "the HC read and add of 4 residual streams, Zipf(1.1) expert popularity"),
+    "q4k_decode_streamed": dict(type=abi.GGUF_Q4_K, tokens=1, steps=512, warmup=0, streamed=448,
+                                label="Q4_K experts, decode batch 1, routed experts streamed from a file through a pool of 448 "
+                                      "slots for 512 experts"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=100, warmup=10,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),
@@ -644,10 +647,110 @@ def run_hc(args, ctx, name, steps, warmup, cpu_seconds):
     }
 
 
+def run_streamed(args, ctx, name, steps, cpu_seconds):
+    """A layer whose routed experts stay in a file (here: in the page cache of a file written just before) and reach the
+    GPU through an expert pool with fewer slots than experts: per token the router and the routing (first device call),
+    the pool's acquire (misses are read by the pool's reader threads and stored in the device layout), the expert kernels
+    on the pool's slots (second device call), the release.  Wall time of the host call per token over a seeded token
+    stream, after one pass that fills the pool; the same with a slot for every expert (no misses) beside it."""
+    import tempfile
+    api, hip, tools = ctx
+    wl = WORKLOADS[name]
+    cfg = workloads.measured_config()
+    weights = pf.LayerWeights.synthetic(cfg, wl["type"], seed=args.seed)
+    x, info = workloads.decode_tokens(weights, steps, seed=args.seed, min_margin=0.0)
+    sizes = [weights.raw[j].size // cfg.experts for j in (1, 2, 3)]
+    folder = tempfile.mkdtemp(prefix="pf_bench_")
+    path = os.path.join(folder, "experts.bin")
+    offsets, at = [], 4096
+    with open(path, "wb") as f:
+        f.write(bytes(4096))
+        for j in (1, 2, 3):
+            offsets.append(at)
+            weights.raw[j].tofile(f)
+            at += weights.raw[j].size
+    fd = os.open(path, os.O_RDONLY)
+    table = (abi.QW4ExpertLayer * 1)(abi.QW4ExpertLayer((C.c_uint64 * 3)(*offsets)))
+    h, i = cfg.hidden_size, cfg.intermediate
+    err, handle = abi.Qwen4Error(), C.c_void_p()
+    struct = weights.without_routed_bytes()
+    assert api.create_streamed(C.byref(cfg), C.byref(struct), C.byref(handle), C.byref(err)) == abi.QW4_OK, err.detail
+    cpu_api, kind = cpu_api_and_kind()
+    sample = args.cpu_sample or max(1, int(cpu_seconds / 0.14))
+    with pf.MoeLayer(cpu_api, cfg, weights, 1) as cpu:
+        c0 = time.perf_counter()
+        want = [cpu.forward(x[b:b + 1])[1:] for b in range(sample)]
+        cpu_s = time.perf_counter() - c0
+    results, parity = {}, None
+    with pf.MoeLayer(api, cfg, weights, 16, handle=handle) as layer:
+        for slots in (wl["streamed"], cfg.experts):
+            pool = api.pool_create(fd, table, 1, cfg.experts, (C.c_size_t * 3)(*sizes), slots)
+            assert pool and api.pool_set_formats(pool, (C.c_uint32 * 3)(*weights.types[1:4]), (C.c_size_t * 3)(h, h, cfg.down_physical),
+                                                 (C.c_size_t * 3)(i, i, h)) == 0
+            y = np.zeros((1, h), np.float32)
+            ids = np.zeros((1, cfg.top_k), np.uint32)
+            w = np.zeros((1, cfg.top_k), np.float32)
+            routes = abi.Qwen4MoeRoutes(abi.u32_view(ids), abi.f32_view(w))
+
+            def forward(row):
+                st = api.forward_streamed(layer.handle, pool, 0, abi.f32_view(row), abi.f32_view(y), C.byref(routes), layer.work,
+                                          C.byref(layer.err))
+                assert st == abi.QW4_OK, layer.err.detail
+
+            for b in range(steps):                      # fills the pool
+                forward(np.ascontiguousarray(x[b:b + 1]))
+            before = api.pool_stats(pool)
+            t0 = time.perf_counter()
+            for b in range(steps):
+                forward(np.ascontiguousarray(x[b:b + 1]))
+            wall = time.perf_counter() - t0
+            after = api.pool_stats(pool)
+            misses = after.misses - before.misses
+            results[slots] = {"us_per_token": round(wall / steps * 1e6, 1), "misses_per_token": round(misses / steps, 3),
+                              "miss_rate_per_routed_expert": round(misses / (steps * cfg.top_k), 4),
+                              "MB_read_per_token": round((after.bytes_read - before.bytes_read) / steps / 1e6, 3),
+                              "acquire_us_per_token": round((after.acquire_ns - before.acquire_ns) / steps / 1e3, 1)}
+            if parity is None:
+                got = []
+                for b in range(sample):
+                    forward(np.ascontiguousarray(x[b:b + 1]))
+                    got.append((y.copy(), ids.copy(), w.copy()))
+                parity = {"ids_equal": bool(all((g[1] == c[1]).all() for g, c in zip(got, want))),
+                          "within_1e-3_abs_1e-4_rel": bool(all((np.abs(g[0] - c[0]) <= 1e-3 + 1e-4 * np.abs(c[0])).all()
+                                                               for g, c in zip(got, want))),
+                          "max_abs_err": max(float(np.abs(g[0] - c[0]).max()) for g, c in zip(got, want)), "error_word": 0}
+            api.pool_destroy(pool)
+    os.close(fd)
+    os.unlink(path)
+    os.rmdir(folder)
+    main = results[wl["streamed"]]
+    per_miss = (main["us_per_token"] - results[cfg.experts]["us_per_token"]) / max(main["misses_per_token"], 1e-9)
+    return {
+        "metric": "moe_decode_us_per_layer_token", "value": main["us_per_token"], "unit": "us/layer/token (host call, wall clock)",
+        "n_gpus": 1, "steps": steps, "warmup": steps, "ms_per_step": round(main["us_per_token"] * 1e-3, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": DTYPE_DECODE, "data": "synthetic",
+        "config": {"workload": f"one MoE layer, hidden {cfg.hidden_size}, {cfg.experts} experts, top-{cfg.top_k}, intermediate "
+                               f"{cfg.intermediate}, shared {cfg.shared_intermediate}; {wl['label']}; {steps} seeded tokens, each "
+                               "routed to its own experts; the file is in the page cache (written just before)",
+                   "tokens_per_step": 1, "expert_format": FORMAT_LABEL[wl["type"]], "pool_slots": wl["streamed"],
+                   "readers": 8, "inputs": info},
+        "pool": {str(k): v for k, v in results.items()},
+        "us_per_missed_expert": round(per_miss, 1),
+        "GBps_of_missed_experts": round(sum(sizes) / max(per_miss, 1e-9) / 1e3, 2),
+        "roofline": {"bound": "hbm", "kernel": "not a kernel figure: the misses are bound by the file reads and the copies to the GPU",
+                     "achieved": None, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": None, "traffic": None},
+        "cpu_baseline": {"value": round(cpu_s / sample * 1e6, 1), "unit": "us/layer/token", "cores": 1, "kind": kind,
+                         "sample": f"first {sample} tokens, every expert in memory, {cpu_s:.1f} s"},
+        "parity_on_sample": parity,
+    }
+
+
 def run_one(args, ctx, name, cpu_seconds):
     wl = WORKLOADS[name]
     steps = args.steps if args.steps is not None else wl["steps"]
     warmup = args.warmup if args.warmup is not None else wl["warmup"]
+    if wl.get("streamed"):
+        return run_streamed(args, ctx, name, steps, cpu_seconds)
     if name == "q4k_stack48":
         return run_stack(args, ctx, min(steps, 200), warmup, cpu_seconds)
     if wl.get("hc"):

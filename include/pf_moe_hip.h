@@ -241,6 +241,17 @@ int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, size_t n_out, 
 int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, void *region, size_t slot,
                       const void *file_bytes);
 int pf_hip_pool_slot_tiled(uint32_t gguf_type, size_t n_out);
+/* A reader's staging, allocated once: `bytes` of page-locked host memory to read the file into (pf_hip_stage_host),
+ * as much device memory for the bytes on their way into a split or tile kernel, and a stream of the reader's own.
+ * pf_hip_pool_store_staged stores the `file_bytes` the host memory holds like pf_hip_pool_store does (gguf_type
+ * UINT32_MAX: as they are, at region + slot * file_bytes), enqueued on that stream and waited for: it allocates
+ * nothing, and readers with stages of their own run side by side. */
+typedef struct PfHipStage PfHipStage;
+int pf_hip_stage_create(size_t bytes, PfHipStage **out);
+void pf_hip_stage_destroy(PfHipStage *stage);
+void *pf_hip_stage_host(PfHipStage *stage);
+int pf_hip_pool_store_staged(PfHipStage *stage, uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots,
+                             void *region, size_t slot, size_t file_bytes);
 
 /* Minimal device-memory helpers so that a host program can keep inputs resident. */
 int pf_hip_malloc(void **d_ptr, size_t bytes);

@@ -1075,6 +1075,80 @@ extern "C" int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, siz
     return PF_HIP_OK;
 }
 
+// ---- a reader's staging (expert streaming): page-locked host memory the file is read into, device memory the bytes are
+// copied to before a split or tile kernel lays them out in the slot, and a stream of the reader's own, all allocated once
+struct PfHipStage {
+    uint8_t *host, *device;
+    size_t bytes;
+    hipStream_t stream;
+};
+
+extern "C" int pf_hip_stage_create(size_t bytes, PfHipStage **out) {
+    if (!out || !bytes) return PF_HIP_E_ARGUMENT;
+    *out = nullptr;
+    PfHipStage *st = (PfHipStage *)calloc(1, sizeof *st);
+    if (!st) return PF_HIP_E_MEMORY;
+    st->bytes = bytes;
+    hipError_t e = hipHostMalloc((void **)&st->host, bytes, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipMalloc((void **)&st->device, bytes);
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&st->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        pf_set_error("staging of an expert pool's reader", e);
+        if (st->host) (void)hipHostFree(st->host);
+        if (st->device) (void)hipFree(st->device);
+        free(st);
+        return PF_HIP_E_MEMORY;
+    }
+    *out = st;
+    return PF_HIP_OK;
+}
+
+extern "C" void pf_hip_stage_destroy(PfHipStage *st) {
+    if (!st) return;
+    (void)hipStreamDestroy(st->stream);
+    (void)hipHostFree(st->host);
+    (void)hipFree(st->device);
+    free(st);
+}
+
+extern "C" void *pf_hip_stage_host(PfHipStage *st) { return st ? st->host : nullptr; }
+
+// The expert the stage's host memory holds (one expert's slice of one matrix, as the file stores it) into slot `slot` of
+// the matrix's region: gguf_type == UINT32_MAX copies `file_bytes` bytes as they are to region + slot * file_bytes.
+// Enqueued on the stage's stream and waited for: no allocation, and readers with stages of their own run side by side.
+extern "C" int pf_hip_pool_store_staged(PfHipStage *st, uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, void *region,
+                                        size_t slot, size_t file_bytes) {
+    if (!st || !region || slot >= slots || file_bytes > st->bytes) return PF_HIP_E_ARGUMENT;
+    uint8_t *base = static_cast<uint8_t *>(region);
+    if (gguf_type == UINT32_MAX) {
+        HIP_TRY(hipMemcpyAsync(base + slot * file_bytes, st->host, file_bytes, hipMemcpyHostToDevice, st->stream));
+        HIP_TRY(hipStreamSynchronize(st->stream));
+        return PF_HIP_OK;
+    }
+    PfTensorPlace place;
+    if (!pf_tensor_place(gguf_type, k_storage, n_out, slots, &place) || place.gguf_bytes / slots != file_bytes) return PF_HIP_E_ARGUMENT;
+    const size_t head = split_header_bytes(gguf_type);
+    if (!pf_hip_pool_slot_tiled(gguf_type, n_out) && !head) {   // as the file stores it
+        HIP_TRY(hipMemcpyAsync(base + slot * place.expert_bytes, st->host, file_bytes, hipMemcpyHostToDevice, st->stream));
+        HIP_TRY(hipStreamSynchronize(st->stream));
+        return PF_HIP_OK;
+    }
+    HIP_TRY(hipMemcpyAsync(st->device, st->host, file_bytes, hipMemcpyHostToDevice, st->stream));
+    if (pf_hip_pool_slot_tiled(gguf_type, n_out)) {   // Q4_K: the slot in the tile order every kernel family reads
+        pf_launch_q4k_tile(st->device, base + slot * place.expert_bytes, n_out, place.blocks_per_row, st->stream);
+    } else {
+        size_t block, size;
+        block_geometry(gguf_type, &block, &size);
+        const size_t blocks = (size_t)place.blocks_per_row * n_out;
+        uint8_t *payload = base + slot * place.expert_bytes, *scales = base + place.scale_offset + slot * blocks * head;
+        if (gguf_type == PF_IQ2_XXS) pf_launch_iq2_split(st->device, payload, reinterpret_cast<uint16_t *>(scales), blocks, st->stream);
+        else pf_launch_block_split(st->device, payload, scales, blocks, (int)size, (int)head, st->stream);
+    }
+    HIP_TRY(hipGetLastError());
+    HIP_TRY(hipStreamSynchronize(st->stream));
+    return PF_HIP_OK;
+}
+
 // One expert's slice of one matrix, as the file stores it, into slot `slot` of the matrix's region.
 extern "C" int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, void *region, size_t slot,
                                  const void *file_bytes) {

@@ -4,8 +4,10 @@
  * Recency is a counter stamped on a slot whenever it is acquired; the victim of a miss is the slot
  * with the oldest stamp among those nobody pins (fresh pools stamp slot s with s, so slot 0 goes first,
  * as in the reference).  A scan over the slots per miss is enough: pools hold a few thousand slots and
- * a miss costs a file read of megabytes.  Reads go through one staging buffer per reader thread:
- * pread into it, then one copy to the slot's place in the matrix region. */
+ * a miss costs a file read of megabytes.  The readers are threads the pool starts once, at its first miss, each
+ * with a stage of its own (page-locked host memory, device memory and a stream, pf_hip_stage_create): a reader
+ * preads one matrix of one missed expert into its page-locked memory and has it copied (split, tiled) into the
+ * slot on its stream, so no acquire starts a thread or allocates anything. */
 #define _GNU_SOURCE
 #include "../../include/qwen4_expert_pool.h"
 #include "../../include/pf_moe_hip.h"
@@ -17,6 +19,7 @@
 #include <unistd.h>
 
 #define NO_SLOT UINT32_MAX
+#define QW4_POOL_MAX_READERS 64
 
 struct QW4ExpertPool {
     int fd;
@@ -34,6 +37,16 @@ struct QW4ExpertPool {
     bool formatted, used;
     uint32_t type[3];
     size_t k_storage[3], n_out[3], scale_offset[3];
+    /* the readers: started at the first miss; they sleep on `wake` between acquires */
+    pthread_mutex_t lock;
+    pthread_cond_t wake, done;
+    pthread_t thread[QW4_POOL_MAX_READERS];
+    PfHipStage *stage[QW4_POOL_MAX_READERS + 1];   /* the last one is the acquiring thread's own */
+    uint32_t started;
+    uint64_t round;            /* incremented per batch of reads; a reader takes part once per round */
+    uint32_t running;          /* readers still at work on the current round */
+    bool quit, lock_ready;
+    struct Reads *reads;       /* the current round's */
 };
 
 QW4ExpertPool *qw4_pool_create(int fd, const QW4ExpertLayer *layers, uint32_t n_layers, uint32_t experts,
@@ -43,6 +56,8 @@ QW4ExpertPool *qw4_pool_create(int fd, const QW4ExpertLayer *layers, uint32_t n_
     QW4ExpertPool *p = calloc(1, sizeof *p);
     if (!p) return NULL;
     p->fd = fd; p->n_layers = n_layers; p->experts = experts; p->slots = slots; p->readers = 8;
+    if (pthread_mutex_init(&p->lock, NULL) || pthread_cond_init(&p->wake, NULL) || pthread_cond_init(&p->done, NULL)) { free(p); return NULL; }
+    p->lock_ready = true;
     const size_t keys = (size_t)n_layers * experts;
     p->layers = malloc(n_layers * sizeof *p->layers);
     p->where = malloc(keys * sizeof *p->where);
@@ -73,6 +88,15 @@ QW4ExpertPool *qw4_pool_create(int fd, const QW4ExpertLayer *layers, uint32_t n_
 
 void qw4_pool_destroy(QW4ExpertPool *p) {
     if (!p) return;
+    if (p->lock_ready) {
+        pthread_mutex_lock(&p->lock);
+        p->quit = true;
+        pthread_cond_broadcast(&p->wake);
+        pthread_mutex_unlock(&p->lock);
+        for (uint32_t j = 0; j < p->started; j++) pthread_join(p->thread[j], NULL);
+        for (uint32_t j = 0; j <= QW4_POOL_MAX_READERS; j++) pf_hip_stage_destroy(p->stage[j]);
+        pthread_cond_destroy(&p->wake); pthread_cond_destroy(&p->done); pthread_mutex_destroy(&p->lock);
+    }
     for (int m = 0; m < 3; m++)
         if (p->region[m]) pf_hip_free(p->region[m]);
     free(p->layers); free(p->where); free(p->holds); free(p->pins); free(p->stamp); free(p->new_slot); free(p->new_expert);
@@ -134,7 +158,7 @@ QW4PoolStats qw4_pool_stats(const QW4ExpertPool *p) {
  * A job is one matrix of one missed expert; the readers take jobs from a shared counter until none
  * is left.  (The reference hands reader g the jobs g, g + width, ...; which reader reads what does
  * not show in the result.) */
-typedef struct {
+typedef struct Reads {
     QW4ExpertPool *p;
     uint32_t layer, misses;
     atomic_size_t next;
@@ -151,29 +175,89 @@ static int read_exactly(int fd, unsigned char *dst, size_t bytes, uint64_t offse
     return 0;
 }
 
-static void *reader(void *arg) {
-    Reads *r = arg;
-    QW4ExpertPool *p = r->p;
+static size_t widest_matrix(const QW4ExpertPool *p) {
     size_t widest = p->bytes[0];
     for (int m = 1; m < 3; m++) widest = p->bytes[m] > widest ? p->bytes[m] : widest;
-    unsigned char *staging = malloc(widest);
-    if (!staging) { atomic_store(&r->failed, 1); return NULL; }
+    return widest;
+}
+
+/* one reader's share of a round: jobs from the shared counter, through its stage */
+static void read_jobs(Reads *r, PfHipStage *stage) {
+    QW4ExpertPool *p = r->p;
+    unsigned char *host = pf_hip_stage_host(stage);
     for (;;) {
         const size_t job = atomic_fetch_add(&r->next, 1);
         if (job >= (size_t)r->misses * 3 || atomic_load(&r->failed)) break;
         const size_t miss = job / 3;
         const int m = (int)(job % 3);
         const uint64_t from = p->layers[r->layer].offset[m] + (uint64_t)p->new_expert[miss] * p->bytes[m];
-        unsigned char *to = (unsigned char *)p->region[m] + (size_t)p->new_slot[miss] * p->bytes[m];
-        int rc = read_exactly(p->fd, staging, p->bytes[m], from);
-        if (!rc && p->formatted)
-            rc = pf_hip_pool_store(p->type[m], p->k_storage[m], p->n_out[m], p->slots, p->region[m], p->new_slot[miss], staging);
-        else if (!rc)
-            rc = pf_hip_memcpy_h2d(to, staging, p->bytes[m]);
+        int rc = read_exactly(p->fd, host, p->bytes[m], from);
+        if (!rc)
+            rc = pf_hip_pool_store_staged(stage, p->formatted ? p->type[m] : UINT32_MAX, p->k_storage[m], p->n_out[m], p->slots,
+                                          p->region[m], p->new_slot[miss], p->bytes[m]);
         if (rc) atomic_store(&r->failed, 1);
     }
-    free(staging);
+}
+
+typedef struct { QW4ExpertPool *p; uint32_t index; uint64_t round; } ReaderArg;
+
+static void *reader_main(void *arg) {
+    ReaderArg *me = arg;
+    QW4ExpertPool *p = me->p;
+    const uint32_t index = me->index;
+    uint64_t seen = me->round;   /* the rounds before this reader existed are not its business */
+    free(me);
+    pthread_mutex_lock(&p->lock);
+    for (;;) {
+        while (!p->quit && p->round == seen) pthread_cond_wait(&p->wake, &p->lock);
+        if (p->quit) break;
+        seen = p->round;
+        Reads *r = p->reads;
+        pthread_mutex_unlock(&p->lock);
+        read_jobs(r, p->stage[index]);
+        pthread_mutex_lock(&p->lock);
+        if (--p->running == 0) pthread_cond_signal(&p->done);
+    }
+    pthread_mutex_unlock(&p->lock);
     return NULL;
+}
+
+/* Starts readers until `want` of them (besides the acquiring thread) exist; fewer when a thread or a stage cannot be had. */
+static void start_readers(QW4ExpertPool *p, uint32_t want) {
+    const size_t widest = widest_matrix(p);
+    while (p->started < want && p->started < QW4_POOL_MAX_READERS) {
+        const uint32_t index = p->started;
+        if (!p->stage[index] && pf_hip_stage_create(widest, &p->stage[index]) != PF_HIP_OK) break;
+        ReaderArg *arg = malloc(sizeof *arg);
+        if (!arg) break;
+        arg->p = p; arg->index = index; arg->round = p->round;   /* (only the acquiring thread changes it, and it is here) */
+        if (pthread_create(&p->thread[index], NULL, reader_main, arg)) { free(arg); break; }
+        p->started++;
+    }
+}
+
+/* The misses of an acquire, read together: the pool's readers and this thread.  0, or -1 if a read or a store failed. */
+static int read_misses(QW4ExpertPool *p, uint32_t layer, uint32_t misses) {
+    Reads reads = {.p = p, .layer = layer, .misses = misses};
+    atomic_init(&reads.next, 0);
+    atomic_init(&reads.failed, 0);
+    uint32_t width = p->readers < misses * 3 ? p->readers : misses * 3;
+    if (width > QW4_POOL_MAX_READERS) width = QW4_POOL_MAX_READERS;
+    PfHipStage **mine = &p->stage[QW4_POOL_MAX_READERS];
+    if (!*mine && pf_hip_stage_create(widest_matrix(p), mine) != PF_HIP_OK) return -1;
+    if (width > 1) start_readers(p, width - 1);
+    pthread_mutex_lock(&p->lock);
+    p->reads = &reads;
+    p->running = p->started;      /* every started reader wakes, also those this acquire has no job for */
+    p->round++;
+    pthread_cond_broadcast(&p->wake);
+    pthread_mutex_unlock(&p->lock);
+    read_jobs(&reads, *mine);     /* this thread reads too; alone when no other could be started */
+    pthread_mutex_lock(&p->lock);
+    while (p->running) pthread_cond_wait(&p->done, &p->lock);
+    p->reads = NULL;
+    pthread_mutex_unlock(&p->lock);
+    return atomic_load(&reads.failed) ? -1 : 0;
 }
 
 static uint64_t now_ns(void) {
@@ -213,20 +297,7 @@ int qw4_pool_acquire(QW4ExpertPool *p, uint32_t layer, const uint32_t *experts, 
         slots[i] = s;
     }
     /* pass 2: the misses, read together */
-    if (!rc && misses) {
-        Reads reads = {.p = p, .layer = layer, .misses = misses};
-        atomic_init(&reads.next, 0);
-        atomic_init(&reads.failed, 0);
-        uint32_t width = p->readers < misses * 3 ? p->readers : misses * 3;
-        if (width > 64) width = 64;
-        pthread_t thread[64];
-        uint32_t started = 0;
-        for (; started + 1 < width; started++)
-            if (pthread_create(&thread[started], NULL, reader, &reads)) break;
-        reader(&reads);   /* this thread reads too; alone when no other could be started */
-        for (uint32_t j = 0; j < started; j++) pthread_join(thread[j], NULL);
-        if (atomic_load(&reads.failed)) { qw4_pool_release(p, slots, n); rc = -1; }
-    }
+    if (!rc && misses && read_misses(p, layer, misses)) { qw4_pool_release(p, slots, n); rc = -1; }
     if (rc)   /* the slots this call took hold nothing usable: forget them (their recency stays) */
         for (uint32_t j = 0; j < misses; j++) {
             p->where[p->holds[p->new_slot[j]]] = NO_SLOT;

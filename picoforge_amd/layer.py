@@ -35,6 +35,16 @@ class LayerWeights:
     def nbytes(self):
         return sum(b.size for b in self.raw)
 
+    def without_routed_bytes(self):
+        """The same views with the routed tensors' bytes withheld: what pf_moe_create_streamed takes for a layer whose
+        routed experts stay in a file."""
+        struct = abi.Qwen4MoeWeights()
+        C.memmove(C.byref(struct), C.byref(self.struct), C.sizeof(struct))
+        for role in ("gate", "up", "down"):
+            view = getattr(struct, role)
+            view.span.data, view.span.bytes = None, 0
+        return struct
+
     # the two profiles of real checkpoints (src/qwen4_config.c:197-216, src/qwen4_weights.c:91-99):
     # routed gate/up, routed down, shared expert
     PROFILE = {"q2": (abi.GGUF_IQ2_XXS, abi.GGUF_Q2_K, abi.GGUF_Q8_0), "q4": (abi.GGUF_Q4_K, abi.GGUF_MXFP4, abi.GGUF_Q8_0)}

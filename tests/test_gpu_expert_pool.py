@@ -120,12 +120,7 @@ def test_pool_bookkeeping_and_contents(product, tmp_path):
 
 def streamed_weights(weights):
     """The same views with the routed tensors' bytes withheld."""
-    struct = abi.Qwen4MoeWeights()
-    C.memmove(C.byref(struct), C.byref(weights.struct), C.sizeof(struct))
-    for role in ("gate", "up", "down"):
-        view = getattr(struct, role)
-        view.span.data, view.span.bytes = None, 0
-    return struct
+    return weights.without_routed_bytes()
 
 
 @pytest.mark.parametrize("gtype,formatted", [(abi.GGUF_Q4_K, False), (abi.GGUF_F16, False), (abi.GGUF_Q4_K, True),
