@@ -56,6 +56,10 @@ WORKLOADS = {
     "iq2xxs_decode": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=2000, warmup=200, label="IQ2_XXS experts, decode batch 1"),
     "q4k_verify4": dict(type=abi.GGUF_Q4_K, tokens=4, steps=1000, warmup=100,
                         label="Q4_K experts, 4-token verify batch, ~50% expert overlap"),
+    "q4k_verify8": dict(type=abi.GGUF_Q4_K, tokens=8, steps=500, warmup=50,
+                        label="Q4_K experts, 8-token batch of the same process (each token about half of its neighbour's experts)"),
+    "q4k_verify16": dict(type=abi.GGUF_Q4_K, tokens=16, steps=250, warmup=25,
+                         label="Q4_K experts, 16-token batch of the same process: the longest the decode kernels take"),
     "q4k_prefill1024": dict(type=abi.GGUF_Q4_K, tokens=1024, steps=20, warmup=5, label="Q4_K experts, " + PREFILL_LABEL),
     "q4k_prefill2048": dict(type=abi.GGUF_Q4_K, tokens=2048, steps=20, warmup=5,
                             label="Q4_K experts, " + PREFILL_LABEL.replace("1024", "2048") + " (the chunk size of the 48-layer stack)"),
@@ -102,6 +106,10 @@ ALL_CONFIGS = ["iq2xxs_decode", "q4k_verify4", "q4k_prefill1024", "q4k_stack48"]
 DECODE_STAGES = ["pf_k_dec_router (router logits)",
                  "pf_k_dec_gate_up (routing, gate/up + SwiGLU, routed and shared)",
                  "pf_k_dec_down (down products, routed and shared, combine)"]
+ROUTED_DECODE_STAGES = ["pf_k_dec_router (router logits)",
+                        "pf_k_dec_route (top-k of every token, serial-order re-routes)",
+                        "pf_k_dec_gate_up_given (gate/up + SwiGLU of the experts it is given, routed and shared)",
+                        "pf_k_dec_down (down products, routed and shared, combine)"]
 FUSED_DECODE_STAGES = ["pf_k_dec_router (router logits)",
                        "pf_k_dec_fused (routing, gate/up + SwiGLU, activation lines through memory, down products, combine)"]
 GENERAL_STAGES = ["pf_k_pre (router logits, shared gate/up + SwiGLU, shared gate)",
@@ -255,10 +263,10 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
     wl = WORKLOADS[name]
     cfg = layer_config(wl)
     tokens = wl["tokens"]
-    prefill = tokens > 4
+    chunk_inputs = tokens > 16          # a chunk under the Zipf router; shorter batches are correlated tokens
     t0 = time.time()
     weights = pf.LayerWeights.synthetic(cfg, wl["type"], seed=args.seed)
-    if prefill:
+    if chunk_inputs:
         # Zipf(1.1) popularity profile, flattened (logit bias -1.1 * 0.18 * ln rank) so that the busiest
         # expert receives about 150 of the 1024 tokens, as the configuration states
         workloads.zipf_router(weights, seed=args.seed, temperature=0.18)
@@ -276,7 +284,7 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
         unique = float(cfg.top_k)
     else:
         n_inputs = max(1, min(steps, 64))
-        x, info = workloads.verify_batches(weights, n_inputs, seed=args.seed)
+        x, info = workloads.verify_batches(weights, n_inputs, seed=args.seed, group=tokens)
         unique = info["mean_unique_experts"]
     prep_s = time.time() - t0
 
@@ -302,9 +310,12 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
     # groups of every forward; a group's duration is the difference between consecutive plans (it includes
     # the dispatch gap before it, as a profiler's start-to-end time of a dependent kernel does).
     family = hip.moe_kernel_family(moe, work, tokens)
+    prefill = family == 2 or (family == 0 and chunk_inputs)   # accounted as a chunk: bytes of the grouped products, tokens per second
     names = {0: GENERAL_STAGES, 1: DECODE_STAGES, 2: PREFILL_STAGES}[family]
     if family == 1 and hip.moe_decode_launches(moe, work, tokens) == 2:
         names = FUSED_DECODE_STAGES
+    if family == 1 and hip.moe_decode_launches(moe, work, tokens) == 4:
+        names = ROUTED_DECODE_STAGES
     stage_us = [1e-3] * len(names)
     if not args.skip_stages:
         previous = 0.0
@@ -350,6 +361,8 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
                        unique * lb["down"] + lb["shared_down"]]
         if len(names) == 2:
             stage_bytes = [stage_bytes[0], stage_bytes[1] + stage_bytes[2]]
+        if family == 1 and len(names) == 4:   # the routing launch reads the tokens' logits and their noise terms
+            stage_bytes = [stage_bytes[0], tokens * cfg.experts * 8, stage_bytes[1], stage_bytes[2]]
         if family == 0:
             stage_bytes = [lb["routers"] + lb["shared_gate_up"], tokens * cfg.experts * 8, unique * lb["gate_up"],
                            unique * lb["down"] + lb["shared_down"]]

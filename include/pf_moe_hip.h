@@ -89,7 +89,9 @@ int pf_hip_moe_kernel_family(const PfHipMoe *moe, const PfHipWork *work, size_t 
  * SwiGLU; down products and combine), or 2 where one launch takes the whole expert stage (one token,
  * Q4_K or IQ2_XXS throughout, a workspace created with PF_MOE_DECODE_FUSED=1 in the environment, a
  * device with a compute unit per workgroup: an option, slower than the three kernels where it was
- * measured).  0: the forward runs other kernels. */
+ * measured), or 4 where the routing runs in a launch of its own between the router logits and a
+ * gate/up kernel that is given the experts (three tokens or more on the tile-ordered kernels).
+ * 0: the forward runs other kernels. */
 int pf_hip_moe_decode_launches(const PfHipMoe *moe, const PfHipWork *work, size_t tokens);
 /* Device pointers into the workspace, valid after a forward: expert ids
  * [tokens, top_k] uint32, route weights [tokens, top_k], router logits

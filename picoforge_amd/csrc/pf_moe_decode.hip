@@ -2456,19 +2456,31 @@ static PfHipMoeDesc desc_of(const PfKernelArgs &a) {
     return d;
 }
 
+// the routing in a launch of its own, ahead of a gate/up kernel that is given the experts
+// (from three tokens on: with two the routing launch costs more than the workgroups' own routing, 24.8 against 22.9 us,
+// with one 18.4 against 16.5)
+#ifndef PF_ROUTE_FIRST_FROM
+#define PF_ROUTE_FIRST_FROM 3
+#endif
+template <bool POOL>
+static bool routes_first(const PfKernelArgs &a, int tokens) {
+    return !POOL && tokens >= PF_ROUTE_FIRST_FROM && a.hidden <= 64 * Q4G_ITEMS * Q4G_WAVES && a.top_k <= 15;
+}
+
 template <int FG, int FD, int FS, bool POOL = false>
 static void launch_q4t_experts(const PfKernelArgs &a, int tokens, hipStream_t stream, int last) {
     const int H = a.hidden, I = a.inter, Is = a.shared_inter, K = a.top_k;
     // kernel 2: every workgroup extracts the maxima up to its own slot from all of its token's logits; with several
     // tokens the routing runs first, in a launch of its own
-    // (from three tokens on: with two, the routing launch costs more than the workgroups' own routing, 24.8 against 22.9 us)
-    if (!POOL && tokens >= 3 && a.hidden <= 64 * Q4G_ITEMS * Q4G_WAVES && a.top_k <= 15) {
+    if (routes_first<POOL>(a, tokens)) {   // four launches: `last` counts them
         launch_dec_route(a, tokens, stream);
+        if (last < 3) return;
         launch_gate_up_given<FG, FS>(a, tokens, stream);
+        if (last < 4) return;
     } else {
         launch_gate_up_q4t<FG, FS, POOL>(a, tokens, stream);
+        if (last < 3) return;
     }
-    if (last < 3) return;
     const size_t widest = I > Is ? I : Is;
     constexpr bool GRID = FD == PF_IQ2_XXS || FS == PF_IQ2_XXS;
     // rows per workgroup: eight in the tile order; for down tensors kept row by row the fewest that leave no more
@@ -2491,7 +2503,7 @@ static void launch_q4t_experts(const PfKernelArgs &a, int tokens, hipStream_t st
 
 template <int FG, int FD, int FS>
 static void launch_decode_q4t(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
-    const int last = stage_limit ? stage_limit : 3;
+    const int last = stage_limit ? stage_limit : 4;
     pf_launch_dec_router(a, tokens, (a.experts + 3) / 4, stream);
     if (last < 2) return;
     if constexpr (FG == FD && FG == FS && (FG == PF_Q4_K || FG == PF_IQ2_XXS)) {
@@ -2585,7 +2597,7 @@ void pf_launch_decode_stream_experts(const PfKernelArgs &a, int tokens, hipStrea
 
 int pf_decode_launches(const PfKernelArgs &a, int tokens) {
     const int combination = pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq);
-    if (tokens != 1) return 3;
+    if (tokens != 1) return combination != 0 && routes_first<false>(a, tokens) ? 4 : 3;
     if (combination == 1) return fused_applies<PF_Q4_K>(a) ? 2 : 3;
     if (combination == 2) return fused_applies<PF_IQ2_XXS>(a) ? 2 : 3;
     return 3;

@@ -190,7 +190,8 @@ void pf_launch_dec_router(const PfKernelArgs &a, int tokens, int router_blocks, 
 // bytes of the activation lines a workspace needs for the one-launch expert stage of a one-token forward (0: the
 // layer's shape or formats are not taken)
 void pf_decode_fused_scratch(const PfHipMoeDesc &d, size_t *line_bytes);
-// launches per one-token forward on the decode path: 2 with the fused expert stage, else 3
+// launches per forward on the decode path: 2 for one token with the fused expert stage, 4 where the routing runs in a
+// launch of its own (three tokens or more on the tile kernels), else 3
 int pf_decode_launches(const PfKernelArgs &a, int tokens);
 // kernels 2 and 3 of the tile decode path on pool slots, for a Q4_K layer or one in the q4 checkpoint profile (expert
 // streaming: kernel 1 ran in an earlier call)

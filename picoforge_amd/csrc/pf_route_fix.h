@@ -28,71 +28,56 @@
 #include "pf_route_device.h"
 #include "pf_route_fast.h"
 
-// The serial sums.  A sum is one chain of dependent additions, k ascending (4 ns each for a wave alone on its SIMD:
-// 8 us for 2048 values) and the chains of different experts are independent, so one wave runs them all, a lane per
-// candidate: two vector instructions a step whatever the number of candidates.  (A wave per candidate, with the
-// lanes forming the products side by side and the chain fetching them back through v_readlane, costs the same two
-// instructions a step for a single chain: ten candidates on four SIMDs took 30 us.)  What the chain must never do
-// is wait for memory, and a lane reading its own row keeps too little on its way (two to five 128-byte lines a lane:
-// 22-28 us).  So the other waves of the workgroup bring the candidates' rows into LDS, a chunk of every row at a
-// time with coalesced loads, one chunk ahead of the chain (PF_FIX_CHUNK_FLOATS floats of LDS per buffer: chunks of
-// 512 values for up to 16 candidates, 256 up to 32, 128 up to 64), and the chain reads LDS four pieces ahead.
+// The serial sums.  A sum is one chain of dependent additions, k ascending, and the chains of different experts are
+// independent, so one wave runs them all, a lane per candidate: one vector instruction a step whatever the number of
+// candidates.  (A wave per candidate, with the lanes forming the products side by side and the chain fetching them
+// back through v_readlane, costs two instructions a step for a single chain: ten candidates on four SIMDs took 30 us.)
+// What the chain must never do is wait for memory, and a lane reading its own row keeps too little on its way (two to
+// five 128-byte lines a lane: 22-28 us).  So the other waves of the workgroup bring the candidates' rows in with
+// coalesced loads, multiply them by the token's values and leave the products in LDS, a chunk of every row at a time,
+// one chunk ahead of the chain (PF_FIX_CHUNK_FLOATS floats of LDS per buffer: chunks of 512 values for up to 16
+// candidates, 256 up to 32, 128 up to 64), and the chain reads LDS four pieces ahead.  (With the multiplications in the
+// chain's own wave, two instructions a step, 2048 values took 8 us.)
 #define PF_FIX_CHUNK_FLOATS 8448   // 16 rows of 512 + 4 (or 32 of 256 + 4, or 64 of 128 + 4) floats, rounded up
 
-// The chain over one chunk: w = this lane's row of the chunk in LDS, x = the token's values of the chunk in LDS
-// (the same for every lane), pieces = 16-byte pieces in the chunk.  A piece's products are formed between the
-// additions of the piece before it; the LDS reads run a batch of four pieces ahead.
-__device__ __forceinline__ float pf_serial_chunk(float sum, const float *w, const float *x, int pieces) {
+// The chain over one chunk: p = this lane's row of the chunk's PRODUCTS in LDS (each w[k] * x[k] rounded, formed by the
+// waves that brought the row), pieces = 16-byte pieces in the chunk.  The chain is additions only, one vector instruction
+// a step; the LDS reads run a batch of four pieces ahead.
+__device__ __forceinline__ float pf_serial_chunk(float sum, const float *p, int pieces) {
 #pragma clang fp contract(off)
-    const float4 *w4 = reinterpret_cast<const float4 *>(w), *x4 = reinterpret_cast<const float4 *>(x);
-    float4 wa[4], xa[4], wb[4], xb[4];
-    auto fetch = [&](float4 (&wv)[4], float4 (&xv)[4], int first) {   // beyond the chunk: its last batch again, not used
+    const float4 *p4 = reinterpret_cast<const float4 *>(p);
+    float4 a[4], b[4];
+    auto fetch = [&](float4 (&v)[4], int first) {   // beyond the chunk: its last batch again, not used
         const int at = min(first, pieces - 4);
 #pragma unroll
-        for (int j = 0; j < 4; j++) { wv[j] = w4[at + j]; xv[j] = x4[at + j]; }
+        for (int j = 0; j < 4; j++) v[j] = p4[at + j];
     };
-    auto batch = [&](const float4 (&wv)[4], const float4 (&xv)[4]) {
-        float p0 = wv[0].x * xv[0].x, p1 = wv[0].y * xv[0].y, p2 = wv[0].z * xv[0].z, p3 = wv[0].w * xv[0].w;
+    auto batch = [&](const float4 (&v)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int n = j + 1 < 4 ? j + 1 : j;   // the last piece forms its own products again, unused
             __builtin_amdgcn_sched_barrier(0);
-            sum = sum + p0;
-            __builtin_amdgcn_sched_barrier(0);
-            const float n0 = wv[n].x * xv[n].x;
-            __builtin_amdgcn_sched_barrier(0);
-            sum = sum + p1;
-            __builtin_amdgcn_sched_barrier(0);
-            const float n1 = wv[n].y * xv[n].y;
-            __builtin_amdgcn_sched_barrier(0);
-            sum = sum + p2;
-            __builtin_amdgcn_sched_barrier(0);
-            const float n2 = wv[n].z * xv[n].z;
-            __builtin_amdgcn_sched_barrier(0);
-            sum = sum + p3;
-            __builtin_amdgcn_sched_barrier(0);
-            const float n3 = wv[n].w * xv[n].w;
-            __builtin_amdgcn_sched_barrier(0);
-            p0 = n0; p1 = n1; p2 = n2; p3 = n3;
+            sum = sum + v[j].x;
+            sum = sum + v[j].y;
+            sum = sum + v[j].z;
+            sum = sum + v[j].w;
         }
     };
     const int whole = pieces / 8 * 8;
     if (whole > 0) {
-        fetch(wa, xa, 0);
-        for (int b = 0; b < whole; b += 8) {
-            fetch(wb, xb, b + 4);
-            batch(wa, xa);
-            fetch(wa, xa, b + 8);
-            batch(wb, xb);
+        fetch(a, 0);
+        for (int q = 0; q < whole; q += 8) {
+            fetch(b, q + 4);
+            batch(a);
+            fetch(a, q + 8);
+            batch(b);
         }
     }
     for (int j = whole; j < pieces; j++) {   // a last chunk that is not whole batches
-        const float4 wv = w4[j], xv = x4[j];
-        const float p0 = wv.x * xv.x, p1 = wv.y * xv.y, p2 = wv.z * xv.z, p3 = wv.w * xv.w;
-        sum = sum + p0;
-        sum = sum + p1;
-        sum = sum + p2;
-        sum = sum + p3;
+        const float4 v = p4[j];
+        sum = sum + v.x;
+        sum = sum + v.y;
+        sum = sum + v.z;
+        sum = sum + v.w;
     }
     return sum;
 }
@@ -185,8 +170,13 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
                     held[j] = reinterpret_cast<const float4 *>(router + expert * H + first)[piece[j]];
                 }
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (i0 + j * helpers < total) reinterpret_cast<float4 *>(buf + row[j] * pitch)[piece[j]] = held[j];
+                for (int j = 0; j < 4; j++) {   // the products, each rounded once, as the reference forms them before it adds
+                    if (i0 + j * helpers < total) {
+                        const float4 xv = reinterpret_cast<const float4 *>(xs + first)[piece[j]];
+                        reinterpret_cast<float4 *>(buf + row[j] * pitch)[piece[j]] =
+                            float4{held[j].x * xv.x, held[j].y * xv.y, held[j].z * xv.z, held[j].w * xv.w};
+                    }
+                }
             }
         };
         bring(0);
@@ -196,7 +186,7 @@ __device__ __forceinline__ int pf_route_fix_block(const float *router, const flo
                 if (c + 1 < chunks) bring(c + 1);
             } else {   // lanes beyond the rows sum the last row again, unused
                 const int first = c * chunk, pieces = min(chunk, H - first) / 4;
-                sum = pf_serial_chunk(sum, stage + (c & 1) * PF_FIX_CHUNK_FLOATS + min(lane, n - 1) * pitch, xs + first, pieces);
+                sum = pf_serial_chunk(sum, stage + (c & 1) * PF_FIX_CHUNK_FLOATS + min(lane, n - 1) * pitch, pieces);
             }
             __syncthreads();
         }

@@ -71,28 +71,28 @@ def decode_tokens(weights, count, seed, min_margin=1e-3, max_margin=None):
     return np.ascontiguousarray(x), {"drawn": drawn, "kept_fraction": float(sum(len(k) for k in kept) / drawn)}
 
 
-def verify_batches(weights, batches, seed, rho=0.85, min_margin=1e-3):
-    """Groups of 4 consecutive tokens x_t = rho x_(t-1) + sqrt(1-rho^2) n_t (RMS-normalised), which
-    makes adjacent tokens share about half of their top-10 experts; returns x [batches,4,H]
+def verify_batches(weights, batches, seed, rho=0.85, min_margin=1e-3, group=4):
+    """Groups of `group` consecutive tokens x_t = rho x_(t-1) + sqrt(1-rho^2) n_t (RMS-normalised), which
+    makes adjacent tokens share about half of their top-10 experts; returns x [batches,group,H]
     and the achieved mean overlap and mean unique experts per batch."""
     synth, cfg = Synth(), weights.cfg
     out, overlaps, uniques, draw = [], [], [], 0
     while len(out) < batches:
-        n = synth.normal((4 * max(64, batches), cfg.hidden_size), seed * 1000 + draw).reshape(-1, 4, cfg.hidden_size)
+        n = synth.normal((group * max(64, batches), cfg.hidden_size), seed * 1000 + draw).reshape(-1, group, cfg.hidden_size)
         draw += 1
         x = np.empty_like(n)
         x[:, 0] = n[:, 0]
-        for t in range(1, 4):
+        for t in range(1, group):
             x[:, t] = rho * x[:, t - 1] + np.sqrt(1 - rho * rho) * n[:, t]
         x = rms_normalise(x)
         z = router_logits64(weights, x.reshape(-1, cfg.hidden_size))
-        ok = (top_margins(z, cfg.top_k) >= min_margin).reshape(-1, 4).all(axis=1)
-        ids = np.argsort(-z, axis=1, kind="stable")[:, :cfg.top_k].reshape(-1, 4, cfg.top_k)
+        ok = (top_margins(z, cfg.top_k) >= min_margin).reshape(-1, group).all(axis=1)
+        ids = np.argsort(-z, axis=1, kind="stable")[:, :cfg.top_k].reshape(-1, group, cfg.top_k)
         for b in np.nonzero(ok)[0]:
             if len(out) == batches:
                 break
             out.append(x[b])
-            overlaps.append(np.mean([len(set(ids[b, t]) & set(ids[b, t + 1])) / cfg.top_k for t in range(3)]))
+            overlaps.append(np.mean([len(set(ids[b, t]) & set(ids[b, t + 1])) / cfg.top_k for t in range(group - 1)]))
             uniques.append(len(set(ids[b].reshape(-1))))
     return np.ascontiguousarray(np.stack(out)), {"mean_adjacent_overlap": float(np.mean(overlaps)),
                                                   "mean_unique_experts": float(np.mean(uniques))}
