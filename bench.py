@@ -92,6 +92,9 @@ WORKLOADS = {
     "q4k_decode_streamed": dict(type=abi.GGUF_Q4_K, tokens=1, steps=512, warmup=0, streamed=448,
                                 label="Q4_K experts, decode batch 1, routed experts streamed from a file through a pool of 448 "
                                       "slots for 512 experts"),
+    "iq2xxs_decode_streamed": dict(type=abi.GGUF_IQ2_XXS, tokens=1, steps=512, warmup=0, streamed=448,
+                                   label="IQ2_XXS experts, decode batch 1, routed experts streamed from a file through a pool of "
+                                         "448 slots for 512 experts"),
     "q4k_stack48": dict(type=abi.GGUF_Q4_K, tokens=1, steps=100, warmup=10,
                         label="48 independent Q4_K layers resident in HBM, decode batch 1 and 2048-token prefill chunks, "
                               "uniform and Zipf(1.1) expert popularity"),

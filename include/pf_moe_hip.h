@@ -217,11 +217,12 @@ int pf_hip_exact_combine_host(const float *down, const uint64_t *pair_to_row, co
  * regions, the payload bytes of one expert and the offset of the scales in each (pf_hip_pool_region_plan's
  * layout for the pool's slot count), the slot count and the pairs' slots to the second, which runs the
  * expert products and the combine.  pf_hip_moe_forward_* refuse such a layer.
- * tiled_mask, the same in both calls: bit j set when region j holds Q4_K slots in the tile order (what
- * pf_hip_pool_store writes where pf_hip_pool_slot_tiled says so).  With every Q4_K region set -- all three
- * of a layer that is Q4_K throughout, gate and up of one in the q4 checkpoint profile (MXFP4 down, Q8_0
- * shared expert) -- batches of up to 16 tokens run the decode kernels on the slots (the first call the router
- * kernel and the routing, the second the expert kernels); otherwise the general kernels. */
+ * tiled_mask, the same in both calls: bit j set when region j holds Q4_K or IQ2_XXS slots in the tile order
+ * (what pf_hip_pool_store writes where pf_hip_pool_slot_tiled says so).  With every such region set -- all
+ * three of a layer that is Q4_K or IQ2_XXS throughout, gate and up of one in a checkpoint profile (Q4_K with
+ * an MXFP4 down tensor, IQ2_XXS with a Q2_K one; Q8_0 shared expert) -- batches of up to 16 tokens run the
+ * decode kernels on the slots (the first call the router kernel and the routing, the second the expert
+ * kernels); otherwise the general kernels, which read either order. */
 int pf_hip_moe_route_streamed_host(const PfHipMoe *moe, PfHipWork *work, const float *x, size_t x_pitch_bytes,
                                    size_t tokens, uint32_t tiled_mask, uint32_t *ids, uint32_t *error_word);
 int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const void *const regions[3],
@@ -236,8 +237,9 @@ int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *work, const
  * MXFP4 as all payloads, then all scales).  pf_hip_pool_region_plan gives the region's size, the bytes
  * of one expert in the file, the bytes of its payload in a slot and the offset of the scales (0: not split); pf_hip_pool_store copies one
  * expert's file bytes from host memory into a slot, splitting on the device where the format needs it
- * (a Q4_K matrix whose row count is a multiple of 32 goes into the tile order: pf_hip_pool_slot_tiled),
- * and returns when the slot is readable. */
+ * (a Q4_K or IQ2_XXS matrix whose row count is a multiple of 32 goes into the tile order:
+ * pf_hip_pool_slot_tiled; an IQ2_XXS slot in that order holds its block scales inside its chunks, so the
+ * scale offset is 0 and the payload bytes are those of the chunks), and returns when the slot is readable. */
 int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, size_t *region_bytes,
                             size_t *file_expert_bytes, size_t *payload_expert_bytes, size_t *scale_offset);
 int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, void *region, size_t slot,

@@ -311,10 +311,12 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
     // expert): tile-ordered copies of its shared expert's tensors as the resident layer keeps them, so that short batches
     // run the tile decode kernels on pool slots (Q4_K slots in tile order; the routed tensors are not here to be copied).
     if (m->streamed) {
-        bool all_q4k = true, q4_profile = desc->type[1] == PF_Q4_K && desc->type[2] == PF_Q4_K && desc->type[3] == PF_MXFP4;
-        for (int a = 1; a <= 6; a++) all_q4k &= desc->type[a] == PF_Q4_K;
-        for (int a = 4; a <= 6; a++) q4_profile &= desc->type[a] == PF_Q8_0;
-        const int combination = all_q4k ? 1 : q4_profile ? 4 : 0;
+        bool all_q4k = true, all_iq2 = true;
+        bool q4_profile = desc->type[1] == PF_Q4_K && desc->type[2] == PF_Q4_K && desc->type[3] == PF_MXFP4;
+        bool q2_profile = desc->type[1] == PF_IQ2_XXS && desc->type[2] == PF_IQ2_XXS && desc->type[3] == PF_Q2_K;
+        for (int a = 1; a <= 6; a++) { all_q4k &= desc->type[a] == PF_Q4_K; all_iq2 &= desc->type[a] == PF_IQ2_XXS; }
+        for (int a = 4; a <= 6; a++) { q4_profile &= desc->type[a] == PF_Q8_0; q2_profile &= desc->type[a] == PF_Q8_0; }
+        const int combination = all_q4k ? 1 : all_iq2 ? 2 : q2_profile ? 3 : q4_profile ? 4 : 0;
         const char *copy = getenv("PF_MOE_PREFILL_COPY");
         if (combination && pf_decode_supported(*desc) && (!copy || strcmp(copy, "0") != 0)) {
             hipError_t e = hipSuccess;
@@ -326,7 +328,17 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
                     m->total_bytes += m->bytes[a];
                 }
             }
-            for (int a = 4; a <= 5 && e == hipSuccess && combination == 4; a++) {
+            for (int a = 4; a <= 6 && e == hipSuccess && combination == 2; a++) {
+                if (n_out[a] % 32) { e = hipErrorInvalidValue; break; }
+                const size_t bytes = pf_i2t_expert_bytes((int)n_out[a], m->blocks_per_row[a]);
+                e = hipMalloc((void **)&m->w_itile[a], bytes);
+                if (e == hipSuccess) {
+                    pf_launch_iq2_tile(m->w[a], reinterpret_cast<const uint16_t *>(m->w[a] + m->scale_offset[a]), m->w_itile[a],
+                                       (size_t)n_out[a], m->blocks_per_row[a], nullptr);
+                    m->total_bytes += bytes;
+                }
+            }
+            for (int a = 4; a <= 5 && e == hipSuccess && (combination == 4 || combination == 3); a++) {
                 if (n_out[a] % 32 || k_storage[a] % 64) { e = hipErrorInvalidValue; break; }
                 const size_t bytes = pf_q8t_expert_bytes((int)n_out[a], (int)(k_storage[a] / 64));
                 e = hipMalloc((void **)&m->w_qtile[a], bytes);
@@ -338,14 +350,19 @@ extern "C" int pf_hip_moe_create(const PfHipMoeDesc *desc, const void *const hos
             }
             if (e == hipSuccess) e = hipDeviceSynchronize();
             if (e == hipSuccess) {
-                const uint8_t *tiled[8];
-                for (int a = 0; a < 8; a++) tiled[a] = a >= 1 && a <= 3 ? m->w[0] : m->w_tiled[a];   // 1..3: any non-null address, the pool's at forward time
-                const bool slots_tile = n_out[1] % 32 == 0 && (combination == 4 || n_out[3] % 32 == 0);
-                if (slots_tile && pf_decode_tile_layer(m->desc, tiled, m->w_itile, m->w_qtile) == combination) m->stream_decode = combination;
+                const uint8_t *tiled[8], *itiled[8];   // 1..3: any non-null address stands for the pool's at forward time
+                for (int a = 0; a < 8; a++) {
+                    const bool routed = a >= 1 && a <= 3;
+                    tiled[a] = routed && desc->type[a] == PF_Q4_K ? m->w[0] : m->w_tiled[a];
+                    itiled[a] = routed && desc->type[a] == PF_IQ2_XXS ? m->w[0] : m->w_itile[a];
+                }
+                const bool slots_tile = n_out[1] % 32 == 0 && (combination >= 3 || n_out[3] % 32 == 0);
+                if (slots_tile && pf_decode_tile_layer(m->desc, tiled, itiled, m->w_qtile) == combination) m->stream_decode = combination;
             } else {
                 (void)hipGetLastError();   // without the copies the general kernels serve every batch
                 for (int a = 4; a <= 6; a++) {
                     if (m->w_tiled[a]) { (void)hipFree(m->w_tiled[a]); m->w_tiled[a] = nullptr; }
+                    if (m->w_itile[a]) { (void)hipFree(m->w_itile[a]); m->w_itile[a] = nullptr; }
                     if (m->w_qtile[a]) { (void)hipFree(m->w_qtile[a]); m->w_qtile[a] = nullptr; }
                 }
             }
@@ -925,13 +942,35 @@ extern "C" int pf_hip_moe_forward_host(const PfHipMoe *moe, PfHipWork *work, con
 // expert ids; the caller makes those experts resident (qw4_pool_acquire) and passes the pool's device regions and
 // the pairs' slots to the second, which runs the expert products and the combine reading rows at
 // region + slot * expert_bytes.  The general kernels serve both: streaming is bound by the reads that fill the pool.
-extern "C" int pf_hip_pool_slot_tiled(uint32_t gguf_type, size_t n_out) { return gguf_type == PF_Q4_K && n_out % 32 == 0; }
+extern "C" int pf_hip_pool_slot_tiled(uint32_t gguf_type, size_t n_out) {
+    return (gguf_type == PF_Q4_K || gguf_type == PF_IQ2_XXS) && n_out % 32 == 0;
+}
+
+// A pool region of `slots` experts of one matrix in the layout the kernels read a slot in: pf_tensor_place (a resident
+// tensor of `slots` experts; Q4_K tile order has the file's size), or for IQ2_XXS slots in tile order the chunks of
+// pf_decode_addr.h with the block scales inside them.
+struct SlotPlan { size_t region_bytes, file_expert_bytes, expert_bytes, scale_offset; int blocks_per_row; };
+static bool slot_plan(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, SlotPlan *p) {
+    PfTensorPlace place;
+    if (!slots || !n_out || !pf_tensor_place(gguf_type, k_storage, n_out, slots, &place)) return false;
+    p->region_bytes = place.bytes;
+    p->file_expert_bytes = place.gguf_bytes / slots;
+    p->expert_bytes = place.expert_bytes;
+    p->scale_offset = place.scale_offset;
+    p->blocks_per_row = place.blocks_per_row;
+    if (gguf_type == PF_IQ2_XXS && pf_hip_pool_slot_tiled(gguf_type, n_out)) {
+        p->expert_bytes = pf_i2t_expert_bytes((int)n_out, place.blocks_per_row);
+        p->region_bytes = p->expert_bytes * slots;
+        p->scale_offset = 0;
+    }
+    return true;
+}
 
 // Short batches of a streamed layer whose Q4_K pool regions hold tile-ordered slots (all three of a Q4_K layer; gate and
 // up of the q4 checkpoint profile, whose MXFP4 down slots stay row by row) run the tile decode kernels: kernel 1 and the
 // routing kernels in the first call, kernels 2 and 3 reading the pairs' slots in the second.
 static bool streamed_decode(const PfHipMoe *moe, const PfHipWork *work, size_t tokens, uint32_t tiled_mask) {
-    const uint32_t wanted = moe->stream_decode == 1 ? 7u : 3u;
+    const uint32_t wanted = moe->stream_decode <= 2 ? 7u : 3u;   // one format throughout: all three regions; a profile: gate and up
     return moe->stream_decode && tiled_mask == wanted && tokens <= PF_TILE_DECODE_MAX_TOKENS && !work->force_general;
 }
 
@@ -995,11 +1034,15 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
     const size_t H = moe->desc.hidden, K = moe->desc.top_k;
     for (int j = 0; j < 3; j++) {   // a slot holds one expert of each tensor in the device layout of `pool_slots` experts
         PfTensorPlace place;
+        SlotPlan plan;
         const int t = 1 + j;
         const size_t k_storage = t == 3 ? moe->desc.down_physical : moe->desc.hidden;
         if (!regions[j] || !scale_offsets || !pf_tensor_place(moe->desc.type[t], k_storage, (size_t)moe->n_out[t], pool_slots, &place) ||
-            expert_bytes[j] != place.expert_bytes || scale_offsets[j] != place.scale_offset)
+            !slot_plan(moe->desc.type[t], k_storage, (size_t)moe->n_out[t], pool_slots, &plan))
             return PF_HIP_E_ARGUMENT;
+        const bool tiled = (tiled_mask >> j) & 1u;   // a pool of file bytes under split formats is refused further down
+        const size_t want_bytes = tiled ? plan.expert_bytes : place.expert_bytes, want_scales = tiled ? plan.scale_offset : place.scale_offset;
+        if (expert_bytes[j] != want_bytes || scale_offsets[j] != want_scales) return PF_HIP_E_ARGUMENT;
     }
     const bool staged = through_host_block(work, tokens);
     const HostBlock b = host_block(&moe->desc, work->host);
@@ -1014,8 +1057,10 @@ extern "C" int pf_hip_moe_experts_streamed_host(const PfHipMoe *moe, PfHipWork *
         const int t = 1 + j;
         const bool tiled = (tiled_mask >> j) & 1u;
         if (tiled && !pf_hip_pool_slot_tiled(moe->desc.type[t], (size_t)moe->n_out[t])) return PF_HIP_E_ARGUMENT;
-        a.w[t] = tiled ? nullptr : static_cast<const uint8_t *>(regions[j]);    // Q4_K slots in tile order: every kernel's tile reader
-        a.wt[t] = tiled ? static_cast<const uint8_t *>(regions[j]) : nullptr;
+        const bool iq2 = moe->desc.type[t] == PF_IQ2_XXS;
+        a.w[t] = tiled ? nullptr : static_cast<const uint8_t *>(regions[j]);    // slots in tile order: every kernel's tile reader
+        a.wt[t] = tiled && !iq2 ? static_cast<const uint8_t *>(regions[j]) : nullptr;
+        a.wi[t] = tiled && iq2 ? static_cast<const uint8_t *>(regions[j]) : nullptr;
         a.scale_offset[t] = scale_offsets[j];
     }
     a.slots = work->slots;
@@ -1064,14 +1109,14 @@ struct DeviceBlock {   // one allocation, freed on scope exit
 // stores them slot after slot; formats stored split as all payloads, then (256-aligned) all scales.
 extern "C" int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, size_t n_out, size_t slots, size_t *region_bytes,
                                        size_t *file_expert_bytes, size_t *payload_expert_bytes, size_t *scale_offset) {
-    PfTensorPlace place;
-    if (!region_bytes || !file_expert_bytes || !payload_expert_bytes || !scale_offset || !slots || !n_out ||
-        !pf_tensor_place(gguf_type, k_storage, n_out, slots, &place))
+    SlotPlan plan;
+    if (!region_bytes || !file_expert_bytes || !payload_expert_bytes || !scale_offset ||
+        !slot_plan(gguf_type, k_storage, n_out, slots, &plan))
         return PF_HIP_E_ARGUMENT;
-    *region_bytes = place.bytes;
-    *file_expert_bytes = place.gguf_bytes / slots;
-    *payload_expert_bytes = place.expert_bytes;
-    *scale_offset = place.scale_offset;
+    *region_bytes = plan.region_bytes;
+    *file_expert_bytes = plan.file_expert_bytes;
+    *payload_expert_bytes = plan.expert_bytes;
+    *scale_offset = plan.scale_offset;
     return PF_HIP_OK;
 }
 
@@ -1079,6 +1124,7 @@ extern "C" int pf_hip_pool_region_plan(uint32_t gguf_type, size_t k_storage, siz
 // copied to before a split or tile kernel lays them out in the slot, and a stream of the reader's own, all allocated once
 struct PfHipStage {
     uint8_t *host, *device;
+    uint8_t *split;   // the split form of an IQ2_XXS matrix on its way into the tile order (bytes + 256)
     size_t bytes;
     hipStream_t stream;
 };
@@ -1091,11 +1137,13 @@ extern "C" int pf_hip_stage_create(size_t bytes, PfHipStage **out) {
     st->bytes = bytes;
     hipError_t e = hipHostMalloc((void **)&st->host, bytes, hipHostMallocDefault);
     if (e == hipSuccess) e = hipMalloc((void **)&st->device, bytes);
+    if (e == hipSuccess) e = hipMalloc((void **)&st->split, bytes + 256);
     if (e == hipSuccess) e = hipStreamCreateWithFlags(&st->stream, hipStreamNonBlocking);
     if (e != hipSuccess) {
         pf_set_error("staging of an expert pool's reader", e);
         if (st->host) (void)hipHostFree(st->host);
         if (st->device) (void)hipFree(st->device);
+        if (st->split) (void)hipFree(st->split);
         free(st);
         return PF_HIP_E_MEMORY;
     }
@@ -1108,6 +1156,7 @@ extern "C" void pf_hip_stage_destroy(PfHipStage *st) {
     (void)hipStreamDestroy(st->stream);
     (void)hipHostFree(st->host);
     (void)hipFree(st->device);
+    (void)hipFree(st->split);
     free(st);
 }
 
@@ -1126,7 +1175,10 @@ extern "C" int pf_hip_pool_store_staged(PfHipStage *st, uint32_t gguf_type, size
         return PF_HIP_OK;
     }
     PfTensorPlace place;
-    if (!pf_tensor_place(gguf_type, k_storage, n_out, slots, &place) || place.gguf_bytes / slots != file_bytes) return PF_HIP_E_ARGUMENT;
+    SlotPlan plan;
+    if (!pf_tensor_place(gguf_type, k_storage, n_out, slots, &place) || !slot_plan(gguf_type, k_storage, n_out, slots, &plan) ||
+        plan.file_expert_bytes != file_bytes)
+        return PF_HIP_E_ARGUMENT;
     const size_t head = split_header_bytes(gguf_type);
     if (!pf_hip_pool_slot_tiled(gguf_type, n_out) && !head) {   // as the file stores it
         HIP_TRY(hipMemcpyAsync(base + slot * place.expert_bytes, st->host, file_bytes, hipMemcpyHostToDevice, st->stream));
@@ -1134,7 +1186,15 @@ extern "C" int pf_hip_pool_store_staged(PfHipStage *st, uint32_t gguf_type, size
         return PF_HIP_OK;
     }
     HIP_TRY(hipMemcpyAsync(st->device, st->host, file_bytes, hipMemcpyHostToDevice, st->stream));
-    if (pf_hip_pool_slot_tiled(gguf_type, n_out)) {   // Q4_K: the slot in the tile order every kernel family reads
+    if (pf_hip_pool_slot_tiled(gguf_type, n_out) && gguf_type == PF_IQ2_XXS) {
+        // payloads and scales apart (the upload's split kernel, into the stage), then into the slot in tile order
+        PfTensorPlace one;
+        if (!pf_tensor_place(gguf_type, k_storage, n_out, 1, &one) || one.bytes > st->bytes + 256) return PF_HIP_E_ARGUMENT;
+        const size_t blocks = (size_t)one.blocks_per_row * n_out;
+        pf_launch_iq2_split(st->device, st->split, reinterpret_cast<uint16_t *>(st->split + one.scale_offset), blocks, st->stream);
+        pf_launch_iq2_tile(st->split, reinterpret_cast<const uint16_t *>(st->split + one.scale_offset), base + slot * plan.expert_bytes,
+                           n_out, one.blocks_per_row, st->stream);
+    } else if (pf_hip_pool_slot_tiled(gguf_type, n_out)) {   // Q4_K: the slot in the tile order every kernel family reads
         pf_launch_q4k_tile(st->device, base + slot * place.expert_bytes, n_out, place.blocks_per_row, st->stream);
     } else {
         size_t block, size;
@@ -1157,6 +1217,22 @@ extern "C" int pf_hip_pool_store(uint32_t gguf_type, size_t k_storage, size_t n_
         return PF_HIP_E_ARGUMENT;
     uint8_t *base = static_cast<uint8_t *>(region);
     const size_t head = split_header_bytes(gguf_type), file_expert = place.gguf_bytes / slots;
+    if (pf_hip_pool_slot_tiled(gguf_type, n_out) && gguf_type == PF_IQ2_XXS) {
+        PfTensorPlace one;
+        SlotPlan plan;
+        if (!pf_tensor_place(gguf_type, k_storage, n_out, 1, &one) || !slot_plan(gguf_type, k_storage, n_out, slots, &plan)) return PF_HIP_E_ARGUMENT;
+        DeviceBlock staging, split;
+        HIP_TRY(hipMalloc((void **)&staging.p, file_expert));
+        HIP_TRY(hipMalloc((void **)&split.p, one.bytes));
+        HIP_TRY(hipMemcpy(staging.p, file_bytes, file_expert, hipMemcpyHostToDevice));
+        const size_t blocks = (size_t)one.blocks_per_row * n_out;
+        pf_launch_iq2_split(staging.p, split.p, reinterpret_cast<uint16_t *>(split.p + one.scale_offset), blocks, nullptr);
+        pf_launch_iq2_tile(split.p, reinterpret_cast<const uint16_t *>(split.p + one.scale_offset), base + slot * plan.expert_bytes, n_out,
+                           one.blocks_per_row, nullptr);
+        HIP_TRY(hipGetLastError());
+        HIP_TRY(hipStreamSynchronize(nullptr));
+        return PF_HIP_OK;
+    }
     if (pf_hip_pool_slot_tiled(gguf_type, n_out)) {   // Q4_K: the slot in the tile order every kernel family reads
         DeviceBlock staging;
         HIP_TRY(hipMalloc((void **)&staging.p, file_expert));

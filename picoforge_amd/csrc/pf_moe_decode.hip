@@ -2583,6 +2583,8 @@ void pf_launch_decode_iq2(const PfKernelArgs &a, int tokens, hipStream_t stream,
 void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit);
 void pf_launch_decode_q4profile_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);
+void pf_launch_decode_iq2_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);
+void pf_launch_decode_q2profile_experts(const PfKernelArgs &a, int tokens, hipStream_t stream);
 
 #if PF_DECODE_PART == 0
 void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
@@ -2591,8 +2593,12 @@ void pf_launch_decode_q4k(const PfKernelArgs &a, int tokens, hipStream_t stream,
 }
 
 void pf_launch_decode_stream_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
-    if (decode_combination(a.type) == 4) pf_launch_decode_q4profile_experts(a, tokens, stream);
-    else launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K, true>(a, tokens, stream, 3);
+    switch (decode_combination(a.type)) {
+    case 2: pf_launch_decode_iq2_experts(a, tokens, stream); break;
+    case 3: pf_launch_decode_q2profile_experts(a, tokens, stream); break;
+    case 4: pf_launch_decode_q4profile_experts(a, tokens, stream); break;
+    default: launch_q4t_experts<PF_Q4_K, PF_Q4_K, PF_Q4_K, true>(a, tokens, stream, 3);
+    }
 }
 
 int pf_decode_launches(const PfKernelArgs &a, int tokens) {
@@ -2618,11 +2624,19 @@ void pf_launch_decode_iq2(const PfKernelArgs &a, int tokens, hipStream_t stream,
         launch_decode_q4t<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit);
     else launch_decode_tokens<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS>(a, tokens, stream, stage_limit);
 }
+
+void pf_launch_decode_iq2_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
+    launch_q4t_experts<PF_IQ2_XXS, PF_IQ2_XXS, PF_IQ2_XXS, true>(a, tokens, stream, 3);
+}
 #elif PF_DECODE_PART == 2
 void pf_launch_decode_q2profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {
     if (pf_decode_tile_layer(desc_of(a), a.wt, a.wi, a.wq) == 3)
         launch_decode_q4t<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit);
     else launch_decode_tokens<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0>(a, tokens, stream, stage_limit);
+}
+
+void pf_launch_decode_q2profile_experts(const PfKernelArgs &a, int tokens, hipStream_t stream) {
+    launch_q4t_experts<PF_IQ2_XXS, PF_Q2_K, PF_Q8_0, true>(a, tokens, stream, 3);
 }
 #else
 void pf_launch_decode_q4profile(const PfKernelArgs &a, int tokens, hipStream_t stream, int stage_limit) {

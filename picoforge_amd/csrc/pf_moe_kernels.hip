@@ -130,6 +130,38 @@ __device__ __forceinline__ float dot_row_iq2(const uint8_t *payload, const uint1
     return acc;
 }
 
+// The same product on the tile-ordered copy (pf_decode_addr.h: per 32-row tile and 256-block the rows' 16-byte pieces of
+// each 64-weight run, two groups a piece, then the rows' block scales): row n of the expert whose tiles start at
+// `expert`.  Pool slots of a streamed layer are kept in this order for the decode kernels; longer batches read them here.
+__device__ __forceinline__ float dot_row_iq2_tiled(const uint8_t *expert, int n, const float *x, int nblk, int lane,
+                                                   const uint64_t *grid) {
+    const int ngroups = nblk * 8, row_in_tile = n & 31;
+    float acc = 0.0f;
+    for (int gi = lane; gi < ngroups; gi += PF_WAVE) {
+        const uint8_t *chunk = expert + pf_i2t_chunk_at(0, 0, n >> 5, nblk, gi >> 3);
+        const uint2 p = *reinterpret_cast<const uint2 *>(chunk + pf_i2t_piece_at((gi & 7) >> 1, row_in_tile) + 8 * (gi & 1));
+        const float d = pf_half_bits_to_float(*reinterpret_cast<const uint16_t *>(chunk + pf_i2t_scale_at(row_in_tile)));
+        const uint32_t idx = p.x, word = p.y;
+        const float scale = d * (float)(2u * (word >> 28) + 1u) * 0.125f;
+        const float *xg = x + 32 * gi;
+        float gacc = 0.0f;
+#pragma unroll
+        for (int slot = 0; slot < 4; slot++) {
+            const uint64_t mags = grid[(idx >> (8 * slot)) & 255u];
+            uint32_t signs = (word >> (7 * slot)) & 127u;
+            signs |= pf_parity7(signs) << 7;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float m = (float)(uint32_t)((mags >> (8 * e)) & 255u);
+                const float xv = xg[8 * slot + e];
+                gacc = fmaf((signs >> e) & 1u ? -m : m, xv, gacc);
+            }
+        }
+        acc = fmaf(scale, gacc, acc);
+    }
+    return acc;
+}
+
 // F16 / BF16 rows: two values per lane and step.
 template <bool BF>
 __device__ __forceinline__ float dot_row_16(const uint8_t *row, const float *x, int K, int lane) {
@@ -231,8 +263,9 @@ __device__ __forceinline__ float dot_tensor_row(const PfKernelArgs &a, int t, si
         break;
     case PF_MXFP4: v = dot_row_mxfp4(row, scales + first_block, x, a.blocks_per_row[t], lane); break;
     default:
-        v = dot_row_iq2(row, reinterpret_cast<const uint16_t *>(scales) + first_block, x, a.blocks_per_row[t], lane,
-                        grid);
+        v = a.w[t] ? dot_row_iq2(row, reinterpret_cast<const uint16_t *>(scales) + first_block, x, a.blocks_per_row[t], lane, grid)
+                   : dot_row_iq2_tiled(a.wi[t] + e * pf_i2t_expert_bytes(a.n_out[t], a.blocks_per_row[t]), (int)n, x,
+                                       a.blocks_per_row[t], lane, grid);
     }
     return pf_wave_sum(v);
 }

@@ -201,13 +201,14 @@ def test_streamed_layer_matches_the_cpu_path(product, oracle, tmp_path, gtype, f
     os.close(fd)
 
 
-@pytest.mark.parametrize("expert_type", [abi.GGUF_Q4_K, "q4"])
+@pytest.mark.parametrize("expert_type", [abi.GGUF_Q4_K, "q4", abi.GGUF_IQ2_XXS, "q2"])
 def test_streamed_layer_on_the_decode_kernels(product, oracle, tmp_path, expert_type):
-    """A layer of a shape the decode kernels cover, Q4_K throughout or in the q4 checkpoint profile (Q4_K gate and up,
-    MXFP4 down, Q8_0 shared expert), streamed through a pool that was told its formats: the Q4_K slots are kept in the
-    tile order and batches of up to 16 tokens run the decode kernels on them (the router kernel and the routing in the
-    first device call, the expert kernels on the pairs' slots in the second); longer batches run the general kernels
-    on the same slots.  56 slots for 64 experts: evictions on the way."""
+    """A layer of a shape the decode kernels cover -- Q4_K throughout, IQ2_XXS throughout, or in a checkpoint profile (Q4_K
+    gate and up with an MXFP4 down tensor, IQ2_XXS gate and up with a Q2_K one; the shared expert Q8_0) -- streamed
+    through a pool that was told its formats: the Q4_K and IQ2_XXS slots are kept in the tile order and batches of up to
+    16 tokens run the decode kernels on them (the router kernel and the routing in the first device call, the expert
+    kernels on the pairs' slots in the second); longer batches run the general kernels on the same slots.  56 slots for
+    64 experts: evictions on the way."""
     cfg = abi.moe_config(512, 64, 4, 256, 256)
     tokens = 40
     weights, x = make_layer_inputs(cfg, expert_type, tokens, seed=67)
