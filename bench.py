@@ -336,7 +336,8 @@ def run_layer(args, ctx, name, steps, warmup, cpu_seconds):
     lb = workloads.layer_bytes(wl["type"], cfg)
     i, s_i, k = cfg.intermediate, cfg.shared_intermediate, cfg.top_k
     extra = {}
-    if tokens == 1 and args.margin_window == (1e-3, None) and name in ("q4k_decode", "iq2xxs_decode") and not wl.get("custom_shape"):
+    if tokens == 1 and args.margin_window == (1e-3, None) and name in ("q4k_decode", "iq2xxs_decode") and not wl.get("custom_shape") \
+            and not under_tracer():   # a profiled run keeps to the plans it is there to look at
         extra["unfiltered_inputs"] = unfiltered_decode(args, ctx, weights, layer, n_inputs, steps, warmup, us_per_token)
     if prefill:
         # algorithmic bytes per launch: weights of the active experts once, activations once
@@ -774,7 +775,7 @@ def run_one(args, ctx, name, cpu_seconds):
     return run_layer(args, ctx, name, steps, warmup, cpu_seconds)
 
 
-TRACED_DISPATCH_LIMIT = 1024
+TRACED_GRAPH_NODES_LIMIT = 512
 
 
 def under_tracer():
@@ -826,18 +827,24 @@ def main():
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every box has one GPU); use --gpus 1")
 
     if under_tracer():
-        # a replay that enqueues several thousand traced graph dispatches has ended the profiled process inside the tracer
-        # (cause unexplained; 768-960 dispatches a replay ran clean): keep traced runs below that
+        # A profiled run has ended inside the tracer (a segmentation fault below a graph launch; cause unexplained) whenever
+        # the graphs it had instantiated held 640 kernel nodes or more in all, and never with 500 or fewer: refuse such a run.
         names = [args.workload] if args.workload != "all" else [HEADLINE] + ALL_CONFIGS
         for name in names:
             steps = args.steps if args.steps is not None else WORKLOADS[name]["steps"]
-            per_forward = 10 if WORKLOADS[name]["tokens"] > 4 else 4
+            wl_tokens = WORKLOADS[name]["tokens"]
+            per_forward = 10 if wl_tokens > 16 else (3 if wl_tokens < 3 else 4)
             if name == "q4k_stack48":
                 per_forward *= args.layers
-            if steps * per_forward > TRACED_DISPATCH_LIMIT:
-                sys.exit(f"under a profiler's tracer, {name} with --steps {steps} would enqueue about {steps * per_forward} traced "
-                         f"graph dispatches in one replay; keep it below {TRACED_DISPATCH_LIMIT} (e.g. --steps "
-                         f"{TRACED_DISPATCH_LIMIT // per_forward})")
+            forwards = min(steps, 64) + (steps % 64 if steps > 64 else 0)         # the 64-forward graph and the remainder's
+            nodes = forwards * per_forward
+            if WORKLOADS[name].get("hc"):
+                nodes = forwards * (3 * per_forward + 3)                          # the chain with the add folded, with its own kernel, the block alone
+            elif not args.skip_stages:
+                nodes += min(steps, 64) * per_forward * 3 // 2                    # the plans of the first 1, 2, ... kernels
+            if nodes > TRACED_GRAPH_NODES_LIMIT:
+                sys.exit(f"under a profiler's tracer, {name} with --steps {steps} would instantiate graphs of about {nodes} kernel "
+                         f"nodes; keep it to {TRACED_GRAPH_NODES_LIMIT} (--skip-stages, fewer steps, or a step count that is a multiple of 64)")
     api = pf.load_product()
     hip = api.hip
     if hip.device_count() < 1:
