@@ -66,6 +66,24 @@ def test_decode_kernels_match_oracle_and_general_kernels(product, oracle, h, e, 
             assert_parity(y, ids, w, *want, label="general kernels on a decode shape")
 
 
+@pytest.mark.parametrize("h,e,k,i,s,gtype", DECODE)
+def test_decode_kernels_on_batches_of_up_to_sixteen_tokens(product, oracle, h, e, k, i, s, gtype):
+    """From six tokens the down products run 64 output rows a workgroup with the digits as scalar operands: batches
+    on either side of that switch, whole and ragged, against the oracle."""
+    print(f"case decode batches h={h} e={e} k={k} i={i} s={s} type={gtype}", flush=True)
+    cfg = abi.moe_config(h, e, k, i, s)
+    weights, x = make_layer_inputs(cfg, gtype, 16, seed=3 * h + e + gtype)
+    x[9] = x[8]                                   # two identical tokens share every expert
+    want = forward_with(oracle, cfg, weights, x)
+    with pf.MoeLayer(product, cfg, weights, 16) as layer:
+        if product.hip.moe_kernel_family(*layer.device_handles(), 16) != 1:
+            pytest.skip("batches of 16 tokens of this layer run the prefill kernels")
+        for tokens in (5, 6, 7, 9, 13, 16):
+            print(f"  tokens={tokens}", flush=True)
+            _, y, ids, w = layer.forward(x[:tokens])
+            assert_parity(y, ids, w, want[0][:tokens], want[1][:tokens], want[2][:tokens], label=f"decode T={tokens}")
+
+
 # shapes the matrix-core prefill kernels cover (Q4_K or IQ2_XXS experts, widths in whole 256-blocks), more than 4 tokens
 PREFILL = [
     (256, 16, 4, 256, 256, 5), (256, 16, 4, 256, 256, 33), (512, 8, 3, 256, 512, 70),
