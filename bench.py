@@ -834,11 +834,11 @@ def main():
             steps = args.steps if args.steps is not None else WORKLOADS[name]["steps"]
             wl_tokens = WORKLOADS[name]["tokens"]
             per_forward = 10 if wl_tokens > 16 else (3 if wl_tokens < 3 else 4)
-            if name == "q4k_stack48":
-                per_forward *= args.layers
             forwards = min(steps, 64) + (steps % 64 if steps > 64 else 0)         # the 64-forward graph and the remainder's
             nodes = forwards * per_forward
-            if WORKLOADS[name].get("hc"):
+            if name == "q4k_stack48":                                             # a token and two 2048-token chunks through every layer, on two inputs
+                nodes = 2 * (steps * args.layers * 3 + 2 * args.layers * 10)
+            elif WORKLOADS[name].get("hc"):
                 nodes = forwards * (3 * per_forward + 3)                          # the chain with the add folded, with its own kernel, the block alone
             elif not args.skip_stages:
                 nodes += min(steps, 64) * per_forward * 3 // 2                    # the plans of the first 1, 2, ... kernels

@@ -31,3 +31,8 @@ def test_profiled_runs_keep_their_graphs_small():
     for workload, steps in (("q4k_verify4", "256"), ("q4k_decode", "256"), ("q4k_prefill1024", "20")):
         r = run_bench("--workload", workload, "--steps", steps, "--skip-stages", env=tracer)
         assert "kernel nodes" not in r.stderr
+    # the 48-layer stack replays a token and two 2048-token chunks through every layer: never under a tracer as it is
+    r = run_bench("--workload", "q4k_stack48", "--steps", "3", "--skip-stages", env=tracer)
+    assert r.returncode != 0 and "kernel nodes" in r.stderr
+    r = run_bench("--workload", "q4k_stack48", "--steps", "3", "--layers", "8", "--skip-stages", env=tracer)
+    assert "kernel nodes" not in r.stderr
