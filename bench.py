@@ -507,8 +507,11 @@ def run_stack(args, ctx, steps, warmup, cpu_seconds):
     for l in layers:
         l.close()
     hip.free(d_y)
+    if args.copy_probe:
+        tools.check(tools.lib.pf_bench_copy_probe(args.copy_probe << 20, 3), "copy probe")
     us = out["uniform_decode_us_per_token"]
     alg = layers_n * workloads.algorithmic_bytes_per_token(abi.GGUF_Q4_K)
+    per_layer, traffic_from = measured_traffic("q4k_stack48")   # the three decode kernels of one layer of a stack, cold caches
     return {
         "metric": "moe_stack_decode_us_per_token", "value": round(us, 2), "unit": "us/token (all layers)",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(us * 1e-3, 6),
@@ -522,7 +525,8 @@ def run_stack(args, ctx, steps, warmup, cpu_seconds):
         "algorithmic_bytes_per_step": int(alg),
         "roofline": {"bound": "hbm", "kernel": "whole stack: three decode kernels per layer", "achieved":
                      round(alg / (us * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None},
+                     "frac": round(alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "traffic": None if per_layer is None else int(per_layer) * layers_n, "traffic_from": traffic_from},
         "stack": {k: round(v, 3) for k, v in out.items()}, "stack_spread": spread,
         "cpu_baseline": {"value": round(cpu_s / n * 1e6 * layers_n, 1), "unit": "us/token (all layers)", "cores": 1,
                          "kind": kind, "sample": f"{n} tokens through layer 0 ({cpu_s:.1f} s), times {layers_n} layers: "
